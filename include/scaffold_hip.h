@@ -1,0 +1,153 @@
+/*
+ * scaffold_hip.h -- C ABI of libscaffold_hip.so: the MI355X (gfx950) kernels behind the
+ * ScaFFold 3D U-Net compute hot path (channels-last conv3d forward / data-gradient /
+ * weight-gradient, kernel==stride transposed conv3d, channels-last GroupNorm fwd/bwd).
+ *
+ * Conventions (all entry points):
+ *   - every tensor pointer is a DEVICE pointer on the current HIP device; nothing is
+ *     allocated, freed or synchronised by the library; `stream` is a hipStream_t (NULL =
+ *     the default stream) and all work is enqueued on it;
+ *   - activations are dense NDHWC ("channels_last_3d"): element (n,c,d,h,w) lives at
+ *     (((n*D + d)*H + h)*W + w)*C + c;
+ *   - weights are read where they lie: `w_stride[5]` are ELEMENT strides of the logical
+ *     (Cout, Cin, kd, kh, kw) tensor (for the transposed conv: (Cin, Cout, kd, kh, kw));
+ *   - return value 0 = success, otherwise one of SFH_ERR_*; sfh_last_error() returns a
+ *     thread-local human-readable message for the last failure on this thread;
+ *   - launch geometry (tiles, split counts) is a pure function of the descriptor and dtype,
+ *     and no floating-point atomics are used: the same call gives the same bits.
+ *
+ * Each declaration cites the reference interface (LBANN/ScaFFold) that it stands in for.
+ */
+#ifndef SCAFFOLD_HIP_H
+#define SCAFFOLD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SFH_OK 0
+#define SFH_ERR_INVALID 1     /* contract violation (null pointer, bad enum, inconsistent sizes) */
+#define SFH_ERR_UNSUPPORTED 2 /* a problem this library does not serve (e.g. dgrad at stride != 1) */
+#define SFH_ERR_WORKSPACE 3   /* workspace missing or smaller than *_workspace_bytes() */
+#define SFH_ERR_LAUNCH 4      /* the HIP runtime refused a launch */
+
+/* Element type of activations and weights; accumulation is always fp32. */
+#define SFH_BF16 0
+#define SFH_FP16 1
+#define SFH_FP32 2
+
+/* Flags for the convolution entry points. */
+#define SFH_FLAG_FORCE_GENERIC 1u /* use the direct (non-MFMA) kernels whatever the shape */
+
+/* A convolution problem as torch.nn.functional.conv3d names it (groups == 1). */
+typedef struct sfh_conv3d_desc {
+  int32_t n, cin, in_d, in_h, in_w;
+  int32_t cout, kd, kh, kw;
+  int32_t sd, sh, sw; /* stride   */
+  int32_t pd, ph, pw; /* padding  */
+  int32_t dd, dh, dw; /* dilation */
+} sfh_conv3d_desc;
+
+/* A kernel==stride, padding 0 transposed convolution (the U-Net up-convolution). */
+typedef struct sfh_convT3d_desc {
+  int32_t n, cin, in_d, in_h, in_w;
+  int32_t cout, kd, kh, kw; /* stride == kernel */
+} sfh_convT3d_desc;
+
+/* A GroupNorm problem over a dense (N, S, C) channels-last tensor, S = D*H*W. */
+typedef struct sfh_groupnorm_desc {
+  int32_t n, c, groups;
+  int32_t relu;    /* 1: fuse y = relu(y) into the store / gate the backward on the pre-activation */
+  int64_t spatial; /* S */
+  float eps;
+} sfh_groupnorm_desc;
+
+/* ---- library ------------------------------------------------------------------------ */
+int sfh_version(void);
+const char* sfh_last_error(void);
+/* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
+int sfh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* lds_bytes);
+/* Output spatial extents of a conv3d problem; SFH_ERR_INVALID if the output would be empty. */
+int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]);
+/* 1 if the MFMA implicit-GEMM kernels (rather than the direct kernels) serve this problem
+ * in the given direction: 0 = forward, 1 = data-gradient, 2 = weight-gradient. */
+int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
+
+/* ---- conv3d forward ------------------------------------------------------------------
+ * Stands in for triton_conv3d.conv3d_forward (triton_conv3d/gather_gemm.py:1187) and its
+ * kernel _conv3d_fwd_kernel (gather_gemm.py:112).
+ * y[n,co,od,oh,ow] = bias[co] + sum_{ci,kd,kh,kw} x[n,ci,od*sd+kd*dd-pd,...] * w[co,ci,kd,kh,kw]
+ * bias may be NULL; when given it has Cout elements of the activation dtype.
+ * The workspace holds the weight repacked into MFMA fragment order. */
+size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
+int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w,
+                   const int64_t w_stride[5], const void* bias, void* y, void* workspace,
+                   size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- conv3d data gradient ------------------------------------------------------------
+ * Stands in for triton_conv3d.conv3d_backward_data (triton_conv3d/bwd_data.py:275).
+ * `p` describes the FORWARD problem; gy has its output shape, gx its input shape.
+ * Served for stride 1 and padding <= dilation*(k-1) only (bwd_data.py:250-253). */
+size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
+int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w,
+                     const int64_t w_stride[5], void* gx, void* workspace,
+                     size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- conv3d weight gradient ----------------------------------------------------------
+ * Stands in for triton_conv3d.conv3d_backward_weight (triton_conv3d/reduce_gemm.py:1177),
+ * _conv3d_bwd_weight_kernel (:137) and _reduce_partials_kernel (:396).
+ * gw is written dense as [Cout][kd][kh][kw][Cin] (channels_last_3d for a weight) in the
+ * activation dtype, from fp32 split partials summed in a fixed order.
+ * sfh_conv3d_wgrad_splits() reports the number of partial slices (1 = no workspace pass). */
+int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype);
+size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
+int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw,
+                     void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- transposed conv3d (kernel == stride) forward ------------------------------------
+ * Stands in for triton_conv3d.conv_transpose3d_forward (triton_conv3d/transposed.py:941)
+ * and _convT3d_fwd_kernel (:135).
+ * y[n,oc,d*kd+a,h*kh+b,w*kw+c] = bias[oc] + sum_ic x[n,ic,d,h,w] * w[ic,oc,a,b,c].
+ * Its data gradient is sfh_conv3d_fwd at stride k (transposed.py:1073) and its weight
+ * gradient sfh_conv3d_wgrad at stride k with the operands swapped (transposed.py:1113). */
+size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int dtype);
+int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w,
+                    const int64_t w_stride[5], const void* bias, void* y, void* workspace,
+                    size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- GroupNorm forward ---------------------------------------------------------------
+ * Stands in for torch.ops.scaffold_gn.group_norm (ScaFFold/unet/triton_group_norm.py:1339)
+ * and its kernels _stats_partial_kernel (:609) and _normalize_kernel (:697).
+ * x: (N,S,C) of x_dtype; gamma/beta: C elements of param_dtype or NULL; y: (N,S,C) of
+ * y_dtype; mean, rstd: (N, groups) fp32. Statistics and the normalisation are fp32. */
+size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype);
+int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
+                      const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                      float* rstd, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- GroupNorm backward --------------------------------------------------------------
+ * Stands in for torch.ops.scaffold_gn.group_norm_backward (triton_group_norm.py:1394) and
+ * its kernels _bwd_partial_kernel (:813) and _dx_kernel (:908).
+ * x, dx: (N,S,C) of x_dtype; dy: (N,S,C) of dy_dtype (x_dtype, or fp32 when the forward
+ * produced an fp32 output from a 16-bit input); dgamma, dbeta: C fp32 elements each (either
+ * may be NULL).
+ * With p->relu the incoming gradient is gated on the recomputed pre-activation. */
+size_t sfh_groupnorm_bwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype);
+int sfh_groupnorm_bwd(const sfh_groupnorm_desc* p, int x_dtype, int dy_dtype, int param_dtype,
+                      const void* dy, const void* x, const void* gamma, const void* beta, const float* mean,
+                      const float* rstd, void* dx, float* dgamma, float* dbeta, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* ---- measurement helper --------------------------------------------------------------
+ * A plain streaming copy of `bytes` bytes (multiple of 16) used to calibrate achieved HBM
+ * bandwidth and the scale of the FETCH_SIZE / WRITE_SIZE counters. Has no counterpart in the
+ * reference (its bench harness times torch copies, triton_conv3d/bench/harness.py:62). */
+int sfh_stream_copy(const void* src, void* dst, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SCAFFOLD_HIP_H */

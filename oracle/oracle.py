@@ -1,0 +1,390 @@
+"""CPU oracle for the ScaFFold U-Net hot path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the product (``scaffold_amd/``) may import this module: it is the checker, used by
+``tests/``, by ``__graft_entry__.smoke()`` and by the ``cpu_baseline`` leg of ``bench.py``.
+
+What it restates, and what pins each function (so a dropped term, a wrong sign or a transposed
+operand fails a test in ``tests/test_oracle.py``):
+
+======================  =========================================================  =====================================
+function                reference it follows                                        pinned by
+======================  =========================================================  =====================================
+``conv_reference``      ``triton_conv3d/reference.py:201-238`` (fp64 ``F.conv3d`` /   brute-force C loops (``conv_ref.c``),
+                        ``F.conv_transpose3d`` + ``torch.autograd.grad``)            delta-input closed form, adjoint
+                                                                                     identities <conv x, g> = <x, dgrad g>
+``make_inputs``         ``reference.py:63-138`` (seeded operands, ``{-1,0,1}`` exact   value-set / density / determinism checks
+                        draw with activation thinning)
+``exact_density``       ``reference.py:141-174`` closed form                         hand-computed values
+``is_exactly_repr...``  ``reference.py:177-193``                                     integers at / beyond the mantissa limit
+``compare``,            ``reference.py:289-361`` (RMS-normalised error; bound =        hand-computed report / bound
+``error_bound``         8 u32 sqrt(K) rms + 2 r u_dtype peak)
+``group_norm_reference``  ``tests/test_triton_group_norm.py:114-129`` (fp64             independent from-scratch formula
+                        ``F.group_norm`` + ``F.relu`` + autograd)                     (``group_norm_manual``), C loops,
+                                                                                     zero-variance / one-element-group cases
+``train_step_loss``     ``ScaFFold/utils/trainer.py:640-663`` (fp32 log-softmax,      closed form on a two-voxel example
+                        CE + 1 - mean foreground Dice, eps 1e-6)
+======================  =========================================================  =====================================
+
+The reference's own oracle *is* a library routine (torch in fp64), so this file calls the same
+routine; the reference's Python is read, never imported.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Optional, Sequence
+
+import torch
+import torch.nn.functional as F
+
+MANTISSA_BITS = {torch.float64: 53, torch.float32: 24, torch.bfloat16: 8, torch.float16: 11}
+
+
+def unit_roundoff(dtype: torch.dtype) -> float:
+    return 2.0 ** -MANTISSA_BITS[dtype]
+
+
+def _triple(v):
+    return (v, v, v) if isinstance(v, int) else tuple(int(a) for a in v)
+
+
+@dataclasses.dataclass(frozen=True)
+class ConvProblem:
+    """One convolution: logical NCDHW shapes, FLOPs and compulsory bytes (``triton_conv3d/shapes.py:288-340``)."""
+
+    n: int
+    cin: int
+    cout: int
+    spatial: tuple  # input (D, H, W)
+    kernel: tuple = (3, 3, 3)
+    stride: tuple = (1, 1, 1)
+    padding: tuple = (1, 1, 1)
+    transposed: bool = False
+    bias: bool = False
+    dtype: torch.dtype = torch.bfloat16
+
+    @property
+    def input_shape(self):
+        return (self.n, self.cin, *self.spatial)
+
+    @property
+    def weight_shape(self):
+        return ((self.cin, self.cout) if self.transposed else (self.cout, self.cin)) + tuple(self.kernel)
+
+    @property
+    def output_spatial(self):
+        if self.transposed:
+            return tuple((i - 1) * s - 2 * p + k for i, s, p, k in zip(self.spatial, self.stride, self.padding, self.kernel))
+        return tuple((i + 2 * p - k) // s + 1 for i, s, p, k in zip(self.spatial, self.stride, self.padding, self.kernel))
+
+    @property
+    def output_shape(self):
+        return (self.n, self.cout, *self.output_spatial)
+
+    @property
+    def taps(self):
+        return self.kernel[0] * self.kernel[1] * self.kernel[2]
+
+    def flops(self) -> int:
+        """2*N*vol*Cin*Cout*taps; for a k == s transposed conv ``vol`` is the INPUT volume."""
+        vol = math.prod(self.spatial if self.transposed else self.output_spatial)
+        return 2 * self.n * vol * self.cin * self.cout * self.taps
+
+    def bytes(self) -> int:
+        """x + w + y once each."""
+        item = torch.empty((), dtype=self.dtype).element_size()
+        return item * (math.prod(self.input_shape) + math.prod(self.weight_shape) + math.prod(self.output_shape))
+
+    def gemm_shape(self, direction: str = "fwd"):
+        """(M, N, K) of the GEMM each direction runs."""
+        vox_out = self.n * math.prod(self.output_spatial)
+        vox_in = self.n * math.prod(self.spatial)
+        if self.transposed:
+            if direction == "fwd":
+                return (vox_in, self.cout * self.taps, self.cin)
+            if direction == "bwd-data":
+                return (vox_in, self.cin, self.cout * self.taps)
+            return (self.cin, self.cout * self.taps, vox_in)
+        if direction == "fwd":
+            return (vox_out, self.cout, self.cin * self.taps)
+        if direction == "bwd-data":
+            return (vox_in, self.cin, self.cout * self.taps)
+        return (self.cout, self.cin * self.taps, vox_out)
+
+
+# ---------------------------------------------------------------------------------------------
+# operands
+# ---------------------------------------------------------------------------------------------
+def make_inputs(problem: ConvProblem, *, seed: int = 0, exact: bool = False, density: Optional[float] = None,
+                channels_last: bool = True, dtype: Optional[torch.dtype] = None) -> dict:
+    """Input, weight, bias and upstream gradient, drawn on the CPU generator (identical bits on
+    every machine).  ``exact=True`` draws from {-1, 0, 1}; ``density`` then thins the two
+    activations (never the weight) so realised sums stay inside the mantissa."""
+    dtype = dtype or problem.dtype
+    thin = exact and density is not None and density < 1.0
+
+    def draw(shape, offset, activation=False):
+        g = torch.Generator().manual_seed(seed + offset)
+        if exact:
+            t = torch.randint(-1, 2, shape, generator=g, dtype=torch.int8).to(dtype)
+            if thin and activation:
+                gm = torch.Generator().manual_seed(seed + offset + (1 << 20))
+                t = t * (torch.rand(shape, generator=gm) < density).to(dtype)
+            return t
+        return torch.randn(shape, generator=g, dtype=torch.float32).to(dtype)
+
+    fmt = torch.channels_last_3d if channels_last else torch.contiguous_format
+    out = {
+        "input": draw(problem.input_shape, 0, True).contiguous(memory_format=fmt),
+        "weight": draw(problem.weight_shape, 1).contiguous(memory_format=fmt),
+        "grad_output": draw(problem.output_shape, 2, True).contiguous(memory_format=fmt),
+        "bias": draw((problem.cout,), 3) if problem.bias else None,
+    }
+    return out
+
+
+def exact_density(problem: ConvProblem, direction: str = "fwd", *, dtype=None, headroom: float = 4.0) -> float:
+    """q = min(1, (1.5 * 2^mant / headroom / sqrt(2 ln(MN)))^2 / K)."""
+    dtype = dtype or problem.dtype
+    m, n, k = problem.gemm_shape(direction)
+    if k <= 0 or m * n <= 0:
+        return 1.0
+    limit = 2 ** MANTISSA_BITS[dtype] / headroom
+    spread = math.sqrt(2.0 * math.log(max(m * n, 2)))
+    return min(1.0, (1.5 * limit / spread) ** 2 / k)
+
+
+def is_exactly_representable(result: torch.Tensor, dtype: torch.dtype) -> bool:
+    finite = result[torch.isfinite(result)]
+    if finite.numel() == 0:
+        return True
+    return bool(torch.equal(finite, finite.round()) and finite.abs().max().item() < 2 ** MANTISSA_BITS[dtype])
+
+
+# ---------------------------------------------------------------------------------------------
+# convolution references
+# ---------------------------------------------------------------------------------------------
+def _conv(problem: ConvProblem, x, w, b):
+    op = F.conv_transpose3d if problem.transposed else F.conv3d
+    return op(x, w, b, stride=problem.stride, padding=problem.padding)
+
+
+def conv_reference(problem: ConvProblem, operands: dict, direction: str = "fwd", *, dtype=torch.float64) -> torch.Tensor:
+    """The trusted answer in ``dtype`` (fp64): forward value, or the requested gradient via autograd."""
+    x = operands["input"].to(device="cpu", dtype=dtype)
+    w = operands["weight"].to(device="cpu", dtype=dtype)
+    b = operands.get("bias")
+    b = b.to(device="cpu", dtype=dtype) if b is not None else None
+    if direction == "fwd":
+        return _conv(problem, x, w, b)
+    gy = operands["grad_output"].to(device="cpu", dtype=dtype)
+    x = x.detach().requires_grad_(direction == "bwd-data")
+    w = w.detach().requires_grad_(direction != "bwd-data")
+    y = _conv(problem, x, w, b)
+    (grad,) = torch.autograd.grad(y, (x if direction == "bwd-data" else w,), gy)
+    return grad
+
+
+def conv_working_dtype(problem: ConvProblem, operands: dict, direction: str = "fwd") -> torch.Tensor:
+    """The same convolution computed by torch's CPU kernels in the operands' own dtype (the
+    reference's CPU path: its ladders fall to stock ``nn.Conv3d`` off-GPU, ``ScaFFold/unet/conv3d.py:1371-1378``)."""
+    x, w, b = operands["input"], operands["weight"], operands.get("bias")
+    if direction == "fwd":
+        return _conv(problem, x, w, b)
+    gy = operands["grad_output"]
+    x = x.detach().requires_grad_(True)
+    w = w.detach().requires_grad_(True)
+    y = _conv(problem, x, w, b)
+    gx, gw = torch.autograd.grad(y, (x, w), gy)
+    return gx if direction == "bwd-data" else gw
+
+
+# ---------------------------------------------------------------------------------------------
+# comparison / tolerance policy
+# ---------------------------------------------------------------------------------------------
+@dataclasses.dataclass(frozen=True)
+class ErrorReport:
+    max_abs: float
+    max_rel: float  # max_abs / rms(expected)
+    rms_rel: float
+    n_diff: int
+    n_total: int
+
+    @property
+    def bitwise(self) -> bool:
+        return self.n_diff == 0
+
+    def __str__(self) -> str:
+        return (f"max_abs={self.max_abs:.3e} max_rel={self.max_rel:.3e} rms_rel={self.rms_rel:.3e} "
+                f"diff={self.n_diff}/{self.n_total}")
+
+
+def compare(actual: torch.Tensor, expected: torch.Tensor) -> ErrorReport:
+    a = actual.detach().to(device="cpu", dtype=torch.float64)
+    e = expected.detach().to(device="cpu", dtype=torch.float64)
+    if a.shape != e.shape:
+        raise ValueError(f"shape mismatch: {tuple(a.shape)} vs {tuple(e.shape)}")
+    if a.numel() == 0:
+        return ErrorReport(0.0, 0.0, 0.0, 0, 0)
+    diff = (a - e).abs()
+    scale = e.pow(2).mean().sqrt().item()
+    scale = scale if scale > 0 else 1.0
+    return ErrorReport(diff.max().item(), diff.max().item() / scale, diff.pow(2).mean().sqrt().item() / scale,
+                       int((a != e).sum().item()), a.numel())
+
+
+def error_bound(problem: ConvProblem, expected: torch.Tensor, direction: str = "fwd", *, roundings: float = 1.0) -> float:
+    """8 * u_fp32 * sqrt(K) * rms  +  2 * roundings * u_dtype * peak."""
+    k = problem.gemm_shape(direction)[2]
+    e = expected.detach().to(torch.float64)
+    rms = e.pow(2).mean().sqrt().item()
+    peak = e.abs().max().item()
+    return 8.0 * unit_roundoff(torch.float32) * math.sqrt(k) * rms + 2.0 * roundings * unit_roundoff(problem.dtype) * peak
+
+
+def assert_close(actual, expected, problem: ConvProblem, direction: str = "fwd", *, incumbent_error: Optional[ErrorReport] = None,
+                 margin: float = 4.0, roundings: float = 1.0) -> ErrorReport:
+    report = compare(actual, expected)
+    bound = error_bound(problem, expected, direction, roundings=roundings)
+    if incumbent_error is not None:
+        bound = max(bound, margin * incumbent_error.max_abs)
+    if not (report.max_abs <= bound):
+        raise AssertionError(f"{problem} [{direction}]: {report}, bound max_abs <= {bound:.3e}")
+    return report
+
+
+def assert_baseline_tolerance(actual, expected, dtype: torch.dtype, what: str = "") -> ErrorReport:
+    """BASELINE.json's bar: fp32 within 1e-5 relative (to the RMS of the expected tensor);
+    bf16/fp16 within 2e-2 relative + 1e-2 absolute, elementwise."""
+    report = compare(actual, expected)
+    a = actual.detach().to(device="cpu", dtype=torch.float64)
+    e = expected.detach().to(device="cpu", dtype=torch.float64)
+    if dtype is torch.float32:
+        ok = report.max_rel <= 1e-5
+    else:
+        ok = bool(((a - e).abs() <= 1e-2 + 2e-2 * e.abs()).all())
+    if not ok:
+        raise AssertionError(f"{what}: outside BASELINE tolerance for {dtype}: {report}")
+    return report
+
+
+# ---------------------------------------------------------------------------------------------
+# GroupNorm references
+# ---------------------------------------------------------------------------------------------
+def group_norm_reference(x, num_groups, weight=None, bias=None, eps=1e-5, relu=False, grad_output=None, *, dtype=torch.float64):
+    """fp64 ``F.group_norm`` (+``F.relu``); with ``grad_output`` also returns (dx, dweight, dbias)."""
+    xd = x.detach().to(device="cpu", dtype=dtype).requires_grad_(grad_output is not None)
+    wd = None if weight is None else weight.detach().to(device="cpu", dtype=dtype).requires_grad_(grad_output is not None)
+    bd = None if bias is None else bias.detach().to(device="cpu", dtype=dtype).requires_grad_(grad_output is not None)
+    # torch's CPU group_norm backward cannot differentiate a bias without a weight; unit weights are the same function
+    w_arg = wd if (wd is not None or bd is None) else torch.ones(xd.shape[1], dtype=dtype)
+    y = F.group_norm(xd, num_groups, w_arg, bd, eps)
+    if relu:
+        y = F.relu(y)
+    if grad_output is None:
+        return y.detach()
+    wanted = [t for t in (xd, wd, bd) if t is not None]
+    grads = list(torch.autograd.grad(y, wanted, grad_output.detach().to(device="cpu", dtype=dtype)))
+    dx = grads.pop(0)
+    dw = grads.pop(0) if wd is not None else None
+    db = grads.pop(0) if bd is not None else None
+    return y.detach(), dx, dw, db
+
+
+def group_norm_manual(x, num_groups, weight=None, bias=None, eps=1e-5, relu=False, grad_output=None):
+    """The same quantities from the textbook formulas, no autograd and no ``F.group_norm``:
+    mean/var per (n, g), y = (x - mu) rstd gamma + beta, and
+    dx = rstd (g gamma - mean_g(g gamma) - xhat mean_g(g gamma xhat)), dgamma = sum g xhat, dbeta = sum g,
+    where g is the upstream gradient gated by the sign of the pre-activation when ``relu``."""
+    xd = x.detach().to(device="cpu", dtype=torch.float64)
+    n, c = xd.shape[:2]
+    sp = xd.shape[2:]
+    cg = c // num_groups
+    xg = xd.reshape(n, num_groups, cg, -1)
+    mu = xg.mean(dim=(2, 3), keepdim=True)
+    var = ((xg - mu) ** 2).mean(dim=(2, 3), keepdim=True)
+    rstd = 1.0 / torch.sqrt(var + eps)
+    xhat = ((xg - mu) * rstd).reshape(n, c, *sp)
+    shape = (1, c) + (1,) * len(sp)
+    gamma = torch.ones(c, dtype=torch.float64) if weight is None else weight.detach().to(device="cpu", dtype=torch.float64)
+    beta = torch.zeros(c, dtype=torch.float64) if bias is None else bias.detach().to(device="cpu", dtype=torch.float64)
+    pre = xhat * gamma.reshape(shape) + beta.reshape(shape)
+    y = torch.where(pre <= 0, torch.zeros_like(pre), pre) if relu else pre
+    stats = (mu.reshape(n, num_groups), rstd.reshape(n, num_groups))
+    if grad_output is None:
+        return y, stats
+    g = grad_output.detach().to(device="cpu", dtype=torch.float64)
+    if relu:
+        g = torch.where(pre <= 0, torch.zeros_like(g), g)
+    gg = (g * gamma.reshape(shape)).reshape(n, num_groups, cg, -1)
+    xh = xhat.reshape(n, num_groups, cg, -1)
+    c1 = gg.mean(dim=(2, 3), keepdim=True)
+    c2 = (gg * xh).mean(dim=(2, 3), keepdim=True)
+    dx = (rstd * (gg - c1 - xh * c2)).reshape(n, c, *sp)
+    red = (0,) + tuple(range(2, 2 + len(sp)))
+    dw = (g * xhat).sum(dim=red)
+    db = g.sum(dim=red)
+    return y, stats, dx, dw, db
+
+
+#: GroupNorm tolerances relative to max|reference| (``tests/test_triton_group_norm.py:57-78``)
+GN_TOLERANCE = {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 3e-3}
+
+
+def gn_rel_error(actual: torch.Tensor, expected: torch.Tensor) -> float:
+    a = actual.detach().to(device="cpu", dtype=torch.float64)
+    e = expected.detach().to(device="cpu", dtype=torch.float64)
+    denom = max(e.abs().max().item(), 1e-30)
+    return (a - e).abs().max().item() / denom
+
+
+# ---------------------------------------------------------------------------------------------
+# train step recipe (config 5)
+# ---------------------------------------------------------------------------------------------
+def train_step_loss(logits: torch.Tensor, labels: torch.Tensor, n_classes: int, eps: float = 1e-6) -> torch.Tensor:
+    """fp32 log-softmax -> mean cross entropy + (1 - mean foreground soft Dice)
+    (``ScaFFold/utils/trainer.py:640-663``, ``ScaFFold/utils/dice_score.py:101-136``; uniform class weights)."""
+    logp = F.log_softmax(logits.float(), dim=1)
+    ce = F.nll_loss(logp, labels)
+    prob = logp.exp()
+    onehot = F.one_hot(labels, n_classes).movedim(-1, 1).to(prob.dtype)
+    dims = (2, 3, 4)
+    inter = (prob * onehot).sum(dims)
+    sets = prob.sum(dims) + onehot.sum(dims)
+    dice = (2 * inter + eps) / (sets + eps)  # (N, C)
+    return ce + (1.0 - dice[:, 1:].mean())
+
+
+def ifs_volume(size: Sequence[int], *, n_fractals: int = 3, n_classes: int = 10, n_maps: int = 4, iterations: int = 200_000,
+               seed: int = 5000):
+    """Config 5's synthetic sample: voxelised points of random 3-D iterated function systems
+    (``n_maps`` affine maps each, contraction factors U(0.3, 0.7)); returns (occupancy float32
+    (1, 1, D, H, W), labels int64 (1, D, H, W)) with label = class id in 1..n_classes, 0 = background."""
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    d, h, w = (int(v) for v in size)
+    labels = np.zeros((d, h, w), dtype=np.int64)
+    for _ in range(n_fractals):
+        cls = int(rng.integers(1, n_classes + 1))
+        mats, offs = [], []
+        for _ in range(n_maps):
+            q, _r = np.linalg.qr(rng.standard_normal((3, 3)))
+            mats.append(q * rng.uniform(0.3, 0.7))
+            offs.append(rng.uniform(-1.0, 1.0, size=3))
+        mats, offs = np.stack(mats), np.stack(offs)
+        choice = rng.integers(0, n_maps, size=iterations)
+        pts = np.empty((iterations, 3))
+        p = np.zeros(3)
+        for i in range(iterations):
+            p = mats[choice[i]] @ p + offs[choice[i]]
+            pts[i] = p
+        pts = pts[100:]
+        lo, hi = pts.min(0), pts.max(0)
+        scale = (np.array([d, h, w]) - 1) / np.maximum(hi - lo, 1e-9).max()
+        idx = np.clip(np.floor((pts - lo) * scale).astype(np.int64), 0, [d - 1, h - 1, w - 1])
+        labels[idx[:, 0], idx[:, 1], idx[:, 2]] = cls
+    lab = torch.from_numpy(labels)[None]
+    occ = (lab > 0).to(torch.float32)[:, None]
+    return occ, lab

@@ -1,0 +1,172 @@
+"""ctypes binding of ``libscaffold_hip.so`` (the C ABI declared in ``include/scaffold_hip.h``).
+
+The library is the product: there is no Python or CPU fallback behind it.  If the shared
+object has not been built, :func:`lib` raises ``ScaffoldLibraryError`` with the build command,
+and every op that needs it fails with that error.
+
+Error codes map onto the exception classes the reference's entry points raise
+(``triton_conv3d/gather_gemm.py:1228-1232``, ``ScaFFold/unet/triton_group_norm.py:253-277``):
+``SFH_ERR_UNSUPPORTED`` -> ``NotImplementedError``, ``SFH_ERR_INVALID`` / ``SFH_ERR_WORKSPACE``
+-> ``ValueError``, ``SFH_ERR_LAUNCH`` -> :class:`ScaffoldKernelError`.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint32, c_void_p
+
+import torch
+
+__all__ = [
+    "ScaffoldLibraryError",
+    "ScaffoldKernelError",
+    "lib",
+    "lib_path",
+    "check",
+    "ConvDesc",
+    "ConvTDesc",
+    "GroupNormDesc",
+    "dtype_code",
+    "SUPPORTED_DTYPES",
+    "EXPORTED_SYMBOLS",
+]
+
+SFH_OK, SFH_ERR_INVALID, SFH_ERR_UNSUPPORTED, SFH_ERR_WORKSPACE, SFH_ERR_LAUNCH = range(5)
+SFH_FLAG_FORCE_GENERIC = 1
+
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+SUPPORTED_DTYPES = tuple(_DTYPE_CODE)
+
+
+class ScaffoldLibraryError(RuntimeError):
+    """libscaffold_hip.so is missing or does not export the declared ABI."""
+
+
+class ScaffoldKernelError(RuntimeError):
+    """The HIP runtime refused a kernel launch (distinct from a contract violation)."""
+
+
+class ConvDesc(ctypes.Structure):
+    _fields_ = [(k, c_int32) for k in (
+        "n", "cin", "in_d", "in_h", "in_w", "cout", "kd", "kh", "kw",
+        "sd", "sh", "sw", "pd", "ph", "pw", "dd", "dh", "dw")]
+
+
+class ConvTDesc(ctypes.Structure):
+    _fields_ = [(k, c_int32) for k in ("n", "cin", "in_d", "in_h", "in_w", "cout", "kd", "kh", "kw")]
+
+
+class GroupNormDesc(ctypes.Structure):
+    _fields_ = [("n", c_int32), ("c", c_int32), ("groups", c_int32), ("relu", c_int32),
+                ("spatial", c_int64), ("eps", c_float)]
+
+
+_I64x5 = c_int64 * 5
+
+# name -> (restype, argtypes); every symbol include/scaffold_hip.h declares.
+_SIGNATURES = {
+    "sfh_version": (c_int, []),
+    "sfh_last_error": (c_char_p, []),
+    "sfh_device_info": (c_int, [c_char_p, c_size_t, POINTER(c_int32), POINTER(c_int32)]),
+    "sfh_conv3d_out_shape": (c_int, [POINTER(ConvDesc), POINTER(c_int32)]),
+    "sfh_conv3d_uses_mfma": (c_int, [POINTER(ConvDesc), c_int, c_int]),
+    "sfh_conv3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_fwd": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
+                               c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_dgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_dgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
+                                 c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_wgrad_splits": (c_int, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_wgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_wgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,
+                                 c_void_p]),
+    "sfh_convT3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvTDesc), c_int]),
+    "sfh_convT3d_fwd": (c_int, [POINTER(ConvTDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
+                                c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_groupnorm_fwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
+    "sfh_groupnorm_fwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_groupnorm_bwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
+    "sfh_groupnorm_bwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_stream_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lock = threading.Lock()
+_lib = None
+
+
+def lib_path() -> str:
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "libscaffold_hip.so")
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library; raises :class:`ScaffoldLibraryError` if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = lib_path()
+        if not os.path.exists(path):
+            raise ScaffoldLibraryError(
+                f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C scaffold_amd/csrc -j8` (needs hipcc, targets gfx950). There is no fallback path."
+            )
+        try:
+            handle = ctypes.CDLL(path)
+        except OSError as exc:  # missing ROCm runtime, wrong arch, ...
+            raise ScaffoldLibraryError(f"cannot load {path}: {exc}") from exc
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            try:
+                fn = getattr(handle, name)
+            except AttributeError as exc:
+                raise ScaffoldLibraryError(f"{path} does not export {name}; rebuild it") from exc
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+        return _lib
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise NotImplementedError(f"unsupported dtype {dtype}; supported: {SUPPORTED_DTYPES}") from None
+
+
+def check(rc: int, what: str) -> None:
+    """Turn a non-zero return code into the matching exception."""
+    if rc == SFH_OK:
+        return
+    msg = lib().sfh_last_error()
+    msg = msg.decode("utf-8", "replace") if msg else "unknown error"
+    text = f"{what}: {msg}"
+    if rc == SFH_ERR_UNSUPPORTED:
+        raise NotImplementedError(text)
+    if rc in (SFH_ERR_INVALID, SFH_ERR_WORKSPACE):
+        raise ValueError(text)
+    raise ScaffoldKernelError(text)
+
+
+def strides5(t: torch.Tensor):
+    return _I64x5(*[int(s) for s in t.stride()])
+
+
+def stream_ptr(device: torch.device) -> int:
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def workspace(nbytes: int, device: torch.device):
+    """A scratch buffer from torch's caching allocator (None when nothing is needed)."""
+    if nbytes <= 0:
+        return None
+    return torch.empty(int(nbytes), dtype=torch.uint8, device=device)

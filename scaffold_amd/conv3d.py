@@ -1,0 +1,483 @@
+"""Channels-last conv3d forward / data-gradient / weight-gradient on the HIP library.
+
+Same call signatures, argument meaning and error behaviour as the reference's kernel package:
+
+====================================  ==========================================================
+this module                           reference (LBANN/ScaFFold)
+====================================  ==========================================================
+``conv3d_forward``                    ``triton_conv3d/gather_gemm.py:1187``
+``conv3d_backward_data``              ``triton_conv3d/bwd_data.py:275``
+``conv3d_backward_weight``            ``triton_conv3d/reduce_gemm.py:1177``
+``is_supported`` / ``_all``           ``triton_conv3d/gather_gemm.py:945,1036``
+``is_supported_bwd_data``             ``triton_conv3d/bwd_data.py:201``
+``is_supported_bwd_weight``           ``triton_conv3d/reduce_gemm.py:1112``
+``grad_weight_empty``                 ``triton_conv3d/reduce_gemm.py:1023``
+``bwd_data_padding``                  ``triton_conv3d/bwd_data.py:84``
+====================================  ==========================================================
+
+Tensors are PyTorch NCDHW-shaped; memory is ``channels_last_3d`` (NDHWC).  Inputs in another
+layout are converted, never misread.  Outputs are allocated once, directly in the layout the
+kernels store.  ``out=`` / ``workspace=`` are validated, not trusted.  A call the library does
+not serve raises ``NotImplementedError``; a contract violation raises ``ValueError``; the gates
+never raise.  There is no fallback to another backend: a CPU tensor is simply not served.
+
+``config=`` and ``weight_rsck=`` are accepted for signature compatibility.  Tile selection here
+is a pure function of shape inside the library, so ``config`` must be ``None``; ``weight_rsck``
+(the forward's ``(kd, kh, kw, Cin, Cout)`` weight copy) is validated and then read through its
+strides like any other weight layout.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import ConvDesc, SUPPORTED_DTYPES
+
+__all__ = [
+    "conv3d_forward",
+    "conv3d_backward_data",
+    "conv3d_backward_weight",
+    "is_supported",
+    "is_supported_all",
+    "is_supported_bwd_data",
+    "is_supported_bwd_weight",
+    "bwd_data_padding",
+    "grad_weight_empty",
+    "workspace_elements",
+    "split_count",
+    "uses_mfma",
+    "output_shape",
+]
+
+_CL3D = torch.channels_last_3d
+
+
+def _triple(value, name: str) -> tuple[int, int, int]:
+    """``int`` or length-3 sequence of ints -> 3-tuple; anything else is a ValueError/TypeError."""
+    if isinstance(value, bool):
+        raise TypeError(f"{name} must be an int or three ints, got {value!r}")
+    if isinstance(value, int):
+        return (value, value, value)
+    seq = tuple(value)  # TypeError for non-iterables such as None or 1.5
+    if len(seq) != 3 or not all(isinstance(v, int) and not isinstance(v, bool) for v in seq):
+        raise ValueError(f"{name} must be an int or three ints, got {value!r}")
+    return seq  # type: ignore[return-value]
+
+
+def output_shape(in_shape: Sequence[int], weight_shape: Sequence[int], stride, padding, dilation) -> tuple[int, ...]:
+    """NCDHW output shape of a conv3d, ``floor((in + 2p - dil(k-1) - 1)/s) + 1`` per axis."""
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    n, cout = int(in_shape[0]), int(weight_shape[0])
+    sp = tuple(
+        (int(in_shape[2 + i]) + 2 * p[i] - d[i] * (int(weight_shape[2 + i]) - 1) - 1) // s[i] + 1 for i in range(3)
+    )
+    return (n, cout) + sp
+
+
+def bwd_data_padding(padding, dilation, kernel) -> tuple[int, int, int]:
+    """Padding of the gather that computes the data gradient: ``dil*(k-1) - p`` per axis."""
+    p, d, k = _triple(padding, "padding"), _triple(dilation, "dilation"), _triple(kernel, "kernel")
+    return (d[0] * (k[0] - 1) - p[0], d[1] * (k[1] - 1) - p[1], d[2] * (k[2] - 1) - p[2])
+
+
+def _desc(n, cin, in_sp, cout, k, s, p, d) -> ConvDesc:
+    return ConvDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2], s[0], s[1], s[2],
+                    p[0], p[1], p[2], d[0], d[1], d[2])
+
+
+# ---------------------------------------------------------------------------------------------
+# gates
+# ---------------------------------------------------------------------------------------------
+def is_supported(x, w, bias=None, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
+    """Whether :func:`conv3d_forward` serves this call.  Total: never raises."""
+    try:
+        if groups != 1:
+            return False
+        if not isinstance(x, torch.Tensor) or not isinstance(w, torch.Tensor):
+            return False
+        if x.dim() != 5 or w.dim() != 5:
+            return False
+        if x.dtype != w.dtype or x.dtype not in SUPPORTED_DTYPES:
+            return False
+        if not x.is_cuda or not w.is_cuda or x.device != w.device:
+            return False
+        if bias is not None:
+            if not isinstance(bias, torch.Tensor) or bias.dim() != 1 or bias.shape[0] != w.shape[0]:
+                return False
+            if bias.dtype != x.dtype or bias.device != x.device or bias.stride(0) != 1:
+                return False
+        if x.shape[1] != w.shape[1]:
+            return False
+        s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+        k = tuple(int(v) for v in w.shape[2:])
+        if min(s + d) < 1 or min(p) < 0:
+            return False
+        if min(int(v) for v in x.shape[2:]) < 1 or min(k) < 1:
+            return False
+        if w.shape[0] < 1 or w.shape[1] < 1:
+            return False
+        for i in range(3):
+            if int(x.shape[2 + i]) + 2 * p[i] < d[i] * (k[i] - 1) + 1:
+                return False
+        return True
+    except (TypeError, ValueError, AttributeError):
+        return False
+
+
+def is_supported_bwd_data(grad_output, weight, input_shape, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
+    """Whether :func:`conv3d_backward_data` serves this call: stride 1 and ``p <= dil*(k-1)`` only."""
+    try:
+        if groups != 1:
+            return False
+        if not isinstance(grad_output, torch.Tensor) or not isinstance(weight, torch.Tensor):
+            return False
+        shape = tuple(int(v) for v in input_shape)
+        if grad_output.dim() != 5 or weight.dim() != 5 or len(shape) != 5:
+            return False
+        if grad_output.dtype != weight.dtype or grad_output.dtype not in SUPPORTED_DTYPES:
+            return False
+        if not grad_output.is_cuda or not weight.is_cuda or grad_output.device != weight.device:
+            return False
+        s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+        k = tuple(int(v) for v in weight.shape[2:])
+        if min(d) < 1 or min(p) < 0 or min(k) < 1 or s != (1, 1, 1):
+            return False
+        if any(p[i] > d[i] * (k[i] - 1) for i in range(3)):
+            return False
+        n, cin, *in_sp = shape
+        if weight.shape[0] != grad_output.shape[1] or weight.shape[1] != cin or grad_output.shape[0] != n:
+            return False
+        if n < 1 or min(in_sp) < 1:
+            return False
+        for i in range(3):
+            if int(grad_output.shape[2 + i]) != in_sp[i] + 2 * p[i] - d[i] * (k[i] - 1):
+                return False
+        return True
+    except (TypeError, ValueError, AttributeError):
+        return False
+
+
+def is_supported_bwd_weight(input, weight_shape, grad_output, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
+    """Whether :func:`conv3d_backward_weight` serves this call (any stride)."""
+    try:
+        if groups != 1:
+            return False
+        if not isinstance(input, torch.Tensor) or not isinstance(grad_output, torch.Tensor):
+            return False
+        ws = tuple(int(v) for v in weight_shape)
+        if input.dim() != 5 or grad_output.dim() != 5 or len(ws) != 5:
+            return False
+        if input.dtype != grad_output.dtype or input.dtype not in SUPPORTED_DTYPES:
+            return False
+        if not input.is_cuda or not grad_output.is_cuda or input.device != grad_output.device:
+            return False
+        s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+        cout, cin, *k = ws
+        if min(s + d + tuple(k)) < 1 or min(p) < 0 or cout < 1 or cin < 1:
+            return False
+        n, in_c, *in_sp = (int(v) for v in input.shape)
+        if in_c != cin or grad_output.shape[1] != cout or grad_output.shape[0] != n:
+            return False
+        for i in range(3):
+            eff = d[i] * (k[i] - 1) + 1
+            if in_sp[i] + 2 * p[i] < eff:
+                return False
+            if int(grad_output.shape[2 + i]) != (in_sp[i] + 2 * p[i] - eff) // s[i] + 1:
+                return False
+        return True
+    except (TypeError, ValueError, AttributeError):
+        return False
+
+
+def is_supported_all(x, w, bias=None, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
+    """Whether all three directions of this convolution are served (the gate for a caller
+    that will differentiate): the forward accepts strides the data gradient refuses."""
+    if not is_supported(x, w, bias, stride, padding, dilation, groups):
+        return False
+    try:
+        gshape = output_shape(x.shape, w.shape, stride, padding, dilation)
+        grad = x.new_empty((1, 1, 1, 1, 1)).expand(gshape)  # metadata-only stand-in
+        return is_supported_bwd_data(grad, w, tuple(x.shape), stride, padding, dilation, groups) and \
+            is_supported_bwd_weight(x, tuple(w.shape), grad, stride, padding, dilation, groups)
+    except (TypeError, ValueError, AttributeError, RuntimeError):
+        return False
+
+
+# ---------------------------------------------------------------------------------------------
+# helpers
+# ---------------------------------------------------------------------------------------------
+def _check_out(y: torch.Tensor, shape: tuple[int, ...], like: torch.Tensor) -> None:
+    if tuple(y.shape) != tuple(shape):
+        raise ValueError(f"out= must have shape {tuple(shape)}, got {tuple(y.shape)}")
+    if y.dtype != like.dtype:
+        raise ValueError(f"out= must have dtype {like.dtype}, got {y.dtype}")
+    if y.device != like.device:
+        raise ValueError(f"out= must be on {like.device}, got {y.device}")
+    if not y.is_contiguous(memory_format=_CL3D):
+        raise ValueError(f"out= must be channels_last_3d (channel stride 1); got strides {tuple(y.stride())}")
+
+
+def _check_weight_rsck(wr: torch.Tensor, shape: tuple[int, ...], like: torch.Tensor) -> None:
+    if tuple(wr.shape) != tuple(shape):
+        raise ValueError(f"weight_rsck= must have shape {tuple(shape)} (kd, kh, kw, Cin, Cout), got {tuple(wr.shape)}")
+    if wr.dtype != like.dtype:
+        raise ValueError(f"weight_rsck= must have dtype {like.dtype}, got {wr.dtype}")
+    if wr.device != like.device:
+        raise ValueError(f"weight_rsck= must be on {like.device}, got {wr.device}")
+    if not wr.is_contiguous():
+        raise ValueError(f"weight_rsck= must be contiguous; got strides {tuple(wr.stride())}")
+
+
+def _no_config(config) -> None:
+    if config is not None:
+        raise ValueError("config= is not supported: tile selection is a pure function of shape inside the HIP library")
+
+
+def _flags(force_generic: bool) -> int:
+    return _lib.SFH_FLAG_FORCE_GENERIC if force_generic else 0
+
+
+def uses_mfma(in_shape, weight_shape, stride, padding, dilation, dtype, direction: str = "fwd") -> bool:
+    """Whether the MFMA implicit-GEMM kernels (rather than the direct ones) serve a problem."""
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    n, cin, *in_sp = (int(v) for v in in_shape)
+    cout, _, *k = (int(v) for v in weight_shape)
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    code = {"fwd": 0, "bwd-data": 1, "bwd-weight": 2}[direction]
+    return bool(_lib.lib().sfh_conv3d_uses_mfma(ctypes.byref(desc), _lib.dtype_code(dtype), code))
+
+
+def split_count(in_shape, weight_shape, stride, padding, dilation, dtype) -> int:
+    """Number of fp32 partial slices the weight gradient reduces (1 = no workspace)."""
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    n, cin, *in_sp = (int(v) for v in in_shape)
+    cout, _, *k = (int(v) for v in weight_shape)
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    return int(_lib.lib().sfh_conv3d_wgrad_splits(ctypes.byref(desc), _lib.dtype_code(dtype)))
+
+
+def workspace_elements(splits: int, cout: int, cin: int, kernel: Sequence[int]) -> int:
+    """fp32 elements :func:`conv3d_backward_weight` needs for ``splits`` partial slices."""
+    k = _triple(kernel, "kernel")
+    return int(splits) * int(cout) * int(cin) * k[0] * k[1] * k[2]
+
+
+def grad_weight_empty(cout: int, cin: int, kernel: Sequence[int], *, dtype, device) -> torch.Tensor:
+    """An empty ``(Cout, Cin, kd, kh, kw)`` gradient in the layout the kernel writes:
+    ``[Cout][kd][kh][kw][Cin]`` in memory, i.e. ``channels_last_3d``."""
+    k = _triple(kernel, "kernel")
+    return torch.empty((cout, cin, *k), dtype=dtype, device=device, memory_format=_CL3D)
+
+
+# ---------------------------------------------------------------------------------------------
+# forward
+# ---------------------------------------------------------------------------------------------
+def conv3d_forward(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    stride=1,
+    padding=0,
+    dilation=1,
+    groups: int = 1,
+    *,
+    config=None,
+    weight_rsck: Optional[torch.Tensor] = None,
+    weight_flip: bool = False,
+    out: Optional[torch.Tensor] = None,
+    force_generic: bool = False,
+) -> torch.Tensor:
+    """Forward 3-D convolution; input and output are ``channels_last_3d``.
+
+    The weight is read where it lies (its strides are handed to the library), so a
+    ``channels_last_3d`` parameter, PyTorch's default layout and an RSCK copy all work without
+    a host-side transform and give bitwise identical results.  ``weight_flip`` consumes the
+    taps mirrored in all three axes (the data gradient's view of the weight).
+    """
+    if not is_supported(x, w, bias, stride, padding, dilation, groups):
+        raise NotImplementedError(
+            f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)} "
+            f"w={tuple(getattr(w, 'shape', ()))} stride={stride} padding={padding} dilation={dilation} groups={groups}"
+        )
+    _no_config(config)
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    k = tuple(int(v) for v in w.shape[2:])
+    x = x.contiguous(memory_format=_CL3D)
+    n, cin, *in_sp = (int(v) for v in x.shape)
+    cout = int(w.shape[0])
+    y_shape = output_shape(x.shape, w.shape, s, p, d)
+    if out is None:
+        y = torch.empty(y_shape, device=x.device, dtype=x.dtype, memory_format=_CL3D)
+    else:
+        y = out
+        _check_out(y, y_shape, x)
+    if weight_rsck is not None:
+        _check_weight_rsck(weight_rsck, (*k, cin, cout), x)
+        w_eff = weight_rsck.permute(4, 3, 0, 1, 2)  # (Cout, Cin, kd, kh, kw) view of the RSCK buffer
+    else:
+        w_eff = w
+    if weight_flip:
+        w_eff = w_eff.flip(2, 3, 4)  # small copy; the data-gradient entry point flips inside the library instead
+    if n == 0:
+        return y
+    L = _lib.lib()
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    code = _lib.dtype_code(x.dtype)
+    with torch.cuda.device(x.device):
+        ws = _lib.workspace(L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
+        rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(bias),
+                              _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
+                              _lib.stream_ptr(x.device))
+    _lib.check(rc, "conv3d_forward")
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# data gradient
+# ---------------------------------------------------------------------------------------------
+def conv3d_backward_data(
+    grad_output: torch.Tensor,
+    weight: torch.Tensor,
+    input_shape: Sequence[int],
+    stride=1,
+    padding=0,
+    dilation=1,
+    groups: int = 1,
+    *,
+    config=None,
+    weight_rsck: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    force_generic: bool = False,
+) -> torch.Tensor:
+    """Gradient of a conv3d with respect to its input (stride 1 only).
+
+    Computed as a gather over ``grad_output`` with the channel roles of the weight swapped, the
+    taps mirrored and padding ``dil*(k-1) - p``; the swap and the mirror happen while the library
+    repacks the weight, so no transformed copy of the weight is made here.
+    """
+    if not is_supported_bwd_data(grad_output, weight, input_shape, stride, padding, dilation, groups):
+        raise NotImplementedError(
+            f"unsupported: grad_output={tuple(getattr(grad_output, 'shape', ()))}/{getattr(grad_output, 'dtype', None)} "
+            f"w={tuple(getattr(weight, 'shape', ()))} input_shape={tuple(input_shape)} stride={stride} "
+            f"padding={padding} dilation={dilation} groups={groups}"
+        )
+    _no_config(config)
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    k = tuple(int(v) for v in weight.shape[2:])
+    n, cin, *in_sp = (int(v) for v in input_shape)
+    cout = int(weight.shape[0])
+    gy = grad_output.contiguous(memory_format=_CL3D)
+    gx_shape = (n, cin, *in_sp)
+    if out is None:
+        gx = torch.empty(gx_shape, device=gy.device, dtype=gy.dtype, memory_format=_CL3D)
+    else:
+        gx = out
+        _check_out(gx, gx_shape, gy)
+    if weight_rsck is not None:
+        _check_weight_rsck(weight_rsck, (*k, cin, cout), gy)
+        w_eff = weight_rsck.permute(4, 3, 0, 1, 2)
+    else:
+        w_eff = weight
+    L = _lib.lib()
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    code = _lib.dtype_code(gy.dtype)
+    with torch.cuda.device(gy.device):
+        ws = _lib.workspace(L.sfh_conv3d_dgrad_workspace_bytes(ctypes.byref(desc), code), gy.device)
+        rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(gx),
+                                _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
+                                _lib.stream_ptr(gy.device))
+    _lib.check(rc, "conv3d_backward_data")
+    return gx
+
+
+# ---------------------------------------------------------------------------------------------
+# weight gradient
+# ---------------------------------------------------------------------------------------------
+def _validate_gw_out(gw: torch.Tensor, cout: int, cin: int, k, dtype, device) -> Optional[str]:
+    want_shape = (cout, cin, *k)
+    if tuple(gw.shape) != want_shape:
+        return f"shape must be {want_shape} (Cout x Cin x kernel); got {tuple(gw.shape)}"
+    if gw.device != device:
+        return f"device must be {device}; got {gw.device}"
+    if gw.dtype != dtype:
+        return f"dtype must match the operands' {dtype}; got {gw.dtype}"
+    taps = k[0] * k[1] * k[2]
+    want = (taps * cin, 1, k[1] * k[2] * cin, k[2] * cin, cin)
+    got = tuple(gw.stride())
+    # A size-1 dimension's stride is unobservable; compare only the ones that matter.
+    if not all(g == w for g, w, extent in zip(got, want, want_shape) if extent > 1):
+        return f"must have channels_last_3d strides ([Cout][tap][Cin] in memory); want {want}, got {got}"
+    return None
+
+
+def conv3d_backward_weight(
+    input: torch.Tensor,
+    weight_shape: Sequence[int],
+    grad_output: torch.Tensor,
+    stride=1,
+    padding=0,
+    dilation=1,
+    groups: int = 1,
+    *,
+    deterministic: bool = True,
+    config=None,
+    workspace: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    force_generic: bool = False,
+) -> torch.Tensor:
+    """Gradient of a conv3d with respect to its weight, returned ``channels_last_3d``.
+
+    Split-K over the output voxels with fp32 partial slices at fixed workspace slots and an
+    ordered reduction; there is no atomic variant, so ``deterministic=False`` is refused rather
+    than silently served by the deterministic path.
+    """
+    if not is_supported_bwd_weight(input, weight_shape, grad_output, stride, padding, dilation, groups):
+        raise NotImplementedError(
+            f"unsupported: input={tuple(getattr(input, 'shape', ()))}/{getattr(input, 'dtype', None)} "
+            f"weight_shape={tuple(weight_shape)} grad_output={tuple(getattr(grad_output, 'shape', ()))} "
+            f"stride={stride} padding={padding} dilation={dilation} groups={groups}"
+        )
+    _no_config(config)
+    if not deterministic:
+        raise NotImplementedError("deterministic=False: this library has no atomic weight-gradient path")
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    cout, cin, *k = (int(v) for v in weight_shape)
+    x = input.contiguous(memory_format=_CL3D)
+    gy = grad_output.contiguous(memory_format=_CL3D)
+    n, _, *in_sp = (int(v) for v in x.shape)
+    if out is None:
+        gw = grad_weight_empty(cout, cin, k, dtype=x.dtype, device=x.device)
+    else:
+        gw = out
+        why = _validate_gw_out(gw, cout, cin, tuple(k), x.dtype, x.device)
+        if why is not None:
+            raise ValueError(f"out= is not usable for this problem: {why}")
+    L = _lib.lib()
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    code = _lib.dtype_code(x.dtype)
+    if n == 0:
+        return gw.zero_()
+    with torch.cuda.device(x.device):
+        need = 0 if force_generic else int(L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(desc), code))
+        if workspace is None:
+            ws = _lib.workspace(need, x.device)
+            ws_bytes = 0 if ws is None else ws.numel()
+        else:
+            have = workspace.numel() * workspace.element_size()
+            if workspace.dtype is not torch.float32 or have < need or workspace.device != x.device \
+                    or not workspace.is_contiguous():
+                splits = int(L.sfh_conv3d_wgrad_splits(ctypes.byref(desc), code))
+                raise ValueError(
+                    f"workspace must be a contiguous float32 tensor on {x.device} of at least {need // 4} elements "
+                    f"({need / 2**20:.1f} MiB) -- {splits} splits x {cout} Cout x {k[0] * k[1] * k[2]} taps x {cin} Cin; "
+                    f"got {workspace.numel()} of {workspace.dtype}"
+                )
+            ws, ws_bytes = workspace, have
+        rc = L.sfh_conv3d_wgrad(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(ws), ws_bytes,
+                                _flags(force_generic), _lib.stream_ptr(x.device))
+    _lib.check(rc, "conv3d_backward_weight")
+    return gw

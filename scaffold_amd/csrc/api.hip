@@ -1,0 +1,286 @@
+// extern "C" entry points of libscaffold_hip.so: argument checking, kernel selection (a pure
+// function of descriptor and dtype), workspace carving. No allocation, no synchronisation.
+#include <string.h>
+
+#include "common.hpp"
+#include "conv_direct.hpp"
+#include "conv_mfma.hpp"
+#include "wgrad_mfma.hpp"
+
+namespace sfh {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return SFH_OK;
+  return fail(SFH_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString(e));
+}
+
+namespace {
+
+int check_conv(const sfh_conv3d_desc* p, int dtype, int32_t out[3]) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "conv3d: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "conv3d: bad dtype %d", dtype);
+  if (p->n < 0 || p->cin < 1 || p->cout < 1 || p->in_d < 1 || p->in_h < 1 || p->in_w < 1)
+    return fail(SFH_ERR_INVALID, "conv3d: bad extents n=%d cin=%d cout=%d in=%dx%dx%d", p->n, p->cin, p->cout, p->in_d, p->in_h,
+                p->in_w);
+  if (p->kd < 1 || p->kh < 1 || p->kw < 1 || p->sd < 1 || p->sh < 1 || p->sw < 1 || p->dd < 1 || p->dh < 1 || p->dw < 1 ||
+      p->pd < 0 || p->ph < 0 || p->pw < 0)
+    return fail(SFH_ERR_INVALID, "conv3d: kernel/stride/dilation must be >= 1 and padding >= 0");
+  const int in[3] = {p->in_d, p->in_h, p->in_w}, k[3] = {p->kd, p->kh, p->kw}, s[3] = {p->sd, p->sh, p->sw},
+            pad[3] = {p->pd, p->ph, p->pw}, dil[3] = {p->dd, p->dh, p->dw};
+  for (int i = 0; i < 3; ++i) {
+    const int64_t eff = (int64_t)dil[i] * (k[i] - 1) + 1;
+    if ((int64_t)in[i] + 2 * pad[i] < eff) return fail(SFH_ERR_INVALID, "conv3d: kernel wider than the padded input on axis %d", i);
+    out[i] = (int32_t)(((int64_t)in[i] + 2 * pad[i] - eff) / s[i] + 1);
+  }
+  return SFH_OK;
+}
+
+bool is_unit(const sfh_conv3d_desc& p) {
+  return p.sd == 1 && p.sh == 1 && p.sw == 1 && p.dd == 1 && p.dh == 1 && p.dw == 1;
+}
+
+MfmaConvArgs fwd_mfma_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  MfmaConvArgs a{};
+  a.n = p.n; a.cred = p.cin; a.id = p.in_d; a.ih = p.in_h; a.iw = p.in_w;
+  a.cout = p.cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
+  a.kd = p.kd; a.kh = p.kh; a.kw = p.kw; a.pd = p.pd; a.ph = p.ph; a.pw = p.pw;
+  return a;
+}
+
+// The data gradient as a gather over gy: reduction channels = Cout, produced = Cin,
+// padding dil*(k-1) - p, output extents = the forward's input extents.
+MfmaConvArgs dgrad_mfma_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  MfmaConvArgs a{};
+  a.n = p.n; a.cred = p.cout; a.id = out[0]; a.ih = out[1]; a.iw = out[2];
+  a.cout = p.cin; a.od = p.in_d; a.oh = p.in_h; a.ow = p.in_w;
+  a.kd = p.kd; a.kh = p.kh; a.kw = p.kw;
+  a.pd = (p.kd - 1) - p.pd; a.ph = (p.kh - 1) - p.ph; a.pw = (p.kw - 1) - p.pw;
+  return a;
+}
+
+bool fwd_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return is_unit(p) && mfma_conv_supported(fwd_mfma_args(p, out), dtype);
+}
+
+int check_dgrad(const sfh_conv3d_desc& p) {
+  if (p.sd != 1 || p.sh != 1 || p.sw != 1)
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad: served at stride 1 only (got %d,%d,%d)", p.sd, p.sh, p.sw);
+  if (p.pd > p.dd * (p.kd - 1) || p.ph > p.dh * (p.kh - 1) || p.pw > p.dw * (p.kw - 1))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad: padding must not exceed dilation*(k-1)");
+  if (p.n < 1) return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad: empty batch");
+  return SFH_OK;
+}
+
+bool dgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return is_unit(p) && mfma_conv_supported(dgrad_mfma_args(p, out), dtype);
+}
+
+WgradArgs wgrad_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  WgradArgs a{};
+  a.n = p.n; a.cin = p.cin; a.id = p.in_d; a.ih = p.in_h; a.iw = p.in_w;
+  a.cout = p.cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
+  a.pd = p.pd; a.ph = p.ph; a.pw = p.pw;
+  return a;
+}
+
+bool wgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return is_unit(p) && p.kd == 3 && p.kh == 3 && p.kw == 3 && p.n >= 1 && mfma_wgrad_supported(wgrad_args(p, out), dtype);
+}
+
+__global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < n; i += stride) dst[i] = src[i];
+}
+
+}  // namespace
+}  // namespace sfh
+
+using namespace sfh;
+
+extern "C" int sfh_version(void) { return 100; }
+
+extern "C" const char* sfh_last_error(void) { return g_error; }
+
+extern "C" int sfh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* lds_bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(SFH_ERR_LAUNCH, "no HIP device");
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return fail(SFH_ERR_LAUNCH, "hipGetDeviceProperties failed");
+  if (name != nullptr && name_len > 0) {
+    strncpy(name, prop.gcnArchName, name_len - 1);
+    name[name_len - 1] = 0;
+  }
+  if (compute_units != nullptr) *compute_units = prop.multiProcessorCount;
+  if (lds_bytes != nullptr) *lds_bytes = (int32_t)prop.sharedMemPerBlock;
+  return SFH_OK;
+}
+
+extern "C" int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]) {
+  if (out_dhw == nullptr) return fail(SFH_ERR_INVALID, "conv3d: null output");
+  return check_conv(p, SFH_FP32, out_dhw);
+}
+
+extern "C" int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (direction == 0) return fwd_uses_mfma(*p, dtype, out) ? 1 : 0;
+  if (direction == 1) return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)) ? 1 : 0;
+  return wgrad_uses_mfma(*p, dtype, out) ? 1 : 0;
+}
+
+// ---- forward ---------------------------------------------------------------------------
+extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (!fwd_uses_mfma(*p, dtype, out)) return 0;
+  return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out));
+}
+
+extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                              const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (x == nullptr || w == nullptr || y == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d fwd: null tensor");
+  if (p->n == 0) return SFH_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_mfma(*p, dtype, out)) {
+    const MfmaConvArgs a = fwd_mfma_args(*p, out);
+    const size_t need = mfma_conv_packed_weight_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
+      return rc;
+    return mfma_conv_gather(a, dtype, x, workspace, bias, y, st);
+  }
+  DirectConvArgs a{};
+  a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;
+  a.cout = p->cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
+  a.kd = p->kd; a.kh = p->kh; a.kw = p->kw; a.sd = p->sd; a.sh = p->sh; a.sw = p->sw;
+  a.pd = p->pd; a.ph = p->ph; a.pw = p->pw; a.dd = p->dd; a.dh = p->dh; a.dw = p->dw;
+  a.flip = 0;
+  a.ws_co = w_stride[0]; a.ws_ci = w_stride[1]; a.ws_kd = w_stride[2]; a.ws_kh = w_stride[3]; a.ws_kw = w_stride[4];
+  return direct_conv_gather(a, dtype, x, w, bias, y, st);
+}
+
+// ---- data gradient ---------------------------------------------------------------------
+extern "C" size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (check_dgrad(*p) != SFH_OK || !dgrad_uses_mfma(*p, dtype, out)) return 0;
+  return mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out));
+}
+
+extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
+                                void* gx, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (int rc = check_dgrad(*p)) return rc;
+  if (gy == nullptr || w == nullptr || gx == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d dgrad: null tensor");
+  hipStream_t st = (hipStream_t)stream;
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && dgrad_uses_mfma(*p, dtype, out)) {
+    const MfmaConvArgs a = dgrad_mfma_args(*p, out);
+    const size_t need = mfma_conv_packed_weight_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    // produced channel = Cin (stride w_stride[1]), reduction channel = Cout (w_stride[0]), taps flipped
+    if (int rc = mfma_pack_weight(a, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, workspace, st))
+      return rc;
+    return mfma_conv_gather(a, dtype, gy, workspace, nullptr, gx, st);
+  }
+  DirectConvArgs a{};
+  a.n = p->n; a.cin = p->cout; a.id = out[0]; a.ih = out[1]; a.iw = out[2];
+  a.cout = p->cin; a.od = p->in_d; a.oh = p->in_h; a.ow = p->in_w;
+  a.kd = p->kd; a.kh = p->kh; a.kw = p->kw; a.sd = 1; a.sh = 1; a.sw = 1;
+  a.pd = p->dd * (p->kd - 1) - p->pd; a.ph = p->dh * (p->kh - 1) - p->ph; a.pw = p->dw * (p->kw - 1) - p->pw;
+  a.dd = p->dd; a.dh = p->dh; a.dw = p->dw;
+  a.flip = 1;
+  a.ws_co = w_stride[1]; a.ws_ci = w_stride[0]; a.ws_kd = w_stride[2]; a.ws_kh = w_stride[3]; a.ws_kw = w_stride[4];
+  return direct_conv_gather(a, dtype, gy, w, nullptr, gx, st);
+}
+
+// ---- weight gradient -------------------------------------------------------------------
+extern "C" int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (!wgrad_uses_mfma(*p, dtype, out)) return 1;
+  return mfma_wgrad_splits(wgrad_args(*p, out));
+}
+
+extern "C" size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (!wgrad_uses_mfma(*p, dtype, out)) return 0;
+  return mfma_wgrad_workspace_bytes(wgrad_args(*p, out));
+}
+
+extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* workspace,
+                                size_t workspace_bytes, uint32_t flags, void* stream) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (x == nullptr || gy == nullptr || gw == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad: null tensor");
+  hipStream_t st = (hipStream_t)stream;
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_mfma(*p, dtype, out)) {
+    const WgradArgs a = wgrad_args(*p, out);
+    const size_t need = mfma_wgrad_workspace_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    return mfma_wgrad(a, dtype, x, gy, gw, workspace, st);
+  }
+  DirectConvArgs a{};
+  a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;
+  a.cout = p->cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
+  a.kd = p->kd; a.kh = p->kh; a.kw = p->kw; a.sd = p->sd; a.sh = p->sh; a.sw = p->sw;
+  a.pd = p->pd; a.ph = p->ph; a.pw = p->pw; a.dd = p->dd; a.dh = p->dh; a.dw = p->dw;
+  return direct_conv_wgrad(a, dtype, x, gy, gw, st);
+}
+
+// ---- transposed convolution ------------------------------------------------------------
+static int check_convT(const sfh_convT3d_desc* p, int dtype) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "convT3d: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "convT3d: bad dtype %d", dtype);
+  if (p->n < 0 || p->cin < 1 || p->cout < 1 || p->in_d < 1 || p->in_h < 1 || p->in_w < 1 || p->kd < 1 || p->kh < 1 || p->kw < 1)
+    return fail(SFH_ERR_INVALID, "convT3d: bad extents");
+  return SFH_OK;
+}
+
+extern "C" size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int dtype) {
+  if (check_convT(p, dtype) != SFH_OK) return 0;
+  return 0;
+}
+
+extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                               const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  (void)workspace; (void)workspace_bytes; (void)flags;
+  if (int rc = check_convT(p, dtype)) return rc;
+  if (x == nullptr || w == nullptr || y == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
+  if (p->n == 0) return SFH_OK;
+  return direct_convT(*p, dtype, w_stride, x, w, bias, y, (hipStream_t)stream);
+}
+
+// ---- measurement helper ----------------------------------------------------------------
+extern "C" int sfh_stream_copy(const void* src, void* dst, size_t bytes, void* stream) {
+  if (src == nullptr || dst == nullptr || bytes % 16 != 0) return fail(SFH_ERR_INVALID, "stream copy: need 16-byte multiples");
+  if (bytes == 0) return SFH_OK;
+  hipLaunchKernelGGL(stream_copy_kernel, dim3(kComputeUnits * 4), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
+                     (uint4*)dst, bytes / 16);
+  return check_launch("stream_copy_kernel");
+}

@@ -1,0 +1,82 @@
+// Shared device/host helpers for libscaffold_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/scaffold_hip.h"
+
+namespace sfh {
+
+// ---- error plumbing -----------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+// Checks the launch status of the kernel that was just enqueued.
+int check_launch(const char* what);
+
+// ---- element types ------------------------------------------------------------------
+// Storage types are raw bit patterns; arithmetic is always done in float.
+struct bf16_t { uint16_t bits; };
+struct fp16_t { _Float16 v; };
+
+__device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((uint32_t)x.bits) << 16); }
+__device__ __forceinline__ float to_float(fp16_t x) { return (float)x.v; }
+__device__ __forceinline__ float to_float(float x) { return x; }
+
+// Round-to-nearest-even fp32 -> bf16 (NaN stays NaN, quietened).
+__device__ __forceinline__ uint16_t bf16_bits_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct elem;
+template <> struct elem<bf16_t> {
+  static __device__ __forceinline__ bf16_t from_float(float f) { bf16_t r; r.bits = bf16_bits_rne(f); return r; }
+};
+template <> struct elem<fp16_t> {
+  static __device__ __forceinline__ fp16_t from_float(float f) { fp16_t r; r.v = (_Float16)f; return r; }
+};
+template <> struct elem<float> {
+  static __device__ __forceinline__ float from_float(float f) { return f; }
+};
+
+// Two bf16 packed in a dword -> two floats, and back.
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)bf16_bits_rne(lo) | ((uint32_t)bf16_bits_rne(hi) << 16);
+}
+__device__ __forceinline__ uint32_t pack_fp16x2(float lo, float hi) {
+  union { _Float16 h[2]; uint32_t u; } r;
+  r.h[0] = (_Float16)lo; r.h[1] = (_Float16)hi;
+  return r.u;
+}
+__device__ __forceinline__ float fp16_lo(uint32_t u) { union { uint32_t u; _Float16 h[2]; } r; r.u = u; return (float)r.h[0]; }
+__device__ __forceinline__ float fp16_hi(uint32_t u) { union { uint32_t u; _Float16 h[2]; } r; r.u = u; return (float)r.h[1]; }
+
+inline size_t dtype_size(int dtype) { return dtype == SFH_FP32 ? 4 : 2; }
+inline bool dtype_ok(int dtype) { return dtype == SFH_BF16 || dtype == SFH_FP16 || dtype == SFH_FP32; }
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Number of compute units the launch heuristics are written for (MI355X).
+constexpr int kComputeUnits = 256;
+constexpr int kXcds = 8;
+
+// Maps the hardware workgroup id (dispatched round-robin over the 8 XCDs) to a logical
+// tile id such that every XCD, and so every L2, works on one contiguous range of tiles.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total) {
+  const uint32_t per = total / kXcds, rem = total % kXcds;
+  const uint32_t xcd = pid % kXcds, slot = pid / kXcds;
+  // XCDs [0, rem) own per+1 tiles, the rest own per tiles.
+  const uint32_t start = xcd * per + (xcd < rem ? xcd : rem);
+  return start + slot;
+}
+
+}  // namespace sfh

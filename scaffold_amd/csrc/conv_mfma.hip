@@ -1,0 +1,278 @@
+// MFMA implicit-GEMM convolution for gfx950: stride 1, dilation 1, kernel extents <= 3,
+// bf16 / fp16 operands, fp32 accumulation, one rounding on store.
+//
+// GEMM view (triton_conv3d/gather_gemm.py:112-341): M = output voxels, N = produced channels,
+// K = taps x reduction channels. What is different here is where the operands live:
+//
+//   * A workgroup owns a TD x TH x TW brick of output voxels and stages the matching input
+//     brick INCLUDING its halo in LDS once per 32-channel chunk; all taps then read it at a
+//     constant offset, so an input voxel is fetched from memory once per brick instead of once
+//     per tap.
+//   * LDS layout is four "planes" per chunk, plane p holding channels [8p, 8p+8) of every brick
+//     voxel as one 16-byte unit. A wavefront's activation fragment for 32 consecutive voxels is
+//     then 512 contiguous bytes per half-wave: ds_read_b128 without bank conflicts, no padding
+//     between voxels, and every (tap, k-step) is an immediate offset from one per-lane base.
+//     Planes are spaced 64 bytes (mod 256) apart so the staging writes do not conflict either.
+//   * The weight is repacked once per call (a few hundred KB) into MFMA fragment order, so a
+//     wavefront fetches the fragment for (tap, k-step) as one contiguous 1 KiB global load that
+//     hits in L1/L2; it is reused across the wave's four 32-voxel sub-tiles.
+//   * v_mfma_f32_32x32x16 with the WEIGHT as the row operand: a lane then ends up holding, for
+//     one voxel, four runs of four consecutive output channels, which are stored as 8-byte pieces.
+//
+// The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
+// padding k-1-p (triton_conv3d/bwd_data.py:344-363).
+#include "conv_mfma.hpp"
+
+namespace sfh {
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+};
+template <> struct Mma<fp16_t> {
+  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_fp16x2(lo, hi); }
+};
+
+constexpr int kChunk = 32;  // reduction channels staged per pass (4 planes of 8)
+
+constexpr int plane_bytes(int voxels) {
+  // smallest size >= voxels*16 that is 64 modulo 256
+  int b = voxels * 16;
+  int r = ((b - 64 + 255) / 256) * 256 + 64;
+  return r;
+}
+
+template <int TD_, int TH_, int TW_, int KD_, int KH_, int KW_, int NSUB_>
+struct Tile {
+  static constexpr int TD = TD_, TH = TH_, TW = TW_, KD = KD_, KH = KH_, KW = KW_, NSUB = NSUB_;
+  static constexpr int BD = TD + KD - 1, BH = TH + KH - 1, BW = TW + KW - 1;
+  static constexpr int BV = BD * BH * BW;            // brick voxels
+  static constexpr int PLANE = plane_bytes(BV);
+  static constexpr int LDS = 4 * PLANE;
+  static constexpr int TAPS = KD * KH * KW;
+  static constexpr int SUBTILES = TD * TH * TW / 32;  // 32-voxel MFMA column blocks
+  static constexpr int MS = SUBTILES / 4;             // per wavefront
+  static_assert(TD * TH * TW % 128 == 0, "tile must split into 4 wavefronts of 32-voxel sub-tiles");
+  static_assert(LDS <= 80 * 1024, "two workgroups must fit in the 160 KB LDS of a CU");
+  static_assert(2 * PLANE + ((KD - 1) * BH * BW + (KH - 1) * BW + KW - 1) * 16 < 65536, "ds_read immediate range");
+};
+
+template <typename T, typename C>
+__global__ void __launch_bounds__(256, 2)
+conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
+                 T* __restrict__ y, int tiles_d, int tiles_h, int tiles_w, int nblocks, uint32_t total) {
+  __shared__ __attribute__((aligned(16))) char lds[C::LDS];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 31, kg = lane >> 5;
+
+  uint32_t t = xcd_remap(blockIdx.x, total);
+  const int nb = t % nblocks; t /= nblocks;
+  const int tw_i = t % tiles_w; t /= tiles_w;
+  const int th_i = t % tiles_h; t /= tiles_h;
+  const int td_i = t % tiles_d;
+  const int n = t / tiles_d;
+  const int od0 = td_i * C::TD, oh0 = th_i * C::TH, ow0 = tw_i * C::TW;
+
+  // Per-lane LDS byte offset of the sub-tile voxel at tap (0,0,0), in the lane's k-half plane.
+  int lbase[C::MS];
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms) {
+    const int v = (wave * C::MS + ms) * 32 + j;
+    const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
+    lbase[ms] = kg * C::PLANE + ((td * C::BH + th) * C::BW + tw) * 16;
+  }
+
+  f32x16_t acc[C::MS][C::NSUB];
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms)
+#pragma unroll
+    for (int ns = 0; ns < C::NSUB; ++ns)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ms][ns][r] = 0.f;
+
+  const int ncc = a.cred / kChunk;
+  const int id0 = od0 - a.pd, ih0 = oh0 - a.ph, iw0 = ow0 - a.pw;
+  constexpr int PIECES = C::BV * 4;
+  constexpr int ITERS = (PIECES + 255) / 256;
+  constexpr int BATCH = 8;
+  constexpr int FRAG = 512;  // elements per packed (tap, k-step) fragment: 64 lanes x 8
+
+  for (int cc = 0; cc < ncc; ++cc) {
+    __syncthreads();  // every wave is done reading the previous chunk
+    {
+      const T* xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cred + cc * kChunk;
+#pragma unroll
+      for (int it0 = 0; it0 < ITERS; it0 += BATCH) {
+        uint4 v[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          if (it0 + u < ITERS) {
+            const int p = (it0 + u) * 256 + tid;
+            v[u] = make_uint4(0, 0, 0, 0);
+            if (p < PIECES) {
+              const int vox = p >> 2, piece = p & 3;
+              const int bw = vox % C::BW, bh = (vox / C::BW) % C::BH, bd = vox / (C::BW * C::BH);
+              const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
+              if ((unsigned)id < (unsigned)a.id && (unsigned)ih < (unsigned)a.ih && (unsigned)iw < (unsigned)a.iw)
+                v[u] = *reinterpret_cast<const uint4*>(xn + (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8);
+            }
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          if (it0 + u < ITERS) {
+            const int p = (it0 + u) * 256 + tid;
+            if (p < PIECES) *reinterpret_cast<uint4*>(lds + (p & 3) * C::PLANE + (p >> 2) * 16) = v[u];
+          }
+        }
+      }
+    }
+    __syncthreads();
+
+    const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
+    const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
+#pragma unroll
+    for (int tap = 0; tap < C::TAPS; ++tap) {
+      constexpr int KHW = C::KH * C::KW;
+      const int kd = tap / KHW, kh = (tap / C::KW) % C::KH, kw = tap % C::KW;
+      const int tapoff = ((kd * C::BH + kh) * C::BW + kw) * 16;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        uint4 wf[C::NSUB];
+#pragma unroll
+        for (int ns = 0; ns < C::NSUB; ++ns)
+          wf[ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + (tap * 2 + ks) * FRAG);
+#pragma unroll
+        for (int ms = 0; ms < C::MS; ++ms) {
+          const uint4 af = *reinterpret_cast<const uint4*>(lds + lbase[ms] + tapoff + ks * 2 * C::PLANE);
+#pragma unroll
+          for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma<T>::run(wf[ns], af, acc[ms][ns]);
+        }
+      }
+    }
+  }
+
+  // Epilogue. Accumulator register r of a lane is output channel 8*(r/4) + 4*kg + r%4 of the
+  // sub-tile's voxel j: four runs of four consecutive channels per 32-channel block.
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms) {
+    const int v = (wave * C::MS + ms) * 32 + j;
+    const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
+    const int od = od0 + td, oh = oh0 + th, ow = ow0 + tw;
+    if (od >= a.od || oh >= a.oh || ow >= a.ow) continue;
+    T* yp = y + ((((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cout + nb * C::NSUB * 32;
+#pragma unroll
+    for (int ns = 0; ns < C::NSUB; ++ns) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int co = ns * 32 + 8 * g + 4 * kg;
+        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+        if (bias != nullptr) {
+          const T* bp = bias + nb * C::NSUB * 32 + co;
+          b0 = to_float(bp[0]); b1 = to_float(bp[1]); b2 = to_float(bp[2]); b3 = to_float(bp[3]);
+        }
+        uint2 o;
+        o.x = Mma<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
+        o.y = Mma<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
+        *reinterpret_cast<uint2*>(yp + co) = o;
+      }
+    }
+  }
+}
+
+// One thread per packed element.
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, T* __restrict__ packed, int cout, int cred,
+                                                          int kd, int kh, int kw, int64_t s_out, int64_t s_red, int64_t s_kd,
+                                                          int64_t s_kh, int64_t s_kw, int flip, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int taps = kd * kh * kw;
+  int64_t r = idx;
+  const int e = (int)(r % 8); r /= 8;
+  const int lane = (int)(r % 64); r /= 64;
+  const int ks = (int)(r % 2); r /= 2;
+  int tap = (int)(r % taps); r /= taps;
+  const int ncc = cred / kChunk;
+  const int cc = (int)(r % ncc);
+  const int nblk = (int)(r / ncc);
+  const int co = nblk * 32 + (lane & 31);
+  const int ci = cc * kChunk + ks * 16 + (lane >> 5) * 8 + e;
+  if (flip) tap = taps - 1 - tap;
+  const int tkw = tap % kw, tkh = (tap / kw) % kh, tkd = tap / (kw * kh);
+  packed[idx] = w[co * s_out + ci * s_red + tkd * s_kd + tkh * s_kh + tkw * s_kw];
+}
+
+template <typename T, typename C>
+int launch_cfg(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+  const int tiles_d = (int)cdiv(a.od, C::TD), tiles_h = (int)cdiv(a.oh, C::TH), tiles_w = (int)cdiv(a.ow, C::TW);
+  const int nblocks = a.cout / (32 * C::NSUB);
+  const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks;
+  if (total == 0) return SFH_OK;
+  if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: %lld workgroups exceed the grid limit", (long long)total);
+  hipLaunchKernelGGL((conv_mfma_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
+                     (const T*)bias, (T*)y, tiles_d, tiles_h, tiles_w, nblocks, (uint32_t)total);
+  return check_launch("conv_mfma_kernel");
+}
+
+template <typename T, int NSUB>
+int launch_k333(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+  // Brick shape follows the row length: 32-voxel sub-tiles are one, two or four W rows.
+  if (a.ow > 16) return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
+  if (a.ow > 8) return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
+  return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
+}
+
+template <typename T>
+int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+  if (a.cout % 64 == 0) return launch_k333<T, 2>(a, x, packed, bias, y, st);
+  return launch_k333<T, 1>(a, x, packed, bias, y, st);
+}
+
+}  // namespace
+
+bool mfma_conv_supported(const MfmaConvArgs& a, int dtype) {
+  if (dtype != SFH_BF16 && dtype != SFH_FP16) return false;
+  if (a.kd != 3 || a.kh != 3 || a.kw != 3) return false;
+  if (a.cred % kChunk != 0 || a.cout % 32 != 0) return false;
+  if (a.pd < 0 || a.ph < 0 || a.pw < 0 || a.pd > 2 || a.ph > 2 || a.pw > 2) return false;
+  if (a.n < 1 || a.od < 1 || a.oh < 1 || a.ow < 1) return false;
+  return true;
+}
+
+size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a) {
+  return align_up((size_t)a.cout * a.cred * a.kd * a.kh * a.kw * 2, 256);
+}
+
+int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd, int64_t s_kh,
+                     int64_t s_kw, int flip, void* packed, hipStream_t st) {
+  const int64_t total = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw;
+  const unsigned blocks = (unsigned)cdiv(total, 256);
+  if (dtype == SFH_BF16)
+    hipLaunchKernelGGL(pack_weight_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)w, (bf16_t*)packed, a.cout,
+                       a.cred, a.kd, a.kh, a.kw, s_out, s_red, s_kd, s_kh, s_kw, flip, total);
+  else
+    hipLaunchKernelGGL(pack_weight_kernel<fp16_t>, dim3(blocks), dim3(256), 0, st, (const fp16_t*)w, (fp16_t*)packed, a.cout,
+                       a.cred, a.kd, a.kh, a.kw, s_out, s_red, s_kd, s_kh, s_kw, flip, total);
+  return check_launch("pack_weight_kernel");
+}
+
+int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
+                     hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st);
+  return launch_typed<fp16_t>(a, x, packed, bias, y, st);
+}
+
+}  // namespace sfh

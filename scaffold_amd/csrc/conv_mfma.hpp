@@ -1,0 +1,28 @@
+// Host-side interface of the MFMA implicit-GEMM convolution kernels (bf16 / fp16 only).
+#pragma once
+#include "common.hpp"
+
+namespace sfh {
+
+// A stride-1, dilation-1 gather convolution in the roles the kernel sees them: `cred` reduction
+// channels (a multiple of 32), `cout` produced channels (a multiple of 32), kernel extents in
+// 1..3. The forward passes (Cin, Cout, padding); the data gradient passes (Cout, Cin, k-1-p)
+// with the weight packed transposed and tap-flipped.
+struct MfmaConvArgs {
+  int n, cred, id, ih, iw;
+  int cout, od, oh, ow;
+  int kd, kh, kw, pd, ph, pw;
+};
+
+bool mfma_conv_supported(const MfmaConvArgs& a, int dtype);
+size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a);
+// Repacks the weight into per-wavefront MFMA fragment order:
+//   packed[cout/32][cred/32][tap][kstep(2)][lane(64)][8]
+// with lane = (cout % 32) + 32 * (cred % 16 / 8). `s_out`, `s_red`, `s_kd/kh/kw` are element
+// strides of the source for the produced channel, the reduction channel and the taps.
+int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd,
+                     int64_t s_kh, int64_t s_kw, int flip, void* packed, hipStream_t st);
+int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
+                     hipStream_t st);
+
+}  // namespace sfh

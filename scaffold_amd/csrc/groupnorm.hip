@@ -1,0 +1,839 @@
+// Channels-last GroupNorm forward / backward for a dense (N, S, C) tensor.
+//
+// Statistics are fp32 and computed in one streaming pass with SHIFTED sums: every workgroup
+// first derives, for each group, the same shift K (the mean of the group's channels over the
+// first voxels of the sample) and then accumulates sum(x-K) and sum((x-K)^2). Because the shift
+// is within a fraction of a standard deviation of the true mean, var = S2/m - (S1/m)^2 does not
+// cancel the way E[x^2]-E[x]^2 does at mean >> std, and because every workgroup of a sample
+// uses the identical shift the partial sums add without a pairwise (Chan) correction. This is
+// the role the corrected two-pass tile statistics + Welford merge play in the reference
+// (ScaFFold/unet/triton_group_norm.py:148-165,594-694).
+//
+// Launch chain (no atomics, partials at fixed scratch slots, fixed-order sums):
+//   forward : gn_stats_partial -> gn_stats_finalize -> gn_normalize          (3*B bytes streamed)
+//   backward: gn_bwd_partial   -> gn_bwd_finalize   -> gn_dx                 (5*B bytes streamed)
+// The fused ReLU is spelled `y <= 0 ? 0 : y` and the backward gate `pre <= 0 ? 0 : dy` so that
+// NaN propagates exactly as F.relu / threshold_backward do (triton_group_norm.py:176-198), and
+// the gate is evaluated on the pre-activation recomputed with the forward's own expression.
+//
+// Two code paths, chosen by shape only: the vector path (16-byte loads, a thread owns a fixed
+// set of channels) when C is a multiple of the vector width and the channels of a thread fall
+// into whole groups; the scalar path (one workgroup per (sample, group)) otherwise.
+#include "common.hpp"
+
+namespace sfh {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kShiftRows = 32;   // voxels that define the shift K
+constexpr int kMaxSplit = 2048;  // workgroups per sample
+
+struct GnPlan {
+  bool vector;
+  int vec;    // elements per thread and row
+  int tpr;    // threads per voxel row = C / vec
+  int rpp;    // voxel rows per pass of a workgroup
+  int slots;  // group slots per thread: max(1, vec / (C/G))
+  int nsplit; // workgroups per sample (reduction and elementwise passes alike)
+  int64_t rows_per_split;
+};
+
+GnPlan make_plan(const sfh_groupnorm_desc& p, int x_dtype, bool aligned) {
+  GnPlan pl{};
+  pl.vec = x_dtype == SFH_FP32 ? 4 : 8;
+  const int cg = p.c / p.groups;
+  pl.vector = aligned && p.c % pl.vec == 0 && p.c / pl.vec <= kBlock && (cg % pl.vec == 0 || pl.vec % cg == 0);
+  if (!pl.vector) {
+    pl.nsplit = 1;
+    pl.rows_per_split = p.spatial;
+    return pl;
+  }
+  pl.tpr = p.c / pl.vec;
+  pl.rpp = kBlock / pl.tpr;
+  pl.slots = cg >= pl.vec ? 1 : pl.vec / cg;
+  int64_t rows = (int64_t)pl.rpp * 16;  // 16 passes of 4 KiB per workgroup
+  if (cdiv(p.spatial, rows) > kMaxSplit) rows = cdiv(cdiv(p.spatial, kMaxSplit), pl.rpp) * pl.rpp;
+  pl.rows_per_split = rows;
+  pl.nsplit = (int)cdiv(p.spatial, rows);
+  return pl;
+}
+
+// ---- element vector load/store ------------------------------------------------------------
+template <typename T, int V> struct Ld;
+template <int V> struct Ld<bf16_t, V> {
+  static __device__ __forceinline__ void run(const bf16_t* p, float (&f)[V]) {
+    if constexpr (V == 8) {
+      const uint4 v = *reinterpret_cast<const uint4*>(p);
+      f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+      f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+    } else {
+      const uint2 v = *reinterpret_cast<const uint2*>(p);
+      f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+    }
+  }
+};
+template <int V> struct Ld<fp16_t, V> {
+  static __device__ __forceinline__ void run(const fp16_t* p, float (&f)[V]) {
+    if constexpr (V == 8) {
+      const uint4 v = *reinterpret_cast<const uint4*>(p);
+      f[0] = fp16_lo(v.x); f[1] = fp16_hi(v.x); f[2] = fp16_lo(v.y); f[3] = fp16_hi(v.y);
+      f[4] = fp16_lo(v.z); f[5] = fp16_hi(v.z); f[6] = fp16_lo(v.w); f[7] = fp16_hi(v.w);
+    } else {
+      const uint2 v = *reinterpret_cast<const uint2*>(p);
+      f[0] = fp16_lo(v.x); f[1] = fp16_hi(v.x); f[2] = fp16_lo(v.y); f[3] = fp16_hi(v.y);
+    }
+  }
+};
+template <int V> struct Ld<float, V> {
+  static __device__ __forceinline__ void run(const float* p, float (&f)[V]) {
+#pragma unroll
+    for (int i = 0; i < V / 4; ++i) {
+      const float4 v = *reinterpret_cast<const float4*>(p + 4 * i);
+      f[4 * i] = v.x; f[4 * i + 1] = v.y; f[4 * i + 2] = v.z; f[4 * i + 3] = v.w;
+    }
+  }
+};
+
+template <typename T, int V> struct St;
+template <int V> struct St<bf16_t, V> {
+  static __device__ __forceinline__ void run(bf16_t* p, const float (&f)[V]) {
+    uint32_t u[V / 2];
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) u[i] = pack_bf16x2(f[2 * i], f[2 * i + 1]);
+    if constexpr (V == 8) *reinterpret_cast<uint4*>(p) = make_uint4(u[0], u[1], u[2], u[3]);
+    else *reinterpret_cast<uint2*>(p) = make_uint2(u[0], u[1]);
+  }
+};
+template <int V> struct St<fp16_t, V> {
+  static __device__ __forceinline__ void run(fp16_t* p, const float (&f)[V]) {
+    uint32_t u[V / 2];
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) u[i] = pack_fp16x2(f[2 * i], f[2 * i + 1]);
+    if constexpr (V == 8) *reinterpret_cast<uint4*>(p) = make_uint4(u[0], u[1], u[2], u[3]);
+    else *reinterpret_cast<uint2*>(p) = make_uint2(u[0], u[1]);
+  }
+};
+template <int V> struct St<float, V> {
+  static __device__ __forceinline__ void run(float* p, const float (&f)[V]) {
+#pragma unroll
+    for (int i = 0; i < V / 4; ++i)
+      *reinterpret_cast<float4*>(p + 4 * i) = make_float4(f[4 * i], f[4 * i + 1], f[4 * i + 2], f[4 * i + 3]);
+  }
+};
+
+template <typename T> struct VecOf { static constexpr int N = 8; };
+template <> struct VecOf<float> { static constexpr int N = 4; };
+
+__device__ __forceinline__ float load_param(const void* p, int dtype, int i, float dflt) {
+  if (p == nullptr) return dflt;
+  if (dtype == SFH_FP32) return static_cast<const float*>(p)[i];
+  if (dtype == SFH_BF16) return to_float(static_cast<const bf16_t*>(p)[i]);
+  return to_float(static_cast<const fp16_t*>(p)[i]);
+}
+
+__device__ __forceinline__ float relu_keep_nan(float y) { return y <= 0.f ? 0.f : y; }
+
+// Fixed-order sum over a 64-lane wavefront; lane 0 holds the result.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+// Sums NVAL per-thread values over the voxel rows of the workgroup (threads sharing a channel
+// vector cv) with a fixed binary tree. Afterwards buf[v * kBlock + cv], cv < tpr, holds the
+// totals. buf needs NVAL * kBlock floats.
+template <int NVAL>
+__device__ __forceinline__ void block_row_reduce(const float (&val)[NVAL], float* buf, int tpr, int rpp, bool active) {
+  const int tid = threadIdx.x;
+  const int r = tid / tpr;
+  __syncthreads();
+  if (active) {
+#pragma unroll
+    for (int v = 0; v < NVAL; ++v) buf[v * kBlock + tid] = val[v];
+  }
+  __syncthreads();
+  int top = 1;
+  while (top < rpp) top <<= 1;
+  for (int stride = top >> 1; stride > 0; stride >>= 1) {
+    if (active && r < stride && r + stride < rpp) {
+#pragma unroll
+      for (int v = 0; v < NVAL; ++v) buf[v * kBlock + tid] += buf[v * kBlock + tid + stride * tpr];
+    }
+    __syncthreads();
+  }
+}
+
+// Folds the per-channel-vector totals of NQ quantities (SLOTS slots each, value index
+// q * SLOTS + s) into per-group totals out[q * G + g].
+template <int SLOTS, int NQ>
+__device__ __forceinline__ void fold_groups(const float* buf, float* out, int G, int cg, int vec) {
+  for (int g = threadIdx.x; g < G; g += kBlock) {
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      float s = 0.f;
+      if (SLOTS > 1) {
+        s = buf[(q * SLOTS + (g % SLOTS)) * kBlock + g / SLOTS];
+      } else {
+        const int per = cg / vec;
+        for (int k = 0; k < per; ++k) s += buf[q * kBlock + g * per + k];
+      }
+      out[q * G + g] = s;
+    }
+  }
+  __syncthreads();
+}
+
+// ---- forward: partial statistics (vector path) --------------------------------------------
+// scratch (floats): shift[N][G] | part[N][nsplit][2][G]
+template <typename T, int SLOTS>
+__global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__ x, float* __restrict__ shift,
+                                                           float* __restrict__ part, int64_t S, int C, int G, int tpr, int rpp,
+                                                           int nsplit, int64_t rows_per_split) {
+  constexpr int V = VecOf<T>::N;
+  extern __shared__ float smem[];
+  float* buf = smem;                        // 2 * SLOTS * kBlock
+  float* out = smem + 2 * SLOTS * kBlock;   // 2 * G
+  const int tid = threadIdx.x;
+  const int n = blockIdx.y, split = blockIdx.x;
+  const int cg = C / G;
+  const int r = tid / tpr, cv = tid - r * tpr;
+  const bool active = r < rpp;
+  const T* xs = x + (int64_t)n * S * C + cv * V;
+
+  // Shift K: mean of every group over the first voxels of the sample, bit-identical in every
+  // workgroup of the sample because it is computed from the same rows in the same order.
+  const int64_t krows = S < kShiftRows ? S : kShiftRows;
+  float kv[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) kv[s] = 0.f;
+  if (active) {
+    for (int64_t row = r; row < krows; row += rpp) {
+      float f[V];
+      Ld<T, V>::run(xs + row * C, f);
+#pragma unroll
+      for (int e = 0; e < V; ++e) kv[e * SLOTS / V] += f[e];
+    }
+  }
+  block_row_reduce<SLOTS>(kv, buf, tpr, rpp, active);
+  fold_groups<SLOTS, 1>(buf, out, G, cg, V);
+  const float kinv = 1.f / ((float)krows * (float)cg);
+  float K[SLOTS];
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) {
+    const int g = (SLOTS > 1) ? cv * SLOTS + s : (cv * V) / cg;
+    K[s] = active ? out[g] * kinv : 0.f;
+  }
+  if (split == 0)
+    for (int g = tid; g < G; g += kBlock) shift[n * G + g] = out[g] * kinv;
+
+  float acc[2 * SLOTS];
+#pragma unroll
+  for (int s = 0; s < 2 * SLOTS; ++s) acc[s] = 0.f;
+  const int64_t begin = (int64_t)split * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  if (active) {
+    int64_t row = begin + r;
+    const int64_t step = rpp;
+    for (; row + 3 * step < end; row += 4 * step) {  // four independent loads in flight
+      float f0[V], f1[V], f2[V], f3[V];
+      Ld<T, V>::run(xs + row * C, f0);
+      Ld<T, V>::run(xs + (row + step) * C, f1);
+      Ld<T, V>::run(xs + (row + 2 * step) * C, f2);
+      Ld<T, V>::run(xs + (row + 3 * step) * C, f3);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int s = e * SLOTS / V;
+        const float d0 = f0[e] - K[s], d1 = f1[e] - K[s], d2 = f2[e] - K[s], d3 = f3[e] - K[s];
+        acc[s] += (d0 + d1) + (d2 + d3);
+        float q = acc[SLOTS + s];
+        q = fmaf(d0, d0, q); q = fmaf(d1, d1, q); q = fmaf(d2, d2, q); q = fmaf(d3, d3, q);
+        acc[SLOTS + s] = q;
+      }
+    }
+    for (; row < end; row += step) {
+      float f0[V];
+      Ld<T, V>::run(xs + row * C, f0);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int s = e * SLOTS / V;
+        const float d0 = f0[e] - K[s];
+        acc[s] += d0;
+        acc[SLOTS + s] = fmaf(d0, d0, acc[SLOTS + s]);
+      }
+    }
+  }
+  block_row_reduce<2 * SLOTS>(acc, buf, tpr, rpp, active);
+  fold_groups<SLOTS, 2>(buf, out, G, cg, V);
+  float* dst = part + ((int64_t)n * nsplit + split) * 2 * G;
+  for (int i = tid; i < 2 * G; i += kBlock) dst[i] = out[i];
+}
+
+// One 64-lane workgroup per (group, sample): fixed-order sum of the split partials, then
+// mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps).
+__global__ void __launch_bounds__(64) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
+                                                        float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
+                                                        float m, float eps) {
+  const int g = blockIdx.x, n = blockIdx.y;
+  float s1 = 0.f, s2 = 0.f;
+  for (int i = threadIdx.x; i < nsplit; i += 64) {
+    const float* p = part + ((int64_t)n * nsplit + i) * 2 * G;
+    s1 += p[g];
+    s2 += p[G + g];
+  }
+  s1 = wave_sum(s1);
+  s2 = wave_sum(s2);
+  if (threadIdx.x == 0) {
+    const float d = s1 / m;
+    float var = s2 / m - d * d;
+    var = var < 0.f ? 0.f : var;
+    mean[n * G + g] = shift[n * G + g] + d;
+    rstd[n * G + g] = 1.f / sqrtf(var + eps);
+  }
+}
+
+// ---- forward: normalise + affine (+ReLU) (vector path) ------------------------------------
+template <typename T, typename TO>
+__global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, TO* __restrict__ y, const float* __restrict__ mean,
+                                                       const float* __restrict__ rstd, const void* __restrict__ gamma,
+                                                       const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
+                                                       int tpr, int rpp, int64_t rows_per_split, int relu) {
+  constexpr int V = VecOf<T>::N;
+  const int tid = threadIdx.x;
+  const int n = blockIdx.y;
+  const int cg = C / G;
+  const int r = tid / tpr, cv = tid - r * tpr;
+  if (r >= rpp) return;
+  float mu[V], rs[V], ga[V], be[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int c = cv * V + e;
+    mu[e] = mean[n * G + c / cg];
+    rs[e] = rstd[n * G + c / cg];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
+  }
+  const int64_t base = (int64_t)n * S * C + cv * V;
+  const T* xs = x + base;
+  TO* ys = y + base;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  for (; row + 3 * step < end; row += 4 * step) {
+    float f[4][V];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) Ld<T, V>::run(xs + (row + u * step) * C, f[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float o[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float xh = (f[u][e] - mu[e]) * rs[e];
+        const float v = fmaf(xh, ga[e], be[e]);
+        o[e] = relu ? relu_keep_nan(v) : v;
+      }
+      St<TO, V>::run(ys + (row + u * step) * C, o);
+    }
+  }
+  for (; row < end; row += step) {
+    float f[V], o[V];
+    Ld<T, V>::run(xs + row * C, f);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float xh = (f[e] - mu[e]) * rs[e];
+      const float v = fmaf(xh, ga[e], be[e]);
+      o[e] = relu ? relu_keep_nan(v) : v;
+    }
+    St<TO, V>::run(ys + row * C, o);
+  }
+}
+
+// ---- backward: per-channel partial sums (vector path) --------------------------------------
+// part (floats): [N][nsplit][2][C]  with q = 0: sum dy'*xhat, q = 1: sum dy'
+template <typename T, typename TG>
+__global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x, const TG* __restrict__ dy,
+                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                         const void* __restrict__ gamma, const void* __restrict__ beta,
+                                                         int param_dtype, float* __restrict__ part, int64_t S, int C, int G,
+                                                         int tpr, int rpp, int nsplit, int64_t rows_per_split, int relu) {
+  constexpr int V = VecOf<T>::N;
+  extern __shared__ float smem[];  // 2 * V * kBlock
+  const int tid = threadIdx.x;
+  const int n = blockIdx.y, split = blockIdx.x;
+  const int cg = C / G;
+  const int r = tid / tpr, cv = tid - r * tpr;
+  const bool active = r < rpp;
+  float mu[V], rs[V], ga[V], be[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int c = active ? cv * V + e : 0;
+    mu[e] = mean[n * G + c / cg];
+    rs[e] = rstd[n * G + c / cg];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
+  }
+  float acc[2 * V];
+#pragma unroll
+  for (int e = 0; e < 2 * V; ++e) acc[e] = 0.f;
+  if (active) {
+    const int64_t base = (int64_t)n * S * C + cv * V;
+    const T* xs = x + base;
+    const TG* gs = dy + base;
+    const int64_t begin = (int64_t)split * rows_per_split;
+    int64_t end = begin + rows_per_split;
+    if (end > S) end = S;
+    const int64_t step = rpp;
+    int64_t row = begin + r;
+    for (; row + step < end; row += 2 * step) {
+      float f0[V], g0[V], f1[V], g1[V];
+      Ld<T, V>::run(xs + row * C, f0);
+      Ld<TG, V>::run(gs + row * C, g0);
+      Ld<T, V>::run(xs + (row + step) * C, f1);
+      Ld<TG, V>::run(gs + (row + step) * C, g1);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float xh0 = (f0[e] - mu[e]) * rs[e], xh1 = (f1[e] - mu[e]) * rs[e];
+        float d0 = g0[e], d1 = g1[e];
+        if (relu) {
+          d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
+          d1 = fmaf(xh1, ga[e], be[e]) <= 0.f ? 0.f : d1;
+        }
+        acc[e] = fmaf(d0, xh0, acc[e]);
+        acc[e] = fmaf(d1, xh1, acc[e]);
+        acc[V + e] += d0 + d1;
+      }
+    }
+    for (; row < end; row += step) {
+      float f0[V], g0[V];
+      Ld<T, V>::run(xs + row * C, f0);
+      Ld<TG, V>::run(gs + row * C, g0);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float xh0 = (f0[e] - mu[e]) * rs[e];
+        float d0 = g0[e];
+        if (relu) d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
+        acc[e] = fmaf(d0, xh0, acc[e]);
+        acc[V + e] += d0;
+      }
+    }
+  }
+  block_row_reduce<2 * V>(acc, smem, tpr, rpp, active);
+  float* dst = part + ((int64_t)n * nsplit + split) * 2 * C;
+  for (int i = tid; i < 2 * C; i += kBlock) {
+    const int q = i / C, c = i - q * C;
+    dst[i] = smem[(q * V + c % V) * kBlock + c / V];
+  }
+}
+
+// Workgroups [0, N*G): coef[n][g] = (A, B) with A = mean(dy'*gamma), B = mean(dy'*gamma*xhat)
+// over the group. Workgroups [N*G, N*G + C): dgamma[c], dbeta[c] summed over samples and splits.
+__global__ void __launch_bounds__(64) gn_bwd_finalize(const float* __restrict__ part, const void* __restrict__ gamma,
+                                                      int param_dtype, float* __restrict__ coef, float* __restrict__ dgamma,
+                                                      float* __restrict__ dbeta, int N, int C, int G, int nsplit, float m) {
+  const int b = blockIdx.x;
+  const int cg = C / G;
+  if (b < N * G) {
+    const int n = b / G, g = b - n * G;
+    float s1 = 0.f, s2 = 0.f;
+    const int total = cg * nsplit;
+    for (int i = threadIdx.x; i < total; i += 64) {
+      const int cc = i / nsplit, sp = i - cc * nsplit;
+      const int c = g * cg + cc;
+      const float w = load_param(gamma, param_dtype, c, 1.f);
+      const float* p = part + ((int64_t)n * nsplit + sp) * 2 * C;
+      s1 = fmaf(w, p[c], s1);
+      s2 = fmaf(w, p[C + c], s2);
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (threadIdx.x == 0) {
+      coef[(n * G + g) * 2] = s2 / m;
+      coef[(n * G + g) * 2 + 1] = s1 / m;
+    }
+  } else {
+    const int c = b - N * G;
+    float s1 = 0.f, s2 = 0.f;
+    const int total = N * nsplit;
+    for (int i = threadIdx.x; i < total; i += 64) {
+      const float* p = part + (int64_t)i * 2 * C;
+      s1 += p[c];
+      s2 += p[C + c];
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (threadIdx.x == 0) {
+      if (dgamma != nullptr) dgamma[c] = s1;
+      if (dbeta != nullptr) dbeta[c] = s2;
+    }
+  }
+}
+
+// dx = rstd * (dy'*gamma - A - xhat*B)   (ScaFFold/unet/triton_group_norm.py:908-1043)
+template <typename T, typename TG>
+__global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const TG* __restrict__ dy, T* __restrict__ dx,
+                                                const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                const void* __restrict__ gamma, const void* __restrict__ beta, int param_dtype,
+                                                const float* __restrict__ coef, int64_t S, int C, int G, int tpr, int rpp,
+                                                int64_t rows_per_split, int relu) {
+  constexpr int V = VecOf<T>::N;
+  const int tid = threadIdx.x;
+  const int n = blockIdx.y;
+  const int cg = C / G;
+  const int r = tid / tpr, cv = tid - r * tpr;
+  if (r >= rpp) return;
+  float mu[V], rs[V], ga[V], be[V], ca[V], cb[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int c = cv * V + e;
+    const int g = c / cg;
+    mu[e] = mean[n * G + g];
+    rs[e] = rstd[n * G + g];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
+    ca[e] = coef[(n * G + g) * 2];
+    cb[e] = coef[(n * G + g) * 2 + 1];
+  }
+  const int64_t base = (int64_t)n * S * C + cv * V;
+  const T* xs = x + base;
+  const TG* gs = dy + base;
+  T* ds = dx + base;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  for (; row + step < end; row += 2 * step) {
+    float f[2][V], g[2][V];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      Ld<T, V>::run(xs + (row + u * step) * C, f[u]);
+      Ld<TG, V>::run(gs + (row + u * step) * C, g[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      float o[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float xh = (f[u][e] - mu[e]) * rs[e];
+        float d = g[u][e];
+        if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
+        // the product is rounded on its own (no contraction) so that a one-element group, whose mean of
+        // dy*gamma is that same rounded product, cancels to an exact zero
+        o[e] = rs[e] * ((__fmul_rn(d, ga[e]) - ca[e]) - xh * cb[e]);
+      }
+      St<T, V>::run(ds + (row + u * step) * C, o);
+    }
+  }
+  for (; row < end; row += step) {
+    float f[V], g[V], o[V];
+    Ld<T, V>::run(xs + row * C, f);
+    Ld<TG, V>::run(gs + row * C, g);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float xh = (f[e] - mu[e]) * rs[e];
+      float d = g[e];
+      if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
+      o[e] = rs[e] * ((__fmul_rn(d, ga[e]) - ca[e]) - xh * cb[e]);
+    }
+    St<T, V>::run(ds + row * C, o);
+  }
+}
+
+// ---- scalar path: one workgroup per (group, sample) ---------------------------------------
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  __syncthreads();
+  red[threadIdx.x] = v;
+  __syncthreads();
+  for (int s = kBlock / 2; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+    __syncthreads();
+  }
+  return red[0];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) gn_scalar_stats(const T* __restrict__ x, float* __restrict__ mean,
+                                                          float* __restrict__ rstd, int64_t S, int C, int G, float eps) {
+  __shared__ float red[kBlock];
+  const int g = blockIdx.x, n = blockIdx.y;
+  const int cg = C / G;
+  const T* xs = x + (int64_t)n * S * C + g * cg;
+  const int64_t m = S * cg;
+  // shift: mean over the first voxels
+  const int64_t km = (S < kShiftRows ? S : kShiftRows) * cg;
+  float k = 0.f;
+  for (int64_t i = threadIdx.x; i < km; i += kBlock) k += to_float(xs[(i / cg) * C + i % cg]);
+  const float K = block_sum(k, red) / (float)km;
+  float s1 = 0.f, s2 = 0.f;
+  for (int64_t i = threadIdx.x; i < m; i += kBlock) {
+    const float d = to_float(xs[(i / cg) * C + i % cg]) - K;
+    s1 += d;
+    s2 = fmaf(d, d, s2);
+  }
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  if (threadIdx.x == 0) {
+    const float d = s1 / (float)m;
+    float var = s2 / (float)m - d * d;
+    var = var < 0.f ? 0.f : var;
+    mean[n * G + g] = K + d;
+    rstd[n * G + g] = 1.f / sqrtf(var + eps);
+  }
+}
+
+template <typename T, typename TO>
+__global__ void __launch_bounds__(kBlock) gn_scalar_normalize(const T* __restrict__ x, TO* __restrict__ y,
+                                                              const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                              const void* __restrict__ gamma, const void* __restrict__ beta,
+                                                              int param_dtype, int64_t S, int C, int G, int64_t total, int relu) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % C);
+  const int n = (int)(i / ((int64_t)S * C));
+  const int g = c / (C / G);
+  const float xh = (to_float(x[i]) - mean[n * G + g]) * rstd[n * G + g];
+  const float v = fmaf(xh, load_param(gamma, param_dtype, c, 1.f), load_param(beta, param_dtype, c, 0.f));
+  y[i] = elem<TO>::from_float(relu ? relu_keep_nan(v) : v);
+}
+
+// Per (group, sample): per-channel sums into chan[n][2][C], then coef[n][g].
+template <typename T, typename TG>
+__global__ void __launch_bounds__(kBlock) gn_scalar_bwd_sums(const T* __restrict__ x, const TG* __restrict__ dy,
+                                                             const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                             const void* __restrict__ gamma, const void* __restrict__ beta,
+                                                             int param_dtype, float* __restrict__ chan, float* __restrict__ coef,
+                                                             int64_t S, int C, int G, int relu) {
+  __shared__ float red[kBlock];
+  const int g = blockIdx.x, n = blockIdx.y;
+  const int cg = C / G;
+  const float mu = mean[n * G + g], rs = rstd[n * G + g];
+  float a1 = 0.f, a2 = 0.f;
+  for (int cc = 0; cc < cg; ++cc) {
+    const int c = g * cg + cc;
+    const float w = load_param(gamma, param_dtype, c, 1.f), b = load_param(beta, param_dtype, c, 0.f);
+    const T* xs = x + (int64_t)n * S * C + c;
+    const TG* gs = dy + (int64_t)n * S * C + c;
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t s = threadIdx.x; s < S; s += kBlock) {
+      const float xh = (to_float(xs[s * C]) - mu) * rs;
+      float d = to_float(gs[s * C]);
+      if (relu) d = fmaf(xh, w, b) <= 0.f ? 0.f : d;
+      s1 = fmaf(d, xh, s1);
+      s2 += d;
+    }
+    s1 = block_sum(s1, red);
+    s2 = block_sum(s2, red);
+    if (threadIdx.x == 0) {
+      chan[((int64_t)n * 2) * C + c] = s1;
+      chan[((int64_t)n * 2 + 1) * C + c] = s2;
+    }
+    a1 = fmaf(w, s1, a1);
+    a2 = fmaf(w, s2, a2);
+  }
+  if (threadIdx.x == 0) {
+    const float m = (float)S * (float)cg;
+    coef[(n * G + g) * 2] = a2 / m;
+    coef[(n * G + g) * 2 + 1] = a1 / m;
+  }
+}
+
+__global__ void __launch_bounds__(kBlock) gn_scalar_dparam(const float* __restrict__ chan, float* __restrict__ dgamma,
+                                                           float* __restrict__ dbeta, int N, int C) {
+  const int c = blockIdx.x * kBlock + threadIdx.x;
+  if (c >= C) return;
+  float s1 = 0.f, s2 = 0.f;
+  for (int n = 0; n < N; ++n) {
+    s1 += chan[((int64_t)n * 2) * C + c];
+    s2 += chan[((int64_t)n * 2 + 1) * C + c];
+  }
+  if (dgamma != nullptr) dgamma[c] = s1;
+  if (dbeta != nullptr) dbeta[c] = s2;
+}
+
+template <typename T, typename TG>
+__global__ void __launch_bounds__(kBlock) gn_scalar_dx(const T* __restrict__ x, const TG* __restrict__ dy, T* __restrict__ dx,
+                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                       const void* __restrict__ gamma, const void* __restrict__ beta,
+                                                       int param_dtype, const float* __restrict__ coef, int64_t S, int C, int G,
+                                                       int64_t total, int relu) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= total) return;
+  const int c = (int)(i % C);
+  const int n = (int)(i / ((int64_t)S * C));
+  const int g = c / (C / G);
+  const float rs = rstd[n * G + g];
+  const float w = load_param(gamma, param_dtype, c, 1.f), b = load_param(beta, param_dtype, c, 0.f);
+  const float xh = (to_float(x[i]) - mean[n * G + g]) * rs;
+  float d = to_float(dy[i]);
+  if (relu) d = fmaf(xh, w, b) <= 0.f ? 0.f : d;
+  dx[i] = elem<T>::from_float(rs * ((__fmul_rn(d, w) - coef[(n * G + g) * 2]) - xh * coef[(n * G + g) * 2 + 1]));
+}
+
+// ---- host-side dispatch --------------------------------------------------------------------
+int check_desc(const sfh_groupnorm_desc* p, int x_dtype) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null descriptor");
+  if (!dtype_ok(x_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad dtype %d", x_dtype);
+  if (p->n < 1 || p->c < 1 || p->spatial < 1 || p->groups < 1 || p->c % p->groups != 0)
+    return fail(SFH_ERR_INVALID, "groupnorm: need N,C,S >= 1 and C %% groups == 0 (N=%d C=%d S=%lld G=%d)", p->n, p->c,
+                (long long)p->spatial, p->groups);
+  if (p->n > 65535) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: N=%d exceeds the grid limit", p->n);
+  return SFH_OK;
+}
+
+bool aligned16(const void* a) { return (reinterpret_cast<uintptr_t>(a) & 15u) == 0; }
+
+size_t fwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
+  return (size_t)p.n * p.groups + (size_t)p.n * pl.nsplit * 2 * p.groups;
+}
+size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
+  // coef[N][G][2] | part[N][nsplit][2][C]   (scalar path: chan[N][2][C] in the part slot)
+  return (size_t)p.n * p.groups * 2 + (size_t)p.n * pl.nsplit * 2 * p.c;
+}
+
+template <typename T, typename TO>
+int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
+              void* y, float* mean, float* rstd, float* ws, hipStream_t st) {
+  const int G = p.groups, C = p.c;
+  const int64_t S = p.spatial;
+  if (!pl.vector) {
+    hipLaunchKernelGGL(gn_scalar_stats<T>, dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, mean, rstd, S, C, G, p.eps);
+    if (int rc = check_launch("gn_scalar_stats")) return rc;
+    const int64_t total = (int64_t)p.n * S * C;
+    if (cdiv(total, kBlock) > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: tensor too large for the scalar path");
+    hipLaunchKernelGGL((gn_scalar_normalize<T, TO>), dim3((unsigned)cdiv(total, kBlock)), dim3(kBlock), 0, st, (const T*)x,
+                       (TO*)y, mean, rstd, gamma, beta, param_dtype, S, C, G, total, p.relu);
+    return check_launch("gn_scalar_normalize");
+  }
+  float* shift = ws;
+  float* part = ws + (size_t)p.n * G;
+  const size_t lds = (size_t)(2 * pl.slots * kBlock + 2 * G) * sizeof(float);
+  const dim3 grid(pl.nsplit, p.n);
+#define SFH_GN_STATS(SL)                                                                                                   \
+  hipLaunchKernelGGL((gn_stats_partial<T, SL>), grid, dim3(kBlock), lds, st, (const T*)x, shift, part, S, C, G, pl.tpr, \
+                     pl.rpp, pl.nsplit, pl.rows_per_split)
+  switch (pl.slots) {
+    case 1: SFH_GN_STATS(1); break;
+    case 2: SFH_GN_STATS(2); break;
+    case 4: SFH_GN_STATS(4); break;
+    default: SFH_GN_STATS(8); break;
+  }
+#undef SFH_GN_STATS
+  if (int rc = check_launch("gn_stats_partial")) return rc;
+  const float m = (float)S * (float)(C / G);
+  hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, pl.nsplit, m, p.eps);
+  if (int rc = check_launch("gn_stats_finalize")) return rc;
+  hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), 0, st, (const T*)x, (TO*)y, mean, rstd, gamma, beta,
+                     param_dtype, S, C, G, pl.tpr, pl.rpp, pl.rows_per_split, p.relu);
+  return check_launch("gn_normalize");
+}
+
+template <typename T, typename TG>
+int bwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* dy, const void* x, const void* gamma,
+              const void* beta, const float* mean, const float* rstd, void* dx, float* dgamma, float* dbeta, float* ws,
+              hipStream_t st) {
+  const int G = p.groups, C = p.c;
+  const int64_t S = p.spatial;
+  float* coef = ws;
+  float* part = ws + (size_t)p.n * G * 2;
+  if (!pl.vector) {
+    hipLaunchKernelGGL((gn_scalar_bwd_sums<T, TG>), dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, (const TG*)dy, mean, rstd,
+                       gamma, beta, param_dtype, part, coef, S, C, G, p.relu);
+    if (int rc = check_launch("gn_scalar_bwd_sums")) return rc;
+    if (dgamma != nullptr || dbeta != nullptr) {
+      hipLaunchKernelGGL(gn_scalar_dparam, dim3((unsigned)cdiv(C, kBlock)), dim3(kBlock), 0, st, part, dgamma, dbeta, p.n, C);
+      if (int rc = check_launch("gn_scalar_dparam")) return rc;
+    }
+    const int64_t total = (int64_t)p.n * S * C;
+    if (cdiv(total, kBlock) > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: tensor too large for the scalar path");
+    hipLaunchKernelGGL((gn_scalar_dx<T, TG>), dim3((unsigned)cdiv(total, kBlock)), dim3(kBlock), 0, st, (const T*)x,
+                       (const TG*)dy, (T*)dx, mean, rstd, gamma, beta, param_dtype, coef, S, C, G, total, p.relu);
+    return check_launch("gn_scalar_dx");
+  }
+  constexpr int V = VecOf<T>::N;
+  const dim3 grid(pl.nsplit, p.n);
+  hipLaunchKernelGGL((gn_bwd_partial<T, TG>), grid, dim3(kBlock), (size_t)2 * V * kBlock * sizeof(float), st, (const T*)x,
+                     (const TG*)dy, mean, rstd, gamma, beta, param_dtype, part, S, C, G, pl.tpr, pl.rpp, pl.nsplit,
+                     pl.rows_per_split, p.relu);
+  if (int rc = check_launch("gn_bwd_partial")) return rc;
+  const float m = (float)S * (float)(C / G);
+  hipLaunchKernelGGL(gn_bwd_finalize, dim3(p.n * G + C), dim3(64), 0, st, part, gamma, param_dtype, coef, dgamma, dbeta, p.n, C,
+                     G, pl.nsplit, m);
+  if (int rc = check_launch("gn_bwd_finalize")) return rc;
+  hipLaunchKernelGGL((gn_dx<T, TG>), grid, dim3(kBlock), 0, st, (const T*)x, (const TG*)dy, (T*)dx, mean, rstd, gamma, beta,
+                     param_dtype, coef, S, C, G, pl.tpr, pl.rpp, pl.rows_per_split, p.relu);
+  return check_launch("gn_dx");
+}
+
+}  // namespace
+}  // namespace sfh
+
+using namespace sfh;
+
+extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype) {
+  if (check_desc(p, x_dtype) != SFH_OK) return 0;
+  // Sized for the vector path whatever the pointer alignment turns out to be.
+  const GnPlan pl = make_plan(*p, x_dtype, true);
+  return align_up(fwd_ws_floats(*p, pl) * sizeof(float), 256);
+}
+
+extern "C" int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
+                                 const void* gamma, const void* beta, void* y, float* mean, float* rstd, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  if (int rc = check_desc(p, x_dtype)) return rc;
+  if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
+  if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
+  const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(y));
+  if (pl.vector) {
+    const size_t need = fwd_ws_floats(*p, pl) * sizeof(float);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "groupnorm fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  float* ws = (float*)workspace;
+#define SFH_GN_FWD(TX, TY) return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, mean, rstd, ws, st)
+  if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
+  if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
+  if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
+  if (x_dtype == SFH_FP16 && y_dtype == SFH_FP16) SFH_GN_FWD(fp16_t, fp16_t);
+  if (x_dtype == SFH_FP16 && y_dtype == SFH_FP32) SFH_GN_FWD(fp16_t, float);
+  if (x_dtype == SFH_FP16 && y_dtype == SFH_BF16) SFH_GN_FWD(fp16_t, bf16_t);
+  if (x_dtype == SFH_FP32 && y_dtype == SFH_FP32) SFH_GN_FWD(float, float);
+  if (x_dtype == SFH_FP32 && y_dtype == SFH_BF16) SFH_GN_FWD(float, bf16_t);
+  SFH_GN_FWD(float, fp16_t);
+#undef SFH_GN_FWD
+}
+
+extern "C" size_t sfh_groupnorm_bwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype) {
+  if (check_desc(p, x_dtype) != SFH_OK) return 0;
+  const GnPlan pl = make_plan(*p, x_dtype, true);
+  return align_up(bwd_ws_floats(*p, pl) * sizeof(float), 256);
+}
+
+extern "C" int sfh_groupnorm_bwd(const sfh_groupnorm_desc* p, int x_dtype, int dy_dtype, int param_dtype, const void* dy,
+                                 const void* x, const void* gamma, const void* beta, const float* mean, const float* rstd,
+                                 void* dx, float* dgamma, float* dbeta, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = check_desc(p, x_dtype)) return rc;
+  if (!dtype_ok(dy_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad gradient/param dtype");
+  if (dy_dtype != x_dtype && dy_dtype != SFH_FP32)
+    return fail(SFH_ERR_UNSUPPORTED, "groupnorm bwd: the gradient must have the input's dtype or fp32");
+  if (dy == nullptr || x == nullptr || dx == nullptr || mean == nullptr || rstd == nullptr)
+    return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
+  const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(dy) && aligned16(dx));
+  const size_t need = bwd_ws_floats(*p, pl) * sizeof(float);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "groupnorm bwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  hipStream_t st = (hipStream_t)stream;
+  float* ws = (float*)workspace;
+#define SFH_GN_BWD(TX, TG) \
+  return bwd_typed<TX, TG>(*p, pl, param_dtype, dy, x, gamma, beta, mean, rstd, dx, dgamma, dbeta, ws, st)
+  if (x_dtype == SFH_BF16 && dy_dtype == SFH_BF16) SFH_GN_BWD(bf16_t, bf16_t);
+  if (x_dtype == SFH_BF16) SFH_GN_BWD(bf16_t, float);
+  if (x_dtype == SFH_FP16 && dy_dtype == SFH_FP16) SFH_GN_BWD(fp16_t, fp16_t);
+  if (x_dtype == SFH_FP16) SFH_GN_BWD(fp16_t, float);
+  SFH_GN_BWD(float, float);
+#undef SFH_GN_BWD
+}

@@ -1,0 +1,19 @@
+// Host-side interface of the MFMA weight-gradient kernel (3x3x3, stride 1, bf16 / fp16).
+#pragma once
+#include "common.hpp"
+
+namespace sfh {
+
+struct WgradArgs {
+  int n, cin, id, ih, iw;
+  int cout, od, oh, ow;
+  int pd, ph, pw;
+};
+
+bool mfma_wgrad_supported(const WgradArgs& a, int dtype);
+// Number of fp32 partial slices [Cout][27][Cin]; a pure function of the shape.
+int mfma_wgrad_splits(const WgradArgs& a);
+size_t mfma_wgrad_workspace_bytes(const WgradArgs& a);
+int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, void* workspace, hipStream_t st);
+
+}  // namespace sfh

@@ -1,0 +1,307 @@
+"""Channels-last GroupNorm (+ fused ReLU) forward / backward on the HIP library.
+
+Mirrors ``ScaFFold/unet/triton_group_norm.py``: the dispatcher ops
+``torch.ops.scaffold_gn.group_norm`` / ``group_norm_backward`` (:1339-1436) with fake kernels and
+an autograd formula (:1439-1479), the gate ``is_supported`` (:1541) and the public
+``group_norm`` function (there called ``triton_group_norm``, :1610; the old name is kept as an
+alias so callers can switch by changing an import).
+
+Contract kept from the reference:
+
+* statistics and the normalisation are fp32 whatever the storage dtype; the result is rounded once;
+* ``out_dtype=MATCH_STOCK_DTYPE`` reproduces ``F.group_norm`` (fp32 inside autocast, the input's
+  dtype outside), ``None`` means the input's dtype, an explicit dtype is honoured;
+* ``activation="relu"`` is fused into the store and the backward gates on the recomputed
+  pre-activation; NaN propagates like ``F.relu`` / ``threshold_backward``;
+* ``mean`` / ``rstd`` are non-differentiable backward state; the backward op has no autograd
+  formula, so double backward raises;
+* every shape ``F.group_norm`` rejects is rejected with the same exception type.
+
+Difference from the reference: inputs the gate refuses are **not** routed to ``F.group_norm``.
+``group_norm`` raises ``NotImplementedError`` for them -- this package has no second backend.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import GroupNormDesc
+
+__all__ = [
+    "group_norm",
+    "triton_group_norm",
+    "is_supported",
+    "SUPPORTED_ACTIVATIONS",
+    "SUPPORTED_DTYPES",
+    "MATCH_STOCK_DTYPE",
+]
+
+SUPPORTED_ACTIVATIONS = (None, "relu")
+SUPPORTED_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+_CL3D = torch.channels_last_3d
+
+
+def _one_value_per_channel(input, num_groups: int) -> bool:
+    """``F.group_norm`` raises for ``N * (C/G) * S == 1``, i.e. numel == C == num_groups."""
+    channels = input.shape[1]
+    return channels == num_groups and input.numel() == channels
+
+
+def _validate(input, num_groups, weight, bias, activation) -> None:
+    if activation not in SUPPORTED_ACTIVATIONS:
+        raise ValueError(f"activation must be one of {SUPPORTED_ACTIVATIONS}, got {activation!r}")
+    if input.dim() != 5:
+        raise ValueError(f"expected a 5-D NCDHW tensor, got {tuple(input.shape)}")
+    if num_groups <= 0 or input.shape[1] % num_groups != 0:
+        raise ValueError(f"num_channels={input.shape[1]} is not divisible by num_groups={num_groups}")
+    if _one_value_per_channel(input, num_groups):
+        raise ValueError(
+            f"Expected more than 1 value per channel when training, got input size {tuple(input.shape)} "
+            f"with num_groups={num_groups}"
+        )
+    if input.dtype not in SUPPORTED_DTYPES:
+        raise ValueError(f"unsupported input dtype {input.dtype}")
+    if not input.is_contiguous(memory_format=_CL3D):
+        raise ValueError("input must be channels_last_3d-contiguous")
+    for name, t in (("weight", weight), ("bias", bias)):
+        if t is not None and t.numel() != input.shape[1]:
+            raise ValueError(f"{name} has {t.numel()} elements, expected {input.shape[1]}")
+
+
+def _param_dtype(weight, bias, input) -> torch.dtype:
+    for t in (weight, bias):
+        if t is not None:
+            return t.dtype
+    return input.dtype
+
+
+def _desc(input, num_groups: int, eps: float, activation) -> GroupNormDesc:
+    n, c = int(input.shape[0]), int(input.shape[1])
+    spatial = int(input.shape[2]) * int(input.shape[3]) * int(input.shape[4])
+    return GroupNormDesc(n, c, int(num_groups), 1 if activation == "relu" else 0, spatial, float(eps))
+
+
+@torch.library.custom_op("scaffold_gn::group_norm", mutates_args=(), device_types="cuda")
+def _group_norm_op(
+    input: torch.Tensor,
+    num_groups: int,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+    activation: Optional[str],
+    out_dtype: Optional[torch.dtype],
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Channels-last GroupNorm forward: ``(output, mean, rstd)``; mean/rstd are ``(N, G)`` fp32."""
+    _validate(input, num_groups, weight, bias, activation)
+    weight = None if weight is None else weight.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    if weight is not None and bias is not None and weight.dtype != bias.dtype:
+        bias = bias.to(weight.dtype)
+    odt = out_dtype or input.dtype
+    n = int(input.shape[0])
+    out = torch.empty_like(input, dtype=odt)  # keeps the channels_last_3d strides
+    mean = torch.empty((n, num_groups), dtype=torch.float32, device=input.device)
+    rstd = torch.empty((n, num_groups), dtype=torch.float32, device=input.device)
+    if input.numel() == 0:
+        return out, mean, rstd
+    L = _lib.lib()
+    desc = _desc(input, num_groups, eps, activation)
+    xcode = _lib.dtype_code(input.dtype)
+    with torch.cuda.device(input.device):
+        ws = _lib.workspace(L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
+        rc = L.sfh_groupnorm_fwd(
+            ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+            _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
+            _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+    _lib.check(rc, "group_norm")
+    return out, mean, rstd
+
+
+@_group_norm_op.register_fake
+def _(input, num_groups, weight, bias, eps, activation, out_dtype):
+    out = torch.empty_like(input, dtype=out_dtype or input.dtype)
+    mean = input.new_empty((input.shape[0], num_groups), dtype=torch.float32)
+    rstd = input.new_empty((input.shape[0], num_groups), dtype=torch.float32)
+    return out, mean, rstd
+
+
+@torch.library.custom_op("scaffold_gn::group_norm_backward", mutates_args=(), device_types="cuda")
+def _group_norm_backward_op(
+    grad_out: torch.Tensor,
+    input: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    mean: torch.Tensor,
+    rstd: torch.Tensor,
+    num_groups: int,
+    activation: Optional[str],
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(d_input, d_weight, d_bias)``; the parameter gradients are empty when the parameter is None.
+    ``d_input`` has the input's dtype and is channels_last_3d."""
+    if not grad_out.is_contiguous(memory_format=_CL3D):
+        grad_out = grad_out.contiguous(memory_format=_CL3D)
+    if not input.is_contiguous(memory_format=_CL3D):
+        input = input.contiguous(memory_format=_CL3D)
+    if grad_out.dtype != input.dtype and grad_out.dtype != torch.float32:
+        grad_out = grad_out.to(input.dtype)
+    weight = None if weight is None else weight.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    if weight is not None and bias is not None and weight.dtype != bias.dtype:
+        bias = bias.to(weight.dtype)
+    channels = int(input.shape[1])
+    d_input = torch.empty_like(input, memory_format=_CL3D)
+    dw32 = torch.empty(channels, dtype=torch.float32, device=input.device) if weight is not None else None
+    db32 = torch.empty(channels, dtype=torch.float32, device=input.device) if bias is not None else None
+    if input.numel() > 0:
+        L = _lib.lib()
+        desc = _desc(input, num_groups, 0.0, activation)
+        xcode = _lib.dtype_code(input.dtype)
+        with torch.cuda.device(input.device):
+            ws = _lib.workspace(L.sfh_groupnorm_bwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
+            rc = L.sfh_groupnorm_bwd(
+                ctypes.byref(desc), xcode, _lib.dtype_code(grad_out.dtype),
+                _lib.dtype_code(_param_dtype(weight, bias, input)), _lib.ptr(grad_out), _lib.ptr(input), _lib.ptr(weight),
+                _lib.ptr(bias), _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(d_input), _lib.ptr(dw32), _lib.ptr(db32),
+                _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+        _lib.check(rc, "group_norm_backward")
+    else:
+        if dw32 is not None:
+            dw32.zero_()
+        if db32 is not None:
+            db32.zero_()
+    d_weight = input.new_empty(0, dtype=torch.float32) if weight is None else dw32.to(weight.dtype)
+    d_bias = input.new_empty(0, dtype=torch.float32) if bias is None else db32.to(bias.dtype)
+    return d_input, d_weight, d_bias
+
+
+@_group_norm_backward_op.register_fake
+def _(grad_out, input, weight, bias, mean, rstd, num_groups, activation):
+    channels = input.shape[1]
+    d_input = torch.empty_like(input, memory_format=_CL3D)
+    d_weight = input.new_empty(channels if weight is not None else 0,
+                               dtype=weight.dtype if weight is not None else torch.float32)
+    d_bias = input.new_empty(channels if bias is not None else 0,
+                             dtype=bias.dtype if bias is not None else torch.float32)
+    return d_input, d_weight, d_bias
+
+
+def _setup_context(ctx, inputs, output):
+    input, num_groups, weight, bias, eps, activation, out_dtype = inputs
+    _out, mean, rstd = output
+    ctx.mark_non_differentiable(mean, rstd)
+    ctx.save_for_backward(input, weight, bias, mean, rstd)
+    ctx.num_groups = num_groups
+    ctx.activation = activation
+    ctx.needs = (ctx.needs_input_grad[0], ctx.needs_input_grad[2], ctx.needs_input_grad[3])
+
+
+def _autograd_backward(ctx, grad_out, grad_mean, grad_rstd):
+    input, weight, bias, mean, rstd = ctx.saved_tensors
+    need_x, need_w, need_b = ctx.needs
+    if not (need_x or need_w or need_b):
+        return None, None, None, None, None, None, None
+    d_input, d_weight, d_bias = torch.ops.scaffold_gn.group_norm_backward(
+        grad_out, input, weight, bias, mean, rstd, ctx.num_groups, ctx.activation
+    )
+    return (d_input if need_x else None, None, d_weight if need_w else None, d_bias if need_b else None, None, None, None)
+
+
+torch.library.register_autograd("scaffold_gn::group_norm", _autograd_backward, setup_context=_setup_context)
+
+
+# ---------------------------------------------------------------------------------------------
+# public API
+# ---------------------------------------------------------------------------------------------
+def _autocast_active(input: torch.Tensor) -> bool:
+    try:
+        return bool(torch.is_autocast_enabled(input.device.type))
+    except (RuntimeError, TypeError):
+        return False
+
+
+class _MatchStockDtype:
+    __slots__ = ()
+
+    def __repr__(self):
+        return "MATCH_STOCK_DTYPE"
+
+
+#: default ``out_dtype``: what ``F.group_norm`` would return (fp32 inside autocast, else the input's dtype)
+MATCH_STOCK_DTYPE = _MatchStockDtype()
+
+
+def _resolve_out_dtype(input: torch.Tensor, out_dtype) -> Optional[torch.dtype]:
+    if out_dtype is MATCH_STOCK_DTYPE:
+        if input.dtype is not torch.float32 and _autocast_active(input):
+            return torch.float32
+        return None
+    return out_dtype
+
+
+def is_supported(input, num_groups: int, weight=None, bias=None, activation: Optional[str] = None) -> bool:
+    """Whether the HIP kernels serve this call: a 5-D CUDA tensor, ``channels_last_3d``-contiguous,
+    fp32/bf16/fp16, C divisible by ``num_groups``, affine parameters of the input's dtype (or fp32 under
+    autocast), and not one of the shapes ``F.group_norm`` itself rejects.  Total and side-effect free."""
+    try:
+        if activation not in SUPPORTED_ACTIVATIONS:
+            return False
+        if not isinstance(input, torch.Tensor) or input.device.type != "cuda":
+            return False
+        if input.dim() != 5 or input.dtype not in SUPPORTED_DTYPES:
+            return False
+        if not isinstance(num_groups, int) or isinstance(num_groups, bool) or num_groups <= 0:
+            return False
+        channels = input.shape[1]
+        if channels % num_groups != 0 or input.numel() == 0:
+            return False
+        if _one_value_per_channel(input, num_groups):
+            return False
+        if not input.is_contiguous(memory_format=_CL3D):
+            return False
+        for t in (weight, bias):
+            if t is None:
+                continue
+            if not isinstance(t, torch.Tensor) or t.dim() != 1 or t.numel() != channels or t.device != input.device:
+                return False
+            if t.dtype is not input.dtype:
+                if t.dtype is not torch.float32 or not _autocast_active(input):
+                    return False
+        return True
+    except (TypeError, ValueError, AttributeError):
+        return False
+
+
+def group_norm(input, num_groups: int, weight=None, bias=None, eps: float = 1e-5, activation: Optional[str] = None, *,
+               out_dtype=MATCH_STOCK_DTYPE):
+    """``F.group_norm(input, num_groups, weight, bias, eps)`` (then ``F.relu`` when ``activation="relu"``)
+    on a channels_last_3d CUDA tensor.  Raises ``NotImplementedError`` for calls :func:`is_supported` refuses."""
+    if activation not in SUPPORTED_ACTIVATIONS:
+        raise ValueError(f"activation must be one of {SUPPORTED_ACTIVATIONS}, got {activation!r}")
+    if not (out_dtype is MATCH_STOCK_DTYPE or out_dtype is None or out_dtype in SUPPORTED_DTYPES):
+        raise ValueError(
+            f"out_dtype must be MATCH_STOCK_DTYPE, None (the input's dtype) or one of {SUPPORTED_DTYPES}, got {out_dtype!r}"
+        )
+    if not is_supported(input, num_groups, weight, bias, activation):
+        if isinstance(input, torch.Tensor) and input.dim() == 5 and input.is_cuda:
+            # shapes F.group_norm rejects keep F.group_norm's own exception type
+            if isinstance(num_groups, int) and num_groups > 0 and input.shape[1] % num_groups == 0 \
+                    and _one_value_per_channel(input, num_groups):
+                raise ValueError(
+                    f"Expected more than 1 value per channel when training, got input size {tuple(input.shape)}"
+                )
+        raise NotImplementedError(
+            f"unsupported group_norm call: input={tuple(getattr(input, 'shape', ()))}/{getattr(input, 'dtype', None)} on "
+            f"{getattr(input, 'device', None)}, num_groups={num_groups}; needs a channels_last_3d CUDA tensor"
+        )
+    out, _mean, _rstd = torch.ops.scaffold_gn.group_norm(
+        input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype)
+    )
+    return out
+
+
+#: the reference's name for :func:`group_norm`
+triton_group_norm = group_norm

@@ -1,0 +1,176 @@
+"""Drop-in ``nn.Module``s over the HIP ops: ``FastConv3d``, ``FastConvTranspose3d``, ``FastGroupNorm``.
+
+They stand where the reference's adapters stand (``ScaFFold/unet/conv3d.py:1235-1479,1790-1904``,
+``ScaFFold/unet/group_norm.py:556-808``) and keep their contract:
+
+* same parameters under the same names and no buffers, so ``state_dict`` keys and shapes are
+  those of ``nn.Conv3d`` / ``nn.ConvTranspose3d`` / ``nn.GroupNorm`` in both directions;
+* under ``torch.autocast`` only exactly-fp32 operands are cast, and the cast is an ordinary
+  autograd node *outside* the kernel's node, so an fp32 parameter receives an fp32 gradient
+  (``conv3d.py:446-480``);
+* the autograd nodes save ``(x, weight)`` after the launch, compute the bias gradient as
+  ``grad_output.sum((0, 2, 3, 4))`` (``conv3d.py:1231``) and are once-differentiable: a second
+  differentiation raises instead of returning zeros;
+* ``FastGroupNorm`` returns its input's dtype (not fp32) inside autocast and applies the ReLU
+  when ``activation="relu"``.
+
+What is deliberately absent: the reference's fallback ladder (Triton -> MIOpen, compiled ->
+eager), its latches, the hardware allowlist and the mesh-wide vote.  There is one backend here;
+a call it does not serve raises ``NotImplementedError``.
+
+``FastConv3d.shard_halo`` reproduces the compute shape of one DistConv depth shard on a single
+GPU: the input is extended by one voxel of (zero) halo on each depth face and the convolution
+runs with depth padding 0, which is what the reference's own halo exchange hands its kernel
+(``conv3d.py:648-677,748-792``); with no neighbour the halo is zero and the result equals the
+ordinary padded convolution.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.autograd.function import once_differentiable
+
+from . import conv3d as _c3
+from . import groupnorm as _gn
+from . import transposed as _ct
+
+__all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand"]
+
+_CL3D = torch.channels_last_3d
+
+
+def autocast_dtype(tensor: torch.Tensor) -> Optional[torch.dtype]:
+    """The dtype autocast would cast a convolution's operands to on this device, or ``None``."""
+    try:
+        if not torch.is_autocast_enabled(tensor.device.type):
+            return None
+        return torch.get_autocast_dtype(tensor.device.type)
+    except (RuntimeError, TypeError):
+        return None
+
+
+def cast_operand(tensor: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
+    """ATen's ``cached_cast`` rule: only an exactly-fp32 tensor is narrowed."""
+    if tensor is None or dtype is None or tensor.dtype is not torch.float32:
+        return tensor
+    return tensor.to(dtype)
+
+
+class _Conv3dFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, stride, padding, dilation):
+        y = _c3.conv3d_forward(x, weight, bias, stride, padding, dilation, 1)
+        ctx.save_for_backward(x, weight)
+        ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        x, weight = ctx.saved_tensors
+        stride, padding, dilation, has_bias, bias_dtype = ctx.conv_args
+        needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
+        grad_output = grad_output.contiguous(memory_format=_CL3D)
+        grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1) if needs_x else None
+        grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1) if needs_w else None
+        grad_b = grad_output.sum(dim=(0, 2, 3, 4)).to(bias_dtype) if (has_bias and needs_b) else None
+        return grad_x, grad_w, grad_b, None, None, None
+
+
+class _ConvTranspose3dFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, stride):
+        y = _ct.conv_transpose3d_forward(x, weight, bias, stride, 0, 0, 1, 1)
+        ctx.save_for_backward(x, weight)
+        ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype)
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_output):
+        x, weight = ctx.saved_tensors
+        stride, has_bias, bias_dtype = ctx.conv_args
+        needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
+        grad_output = grad_output.contiguous(memory_format=_CL3D)
+        grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1) if needs_x else None
+        grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1) if needs_w else None
+        grad_b = grad_output.sum(dim=(0, 2, 3, 4)).to(bias_dtype) if (has_bias and needs_b) else None
+        return grad_x, grad_w, grad_b, None
+
+
+def _wants_grad(*tensors) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
+
+
+class FastConv3d(nn.Conv3d):
+    """``nn.Conv3d`` served by the HIP kernels.  ``__init__`` is inherited unchanged."""
+
+    #: emulate one depth shard: zero halo on both depth faces + depth padding 0
+    shard_halo = False
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.padding_mode != "zeros" or isinstance(self.padding, str):
+            raise NotImplementedError(f"FastConv3d: padding_mode={self.padding_mode!r} padding={self.padding!r}")
+        dt = autocast_dtype(x)
+        x = cast_operand(x, dt)
+        w = cast_operand(self.weight, dt)
+        b = cast_operand(self.bias, dt)
+        padding = tuple(self.padding)
+        if self.shard_halo and padding[0] > 0:
+            # (N, C, D, H, W): extend D by the halo the neighbours would have sent
+            x = F.pad(x, (0, 0, 0, 0, padding[0], padding[0]))
+            padding = (0, padding[1], padding[2])
+        x = x.contiguous(memory_format=_CL3D)
+        gate = _c3.is_supported_all if _wants_grad(x, w, b) else _c3.is_supported
+        if not gate(x, w, b, self.stride, padding, self.dilation, self.groups):
+            raise NotImplementedError(
+                f"FastConv3d: not served: x={tuple(x.shape)}/{x.dtype} on {x.device}, weight={tuple(w.shape)}/{w.dtype}, "
+                f"stride={self.stride} padding={padding} dilation={self.dilation} groups={self.groups}"
+            )
+        return _Conv3dFn.apply(x, w, b, tuple(self.stride), padding, tuple(self.dilation))
+
+
+class FastConvTranspose3d(nn.ConvTranspose3d):
+    """``nn.ConvTranspose3d`` at ``kernel == stride`` served by the HIP kernels."""
+
+    def forward(self, x: torch.Tensor, output_size=None) -> torch.Tensor:
+        if output_size is not None:
+            raise NotImplementedError("FastConvTranspose3d: output_size is not supported")
+        dt = autocast_dtype(x)
+        x = cast_operand(x, dt)
+        w = cast_operand(self.weight, dt)
+        b = cast_operand(self.bias, dt)
+        x = x.contiguous(memory_format=_CL3D)
+        gate = _ct.is_supported_transposed_all if _wants_grad(x, w, b) else _ct.is_supported_transposed
+        if not gate(x, w, b, self.stride, self.padding, self.output_padding, self.dilation, self.groups):
+            raise NotImplementedError(
+                f"FastConvTranspose3d: not served: x={tuple(x.shape)}/{x.dtype} on {x.device}, weight={tuple(w.shape)}, "
+                f"stride={self.stride} padding={self.padding} output_padding={self.output_padding} "
+                f"dilation={self.dilation} groups={self.groups}"
+            )
+        return _ConvTranspose3dFn.apply(x, w, b, tuple(self.stride))
+
+
+class FastGroupNorm(nn.GroupNorm):
+    """``nn.GroupNorm`` (+ optional fused ReLU) served by the HIP kernels; output dtype = input dtype."""
+
+    activation = None  # class-level default: not a parameter, buffer or state-dict key
+
+    def __init__(self, num_groups, num_channels, eps=1e-5, affine=True, device=None, dtype=None, activation=None):
+        super().__init__(num_groups, num_channels, eps=eps, affine=affine, device=device, dtype=dtype)
+        if activation not in _gn.SUPPORTED_ACTIVATIONS:
+            raise ValueError(f"activation must be one of {_gn.SUPPORTED_ACTIVATIONS}, got {activation!r}")
+        self.activation = activation
+
+    def extra_repr(self) -> str:
+        base = super().extra_repr()
+        return base if self.activation is None else f"{base}, activation={self.activation!r}"
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.dim() == 5 and not x.is_contiguous(memory_format=_CL3D):
+            x = x.contiguous(memory_format=_CL3D)
+        return _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None)

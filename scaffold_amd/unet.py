@@ -1,0 +1,170 @@
+"""The ScaFFold 3D U-Net over the HIP ops, with the widths BASELINE's configs need as arguments.
+
+Structure, child names and therefore ``state_dict`` keys follow the reference model
+(``ScaFFold/unet/unet_model.py:27-162``, ``ScaFFold/unet/unet_parts.py:107-240``):
+``down_list[0]`` is a DoubleConv, ``down_list[i]`` is MaxPool3d(2) + DoubleConv, ``up_list[i]`` is
+ConvTranspose3d(k=2, s=2) -> pad -> skip concat -> DoubleConv, ``up_list[-1]`` is the 1x1x1 head.
+DoubleConv is ``(conv3 -> GroupNorm(+ReLU) -> Identity) x 2``: the ReLU is fused into the GroupNorm
+and ``nn.Identity`` keeps the positional names of a conv/norm/relu Sequential.
+
+The reference hard-codes a base width of 64 (``unet_model.py:68``); here ``base_width`` is an
+argument (32 for the benchmark configuration).  ``stock=True`` builds the identical architecture
+from ``nn.Conv3d`` / ``nn.ConvTranspose3d`` / ``nn.GroupNorm`` + ``F.relu``: the comparison arm of the
+parity tests, with interchangeable state dicts.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+import torch.utils.checkpoint
+
+from .modules import FastConv3d, FastConvTranspose3d, FastGroupNorm, autocast_dtype
+
+__all__ = ["UNet", "DoubleConv", "Down", "Up", "OutConv", "skip_concat"]
+
+
+class _StockGroupNormRelu(nn.GroupNorm):
+    """Stock arm: ``F.group_norm`` then ``F.relu``, returned in the input's dtype (the contract of
+    ``FastGroupNorm``, ``ScaFFold/unet/group_norm.py:572-599``)."""
+
+    activation = None
+
+    def __init__(self, num_groups, num_channels, eps=1e-5, affine=True, device=None, dtype=None, activation=None):
+        super().__init__(num_groups, num_channels, eps=eps, affine=affine, device=device, dtype=dtype)
+        self.activation = activation
+
+    def forward(self, x):
+        y = F.group_norm(x, self.num_groups, self.weight, self.bias, self.eps)
+        if self.activation == "relu":
+            y = F.relu(y)
+        return y if y.dtype is x.dtype else y.to(x.dtype)
+
+
+def _conv3d(stock, cin, cout, **kw):
+    return (nn.Conv3d if stock else FastConv3d)(cin, cout, **kw)
+
+
+def _conv_transpose3d(stock, cin, cout, **kw):
+    return (nn.ConvTranspose3d if stock else FastConvTranspose3d)(cin, cout, **kw)
+
+
+def _group_norm(stock, groups, channels, activation=None):
+    if channels % groups != 0:
+        raise ValueError(f"group_norm_groups={groups} must evenly divide num_channels={channels}")
+    return (_StockGroupNormRelu if stock else FastGroupNorm)(groups, channels, activation=activation)
+
+
+def _consumer_dtype(*tensors):
+    """The dtype the convolution after a concat will read: autocast's when it narrows, else the widest."""
+    dtype = tensors[0].dtype
+    for t in tensors[1:]:
+        dtype = torch.promote_types(dtype, t.dtype)
+    ac = autocast_dtype(tensors[0])
+    if ac is None or dtype is not torch.float32:
+        return dtype
+    return ac
+
+
+def skip_concat(skip, upsampled):
+    """``torch.cat([skip, upsampled], 1)`` at the consumer's dtype (``unet_parts.py:107-120``)."""
+    dtype = _consumer_dtype(skip, upsampled)
+    return torch.cat([skip.to(dtype), upsampled.to(dtype)], dim=1)
+
+
+class DoubleConv(nn.Module):
+    def __init__(self, in_channels, out_channels, group_norm_groups, mid_channels=None, stock=False):
+        super().__init__()
+        mid = mid_channels or out_channels
+        self.double_conv = nn.Sequential(
+            _conv3d(stock, in_channels, mid, kernel_size=3, padding=1, bias=False),
+            _group_norm(stock, group_norm_groups, mid, activation="relu"),
+            nn.Identity(),
+            _conv3d(stock, mid, out_channels, kernel_size=3, padding=1, bias=False),
+            _group_norm(stock, group_norm_groups, out_channels, activation="relu"),
+            nn.Identity(),
+        )
+
+    def forward(self, x):
+        return self.double_conv(x)
+
+
+class Down(nn.Module):
+    def __init__(self, in_channels, out_channels, group_norm_groups, stock=False):
+        super().__init__()
+        self.maxpool_conv = nn.Sequential(nn.MaxPool3d(2), DoubleConv(in_channels, out_channels, group_norm_groups, stock=stock))
+
+    def forward(self, x):
+        return self.maxpool_conv(x)
+
+
+class Up(nn.Module):
+    def __init__(self, in_channels, out_channels, group_norm_groups, stock=False):
+        super().__init__()
+        self.up = _conv_transpose3d(stock, in_channels, in_channels // 2, kernel_size=2, stride=2)
+        self.conv = DoubleConv(in_channels, out_channels, group_norm_groups, stock=stock)
+
+    def forward(self, x1, x2):
+        x1 = self.up(x1)
+        dz, dy, dx = (x2.size(i) - x1.size(i) for i in (2, 3, 4))
+        if dx or dy or dz:
+            x1 = F.pad(x1, [dx // 2, dx - dx // 2, dy // 2, dy - dy // 2, dz // 2, dz - dz // 2])
+        return self.conv(skip_concat(x2, x1))
+
+
+class OutConv(nn.Module):
+    def __init__(self, in_channels, out_channels, stock=False):
+        super().__init__()
+        self.conv = _conv3d(stock, in_channels, out_channels, kernel_size=1)
+
+    def forward(self, x):
+        return self.conv(x)
+
+
+class UNet(nn.Module):
+    """``layers`` down/up stages (4 at problem scale 7), widths ``base_width * 2**i``."""
+
+    def __init__(self, n_channels, n_classes, layers=4, group_norm_groups=8, base_width=32, stock=False):
+        super().__init__()
+        if layers < 1:
+            raise ValueError(f"UNet requires layers >= 1, got layers={layers}")
+        self.n_channels, self.n_classes, self.layers = n_channels, n_classes, layers
+        self.group_norm_groups, self.base_width, self.stock = group_norm_groups, base_width, stock
+        self.checkpointing = False
+        g = group_norm_groups
+        width = base_width
+        self.down_list = nn.ModuleList([DoubleConv(n_channels, width, g, stock=stock)])
+        for _ in range(layers):
+            self.down_list.append(Down(width, width * 2, g, stock=stock))
+            width *= 2
+        self.up_list = nn.ModuleList()
+        for _ in range(layers):
+            self.up_list.append(Up(width, width // 2, g, stock=stock))
+            width //= 2
+        self.up_list.append(OutConv(width, n_classes, stock=stock))
+
+    def use_checkpointing(self):
+        self.checkpointing = True
+
+    def set_shard_halo(self, enabled: bool = True):
+        """Run every 3x3x3 convolution in the depth-shard form (zero halo + depth padding 0)."""
+        for m in self.modules():
+            if isinstance(m, FastConv3d):
+                m.shard_halo = bool(enabled)
+        return self
+
+    def _run(self, block, *inputs):
+        if self.checkpointing:
+            return torch.utils.checkpoint.checkpoint(block, *inputs, use_reentrant=False)
+        return block(*inputs)
+
+    def forward(self, x):
+        feats = [self._run(self.down_list[0], x)]
+        for i in range(1, self.layers + 1):
+            feats.append(self._run(self.down_list[i], feats[-1]))
+        feats.reverse()
+        out = feats[0]
+        for i in range(self.layers):
+            out = self._run(self.up_list[i], out, feats[i + 1])
+        return self._run(self.up_list[-1], out)

@@ -1,0 +1,287 @@
+"""GPU parity of the conv3d family against the fp64 oracle, through the C ABI.
+
+Standards, as in the reference's kernel suite (``triton_conv3d/reference.py:4-18``):
+1. bitwise on {-1,0,1} operands whose sums are exactly representable (catches a wrong voxel / tap /
+   channel, which a tolerance hides), each with the shapes that exercise partial tiles and padding forms;
+2. the K/dtype-derived ``error_bound`` on Gaussian operands, plus BASELINE.json's tolerance
+   (fp32 1e-5 relative, bf16 2e-2 relative + 1e-2 absolute);
+3. fp32 must really accumulate in fp32 (``max_abs < 1e-4 * peak``).
+"""
+
+import pytest
+import torch
+
+import scaffold_amd as sa
+from oracle import oracle as orc
+from scaffold_amd import conv3d as c3
+
+pytestmark = pytest.mark.gpu
+
+DIRS = ("fwd", "bwd-data", "bwd-weight")
+
+
+def run(problem, ops, direction, device, **kw):
+    x, w, gy = (ops[k].to(device) for k in ("input", "weight", "grad_output"))
+    b = ops["bias"].to(device) if ops["bias"] is not None else None
+    s, p = problem.stride, problem.padding
+    if problem.transposed:
+        if direction == "fwd":
+            return sa.conv_transpose3d_forward(x, w, b, s, 0, 0, 1, 1, **kw)
+        if direction == "bwd-data":
+            return sa.conv_transpose3d_backward_data(gy, w, x.shape, s, 0, 0, 1, 1, **kw)
+        return sa.conv_transpose3d_backward_weight(x, w.shape, gy, s, 0, 0, 1, 1, **kw)
+    if direction == "fwd":
+        return sa.conv3d_forward(x, w, b, s, p, 1, 1, **kw)
+    if direction == "bwd-data":
+        return sa.conv3d_backward_data(gy, w, x.shape, s, p, 1, 1, **kw)
+    return sa.conv3d_backward_weight(x, w.shape, gy, s, p, 1, 1, **kw)
+
+
+def check_exact(problem, direction, device, seed=0, **kw):
+    """Bitwise standard; thins the activations until the fp64 result is exactly representable."""
+    density = orc.exact_density(problem, direction)
+    for _ in range(6):
+        ops = orc.make_inputs(problem, seed=seed, exact=True, density=density)
+        ref = orc.conv_reference(problem, ops, direction)
+        if orc.is_exactly_representable(ref, problem.dtype):
+            break
+        density *= 0.5
+    else:
+        pytest.skip("no exactly representable draw")
+    assert ref.abs().max() > 0, "degenerate draw"
+    got = run(problem, ops, direction, device, **kw)
+    rep = orc.compare(got, ref)
+    assert rep.bitwise, f"{problem} [{direction}] {kw}: {rep}"
+    return got
+
+
+# --- shapes -------------------------------------------------------------------------------------
+# MFMA-tiled: 3x3x3, stride 1, channels multiples of 32; spatial extents chosen to hit all three
+# brick shapes (W > 16, 9..16, <= 8), partial tiles, and the three padding forms of a depth shard.
+MFMA_SHAPES = [
+    # (cin, cout, spatial, padding)
+    (32, 32, (8, 8, 32), (1, 1, 1)),
+    (32, 32, (5, 7, 33), (1, 1, 1)),
+    (32, 64, (6, 9, 40), (0, 1, 1)),
+    (64, 32, (6, 6, 18), (0, 0, 0)),
+    (64, 64, (9, 10, 16), (1, 1, 1)),
+    (32, 96, (4, 13, 13), (1, 1, 1)),
+    (96, 32, (10, 8, 8), (1, 1, 1)),
+    (32, 32, (3, 5, 7), (1, 1, 1)),
+    (128, 64, (4, 4, 4), (1, 1, 1)),
+    (32, 32, (2, 2, 2), (1, 1, 1)),
+    (32, 32, (4, 6, 20), (2, 2, 2)),
+]
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("cin,cout,spatial,padding", MFMA_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_exact(device, dtype, cin, cout, spatial, padding, direction):
+    if direction == "bwd-data" and any(p > 2 for p in padding):
+        pytest.skip("p > k-1")
+    prob = orc.ConvProblem(n=2 if spatial[2] < 30 else 1, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=dtype)
+    assert c3.uses_mfma(prob.input_shape, prob.weight_shape, 1, padding, 1, dtype, direction)
+    got = check_exact(prob, direction, device)
+    # the direct kernels must agree bit for bit on the same exact draw
+    check_exact(prob, direction, device, force_generic=True)
+    if direction == "bwd-weight":
+        assert got.is_contiguous(memory_format=torch.channels_last_3d) or got.shape[2:] == (1, 1, 1)
+
+
+# Shapes only the direct kernels serve: odd channel counts, strides, dilation, other kernel sizes,
+# fp32 (``triton_conv3d/shapes.py:611-684`` edge list).
+DIRECT_SHAPES = [
+    # (n, cin, cout, spatial, kernel, stride, padding, bias)
+    (1, 3, 6, (13, 13, 13), (3, 3, 3), (1, 1, 1), (1, 1, 1), False),
+    (2, 5, 7, (1, 8, 8), (1, 3, 3), (1, 1, 1), (0, 1, 1), True),
+    (1, 17, 6, (2, 31, 3), (3, 3, 3), (1, 1, 1), (1, 1, 1), False),
+    (3, 8, 8, (5, 6, 7), (3, 3, 3), (2, 2, 2), (1, 1, 1), True),
+    (1, 16, 11, (6, 6, 6), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),
+    (1, 1, 32, (6, 7, 9), (3, 3, 3), (1, 1, 1), (1, 1, 1), False),
+    (1, 4, 4, (2, 2, 2), (3, 3, 3), (1, 1, 1), (1, 1, 1), False),
+    (1, 8, 4, (8, 8, 8), (2, 2, 2), (2, 2, 2), (0, 0, 0), False),
+]
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("n,cin,cout,spatial,kernel,stride,padding,bias", DIRECT_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_direct_exact(device, dtype, n, cin, cout, spatial, kernel, stride, padding, bias, direction):
+    if direction == "bwd-data" and stride != (1, 1, 1):
+        pytest.skip("the data gradient is served at stride 1 only")
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, kernel=kernel, stride=stride, padding=padding,
+                           bias=bias, dtype=dtype)
+    check_exact(prob, direction, device)
+
+
+def test_dilation_and_anisotropic_stride(device):
+    x = torch.randint(-1, 2, (1, 4, 9, 10, 11), dtype=torch.float32)
+    w = torch.randint(-1, 2, (5, 4, 3, 2, 3), dtype=torch.float32)
+    ref = torch.nn.functional.conv3d(x.double(), w.double(), None, (1, 2, 1), (2, 0, 1), (2, 1, 1))
+    got = sa.conv3d_forward(x.to(device).contiguous(memory_format=torch.channels_last_3d), w.to(device), None, (1, 2, 1),
+                            (2, 0, 1), (2, 1, 1))
+    assert torch.equal(got.cpu().double(), ref)
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_gaussian_tolerance(device, dtype, direction):
+    prob = orc.ConvProblem(n=1, cin=64, cout=64, spatial=(12, 20, 36), dtype=dtype)
+    ops = orc.make_inputs(prob, seed=3)
+    ops["weight"] = (ops["weight"].float() / (prob.cin * 27) ** 0.5).to(dtype)
+    ref = orc.conv_reference(prob, ops, direction)
+    got = run(prob, ops, direction, device)
+    orc.assert_close(got, ref, prob, direction)
+    if dtype is torch.bfloat16:
+        orc.assert_baseline_tolerance(got, ref, dtype, f"{direction}")
+
+
+@pytest.mark.parametrize("direction", DIRS)
+def test_fp32_is_true_fp32(device, direction):
+    """Config 1 of BASELINE.json: 32->32 at 32^3 in fp32, fwd + dgrad + wgrad."""
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(32, 32, 32), dtype=torch.float32)
+    g = torch.Generator().manual_seed(1000)
+    x = torch.randn(prob.input_shape, generator=g).contiguous(memory_format=torch.channels_last_3d)
+    bound = 1.0 / (prob.cin * 27) ** 0.5
+    w = ((torch.rand(prob.weight_shape, generator=torch.Generator().manual_seed(1001)) * 2 - 1) * bound).contiguous(
+        memory_format=torch.channels_last_3d)
+    gy = torch.randn(prob.output_shape, generator=torch.Generator().manual_seed(1002)).contiguous(
+        memory_format=torch.channels_last_3d)
+    ops = {"input": x, "weight": w, "grad_output": gy, "bias": None}
+    ref = orc.conv_reference(prob, ops, direction)
+    got = run(prob, ops, direction, device)
+    rep = orc.compare(got, ref)
+    assert rep.max_abs < 1e-4 * ref.abs().max().item(), rep
+    orc.assert_baseline_tolerance(got, ref, torch.float32, direction)
+
+
+# --- transposed convolution ---------------------------------------------------------------------
+CONVT_SHAPES = [
+    (1, 128, 64, (4, 4, 4), (2, 2, 2), True),
+    (2, 64, 32, (3, 5, 6), (2, 2, 2), True),
+    (1, 5, 7, (2, 3, 4), (2, 2, 2), False),
+    (1, 8, 8, (2, 2, 3), (1, 2, 3), True),
+]
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("n,cin,cout,spatial,kernel,bias", CONVT_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_transposed_exact(device, dtype, n, cin, cout, spatial, kernel, bias, direction):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, kernel=kernel, stride=kernel, padding=(0, 0, 0),
+                           transposed=True, bias=bias, dtype=dtype)
+    got = check_exact(prob, direction, device)
+    assert tuple(got.shape) == {"fwd": prob.output_shape, "bwd-data": prob.input_shape, "bwd-weight": prob.weight_shape}[direction]
+
+
+def test_transposed_bias_is_per_channel_not_per_tap(device):
+    x = torch.zeros((1, 4, 2, 2, 2), dtype=torch.float32, device=device).contiguous(memory_format=torch.channels_last_3d)
+    w = torch.zeros((4, 3, 2, 2, 2), dtype=torch.float32, device=device)
+    b = torch.tensor([1.0, 2.0, 3.0], device=device)
+    y = sa.conv_transpose3d_forward(x, w, b, 2)
+    assert torch.equal(y, b.view(1, 3, 1, 1, 1).expand_as(y))
+
+
+# --- layouts, out=, determinism -----------------------------------------------------------------
+def test_weight_layouts_give_identical_bits(device):
+    prob = orc.ConvProblem(n=1, cin=32, cout=64, spatial=(6, 8, 20), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=5)
+    x = ops["input"].to(device)
+    w_cl = ops["weight"].to(device)                       # channels_last_3d
+    w_std = w_cl.contiguous()                              # PyTorch default
+    w_rsck = w_cl.permute(2, 3, 4, 1, 0).contiguous()      # (kd, kh, kw, Cin, Cout)
+    y0 = sa.conv3d_forward(x, w_cl, None, 1, 1)
+    y1 = sa.conv3d_forward(x, w_std, None, 1, 1)
+    y2 = sa.conv3d_forward(x, w_cl, None, 1, 1, weight_rsck=w_rsck)
+    assert torch.equal(y0, y1) and torch.equal(y0, y2)
+    gy = ops["grad_output"].to(device)
+    g0 = sa.conv3d_backward_data(gy, w_cl, x.shape, 1, 1)
+    g1 = sa.conv3d_backward_data(gy, w_std, x.shape, 1, 1)
+    g2 = sa.conv3d_backward_data(gy, w_cl, x.shape, 1, 1, weight_rsck=w_rsck)
+    assert torch.equal(g0, g1) and torch.equal(g0, g2)
+
+
+def test_ncdhw_input_is_converted_not_misread(device):
+    prob = orc.ConvProblem(n=2, cin=32, cout=32, spatial=(4, 6, 10), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=9, exact=True, density=0.3)
+    ref = orc.conv_reference(prob, ops, "fwd")
+    x_ncdhw = ops["input"].contiguous().to(device)
+    assert not x_ncdhw.is_contiguous(memory_format=torch.channels_last_3d)
+    y = sa.conv3d_forward(x_ncdhw, ops["weight"].to(device), None, 1, 1)
+    assert y.is_contiguous(memory_format=torch.channels_last_3d)
+    assert orc.compare(y, ref).bitwise
+
+
+def test_weight_flip_matches_flipped_weight(device):
+    prob = orc.ConvProblem(n=1, cin=8, cout=8, spatial=(5, 5, 5), dtype=torch.float32)
+    ops = orc.make_inputs(prob, seed=2, exact=True)
+    x, w = ops["input"].to(device), ops["weight"].to(device)
+    y = sa.conv3d_forward(x, w, None, 1, 1, weight_flip=True)
+    ref = torch.nn.functional.conv3d(ops["input"].double(), ops["weight"].double().flip(2, 3, 4), None, 1, 1)
+    assert torch.equal(y.cpu().double(), ref)
+
+
+def test_out_and_workspace_are_validated(device):
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(4, 4, 8), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=1)
+    x, w, gy = (ops[k].to(device) for k in ("input", "weight", "grad_output"))
+    good = torch.empty(prob.output_shape, dtype=x.dtype, device=device, memory_format=torch.channels_last_3d)
+    assert sa.conv3d_forward(x, w, None, 1, 1, out=good) is good
+    with pytest.raises(ValueError):
+        sa.conv3d_forward(x, w, None, 1, 1, out=torch.empty(prob.output_shape, dtype=x.dtype, device=device))  # NCDHW
+    with pytest.raises(ValueError):
+        sa.conv3d_forward(x, w, None, 1, 1, out=good[:, :16])
+    with pytest.raises(ValueError):
+        sa.conv3d_forward(x, w, None, 1, 1, out=good.float())
+    with pytest.raises(ValueError):
+        sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, workspace=torch.empty(8, dtype=torch.float32, device=device))
+    with pytest.raises(ValueError):
+        sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, out=torch.empty(w.shape, dtype=x.dtype, device=device).contiguous())
+    splits = c3.split_count(x.shape, w.shape, 1, 1, 1, x.dtype)
+    ws = torch.empty(c3.workspace_elements(splits, 32, 32, (3, 3, 3)), dtype=torch.float32, device=device)
+    gw = sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, workspace=ws)
+    assert torch.equal(gw, sa.conv3d_backward_weight(x, w.shape, gy, 1, 1))
+    with pytest.raises(NotImplementedError):
+        sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, deterministic=False)
+    with pytest.raises(NotImplementedError):
+        sa.conv3d_backward_data(gy, w, x.shape, 2, 1)
+    with pytest.raises(NotImplementedError):
+        sa.conv3d_forward(x.cpu(), w.cpu(), None, 1, 1)
+
+
+def test_same_call_same_bits(device):
+    prob = orc.ConvProblem(n=1, cin=64, cout=64, spatial=(8, 16, 40), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=4)
+    outs = []
+    for _ in range(3):
+        # scratch comes from torch.empty: poison the allocator's free blocks between calls
+        junk = torch.full((1 << 22,), float("nan"), device=device)
+        del junk
+        outs.append(tuple(run(prob, ops, d, device).clone() for d in DIRS))
+    for o in outs[1:]:
+        for a, b in zip(outs[0], o):
+            assert torch.equal(a, b)
+
+
+def test_empty_batch_forward(device):
+    x = torch.empty((0, 32, 4, 4, 4), dtype=torch.bfloat16, device=device).contiguous(memory_format=torch.channels_last_3d)
+    w = torch.empty((32, 32, 3, 3, 3), dtype=torch.bfloat16, device=device)
+    assert sa.conv3d_forward(x, w, None, 1, 1).shape == (0, 32, 4, 4, 4)
+
+
+# --- shard boundary -----------------------------------------------------------------------------
+def test_depth_shard_with_halo_equals_slice_of_full_volume(device):
+    """A (D_loc + 2) x H x W slab convolved at padding (0,1,1) is the D-slice of the full-volume
+    convolution (``tests/helpers/rank_scripts/conv3d_shards_2rank.py:96-98`` without the second rank)."""
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(16, 12, 20), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=8, exact=True, density=0.25)
+    full = orc.conv_reference(prob, ops, "fwd")
+    if not orc.is_exactly_representable(full, torch.bfloat16):
+        pytest.skip("draw not exact")
+    x, w = ops["input"], ops["weight"].to(device)
+    lo = torch.cat([torch.zeros_like(x[:, :, :1]), x[:, :, :9]], dim=2).contiguous(memory_format=torch.channels_last_3d)
+    hi = torch.cat([x[:, :, 7:], torch.zeros_like(x[:, :, :1])], dim=2).contiguous(memory_format=torch.channels_last_3d)
+    y_lo = sa.conv3d_forward(lo.to(device), w, None, 1, (0, 1, 1))
+    y_hi = sa.conv3d_forward(hi.to(device), w, None, 1, (0, 1, 1))
+    assert torch.equal(torch.cat([y_lo, y_hi], dim=2).cpu().double(), full)
