@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Throughput of the ScaFFold U-Net hot path on one MI355X.
+
+``python bench.py [--steps K] [--warmup W]`` prints ONE JSON line.
+
+The workload (``config.workload``) is BASELINE.json's headline convolution: the 3x3x3, 32->32 channel,
+stride-1 convolution of the first encoder level on a 128^3 volume, bf16 NDHWC, N=1 (config 3 of
+BASELINE.json).  One *step* is one pass of the hot path over that batch: forward + data gradient +
+weight gradient, operands resident in HBM.  ``value`` is the algorithmic FLOPs of the three directions
+(3 x 2*M*N*K) divided by the measured step time.
+
+Also on the line:
+* ``roofline``: the dominant kernel (the MFMA implicit-GEMM kernel, forward direction), timed on its own
+  with HIP events on the launch stream, against the dense bf16 MFMA peak of 2.5 PFLOP/s;
+* ``cpu_baseline``: the reference's CPU path for the same op (stock torch ``conv3d`` + autograd on
+  channels_last_3d bf16 tensors, which is what the reference's ladders fall to off-GPU), timed on the
+  host cores of this box on a bounded sample of the workload;
+* ``details``: per-direction TFLOP/s, GroupNorm (config 2) GB/s against the 8 TB/s HBM peak, and the
+  U-Net train step of one depth shard (config 5) in ms.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+CL = torch.channels_last_3d
+
+
+def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
+    """Average GPU time of ``fn`` over ``iters`` back-to-back calls, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def conv_operands(cin, cout, spatial, device, seed=3000):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((1, cin, *spatial), generator=g, dtype=torch.float32).to(torch.bfloat16).contiguous(memory_format=CL)
+    bound = 1.0 / math.sqrt(cin * 27)
+    w = ((torch.rand((cout, cin, 3, 3, 3), generator=g) * 2 - 1) * bound).to(torch.bfloat16).contiguous(memory_format=CL)
+    gy = torch.randn((1, cout, *spatial), generator=g, dtype=torch.float32).to(torch.bfloat16).contiguous(memory_format=CL)
+    return x.to(device), w.to(device), gy.to(device)
+
+
+def bench_conv(args, device):
+    import scaffold_amd as sa
+
+    cin = cout = 32
+    spatial = (128, 128, 128)
+    x, w, gy = conv_operands(cin, cout, spatial, device)
+    flops = 2 * math.prod(spatial) * cin * cout * 27
+    y = torch.empty_like(gy)
+    gx = torch.empty_like(x)
+    gw = sa.grad_weight_empty(cout, cin, (3, 3, 3), dtype=x.dtype, device=device)
+
+    def fwd():
+        sa.conv3d_forward(x, w, None, 1, 1, 1, out=y)
+
+    def dgrad():
+        sa.conv3d_backward_data(gy, w, x.shape, 1, 1, 1, out=gx)
+
+    def wgrad():
+        sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, 1, out=gw)
+
+    def step():
+        fwd()
+        dgrad()
+        wgrad()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = max(e0.elapsed_time(e1) / args.steps, 1e-9)
+    per_dir = {name: event_time_ms(fn, max(args.steps, 5)) for name, fn in (("fwd", fwd), ("dgrad", dgrad), ("wgrad", wgrad))}
+    return {
+        "flops_per_direction": flops,
+        "ms_per_step": ms_per_step,
+        "wall_ms_per_step": wall_ms,
+        "per_direction_ms": per_dir,
+        "per_direction_tflops": {k: flops / (v * 1e-3) / 1e12 for k, v in per_dir.items()},
+        "bytes_compulsory": 2 * (x.numel() + w.numel() + y.numel()),
+    }
+
+
+def bench_groupnorm(args, device):
+    """Config 2: N=2, C=64, 64^3, 8 groups, bf16, fused ReLU; algorithmic bytes 3B forward / 5B backward."""
+    import scaffold_amd.groupnorm  # noqa: F401  (registers torch.ops.scaffold_gn.*)
+
+    g = torch.Generator().manual_seed(2000)
+    shape = (2, 64, 64, 64, 64)
+    x = (torch.randn(shape, generator=g) * 3 + 0.5).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    gamma = (1 + 0.1 * torch.randn(64, generator=g)).to(device)
+    beta = (0.1 * torch.randn(64, generator=g)).to(device)
+    dy = torch.randn(shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    B = x.numel() * x.element_size()
+    out, mean, rstd = torch.ops.scaffold_gn.group_norm(x, 8, gamma, beta, 1e-5, "relu", None)
+    fwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm(x, 8, gamma, beta, 1e-5, "relu", None), 10)
+    bwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm_backward(dy, x, gamma, beta, mean, rstd, 8, "relu"), 10)
+    return {
+        "tensor_bytes": B,
+        "fwd_ms": fwd_ms, "fwd_gbs": 3 * B / (fwd_ms * 1e-3) / 1e9, "fwd_frac_of_hbm_peak": 3 * B / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "bwd_ms": bwd_ms, "bwd_gbs": 5 * B / (bwd_ms * 1e-3) / 1e9, "bwd_frac_of_hbm_peak": 5 * B / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
+
+
+def bench_unet_step(args, device):
+    """Config 5: one Adam step of the base-32, 5-level U-Net on a 64x128x128 depth shard (zero halo),
+    bf16 autocast, fp32 master weights, CE + Dice loss, gradient clipping at 1.0."""
+    import scaffold_amd as sa
+    from oracle.oracle import train_step_loss  # loss recipe only; the model and kernels are the product's
+
+    torch.manual_seed(5001)
+    model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True)
+    g = torch.Generator().manual_seed(5000)
+    occ = (torch.rand((1, 1, 64, 128, 128), generator=g) < 0.05).float().contiguous(memory_format=CL).to(device)
+    lab = torch.randint(0, 11, (1, 64, 128, 128), generator=g).to(device)
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(occ)
+        loss = train_step_loss(logits, lab, 11)
+        loss.backward()
+        torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        return loss
+
+    ms = event_time_ms(step, 3, warmup=2)
+    return {"ms_per_step": ms, "input": "1x1x64x128x128 occupancy (5% ones), zero depth halo, padding (0,1,1)"}
+
+
+def cpu_baseline():
+    """The reference's CPU path (torch conv3d + autograd, channels_last_3d bf16) on a 1/8 sample (64^3)."""
+    import torch.nn.functional as F
+
+    cin = cout = 32
+    spatial = (64, 64, 64)
+    g = torch.Generator().manual_seed(3000)
+    x = torch.randn((1, cin, *spatial), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).requires_grad_(True)
+    w = (torch.randn((cout, cin, 3, 3, 3), generator=g) / math.sqrt(cin * 27)).to(torch.bfloat16).contiguous(memory_format=CL).requires_grad_(True)
+    gy = torch.randn((1, cout, *spatial), generator=g).to(torch.bfloat16).contiguous(memory_format=CL)
+    flops = 3 * 2 * math.prod(spatial) * cin * cout * 27
+
+    def once():
+        y = F.conv3d(x, w, None, 1, 1)
+        torch.autograd.grad(y, (x, w), gy)
+
+    once()
+    times = []
+    budget = time.perf_counter() + 25.0
+    while len(times) < 3 and time.perf_counter() < budget:
+        t0 = time.perf_counter()
+        once()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[len(times) // 2]
+    return {
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"torch CPU conv3d fwd+dgrad+wgrad, bf16 channels_last_3d, 32->32 3x3x3 on 64^3 (1/8 of the workload), "
+                  f"median of {len(times)} runs, {t * 1e3:.1f} ms each",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--skip-unet", action="store_true", help="omit the U-Net train step")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (one process, one MI355X); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU fallback exists for the hot path)", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    conv = bench_conv(args, device)
+    details = {"conv": conv}
+    try:
+        details["groupnorm_cfg2"] = bench_groupnorm(args, device)
+    except Exception as exc:  # report, do not hide
+        details["groupnorm_cfg2"] = {"error": repr(exc)}
+    if not args.skip_unet:
+        try:
+            details["unet_step_cfg5"] = bench_unet_step(args, device)
+        except Exception as exc:
+            details["unet_step_cfg5"] = {"error": repr(exc)}
+    flops = conv["flops_per_direction"]
+    fwd_ms = conv["per_direction_ms"]["fwd"]
+    achieved = flops / (fwd_ms * 1e-3) / 1e12
+    line = {
+        "metric": "conv3d fwd+dgrad+wgrad TFLOP/s @128^3 bf16 (U-Net level-0 conv 32->32, 1 GPU)",
+        "value": 3 * flops / (conv["ms_per_step"] * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": conv["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "conv3d 3x3x3 stride 1 pad 1, Cin=Cout=32, 128^3, N=1, NDHWC bf16: fwd + dgrad + wgrad "
+                               "(BASELINE.json config 3, first encoder level)"},
+        "roofline": {
+            "bound": "mfma", "kernel": "conv_mfma_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+            "flops_per_launch": flops, "avg_launch_ms": fwd_ms,
+        },
+        "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
+        "details": details,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

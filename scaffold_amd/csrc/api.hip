@@ -169,7 +169,7 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
       return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
-    return mfma_conv_gather(a, dtype, x, workspace, bias, y, st);
+    return mfma_conv_persist(a, dtype, x, workspace, bias, y, st);
   }
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;
@@ -204,7 +204,7 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
     // produced channel = Cin (stride w_stride[1]), reduction channel = Cout (w_stride[0]), taps flipped
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, workspace, st))
       return rc;
-    return mfma_conv_gather(a, dtype, gy, workspace, nullptr, gx, st);
+    return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, st);
   }
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cout; a.id = out[0]; a.ih = out[1]; a.iw = out[2];

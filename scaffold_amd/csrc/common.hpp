@@ -26,12 +26,11 @@ __device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(((u
 __device__ __forceinline__ float to_float(fp16_t x) { return (float)x.v; }
 __device__ __forceinline__ float to_float(float x) { return x; }
 
-// Round-to-nearest-even fp32 -> bf16 (NaN stays NaN, quietened).
+// Round-to-nearest-even fp32 -> bf16 (NaN stays NaN): gfx950's v_cvt_pk_bf16_f32, no branches.
+typedef __bf16 sfh_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float sfh_f32x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint16_t bf16_bits_rne(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 template <typename T> struct elem;
@@ -49,7 +48,8 @@ template <> struct elem<float> {
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)bf16_bits_rne(lo) | ((uint32_t)bf16_bits_rne(hi) << 16);
+  const sfh_f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, sfh_bf16x2_t));
 }
 __device__ __forceinline__ uint32_t pack_fp16x2(float lo, float hi) {
   union { _Float16 h[2]; uint32_t u; } r;

@@ -68,6 +68,14 @@ struct Tile {
   static_assert(2 * PLANE + ((KD - 1) * BH * BW + (KH - 1) * BW + KW - 1) * 16 < 65536, "ds_read immediate range");
 };
 
+// LDS byte offset, relative to a lane's sub-tile base, of iteration it = tap*2 + kstep.
+template <typename C>
+__device__ __forceinline__ constexpr int lds_off(int it) {
+  const int tap = it / 2, ks = it % 2;
+  const int kd = tap / (C::KH * C::KW), kh = (tap / C::KW) % C::KH, kw = tap % C::KW;
+  return ((kd * C::BH + kh) * C::BW + kw) * 16 + ks * 2 * C::PLANE;
+}
+
 template <typename T, typename C>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
@@ -106,7 +114,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   const int id0 = od0 - a.pd, ih0 = oh0 - a.ph, iw0 = ow0 - a.pw;
   constexpr int PIECES = C::BV * 4;
   constexpr int ITERS = (PIECES + 255) / 256;
-  constexpr int BATCH = 8;
+  // staging loads in flight before the first LDS write: all of them when registers allow
+  constexpr int BATCH = C::NSUB == 1 ? ITERS : 8;
   constexpr int FRAG = 512;  // elements per packed (tap, k-step) fragment: 64 lanes x 8
 
   for (int cc = 0; cc < ncc; ++cc) {
@@ -141,26 +150,39 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     }
     __syncthreads();
 
+    // Software pipeline over the TAPS*2 (tap, k-step) iterations of this chunk: the weight fragment
+    // of iteration it+WDEPTH and the activation fragments of iteration it+1 are requested before the
+    // MFMAs of iteration it are issued, so L2 and LDS latency overlap the matrix pipe.
     const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
     const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
+    constexpr int NIT = C::TAPS * 2;
+    constexpr int WDEPTH = NIT < 6 ? NIT : 6;
+    uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
+    uint4 aq[2][C::MS];
 #pragma unroll
-    for (int tap = 0; tap < C::TAPS; ++tap) {
-      constexpr int KHW = C::KH * C::KW;
-      const int kd = tap / KHW, kh = (tap / C::KW) % C::KH, kw = tap % C::KW;
-      const int tapoff = ((kd * C::BH + kh) * C::BW + kw) * 16;
+    for (int it = 0; it < WDEPTH; ++it)
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        uint4 wf[C::NSUB];
+      for (int ns = 0; ns < C::NSUB; ++ns) wq[it][ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + it * FRAG);
+#pragma unroll
+    for (int ms = 0; ms < C::MS; ++ms) aq[0][ms] = *reinterpret_cast<const uint4*>(lds + lbase[ms] + lds_off<C>(0));
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+      if (it + WDEPTH < NIT) {
 #pragma unroll
         for (int ns = 0; ns < C::NSUB; ++ns)
-          wf[ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + (tap * 2 + ks) * FRAG);
-#pragma unroll
-        for (int ms = 0; ms < C::MS; ++ms) {
-          const uint4 af = *reinterpret_cast<const uint4*>(lds + lbase[ms] + tapoff + ks * 2 * C::PLANE);
-#pragma unroll
-          for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma<T>::run(wf[ns], af, acc[ms][ns]);
-        }
+          wq[it + WDEPTH][ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + (it + WDEPTH) * FRAG);
       }
+      if (it + 1 < NIT) {
+#pragma unroll
+        for (int ms = 0; ms < C::MS; ++ms)
+          aq[(it + 1) & 1][ms] = *reinterpret_cast<const uint4*>(lds + lbase[ms] + lds_off<C>(it + 1));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ms = 0; ms < C::MS; ++ms)
+#pragma unroll
+        for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma<T>::run(wq[it][ns], aq[it & 1][ms], acc[ms][ns]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 

@@ -24,5 +24,8 @@ int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_
                      int64_t s_kh, int64_t s_kw, int flip, void* packed, hipStream_t st);
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                      hipStream_t st);
+// Same contract, persistent one-workgroup-per-CU kernel with register-resident weights.
+int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
+                      hipStream_t st);
 
 }  // namespace sfh

@@ -21,6 +21,11 @@
 // into whole groups; the scalar path (one workgroup per (sample, group)) otherwise.
 #include "common.hpp"
 
+// No implicit mul+add contraction in this file: every FMA is written as fmaf(). The forward and the
+// backward then round the pre-activation identically, and dy*gamma minus its own group mean cancels
+// to an exact zero for one-element groups.
+#pragma clang fp contract(off)
+
 namespace sfh {
 
 namespace {
@@ -521,9 +526,7 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
         const float xh = (f[u][e] - mu[e]) * rs[e];
         float d = g[u][e];
         if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
-        // the product is rounded on its own (no contraction) so that a one-element group, whose mean of
-        // dy*gamma is that same rounded product, cancels to an exact zero
-        o[e] = rs[e] * ((__fmul_rn(d, ga[e]) - ca[e]) - xh * cb[e]);
+        o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
       }
       St<T, V>::run(ds + (row + u * step) * C, o);
     }
@@ -537,7 +540,7 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
       const float xh = (f[e] - mu[e]) * rs[e];
       float d = g[e];
       if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
-      o[e] = rs[e] * ((__fmul_rn(d, ga[e]) - ca[e]) - xh * cb[e]);
+      o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
     }
     St<T, V>::run(ds + row * C, o);
   }
@@ -670,7 +673,7 @@ __global__ void __launch_bounds__(kBlock) gn_scalar_dx(const T* __restrict__ x, 
   const float xh = (to_float(x[i]) - mean[n * G + g]) * rs;
   float d = to_float(dy[i]);
   if (relu) d = fmaf(xh, w, b) <= 0.f ? 0.f : d;
-  dx[i] = elem<T>::from_float(rs * ((__fmul_rn(d, w) - coef[(n * G + g) * 2]) - xh * coef[(n * G + g) * 2 + 1]));
+  dx[i] = elem<T>::from_float(rs * ((d * w - coef[(n * G + g) * 2]) - xh * coef[(n * G + g) * 2 + 1]));
 }
 
 // ---- host-side dispatch --------------------------------------------------------------------
