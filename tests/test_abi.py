@@ -1,0 +1,106 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol include/scaffold_hip.h declares, and its
+pure host entry points (shape, plan and workspace queries, argument checking) behave."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from scaffold_amd import _lib
+from scaffold_amd._lib import ConvDesc, ConvTDesc, GroupNormDesc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "scaffold_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sfh_[a-zA-Z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_symbols()
+    assert len(names) >= 18
+    handle = ctypes.CDLL(_lib.lib_path())
+    for name in names:
+        assert hasattr(handle, name), f"{name} is declared in scaffold_hip.h but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names, "the ctypes binding and the header disagree"
+    assert _lib.lib().sfh_version() >= 100
+
+
+def conv_desc(n=1, cin=32, sp=(16, 16, 16), cout=32, k=(3, 3, 3), s=(1, 1, 1), p=(1, 1, 1), d=(1, 1, 1)):
+    return ConvDesc(n, cin, *sp, cout, *k, *s, *p, *d)
+
+
+def test_out_shape_and_argument_checks():
+    L = _lib.lib()
+    out = (ctypes.c_int32 * 3)()
+    assert L.sfh_conv3d_out_shape(ctypes.byref(conv_desc(p=(0, 1, 1))), out) == 0 and list(out) == [14, 16, 16]
+    assert L.sfh_conv3d_out_shape(ctypes.byref(conv_desc(sp=(7, 8, 9), k=(2, 3, 1), s=(2, 1, 3), p=(1, 0, 2), d=(1, 2, 1))), out) == 0
+    assert list(out) == list(torch.nn.functional.conv3d(torch.empty((1, 32, 7, 8, 9), device="meta"),
+                                                        torch.empty((32, 32, 2, 3, 1), device="meta"), None, (2, 1, 3),
+                                                        (1, 0, 2), (1, 2, 1)).shape[2:])
+    # kernel wider than the padded input, zero stride, null descriptor: contract violations with a message
+    assert L.sfh_conv3d_out_shape(ctypes.byref(conv_desc(sp=(2, 2, 2), p=(0, 0, 0))), out) == _lib.SFH_ERR_INVALID
+    assert b"wider" in L.sfh_last_error()
+    assert L.sfh_conv3d_out_shape(ctypes.byref(conv_desc(s=(0, 1, 1))), out) == _lib.SFH_ERR_INVALID
+    assert L.sfh_conv3d_out_shape(None, out) == _lib.SFH_ERR_INVALID
+    with pytest.raises(ValueError):
+        _lib.check(_lib.SFH_ERR_INVALID, "x")
+    with pytest.raises(NotImplementedError):
+        _lib.check(_lib.SFH_ERR_UNSUPPORTED, "x")
+    with pytest.raises(_lib.ScaffoldKernelError):
+        _lib.check(_lib.SFH_ERR_LAUNCH, "x")
+
+
+def test_kernel_selection_is_a_pure_function_of_the_problem():
+    L = _lib.lib()
+    bf16, fp32 = 0, 2
+    d = conv_desc(sp=(128, 128, 128))
+    assert [L.sfh_conv3d_uses_mfma(ctypes.byref(d), bf16, i) for i in range(3)] == [1, 1, 1]
+    assert [L.sfh_conv3d_uses_mfma(ctypes.byref(d), fp32, i) for i in range(3)] == [0, 0, 0]          # fp32 is true fp32
+    assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(cin=3)), bf16, 0) == 0                         # odd channels
+    assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(s=(2, 2, 2))), bf16, 0) == 0                   # strided
+    assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(p=(0, 1, 1))), bf16, 1) == 1                   # shard form dgrad
+    # workspace sizes: packed weight for fwd/dgrad, splits * Cout * 27 * Cin fp32 for wgrad
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(d), bf16) == 32 * 32 * 27 * 2
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(d), fp32) == 0
+    splits = L.sfh_conv3d_wgrad_splits(ctypes.byref(d), bf16)
+    assert splits >= 1 and splits == L.sfh_conv3d_wgrad_splits(ctypes.byref(d), bf16)
+    assert L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(d), bf16) == splits * 32 * 27 * 32 * 4
+    assert L.sfh_conv3d_wgrad_splits(ctypes.byref(d), fp32) == 1
+
+
+def test_wgrad_split_plan_partitions_the_bricks():
+    """Every brick belongs to exactly one split: splits * ceil(bricks / splits) covers, (splits-1) * that does not."""
+    L = _lib.lib()
+    for sp in [(128, 128, 128), (64, 64, 64), (9, 10, 16), (5, 7, 33), (8, 8, 8), (2, 2, 2)]:
+        for cin, cout in [(32, 32), (64, 128), (512, 512)]:
+            d = conv_desc(cin=cin, cout=cout, sp=sp)
+            splits = L.sfh_conv3d_wgrad_splits(ctypes.byref(d), 0)
+            tw, td, th = (32, 2, 4) if sp[2] > 16 else ((16, 2, 8) if sp[2] > 8 else (8, 4, 8))
+            bricks = -(-sp[0] // td) * -(-sp[1] // th) * -(-sp[2] // tw)
+            per = -(-bricks // splits)
+            assert 1 <= splits <= bricks and splits * per >= bricks and (splits - 1) * per < bricks
+
+
+def test_groupnorm_workspace_and_checks():
+    L = _lib.lib()
+    d = GroupNormDesc(2, 64, 8, 1, 64 ** 3, 1e-5)
+    fwd = L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(d), 0)
+    bwd = L.sfh_groupnorm_bwd_workspace_bytes(ctypes.byref(d), 0)
+    assert fwd > 0 and bwd > fwd and fwd % 256 == 0
+    assert L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(GroupNormDesc(2, 64, 7, 0, 8, 1e-5)), 0) == 0   # C % G != 0
+    rc = L.sfh_groupnorm_fwd(ctypes.byref(d), 0, 0, 2, None, None, None, None, None, None, None, 0, None)
+    assert rc == _lib.SFH_ERR_INVALID and b"null" in L.sfh_last_error()
+
+
+def test_transposed_and_copy_entry_points_check_arguments():
+    L = _lib.lib()
+    d = ConvTDesc(1, 128, 32, 32, 32, 64, 2, 2, 2)
+    assert L.sfh_convT3d_fwd_workspace_bytes(ctypes.byref(d), 0) >= 0
+    strides = (ctypes.c_int64 * 5)(512, 1, 256, 128, 64)
+    assert L.sfh_convT3d_fwd(ctypes.byref(d), 0, None, None, strides, None, None, None, 0, 0, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_stream_copy(None, None, 64, None) == _lib.SFH_ERR_INVALID

@@ -1,0 +1,207 @@
+"""GPU parity at the module / network level, and of the kernels against the committed golden vectors.
+
+Mirrors the reference's module-level tests: all three directions through autograd against the stock op
+(``tests/test_conv3d.py:1170-1217``), autocast dtypes (``:1248-1284``), second-order differentiation raising
+(``:1733-1739``), and whole-network gradients with the two-arm structure of ``tests/test_groupnorm.py:1174-1228``
+(fp32: per-parameter relative L2 < 1e-4; bf16 autocast: relative L2 of the concatenated gradient < 5e-2)."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import scaffold_amd as sa
+from oracle import oracle as orc
+from scaffold_amd.modules import FastConv3d, FastConvTranspose3d, FastGroupNorm
+from scaffold_amd.unet import UNet
+
+pytestmark = pytest.mark.gpu
+CL = torch.channels_last_3d
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "hotpath_small.npz"))
+
+
+def g(name, device, dtype=torch.float32):
+    t = torch.from_numpy(GOLD[name]).to(dtype)
+    return (t.contiguous(memory_format=CL) if t.dim() == 5 else t).to(device)
+
+
+def test_kernels_reproduce_the_golden_vectors(device):
+    """Small-integer problems: fp32 results must equal the committed brute-force answers exactly."""
+    x, w, b, gy = (g(k, device) for k in ("conv_x", "conv_w", "conv_b", "conv_gy"))
+    assert torch.equal(sa.conv3d_forward(x, w, b, 1, (0, 1, 1)).cpu().double(), torch.from_numpy(GOLD["conv_y"]))
+    assert torch.equal(sa.conv3d_backward_data(gy, w, x.shape, 1, (0, 1, 1)).cpu().double(), torch.from_numpy(GOLD["conv_gx"]))
+    assert torch.equal(sa.conv3d_backward_weight(x, w.shape, gy, 1, (0, 1, 1)).cpu().double(), torch.from_numpy(GOLD["conv_gw"]))
+    x2, w2, gy2 = g("sconv_x", device), g("sconv_w", device), g("sconv_gy", device)
+    assert torch.equal(sa.conv3d_forward(x2, w2, None, (2, 1, 3), (1, 0, 2), (1, 2, 1)).cpu().double(), torch.from_numpy(GOLD["sconv_y"]))
+    assert torch.equal(sa.conv3d_backward_weight(x2, w2.shape, gy2, (2, 1, 3), (1, 0, 2), (1, 2, 1)).cpu().double(),
+                       torch.from_numpy(GOLD["sconv_gw"]))
+    xt, wt, bt = g("convt_x", device), g("convt_w", device), g("convt_b", device)
+    assert torch.equal(sa.conv_transpose3d_forward(xt, wt, bt, 2).cpu().double(), torch.from_numpy(GOLD["convt_y"]))
+    xg, gamma, beta, dy = g("gn_x", device), g("gn_gamma", device), g("gn_beta", device), g("gn_dy", device)
+    out, mean, rstd = torch.ops.scaffold_gn.group_norm(xg, 4, gamma, beta, 1e-5, "relu", None)
+    dx, dgamma, dbeta = torch.ops.scaffold_gn.group_norm_backward(dy, xg, gamma, beta, mean, rstd, 4, "relu")
+    for got, name in ((out, "gn_y"), (mean, "gn_mean"), (rstd, "gn_rstd"), (dx, "gn_dx"), (dgamma, "gn_dgamma"), (dbeta, "gn_dbeta")):
+        assert orc.gn_rel_error(got, torch.from_numpy(GOLD[name])) <= 1e-5, name
+
+
+def _grads(module, x, gy):
+    x = x.clone().requires_grad_(True)
+    y = module(x)
+    y.backward(gy)
+    return y.detach(), x.grad, {k: p.grad for k, p in module.named_parameters()}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fastconv3d_matches_stock_in_all_directions(device, dtype):
+    torch.manual_seed(0)
+    stock = nn.Conv3d(32, 64, 3, padding=1, bias=True).double()
+    fast = FastConv3d(32, 64, 3, padding=1, bias=True).to(device).to(dtype).to(memory_format=CL)
+    fast.load_state_dict({k: v.to(dtype) for k, v in stock.state_dict().items()})
+    stock.load_state_dict({k: v.double() for k, v in fast.state_dict().items()})  # identical (rounded) parameters
+    x = torch.randn(2, 32, 6, 10, 12).to(dtype)
+    gy = torch.randn(2, 64, 6, 10, 12).to(dtype)
+    y0, gx0, gp0 = _grads(stock, x.double(), gy.double())
+    y1, gx1, gp1 = _grads(fast, x.to(device).contiguous(memory_format=CL), gy.to(device).contiguous(memory_format=CL))
+    prob = orc.ConvProblem(n=2, cin=32, cout=64, spatial=(6, 10, 12), bias=True, dtype=dtype)
+    orc.assert_close(y1, y0, prob, "fwd")
+    orc.assert_close(gx1, gx0, prob, "bwd-data")
+    orc.assert_close(gp1["weight"], gp0["weight"], prob, "bwd-weight")
+    assert orc.gn_rel_error(gp1["bias"], gp0["bias"]) <= (1e-5 if dtype is torch.float32 else 2e-2)   # gy.sum((0,2,3,4))
+    assert y1.dtype is dtype and gx1.dtype is dtype and gp1["weight"].dtype is dtype and y1.is_contiguous(memory_format=CL)
+
+
+def test_autocast_casts_outside_the_node_and_returns_fp32_parameter_grads(device):
+    fast = FastConv3d(32, 32, 3, padding=1, bias=False).to(device).to(memory_format=CL)
+    up = FastConvTranspose3d(32, 32, 2, stride=2).to(device).to(memory_format=CL)
+    gn = FastGroupNorm(8, 32, activation="relu").to(device)
+    x = torch.randn(1, 32, 4, 8, 8, device=device).contiguous(memory_format=CL).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        h = fast(x)
+        assert h.dtype is torch.bfloat16
+        h = gn(h)
+        assert h.dtype is torch.bfloat16           # the input's dtype, not autocast's fp32 policy
+        y = up(h)
+        assert y.dtype is torch.bfloat16 and y.shape == (1, 32, 8, 16, 16)
+    y.float().sum().backward()
+    assert x.grad.dtype is torch.float32 and fast.weight.grad.dtype is torch.float32
+    assert up.weight.grad.dtype is torch.float32 and up.bias.grad.dtype is torch.float32 and gn.weight.grad.dtype is torch.float32
+    # outside autocast an fp32 model computes in fp32
+    assert fast(x.detach()).dtype is torch.float32
+
+
+def test_second_order_differentiation_raises(device):
+    fast = FastConv3d(8, 8, 3, padding=1).to(device)
+    x = torch.randn(1, 8, 4, 4, 4, device=device).requires_grad_(True)
+    (gx,) = torch.autograd.grad(fast(x).sum(), x, create_graph=True)
+    with pytest.raises(RuntimeError):
+        gx.sum().backward()
+    with torch.no_grad():
+        assert fast(x).shape == (1, 8, 4, 4, 4)
+    with torch.inference_mode():
+        assert fast(x).shape == (1, 8, 4, 4, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transposed_module_matches_stock(device, dtype):
+    torch.manual_seed(1)
+    stock = nn.ConvTranspose3d(64, 32, 2, stride=2).double()
+    fast = FastConvTranspose3d(64, 32, 2, stride=2).to(device).to(dtype).to(memory_format=CL)
+    fast.load_state_dict({k: v.to(dtype) for k, v in stock.state_dict().items()})
+    stock.load_state_dict({k: v.double() for k, v in fast.state_dict().items()})
+    x = torch.randn(1, 64, 4, 5, 6).to(dtype)
+    gy = torch.randn(1, 32, 8, 10, 12).to(dtype)
+    y0, gx0, gp0 = _grads(stock, x.double(), gy.double())
+    y1, gx1, gp1 = _grads(fast, x.to(device).contiguous(memory_format=CL), gy.to(device).contiguous(memory_format=CL))
+    tol = 1e-5 if dtype is torch.float32 else 2e-2
+    for a, b in ((y1, y0), (gx1, gx0), (gp1["weight"], gp0["weight"]), (gp1["bias"], gp0["bias"])):
+        assert orc.gn_rel_error(a, b) <= tol
+    assert gp1["weight"].shape == (64, 32, 2, 2, 2)
+
+
+def _two_arms(device, dtype_autocast, layers=2, base=32, size=(16, 16, 32), shard=False):
+    torch.manual_seed(7)
+    stock = UNet(1, 5, layers=layers, base_width=base, stock=True)
+    ours = UNet(1, 5, layers=layers, base_width=base).to(device).to(memory_format=CL)
+    ours.load_state_dict(stock.state_dict())
+    if shard:
+        ours.set_shard_halo(True)
+    g0 = torch.Generator().manual_seed(8)
+    x = (torch.rand((1, 1, *size), generator=g0) < 0.05).float()
+    lab = torch.randint(0, 5, (1, *size), generator=g0)
+    return stock, ours, x, lab
+
+
+def _step(model, x, lab, autocast_device=None):
+    if autocast_device is None:
+        logits = model(x)
+    else:
+        with torch.autocast(autocast_device, dtype=torch.bfloat16):
+            logits = model(x)
+    loss = orc.train_step_loss(logits, lab, 5)
+    loss.backward()
+    return loss.detach(), logits.detach()
+
+
+def test_unet_fp32_gradients_match_stock_per_parameter(device):
+    stock, ours, x, lab = _two_arms(device, None)
+    stock = stock.double()
+    l0, y0 = _step(stock, x.double(), lab)
+    l1, y1 = _step(ours, x.to(device).contiguous(memory_format=CL), lab.to(device))
+    assert abs(l0.item() - l1.item()) <= 1e-5 * abs(l0.item())
+    assert orc.gn_rel_error(y1, y0) <= 1e-4
+    worst = 0.0
+    for (k, p0), (_, p1) in zip(stock.named_parameters(), ours.named_parameters()):
+        rel = (p1.grad.cpu().double() - p0.grad).norm() / p0.grad.norm().clamp_min(1e-30)
+        worst = max(worst, rel.item())
+        assert rel < 1e-4, (k, rel.item())
+
+
+def test_unet_bf16_autocast_train_step_matches_stock(device):
+    """Config 5 in small: bf16 autocast, fp32 master weights, CE + Dice, clip 1.0, one Adam step; our arm on the
+    GPU against the stock-module arm on the host cores."""
+    stock, ours, x, lab = _two_arms(device, torch.bfloat16)
+    opt0 = torch.optim.Adam(stock.parameters(), lr=1e-3)
+    opt1 = torch.optim.Adam(ours.parameters(), lr=1e-3)
+    l0, _ = _step(stock, x, lab, "cpu")
+    l1, _ = _step(ours, x.to(device).contiguous(memory_format=CL), lab.to(device), "cuda")
+    assert abs(l0.item() - l1.item()) <= 2e-2 * abs(l0.item())
+    g0 = torch.cat([p.grad.flatten().double() for p in stock.parameters()])
+    g1 = torch.cat([p.grad.flatten().cpu().double() for p in ours.parameters()])
+    assert all(p.grad.dtype is torch.float32 for p in ours.parameters())
+    assert ((g1 - g0).norm() / g0.norm()).item() < 5e-2
+    init = torch.cat([p.detach().flatten().double() for p in stock.parameters()])
+    for m, o in ((stock, opt0), (ours, opt1)):
+        torch.nn.utils.clip_grad_norm_(m.parameters(), 1.0)
+        o.step()
+    w0 = torch.cat([p.detach().flatten().double() for p in stock.parameters()])
+    w1 = torch.cat([p.detach().flatten().cpu().double() for p in ours.parameters()])
+    # Adam's first update is lr * sign(g): it amplifies the sign of gradients that are noise in bf16, so the
+    # bounded quantities are the step size and the agreement of the two update directions, not w itself.
+    u0, u1 = w0 - init, w1 - init
+    assert u0.abs().max() <= 1.001e-3 and u1.abs().max() <= 1.001e-3
+    assert (torch.dot(u0, u1) / (u0.norm() * u1.norm())).item() > 0.9
+
+
+def test_shard_halo_form_is_bitwise_the_padded_form(device):
+    """Zero depth halo + depth padding 0 (what a single DistConv shard computes) equals padding 1."""
+    _, ours, x, _ = _two_arms(device, torch.bfloat16)
+    xd = x.to(device).contiguous(memory_format=CL)
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        y_pad = ours(xd)
+        ours.set_shard_halo(True)
+        y_halo = ours(xd)
+    assert torch.equal(y_pad, y_halo)
+
+
+def test_up_equals_explicit_cat(device):
+    from scaffold_amd.unet import Up
+
+    torch.manual_seed(3)
+    up = Up(64, 32, 8).to(device).to(memory_format=CL)
+    x1 = torch.randn(1, 64, 4, 4, 8, device=device).contiguous(memory_format=CL)
+    x2 = torch.randn(1, 32, 8, 8, 16, device=device).contiguous(memory_format=CL)
+    want = up.conv(torch.cat([x2, up.up(x1)], dim=1))
+    assert torch.equal(up(x1, x2), want)
