@@ -36,6 +36,9 @@ if ROOT not in sys.path:
 
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the forward kernel on the bench workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
+# counter runs of this script scaled by the same counters on the 256 MiB copy kernel (profiles/ holds the runs).
+CONV_FWD_HBM_TRAFFIC_BYTES = int((108831.8 * 2.000 + 131073.9) * 1024)
 CL = torch.channels_last_3d
 
 
@@ -111,8 +114,14 @@ def bench_conv(args, device):
 
 
 def bench_groupnorm(args, device):
-    """Config 2: N=2, C=64, 64^3, 8 groups, bf16, fused ReLU; algorithmic bytes 3B forward / 5B backward."""
+    """Config 2: N=2, C=64, 64^3, 8 groups, bf16, fused ReLU; algorithmic bytes 3B forward / 5B backward.
+
+    Timed twice: through the C ABI directly (what a compiled caller sees; the launch chain keeps the GPU busy)
+    and through the registered torch operator (adds the Python dispatcher and output allocation per call)."""
+    import ctypes
+
     import scaffold_amd.groupnorm  # noqa: F401  (registers torch.ops.scaffold_gn.*)
+    from scaffold_amd import _lib
 
     g = torch.Generator().manual_seed(2000)
     shape = (2, 64, 64, 64, 64)
@@ -122,13 +131,53 @@ def bench_groupnorm(args, device):
     dy = torch.randn(shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
     B = x.numel() * x.element_size()
     out, mean, rstd = torch.ops.scaffold_gn.group_norm(x, 8, gamma, beta, 1e-5, "relu", None)
-    fwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm(x, 8, gamma, beta, 1e-5, "relu", None), 10)
-    bwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm_backward(dy, x, gamma, beta, mean, rstd, 8, "relu"), 10)
+    op_fwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm(x, 8, gamma, beta, 1e-5, "relu", None), 10)
+    op_bwd_ms = event_time_ms(lambda: torch.ops.scaffold_gn.group_norm_backward(dy, x, gamma, beta, mean, rstd, 8, "relu"), 10)
+
+    BF16, FP32 = _lib.dtype_code(torch.bfloat16), _lib.dtype_code(torch.float32)
+    L = _lib.lib()
+    desc = _lib.GroupNormDesc(2, 64, 8, 1, 64 ** 3, 1e-5)
+    dref = ctypes.byref(desc)
+    ws_f = torch.empty(max(1, L.sfh_groupnorm_fwd_workspace_bytes(dref, BF16)), dtype=torch.uint8, device=device)
+    ws_b = torch.empty(max(1, L.sfh_groupnorm_bwd_workspace_bytes(dref, BF16)), dtype=torch.uint8, device=device)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    dgamma, dbeta = torch.empty_like(gamma), torch.empty_like(beta)
+    stream = torch.cuda.current_stream().cuda_stream
+    P = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+
+    def abi_fwd():
+        _lib.check(L.sfh_groupnorm_fwd(dref, BF16, BF16, FP32, P(x), P(gamma), P(beta), P(y),
+                                       P(mean), P(rstd), P(ws_f), ws_f.numel(), stream), "sfh_groupnorm_fwd")
+
+    def abi_bwd():
+        _lib.check(L.sfh_groupnorm_bwd(dref, BF16, BF16, FP32, P(dy), P(x), P(gamma), P(beta),
+                                       P(mean), P(rstd), P(dx), P(dgamma), P(dbeta), P(ws_b), ws_b.numel(), stream), "sfh_groupnorm_bwd")
+
+    fwd_ms = event_time_ms(abi_fwd, 20)
+    bwd_ms = event_time_ms(abi_bwd, 20)
     return {
         "tensor_bytes": B,
         "fwd_ms": fwd_ms, "fwd_gbs": 3 * B / (fwd_ms * 1e-3) / 1e9, "fwd_frac_of_hbm_peak": 3 * B / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bwd_ms": bwd_ms, "bwd_gbs": 5 * B / (bwd_ms * 1e-3) / 1e9, "bwd_frac_of_hbm_peak": 5 * B / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "torch_op_fwd_ms": op_fwd_ms, "torch_op_bwd_ms": op_bwd_ms,
     }
+
+
+def copy_calibration(device, mib=256, reps=4):
+    """Runs the library's plain copy kernel on a buffer of known size, so that a counter run of this script
+    also holds FETCH_SIZE / WRITE_SIZE for a launch whose HBM traffic is known exactly."""
+    import ctypes
+
+    from scaffold_amd import _lib
+
+    L = _lib.lib()
+    src = torch.empty(mib << 20, dtype=torch.uint8, device=device).fill_(1)
+    dst = torch.empty_like(src)
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(reps):
+        _lib.check(L.sfh_stream_copy(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), src.numel(), stream), "sfh_stream_copy")
+    torch.cuda.synchronize()
+    return {"bytes_read": src.numel(), "bytes_written": src.numel(), "launches": reps}
 
 
 def bench_unet_step(args, device):
@@ -196,6 +245,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--skip-unet", action="store_true", help="omit the U-Net train step")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch the plain copy kernel on 256 MiB (reference point for HBM counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (one process, one MI355X); "
@@ -207,6 +258,8 @@ def main():
     device = torch.device("cuda:0")
     conv = bench_conv(args, device)
     details = {"conv": conv}
+    if args.copy_calibration:
+        details["copy_calibration"] = copy_calibration(device)
     try:
         details["groupnorm_cfg2"] = bench_groupnorm(args, device)
     except Exception as exc:  # report, do not hide
@@ -235,8 +288,8 @@ def main():
         "config": {"workload": "conv3d 3x3x3 stride 1 pad 1, Cin=Cout=32, 128^3, N=1, NDHWC bf16: fwd + dgrad + wgrad "
                                "(BASELINE.json config 3, first encoder level)"},
         "roofline": {
-            "bound": "mfma", "kernel": "conv_mfma_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+            "bound": "mfma", "kernel": "conv_persist_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": CONV_FWD_HBM_TRAFFIC_BYTES,
             "flops_per_launch": flops, "avg_launch_ms": fwd_ms,
         },
         "cpu_baseline": None if args.skip_cpu else cpu_baseline(),

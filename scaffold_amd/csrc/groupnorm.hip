@@ -434,27 +434,40 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
   }
 }
 
+// Fixed-order sum over a 256-thread workgroup (wavefront trees, then the four wave totals in order).
+__device__ __forceinline__ float block_sum256(float v, float* red4) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red4[0] + red4[1]) + (red4[2] + red4[3]);
+}
+
 // Workgroups [0, N*G): coef[n][g] = (A, B) with A = mean(dy'*gamma), B = mean(dy'*gamma*xhat)
 // over the group. Workgroups [N*G, N*G + C): dgamma[c], dbeta[c] summed over samples and splits.
-__global__ void __launch_bounds__(64) gn_bwd_finalize(const float* __restrict__ part, const void* __restrict__ gamma,
-                                                      int param_dtype, float* __restrict__ coef, float* __restrict__ dgamma,
-                                                      float* __restrict__ dbeta, int N, int C, int G, int nsplit, float m) {
+__global__ void __launch_bounds__(kBlock) gn_bwd_finalize(const float* __restrict__ part, const void* __restrict__ gamma,
+                                                          int param_dtype, float* __restrict__ coef, float* __restrict__ dgamma,
+                                                          float* __restrict__ dbeta, int N, int C, int G, int nsplit, float m) {
+  __shared__ float red4[4];
   const int b = blockIdx.x;
   const int cg = C / G;
   if (b < N * G) {
     const int n = b / G, g = b - n * G;
     float s1 = 0.f, s2 = 0.f;
-    const int total = cg * nsplit;
-    for (int i = threadIdx.x; i < total; i += 64) {
-      const int cc = i / nsplit, sp = i - cc * nsplit;
+    for (int cc = 0; cc < cg; ++cc) {
       const int c = g * cg + cc;
       const float w = load_param(gamma, param_dtype, c, 1.f);
-      const float* p = part + ((int64_t)n * nsplit + sp) * 2 * C;
-      s1 = fmaf(w, p[c], s1);
-      s2 = fmaf(w, p[C + c], s2);
+      float t1 = 0.f, t2 = 0.f;
+      for (int sp = threadIdx.x; sp < nsplit; sp += kBlock) {
+        const float* p = part + ((int64_t)n * nsplit + sp) * 2 * C;
+        t1 += p[c];
+        t2 += p[C + c];
+      }
+      s1 = fmaf(w, t1, s1);
+      s2 = fmaf(w, t2, s2);
     }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
+    s1 = block_sum256(s1, red4);
+    s2 = block_sum256(s2, red4);
     if (threadIdx.x == 0) {
       coef[(n * G + g) * 2] = s2 / m;
       coef[(n * G + g) * 2 + 1] = s1 / m;
@@ -463,13 +476,13 @@ __global__ void __launch_bounds__(64) gn_bwd_finalize(const float* __restrict__ 
     const int c = b - N * G;
     float s1 = 0.f, s2 = 0.f;
     const int total = N * nsplit;
-    for (int i = threadIdx.x; i < total; i += 64) {
+    for (int i = threadIdx.x; i < total; i += kBlock) {
       const float* p = part + (int64_t)i * 2 * C;
       s1 += p[c];
       s2 += p[C + c];
     }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
+    s1 = block_sum256(s1, red4);
+    s2 = block_sum256(s2, red4);
     if (threadIdx.x == 0) {
       if (dgamma != nullptr) dgamma[c] = s1;
       if (dbeta != nullptr) dbeta[c] = s2;
@@ -763,7 +776,7 @@ int bwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
                      pl.rows_per_split, p.relu);
   if (int rc = check_launch("gn_bwd_partial")) return rc;
   const float m = (float)S * (float)(C / G);
-  hipLaunchKernelGGL(gn_bwd_finalize, dim3(p.n * G + C), dim3(64), 0, st, part, gamma, param_dtype, coef, dgamma, dbeta, p.n, C,
+  hipLaunchKernelGGL(gn_bwd_finalize, dim3(p.n * G + C), dim3(kBlock), 0, st, part, gamma, param_dtype, coef, dgamma, dbeta, p.n, C,
                      G, pl.nsplit, m);
   if (int rc = check_launch("gn_bwd_finalize")) return rc;
   hipLaunchKernelGGL((gn_dx<T, TG>), grid, dim3(kBlock), 0, st, (const T*)x, (const TG*)dy, (T*)dx, mean, rstd, gamma, beta,

@@ -285,3 +285,52 @@ def test_depth_shard_with_halo_equals_slice_of_full_volume(device):
     y_lo = sa.conv3d_forward(lo.to(device), w, None, 1, (0, 1, 1))
     y_hi = sa.conv3d_forward(hi.to(device), w, None, 1, (0, 1, 1))
     assert torch.equal(torch.cat([y_lo, y_hi], dim=2).cpu().double(), full)
+
+
+# --- full size: properties that do not need the CPU oracle --------------------------------------
+def test_full_size_128cube_properties(device):
+    """BASELINE's headline conv (32 -> 32, 3x3x3, 128^3, bf16) on the exact standard: the fp64 oracle would
+    take minutes on the host, so the full-size launch is pinned by size-independent properties.  Operands are
+    in {-1,0,1}, thinned so every partial sum is an integer below 2^8 and the results are exact in bf16:
+    (1) the tiled MFMA kernels agree bitwise with the untiled direct kernels (two independent index paths,
+        the direct ones pinned against the oracle at small sizes above);
+    (2) the three directions are adjoint to one another exactly: <fwd(x), g> = <x, dgrad(g)> = <w, wgrad(x, g)>;
+    (3) the top-left corner equals the oracle on that corner's receptive field."""
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(128, 128, 128), dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(128)
+    shape = (1, 32, 128, 128, 128)
+    cl = torch.channels_last_3d
+
+    def draw(shp, density):
+        keep = torch.rand(shp, generator=g) < density
+        sign = torch.randint(0, 2, shp, generator=g) * 2 - 1
+        return (keep * sign).to(torch.bfloat16)
+
+    x = draw(shape, 0.02).contiguous(memory_format=cl).to(device)
+    gy = draw(shape, 0.02).contiguous(memory_format=cl).to(device)
+    w = draw((32, 32, 3, 3, 3), 0.5).contiguous(memory_format=cl).to(device)
+
+    y = sa.conv3d_forward(x, w, None, 1, 1)
+    gx = sa.conv3d_backward_data(gy, w, x.shape, 1, 1)
+    gw = sa.conv3d_backward_weight(x, w.shape, gy, 1, 1)
+    assert c3.uses_mfma(x.shape, w.shape, 1, 1, 1, torch.bfloat16, "fwd")
+    assert y.abs().max() > 0 and y.abs().max() < 256 and gx.abs().max() < 256
+    # the weight gradient sums over 2M voxels: exact only while it stays below 2^8 in bf16
+    assert gw.abs().max() <= 256, "draw too dense for an exact bf16 weight gradient"
+
+    y_d = sa.conv3d_forward(x, w, None, 1, 1, force_generic=True)
+    gx_d = sa.conv3d_backward_data(gy, w, x.shape, 1, 1, force_generic=True)
+    assert torch.equal(y, y_d)
+    assert torch.equal(gx, gx_d)
+
+    lhs = (y.double() * gy.double()).sum().item()
+    mid = (x.double() * gx.double()).sum().item()
+    assert lhs == mid
+    if gw.abs().max() < 256:
+        rhs = (w.double() * gw.double()).sum().item()
+        assert lhs == rhs
+
+    corner = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(10, 10, 40), dtype=torch.bfloat16)
+    xc = x[:, :, :10, :10, :40].cpu().contiguous(memory_format=cl)
+    ref = orc.conv_reference(corner, {"input": xc, "weight": w.cpu(), "bias": None, "grad_output": None}, "fwd")
+    assert torch.equal(y[:, :, :9, :9, :39].cpu().double(), ref[:, :, :9, :9, :39])
