@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
+#include "conv_thin.hpp"
 #include "wgrad_mfma.hpp"
 
 namespace sfh {
@@ -105,6 +106,74 @@ bool wgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) 
   return is_unit(p) && p.kd == 3 && p.kh == 3 && p.kw == 3 && p.n >= 1 && mfma_wgrad_supported(wgrad_args(p, out), dtype);
 }
 
+// ---- thin-channel problems (Cin == 1 stems, 1x1x1 heads) ---------------------------------------
+bool is_pointwise(const sfh_conv3d_desc& p) {
+  return p.kd == 1 && p.kh == 1 && p.kw == 1 && p.sd == 1 && p.sh == 1 && p.sw == 1 && p.pd == 0 && p.ph == 0 && p.pw == 0;
+}
+
+bool is_one_channel_cube(const sfh_conv3d_desc& p) {
+  return p.cin == 1 && p.kd == p.kh && p.kh == p.kw && (p.kd == 2 || p.kd == 3);
+}
+
+ThinArgs thin_base(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  ThinArgs a{};
+  a.n = p.n; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
+  a.td = p.in_d; a.th = p.in_h; a.tw = p.in_w;
+  a.sd = p.sd; a.sh = p.sh; a.sw = p.sw; a.pd = p.pd; a.ph = p.ph; a.pw = p.pw; a.dd = p.dd; a.dh = p.dh; a.dw = p.dw;
+  return a;
+}
+
+enum ThinKind { kThinNone = 0, kThinWideOut, kThinOut, kThinReduce };
+
+// Forward: y[v][co]. Returns the kernel family and fills `a` (weight strides left to the caller).
+ThinKind thin_fwd_plan(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], ThinArgs& a) {
+  a = thin_base(p, out);
+  if (is_one_channel_cube(p)) {
+    a.K = p.kd; a.J = p.kd * p.kh * p.kw; a.ct = 1; a.cw = p.cout;
+    return thin_supported(a, dtype) ? kThinWideOut : kThinNone;
+  }
+  if (!is_pointwise(p)) return kThinNone;
+  a.K = 0;
+  a.J = p.cin; a.ct = p.cin; a.cw = p.cout;
+  if (p.cin <= 32 && thin_supported(a, dtype)) return kThinWideOut;
+  a.J = p.cout; a.ct = p.cout; a.cw = p.cin;
+  if (p.cout <= 32 && thin_supported(a, dtype)) return kThinOut;
+  return kThinNone;
+}
+
+// Data gradient of a pointwise conv: gx[v][ci] = sum_co gy[v][co] * w[co][ci].
+ThinKind thin_dgrad_plan(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], ThinArgs& a) {
+  a = thin_base(p, out);
+  if (!is_pointwise(p)) return kThinNone;
+  a.K = 0;
+  a.J = p.cout; a.ct = p.cout; a.cw = p.cin;
+  if (p.cout <= 32 && thin_supported(a, dtype)) return kThinWideOut;
+  a.J = p.cin; a.ct = p.cin; a.cw = p.cout;
+  if (p.cin <= 32 && thin_supported(a, dtype)) return kThinOut;
+  return kThinNone;
+}
+
+// Weight gradient, dense [Cout][taps][Cin]. `thin_is_x` tells which operand is the thin one.
+ThinKind thin_wgrad_plan(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], ThinArgs& a, bool& thin_is_x) {
+  a = thin_base(p, out);
+  if (p.n < 1) return kThinNone;
+  if (is_one_channel_cube(p)) {
+    a.K = p.kd; a.J = p.kd * p.kh * p.kw; a.ct = 1; a.cw = p.cout;
+    a.so_wide = a.J; a.so_thin = 1;
+    thin_is_x = true;
+    return thin_supported(a, dtype) ? kThinReduce : kThinNone;
+  }
+  if (!is_pointwise(p)) return kThinNone;
+  a.K = 0;
+  a.J = p.cout; a.ct = p.cout; a.cw = p.cin; a.so_wide = 1; a.so_thin = p.cin;
+  thin_is_x = false;
+  if (p.cout <= 32 && thin_supported(a, dtype)) return kThinReduce;
+  a.J = p.cin; a.ct = p.cin; a.cw = p.cout; a.so_wide = p.cin; a.so_thin = 1;
+  thin_is_x = true;
+  if (p.cin <= 32 && thin_supported(a, dtype)) return kThinReduce;
+  return kThinNone;
+}
+
 __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n) {
   size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * 256;
@@ -171,6 +240,19 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
       return rc;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, st);
   }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
+    ThinArgs t;
+    const ThinKind kind = thin_fwd_plan(*p, dtype, out, t);
+    t.ws_kd = w_stride[2]; t.ws_kh = w_stride[3]; t.ws_kw = w_stride[4];
+    if (kind == kThinWideOut) {
+      t.ws_wide = w_stride[0]; t.ws_thin = w_stride[1];
+      return thin_wide_out(t, dtype, x, w, bias, y, st);
+    }
+    if (kind == kThinOut) {
+      t.ws_wide = w_stride[1]; t.ws_thin = w_stride[0];
+      return thin_out(t, dtype, x, w, bias, y, st);
+    }
+  }
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;
   a.cout = p->cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];
@@ -206,6 +288,18 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
       return rc;
     return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, st);
   }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
+    ThinArgs t;
+    const ThinKind kind = thin_dgrad_plan(*p, dtype, out, t);
+    if (kind == kThinWideOut) {
+      t.ws_wide = w_stride[1]; t.ws_thin = w_stride[0];
+      return thin_wide_out(t, dtype, gy, w, nullptr, gx, st);
+    }
+    if (kind == kThinOut) {
+      t.ws_wide = w_stride[0]; t.ws_thin = w_stride[1];
+      return thin_out(t, dtype, gy, w, nullptr, gx, st);
+    }
+  }
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cout; a.id = out[0]; a.ih = out[1]; a.iw = out[2];
   a.cout = p->cin; a.od = p->in_d; a.oh = p->in_h; a.ow = p->in_w;
@@ -221,15 +315,21 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
 extern "C" int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (!wgrad_uses_mfma(*p, dtype, out)) return 1;
-  return mfma_wgrad_splits(wgrad_args(*p, out));
+  if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_splits(wgrad_args(*p, out));
+  ThinArgs t;
+  bool thin_is_x;
+  if (thin_wgrad_plan(*p, dtype, out, t, thin_is_x) == kThinReduce) return thin_reduce_splits(t);
+  return 1;
 }
 
 extern "C" size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (!wgrad_uses_mfma(*p, dtype, out)) return 0;
-  return mfma_wgrad_workspace_bytes(wgrad_args(*p, out));
+  if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_workspace_bytes(wgrad_args(*p, out));
+  ThinArgs t;
+  bool thin_is_x;
+  if (thin_wgrad_plan(*p, dtype, out, t, thin_is_x) == kThinReduce) return thin_reduce_workspace_bytes(t);
+  return 0;
 }
 
 extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* workspace,
@@ -244,6 +344,16 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     return mfma_wgrad(a, dtype, x, gy, gw, workspace, st);
+  }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
+    ThinArgs t;
+    bool thin_is_x = false;
+    if (thin_wgrad_plan(*p, dtype, out, t, thin_is_x) == kThinReduce) {
+      const size_t need = thin_reduce_workspace_bytes(t);
+      if (workspace == nullptr || workspace_bytes < need)
+        return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+      return thin_is_x ? thin_reduce(t, dtype, x, gy, gw, workspace, st) : thin_reduce(t, dtype, gy, x, gw, workspace, st);
+    }
   }
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;

@@ -115,6 +115,47 @@ def test_direct_exact(device, dtype, n, cin, cout, spatial, kernel, stride, padd
     check_exact(prob, direction, device)
 
 
+# Thin-channel problems: the one-channel 3x3x3 / 2x2x2 stem forms and the 1x1x1 head forms (thin input,
+# thin output), each also checked bit for bit against the direct kernels on the same draw.
+THIN_SHAPES = [
+    # (n, cin, cout, spatial, kernel, stride, padding, bias)
+    (1, 1, 32, (9, 10, 21), (3, 3, 3), (1, 1, 1), (1, 1, 1), True),     # U-Net stem
+    (2, 1, 32, (6, 12, 12), (3, 3, 3), (1, 1, 1), (0, 1, 1), False),    # stem of a depth shard
+    (1, 1, 64, (9, 9, 9), (3, 3, 3), (2, 2, 2), (1, 1, 1), False),
+    (1, 1, 16, (8, 8, 8), (2, 2, 2), (2, 2, 2), (0, 0, 0), True),
+    (1, 32, 11, (7, 9, 13), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),     # U-Net head
+    (2, 64, 3, (4, 5, 6), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),
+    (1, 11, 32, (5, 6, 7), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),      # thin input, wide output
+    (1, 32, 32, (4, 4, 9), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),
+    (1, 2, 8, (30, 30, 30), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),    # several splits in the weight gradient
+]
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("n,cin,cout,spatial,kernel,stride,padding,bias", THIN_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_thin_exact(device, dtype, n, cin, cout, spatial, kernel, stride, padding, bias, direction):
+    if direction == "bwd-data" and stride != (1, 1, 1):
+        pytest.skip("the data gradient is served at stride 1 only")
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, kernel=kernel, stride=stride, padding=padding,
+                           bias=bias, dtype=dtype)
+    got = check_exact(prob, direction, device)
+    ref = check_exact(prob, direction, device, force_generic=True)
+    assert torch.equal(got, ref)
+
+
+def test_thin_gaussian_within_tolerance(device):
+    """Head and stem at Gaussian operands: fp32 within 1e-5 relative, bf16 within 2e-2 relative + 1e-2 absolute."""
+    for dtype in (torch.float32, torch.bfloat16):
+        for cin, cout, k, pad in ((1, 32, 3, 1), (32, 11, 1, 0)):
+            prob = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=(12, 16, 20), kernel=(k, k, k), padding=(pad, pad, pad),
+                                   bias=True, dtype=dtype)
+            ops = orc.make_inputs(prob, seed=21)
+            for direction in DIRS:
+                got = run(prob, ops, direction, device)
+                orc.assert_baseline_tolerance(got, orc.conv_reference(prob, ops, direction), dtype)
+
+
 def test_dilation_and_anisotropic_stride(device):
     x = torch.randint(-1, 2, (1, 4, 9, 10, 11), dtype=torch.float32)
     w = torch.randint(-1, 2, (5, 4, 3, 2, 3), dtype=torch.float32)
