@@ -5,6 +5,7 @@
 #include "common.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
+#include "conv_patch.hpp"
 #include "conv_thin.hpp"
 #include "wgrad_mfma.hpp"
 
@@ -104,6 +105,48 @@ WgradArgs wgrad_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
 
 bool wgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return is_unit(p) && p.kd == 3 && p.kh == 3 && p.kw == 3 && p.n >= 1 && mfma_wgrad_supported(wgrad_args(p, out), dtype);
+}
+
+// ---- 2x2x2, stride-2, unpadded problems (the up-convolution family) ------------------------------
+bool is_patch(const sfh_conv3d_desc& p) {
+  return p.kd == 2 && p.kh == 2 && p.kw == 2 && p.sd == 2 && p.sh == 2 && p.sw == 2 && p.pd == 0 && p.ph == 0 && p.pw == 0 &&
+         p.dd == 1 && p.dh == 1 && p.dw == 1;
+}
+
+// The strided convolution's input is the big volume, its output the small one.
+PatchArgs patch_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  PatchArgs a{};
+  a.n = p.n;
+  a.cbig = p.cin; a.bd = p.in_d; a.bh = p.in_h; a.bw = p.in_w;
+  a.csmall = p.cout; a.sd = out[0]; a.sh = out[1]; a.sw = out[2];
+  return a;
+}
+
+bool fwd_uses_patch(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return is_patch(p) && patch_supported(patch_args(p, out), dtype);
+}
+
+bool wgrad_uses_patch(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return is_patch(p) && patch_reduce_supported(patch_args(p, out), dtype);
+}
+
+// Weight of the strided convolution in fragment order: produced = Cout, reduced = Cin.
+MfmaConvArgs patch_pack_args(int produced, int reduced) {
+  MfmaConvArgs a{};
+  a.cout = produced; a.cred = reduced; a.kd = 2; a.kh = 2; a.kw = 2;
+  return a;
+}
+
+PatchArgs convT_patch_args(const sfh_convT3d_desc& p) {
+  PatchArgs a{};
+  a.n = p.n;
+  a.cbig = p.cout; a.bd = 2 * p.in_d; a.bh = 2 * p.in_h; a.bw = 2 * p.in_w;
+  a.csmall = p.cin; a.sd = p.in_d; a.sh = p.in_h; a.sw = p.in_w;
+  return a;
+}
+
+bool convT_uses_patch(const sfh_convT3d_desc& p, int dtype) {
+  return p.kd == 2 && p.kh == 2 && p.kw == 2 && p.n >= 1 && patch_supported(convT_patch_args(p), dtype);
 }
 
 // ---- thin-channel problems (Cin == 1 stems, 1x1x1 heads) ---------------------------------------
@@ -211,15 +254,16 @@ extern "C" int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]
 extern "C" int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (direction == 0) return fwd_uses_mfma(*p, dtype, out) ? 1 : 0;
+  if (direction == 0) return (fwd_uses_mfma(*p, dtype, out) || fwd_uses_patch(*p, dtype, out)) ? 1 : 0;
   if (direction == 1) return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)) ? 1 : 0;
-  return wgrad_uses_mfma(*p, dtype, out) ? 1 : 0;
+  return (wgrad_uses_mfma(*p, dtype, out) || wgrad_uses_patch(*p, dtype, out)) ? 1 : 0;
 }
 
 // ---- forward ---------------------------------------------------------------------------
 extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (fwd_uses_patch(*p, dtype, out)) return mfma_conv_packed_weight_bytes(patch_pack_args(p->cout, p->cin));
   if (!fwd_uses_mfma(*p, dtype, out)) return 0;
   return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out));
 }
@@ -239,6 +283,15 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, st);
+  }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_patch(*p, dtype, out)) {
+    const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);
+    const size_t need = mfma_conv_packed_weight_bytes(pk);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    if (int rc = mfma_pack_weight(pk, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
+      return rc;
+    return patch_gather(patch_args(*p, out), dtype, x, workspace, bias, y, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
     ThinArgs t;
@@ -316,6 +369,7 @@ extern "C" int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_splits(wgrad_args(*p, out));
+  if (wgrad_uses_patch(*p, dtype, out)) return patch_reduce_splits(patch_args(*p, out));
   ThinArgs t;
   bool thin_is_x;
   if (thin_wgrad_plan(*p, dtype, out, t, thin_is_x) == kThinReduce) return thin_reduce_splits(t);
@@ -326,6 +380,7 @@ extern "C" size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_workspace_bytes(wgrad_args(*p, out));
+  if (wgrad_uses_patch(*p, dtype, out)) return patch_reduce_workspace_bytes(patch_args(*p, out));
   ThinArgs t;
   bool thin_is_x;
   if (thin_wgrad_plan(*p, dtype, out, t, thin_is_x) == kThinReduce) return thin_reduce_workspace_bytes(t);
@@ -344,6 +399,13 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     return mfma_wgrad(a, dtype, x, gy, gw, workspace, st);
+  }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_patch(*p, dtype, out)) {
+    const PatchArgs a = patch_args(*p, out);
+    const size_t need = patch_reduce_workspace_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    return patch_reduce(a, dtype, gy, x, gw, workspace, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
     ThinArgs t;
@@ -374,15 +436,26 @@ static int check_convT(const sfh_convT3d_desc* p, int dtype) {
 
 extern "C" size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int dtype) {
   if (check_convT(p, dtype) != SFH_OK) return 0;
+  if (convT_uses_patch(*p, dtype)) return mfma_conv_packed_weight_bytes(patch_pack_args(p->cout, p->cin));
   return 0;
 }
 
 extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
                                const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
-  (void)workspace; (void)workspace_bytes; (void)flags;
   if (int rc = check_convT(p, dtype)) return rc;
   if (x == nullptr || w == nullptr || y == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
   if (p->n == 0) return SFH_OK;
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && convT_uses_patch(*p, dtype)) {
+    // produced channel = Cout (w_stride[1]), reduced channel = Cin (w_stride[0])
+    const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);
+    const size_t need = mfma_conv_packed_weight_bytes(pk);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "convT3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    if (int rc = mfma_pack_weight(pk, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
+      return rc;
+    return patch_scatter(convT_patch_args(*p), dtype, x, workspace, bias, y, st);
+  }
   return direct_convT(*p, dtype, w_stride, x, w, bias, y, (hipStream_t)stream);
 }
 

@@ -1,0 +1,344 @@
+// MFMA kernels for 2x2x2, stride-2, unpadded convolutions between a BIG and a SMALL volume: the U-Net's
+// transposed up-convolution (triton_conv3d/transposed.py:135-319), its data gradient (a stride-2
+// convolution, transposed.py:1073) and its weight gradient (transposed.py:1113).
+//
+// Windows do not overlap, so there is no halo and nothing to reuse between neighbouring voxels: the
+// three kernels are HBM-bound GEMMs with M = small voxels. The gather and the scatter take both MFMA
+// operands straight from global memory (a lane's fragment is 8 consecutive channels of one voxel, one
+// 16-byte load; the weight is pre-packed in fragment order and stays in L1/L2). The weight gradient
+// contracts over voxels, so both operands must be transposed: tiles are staged in LDS in their natural
+// [voxel][channel] layout and read with ds_read_b64_tr_b16, which hands each lane four consecutive
+// voxels of one channel.
+#include "conv_patch.hpp"
+#include "mma.hpp"
+
+namespace sfh {
+namespace {
+
+constexpr int kTaps = 8;
+
+struct Voxel { int nn, d, h, w; };
+
+__device__ __forceinline__ Voxel decode_small(const PatchArgs& a, int64_t v) {
+  Voxel r;
+  if (v <= 0x7fffffffLL) {  // 32-bit arithmetic when it fits
+    uint32_t t = (uint32_t)v;
+    r.w = (int)(t % (uint32_t)a.sw); t /= (uint32_t)a.sw;
+    r.h = (int)(t % (uint32_t)a.sh); t /= (uint32_t)a.sh;
+    r.d = (int)(t % (uint32_t)a.sd);
+    r.nn = (int)(t / (uint32_t)a.sd);
+    return r;
+  }
+  r.w = (int)(v % a.sw);
+  int64_t t = v / a.sw;
+  r.h = (int)(t % a.sh);
+  t /= a.sh;
+  r.d = (int)(t % a.sd);
+  r.nn = (int)(t / a.sd);
+  return r;
+}
+
+__device__ __forceinline__ int64_t big_index(const PatchArgs& a, const Voxel& v, int tap) {
+  return (((int64_t)v.nn * a.bd + 2 * v.d + (tap >> 2)) * a.bh + 2 * v.h + ((tap >> 1) & 1)) * a.bw + 2 * v.w + (tap & 1);
+}
+
+template <typename T>
+__device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// Stores result block `acc` (32 produced channels x 32 voxels): this lane's voxel row starts at `row`
+// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given.
+template <typename T>
+__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg) {
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int c = 8 * g + 4 * kg;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = acc[4 * g + i] + (bias != nullptr ? to_float(bias[c0 + c + i]) : 0.f);
+    uint2 o;
+    o.x = Mma32<T>::pack2(v[0], v[1]);
+    o.y = Mma32<T>::pack2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(row + c) = o;
+  }
+}
+
+// ---- gather: stride-2 convolution --------------------------------------------------------------
+// A wavefront owns 32 small voxels x NB blocks of 32 produced channels. grid = (voxel tiles of 128, groups of NB blocks).
+template <typename T, int NB>
+__global__ void __launch_bounds__(256) patch_gather_kernel(PatchArgs a, const T* __restrict__ big, const T* __restrict__ packed,
+                                                           const T* __restrict__ bias, T* __restrict__ small, int64_t total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 5;
+  const int64_t v = (int64_t)blockIdx.x * 128 + wave * 32 + (lane & 31);
+  const bool valid = v < total;
+  const Voxel vx = decode_small(a, valid ? v : total - 1);
+  const int nchunks = a.cbig / 32;
+  const int blk0 = blockIdx.y * NB;
+  f32x16_t acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+  for (int tap = 0; tap < kTaps; ++tap) {
+    const T* src = big + big_index(a, vx, tap) * a.cbig + kg * 8;
+    for (int cc = 0; cc < nchunks; ++cc) {
+      uint4 bf[2], wf[2][NB];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        bf[ks] = load16(src + cc * 32 + ks * 16);
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          wf[ks][b] = load16(packed + (((((int64_t)(blk0 + b) * nchunks + cc) * kTaps + tap) * 2 + ks) * 64 + lane) * 8);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) acc[b] = Mma32<T>::run(wf[ks][b], bf[ks], acc[b]);
+    }
+  }
+  if (!valid) return;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) store_block<T>(acc[b], small + v * a.csmall + (blk0 + b) * 32, bias, (blk0 + b) * 32, kg);
+}
+
+// ---- scatter: transposed convolution -----------------------------------------------------------
+// A wavefront owns 32 small voxels x one block of 32 big channels x all 8 taps. grid = (voxel tiles of 128, cbig / 32).
+template <typename T>
+__global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T* __restrict__ small, const T* __restrict__ packed,
+                                                            const T* __restrict__ bias, T* __restrict__ big, int64_t total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 5;
+  const int64_t v = (int64_t)blockIdx.x * 128 + wave * 32 + (lane & 31);
+  const bool valid = v < total;
+  const int64_t vc = valid ? v : total - 1;
+  const int nchunks = a.csmall / 32;
+  const int blk = blockIdx.y;
+  f32x16_t acc[kTaps];
+#pragma unroll
+  for (int t = 0; t < kTaps; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  const T* src = small + vc * a.csmall + kg * 8;
+  for (int cc = 0; cc < nchunks; ++cc) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const uint4 sf = load16(src + cc * 32 + ks * 16);
+      uint4 wf[kTaps];
+#pragma unroll
+      for (int t = 0; t < kTaps; ++t)
+        wf[t] = load16(packed + (((((int64_t)blk * nchunks + cc) * kTaps + t) * 2 + ks) * 64 + lane) * 8);
+#pragma unroll
+      for (int t = 0; t < kTaps; ++t) acc[t] = Mma32<T>::run(wf[t], sf, acc[t]);
+    }
+  }
+  if (!valid) return;
+  const Voxel vx = decode_small(a, v);
+#pragma unroll
+  for (int t = 0; t < kTaps; ++t) store_block<T>(acc[t], big + big_index(a, vx, t) * a.cbig + blk * 32, bias, blk * 32, kg);
+}
+
+// ---- reduce: weight gradient -------------------------------------------------------------------
+constexpr int kVx = 32;             // voxels staged per round (two k-steps of 16)
+constexpr int kSmallTile = 64;      // small channels per workgroup (two row blocks)
+constexpr int kSRow = kSmallTile + 8;  // LDS row strides in elements: 16-byte aligned, off the 128-byte period
+constexpr int kBRow = 32 + 8;
+
+// Operand fragment (32 channels x 16 voxels) from a natural-layout LDS tile: `tile` points at the first
+// of the 16 voxel rows, channel 0 of the block. Within each group of 16 lanes the transposing read takes
+// lane m's address as (voxel m / 4, channels 4 * (m % 4) .. + 3) and returns to lane m channel m of the
+// four voxels, so two reads give a lane its 8 voxels of the k-step.
+template <typename T>
+__device__ __forceinline__ uint4 tr_fragment(const T* tile, int row_stride, int lane) {
+  typedef short v4s __attribute__((__vector_size__(4 * sizeof(short))));
+  const int g = lane >> 4, m = lane & 15;
+  const T* p0 = tile + ((g >> 1) * 8 + (m >> 2)) * row_stride + (g & 1) * 16 + 4 * (m & 3);
+  const T* p1 = p0 + 4 * row_stride;
+  const v4s r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p0));
+  const v4s r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)(p1));
+  uint4 out;
+  out.x = __builtin_bit_cast(uint2, r0).x; out.y = __builtin_bit_cast(uint2, r0).y;
+  out.z = __builtin_bit_cast(uint2, r1).x; out.w = __builtin_bit_cast(uint2, r1).y;
+  return out;
+}
+
+// grid = (splits, csmall / 64, cbig / 32). Wavefront w accumulates taps 2w and 2w + 1 for both row blocks.
+template <typename T>
+__global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T* __restrict__ small, const T* __restrict__ big,
+                                                           float* __restrict__ part, int64_t total, int64_t per_split) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) T s_tile[kVx * kSRow];
+  __shared__ __attribute__((aligned(16))) T b_tile[kTaps * kVx * kBRow];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int cs0 = blockIdx.y * kSmallTile, cb0 = blockIdx.z * 32;
+  const int64_t begin = (int64_t)blockIdx.x * per_split;
+  int64_t end = begin + per_split;
+  if (end > total) end = total;
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  const int s_vox = tid >> 3, s_piece = tid & 7;          // small tile: 32 voxels x 8 pieces of 16 bytes
+  const int b_vox = (tid >> 2) & 31, b_piece = tid & 3;   // big tiles: 4 taps (tid/128, +2, +4, +6) of one voxel
+  const int b_tap0 = tid >> 7;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int64_t v0 = begin; v0 < end; v0 += kVx) {
+    uint4 sv = zero, bv[4] = {zero, zero, zero, zero};
+    if (v0 + s_vox < end) sv = load16(small + (v0 + s_vox) * a.csmall + cs0 + s_piece * 8);
+    if (v0 + b_vox < end) {
+      const Voxel vx = decode_small(a, v0 + b_vox);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) bv[i] = load16(big + big_index(a, vx, b_tap0 + 2 * i) * a.cbig + cb0 + b_piece * 8);
+    }
+    __syncthreads();  // the previous round's reads are done
+    *reinterpret_cast<uint4*>(s_tile + s_vox * kSRow + s_piece * 8) = sv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<uint4*>(b_tile + ((b_tap0 + 2 * i) * kVx + b_vox) * kBRow + b_piece * 8) = bv[i];
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      uint4 af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = tr_fragment<T>(s_tile + ks * 16 * kSRow + i * 32, kSRow, lane);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[j] = tr_fragment<T>(b_tile + ((2 * wave + j) * kVx + ks * 16) * kBRow, kBRow, lane);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mma32<T>::run(af[i], bf[j], acc[i][j]);
+    }
+  }
+  // part[split][cs][tap][cb]: a lane holds column cb = lane % 32 and 16 rows of each block
+  float* dst = part + (int64_t)blockIdx.x * a.csmall * kTaps * a.cbig;
+  const int col = lane & 31, kg = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int cs = cs0 + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
+        dst[((int64_t)cs * kTaps + 2 * wave + j) * a.cbig + cb0 + col] = acc[i][j][r];
+      }
+#endif
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) patch_reduce_finalize(const float* __restrict__ part, T* __restrict__ g, int64_t nelem,
+                                                             int splits) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= nelem) return;
+  float s = 0.f;
+  for (int sp = 0; sp < splits; ++sp) s += part[(int64_t)sp * nelem + e];
+  g[e] = elem<T>::from_float(s);
+}
+
+int64_t small_voxels(const PatchArgs& a) { return (int64_t)a.n * a.sd * a.sh * a.sw; }
+
+// Produced-channel blocks per wavefront: as many as keep at least two wavefronts per SIMD busy.
+int gather_blocks(const PatchArgs& a) {
+  const int nblk = a.csmall / 32;
+  const int64_t wave_tiles = cdiv(small_voxels(a), 32);
+  int nb = 8;
+  while (nb > 1 && (nblk % nb != 0 || wave_tiles * (nblk / nb) < 2048)) nb >>= 1;
+  return nb;
+}
+
+template <typename T>
+int launch_gather(const PatchArgs& a, const void* big, const void* packed, const void* bias, void* small, hipStream_t st) {
+  const int64_t total = small_voxels(a);
+  const int nb = gather_blocks(a);
+  const dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.csmall / 32 / nb));
+#define SFH_PATCH_GATHER(NB)                                                                                              \
+  hipLaunchKernelGGL((patch_gather_kernel<T, NB>), grid, dim3(256), 0, st, a, (const T*)big, (const T*)packed, (const T*)bias, \
+                     (T*)small, total)
+  if (nb == 8) SFH_PATCH_GATHER(8);
+  else if (nb == 4) SFH_PATCH_GATHER(4);
+  else if (nb == 2) SFH_PATCH_GATHER(2);
+  else SFH_PATCH_GATHER(1);
+#undef SFH_PATCH_GATHER
+  return check_launch("patch_gather_kernel");
+}
+
+template <typename T>
+int launch_scatter(const PatchArgs& a, const void* small, const void* packed, const void* bias, void* big, hipStream_t st) {
+  const int64_t total = small_voxels(a);
+  const dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
+  hipLaunchKernelGGL((patch_scatter_kernel<T>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
+                     (T*)big, total);
+  return check_launch("patch_scatter_kernel");
+}
+
+struct ReducePlan { int splits; int64_t per_split; };
+
+ReducePlan reduce_plan(const PatchArgs& a) {
+  const int64_t total = small_voxels(a);
+  const int64_t tiles = (int64_t)(a.csmall / kSmallTile) * (a.cbig / 32);
+  const int64_t rounds = cdiv(total, kVx);
+  int64_t splits = cdiv(4 * kComputeUnits, tiles);
+  if (splits > rounds) splits = rounds;
+  if (splits < 1) splits = 1;
+  ReducePlan p;
+  p.per_split = cdiv(rounds, splits) * kVx;
+  p.splits = (int)cdiv(total, p.per_split);
+  return p;
+}
+
+template <typename T>
+int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* g, void* ws, hipStream_t st) {
+  const ReducePlan p = reduce_plan(a);
+  const int64_t total = small_voxels(a);
+  const dim3 grid((unsigned)p.splits, (unsigned)(a.csmall / kSmallTile), (unsigned)(a.cbig / 32));
+  hipLaunchKernelGGL((patch_reduce_kernel<T>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)big, (float*)ws, total,
+                     p.per_split);
+  if (int rc = check_launch("patch_reduce_kernel")) return rc;
+  const int64_t nelem = (int64_t)a.csmall * kTaps * a.cbig;
+  hipLaunchKernelGGL((patch_reduce_finalize<T>), dim3((unsigned)cdiv(nelem, 256)), dim3(256), 0, st, (const float*)ws, (T*)g, nelem,
+                     p.splits);
+  return check_launch("patch_reduce_finalize");
+}
+
+bool geometry_ok(const PatchArgs& a, int dtype) {
+  if (dtype != SFH_BF16 && dtype != SFH_FP16) return false;
+  if (a.n < 1 || a.sd < 1 || a.sh < 1 || a.sw < 1) return false;
+  if (a.bd < 2 * a.sd || a.bh < 2 * a.sh || a.bw < 2 * a.sw) return false;
+  if (cdiv(small_voxels(a), 128) > 0x7fffffffLL) return false;
+  return true;
+}
+
+}  // namespace
+
+bool patch_supported(const PatchArgs& a, int dtype) {
+  return geometry_ok(a, dtype) && a.cbig % 32 == 0 && a.csmall % 32 == 0 && a.cbig / 32 <= 65535 && a.csmall / 32 <= 65535;
+}
+
+bool patch_reduce_supported(const PatchArgs& a, int dtype) {
+  return geometry_ok(a, dtype) && a.cbig % 32 == 0 && a.csmall % kSmallTile == 0 && a.cbig / 32 <= 65535 &&
+         a.csmall / kSmallTile <= 65535;
+}
+
+int patch_gather(const PatchArgs& a, int dtype, const void* big, const void* packed, const void* bias, void* small, hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_gather<bf16_t>(a, big, packed, bias, small, st);
+  return launch_gather<fp16_t>(a, big, packed, bias, small, st);
+}
+
+int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_scatter<bf16_t>(a, small, packed, bias, big, st);
+  return launch_scatter<fp16_t>(a, small, packed, bias, big, st);
+}
+
+int patch_reduce_splits(const PatchArgs& a) { return reduce_plan(a).splits; }
+
+size_t patch_reduce_workspace_bytes(const PatchArgs& a) {
+  return (size_t)reduce_plan(a).splits * a.csmall * kTaps * a.cbig * sizeof(float);
+}
+
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, void* ws, hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_reduce<bf16_t>(a, small, big, g, ws, st);
+  return launch_reduce<fp16_t>(a, small, big, g, ws, st);
+}
+
+}  // namespace sfh

@@ -1,0 +1,30 @@
+// Host-side interface of the MFMA kernels for 2x2x2, stride-2, unpadded convolutions: the U-Net's
+// transposed up-convolution and its two gradients (bf16 / fp16).
+#pragma once
+#include "common.hpp"
+
+namespace sfh {
+
+// A BIG volume (cbig channels, extents bd x bh x bw) and a SMALL one (csmall channels, extents
+// sd x sh x sw, 2 * s? <= b?): small voxel v and tap (a,b,c) in {0,1}^3 meet big voxel 2v + tap.
+//   gather  : small[v][cs] = bias[cs] + sum_{tap,cb} big[2v+tap][cb] * W(cs, cb, tap)     (conv, stride 2)
+//   scatter : big[2v+tap][cb] = bias[cb] + sum_cs small[v][cs] * W(cs, cb, tap)            (transposed conv)
+//   reduce  : G[cs][tap][cb] = sum_v small[v][cs] * big[2v+tap][cb]                         (weight gradient)
+struct PatchArgs {
+  int n;
+  int cbig, bd, bh, bw;
+  int csmall, sd, sh, sw;
+};
+
+bool patch_supported(const PatchArgs& a, int dtype);         // gather and scatter
+bool patch_reduce_supported(const PatchArgs& a, int dtype);
+// `packed` holds the weight in MFMA fragment order [produced/32][reduced/32][tap][kstep][lane][8]
+// (mfma_pack_weight): produced = csmall for gather, cbig for scatter.
+int patch_gather(const PatchArgs& a, int dtype, const void* big, const void* packed, const void* bias, void* small, hipStream_t st);
+int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st);
+int patch_reduce_splits(const PatchArgs& a);
+size_t patch_reduce_workspace_bytes(const PatchArgs& a);
+// g: dense [csmall][8][cbig] in the element type, from fp32 partial slices in ws summed in split order
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, void* ws, hipStream_t st);
+
+}  // namespace sfh

@@ -203,17 +203,36 @@ CONVT_SHAPES = [
     (2, 64, 32, (3, 5, 6), (2, 2, 2), True),
     (1, 5, 7, (2, 3, 4), (2, 2, 2), False),
     (1, 8, 8, (2, 2, 3), (1, 2, 3), True),
+    # the MFMA 2x2x2 family: every U-Net up-convolution channel pair, ragged voxel counts
+    (1, 512, 256, (2, 3, 4), (2, 2, 2), True),
+    (1, 256, 128, (3, 5, 7), (2, 2, 2), False),
+    (1, 64, 32, (9, 6, 11), (2, 2, 2), True),
+    (2, 64, 96, (4, 4, 5), (2, 2, 2), False),
+    (1, 32, 32, (1, 1, 1), (2, 2, 2), True),
 ]
 
 
 @pytest.mark.parametrize("direction", DIRS)
 @pytest.mark.parametrize("n,cin,cout,spatial,kernel,bias", CONVT_SHAPES)
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_transposed_exact(device, dtype, n, cin, cout, spatial, kernel, bias, direction):
     prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, kernel=kernel, stride=kernel, padding=(0, 0, 0),
                            transposed=True, bias=bias, dtype=dtype)
     got = check_exact(prob, direction, device)
     assert tuple(got.shape) == {"fwd": prob.output_shape, "bwd-data": prob.input_shape, "bwd-weight": prob.weight_shape}[direction]
+    # the direct kernels must give the same bits on the same exact draw
+    assert torch.equal(got, check_exact(prob, direction, device, force_generic=True))
+
+
+@pytest.mark.parametrize("direction", DIRS)
+def test_transposed_gaussian_tolerance(device, direction):
+    """cfg4's up-convolution (128 -> 64) at Gaussian operands, bf16: 2e-2 relative + 1e-2 absolute."""
+    prob = orc.ConvProblem(n=1, cin=128, cout=64, spatial=(8, 8, 8), kernel=(2, 2, 2), stride=(2, 2, 2), padding=(0, 0, 0),
+                           transposed=True, bias=True, dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=40)
+    ops["weight"] = (ops["weight"].float() / (prob.cin * 8) ** 0.5).to(torch.bfloat16)
+    got = run(prob, ops, direction, device)
+    orc.assert_baseline_tolerance(got, orc.conv_reference(prob, ops, direction), torch.bfloat16, direction)
 
 
 def test_transposed_bias_is_per_channel_not_per_tap(device):
