@@ -107,6 +107,15 @@ size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
 int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw,
                      void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
+/* ---- bias gradient --------------------------------------------------------------------
+ * Stands in for `grad_output.sum((0, 2, 3, 4))` in the reference's autograd functions
+ * (ScaFFold/unet/conv3d.py:1231 for conv3d, :1786 for the transposed conv).
+ * g: dense (rows, channels) of `dtype` (rows = N*D*H*W of a channels-last gradient);
+ * gb: `channels` elements of `out_dtype`; fp32 accumulation in a fixed order. */
+size_t sfh_bias_grad_workspace_bytes(int64_t rows, int32_t channels);
+int sfh_bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int32_t channels, void* gb,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- transposed conv3d (kernel == stride) forward ------------------------------------
  * Stands in for triton_conv3d.conv_transpose3d_forward (triton_conv3d/transposed.py:941)
  * and _convT3d_fwd_kernel (:135).

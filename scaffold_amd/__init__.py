@@ -18,7 +18,7 @@ _EXPORTS = {
     "conv3d_forward": "conv3d", "conv3d_backward_data": "conv3d", "conv3d_backward_weight": "conv3d",
     "is_supported": "conv3d", "is_supported_all": "conv3d", "is_supported_bwd_data": "conv3d",
     "is_supported_bwd_weight": "conv3d", "bwd_data_padding": "conv3d", "grad_weight_empty": "conv3d",
-    "workspace_elements": "conv3d", "split_count": "conv3d",
+    "workspace_elements": "conv3d", "split_count": "conv3d", "bias_grad": "conv3d",
     "conv_transpose3d_forward": "transposed", "conv_transpose3d_backward_data": "transposed",
     "conv_transpose3d_backward_weight": "transposed", "is_supported_transposed": "transposed",
     "is_supported_transposed_all": "transposed", "is_supported_transposed_bwd_data": "transposed",

@@ -41,6 +41,7 @@ __all__ = [
     "conv3d_forward",
     "conv3d_backward_data",
     "conv3d_backward_weight",
+    "bias_grad",
     "is_supported",
     "is_supported_all",
     "is_supported_bwd_data",
@@ -271,6 +272,32 @@ def grad_weight_empty(cout: int, cin: int, kernel: Sequence[int], *, dtype, devi
     ``[Cout][kd][kh][kw][Cin]`` in memory, i.e. ``channels_last_3d``."""
     k = _triple(kernel, "kernel")
     return torch.empty((cout, cin, *k), dtype=dtype, device=device, memory_format=_CL3D)
+
+
+def bias_grad(grad_output: torch.Tensor, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Bias gradient of a (transposed) convolution: ``grad_output.sum((0, 2, 3, 4))`` with fp32 accumulation in a
+    fixed order, rounded once to ``dtype`` (default: ``grad_output``'s) -- the expression the reference's autograd
+    functions use (``ScaFFold/unet/conv3d.py:1231``, ``:1786``)."""
+    if not isinstance(grad_output, torch.Tensor) or grad_output.dim() != 5 or not grad_output.is_cuda \
+            or grad_output.dtype not in _lib.SUPPORTED_DTYPES:
+        raise NotImplementedError(f"unsupported: grad_output={getattr(grad_output, 'shape', None)}/"
+                                  f"{getattr(grad_output, 'dtype', None)}")
+    out_dtype = grad_output.dtype if dtype is None else dtype
+    if out_dtype not in _lib.SUPPORTED_DTYPES:
+        raise NotImplementedError(f"unsupported bias dtype {out_dtype}")
+    g = grad_output.contiguous(memory_format=_CL3D)
+    n, c, d, h, w = (int(v) for v in g.shape)
+    gb = torch.empty((c,), dtype=out_dtype, device=g.device)
+    rows = n * d * h * w
+    if rows == 0:
+        return gb.zero_()
+    L = _lib.lib()
+    with torch.cuda.device(g.device):
+        ws = _lib.workspace(int(L.sfh_bias_grad_workspace_bytes(rows, c)), g.device)
+        rc = L.sfh_bias_grad(_lib.dtype_code(g.dtype), _lib.dtype_code(out_dtype), _lib.ptr(g), rows, c, _lib.ptr(gb),
+                             _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(g.device))
+    _lib.check(rc, "bias_grad")
+    return gb
 
 
 # ---------------------------------------------------------------------------------------------

@@ -7,6 +7,7 @@
 #include "conv_mfma.hpp"
 #include "conv_patch.hpp"
 #include "conv_thin.hpp"
+#include "reduce.hpp"
 #include "wgrad_mfma.hpp"
 
 namespace sfh {
@@ -423,6 +424,23 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
   a.kd = p->kd; a.kh = p->kh; a.kw = p->kw; a.sd = p->sd; a.sh = p->sh; a.sw = p->sw;
   a.pd = p->pd; a.ph = p->ph; a.pw = p->pw; a.dd = p->dd; a.dh = p->dh; a.dw = p->dw;
   return direct_conv_wgrad(a, dtype, x, gy, gw, st);
+}
+
+// ---- bias gradient ---------------------------------------------------------------------
+extern "C" size_t sfh_bias_grad_workspace_bytes(int64_t rows, int32_t channels) {
+  if (rows < 1 || channels < 1) return 0;
+  return bias_grad_workspace_bytes(rows, channels);
+}
+
+extern "C" int sfh_bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int32_t channels, void* gb, void* workspace,
+                             size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype) || !dtype_ok(out_dtype)) return fail(SFH_ERR_INVALID, "bias grad: bad dtype %d / %d", dtype, out_dtype);
+  if (rows < 1 || channels < 1) return fail(SFH_ERR_INVALID, "bias grad: bad extents rows=%lld channels=%d", (long long)rows, channels);
+  if (g == nullptr || gb == nullptr) return fail(SFH_ERR_INVALID, "bias grad: null tensor");
+  const size_t need = bias_grad_workspace_bytes(rows, channels);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "bias grad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  return bias_grad(dtype, out_dtype, g, rows, channels, gb, workspace, (hipStream_t)stream);
 }
 
 // ---- transposed convolution ------------------------------------------------------------

@@ -11,6 +11,7 @@
 // voxels of one channel.
 #include "conv_patch.hpp"
 #include "mma.hpp"
+#include "reduce.hpp"
 
 namespace sfh {
 namespace {
@@ -226,16 +227,6 @@ __global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T*
 #endif
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) patch_reduce_finalize(const float* __restrict__ part, T* __restrict__ g, int64_t nelem,
-                                                             int splits) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= nelem) return;
-  float s = 0.f;
-  for (int sp = 0; sp < splits; ++sp) s += part[(int64_t)sp * nelem + e];
-  g[e] = elem<T>::from_float(s);
-}
-
 int64_t small_voxels(const PatchArgs& a) { return (int64_t)a.n * a.sd * a.sh * a.sw; }
 
 // Produced-channel blocks per wavefront: as many as keep at least two wavefronts per SIMD busy.
@@ -296,9 +287,7 @@ int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* 
                      p.per_split);
   if (int rc = check_launch("patch_reduce_kernel")) return rc;
   const int64_t nelem = (int64_t)a.csmall * kTaps * a.cbig;
-  hipLaunchKernelGGL((patch_reduce_finalize<T>), dim3((unsigned)cdiv(nelem, 256)), dim3(256), 0, st, (const float*)ws, (T*)g, nelem,
-                     p.splits);
-  return check_launch("patch_reduce_finalize");
+  return sum_slices(__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16, (const float*)ws, g, nelem, p.splits, st);
 }
 
 bool geometry_ok(const PatchArgs& a, int dtype) {

@@ -13,6 +13,7 @@
 // The reference serves these shapes with the same implicit-GEMM kernels at small tile sizes
 // (triton_conv3d/gather_gemm.py:493-560, reduce_gemm.py:655-700).
 #include "conv_thin.hpp"
+#include "reduce.hpp"
 #include "vec_io.hpp"
 
 namespace sfh {
@@ -142,8 +143,8 @@ __global__ void __launch_bounds__(kBlock) thin_out_kernel(ThinArgs a, const T* _
 
 // ---- reduce (weight gradient) ----------------------------------------------------------------
 // Thread = (voxel row, V wide channels) with J x V fp32 accumulators; a workgroup owns a contiguous
-// voxel range and leaves one fp32 partial slice part[split][J][cw]; thin_reduce_finalize sums the
-// slices in a fixed order.
+// voxel range and leaves one fp32 partial slice, already in the layout of the weight gradient; the
+// slices are then summed in a fixed order.
 template <typename T, int K, int J>
 __global__ void __launch_bounds__(kBlock) thin_reduce_kernel(ThinArgs a, const T* __restrict__ thin, const T* __restrict__ wide,
                                                              float* __restrict__ part, int64_t total, int64_t per_split) {
@@ -177,7 +178,7 @@ __global__ void __launch_bounds__(kBlock) thin_reduce_kernel(ThinArgs a, const T
     }
   }
   // Fold the voxel rows: JC thin values at a time through LDS, columns summed in row order.
-  float* dst = part + (int64_t)blockIdx.x * J * a.cw;
+  float* dst = part + (int64_t)blockIdx.x * a.J * a.cw;
 #pragma unroll
   for (int j0 = 0; j0 < J; j0 += JC) {
     __syncthreads();
@@ -190,24 +191,13 @@ __global__ void __launch_bounds__(kBlock) thin_reduce_kernel(ThinArgs a, const T
     __syncthreads();
     for (int i = tid; i < JC * a.cw; i += kBlock) {
       const int jj = i / a.cw, c = i - jj * a.cw;
-      if (j0 + jj < J) {
+      if (j0 + jj < a.J) {
         float sum = 0.f;
         for (int rr = 0; rr < rpp; ++rr) sum += buf[(jj * rpp + rr) * a.cw + c];
-        dst[(j0 + jj) * a.cw + c] = sum;
+        dst[(int64_t)c * a.so_wide + (int64_t)(j0 + jj) * a.so_thin] = sum;
       }
     }
   }
-}
-
-template <typename T, int J>
-__global__ void __launch_bounds__(kBlock) thin_reduce_finalize(ThinArgs a, const float* __restrict__ part, T* __restrict__ gw,
-                                                               int nsplit) {
-  const int i = blockIdx.x * kBlock + threadIdx.x;
-  if (i >= a.J * a.cw) return;
-  const int j = i / a.cw, c = i - j * a.cw;
-  float s = 0.f;
-  for (int sp = 0; sp < nsplit; ++sp) s += part[((int64_t)sp * J + j) * a.cw + c];
-  gw[(int64_t)c * a.so_wide + (int64_t)j * a.so_thin] = elem<T>::from_float(s);
 }
 
 int wide_channels_ok(const ThinArgs& a, int dtype) {
@@ -247,9 +237,8 @@ int launch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* g
   hipLaunchKernelGGL((thin_reduce_kernel<T, K, J>), dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide,
                      (float*)ws, total, per);
   if (int rc = check_launch("thin_reduce_kernel")) return rc;
-  hipLaunchKernelGGL((thin_reduce_finalize<T, J>), dim3((unsigned)cdiv((int64_t)a.J * a.cw, kBlock)), dim3(kBlock), 0, st, a,
-                     (const float*)ws, (T*)gw, nsplit);
-  return check_launch("thin_reduce_finalize");
+  const int dtype = sizeof(T) == 4 ? SFH_FP32 : (__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16);
+  return sum_slices(dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
 }
 
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
@@ -293,8 +282,7 @@ int thin_reduce_splits(const ThinArgs& a) {
 }
 
 size_t thin_reduce_workspace_bytes(const ThinArgs& a) {
-  const int jpad = a.K == 3 ? 27 : a.K == 2 ? 8 : a.J <= 4 ? 4 : a.J <= 16 ? 16 : 32;
-  return (size_t)thin_reduce_splits(a) * jpad * a.cw * sizeof(float);
+  return (size_t)thin_reduce_splits(a) * a.J * a.cw * sizeof(float);
 }
 
 #define SFH_THIN_BY_DTYPE(fn, ...)                         \

@@ -1,0 +1,136 @@
+// Deterministic fp32 reductions: the sum over split-K partial slices, and per-channel sums of a
+// channels-last tensor (the bias gradient, ScaFFold/unet/conv3d.py:1231,1786). No atomics: every
+// partial has a fixed slot and every sum a fixed order, so a call gives the same bits every time.
+#include "reduce.hpp"
+
+namespace sfh {
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_flat(const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
+                                                          int splits) {
+  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (e >= nelem) return;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int sp = 0;
+  for (; sp + 3 < splits; sp += 4) {
+    s0 += part[(int64_t)sp * nelem + e];
+    s1 += part[(int64_t)(sp + 1) * nelem + e];
+    s2 += part[(int64_t)(sp + 2) * nelem + e];
+    s3 += part[(int64_t)(sp + 3) * nelem + e];
+  }
+  for (; sp < splits; ++sp) s0 += part[(int64_t)sp * nelem + e];
+  out[e] = elem<T>::from_float((s0 + s1) + (s2 + s3));
+}
+
+// Many slices, few elements: 16 elements x 16 slice lanes per workgroup; lane l sums slices l, l+16, ...
+// and the 16 lane totals are added in lane order.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_grouped(const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
+                                                             int splits) {
+  __shared__ float buf[16][17];
+  const int el = threadIdx.x & 15, sl = threadIdx.x >> 4;
+  const int64_t e = (int64_t)blockIdx.x * 16 + el;
+  float s = 0.f;
+  if (e < nelem)
+    for (int sp = sl; sp < splits; sp += 16) s += part[(int64_t)sp * nelem + e];
+  buf[sl][el] = s;
+  __syncthreads();
+  if (sl == 0 && e < nelem) {
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += buf[i][el];
+    out[e] = elem<T>::from_float(t);
+  }
+}
+
+template <typename T>
+int launch_sum(const float* part, void* out, int64_t nelem, int splits, hipStream_t st) {
+  if (nelem <= 0) return SFH_OK;
+  if (splits >= 32 && nelem <= (1 << 22)) {
+    hipLaunchKernelGGL(sum_slices_grouped<T>, dim3((unsigned)cdiv(nelem, 16)), dim3(kBlock), 0, st, part, (T*)out, nelem, splits);
+    return check_launch("sum_slices_grouped");
+  }
+  hipLaunchKernelGGL(sum_slices_flat<T>, dim3((unsigned)cdiv(nelem, kBlock)), dim3(kBlock), 0, st, part, (T*)out, nelem, splits);
+  return check_launch("sum_slices_flat");
+}
+
+// Per-channel partial sums: thread = (row slot, channel); a workgroup walks its row range with rpp rows per
+// pass (consecutive threads read consecutive elements), folds the row slots through LDS and writes
+// part[block][channel chunk]. Channel chunks of at most 256 lie along grid.y.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) channel_partial(const T* __restrict__ g, float* __restrict__ part, int64_t rows, int C,
+                                                          int64_t rows_per_block) {
+  __shared__ float buf[kBlock];
+  const int c0 = blockIdx.y * kBlock;
+  const int cw = (C - c0) < kBlock ? (C - c0) : kBlock;
+  const int rpp = kBlock / cw;
+  const int tid = threadIdx.x;
+  const int r = tid / cw, c = tid - r * cw;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_block;
+  int64_t end = begin + rows_per_block;
+  if (end > rows) end = rows;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (r < rpp) {
+    const T* p = g + c0 + c;
+    int64_t row = begin + r;
+    for (; row + 3 * (int64_t)rpp < end; row += 4 * (int64_t)rpp) {
+      s0 += to_float(p[row * C]);
+      s1 += to_float(p[(row + rpp) * C]);
+      s2 += to_float(p[(row + 2 * rpp) * C]);
+      s3 += to_float(p[(row + 3 * rpp) * C]);
+    }
+    for (; row < end; row += rpp) s0 += to_float(p[row * C]);
+  }
+  buf[tid] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (tid < cw) {
+    float t = 0.f;
+    for (int i = 0; i < rpp; ++i) t += buf[i * cw + tid];
+    part[(int64_t)blockIdx.x * C + c0 + tid] = t;
+  }
+}
+
+int bias_blocks(int64_t rows) {
+  int64_t n = cdiv(rows, 1024);
+  if (n > kComputeUnits * 4) n = kComputeUnits * 4;
+  return (int)(n < 1 ? 1 : n);
+}
+
+template <typename T>
+int launch_bias(const void* g, int64_t rows, int C, float* ws, hipStream_t st) {
+  const int nblk = bias_blocks(rows);
+  const int64_t per = cdiv(rows, nblk);
+  hipLaunchKernelGGL(channel_partial<T>, dim3((unsigned)nblk, (unsigned)cdiv(C, kBlock)), dim3(kBlock), 0, st, (const T*)g, ws, rows, C,
+                     per);
+  return check_launch("channel_partial");
+}
+
+}  // namespace
+
+int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st) {
+  switch (dtype) {
+    case SFH_BF16: return launch_sum<bf16_t>(part, out, nelem, splits, st);
+    case SFH_FP16: return launch_sum<fp16_t>(part, out, nelem, splits, st);
+    default: return launch_sum<float>(part, out, nelem, splits, st);
+  }
+}
+
+size_t bias_grad_workspace_bytes(int64_t rows, int channels) {
+  return (size_t)bias_blocks(rows) * channels * sizeof(float);
+}
+
+int bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int channels, void* gb, void* ws, hipStream_t st) {
+  int rc;
+  switch (dtype) {
+    case SFH_BF16: rc = launch_bias<bf16_t>(g, rows, channels, (float*)ws, st); break;
+    case SFH_FP16: rc = launch_bias<fp16_t>(g, rows, channels, (float*)ws, st); break;
+    default: rc = launch_bias<float>(g, rows, channels, (float*)ws, st); break;
+  }
+  if (rc != SFH_OK) return rc;
+  return sum_slices(out_dtype, (const float*)ws, gb, channels, bias_blocks(rows), st);
+}
+
+}  // namespace sfh

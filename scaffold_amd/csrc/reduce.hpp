@@ -1,0 +1,15 @@
+// Deterministic reductions shared by the weight-gradient kernels, and the bias gradient.
+#pragma once
+#include "common.hpp"
+
+namespace sfh {
+
+// out[e] = sum over s < splits, in index order within fixed groups, of part[s * nelem + e]; one rounding to `dtype`.
+int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st);
+
+// gb[c] = sum over rows of g[row * channels + c] for a dense (rows, channels) tensor of `dtype`; fp32
+// accumulation through partial slices in `ws`, result rounded once to `out_dtype`.
+size_t bias_grad_workspace_bytes(int64_t rows, int channels);
+int bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int channels, void* gb, void* ws, hipStream_t st);
+
+}  // namespace sfh

@@ -22,6 +22,7 @@
 // workgroup's K range are processed one after another; two workgroups per CU overlap one's
 // staging with the other's MFMAs.
 #include "wgrad_mfma.hpp"
+#include "reduce.hpp"
 
 namespace sfh {
 namespace {
@@ -275,24 +276,6 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   }
 }
 
-// gw[e] = sum over splits, in index order, of ws[split][e]; one rounding to T.
-template <typename T>
-__global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ ws, T* __restrict__ gw, int64_t nelem,
-                                                           int splits) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (e >= nelem) return;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  int sp = 0;
-  for (; sp + 3 < splits; sp += 4) {
-    s0 += ws[(int64_t)sp * nelem + e];
-    s1 += ws[(int64_t)(sp + 1) * nelem + e];
-    s2 += ws[(int64_t)(sp + 2) * nelem + e];
-    s3 += ws[(int64_t)(sp + 3) * nelem + e];
-  }
-  for (; sp < splits; ++sp) s0 += ws[(int64_t)sp * nelem + e];
-  gw[e] = elem<T>::from_float((s0 + s1) + (s2 + s3));
-}
-
 struct Plan {
   int tw;  // 32, 16 or 8
   int tiles_d, tiles_h, tiles_w, ntiles;
@@ -338,8 +321,7 @@ int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, vo
   else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st);
   if (rc != SFH_OK) return rc;
   const int64_t nelem = (int64_t)a.cout * 27 * a.cin;
-  hipLaunchKernelGGL(wgrad_reduce_kernel<T>, dim3((unsigned)cdiv(nelem, 256)), dim3(256), 0, st, ws, (T*)gw, nelem, p.splits);
-  return check_launch("wgrad_reduce_kernel");
+  return sum_slices(__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16, ws, gw, nelem, p.splits, st);
 }
 
 }  // namespace

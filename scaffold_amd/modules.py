@@ -77,7 +77,7 @@ class _Conv3dFn(torch.autograd.Function):
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1) if needs_x else None
         grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1) if needs_w else None
-        grad_b = grad_output.sum(dim=(0, 2, 3, 4)).to(bias_dtype) if (has_bias and needs_b) else None
+        grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
         return grad_x, grad_w, grad_b, None, None, None
 
 
@@ -98,7 +98,7 @@ class _ConvTranspose3dFn(torch.autograd.Function):
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1) if needs_x else None
         grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1) if needs_w else None
-        grad_b = grad_output.sum(dim=(0, 2, 3, 4)).to(bias_dtype) if (has_bias and needs_b) else None
+        grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
         return grad_x, grad_w, grad_b, None
 
 

@@ -394,3 +394,28 @@ def test_full_size_128cube_properties(device):
     xc = x[:, :, :10, :10, :40].cpu().contiguous(memory_format=cl)
     ref = orc.conv_reference(corner, {"input": xc, "weight": w.cpu(), "bias": None, "grad_output": None}, "fwd")
     assert torch.equal(y[:, :, :9, :9, :39].cpu().double(), ref[:, :, :9, :9, :39])
+
+
+# --- bias gradient --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 11, 7, 9, 13), (2, 32, 4, 5, 6), (1, 300, 2, 3, 3), (1, 1, 5, 5, 5), (1, 64, 33, 32, 31)])
+def test_bias_grad_matches_sum(device, dtype, shape):
+    """``grad_output.sum((0, 2, 3, 4))`` (``ScaFFold/unet/conv3d.py:1231``): bitwise on integer-valued gradients whose
+    sums are exactly representable, within the dtype's rounding of an fp64 sum on Gaussian ones."""
+    g = torch.Generator().manual_seed(7)
+    exact = torch.randint(-1, 2, shape, generator=g).to(dtype)
+    keep = torch.rand(shape, generator=g) < min(1.0, 100.0 / (shape[2] * shape[3] * shape[4]))
+    exact = (exact * keep).contiguous(memory_format=torch.channels_last_3d)
+    ref = exact.double().sum((0, 2, 3, 4))
+    got = sa.bias_grad(exact.to(device), torch.float32)
+    assert got.dtype is torch.float32 and torch.equal(got.cpu().double(), ref)
+    if orc.is_exactly_representable(ref, dtype):
+        assert torch.equal(sa.bias_grad(exact.to(device)).cpu().double(), ref)
+    gauss = torch.randn(shape, generator=g).to(dtype).contiguous(memory_format=torch.channels_last_3d)
+    ref = gauss.double().sum((0, 2, 3, 4))
+    got = sa.bias_grad(gauss.to(device), torch.float32).cpu().double()
+    assert (got - ref).abs().max() <= 1e-5 * gauss.double().abs().sum((0, 2, 3, 4)).max()
+    # an NCDHW-contiguous gradient is converted, not misread
+    assert torch.equal(sa.bias_grad(gauss.contiguous().to(device), torch.float32).cpu().double(), got)
+    # same call, same bits
+    assert torch.equal(sa.bias_grad(gauss.to(device), torch.float32).cpu().double(), got)
