@@ -18,9 +18,9 @@
 // different bank groups.
 //
 // A workgroup is four wavefronts; each owns 6-7 of the 27 taps (whole brick rows where possible)
-// and all 32x32 (co, ci) outputs of those taps: 112 accumulator registers. Tiles of the
-// workgroup's K range are processed one after another; two workgroups per CU overlap one's
-// staging with the other's MFMAs.
+// and all 32x32 (co, ci) outputs of those taps: 112 accumulator registers. One workgroup per CU
+// walks the tiles of its K range; the next tile's operands are fetched into registers before the
+// current tile's MFMAs start, so global-memory latency is hidden behind the compute.
 #include "wgrad_mfma.hpp"
 #include "reduce.hpp"
 
@@ -43,7 +43,7 @@ template <> struct Mma<fp16_t> {
   }
 };
 
-constexpr int kTargetWorkgroups = 2 * kComputeUnits;
+constexpr int kTargetWorkgroups = kComputeUnits;
 
 constexpr int odd16(int bytes) {  // smallest odd multiple of 16 that is >= bytes
   int u = (bytes + 15) / 16;
@@ -65,14 +65,7 @@ struct WTile {
   static constexpr int XITEMS = NBR * NQX * 4;
   static_assert(TD * TH * TW == 256, "one gy staging item per thread");
   static_assert(TH % 2 == 0, "an 8-voxel row pair must not straddle a depth slice");
-  static_assert(LDS <= 80 * 1024, "two workgroups per CU");
-};
-
-// Brick row (kd*3 + kh) sets of the four wavefronts; wave w < 3 also owns tap (2,2,kw=w).
-template <int WAVE> struct WaveTaps {
-  static constexpr int R0 = 2 * WAVE, R1 = 2 * WAVE + 1;
-  static constexpr bool EXTRA = WAVE < 3;
-  static constexpr int NACC = EXTRA ? 7 : 6;
+  static_assert(2 * LDS <= 160 * 1024, "two buffers in the 160 KB LDS of a CU");
 };
 
 // d0..d3 hold the same channel pair (even channel in the low half) of four consecutive voxels;
@@ -110,48 +103,85 @@ __device__ __forceinline__ constexpr int x_window_off(int ks, int kd, int kh) {
   }
 }
 
-template <typename T, typename C, int WAVE>
-__device__ __forceinline__ void wave_compute(const char* lds, int lane, f32x16_t (&acc)[7]) {
-  using W = WaveTaps<WAVE>;
+// Fragments of one k-step for a wavefront: the gy fragment, the nine-element windows of its two brick rows,
+// and the window of its extra tap (already positioned on that tap's first element pair).
+struct KFrags {
+  uint4 af;
+  uint4 lo0, lo1;
+  uint32_t nx0, nx1;
+  uint32_t xw[5];
+};
+
+template <typename C>
+__device__ __forceinline__ KFrags load_frags(const char* gsrc, const char* row0, const char* row1, const char* rowx, int ks) {
+  const int koff = x_window_off<C>(ks, 0, 0);
+  KFrags f;
+  f.af = *reinterpret_cast<const uint4*>(gsrc + ks * 32);
+  f.lo0 = *reinterpret_cast<const uint4*>(row0 + koff);
+  f.nx0 = *reinterpret_cast<const uint32_t*>(row0 + koff + 16);
+  f.lo1 = *reinterpret_cast<const uint4*>(row1 + koff);
+  f.nx1 = *reinterpret_cast<const uint32_t*>(row1 + koff + 16);
+#pragma unroll
+  for (int i = 0; i < 5; ++i) f.xw[i] = *reinterpret_cast<const uint32_t*>(rowx + koff + 4 * i);
+  return f;
+}
+
+// All four wavefronts run this one straight-line code path; what differs per wavefront (its two brick rows
+// and the kw of its extra tap) enters through addresses and one shift amount, so there are no branches and
+// the accumulators stay in place across the tile loop. Wavefront 3 has no 27th tap: it repeats tap (2,2,0)
+// into an accumulator that is never stored (it would otherwise idle at the barrier). The fragments of
+// k-step ks+1 are read from LDS before the MFMAs of k-step ks are issued: with one wavefront per SIMD
+// nothing else hides the LDS latency.
+template <typename T, typename C, typename Hook>
+__device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave, f32x16_t (&acc)[7], Hook&& hook) {
   const int i = lane & 31, kg = lane >> 5;
-  const int gbase = C::GOFF + i * C::GC + kg * 16;
+  const char* gsrc = lds + C::GOFF + i * C::GC + kg * 16;
   // k-half offset inside X: 8 voxels along W, or (TW == 8) the next brick row
   const int xbase = i * C::XC + (C::TW == 8 ? kg * C::XR * 2 : kg * 16);
+  const int r0 = 2 * wave, r1 = 2 * wave + 1;
+  const char* row0 = lds + xbase + ((r0 / 3) * C::BH + r0 % 3) * C::XR * 2;
+  const char* row1 = lds + xbase + ((r1 / 3) * C::BH + r1 % 3) * C::XR * 2;
+  // extra tap (2, 2, kw): kw = 2 starts one dword further, kw = 1 is a 16-bit funnel shift
+  const int kwx = wave < 3 ? wave : 0;
+  const char* rowx = lds + xbase + (2 * C::BH + 2) * C::XR * 2 + (kwx == 2 ? 4 : 0);
+  const uint32_t shx = kwx == 1 ? 16u : 0u;
+  KFrags cur = load_frags<C>(gsrc, row0, row1, rowx, 0);
 #pragma unroll
   for (int ks = 0; ks < C::NKS; ++ks) {
-    const uint4 af = *reinterpret_cast<const uint4*>(lds + gbase + ks * 32);
-#pragma unroll
-    for (int rr = 0; rr < 2; ++rr) {
-      const int row = rr == 0 ? W::R0 : W::R1;
-      const int off = xbase + x_window_off<C>(ks, row / 3, row % 3);
-      const uint4 lo = *reinterpret_cast<const uint4*>(lds + off);
-      const uint32_t nx = *reinterpret_cast<const uint32_t*>(lds + off + 16);
-      const uint4 f1 = shift_one(lo, nx);
-      const uint4 f2 = make_uint4(lo.y, lo.z, lo.w, nx);
-      acc[rr * 3 + 0] = Mma<T>::run(af, lo, acc[rr * 3 + 0]);
-      acc[rr * 3 + 1] = Mma<T>::run(af, f1, acc[rr * 3 + 1]);
-      acc[rr * 3 + 2] = Mma<T>::run(af, f2, acc[rr * 3 + 2]);
-    }
-    if (W::EXTRA) {
-      const int off = xbase + x_window_off<C>(ks, 2, 2);
-      const uint4 lo = *reinterpret_cast<const uint4*>(lds + off);
-      uint4 f = lo;
-      if (WAVE >= 1) {
-        const uint32_t nx = *reinterpret_cast<const uint32_t*>(lds + off + 16);
-        f = WAVE == 1 ? shift_one(lo, nx) : make_uint4(lo.y, lo.z, lo.w, nx);
-      }
-      acc[6] = Mma<T>::run(af, f, acc[6]);
-    }
+    // first MFMA of this k-step, then the LDS reads of the next one, then the other six MFMAs: the wait for
+    // this k-step's fragments comes before any younger read is in flight
+    __builtin_amdgcn_sched_barrier(0);
+    acc[0] = Mma<T>::run(cur.af, cur.lo0, acc[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    KFrags nxt = cur;
+    if (ks + 1 < C::NKS) nxt = load_frags<C>(gsrc, row0, row1, rowx, ks + 1);
+    __builtin_amdgcn_sched_barrier(0);
+    acc[1] = Mma<T>::run(cur.af, shift_one(cur.lo0, cur.nx0), acc[1]);
+    acc[2] = Mma<T>::run(cur.af, make_uint4(cur.lo0.y, cur.lo0.z, cur.lo0.w, cur.nx0), acc[2]);
+    __builtin_amdgcn_sched_barrier(0);
+    hook(ks);  // staging work of the following tiles, between MFMAs
+    __builtin_amdgcn_sched_barrier(0);
+    acc[3] = Mma<T>::run(cur.af, cur.lo1, acc[3]);
+    acc[4] = Mma<T>::run(cur.af, shift_one(cur.lo1, cur.nx1), acc[4]);
+    acc[5] = Mma<T>::run(cur.af, make_uint4(cur.lo1.y, cur.lo1.z, cur.lo1.w, cur.nx1), acc[5]);
+    uint4 fx;
+    fx.x = __builtin_amdgcn_alignbit(cur.xw[1], cur.xw[0], shx);
+    fx.y = __builtin_amdgcn_alignbit(cur.xw[2], cur.xw[1], shx);
+    fx.z = __builtin_amdgcn_alignbit(cur.xw[3], cur.xw[2], shx);
+    fx.w = __builtin_amdgcn_alignbit(cur.xw[4], cur.xw[3], shx);
+    acc[6] = Mma<T>::run(cur.af, fx, acc[6]);
+    __builtin_amdgcn_sched_barrier(0);
+    cur = nxt;
   }
 }
 
-template <typename C, int WAVE>
-__device__ __forceinline__ void wave_store(const f32x16_t (&acc)[7], float* __restrict__ dst, int cin, int lane) {
-  using W = WaveTaps<WAVE>;
+template <typename C>
+__device__ __forceinline__ void wave_store(const f32x16_t (&acc)[7], float* __restrict__ dst, int cin, int lane, int wave) {
   const int j = lane & 31, kg = lane >> 5;
 #pragma unroll
-  for (int t = 0; t < W::NACC; ++t) {
-    const int tap = t < 3 ? W::R0 * 3 + t : (t < 6 ? W::R1 * 3 + (t - 3) : 24 + WAVE);
+  for (int t = 0; t < 7; ++t) {
+    if (t == 6 && wave == 3) break;
+    const int tap = t < 3 ? 6 * wave + t : (t < 6 ? 6 * wave + t : 24 + wave);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int co = 8 * (r / 4) + 4 * kg + (r % 4);
@@ -160,13 +190,150 @@ __device__ __forceinline__ void wave_store(const f32x16_t (&acc)[7], float* __re
   }
 }
 
+// A staging item is (8-channel piece, 4-voxel slot). Within a wavefront the 16 lanes of a quarter share the
+// piece and take 16 consecutive slots: their transposed 8-byte LDS writes to one channel row are then
+// contiguous, and the two pieces of a half-wave land 128 bytes apart (mod 256), i.e. on disjoint banks.
+__device__ __forceinline__ int item_piece(int item) { return (item >> 4) & 3; }
+__device__ __forceinline__ int item_slot(int item) { return ((item >> 6) << 4) | (item & 15); }
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+constexpr uint32_t kOob = 0x80000000u;   // a byte offset no sample reaches: the buffer load returns zeros
+constexpr int kWaitLgkm0 = 0xC07F;       // s_waitcnt immediate (gfx9): lgkmcnt(0), vmcnt and expcnt untouched
+
+// Per-thread staging geometry, fixed for the whole kernel. Slot 0 is the thread's gy item, slots 1..XIT its x
+// items; an item is four consecutive W voxels x 8 channels.
+template <typename C>
+struct Slots {
+  // slots are handed out 16 per wavefront pass of 64 items
+  static constexpr int XIT = ((C::NBR * C::NQX + 15) / 16 * 64 + 255) / 256;
+  static constexpr int N = 1 + XIT;
+  int dst[N];  // LDS byte offset (inside one buffer) of the item's first channel row; -1: the thread has no such item
+  int off[N];  // byte offset of the item's first voxel from the tile origin
+  int crd[N];  // row coordinates relative to the tile origin and first W position: r0 | r1 << 8 | w0 << 16
+  uint4 raw[N][4];
+};
+
+struct TileOrigin { int n, od0, oh0, ow0; };
+
+__device__ __forceinline__ TileOrigin decode_tile(int tile, int tiles_d, int tiles_h, int tiles_w, int td, int th, int tw) {
+  TileOrigin o;
+  int t = tile;
+  o.ow0 = (t % tiles_w) * tw; t /= tiles_w;
+  o.oh0 = (t % tiles_h) * th; t /= tiles_h;
+  o.od0 = (t % tiles_d) * td;
+  o.n = t / tiles_d;
+  return o;
+}
+
+template <typename C>
+__device__ __forceinline__ void init_slots(const WgradArgs& a, int tid, Slots<C>& sl) {
+  {
+    const int piece = item_piece(tid), q = item_slot(tid);
+    const int quad = q % (C::TW / 4), grow = q / (C::TW / 4);
+    const int td = grow / C::TH, th = grow % C::TH, w0 = quad * 4;
+    sl.dst[0] = C::GOFF + (piece * 8) * C::GC + grow * C::TW * 2 + quad * 8;
+    sl.off[0] = ((td * a.oh + th) * a.ow + w0) * a.cout * 2 + piece * 16;
+    sl.crd[0] = td | (th << 8) | (w0 << 16);
+  }
+#pragma unroll
+  for (int it = 0; it < Slots<C>::XIT; ++it) {
+    const int item = it * 256 + tid;
+    const int piece = item_piece(item), q = item_slot(item);
+    const int quad = q % C::NQX, brow = q / C::NQX;
+    const int bd = brow / C::BH, bh = brow % C::BH, w0 = quad * 4;
+    sl.dst[1 + it] = q < C::NBR * C::NQX ? (piece * 8) * C::XC + brow * C::XR * 2 + quad * 8 : -1;
+    sl.off[1 + it] = ((bd * a.ih + bh) * a.iw + w0) * a.cin * 2 + piece * 16;
+    sl.crd[1 + it] = bd | (bh << 8) | (w0 << 16);
+  }
+}
+
+// Issues the four 16-byte loads of slot S for the tile at `o`. Voxels outside the tensor (padding, ragged tiles)
+// get an out-of-range offset, for which the buffer load returns zeros.
+template <typename T, typename C, int S>
+__device__ __forceinline__ void fetch_slot(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ gy, const TileOrigin& o,
+                                           int cib, int cob, Slots<C>& sl) {
+  const int r0 = sl.crd[S] & 0xff, r1 = (sl.crd[S] >> 8) & 0xff, w0 = sl.crd[S] >> 16;
+  if (S == 0) {
+    const int64_t sample = (int64_t)a.od * a.oh * a.ow * a.cout;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gy + o.n * sample), 0, (int)(sample * 2), 0x00020000);
+    const int org = ((o.od0 * a.oh + o.oh0) * a.ow + o.ow0) * a.cout * 2 + cob * 64;
+    // plain integer masks (no short-circuit), so that the selection stays a select and never becomes a branch
+    const int rowok = (int)(o.od0 + r0 < a.od) & (int)(o.oh0 + r1 < a.oh);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ok = rowok & (int)(o.ow0 + w0 + k < a.ow);
+      const uint32_t voff = ok != 0 ? (uint32_t)(org + sl.off[0] + k * a.cout * 2) : kOob;
+      sl.raw[0][k] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, 0));
+    }
+  } else {
+    const int64_t sample = (int64_t)a.id * a.ih * a.iw * a.cin;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x + o.n * sample), 0, (int)(sample * 2), 0x00020000);
+    const int id0 = o.od0 - a.pd, ih0 = o.oh0 - a.ph, iw0 = o.ow0 - a.pw;
+    const int org = ((id0 * a.ih + ih0) * a.iw + iw0) * a.cin * 2 + cib * 64;
+    const int rowok = (int)(sl.dst[S] >= 0) & (int)((unsigned)(id0 + r0) < (unsigned)a.id) & (int)((unsigned)(ih0 + r1) < (unsigned)a.ih);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ok = rowok & (int)(w0 + k < C::TW + 2) & (int)((unsigned)(iw0 + w0 + k) < (unsigned)a.iw);
+      const uint32_t voff = ok != 0 ? (uint32_t)(org + sl.off[S] + k * a.cin * 2) : kOob;
+      sl.raw[S][k] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, 0, 0));
+    }
+  }
+}
+
+// Transposes four voxels x 8 channels (v[k] = voxel k) into 8 channel rows of 4 voxels at dst, dst + stride, ...
+__device__ __forceinline__ void store_transposed(char* dst, int stride, const uint4 (&v)[4]) {
+  const uint32_t d0[4] = {v[0].x, v[0].y, v[0].z, v[0].w}, d1[4] = {v[1].x, v[1].y, v[1].z, v[1].w},
+                 d2[4] = {v[2].x, v[2].y, v[2].z, v[2].w}, d3[4] = {v[3].x, v[3].y, v[3].z, v[3].w};
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    uint2 e0, e1;
+    transpose4(d0[d], d1[d], d2[d], d3[d], e0, e1);
+    *reinterpret_cast<uint2*>(dst + (2 * d) * stride) = e0;
+    *reinterpret_cast<uint2*>(dst + (2 * d + 1) * stride) = e1;
+  }
+}
+
+template <typename C, int S>
+__device__ __forceinline__ void stage_slot(char* buf, const Slots<C>& sl) {
+  if (S == 0 || sl.dst[S] >= 0) store_transposed(buf + sl.dst[S], S == 0 ? C::GC : C::XC, sl.raw[S]);
+}
+
+template <typename T, typename C, int S>
+struct SlotLoop {
+  static __device__ __forceinline__ void fetch_all(const WgradArgs& a, const T* x, const T* gy, const TileOrigin& o, int cib, int cob,
+                                                   Slots<C>& sl) {
+    fetch_slot<T, C, S>(a, x, gy, o, cib, cob, sl);
+    if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::fetch_all(a, x, gy, o, cib, cob, sl);
+  }
+  static __device__ __forceinline__ void stage_all(char* buf, const Slots<C>& sl) {
+    stage_slot<C, S>(buf, sl);
+    if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::stage_all(buf, sl);
+  }
+  // k-step ks of the MFMA loop carries slot (ks - 1) / 3: its raw data (fetched one tile ago) goes to the idle LDS
+  // buffer and its registers are refilled with the tile after next.
+  static __device__ __forceinline__ void at_kstep(int ks, char* idle, const WgradArgs& a, const T* x, const T* gy,
+                                                  const TileOrigin& o2, int cib, int cob, Slots<C>& sl) {
+    if (ks == 1 + 3 * S) {
+      stage_slot<C, S>(idle, sl);
+      fetch_slot<T, C, S>(a, x, gy, o2, cib, cob, sl);
+    }
+    if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::at_kstep(ks, idle, a, x, gy, o2, cib, cob, sl);
+  }
+};
+
+// One workgroup per CU (512 registers per lane), two LDS buffers. While the MFMAs of tile t run out of one
+// buffer, the same instruction stream transposes tile t+1 (fetched into registers during tile t-1) into the other
+// buffer and refills the registers with tile t+2, a slot at a time between MFMAs: global-memory latency has a
+// whole tile period to hide in, and the staging work rides in the issue slots the MFMA pipe leaves free.
 template <typename T, typename C>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, 1)
 wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws, int tiles_d,
                   int tiles_h, int tiles_w, int ntiles, int tiles_per_split, int nblk_ci, int nblk, uint32_t total) {
-  __shared__ __attribute__((aligned(16))) char lds[C::LDS];
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char buf0[C::LDS];
+  __shared__ __attribute__((aligned(16))) char buf1[C::LDS];
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
   uint32_t wg = xcd_remap(blockIdx.x, total);
   const int blk = wg % nblk;
@@ -183,97 +350,35 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   int t_end = t_begin + tiles_per_split;
   if (t_end > ntiles) t_end = ntiles;
 
-  constexpr int XIT = (C::XITEMS + 255) / 256;
-  for (int tile = t_begin; tile < t_end; ++tile) {
-    int t = tile;
-    const int tw_i = t % tiles_w; t /= tiles_w;
-    const int th_i = t % tiles_h; t /= tiles_h;
-    const int td_i = t % tiles_d;
-    const int n = t / tiles_d;
-    const int od0 = td_i * C::TD, oh0 = th_i * C::TH, ow0 = tw_i * C::TW;
-
-    __syncthreads();  // previous tile fully consumed
-    // ---- stage gy tile, transposed: one item (tile row, 4-voxel group, 8-channel piece) per thread
-    {
-      const int piece = tid & 3;
-      const int quad = (tid >> 2) % (C::TW / 4);
-      const int grow = tid / (C::TW);  // (tid >> 2) / (TW / 4)
-      const int td = grow / C::TH, th = grow % C::TH;
-      const int od = od0 + td, oh = oh0 + th;
-      const bool rowok = od < a.od && oh < a.oh;
-      const T* gp = gy + ((((int64_t)n * a.od + od) * a.oh + oh) * a.ow) * a.cout + cob * 32 + piece * 8;
-      uint4 v[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        const int ow = ow0 + quad * 4 + k;
-        v[k] = make_uint4(0, 0, 0, 0);
-        if (rowok && ow < a.ow) v[k] = *reinterpret_cast<const uint4*>(gp + (int64_t)ow * a.cout);
-      }
-      char* dst = lds + C::GOFF + (piece * 8) * C::GC + grow * C::TW * 2 + quad * 8;
-      const uint32_t d0[4] = {v[0].x, v[0].y, v[0].z, v[0].w}, d1[4] = {v[1].x, v[1].y, v[1].z, v[1].w},
-                     d2[4] = {v[2].x, v[2].y, v[2].z, v[2].w}, d3[4] = {v[3].x, v[3].y, v[3].z, v[3].w};
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        uint2 e0, e1;
-        transpose4(d0[d], d1[d], d2[d], d3[d], e0, e1);
-        *reinterpret_cast<uint2*>(dst + (2 * d) * C::GC) = e0;
-        *reinterpret_cast<uint2*>(dst + (2 * d + 1) * C::GC) = e1;
-      }
-    }
-    // ---- stage x brick (with halo), transposed
-    {
-      const int id0 = od0 - a.pd, ih0 = oh0 - a.ph, iw0 = ow0 - a.pw;
-      const T* xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cin + cib * 32;
-#pragma unroll
-      for (int it = 0; it < XIT; ++it) {
-        const int item = it * 256 + tid;
-        if (item < C::XITEMS) {
-          const int piece = item & 3;
-          const int quad = (item >> 2) % C::NQX;
-          const int brow = (item >> 2) / C::NQX;
-          const int bd = brow / C::BH, bh = brow % C::BH;
-          const int id = id0 + bd, ih = ih0 + bh;
-          const bool rowok = (unsigned)id < (unsigned)a.id && (unsigned)ih < (unsigned)a.ih;
-          const T* xp = xn + (((int64_t)id * a.ih + ih) * a.iw) * a.cin + piece * 8;
-          uint4 v[4];
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const int bw = quad * 4 + k;
-            const int iw = iw0 + bw;
-            v[k] = make_uint4(0, 0, 0, 0);
-            if (rowok && bw < C::TW + 2 && (unsigned)iw < (unsigned)a.iw)
-              v[k] = *reinterpret_cast<const uint4*>(xp + (int64_t)iw * a.cin);
-          }
-          char* dst = lds + (piece * 8) * C::XC + brow * C::XR * 2 + quad * 8;
-          const uint32_t d0[4] = {v[0].x, v[0].y, v[0].z, v[0].w}, d1[4] = {v[1].x, v[1].y, v[1].z, v[1].w},
-                         d2[4] = {v[2].x, v[2].y, v[2].z, v[2].w}, d3[4] = {v[3].x, v[3].y, v[3].z, v[3].w};
-#pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            uint2 e0, e1;
-            transpose4(d0[d], d1[d], d2[d], d3[d], e0, e1);
-            *reinterpret_cast<uint2*>(dst + (2 * d) * C::XC) = e0;
-            *reinterpret_cast<uint2*>(dst + (2 * d + 1) * C::XC) = e1;
-          }
-        }
-      }
-    }
-    __syncthreads();
-
-    switch (wave) {
-      case 0: wave_compute<T, C, 0>(lds, lane, acc); break;
-      case 1: wave_compute<T, C, 1>(lds, lane, acc); break;
-      case 2: wave_compute<T, C, 2>(lds, lane, acc); break;
-      default: wave_compute<T, C, 3>(lds, lane, acc); break;
+  if (t_begin < t_end) {
+    Slots<C> sl;
+    init_slots<C>(a, tid, sl);
+    auto origin = [&](int tile) {
+      return decode_tile(tile < t_end ? tile : t_end - 1, tiles_d, tiles_h, tiles_w, C::TD, C::TH, C::TW);
+    };
+    SlotLoop<T, C, 0>::fetch_all(a, x, gy, origin(t_begin), cib, cob, sl);
+    SlotLoop<T, C, 0>::stage_all(buf0, sl);
+    SlotLoop<T, C, 0>::fetch_all(a, x, gy, origin(t_begin + 1), cib, cob, sl);
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __builtin_amdgcn_s_barrier();
+    for (int tile = t_begin; tile < t_end; ++tile) {
+      const bool odd = (tile - t_begin) & 1;
+      char* cur = odd ? buf1 : buf0;
+      char* idle = odd ? buf0 : buf1;
+      // On the last tiles the staged / fetched data is never used; doing the work anyway keeps the loop free of
+      // branches (the fetch is clamped to the split's last tile).
+      const TileOrigin o2 = origin(tile + 2);
+      wave_compute<T, C>(cur, lane, wave, acc, [&](int ks) {
+        SlotLoop<T, C, 0>::at_kstep(ks, idle, a, x, gy, o2, cib, cob, sl);
+      });
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // this wave's LDS writes of the next tile have landed
+      __builtin_amdgcn_s_barrier();            // ... and every wave is done reading the current one
     }
   }
 
   float* dst = ws + ((int64_t)split * a.cout + cob * 32) * 27 * a.cin + cib * 32;
-  switch (wave) {
-    case 0: wave_store<C, 0>(acc, dst, a.cin, lane); break;
-    case 1: wave_store<C, 1>(acc, dst, a.cin, lane); break;
-    case 2: wave_store<C, 2>(acc, dst, a.cin, lane); break;
-    default: wave_store<C, 3>(acc, dst, a.cin, lane); break;
-  }
+  wave_store<C>(acc, dst, a.cin, lane, wave);
+#endif
 }
 
 struct Plan {
@@ -331,6 +436,9 @@ bool mfma_wgrad_supported(const WgradArgs& a, int dtype) {
   if (a.cin % 32 != 0 || a.cout % 32 != 0) return false;
   if (a.pd < 0 || a.ph < 0 || a.pw < 0 || a.pd > 2 || a.ph > 2 || a.pw > 2) return false;
   if (a.n < 1 || a.od < 1 || a.oh < 1 || a.ow < 1) return false;
+  // staging addresses one sample with 32-bit byte offsets
+  const int64_t limit = 0x7ff00000LL;
+  if ((int64_t)a.id * a.ih * a.iw * a.cin * 2 > limit || (int64_t)a.od * a.oh * a.ow * a.cout * 2 > limit) return false;
   const Plan p = make_plan(a);
   if ((int64_t)a.n * p.tiles_d * p.tiles_h * p.tiles_w > 0x7fffffffLL) return false;
   return true;
