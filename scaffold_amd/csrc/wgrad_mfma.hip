@@ -109,7 +109,8 @@ struct KFrags {
   uint4 af;
   uint4 lo0, lo1;
   uint32_t nx0, nx1;
-  uint32_t xw[5];
+  uint4 lox;
+  uint32_t nxx;
 };
 
 template <typename C>
@@ -121,8 +122,8 @@ __device__ __forceinline__ KFrags load_frags(const char* gsrc, const char* row0,
   f.nx0 = *reinterpret_cast<const uint32_t*>(row0 + koff + 16);
   f.lo1 = *reinterpret_cast<const uint4*>(row1 + koff);
   f.nx1 = *reinterpret_cast<const uint32_t*>(row1 + koff + 16);
-#pragma unroll
-  for (int i = 0; i < 5; ++i) f.xw[i] = *reinterpret_cast<const uint32_t*>(rowx + koff + 4 * i);
+  f.lox = *reinterpret_cast<const uint4*>(rowx + koff);
+  f.nxx = *reinterpret_cast<const uint32_t*>(rowx + koff + 16);
   return f;
 }
 
@@ -132,8 +133,8 @@ __device__ __forceinline__ KFrags load_frags(const char* gsrc, const char* row0,
 // into an accumulator that is never stored (it would otherwise idle at the barrier). The fragments of
 // k-step ks+1 are read from LDS before the MFMAs of k-step ks are issued: with one wavefront per SIMD
 // nothing else hides the LDS latency.
-template <typename T, typename C, typename Hook>
-__device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave, f32x16_t (&acc)[7], Hook&& hook) {
+template <typename T, typename C>
+__device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave, f32x16_t (&acc)[7]) {
   const int i = lane & 31, kg = lane >> 5;
   const char* gsrc = lds + C::GOFF + i * C::GC + kg * 16;
   // k-half offset inside X: 8 voxels along W, or (TW == 8) the next brick row
@@ -141,10 +142,11 @@ __device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave
   const int r0 = 2 * wave, r1 = 2 * wave + 1;
   const char* row0 = lds + xbase + ((r0 / 3) * C::BH + r0 % 3) * C::XR * 2;
   const char* row1 = lds + xbase + ((r1 / 3) * C::BH + r1 % 3) * C::XR * 2;
-  // extra tap (2, 2, kw): kw = 2 starts one dword further, kw = 1 is a 16-bit funnel shift
+  // extra tap (2, 2, kw): kw = 1 is a 16-bit funnel shift, kw = 2 takes the next dword (wave-uniform selects)
   const int kwx = wave < 3 ? wave : 0;
-  const char* rowx = lds + xbase + (2 * C::BH + 2) * C::XR * 2 + (kwx == 2 ? 4 : 0);
+  const char* rowx = lds + xbase + (2 * C::BH + 2) * C::XR * 2;
   const uint32_t shx = kwx == 1 ? 16u : 0u;
+  const bool next_dword = kwx == 2;
   KFrags cur = load_frags<C>(gsrc, row0, row1, rowx, 0);
 #pragma unroll
   for (int ks = 0; ks < C::NKS; ++ks) {
@@ -158,17 +160,14 @@ __device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave
     __builtin_amdgcn_sched_barrier(0);
     acc[1] = Mma<T>::run(cur.af, shift_one(cur.lo0, cur.nx0), acc[1]);
     acc[2] = Mma<T>::run(cur.af, make_uint4(cur.lo0.y, cur.lo0.z, cur.lo0.w, cur.nx0), acc[2]);
-    __builtin_amdgcn_sched_barrier(0);
-    hook(ks);  // staging work of the following tiles, between MFMAs
-    __builtin_amdgcn_sched_barrier(0);
     acc[3] = Mma<T>::run(cur.af, cur.lo1, acc[3]);
     acc[4] = Mma<T>::run(cur.af, shift_one(cur.lo1, cur.nx1), acc[4]);
     acc[5] = Mma<T>::run(cur.af, make_uint4(cur.lo1.y, cur.lo1.z, cur.lo1.w, cur.nx1), acc[5]);
     uint4 fx;
-    fx.x = __builtin_amdgcn_alignbit(cur.xw[1], cur.xw[0], shx);
-    fx.y = __builtin_amdgcn_alignbit(cur.xw[2], cur.xw[1], shx);
-    fx.z = __builtin_amdgcn_alignbit(cur.xw[3], cur.xw[2], shx);
-    fx.w = __builtin_amdgcn_alignbit(cur.xw[4], cur.xw[3], shx);
+    fx.x = next_dword ? cur.lox.y : __builtin_amdgcn_alignbit(cur.lox.y, cur.lox.x, shx);
+    fx.y = next_dword ? cur.lox.z : __builtin_amdgcn_alignbit(cur.lox.z, cur.lox.y, shx);
+    fx.z = next_dword ? cur.lox.w : __builtin_amdgcn_alignbit(cur.lox.w, cur.lox.z, shx);
+    fx.w = next_dword ? cur.nxx : __builtin_amdgcn_alignbit(cur.nxx, cur.lox.w, shx);
     acc[6] = Mma<T>::run(cur.af, fx, acc[6]);
     __builtin_amdgcn_sched_barrier(0);
     cur = nxt;
@@ -309,24 +308,27 @@ struct SlotLoop {
     stage_slot<C, S>(buf, sl);
     if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::stage_all(buf, sl);
   }
-  // k-step ks of the MFMA loop carries slot (ks - 1) / 3: its raw data (fetched one tile ago) goes to the idle LDS
-  // buffer and its registers are refilled with the tile after next.
-  static __device__ __forceinline__ void at_kstep(int ks, char* idle, const WgradArgs& a, const T* x, const T* gy,
-                                                  const TileOrigin& o2, int cib, int cob, Slots<C>& sl) {
-    if (ks == 1 + 3 * S) {
-      stage_slot<C, S>(idle, sl);
-      fetch_slot<T, C, S>(a, x, gy, o2, cib, cob, sl);
-    }
-    if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::at_kstep(ks, idle, a, x, gy, o2, cib, cob, sl);
+  // Slot by slot: the raw data fetched one tile ago goes to the idle LDS buffer and the registers are refilled
+  // with the tile after next.
+  static __device__ __forceinline__ void stage_and_refill(char* idle, const WgradArgs& a, const T* x, const T* gy,
+                                                          const TileOrigin& o2, int cib, int cob, Slots<C>& sl) {
+    stage_slot<C, S>(idle, sl);
+    fetch_slot<T, C, S>(a, x, gy, o2, cib, cob, sl);
+    if constexpr (S + 1 < Slots<C>::N) SlotLoop<T, C, S + 1>::stage_and_refill(idle, a, x, gy, o2, cib, cob, sl);
   }
 };
 
-// One workgroup per CU (512 registers per lane), two LDS buffers. While the MFMAs of tile t run out of one
-// buffer, the same instruction stream transposes tile t+1 (fetched into registers during tile t-1) into the other
-// buffer and refills the registers with tile t+2, a slot at a time between MFMAs: global-memory latency has a
-// whole tile period to hide in, and the staging work rides in the issue slots the MFMA pipe leaves free.
+// One 8-wavefront workgroup per CU, two LDS buffers, two kinds of wavefront (one of each per SIMD):
+//   * wavefronts 0..3 only compute: LDS fragment reads, the kw shifts and 112 MFMAs per tile;
+//   * wavefronts 4..7 only stage: while tile t is being computed out of one buffer they transpose tile t+1
+//     (which they fetched into registers during tile t-1) into the other buffer and refill their registers
+//     with tile t+2, so global-memory latency has a whole tile period to hide in.
+// A SIMD issues one vector-ALU instruction per four cycles whatever the number of wavefronts; keeping the
+// staging arithmetic out of the MFMA wavefront's instruction stream (and the two streams on different
+// wavefronts, which issue to different ports concurrently) is what lets the MFMA pipe stay busy.
+// One barrier per tile joins all eight wavefronts.
 template <typename T, typename C>
-__global__ void __launch_bounds__(256, 1)
+__global__ void __launch_bounds__(512)
 wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws, int tiles_d,
                   int tiles_h, int tiles_w, int ntiles, int tiles_per_split, int nblk_ci, int nblk, uint32_t total) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -340,19 +342,15 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   const int split = wg / nblk;
   const int cib = blk % nblk_ci, cob = blk / nblk_ci;
 
-  f32x16_t acc[7];
-#pragma unroll
-  for (int t = 0; t < 7; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
-
   const int t_begin = split * tiles_per_split;
   int t_end = t_begin + tiles_per_split;
   if (t_end > ntiles) t_end = ntiles;
 
-  if (t_begin < t_end) {
+  if (wave >= 4) {
+    // ---- staging wavefronts ----
+    if (t_begin >= t_end) return;
     Slots<C> sl;
-    init_slots<C>(a, tid, sl);
+    init_slots<C>(a, tid - 256, sl);
     auto origin = [&](int tile) {
       return decode_tile(tile < t_end ? tile : t_end - 1, tiles_d, tiles_h, tiles_w, C::TD, C::TH, C::TW);
     };
@@ -362,20 +360,32 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
     __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
     __builtin_amdgcn_s_barrier();
     for (int tile = t_begin; tile < t_end; ++tile) {
-      const bool odd = (tile - t_begin) & 1;
-      char* cur = odd ? buf1 : buf0;
-      char* idle = odd ? buf0 : buf1;
+      char* idle = ((tile - t_begin) & 1) ? buf0 : buf1;
       // On the last tiles the staged / fetched data is never used; doing the work anyway keeps the loop free of
       // branches (the fetch is clamped to the split's last tile).
       const TileOrigin o2 = origin(tile + 2);
-      wave_compute<T, C>(cur, lane, wave, acc, [&](int ks) {
-        SlotLoop<T, C, 0>::at_kstep(ks, idle, a, x, gy, o2, cib, cob, sl);
-      });
-      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // this wave's LDS writes of the next tile have landed
-      __builtin_amdgcn_s_barrier();            // ... and every wave is done reading the current one
+      SlotLoop<T, C, 0>::stage_and_refill(idle, a, x, gy, o2, cib, cob, sl);
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // the LDS writes of the next tile have landed
+      __builtin_amdgcn_s_barrier();            // ... and the compute wavefronts are done reading the current one
     }
+    return;
   }
 
+  // ---- compute wavefronts ----
+  f32x16_t acc[7];
+#pragma unroll
+  for (int t = 0; t < 7; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  if (t_begin < t_end) {
+    __builtin_amdgcn_s_barrier();  // the first tile is staged
+    for (int tile = t_begin; tile < t_end; ++tile) {
+      const char* cur = ((tile - t_begin) & 1) ? buf1 : buf0;
+      asm volatile("" ::: "memory");  // LDS changes behind this wavefront's back: reload every tile
+      wave_compute<T, C>(cur, lane, wave, acc);
+      __builtin_amdgcn_s_barrier();
+    }
+  }
   float* dst = ws + ((int64_t)split * a.cout + cob * 32) * 27 * a.cin + cib * 32;
   wave_store<C>(acc, dst, a.cin, lane, wave);
 #endif
@@ -411,7 +421,7 @@ Plan make_plan(const WgradArgs& a) {
 template <typename T, typename C>
 int launch_tile(const WgradArgs& a, const Plan& p, const void* x, const void* gy, float* ws, hipStream_t st) {
   const int64_t total = (int64_t)p.splits * p.nblk;
-  hipLaunchKernelGGL((wgrad_mfma_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)gy, ws,
+  hipLaunchKernelGGL((wgrad_mfma_kernel<T, C>), dim3((unsigned)total), dim3(512), 0, st, a, (const T*)x, (const T*)gy, ws,
                      p.tiles_d, p.tiles_h, p.tiles_w, p.ntiles, p.tiles_per_split, p.nblk_ci, p.nblk, (uint32_t)total);
   return check_launch("wgrad_mfma_kernel");
 }
