@@ -38,7 +38,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the forward kernel on the bench workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # counter runs of this script scaled by the same counters on the 256 MiB copy kernel (profiles/ holds the runs).
-CONV_FWD_HBM_TRAFFIC_BYTES = int((108831.8 * 2.000 + 131073.9) * 1024)
+CONV_FWD_HBM_TRAFFIC_BYTES = int((109566.3 * 2.000 + 131101.1) * 1024)
 CL = torch.channels_last_3d
 
 
