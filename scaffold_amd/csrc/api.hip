@@ -266,7 +266,7 @@ extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int d
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (fwd_uses_patch(*p, dtype, out)) return mfma_conv_packed_weight_bytes(patch_pack_args(p->cout, p->cin));
   if (!fwd_uses_mfma(*p, dtype, out)) return 0;
-  return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out));
+  return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out)) + mfma_conv_partial_bytes(fwd_mfma_args(*p, out));
 }
 
 extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
@@ -278,12 +278,14 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_mfma(*p, dtype, out)) {
     const MfmaConvArgs a = fwd_mfma_args(*p, out);
-    const size_t need = mfma_conv_packed_weight_bytes(a);
+    const size_t packed_bytes = mfma_conv_packed_weight_bytes(a), partial_bytes = mfma_conv_partial_bytes(a);
+    const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
-    return mfma_conv_persist(a, dtype, x, workspace, bias, y, st);
+    void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
+    return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_patch(*p, dtype, out)) {
     const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);
@@ -322,7 +324,7 @@ extern "C" size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (check_dgrad(*p) != SFH_OK || !dgrad_uses_mfma(*p, dtype, out)) return 0;
-  return mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out));
+  return mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out)) + mfma_conv_partial_bytes(dgrad_mfma_args(*p, out));
 }
 
 extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
@@ -334,13 +336,15 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && dgrad_uses_mfma(*p, dtype, out)) {
     const MfmaConvArgs a = dgrad_mfma_args(*p, out);
-    const size_t need = mfma_conv_packed_weight_bytes(a);
+    const size_t packed_bytes = mfma_conv_packed_weight_bytes(a), partial_bytes = mfma_conv_partial_bytes(a);
+    const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     // produced channel = Cin (stride w_stride[1]), reduction channel = Cout (w_stride[0]), taps flipped
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, workspace, st))
       return rc;
-    return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, st);
+    void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
+    return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
     ThinArgs t;

@@ -22,6 +22,7 @@
 // The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
 // padding k-1-p (triton_conv3d/bwd_data.py:344-363).
 #include "conv_mfma.hpp"
+#include "reduce.hpp"
 
 namespace sfh {
 namespace {
@@ -79,13 +80,15 @@ __device__ __forceinline__ constexpr int lds_off(int it) {
 template <typename T, typename C>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
-                 T* __restrict__ y, int tiles_d, int tiles_h, int tiles_w, int nblocks, uint32_t total) {
+                 T* __restrict__ y, float* __restrict__ partial, int tiles_d, int tiles_h, int tiles_w, int nblocks, int ksplit,
+                 uint32_t total) {
   __shared__ __attribute__((aligned(16))) char lds[C::LDS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int j = lane & 31, kg = lane >> 5;
 
   uint32_t t = xcd_remap(blockIdx.x, total);
+  const int ksp = t % ksplit; t /= ksplit;  // slice of the reduction channels (1 slice unless the grid would underfill the chip)
   const int nb = t % nblocks; t /= nblocks;
   const int tw_i = t % tiles_w; t /= tiles_w;
   const int th_i = t % tiles_h; t /= tiles_h;
@@ -118,7 +121,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   constexpr int BATCH = C::NSUB == 1 ? ITERS : 8;
   constexpr int FRAG = 512;  // elements per packed (tap, k-step) fragment: 64 lanes x 8
 
-  for (int cc = 0; cc < ncc; ++cc) {
+  const int cc_begin = (int)((int64_t)ksp * ncc / ksplit), cc_end = (int)((int64_t)(ksp + 1) * ncc / ksplit);
+  for (int cc = cc_begin; cc < cc_end; ++cc) {
     __syncthreads();  // every wave is done reading the previous chunk
     {
       const T* xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cred + cc * kChunk;
@@ -194,7 +198,19 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
     const int od = od0 + td, oh = oh0 + th, ow = ow0 + tw;
     if (od >= a.od || oh >= a.oh || ow >= a.ow) continue;
-    T* yp = y + ((((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cout + nb * C::NSUB * 32;
+    const int64_t vox = (((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow;
+    if (ksplit > 1) {
+      // fp32 slice of this reduction range; the slices are summed (and the bias added) by sum_slices_bias
+      float* pp = partial + ((int64_t)ksp * a.n * a.od * a.oh * a.ow + vox) * a.cout + nb * C::NSUB * 32;
+#pragma unroll
+      for (int ns = 0; ns < C::NSUB; ++ns)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          *reinterpret_cast<float4*>(pp + ns * 32 + 8 * g + 4 * kg) =
+              make_float4(acc[ms][ns][4 * g], acc[ms][ns][4 * g + 1], acc[ms][ns][4 * g + 2], acc[ms][ns][4 * g + 3]);
+      continue;
+    }
+    T* yp = y + vox * a.cout + nb * C::NSUB * 32;
 #pragma unroll
     for (int ns = 0; ns < C::NSUB; ++ns) {
 #pragma unroll
@@ -237,30 +253,60 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
   packed[idx] = w[co * s_out + ci * s_red + tkd * s_kd + tkh * s_kh + tkw * s_kw];
 }
 
+struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
+
+// Launch geometry, a pure function of the problem: brick shape by row length; two output blocks per workgroup
+// when that still fills the chip, else one; and when even that leaves CUs idle (the deep, small-volume levels)
+// the reduction channels are cut into slices that are summed afterwards.
+GatherPlan gather_plan(const MfmaConvArgs& a) {
+  GatherPlan p{};
+  int td, th, tw;
+  if (a.ow > 16) { p.shape = 0; td = 4; th = 4; tw = 32; }
+  else if (a.ow > 8) { p.shape = 1; td = 4; th = 8; tw = 16; }
+  else { p.shape = 2; td = 8; th = 8; tw = 8; }
+  p.tiles = (int64_t)a.n * cdiv(a.od, td) * cdiv(a.oh, th) * cdiv(a.ow, tw);
+  p.nsub = (a.cout % 64 == 0 && p.tiles * (a.cout / 64) >= kComputeUnits) ? 2 : 1;
+  p.ksplit = 1;
+  const int64_t wgs = p.tiles * (a.cout / (32 * p.nsub));
+  const int ncc = a.cred / kChunk;
+  if (wgs < kComputeUnits && ncc > 1) {
+    int64_t k = cdiv(2 * kComputeUnits, wgs);
+    p.ksplit = (int)(k < ncc ? k : ncc);
+  }
+  return p;
+}
+
 template <typename T, typename C>
-int launch_cfg(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
+               float* partial, hipStream_t st) {
   const int tiles_d = (int)cdiv(a.od, C::TD), tiles_h = (int)cdiv(a.oh, C::TH), tiles_w = (int)cdiv(a.ow, C::TW);
   const int nblocks = a.cout / (32 * C::NSUB);
-  const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks;
+  const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks * p.ksplit;
   if (total == 0) return SFH_OK;
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: %lld workgroups exceed the grid limit", (long long)total);
   hipLaunchKernelGGL((conv_mfma_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
-                     (const T*)bias, (T*)y, tiles_d, tiles_h, tiles_w, nblocks, (uint32_t)total);
+                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total);
   return check_launch("conv_mfma_kernel");
 }
 
 template <typename T, int NSUB>
-int launch_k333(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+int launch_k333(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
+                float* partial, hipStream_t st) {
   // Brick shape follows the row length: 32-voxel sub-tiles are one, two or four W rows.
-  if (a.ow > 16) return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
-  if (a.ow > 8) return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
-  return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, x, packed, bias, y, st);
+  if (p.shape == 0) return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+  if (p.shape == 1) return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+  return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
 }
 
 template <typename T>
-int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
-  if (a.cout % 64 == 0) return launch_k333<T, 2>(a, x, packed, bias, y, st);
-  return launch_k333<T, 1>(a, x, packed, bias, y, st);
+int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, void* partial,
+                 hipStream_t st) {
+  const GatherPlan p = gather_plan(a);
+  if (p.ksplit > 1 && partial == nullptr) return fail(SFH_ERR_WORKSPACE, "conv mfma: the reduction split needs its workspace");
+  const int rc = p.nsub == 2 ? launch_k333<T, 2>(a, p, x, packed, bias, y, (float*)partial, st)
+                             : launch_k333<T, 1>(a, p, x, packed, bias, y, (float*)partial, st);
+  if (rc != SFH_OK || p.ksplit == 1) return rc;
+  return sum_slices_bias(dtype, (const float*)partial, bias, y, (int64_t)a.n * a.od * a.oh * a.ow * a.cout, a.cout, p.ksplit, st);
 }
 
 }  // namespace
@@ -291,10 +337,16 @@ int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_
   return check_launch("pack_weight_kernel");
 }
 
+size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
+  const GatherPlan p = gather_plan(a);
+  if (a.cred == kChunk || p.ksplit == 1) return 0;
+  return align_up((size_t)p.ksplit * a.n * a.od * a.oh * a.ow * a.cout * sizeof(float), 256);
+}
+
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                     hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st);
-  return launch_typed<fp16_t>(a, x, packed, bias, y, st);
+                     void* partial, hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st);
+  return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st);
 }
 
 }  // namespace sfh

@@ -57,6 +57,27 @@ int launch_sum(const float* part, void* out, int64_t nelem, int splits, hipStrea
   return check_launch("sum_slices_flat");
 }
 
+// Four consecutive elements per thread (16-byte loads of every slice), bias added before the one rounding.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __restrict__ part, const T* __restrict__ bias,
+                                                                 T* __restrict__ out, int64_t nelem, int channels, int splits) {
+  const int64_t e = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4;
+  if (e >= nelem) return;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int sp = 0; sp < splits; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (bias != nullptr) {
+    const int c = (int)(e % channels);
+    s.x += to_float(bias[c]); s.y += to_float(bias[c + 1]); s.z += to_float(bias[c + 2]); s.w += to_float(bias[c + 3]);
+  }
+  out[e] = elem<T>::from_float(s.x);
+  out[e + 1] = elem<T>::from_float(s.y);
+  out[e + 2] = elem<T>::from_float(s.z);
+  out[e + 3] = elem<T>::from_float(s.w);
+}
+
 // Per-channel partial sums: thread = (row slot, channel); a workgroup walks its row range with rpp rows per
 // pass (consecutive threads read consecutive elements), folds the row slots through LDS and writes
 // part[block][channel chunk]. Channel chunks of at most 256 lie along grid.y.
@@ -116,6 +137,22 @@ int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int split
     case SFH_FP16: return launch_sum<fp16_t>(part, out, nelem, splits, st);
     default: return launch_sum<float>(part, out, nelem, splits, st);
   }
+}
+
+int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, int64_t nelem, int channels, int splits,
+                    hipStream_t st) {
+  if (nelem <= 0) return SFH_OK;
+  const dim3 grid((unsigned)cdiv(nelem / 4, kBlock));
+  if (dtype == SFH_BF16)
+    hipLaunchKernelGGL(sum_slices_bias_kernel<bf16_t>, grid, dim3(kBlock), 0, st, part, (const bf16_t*)bias, (bf16_t*)out, nelem,
+                       channels, splits);
+  else if (dtype == SFH_FP16)
+    hipLaunchKernelGGL(sum_slices_bias_kernel<fp16_t>, grid, dim3(kBlock), 0, st, part, (const fp16_t*)bias, (fp16_t*)out, nelem,
+                       channels, splits);
+  else
+    hipLaunchKernelGGL(sum_slices_bias_kernel<float>, grid, dim3(kBlock), 0, st, part, (const float*)bias, (float*)out, nelem,
+                       channels, splits);
+  return check_launch("sum_slices_bias_kernel");
 }
 
 size_t bias_grad_workspace_bytes(int64_t rows, int channels) {

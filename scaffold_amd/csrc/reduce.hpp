@@ -7,6 +7,10 @@ namespace sfh {
 // out[e] = sum over s < splits, in index order within fixed groups, of part[s * nelem + e]; one rounding to `dtype`.
 int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st);
 
+// out[e] = bias[e % channels] + sum over s < splits, in index order, of part[s * nelem + e]; nelem a multiple of 4.
+int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, int64_t nelem, int channels, int splits,
+                    hipStream_t st);
+
 // gb[c] = sum over rows of g[row * channels + c] for a dense (rows, channels) tensor of `dtype`; fp32
 // accumulation through partial slices in `ws`, result rounded once to `out_dtype`.
 size_t bias_grad_workspace_bytes(int64_t rows, int channels);

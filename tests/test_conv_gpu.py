@@ -71,6 +71,10 @@ MFMA_SHAPES = [
     (128, 64, (4, 4, 4), (1, 1, 1)),
     (32, 32, (2, 2, 2), (1, 1, 1)),
     (32, 32, (4, 6, 20), (2, 2, 2)),
+    # deep, small-volume levels: the forward / data gradient cut the reduction channels into summed slices
+    (256, 512, (4, 8, 8), (1, 1, 1)),
+    (512, 256, (6, 8, 8), (0, 1, 1)),
+    (128, 256, (8, 16, 16), (1, 1, 1)),
 ]
 
 
