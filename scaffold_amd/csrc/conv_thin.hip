@@ -200,6 +200,157 @@ __global__ void __launch_bounds__(kBlock) thin_reduce_kernel(ThinArgs a, const T
   }
 }
 
+// ---- the one-channel 3x3x3, stride-1 stem through an LDS brick ----------------------------------
+// The generic kernels above fetch the 27 taps of every voxel from global memory one scalar at a time, which
+// makes them instruction-bound. At stride 1 neighbouring voxels share their taps: a workgroup stages the
+// one-channel input brick of a 2 x 4 x 64 voxel tile (with its halo, zero outside the tensor) in LDS as fp32
+// once and every tap becomes an LDS read at an immediate offset.
+constexpr int kSTD = 2, kSTH = 4, kSTW = 64;                       // tile of output voxels
+constexpr int kSBD = kSTD + 2, kSBH = kSTH + 2, kSBW = kSTW + 2;   // brick with halo
+constexpr int kSBV = kSBD * kSBH * kSBW;
+
+struct StemTile { int n, d0, h0, w0; };
+
+__device__ __forceinline__ StemTile stem_tile(const ThinArgs& a, int tile, int tiles_h, int tiles_w, int tiles_d) {
+  StemTile t;
+  t.w0 = (tile % tiles_w) * kSTW; tile /= tiles_w;
+  t.h0 = (tile % tiles_h) * kSTH; tile /= tiles_h;
+  t.d0 = (tile % tiles_d) * kSTD;
+  t.n = tile / tiles_d;
+  return t;
+}
+
+template <typename T>
+__device__ __forceinline__ void stem_stage(const ThinArgs& a, const T* __restrict__ x, const StemTile& t, float* brick) {
+  const int id0 = t.d0 - a.pd, ih0 = t.h0 - a.ph, iw0 = t.w0 - a.pw;
+  for (int i = threadIdx.x; i < kSBV; i += kBlock) {
+    const int bw = i % kSBW, bh = (i / kSBW) % kSBH, bd = i / (kSBW * kSBH);
+    const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
+    float v = 0.f;
+    if ((unsigned)id < (unsigned)a.td && (unsigned)ih < (unsigned)a.th && (unsigned)iw < (unsigned)a.tw)
+      v = to_float(x[(((int64_t)t.n * a.td + id) * a.th + ih) * a.tw + iw]);
+    brick[i] = v;
+  }
+}
+
+// out[v][c] = bias[c] + sum_tap x[v (+) tap] * w[c][tap]. Thread = (voxel slot, V output channels), its V x 27 weights
+// in registers for the whole launch.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) stem_fwd_kernel(ThinArgs a, const T* __restrict__ x, const T* __restrict__ wt,
+                                                          const T* __restrict__ bias, T* __restrict__ out, int tiles_d, int tiles_h,
+                                                          int tiles_w) {
+  constexpr int V = VecOf<T>::N;
+  __shared__ float brick[kSBV];
+  const int tid = threadIdx.x;
+  const int wq = a.cw / V, rpp = kBlock / wq;
+  const int r = tid / wq, q = tid - r * wq;
+  const bool active = r < rpp;
+  float w[27][V], b[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int c = active ? q * V + e : 0;
+    b[e] = bias != nullptr ? to_float(bias[c]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < 27; ++j)
+      w[j][e] = to_float(wt[(int64_t)c * a.ws_wide + (j / 9) * a.ws_kd + ((j / 3) % 3) * a.ws_kh + (j % 3) * a.ws_kw]);
+  }
+  const StemTile t = stem_tile(a, blockIdx.x, tiles_h, tiles_w, tiles_d);
+  stem_stage<T>(a, x, t, brick);
+  __syncthreads();
+  if (!active) return;
+  for (int vi = r; vi < kSTD * kSTH * kSTW; vi += rpp) {
+    const int tw = vi % kSTW, th = (vi / kSTW) % kSTH, td = vi / (kSTW * kSTH);
+    const int od = t.d0 + td, oh = t.h0 + th, ow = t.w0 + tw;
+    if (od >= a.od || oh >= a.oh || ow >= a.ow) continue;
+    const float* src = brick + (td * kSBH + th) * kSBW + tw;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = b[e];
+#pragma unroll
+    for (int j = 0; j < 27; ++j) {
+      const float s = src[((j / 9) * kSBH + (j / 3) % 3) * kSBW + j % 3];
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = fmaf(s, w[j][e], acc[e]);
+    }
+    St<T, V>::run(out + ((((int64_t)t.n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cw + q * V, acc);
+  }
+}
+
+// G[c][tap] = sum_v gy[v][c] * x[v (+) tap]: thread = (voxel slot, V channels) with 27 x V accumulators over the
+// workgroup's range of tiles, folded through LDS into one fp32 slice per workgroup (layout of the weight gradient).
+template <typename T>
+__global__ void __launch_bounds__(kBlock) stem_wgrad_kernel(ThinArgs a, const T* __restrict__ x, const T* __restrict__ gy,
+                                                            float* __restrict__ part, int tiles_d, int tiles_h, int tiles_w,
+                                                            int ntiles, int tiles_per_wg) {
+  constexpr int V = VecOf<T>::N;
+  constexpr int JC = 4;
+  __shared__ float brick[kSBV];
+  __shared__ float buf[JC * kBlock * V];
+  const int tid = threadIdx.x;
+  const int wq = a.cw / V, rpp = kBlock / wq;
+  const int r = tid / wq, q = tid - r * wq;
+  const bool active = r < rpp;
+  float acc[27][V];
+#pragma unroll
+  for (int j = 0; j < 27; ++j)
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[j][e] = 0.f;
+  const int t_begin = blockIdx.x * tiles_per_wg;
+  int t_end = t_begin + tiles_per_wg;
+  if (t_end > ntiles) t_end = ntiles;
+  for (int tile = t_begin; tile < t_end; ++tile) {
+    const StemTile t = stem_tile(a, tile, tiles_h, tiles_w, tiles_d);
+    __syncthreads();  // the previous tile's brick is consumed
+    stem_stage<T>(a, x, t, brick);
+    __syncthreads();
+    if (active) {
+      for (int vi = r; vi < kSTD * kSTH * kSTW; vi += rpp) {
+        const int tw = vi % kSTW, th = (vi / kSTW) % kSTH, td = vi / (kSTW * kSTH);
+        const int od = t.d0 + td, oh = t.h0 + th, ow = t.w0 + tw;
+        if (od >= a.od || oh >= a.oh || ow >= a.ow) continue;
+        float f[V];
+        Ld<T, V>::run(gy + ((((int64_t)t.n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cw + q * V, f);
+        const float* src = brick + (td * kSBH + th) * kSBW + tw;
+#pragma unroll
+        for (int j = 0; j < 27; ++j) {
+          const float s = src[((j / 9) * kSBH + (j / 3) % 3) * kSBW + j % 3];
+#pragma unroll
+          for (int e = 0; e < V; ++e) acc[j][e] = fmaf(s, f[e], acc[j][e]);
+        }
+      }
+    }
+  }
+  float* dst = part + (int64_t)blockIdx.x * 27 * a.cw;
+#pragma unroll
+  for (int j0 = 0; j0 < 27; j0 += JC) {
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int jj = 0; jj < JC; ++jj)
+#pragma unroll
+        for (int e = 0; e < V; ++e) buf[(jj * rpp + r) * a.cw + q * V + e] = (j0 + jj < 27) ? acc[(j0 + jj) % 27][e] : 0.f;
+    }
+    __syncthreads();
+    for (int i = tid; i < JC * a.cw; i += kBlock) {
+      const int jj = i / a.cw, c = i - jj * a.cw;
+      if (j0 + jj < 27) {
+        float sum = 0.f;
+        for (int rr = 0; rr < rpp; ++rr) sum += buf[(jj * rpp + rr) * a.cw + c];
+        dst[(int64_t)c * a.so_wide + (int64_t)(j0 + jj) * a.so_thin] = sum;
+      }
+    }
+  }
+}
+
+bool stem_brick_ok(const ThinArgs& a) {
+  return a.K == 3 && a.sd == 1 && a.sh == 1 && a.sw == 1 && a.dd == 1 && a.dh == 1 && a.dw == 1 && a.pd <= 2 && a.ph <= 2 &&
+         a.pw <= 2;
+}
+
+int64_t stem_tiles(const ThinArgs& a) {
+  return (int64_t)a.n * cdiv(a.od, kSTD) * cdiv(a.oh, kSTH) * cdiv(a.ow, kSTW);
+}
+
 int wide_channels_ok(const ThinArgs& a, int dtype) {
   const int v = dtype == SFH_FP32 ? 4 : 8;
   return a.cw % v == 0 && a.cw / v <= kBlock && a.cw >= v;
@@ -244,6 +395,11 @@ int launch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* g
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
 template <typename T>
 int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
+  if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
+    hipLaunchKernelGGL(stem_fwd_kernel<T>, dim3((unsigned)stem_tiles(a)), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt,
+                       (const T*)bias, (T*)out, (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW));
+    return check_launch("stem_fwd_kernel");
+  }
   if (a.K == 3) return launch_wide_out<T, 3, 27>(a, thin, wt, bias, out, st);
   if (a.K == 2) return launch_wide_out<T, 2, 8>(a, thin, wt, bias, out, st);
   if (a.J <= 4) return launch_wide_out<T, 0, 4>(a, thin, wt, bias, out, st);
@@ -258,6 +414,16 @@ int dispatch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const
 }
 template <typename T>
 int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, void* ws, hipStream_t st) {
+  if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
+    const int nsplit = thin_reduce_splits(a);
+    const int ntiles = (int)stem_tiles(a);
+    const int per = (int)cdiv(ntiles, nsplit);
+    hipLaunchKernelGGL(stem_wgrad_kernel<T>, dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws,
+                       (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW), ntiles, per);
+    if (int rc = check_launch("stem_wgrad_kernel")) return rc;
+    const int dtype = sizeof(T) == 4 ? SFH_FP32 : (__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16);
+    return sum_slices(dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+  }
   if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, ws, st);
   if (a.K == 2) return launch_reduce<T, 2, 8>(a, thin, wide, gw, ws, st);
   if (a.J <= 4) return launch_reduce<T, 0, 4>(a, thin, wide, gw, ws, st);

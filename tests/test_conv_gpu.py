@@ -125,6 +125,8 @@ THIN_SHAPES = [
     # (n, cin, cout, spatial, kernel, stride, padding, bias)
     (1, 1, 32, (9, 10, 21), (3, 3, 3), (1, 1, 1), (1, 1, 1), True),     # U-Net stem
     (2, 1, 32, (6, 12, 12), (3, 3, 3), (1, 1, 1), (0, 1, 1), False),    # stem of a depth shard
+    (1, 1, 32, (5, 9, 70), (3, 3, 3), (1, 1, 1), (1, 1, 1), True),      # several LDS bricks, ragged in every axis
+    (1, 1, 8, (3, 5, 130), (3, 3, 3), (1, 1, 1), (2, 0, 1), False),
     (1, 1, 64, (9, 9, 9), (3, 3, 3), (2, 2, 2), (1, 1, 1), False),
     (1, 1, 16, (8, 8, 8), (2, 2, 2), (2, 2, 2), (0, 0, 0), True),
     (1, 32, 11, (7, 9, 13), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),     # U-Net head
