@@ -230,16 +230,17 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   }
 }
 
-// One thread per packed element.
+// One thread per packed 16-byte piece: the 8 consecutive reduction channels of one (output channel, tap, k-half).
+// With the reduction channel innermost in memory (forward, channels-last weight) that is one 16-byte load;
+// otherwise eight 2-byte loads, each coalesced across the wavefront's 32 consecutive output channels.
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, T* __restrict__ packed, int cout, int cred,
                                                           int kd, int kh, int kw, int64_t s_out, int64_t s_red, int64_t s_kd,
-                                                          int64_t s_kh, int64_t s_kw, int flip, int64_t total) {
+                                                          int64_t s_kh, int64_t s_kw, int flip, int64_t pieces) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= total) return;
+  if (idx >= pieces) return;
   const int taps = kd * kh * kw;
   int64_t r = idx;
-  const int e = (int)(r % 8); r /= 8;
   const int lane = (int)(r % 64); r /= 64;
   const int ks = (int)(r % 2); r /= 2;
   int tap = (int)(r % taps); r /= taps;
@@ -247,10 +248,21 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ 
   const int cc = (int)(r % ncc);
   const int nblk = (int)(r / ncc);
   const int co = nblk * 32 + (lane & 31);
-  const int ci = cc * kChunk + ks * 16 + (lane >> 5) * 8 + e;
+  const int ci = cc * kChunk + ks * 16 + (lane >> 5) * 8;
   if (flip) tap = taps - 1 - tap;
   const int tkw = tap % kw, tkh = (tap / kw) % kh, tkd = tap / (kw * kh);
-  packed[idx] = w[co * s_out + ci * s_red + tkd * s_kd + tkh * s_kh + tkw * s_kw];
+  const T* src = w + co * s_out + ci * s_red + tkd * s_kd + tkh * s_kh + tkw * s_kw;
+  uint4 v;
+  if (s_red == 1 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+    v = *reinterpret_cast<const uint4*>(src);
+  } else {
+    uint16_t h[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = *reinterpret_cast<const uint16_t*>(src + e * s_red);
+    v.x = h[0] | ((uint32_t)h[1] << 16); v.y = h[2] | ((uint32_t)h[3] << 16);
+    v.z = h[4] | ((uint32_t)h[5] << 16); v.w = h[6] | ((uint32_t)h[7] << 16);
+  }
+  *reinterpret_cast<uint4*>(packed + idx * 8) = v;
 }
 
 struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
@@ -326,7 +338,7 @@ size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a) {
 
 int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd, int64_t s_kh,
                      int64_t s_kw, int flip, void* packed, hipStream_t st) {
-  const int64_t total = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw;
+  const int64_t total = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw / 8;  // 16-byte pieces
   const unsigned blocks = (unsigned)cdiv(total, 256);
   if (dtype == SFH_BF16)
     hipLaunchKernelGGL(pack_weight_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)w, (bf16_t*)packed, a.cout,
