@@ -175,8 +175,17 @@ __device__ __forceinline__ void persist_step(const char* cur, char* nxt, int wav
       if (have_store && ps.off[ms] >= 0) *reinterpret_cast<uint2*>(y + ps.off[ms] + 8 * g) = ps.data[ms][g];
     }
     __builtin_amdgcn_sched_barrier(0);
+    if (it == 0 && !STREAM) {
+      // a single-chunk brick starts from zero: the first MFMA takes a zero addend instead of a clearing pass
+      f32x16_t zero;
 #pragma unroll
-    for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+#pragma unroll
+      for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
+    } else {
+#pragma unroll
+      for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+    }
     if (STREAM) wq[it] = *reinterpret_cast<const uint4*>(wnext + it * FRAG);
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -255,6 +264,17 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's part of the brick has landed
   __syncthreads();
 
+  // Output position of this lane's voxel of every sub-tile relative to the brick origin: coordinates (for the
+  // ragged-edge test) and element offset, fixed for the whole launch.
+  int vcoord[C::MS], vrel[C::MS];
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms) {
+    const int v = (wave * C::MS + ms) * 32 + j;
+    const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
+    vcoord[ms] = td | (th << 8) | (tw << 16);
+    vrel[ms] = ((td * a.oh + th) * a.ow + tw) * a.cout + 4 * kg;
+  }
+
   f32x16_t acc[C::MS];
   PendingStore<C> ps;
 #pragma unroll
@@ -272,7 +292,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     // slab to stream into the weight registers during this step (the current one again at the end)
     const T* wnext = wblock + (int64_t)(has_next ? ncc_next : cc) * slab;
 
-    if (cc == 0) {
+    if (STREAM && cc == 0) {
 #pragma unroll
       for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
@@ -287,14 +307,13 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
       // Round the finished brick now; its stores ride along with the next step's MFMAs. Accumulator
       // register 4g+t of a lane is output channel 8g + 4*kg + t of voxel j of the sub-tile: the two
       // k-half lanes of a voxel write adjacent 8-byte halves of a 16-byte piece.
-      const int tw_i = tc.w, th_i = tc.h, td_i = tc.d, n = tc.n;
+      const int od0 = tc.d * C::TD, oh0 = tc.h * C::TH, ow0 = tc.w * C::TW;
+      const int64_t tile_off = ((((int64_t)tc.n * a.od + od0) * a.oh + oh0) * a.ow + ow0) * a.cout + nb * 32;  // wave-uniform
 #pragma unroll
       for (int ms = 0; ms < C::MS; ++ms) {
-        const int v = (wave * C::MS + ms) * 32 + j;
-        const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
-        const int od = td_i * C::TD + td, oh = th_i * C::TH + th, ow = tw_i * C::TW + tw;
-        const bool ok = od < a.od && oh < a.oh && ow < a.ow;
-        ps.off[ms] = ok ? ((((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cout + nb * 32 + 4 * kg : -1;
+        const int td = vcoord[ms] & 0xff, th = (vcoord[ms] >> 8) & 0xff, tw = vcoord[ms] >> 16;
+        const bool ok = od0 + td < a.od && oh0 + th < a.oh && ow0 + tw < a.ow;
+        ps.off[ms] = ok ? tile_off + vrel[ms] : -1;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           if (bias != nullptr) {
