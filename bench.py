@@ -182,9 +182,8 @@ def copy_calibration(device, mib=256, reps=4):
 
 def bench_unet_step(args, device):
     """Config 5: one Adam step of the base-32, 5-level U-Net on a 64x128x128 depth shard (zero halo),
-    bf16 autocast, fp32 master weights, CE + Dice loss, gradient clipping at 1.0."""
+    bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0."""
     import scaffold_amd as sa
-    from oracle.oracle import train_step_loss  # loss recipe only; the model and kernels are the product's
 
     torch.manual_seed(5001)
     model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
@@ -196,7 +195,7 @@ def bench_unet_step(args, device):
     def step():
         with torch.autocast("cuda", dtype=torch.bfloat16):
             logits = model(occ)
-        loss = train_step_loss(logits, lab, 11)
+        loss = sa.ce_dice_loss(logits, lab)
         loss.backward()
         torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
         opt.step()

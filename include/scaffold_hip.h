@@ -150,6 +150,29 @@ int sfh_groupnorm_bwd(const sfh_groupnorm_desc* p, int x_dtype, int dy_dtype, in
                       const float* rstd, void* dx, float* dgamma, float* dbeta, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* ---- loss head ------------------------------------------------------------------------
+ * Stands in for the loss block of the reference's train step (ScaFFold/utils/trainer.py:634-663):
+ * fp32 log-softmax of the class logits, cross entropy summed and divided by its normaliser
+ * (ScaFFold/utils/losses.py:119-214; the voxel count, or the sum of the target weights when class
+ * weights are given), soft Dice per (sample, class) (ScaFFold/utils/dice_score.py:101-136) and
+ *   loss = CE + 1 - mean over samples and classes >= 1 of (2 I + eps) / (P + T + eps).
+ * logits: dense (N, S, classes) of `dtype` (a channels-last (N, classes, D, H, W) tensor);
+ * labels: (N, S) int64, values outside [0, classes) contribute nothing; class_weight: `classes`
+ * floats or NULL; loss: one float; stats: N*3*classes + 2 floats kept for the backward.
+ * The backward writes d loss / d logits * grad_loss[0] in `dtype`. 2 <= classes <= 32. */
+typedef struct sfh_loss_desc {
+  int32_t n, classes;
+  int64_t spatial;
+  float eps;
+} sfh_loss_desc;
+size_t sfh_ce_dice_workspace_bytes(const sfh_loss_desc* p);
+int sfh_ce_dice_fwd(const sfh_loss_desc* p, int dtype, const void* logits, const int64_t* labels,
+                    const float* class_weight, float* loss, float* stats, void* workspace,
+                    size_t workspace_bytes, void* stream);
+int sfh_ce_dice_bwd(const sfh_loss_desc* p, int dtype, const void* logits, const int64_t* labels,
+                    const float* class_weight, const float* stats, const float* grad_loss,
+                    void* dlogits, void* stream);
+
 /* ---- measurement helper --------------------------------------------------------------
  * A plain streaming copy of `bytes` bytes (multiple of 16) used to calibrate achieved HBM
  * bandwidth and the scale of the FETCH_SIZE / WRITE_SIZE counters. Has no counterpart in the

@@ -342,11 +342,13 @@ def gn_rel_error(actual: torch.Tensor, expected: torch.Tensor) -> float:
 # ---------------------------------------------------------------------------------------------
 # train step recipe (config 5)
 # ---------------------------------------------------------------------------------------------
-def train_step_loss(logits: torch.Tensor, labels: torch.Tensor, n_classes: int, eps: float = 1e-6) -> torch.Tensor:
-    """fp32 log-softmax -> mean cross entropy + (1 - mean foreground soft Dice)
-    (``ScaFFold/utils/trainer.py:640-663``, ``ScaFFold/utils/dice_score.py:101-136``; uniform class weights)."""
-    logp = F.log_softmax(logits.float(), dim=1)
-    ce = F.nll_loss(logp, labels)
+def train_step_loss(logits: torch.Tensor, labels: torch.Tensor, n_classes: int, eps: float = 1e-6, class_weight=None,
+                    dtype=torch.float32) -> torch.Tensor:
+    """log-softmax in ``dtype`` -> (weighted) mean cross entropy + (1 - mean foreground soft Dice)
+    (``ScaFFold/utils/trainer.py:640-663``, ``ScaFFold/utils/losses.py:119-214``,
+    ``ScaFFold/utils/dice_score.py:101-136``)."""
+    logp = F.log_softmax(logits.to(dtype), dim=1)
+    ce = F.nll_loss(logp, labels, weight=None if class_weight is None else class_weight.to(dtype))
     prob = logp.exp()
     onehot = F.one_hot(labels, n_classes).movedim(-1, 1).to(prob.dtype)
     dims = (2, 3, 4)

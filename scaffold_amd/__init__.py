@@ -25,6 +25,8 @@ _EXPORTS = {
     "is_supported_transposed_bwd_weight": "transposed", "grad_transposed_weight_empty": "transposed",
     # GroupNorm
     "group_norm": "groupnorm", "triton_group_norm": "groupnorm", "MATCH_STOCK_DTYPE": "groupnorm",
+    # loss head
+    "ce_dice_loss": "losses", "is_supported_loss": "losses",
     # modules / model
     "FastConv3d": "modules", "FastConvTranspose3d": "modules", "FastGroupNorm": "modules",
     "UNet": "unet",

@@ -28,6 +28,7 @@ __all__ = [
     "ConvDesc",
     "ConvTDesc",
     "GroupNormDesc",
+    "LossDesc",
     "dtype_code",
     "SUPPORTED_DTYPES",
     "EXPORTED_SYMBOLS",
@@ -56,6 +57,10 @@ class ConvDesc(ctypes.Structure):
 
 class ConvTDesc(ctypes.Structure):
     _fields_ = [(k, c_int32) for k in ("n", "cin", "in_d", "in_h", "in_w", "cout", "kd", "kh", "kw")]
+
+
+class LossDesc(ctypes.Structure):
+    _fields_ = [("n", c_int32), ("classes", c_int32), ("spatial", c_int64), ("eps", c_float)]
 
 
 class GroupNormDesc(ctypes.Structure):
@@ -93,6 +98,10 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "sfh_bias_grad_workspace_bytes": (c_size_t, [c_int64, c_int32]),
     "sfh_bias_grad": (c_int, [c_int, c_int, c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_ce_dice_workspace_bytes": (c_size_t, [POINTER(LossDesc)]),
+    "sfh_ce_dice_fwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                                c_void_p]),
+    "sfh_ce_dice_bwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_stream_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

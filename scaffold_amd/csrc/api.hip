@@ -7,6 +7,7 @@
 #include "conv_mfma.hpp"
 #include "conv_patch.hpp"
 #include "conv_thin.hpp"
+#include "loss.hpp"
 #include "reduce.hpp"
 #include "wgrad_mfma.hpp"
 
@@ -479,6 +480,39 @@ extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void*
     return patch_scatter(convT_patch_args(*p), dtype, x, workspace, bias, y, st);
   }
   return direct_convT(*p, dtype, w_stride, x, w, bias, y, (hipStream_t)stream);
+}
+
+// ---- loss head -------------------------------------------------------------------------
+static int check_loss(const sfh_loss_desc* p, int dtype) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "ce_dice: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "ce_dice: bad dtype %d", dtype);
+  if (!loss_supported(*p))
+    return fail(SFH_ERR_UNSUPPORTED, "ce_dice: n=%d classes=%d spatial=%lld (2..32 classes, non-empty)", p->n, p->classes,
+                (long long)p->spatial);
+  return SFH_OK;
+}
+
+extern "C" size_t sfh_ce_dice_workspace_bytes(const sfh_loss_desc* p) {
+  if (p == nullptr || !loss_supported(*p)) return 0;
+  return loss_workspace_bytes(*p);
+}
+
+extern "C" int sfh_ce_dice_fwd(const sfh_loss_desc* p, int dtype, const void* logits, const int64_t* labels, const float* class_weight,
+                               float* loss, float* stats, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int rc = check_loss(p, dtype)) return rc;
+  if (logits == nullptr || labels == nullptr || loss == nullptr || stats == nullptr) return fail(SFH_ERR_INVALID, "ce_dice: null tensor");
+  const size_t need = loss_workspace_bytes(*p);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "ce_dice fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  return loss_forward(*p, dtype, logits, labels, class_weight, loss, stats, workspace, (hipStream_t)stream);
+}
+
+extern "C" int sfh_ce_dice_bwd(const sfh_loss_desc* p, int dtype, const void* logits, const int64_t* labels, const float* class_weight,
+                               const float* stats, const float* grad_loss, void* dlogits, void* stream) {
+  if (int rc = check_loss(p, dtype)) return rc;
+  if (logits == nullptr || labels == nullptr || stats == nullptr || grad_loss == nullptr || dlogits == nullptr)
+    return fail(SFH_ERR_INVALID, "ce_dice: null tensor");
+  return loss_backward(*p, dtype, logits, labels, class_weight, stats, grad_loss, dlogits, (hipStream_t)stream);
 }
 
 // ---- measurement helper ----------------------------------------------------------------

@@ -1,0 +1,288 @@
+// Loss head of the U-Net train step, fused: fp32 log-softmax over the class logits of every voxel, the
+// (optionally class-weighted) cross-entropy sum with its normaliser, and the soft-Dice sums per (sample, class)
+// in ONE pass over the logits; the backward is one more pass. This is the block ScaFFold/utils/trainer.py:634-663
+// builds from torch ops (log_softmax -> nll_loss(reduction="none").sum() / normaliser, ScaFFold/utils/losses.py:
+// 119-214; exp -> Dice sums -> (2I + eps) / (P + T + eps), ScaFFold/utils/dice_score.py:101-136; loss =
+// CE + 1 - mean foreground Dice, trainer.py:331-333,660-663). It is bandwidth-bound: 22 B of bf16 logits and an
+// 8-byte label per voxel at 11 classes.
+//
+// No atomics: every workgroup leaves its partial sums in its own slot and one workgroup adds the slots in a
+// fixed order (the reference avoids the atomic fused reduction for the same reason, losses.py:156-160).
+#include "loss.hpp"
+
+namespace sfh {
+namespace {
+
+constexpr int kBlock = 256;
+
+template <typename T> __device__ __forceinline__ float ld(const T* p) { return to_float(*p); }
+
+__device__ __forceinline__ float wave_sum_all(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;  // lane 0 holds the sum
+}
+
+// Quantities per sample: inter[c], psum[c], tsum[c] (3 * C), then the two launch-wide ones: ce_sum, normaliser.
+template <typename T, int CMAX>
+__global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                          const float* __restrict__ cw, float* __restrict__ part, int64_t S, int C,
+                                                          int nsplit, int64_t per_split) {
+  extern __shared__ char smem_raw[];
+  T* tile = reinterpret_cast<T*>(smem_raw);  // kBlock voxels x C logits
+  __shared__ float red[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = blockIdx.y, split = blockIdx.x;
+  const T* src = logits + (int64_t)n * S * C;
+  const int64_t* lab = labels + (int64_t)n * S;
+  float inter[CMAX], psum[CMAX], tsum[CMAX], ce = 0.f, norm = 0.f;
+#pragma unroll
+  for (int c = 0; c < CMAX; ++c) inter[c] = psum[c] = tsum[c] = 0.f;
+  const int64_t begin = (int64_t)split * per_split;
+  int64_t end = begin + per_split;
+  if (end > S) end = S;
+  for (int64_t v0 = begin; v0 < end; v0 += kBlock) {
+    const int nv = (int)((end - v0) < kBlock ? (end - v0) : kBlock);
+    __syncthreads();
+    for (int i = tid; i < nv * C; i += kBlock) tile[i] = src[v0 * C + i];
+    __syncthreads();
+    if (tid < nv) {
+      float x[CMAX];
+      float m = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        x[c] = c < C ? to_float(tile[tid * C + c]) : -INFINITY;
+        m = fmaxf(m, x[c]);
+      }
+      float s = 0.f;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        x[c] = c < C ? expf(x[c] - m) : 0.f;  // x now holds exp(logit - max)
+        s += x[c];
+      }
+      const float inv = 1.f / s, logs = logf(s);
+      const int64_t y = lab[v0 + tid];
+      const bool valid = y >= 0 && y < C;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        const float p = x[c] * inv;
+        const bool hit = valid && c == (int)y;
+        psum[c] += p;
+        inter[c] += hit ? p : 0.f;
+        tsum[c] += hit ? 1.f : 0.f;
+      }
+      if (valid) {
+        const float w = cw != nullptr ? cw[y] : 1.f;
+        // -log p_y = log(sum) - (logit_y - max)
+        ce += w * (logs - (to_float(tile[tid * C + (int)y]) - m));
+        norm += w;
+      }
+    }
+  }
+  // workgroup totals: wavefront trees, then the four wave totals in order
+  float* dst = part + ((int64_t)n * nsplit + split) * (3 * C + 2);
+  auto fold = [&](float v, int slot) {
+    v = wave_sum_all(v);
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    if (tid == 0) dst[slot] = (red[0] + red[1]) + (red[2] + red[3]);
+  };
+#pragma unroll
+  for (int c = 0; c < CMAX; ++c) {
+    if (c < C) {
+      fold(inter[c], c);
+      fold(psum[c], C + c);
+      fold(tsum[c], 2 * C + c);
+    }
+  }
+  fold(ce, 3 * C);
+  fold(norm, 3 * C + 1);
+}
+
+// One workgroup: fixed-order sums of the slots, then the scalar loss.
+// stats: inter[N][C] | psum[N][C] | tsum[N][C] | ce_sum | normaliser
+__global__ void __launch_bounds__(kBlock) ce_dice_finalize(const float* __restrict__ part, float* __restrict__ stats,
+                                                           float* __restrict__ loss, int N, int C, int nsplit, float eps,
+                                                           int unweighted, float count) {
+  __shared__ float tot[2];
+  const int Q = 3 * C + 2;
+  for (int i = threadIdx.x; i < N * 3 * C; i += kBlock) {
+    const int n = i / (3 * C), q = i - n * 3 * C;
+    float s = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) s += part[((int64_t)n * nsplit + sp) * Q + q];
+    stats[(q / C) * N * C + n * C + q % C] = s;
+  }
+  if (threadIdx.x < 2) {
+    float s = 0.f;
+    for (int n = 0; n < N; ++n)
+      for (int sp = 0; sp < nsplit; ++sp) s += part[((int64_t)n * nsplit + sp) * Q + 3 * C + threadIdx.x];
+    if (threadIdx.x == 1 && unweighted) s = count;  // the normaliser of the unweighted mean is the voxel count
+    tot[threadIdx.x] = s;
+    stats[N * 3 * C + threadIdx.x] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const float* inter = stats;
+    const float* psum = stats + N * C;
+    const float* tsum = stats + 2 * N * C;
+    float dice = 0.f;
+    for (int n = 0; n < N; ++n)
+      for (int c = 1; c < C; ++c) {
+        const float two_i = 2.f * inter[n * C + c];
+        float sets = psum[n * C + c] + tsum[n * C + c];
+        if (sets == 0.f) sets = two_i;
+        dice += (two_i + eps) / (sets + eps);
+      }
+    dice /= (float)(N * (C - 1));
+    const float ce = tot[0] / fmaxf(tot[1], 1.1920929e-07f);
+    loss[0] = ce + (1.f - dice);
+  }
+}
+
+// dlogits[v][j] = gl * ( w_y / normaliser * (p_j - [j == y])  +  p_j * (g_j - sum_c g_c p_c) ),
+// g_c = -(1 / (N (C-1))) * d dice_c / d p_c = -(1 / (N (C-1))) * ([c == y] * 2 / den_c - (2 I_c + eps) / den_c^2), g_0 = 0.
+template <typename T, int CMAX>
+__global__ void __launch_bounds__(kBlock) ce_dice_backward(const T* __restrict__ logits, const int64_t* __restrict__ labels,
+                                                           const float* __restrict__ cw, const float* __restrict__ stats,
+                                                           const float* __restrict__ grad_loss, T* __restrict__ dlogits, int64_t S,
+                                                           int N, int C, float eps, int64_t per_split) {
+  extern __shared__ char smem_raw[];
+  T* tile = reinterpret_cast<T*>(smem_raw);
+  __shared__ float ca[CMAX], cb[CMAX];
+  const int tid = threadIdx.x;
+  const int n = blockIdx.y, split = blockIdx.x;
+  const float gl = grad_loss[0];
+  if (tid < CMAX) {
+    float a = 0.f, b = 0.f;
+    if (tid >= 1 && tid < C) {
+      const float two_i = 2.f * stats[n * C + tid];
+      float sets = stats[N * C + n * C + tid] + stats[2 * N * C + n * C + tid];
+      if (sets == 0.f) sets = two_i;
+      const float den = sets + eps, k = -gl / (float)(N * (C - 1));
+      a = k * 2.f / den;
+      b = k * (two_i + eps) / (den * den);
+    }
+    ca[tid] = a;
+    cb[tid] = b;
+  }
+  const float ce_scale = gl / fmaxf(stats[N * 3 * C + 1], 1.1920929e-07f);
+  const T* src = logits + (int64_t)n * S * C;
+  T* dst = dlogits + (int64_t)n * S * C;
+  const int64_t* lab = labels + (int64_t)n * S;
+  const int64_t begin = (int64_t)split * per_split;
+  int64_t end = begin + per_split;
+  if (end > S) end = S;
+  for (int64_t v0 = begin; v0 < end; v0 += kBlock) {
+    const int nv = (int)((end - v0) < kBlock ? (end - v0) : kBlock);
+    __syncthreads();
+    for (int i = tid; i < nv * C; i += kBlock) tile[i] = src[v0 * C + i];
+    __syncthreads();
+    if (tid < nv) {
+      float p[CMAX];
+      float m = -INFINITY;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        p[c] = c < C ? to_float(tile[tid * C + c]) : -INFINITY;
+        m = fmaxf(m, p[c]);
+      }
+      float s = 0.f;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        p[c] = c < C ? expf(p[c] - m) : 0.f;
+        s += p[c];
+      }
+      const float inv = 1.f / s;
+      const int64_t y = lab[v0 + tid];
+      const bool valid = y >= 0 && y < C;
+      float g[CMAX], dot = 0.f, wy = 0.f;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        p[c] *= inv;
+        const bool hit = valid && c == (int)y;
+        g[c] = (hit ? ca[c] : 0.f) - cb[c];
+        dot = fmaf(g[c], p[c], dot);
+        if (hit) wy = cw != nullptr ? cw[c] : 1.f;
+      }
+      const float cs = ce_scale * wy;
+#pragma unroll
+      for (int c = 0; c < CMAX; ++c) {
+        if (c < C) {
+          const bool hit = valid && c == (int)y;
+          const float d = fmaf(p[c], g[c] - dot, cs * (p[c] - (hit ? 1.f : 0.f)));
+          tile[tid * C + c] = elem<T>::from_float(d);
+        }
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < nv * C; i += kBlock) dst[v0 * C + i] = tile[i];
+  }
+}
+
+struct LossPlan { int nsplit; int64_t per_split; };
+
+LossPlan loss_plan(const sfh_loss_desc& p) {
+  LossPlan pl;
+  int64_t want = cdiv(4 * kComputeUnits, p.n);
+  const int64_t tiles = cdiv(p.spatial, kBlock);
+  if (want > tiles) want = tiles;
+  if (want < 1) want = 1;
+  pl.per_split = cdiv(tiles, want) * kBlock;
+  pl.nsplit = (int)cdiv(p.spatial, pl.per_split);
+  return pl;
+}
+
+template <typename T, int CMAX>
+int fwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels, const float* cw, float* loss, float* stats,
+              float* ws, hipStream_t st) {
+  const LossPlan pl = loss_plan(p);
+  const size_t lds = (size_t)kBlock * p.classes * sizeof(T);
+  hipLaunchKernelGGL((ce_dice_partial<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, ws,
+                     p.spatial, p.classes, pl.nsplit, pl.per_split);
+  if (int rc = check_launch("ce_dice_partial")) return rc;
+  hipLaunchKernelGGL(ce_dice_finalize, dim3(1), dim3(kBlock), 0, st, ws, stats, loss, p.n, p.classes, pl.nsplit, p.eps,
+                     cw == nullptr ? 1 : 0, (float)p.n * (float)p.spatial);
+  return check_launch("ce_dice_finalize");
+}
+
+template <typename T, int CMAX>
+int bwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels, const float* cw, const float* stats,
+              const float* grad_loss, void* dlogits, hipStream_t st) {
+  const LossPlan pl = loss_plan(p);
+  const size_t lds = (size_t)kBlock * p.classes * sizeof(T);
+  hipLaunchKernelGGL((ce_dice_backward<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, stats,
+                     grad_loss, (T*)dlogits, p.spatial, p.n, p.classes, p.eps, pl.per_split);
+  return check_launch("ce_dice_backward");
+}
+
+}  // namespace
+
+bool loss_supported(const sfh_loss_desc& p) {
+  return p.n >= 1 && p.classes >= 2 && p.classes <= 32 && p.spatial >= 1 && (int64_t)p.n * cdiv(p.spatial, kBlock) < 0x7fffffffLL;
+}
+
+size_t loss_workspace_bytes(const sfh_loss_desc& p) {
+  return (size_t)p.n * loss_plan(p).nsplit * (3 * p.classes + 2) * sizeof(float);
+}
+
+#define SFH_LOSS_DISPATCH(fn, ...)                                               \
+  if (p.classes <= 16) {                                                         \
+    if (dtype == SFH_BF16) return fn<bf16_t, 16>(__VA_ARGS__);                   \
+    if (dtype == SFH_FP16) return fn<fp16_t, 16>(__VA_ARGS__);                   \
+    return fn<float, 16>(__VA_ARGS__);                                           \
+  }                                                                              \
+  if (dtype == SFH_BF16) return fn<bf16_t, 32>(__VA_ARGS__);                     \
+  if (dtype == SFH_FP16) return fn<fp16_t, 32>(__VA_ARGS__);                     \
+  return fn<float, 32>(__VA_ARGS__);
+
+int loss_forward(const sfh_loss_desc& p, int dtype, const void* logits, const int64_t* labels, const float* cw, float* loss,
+                 float* stats, void* ws, hipStream_t st) {
+  SFH_LOSS_DISPATCH(fwd_typed, p, logits, labels, cw, loss, stats, (float*)ws, st)
+}
+
+int loss_backward(const sfh_loss_desc& p, int dtype, const void* logits, const int64_t* labels, const float* cw, const float* stats,
+                  const float* grad_loss, void* dlogits, hipStream_t st) {
+  SFH_LOSS_DISPATCH(bwd_typed, p, logits, labels, cw, stats, grad_loss, dlogits, st)
+}
+
+}  // namespace sfh

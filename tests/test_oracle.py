@@ -240,3 +240,23 @@ def test_ifs_volume_is_seeded_and_labelled():
     occ2, lab2 = orc.ifs_volume((16, 16, 16), iterations=4000, seed=1)
     assert torch.equal(lab, lab2) and occ.shape == (1, 1, 16, 16, 16) and lab.shape == (1, 16, 16, 16)
     assert 0 < occ.mean() < 0.5 and lab.max() <= 10 and torch.equal(occ[0, 0] > 0, lab[0] > 0)
+
+
+def test_train_step_loss_weighted_ce_closed_form():
+    """Two voxels, two classes, uniform logits: p = 1/2 everywhere, CE = log 2 whatever the weights (weighted mean of
+    equal terms); with logits (a, 0) on the class-0 voxel only that voxel's term changes, weighted by w0 / (w0 + w1)."""
+    import math
+    labels = torch.tensor([[[[0, 1]]]])
+    w = torch.tensor([3.0, 1.0], dtype=torch.float64)
+    logits = torch.zeros((1, 2, 1, 1, 2), dtype=torch.float64)
+    base = orc.train_step_loss(logits, labels, 2, class_weight=w, dtype=torch.float64)
+    dice1 = (2 * 0.5 + 1e-6) / (1.0 + 1.0 + 1e-6)
+    assert abs(base.item() - (math.log(2) + 1 - dice1)) < 1e-12
+    a = 1.3
+    logits[0, 0, 0, 0, 0] = a
+    p0 = math.exp(a) / (math.exp(a) + 1)
+    ce = (3.0 * -math.log(p0) + 1.0 * math.log(2)) / 4.0
+    i1, p1 = 0.5, (1 - p0) + 0.5
+    dice1 = (2 * i1 + 1e-6) / (p1 + 1.0 + 1e-6)
+    got = orc.train_step_loss(logits, labels, 2, class_weight=w, dtype=torch.float64)
+    assert abs(got.item() - (ce + 1 - dice1)) < 1e-12
