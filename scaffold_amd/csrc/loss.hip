@@ -100,42 +100,50 @@ __global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ 
   fold(norm, 3 * C + 1);
 }
 
-// One workgroup: fixed-order sums of the slots, then the scalar loss.
+// One 64-lane workgroup per quantity: lane l adds slots l, l + 64, ... and the lane totals meet in a fixed tree.
 // stats: inter[N][C] | psum[N][C] | tsum[N][C] | ce_sum | normaliser
-__global__ void __launch_bounds__(kBlock) ce_dice_finalize(const float* __restrict__ part, float* __restrict__ stats,
-                                                           float* __restrict__ loss, int N, int C, int nsplit, float eps,
-                                                           int unweighted, float count) {
-  __shared__ float tot[2];
+__global__ void __launch_bounds__(64) ce_dice_sum(const float* __restrict__ part, float* __restrict__ stats, int N, int C, int nsplit,
+                                                  int unweighted, float count) {
   const int Q = 3 * C + 2;
-  for (int i = threadIdx.x; i < N * 3 * C; i += kBlock) {
-    const int n = i / (3 * C), q = i - n * 3 * C;
-    float s = 0.f;
-    for (int sp = 0; sp < nsplit; ++sp) s += part[((int64_t)n * nsplit + sp) * Q + q];
-    stats[(q / C) * N * C + n * C + q % C] = s;
+  const int b = blockIdx.x, lane = threadIdx.x;
+  float s = 0.f;
+  int dst;
+  if (b < N * 3 * C) {
+    const int n = b / (3 * C), q = b - n * 3 * C;
+    const float* src = part + (int64_t)n * nsplit * Q + q;
+    for (int sp = lane; sp < nsplit; sp += 64) s += src[(int64_t)sp * Q];
+    dst = (q / C) * N * C + n * C + q % C;
+  } else {
+    const int q = 3 * C + (b - N * 3 * C);  // ce_sum or normaliser, over all samples
+    for (int i = lane; i < N * nsplit; i += 64) s += part[(int64_t)i * Q + q];
+    dst = b;
   }
-  if (threadIdx.x < 2) {
-    float s = 0.f;
-    for (int n = 0; n < N; ++n)
-      for (int sp = 0; sp < nsplit; ++sp) s += part[((int64_t)n * nsplit + sp) * Q + 3 * C + threadIdx.x];
-    if (threadIdx.x == 1 && unweighted) s = count;  // the normaliser of the unweighted mean is the voxel count
-    tot[threadIdx.x] = s;
-    stats[N * 3 * C + threadIdx.x] = s;
+  s = wave_sum_all(s);
+  if (lane == 0) {
+    if (b == N * 3 * C + 1 && unweighted) s = count;  // the normaliser of the unweighted mean is the voxel count
+    stats[dst] = s;
   }
-  __syncthreads();
+}
+
+__global__ void __launch_bounds__(64) ce_dice_scalar(const float* __restrict__ stats, float* __restrict__ loss, int N, int C, float eps) {
+  // one lane per (sample, foreground class) pass; the Dice terms meet in the fixed wavefront tree
+  const float* inter = stats;
+  const float* psum = stats + N * C;
+  const float* tsum = stats + 2 * N * C;
+  float dice = 0.f;
+  for (int i = threadIdx.x; i < N * C; i += 64) {
+    const int c = i % C;
+    if (c >= 1) {
+      const float two_i = 2.f * inter[i];
+      float sets = psum[i] + tsum[i];
+      if (sets == 0.f) sets = two_i;
+      dice += (two_i + eps) / (sets + eps);
+    }
+  }
+  dice = wave_sum_all(dice);
   if (threadIdx.x == 0) {
-    const float* inter = stats;
-    const float* psum = stats + N * C;
-    const float* tsum = stats + 2 * N * C;
-    float dice = 0.f;
-    for (int n = 0; n < N; ++n)
-      for (int c = 1; c < C; ++c) {
-        const float two_i = 2.f * inter[n * C + c];
-        float sets = psum[n * C + c] + tsum[n * C + c];
-        if (sets == 0.f) sets = two_i;
-        dice += (two_i + eps) / (sets + eps);
-      }
     dice /= (float)(N * (C - 1));
-    const float ce = tot[0] / fmaxf(tot[1], 1.1920929e-07f);
+    const float ce = stats[N * 3 * C] / fmaxf(stats[N * 3 * C + 1], 1.1920929e-07f);
     loss[0] = ce + (1.f - dice);
   }
 }
@@ -240,9 +248,11 @@ int fwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels,
   hipLaunchKernelGGL((ce_dice_partial<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, ws,
                      p.spatial, p.classes, pl.nsplit, pl.per_split);
   if (int rc = check_launch("ce_dice_partial")) return rc;
-  hipLaunchKernelGGL(ce_dice_finalize, dim3(1), dim3(kBlock), 0, st, ws, stats, loss, p.n, p.classes, pl.nsplit, p.eps,
+  hipLaunchKernelGGL(ce_dice_sum, dim3(p.n * 3 * p.classes + 2), dim3(64), 0, st, ws, stats, p.n, p.classes, pl.nsplit,
                      cw == nullptr ? 1 : 0, (float)p.n * (float)p.spatial);
-  return check_launch("ce_dice_finalize");
+  if (int rc = check_launch("ce_dice_sum")) return rc;
+  hipLaunchKernelGGL(ce_dice_scalar, dim3(1), dim3(64), 0, st, stats, loss, p.n, p.classes, p.eps);
+  return check_launch("ce_dice_scalar");
 }
 
 template <typename T, int CMAX>
