@@ -205,3 +205,50 @@ def test_up_equals_explicit_cat(device):
     x2 = torch.randn(1, 32, 8, 8, 16, device=device).contiguous(memory_format=CL)
     want = up.conv(torch.cat([x2, up.up(x1)], dim=1))
     assert torch.equal(up(x1, x2), want)
+
+
+def test_train_step_as_a_hip_graph_replays_to_the_eager_result(device):
+    """The whole step (forward, fused loss, backward, clipping, Adam) captured once and replayed: every replay, with
+    eager work and synchronisations between replays, must give the loss the eager step gives from the same state."""
+    def make():
+        _, ours, x, lab = _two_arms(device, torch.bfloat16, shard=True)
+        opt = torch.optim.Adam(ours.parameters(), lr=1e-3, fused=True, capturable=True)
+        xd, labd = x.to(device).contiguous(memory_format=CL), lab.to(device)
+
+        def step():
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                logits = ours(xd)
+            loss = sa.ce_dice_loss(logits, labd)
+            loss.backward()
+            torch.nn.utils.clip_grad_norm_(ours.parameters(), 1.0)
+            opt.step()
+            opt.zero_grad(set_to_none=False)
+            return loss.detach()
+        return ours, opt, step
+
+    _, _, eager = make()
+    want = [eager().item() for _ in range(4)]
+    model, opt, step = make()
+    init = {k: v.clone() for k, v in model.state_dict().items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    model.load_state_dict(init)
+    for st in opt.state.values():
+        for v in st.values():
+            if torch.is_tensor(v):
+                v.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = step()
+    got = []
+    for _ in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        got.append(static_loss.item())
+        torch.randn(1 << 16, device=device).sum().item()
+    assert got == want
+    assert want[0] != want[1]
