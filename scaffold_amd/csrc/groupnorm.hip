@@ -34,6 +34,7 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kShiftRows = 32;   // voxels that define the shift K
 constexpr int kMaxSplit = 2048;  // workgroups per sample
+constexpr int kFillWorkgroups = 512;   // workgroups a launch aims for when the sample is small
 
 struct GnPlan {
   bool vector;
@@ -58,7 +59,12 @@ GnPlan make_plan(const sfh_groupnorm_desc& p, int x_dtype, bool aligned) {
   pl.tpr = p.c / pl.vec;
   pl.rpp = kBlock / pl.tpr;
   pl.slots = cg >= pl.vec ? 1 : pl.vec / cg;
-  int64_t rows = (int64_t)pl.rpp * 16;  // 16 passes of 4 KiB per workgroup
+  // 16 passes of 4 KiB per workgroup on large samples; fewer on small ones, so that a launch still has about
+  // kFillWorkgroups workgroups and no workgroup walks a long serial chain of dependent loads.
+  const int64_t want = cdiv((int64_t)kFillWorkgroups, std::max(1, p.n));
+  int64_t passes = p.spatial / ((int64_t)pl.rpp * want);
+  passes = std::min<int64_t>(16, std::max<int64_t>(1, passes));
+  int64_t rows = (int64_t)pl.rpp * passes;
   if (cdiv(p.spatial, rows) > kMaxSplit) rows = cdiv(cdiv(p.spatial, kMaxSplit), pl.rpp) * pl.rpp;
   pl.rows_per_split = rows;
   pl.nsplit = (int)cdiv(p.spatial, rows);
@@ -388,18 +394,29 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_finalize(const float* __restric
   const int cg = C / G;
   if (b < N * G) {
     const int n = b / G, g = b - n * G;
+    // One flat index over (split, channel of the group): neighbouring threads read neighbouring channels and every
+    // thread's loads are independent of one another.
     float s1 = 0.f, s2 = 0.f;
-    for (int cc = 0; cc < cg; ++cc) {
-      const int c = g * cg + cc;
-      const float w = load_param(gamma, param_dtype, c, 1.f);
-      float t1 = 0.f, t2 = 0.f;
-      for (int sp = threadIdx.x; sp < nsplit; sp += kBlock) {
-        const float* p = part + ((int64_t)n * nsplit + sp) * 2 * C;
-        t1 += p[c];
-        t2 += p[C + c];
+    const float* base = part + (int64_t)n * nsplit * 2 * C + g * cg;
+    const int total = nsplit * cg;
+    constexpr int U = 8;  // loads in flight per thread
+    for (int i0 = threadIdx.x; i0 < total; i0 += U * kBlock) {
+      float a1[U], a2[U], w[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = i0 + k * kBlock;
+        const int ic = i < total ? i : total - 1;
+        const int sp = ic / cg, cc = ic - sp * cg;
+        const float* p = base + (int64_t)sp * 2 * C + cc;
+        a1[k] = p[0];
+        a2[k] = p[C];
+        w[k] = i < total ? load_param(gamma, param_dtype, g * cg + cc, 1.f) : 0.f;
       }
-      s1 = fmaf(w, t1, s1);
-      s2 = fmaf(w, t2, s2);
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        s1 = fmaf(w[k], a1[k], s1);
+        s2 = fmaf(w[k], a2[k], s2);
+      }
     }
     s1 = block_sum256(s1, red4);
     s2 = block_sum256(s2, red4);
