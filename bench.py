@@ -192,9 +192,9 @@ def bench_unet_step(args, device):
     occ = (torch.rand((1, 1, 64, 128, 128), generator=g) < 0.05).float().contiguous(memory_format=CL).to(device)
     lab = torch.randint(0, 11, (1, 64, 128, 128), generator=g).to(device)
 
-    def make():
+    def make(shard_halo=True):
         torch.manual_seed(5001)
-        model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
+        model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(shard_halo)
         opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=True)
         return model, opt
 
@@ -206,7 +206,7 @@ def bench_unet_step(args, device):
             loss.backward()
             torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
             opt.step()
-            opt.zero_grad(set_to_none=False)
+            opt.zero_grad(set_to_none=True)  # ScaFFold/utils/trainer.py:694
             return loss
         return step
 
@@ -214,6 +214,12 @@ def bench_unet_step(args, device):
     step = step_fn(model, opt)
     ms = event_time_ms(step, 10, warmup=3)
     out = {"ms_per_step": ms, "input": "1x1x64x128x128 occupancy (5% ones), zero depth halo, padding (0,1,1)"}
+    # The same arithmetic without the halo emulation's copies (depth padding 1 inside the kernels; bitwise the same
+    # result): what remains is the cost of the step itself, the difference is the bench's stand-in for DistConv's
+    # halo exchange.
+    model_p, opt_p = make(shard_halo=False)
+    out["ms_per_step_padded_form"] = event_time_ms(step_fn(model_p, opt_p), 10, warmup=3)
+    del model_p, opt_p
 
     # The same step as one HIP graph. Checked before it is reported: from identical initial state, the losses of
     # four graph replays (with eager work and synchronisations between them) must equal those of four eager steps.

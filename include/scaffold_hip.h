@@ -173,6 +173,21 @@ int sfh_ce_dice_bwd(const sfh_loss_desc* p, int dtype, const void* logits, const
                     const float* class_weight, const float* stats, const float* grad_loss,
                     void* dlogits, void* stream);
 
+/* ---- 2x2x2 max pooling --------------------------------------------------------------------
+ * The down-sampling step between U-Net levels, nn.MaxPool3d(2) in the reference
+ * (ScaFFold/unet/unet_parts.py:165), on dense channels-last tensors: x (N, D, H, W, C),
+ * y (N, D/2, H/2, W/2, C) of `dtype`. Stock semantics: odd trailing planes are dropped, ties go to
+ * the first voxel of the cell in depth-major order, a NaN wins over any number. `idx` gets one
+ * byte per output element (which of the eight voxels, kd*4 + kh*2 + kw) and is what the backward
+ * needs besides grad_y; the backward writes every element of grad_x. */
+typedef struct sfh_pool_desc {
+  int32_t n, c, in_d, in_h, in_w;
+} sfh_pool_desc;
+int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, uint8_t* idx,
+                     void* stream);
+int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
+                     void* grad_x, void* stream);
+
 /* ---- measurement helper --------------------------------------------------------------
  * A plain streaming copy of `bytes` bytes (multiple of 16) used to calibrate achieved HBM
  * bandwidth and the scale of the FETCH_SIZE / WRITE_SIZE counters. Has no counterpart in the

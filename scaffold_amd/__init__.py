@@ -27,6 +27,8 @@ _EXPORTS = {
     "group_norm": "groupnorm", "triton_group_norm": "groupnorm", "MATCH_STOCK_DTYPE": "groupnorm",
     # loss head
     "ce_dice_loss": "losses", "is_supported_loss": "losses",
+    # pooling
+    "max_pool3d_2x": "pooling", "is_supported_pool": "pooling", "FastMaxPool3d": "pooling",
     # modules / model
     "FastConv3d": "modules", "FastConvTranspose3d": "modules", "FastGroupNorm": "modules",
     "UNet": "unet",

@@ -29,6 +29,7 @@ __all__ = [
     "ConvTDesc",
     "GroupNormDesc",
     "LossDesc",
+    "PoolDesc",
     "dtype_code",
     "SUPPORTED_DTYPES",
     "EXPORTED_SYMBOLS",
@@ -61,6 +62,10 @@ class ConvTDesc(ctypes.Structure):
 
 class LossDesc(ctypes.Structure):
     _fields_ = [("n", c_int32), ("classes", c_int32), ("spatial", c_int64), ("eps", c_float)]
+
+
+class PoolDesc(ctypes.Structure):
+    _fields_ = [(k, c_int32) for k in ("n", "c", "in_d", "in_h", "in_w")]
 
 
 class GroupNormDesc(ctypes.Structure):
@@ -102,6 +107,8 @@ _SIGNATURES = {
     "sfh_ce_dice_fwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                 c_void_p]),
     "sfh_ce_dice_bwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_maxpool2_fwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_maxpool2_bwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_stream_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -9,6 +9,7 @@
 #include "conv_thin.hpp"
 #include "loss.hpp"
 #include "reduce.hpp"
+#include "pool.hpp"
 #include "wgrad_mfma.hpp"
 
 namespace sfh {
@@ -446,6 +447,32 @@ extern "C" int sfh_bias_grad(int dtype, int out_dtype, const void* g, int64_t ro
   if (workspace == nullptr || workspace_bytes < need)
     return fail(SFH_ERR_WORKSPACE, "bias grad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
   return bias_grad(dtype, out_dtype, g, rows, channels, gb, workspace, (hipStream_t)stream);
+}
+
+// ---- 2x2x2 max pooling -----------------------------------------------------------------
+static int check_pool(const sfh_pool_desc* p, int dtype, const char* what) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "%s: null descriptor", what);
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "%s: bad dtype %d", what, dtype);
+  if (p->n < 0 || p->c < 1 || p->in_d < 1 || p->in_h < 1 || p->in_w < 1)
+    return fail(SFH_ERR_INVALID, "%s: bad extents n=%d c=%d in=(%d,%d,%d)", what, p->n, p->c, p->in_d, p->in_h, p->in_w);
+  return SFH_OK;
+}
+
+extern "C" int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, uint8_t* idx, void* stream) {
+  if (int rc = check_pool(p, dtype, "maxpool fwd")) return rc;
+  if (p->n == 0 || p->in_d < 2 || p->in_h < 2 || p->in_w < 2) return SFH_OK;  // empty output
+  if (x == nullptr || y == nullptr || idx == nullptr) return fail(SFH_ERR_INVALID, "maxpool fwd: null tensor");
+  return maxpool2_fwd(*p, dtype, x, y, idx, (hipStream_t)stream);
+}
+
+extern "C" int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx, void* grad_x,
+                                void* stream) {
+  if (int rc = check_pool(p, dtype, "maxpool bwd")) return rc;
+  if (p->n == 0) return SFH_OK;
+  const bool empty_out = p->in_d < 2 || p->in_h < 2 || p->in_w < 2;
+  if (grad_x == nullptr || (!empty_out && (grad_y == nullptr || idx == nullptr)))
+    return fail(SFH_ERR_INVALID, "maxpool bwd: null tensor");
+  return maxpool2_bwd(*p, dtype, grad_y, idx, grad_x, (hipStream_t)stream);
 }
 
 // ---- transposed convolution ------------------------------------------------------------

@@ -1,0 +1,14 @@
+// 2x2x2, stride-2 max pooling of channels-last volumes (the U-Net's down-sampling step) and its gradient.
+#pragma once
+#include "common.hpp"
+
+namespace sfh {
+
+// y[n][od][oh][ow][c] = max over the 2x2x2 cell; idx holds, per output element, which of the cell's eight voxels
+// (kd * 4 + kh * 2 + kw) supplied it. Odd trailing planes, rows and columns are dropped.
+int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st);
+
+// gx = gy routed to the voxel idx names, zero elsewhere (including dropped odd planes). Writes all of gx.
+int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, void* gx, hipStream_t st);
+
+}  // namespace sfh

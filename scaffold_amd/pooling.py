@@ -1,0 +1,91 @@
+"""``MaxPool3d(2)`` on channels-last volumes: the down-sampling step of the U-Net's ``Down`` block.
+
+The reference calls the stock module there (``ScaFFold/unet/unet_parts.py:165``).  This op keeps its
+semantics (floor mode, ties to the first voxel of the cell, NaN wins) and its result bit for bit, but reads the
+NDHWC tensor where it lies, keeps one byte per output element for the backward instead of an int64 index, and
+writes the input gradient in one pass.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+import torch.nn as nn
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+from ._lib import PoolDesc
+
+__all__ = ["max_pool3d_2x", "is_supported_pool", "FastMaxPool3d"]
+
+_CL3D = torch.channels_last_3d
+
+
+def is_supported_pool(x) -> bool:
+    """Total gate: never raises."""
+    try:
+        return (isinstance(x, torch.Tensor) and x.dim() == 5 and x.is_cuda and x.dtype in _lib.SUPPORTED_DTYPES
+                and x.shape[1] >= 1 and min(x.shape[2:]) >= 1)
+    except Exception:
+        return False
+
+
+class _MaxPool2Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        x = x.contiguous(memory_format=_CL3D)
+        n, c, d, h, w = (int(v) for v in x.shape)
+        y = torch.empty((n, c, d // 2, h // 2, w // 2), dtype=x.dtype, device=x.device, memory_format=_CL3D)
+        idx = torch.empty((n, d // 2, h // 2, w // 2, c), dtype=torch.uint8, device=x.device)
+        desc = PoolDesc(n, c, d, h, w)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().sfh_maxpool2_fwd(ctypes.byref(desc), _lib.dtype_code(x.dtype), _lib.ptr(x), _lib.ptr(y), _lib.ptr(idx),
+                                             _lib.stream_ptr(x.device))
+        _lib.check(rc, "max_pool3d_2x")
+        ctx.save_for_backward(idx)
+        ctx.pool_shape = (n, c, d, h, w)
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_y):
+        (idx,) = ctx.saved_tensors
+        n, c, d, h, w = ctx.pool_shape
+        gy = grad_y.contiguous(memory_format=_CL3D)
+        gx = torch.empty((n, c, d, h, w), dtype=gy.dtype, device=gy.device, memory_format=_CL3D)
+        desc = PoolDesc(n, c, d, h, w)
+        with torch.cuda.device(gy.device):
+            rc = _lib.lib().sfh_maxpool2_bwd(ctypes.byref(desc), _lib.dtype_code(gy.dtype), _lib.ptr(gy), _lib.ptr(idx), _lib.ptr(gx),
+                                             _lib.stream_ptr(gy.device))
+        _lib.check(rc, "max_pool3d_2x backward")
+        return gx
+
+
+def max_pool3d_2x(x: torch.Tensor) -> torch.Tensor:
+    """``F.max_pool3d(x, 2)`` for a 5-D GPU tensor; the result is channels-last."""
+    if not is_supported_pool(x):
+        raise NotImplementedError(f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)}")
+    return _MaxPool2Fn.apply(x)
+
+
+def _all_equal(v, want) -> bool:
+    if isinstance(v, (tuple, list)):
+        return len(v) == 3 and all(int(e) == want for e in v)
+    return int(v) == want
+
+
+class FastMaxPool3d(nn.MaxPool3d):
+    """``nn.MaxPool3d`` whose forward runs the HIP kernel. Only the configuration the U-Net uses exists:
+    ``kernel_size == stride == 2``, no padding, no dilation, floor mode, no returned indices; anything else
+    raises ``NotImplementedError`` at call time."""
+
+    def forward(self, input):
+        stride = self.kernel_size if self.stride is None else self.stride
+        if not (_all_equal(self.kernel_size, 2) and _all_equal(stride, 2) and _all_equal(self.padding, 0)
+                and _all_equal(self.dilation, 1) and not self.ceil_mode and not self.return_indices):
+            raise NotImplementedError(
+                f"FastMaxPool3d supports MaxPool3d(2) only, got kernel_size={self.kernel_size} stride={self.stride} "
+                f"padding={self.padding} dilation={self.dilation} ceil_mode={self.ceil_mode} "
+                f"return_indices={self.return_indices}")
+        return max_pool3d_2x(input)

@@ -21,6 +21,7 @@ import torch.nn.functional as F
 import torch.utils.checkpoint
 
 from .modules import FastConv3d, FastConvTranspose3d, FastGroupNorm, autocast_dtype
+from .pooling import FastMaxPool3d
 
 __all__ = ["UNet", "DoubleConv", "Down", "Up", "OutConv", "skip_concat"]
 
@@ -48,6 +49,10 @@ def _conv3d(stock, cin, cout, **kw):
 
 def _conv_transpose3d(stock, cin, cout, **kw):
     return (nn.ConvTranspose3d if stock else FastConvTranspose3d)(cin, cout, **kw)
+
+
+def _max_pool(stock):
+    return (nn.MaxPool3d if stock else FastMaxPool3d)(2)
 
 
 def _group_norm(stock, groups, channels, activation=None):
@@ -93,7 +98,7 @@ class DoubleConv(nn.Module):
 class Down(nn.Module):
     def __init__(self, in_channels, out_channels, group_norm_groups, stock=False):
         super().__init__()
-        self.maxpool_conv = nn.Sequential(nn.MaxPool3d(2), DoubleConv(in_channels, out_channels, group_norm_groups, stock=stock))
+        self.maxpool_conv = nn.Sequential(_max_pool(stock), DoubleConv(in_channels, out_channels, group_norm_groups, stock=stock))
 
     def forward(self, x):
         return self.maxpool_conv(x)

@@ -222,7 +222,7 @@ def test_train_step_as_a_hip_graph_replays_to_the_eager_result(device):
             loss.backward()
             torch.nn.utils.clip_grad_norm_(ours.parameters(), 1.0)
             opt.step()
-            opt.zero_grad(set_to_none=False)
+            opt.zero_grad(set_to_none=True)
             return loss.detach()
         return ours, opt, step
 
