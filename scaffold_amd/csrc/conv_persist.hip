@@ -29,6 +29,7 @@ namespace {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t sfh_u32x2_t __attribute__((ext_vector_type(2)));
 
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
@@ -109,74 +110,138 @@ constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) 
 // origin: offsets of real voxels are below it, kRange itself (and anything above) reads as zero.
 constexpr int kRange = 0x40000000;
 
-// What a wavefront streams into the other brick buffer during a step: for each of its 64-voxel
-// groups the per-lane buffer offset (out of range = zero fill), or -1 in lanes past the brick's end.
-template <typename C>
-struct BrickFetch {
-  int voff[C::GPW];
-};
-
-// Output of the previous brick, already rounded, waiting to be stored during the next step.
-template <typename C>
-struct PendingStore {
-  uint2 data[C::MS][4];
-  int64_t off[C::MS];  // element offset of the lane's voxel row in y, or -1
-};
-
-// Streams a whole brick at once (used for the first brick of a workgroup).
+// Streams a whole brick at once (used for the first brick of a workgroup). voff: per 64-voxel group the lane's
+// buffer offset (out of range = zero fill), or -1 in lanes past the brick's end.
 template <typename T, typename C>
-__device__ __forceinline__ void fetch_brick(char* dst, int wave, const T* origin, const BrickFetch<C>& bf) {
+__device__ __forceinline__ void fetch_brick(char* dst, int wave, const T* origin, const int (&voff)[C::GPW]) {
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(origin), 0, kRange, 0x00020000);
 #pragma unroll
   for (int k = 0; k < C::GPW; ++k)
-    if (bf.voff[k] != -1) {
+    if (voff[k] != -1) {
 #pragma unroll
       for (int p = 0; p < 4; ++p)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + (wave + 4 * k) * 1024 + p * C::PLANE),
-                                                 16, bf.voff[k] + p * 16, 0, 0, 0);
+                                                 16, voff[k] + p * 16, 0, 0, 0);
     }
 }
 
-// One step: MFMAs over the brick in `cur`; interleaved with them, one instruction at a time so that
-// neither the memory pipe nor the matrix pipe sees a burst: the direct-to-LDS loads of the next brick
-// (even iterations), the stores of the previous brick's output (odd iterations) and, when STREAM, the
-// weight fragments of the next chunk (each right after its last use).
-template <typename T, typename C, bool STREAM>
-__device__ __forceinline__ void persist_step(const char* cur, char* nxt, int wave, const int (&lbase)[C::MS], uint4 (&wq)[C::NIT],
-                                             f32x16_t (&acc)[C::MS], const T* wnext, const T* origin, const BrickFetch<C>& bf,
-                                             const PendingStore<C>& ps, bool have_store, T* __restrict__ y) {
-  constexpr int FRAG = 512;
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(origin), 0, kRange, 0x00020000);
+// Launch-constant geometry of a lane, and what it needs to know about the input.
+template <typename C>
+struct LaneGeom {
+  int lbase[C::MS];   // LDS byte offset of the lane's A-fragment voxel, per sub-tile
+  int gcoord[C::GPW]; // staging: packed brick coordinates of the lane's voxel per group, -1 past the brick
+  int grel[C::GPW];   // staging: byte offset of that voxel from the brick origin in the input
+  int vcoord[C::MS];  // output: packed tile coordinates of the lane's voxel per sub-tile
+  int vrel[C::MS];    // output: byte offset of the lane's first channel from the tile origin in y
+};
+
+// Offsets of the brick of tile `tc` for this lane's groups; returns the (possibly virtual) brick origin. Lanes whose
+// voxel lies outside the input use an out-of-range offset and receive zeros; `live` false turns the whole brick
+// into such lanes (the step after the last has nothing to fetch).
+template <typename T, typename C>
+__device__ __forceinline__ const T* brick_origin(const MfmaConvArgs& a, const T* x, const TileCoord& tc) {
+  const int id0 = tc.d * C::TD - a.pd, ih0 = tc.h * C::TH - a.ph, iw0 = tc.w * C::TW - a.pw;
+  return x + ((((int64_t)tc.n * a.id + id0) * a.ih + ih0) * a.iw + iw0) * a.cred;
+}
+template <typename C>
+__device__ __forceinline__ int brick_group_offset(const MfmaConvArgs& a, const TileCoord& tc, bool live, int gcoord, int grel) {
+  const int id0 = tc.d * C::TD - a.pd, ih0 = tc.h * C::TH - a.ph, iw0 = tc.w * C::TW - a.pw;
+  const int bd = gcoord & 0xff, bh = (gcoord >> 8) & 0xff, bw = (gcoord >> 16) & 0xff;
+  const int inside = ((unsigned)(id0 + bd) < (unsigned)a.id) & ((unsigned)(ih0 + bh) < (unsigned)a.ih) &
+                     ((unsigned)(iw0 + bw) < (unsigned)a.iw) & (int)live;
+  return gcoord < 0 ? -1 : (inside ? grel : kRange);
+}
+// Byte offset of the lane's output piece of sub-tile voxel `vcoord` from the tile origin, or out of range when the
+// voxel lies past the ragged edge of the output (such stores are dropped by the buffer bounds check).
+template <typename C>
+__device__ __forceinline__ int store_offset(const MfmaConvArgs& a, const TileCoord& tc, int vcoord, int vrel) {
+  const int td = vcoord & 0xff, th = (vcoord >> 8) & 0xff, tw = vcoord >> 16;
+  const int ok = (tc.d * C::TD + td < a.od) & (tc.h * C::TH + th < a.oh) & (tc.w * C::TW + tw < a.ow);
+  return ok ? vrel : kRange;
+}
+template <typename T, typename C>
+__device__ __forceinline__ T* tile_origin(const MfmaConvArgs& a, T* y, const TileCoord& tc, int nb) {
+  return y + ((((int64_t)tc.n * a.od + tc.d * C::TD) * a.oh + tc.h * C::TH) * a.ow + tc.w * C::TW) * a.cout + nb * 32;
+}
+
+// Output of a finished brick, rounded, waiting to be stored during the next step. Accumulator register 4g+t of a
+// lane is output channel 8g + 4*kg + t of voxel j of the sub-tile: the two k-half lanes of a voxel write adjacent
+// 8-byte halves of a 16-byte piece.
+template <typename C>
+struct PendingStore {
+  sfh_u32x2_t data[C::MS][4];
+};
+
+template <typename T, typename C, bool BIAS>
+__device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const float (&bias)[16], PendingStore<C>& ps) {
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float v[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) v[t] = BIAS ? acc[ms][4 * g + t] + bias[4 * g + t] : acc[ms][4 * g + t];
+      ps.data[ms][g][0] = Mma<T>::pack2(v[0], v[1]);
+      ps.data[ms][g][1] = Mma<T>::pack2(v[2], v[3]);
+    }
+}
+
+// One step = one output brick. While the 54 x MS MFMAs run over the brick in `cur`, the wavefront also issues, a
+// little in every iteration so that the matrix pipe never waits behind a block of other work:
+//   * the direct-to-LDS loads of the next brick into `nxt` (even iterations),
+//   * the stores of the PREVIOUS brick's rounded result (odd ones); lanes past a ragged edge carry an out-of-range
+//     offset and the buffer bounds check drops their store, so there is no branch,
+//   * the fetch offsets of the brick after the next and the store offsets of this brick (late odd iterations),
+//     written over the ones this step has finished using.
+template <typename T, typename C>
+__device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* cur, char* nxt, int wave, const LaneGeom<C>& lg,
+                                             const uint4 (&wq)[C::NIT], f32x16_t (&acc)[C::MS], const PendingStore<C>& ps,
+                                             const T* fetch_origin, int (&voff)[C::GPW],
+                                             __amdgpu_buffer_rsrc_t done_rsrc, int (&done_off)[C::MS],
+                                             const TileCoord& plan_tc, bool plan_live, const TileCoord& tc) {
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(fetch_origin), 0, kRange, 0x00020000);
   constexpr int NLOAD = C::GPW * 4;
   constexpr int NSTORE = C::MS * 4;
-  static_assert(2 * NLOAD <= C::NIT && 2 * NSTORE <= C::NIT, "one memory instruction per iteration");
+  constexpr int PLAN0 = 2 * NSTORE + 1;             // first (odd) iteration that plans a group
+  constexpr int OFF0 = PLAN0 + 2 * C::GPW;          // first (odd) iteration that computes a store offset
+  static_assert(2 * NLOAD <= C::NIT && OFF0 + 2 * C::MS <= C::NIT + 1, "one piece of side work per iteration");
   // activation fragments are requested ADEPTH iterations ahead of the MFMAs that consume them
   constexpr int ADEPTH = 2;
   uint4 aq[ADEPTH + 1][C::MS];
 #pragma unroll
   for (int d = 0; d < ADEPTH; ++d)
 #pragma unroll
-    for (int ms = 0; ms < C::MS; ++ms) aq[d][ms] = *reinterpret_cast<const uint4*>(cur + lbase[ms] + lds_off<C>(d));
+    for (int ms = 0; ms < C::MS; ++ms) aq[d][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(d));
 #pragma unroll
   for (int it = 0; it < C::NIT; ++it) {
     if (it + ADEPTH < C::NIT) {
 #pragma unroll
       for (int ms = 0; ms < C::MS; ++ms)
-        aq[(it + ADEPTH) % (ADEPTH + 1)][ms] = *reinterpret_cast<const uint4*>(cur + lbase[ms] + lds_off<C>(it + ADEPTH));
+        aq[(it + ADEPTH) % (ADEPTH + 1)][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(it + ADEPTH));
     }
     if (it % 2 == 0 && it / 2 < NLOAD) {
       const int k = (it / 2) / 4, p = (it / 2) % 4;
-      if (bf.voff[k] != -1)
+      // only the last group of a wavefront can have lanes past the end of the brick
+      const bool full = (3 + 4 * k) * 64 + 63 < C::BV;
+      if (full || voff[k] != -1)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(nxt + (wave + 4 * k) * 1024 + p * C::PLANE),
-                                                 16, bf.voff[k] + p * 16, 0, 0, 0);
+                                                 16, voff[k] + p * 16, 0, 0, 0);
     }
     if (it % 2 == 1 && it / 2 < NSTORE) {
       const int ms = (it / 2) / 4, g = (it / 2) % 4;
-      if (have_store && ps.off[ms] >= 0) *reinterpret_cast<uint2*>(y + ps.off[ms] + 8 * g) = ps.data[ms][g];
+      __builtin_amdgcn_raw_buffer_store_b64(ps.data[ms][g], done_rsrc, done_off[ms] + 16 * g, 0, 0);
+    }
+    if (it % 2 == 1 && it >= PLAN0 && (it - PLAN0) / 2 < C::GPW) {
+      const int k = (it - PLAN0) / 2;
+      voff[k] = brick_group_offset<C>(a, plan_tc, plan_live, lg.gcoord[k], lg.grel[k]);  // group k's loads are all issued
+    }
+    if (it % 2 == 1 && it >= OFF0 && (it - OFF0) / 2 < C::MS) {
+      const int ms = (it - OFF0) / 2;
+      done_off[ms] = store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]);  // the previous brick's pieces are all stored
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (it == 0 && !STREAM) {
-      // a single-chunk brick starts from zero: the first MFMA takes a zero addend instead of a clearing pass
+    if (it == 0) {
+      // a brick starts from zero: the first MFMA takes a zero addend instead of a clearing pass
       f32x16_t zero;
 #pragma unroll
       for (int r = 0; r < 16; ++r) zero[r] = 0.f;
@@ -186,14 +251,13 @@ __device__ __forceinline__ void persist_step(const char* cur, char* nxt, int wav
 #pragma unroll
       for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
     }
-    if (STREAM) wq[it] = *reinterpret_cast<const uint4*>(wnext + it * FRAG);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
 
-template <typename T, typename C, bool STREAM>
+template <typename T, typename C, bool BIAS>
 __global__ void __launch_bounds__(256, 1)
-conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
+conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias_ptr,
                     T* __restrict__ y, PersistGeom gm) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space builtins the host pass cannot type-check
   __shared__ __attribute__((aligned(16))) char buf0[C::BRICK];
@@ -209,138 +273,79 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   int tile_end = tile_begin + gm.items_per_wg;
   if (tile_end > gm.ntiles) tile_end = gm.ntiles;
   if (nb >= gm.nblocks || tile_begin >= tile_end) return;
-  const int ncc = a.cred / 32;
-  const int nsteps = (tile_end - tile_begin) * ncc;
+  const int nsteps = tile_end - tile_begin;
 
-  int lbase[C::MS];
+  LaneGeom<C> lg;
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     const int v = (wave * C::MS + ms) * 32 + j;
     const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
-    lbase[ms] = kg * C::PLANE + ((td * C::BH + th) * C::BW + tw) * 16;
+    lg.lbase[ms] = kg * C::PLANE + ((td * C::BH + th) * C::BW + tw) * 16;
+    lg.vcoord[ms] = td | (th << 8) | (tw << 16);
+    lg.vrel[ms] = (((td * a.oh + th) * a.ow + tw) * a.cout + 4 * kg) * 2;
   }
-
-  // Staging role of this lane, fixed for the whole launch: wave w fills the 64-voxel groups
-  // w, w+4, ... of every plane; the lane's voxel inside the brick and its byte offset from the
-  // brick origin in the input tensor.
-  int gcoord[C::GPW], grel[C::GPW];
+  // Staging role of this lane, fixed for the whole launch: wave w fills the 64-voxel groups w, w+4, ... of every
+  // plane; the lane's voxel inside the brick and its byte offset from the brick origin in the input tensor.
 #pragma unroll
   for (int k = 0; k < C::GPW; ++k) {
     const int vox = (wave + 4 * k) * 64 + lane;
     const int bw = vox % C::BW, bh = (vox / C::BW) % C::BH, bd = vox / (C::BW * C::BH);
-    gcoord[k] = vox < C::BV ? (bd | (bh << 8) | (bw << 16)) : -1;
-    grel[k] = (((bd * a.ih + bh) * a.iw + bw) * a.cred) * 2;
+    lg.gcoord[k] = vox < C::BV ? (bd | (bh << 8) | (bw << 16)) : -1;
+    lg.grel[k] = (((bd * a.ih + bh) * a.iw + bw) * a.cred) * 2;
   }
 
   constexpr int FRAG = 512;
-  const int64_t slab = (int64_t)C::NIT * FRAG;  // elements per (output block, chunk) weight slab
-  const T* wblock = wp + (int64_t)nb * ncc * slab + lane * 8;
-
+  const T* wblock = wp + (int64_t)nb * C::NIT * FRAG + lane * 8;
   uint4 wq[C::NIT];
 #pragma unroll
   for (int it = 0; it < C::NIT; ++it) wq[it] = *reinterpret_cast<const uint4*>(wblock + it * FRAG);
-
-  // Buffer descriptor and per-lane offsets of the brick of (tile, chunk). The descriptor is based at the
-  // (possibly virtual) voxel at the brick origin; lanes whose voxel lies outside the input never
-  // dereference it: they use an out-of-range offset and receive zeros.
-  auto plan_brick = [&](const TileCoord& tc, int cc, BrickFetch<C>& bf) -> const T* {
-    const int tw_i = tc.w, th_i = tc.h, td_i = tc.d, n = tc.n;
-    const int id0 = td_i * C::TD - a.pd, ih0 = th_i * C::TH - a.ph, iw0 = tw_i * C::TW - a.pw;
-    const T* origin = x + ((((int64_t)n * a.id + id0) * a.ih + ih0) * a.iw + iw0) * a.cred + cc * 32;
+  float bias[16];
 #pragma unroll
-    for (int k = 0; k < C::GPW; ++k) {
-      const int bd = gcoord[k] & 0xff, bh = (gcoord[k] >> 8) & 0xff, bw = (gcoord[k] >> 16) & 0xff;
-      const bool inside = (unsigned)(id0 + bd) < (unsigned)a.id && (unsigned)(ih0 + bh) < (unsigned)a.ih &&
-                          (unsigned)(iw0 + bw) < (unsigned)a.iw;
-      bf.voff[k] = gcoord[k] < 0 ? -1 : (inside ? grel[k] : kRange);
-    }
-    return origin;
-  };
+  for (int r = 0; r < 16; ++r) bias[r] = BIAS ? to_float(bias_ptr[nb * 32 + 8 * (r / 4) + 4 * kg + (r % 4)]) : 0.f;
 
-  BrickFetch<C> bf;
+  // Bricks in flight: `tc` is computed in this step, `tc1` is fetched during it, `tc2` is planned during it.
   TileCoord tc = decode_tile(tile_begin, gm);
-  const T* origin = plan_brick(tc, 0, bf);
-  fetch_brick<T, C>(buf0, wave, origin, bf);
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's part of the brick has landed
-  __syncthreads();
-
-  // Output position of this lane's voxel of every sub-tile relative to the brick origin: coordinates (for the
-  // ragged-edge test) and element offset, fixed for the whole launch.
-  int vcoord[C::MS], vrel[C::MS];
+  int voff[C::GPW];
 #pragma unroll
-  for (int ms = 0; ms < C::MS; ++ms) {
-    const int v = (wave * C::MS + ms) * 32 + j;
-    const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
-    vcoord[ms] = td | (th << 8) | (tw << 16);
-    vrel[ms] = ((td * a.oh + th) * a.ow + tw) * a.cout + 4 * kg;
-  }
+  for (int k = 0; k < C::GPW; ++k) voff[k] = brick_group_offset<C>(a, tc, true, lg.gcoord[k], lg.grel[k]);
+  fetch_brick<T, C>(buf0, wave, brick_origin<T, C>(a, x, tc), voff);
+  TileCoord tc1 = next_tile(tc, gm);
+#pragma unroll
+  for (int k = 0; k < C::GPW; ++k) voff[k] = brick_group_offset<C>(a, tc1, nsteps > 1, lg.gcoord[k], lg.grel[k]);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's part of the first brick has landed
+  __syncthreads();
 
   f32x16_t acc[C::MS];
   PendingStore<C> ps;
 #pragma unroll
-  for (int ms = 0; ms < C::MS; ++ms) ps.off[ms] = -1;
-  bool have_store = false;
-  int cc = 0;
+  for (int ms = 0; ms < C::MS; ++ms)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) ps.data[ms][g] = sfh_u32x2_t{0u, 0u};
+  int done_off[C::MS];
+#pragma unroll
+  for (int ms = 0; ms < C::MS; ++ms) done_off[ms] = kRange;  // nothing to store during the first step
+  T* done_origin = y;
+
   for (int step = 0; step < nsteps; ++step) {
-    TileCoord ntc = tc;
-    int ncc_next = cc + 1;
-    if (ncc_next == ncc) { ncc_next = 0; ntc = next_tile(tc, gm); }
-    const bool has_next = step + 1 < nsteps;
-    // On the last step the current brick is fetched once more (into the idle buffer) rather than
-    // branching around every interleaved load.
-    origin = plan_brick(has_next ? ntc : tc, has_next ? ncc_next : cc, bf);
-    // slab to stream into the weight registers during this step (the current one again at the end)
-    const T* wnext = wblock + (int64_t)(has_next ? ncc_next : cc) * slab;
-
-    if (STREAM && cc == 0) {
-#pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[ms][r] = 0.f;
-    }
-
-    if (step & 1) persist_step<T, C, STREAM>(buf1, buf0, wave, lbase, wq, acc, wnext, origin, bf, ps, have_store, y);
-    else persist_step<T, C, STREAM>(buf0, buf1, wave, lbase, wq, acc, wnext, origin, bf, ps, have_store, y);
-    have_store = false;
-
-    if (cc == ncc - 1) {
-      // Round the finished brick now; its stores ride along with the next step's MFMAs. Accumulator
-      // register 4g+t of a lane is output channel 8g + 4*kg + t of voxel j of the sub-tile: the two
-      // k-half lanes of a voxel write adjacent 8-byte halves of a 16-byte piece.
-      const int od0 = tc.d * C::TD, oh0 = tc.h * C::TH, ow0 = tc.w * C::TW;
-      const int64_t tile_off = ((((int64_t)tc.n * a.od + od0) * a.oh + oh0) * a.ow + ow0) * a.cout + nb * 32;  // wave-uniform
-#pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms) {
-        const int td = vcoord[ms] & 0xff, th = (vcoord[ms] >> 8) & 0xff, tw = vcoord[ms] >> 16;
-        const bool ok = od0 + td < a.od && oh0 + th < a.oh && ow0 + tw < a.ow;
-        ps.off[ms] = ok ? tile_off + vrel[ms] : -1;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          if (bias != nullptr) {
-            const T* bp = bias + nb * 32 + 8 * g + 4 * kg;
-            ps.data[ms][g].x = Mma<T>::pack2(acc[ms][4 * g] + to_float(bp[0]), acc[ms][4 * g + 1] + to_float(bp[1]));
-            ps.data[ms][g].y = Mma<T>::pack2(acc[ms][4 * g + 2] + to_float(bp[2]), acc[ms][4 * g + 3] + to_float(bp[3]));
-          } else {
-            ps.data[ms][g].x = Mma<T>::pack2(acc[ms][4 * g], acc[ms][4 * g + 1]);
-            ps.data[ms][g].y = Mma<T>::pack2(acc[ms][4 * g + 2], acc[ms][4 * g + 3]);
-          }
-        }
-      }
-      have_store = true;
-    }
-
+    const TileCoord tc2 = next_tile(tc1, gm);
+    const bool live2 = step + 2 < nsteps;
+    const T* fetch_origin = brick_origin<T, C>(a, x, tc1);
+    const __amdgpu_buffer_rsrc_t done_rsrc = __builtin_amdgcn_make_buffer_rsrc(done_origin, 0, kRange, 0x00020000);
+    if (step & 1) persist_step<T, C>(a, buf1, buf0, wave, lg, wq, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
+    else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
+    round_brick<T, C, BIAS>(acc, bias, ps);  // its stores ride along with the next step's MFMAs
+    done_origin = tile_origin<T, C>(a, y, tc, nb);
+    tc = tc1;
+    tc1 = tc2;
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's part of the next brick has landed
     __syncthreads();                            // ... and every wave is done reading the current one
-    tc = ntc;
-    cc = ncc_next;
   }
-  if (have_store) {
+  // the last brick's result
+  const __amdgpu_buffer_rsrc_t done_rsrc = __builtin_amdgcn_make_buffer_rsrc(done_origin, 0, kRange, 0x00020000);
 #pragma unroll
-    for (int ms = 0; ms < C::MS; ++ms)
+  for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        if (ps.off[ms] >= 0) *reinterpret_cast<uint2*>(y + ps.off[ms] + 8 * g) = ps.data[ms][g];
-  }
+    for (int g = 0; g < 4; ++g) __builtin_amdgcn_raw_buffer_store_b64(ps.data[ms][g], done_rsrc, done_off[ms] + 16 * g, 0, 0);
 #endif
 }
 
@@ -360,11 +365,11 @@ int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const 
   gm.items_per_wg = (int)cdiv(gm.ntiles, per_block);
   gm.wgs_per_block = (int)cdiv(gm.ntiles, gm.items_per_wg);
   const unsigned grid = (unsigned)(gm.wgs_per_block * gm.nblocks);
-  if (a.cred == 32)
-    hipLaunchKernelGGL((conv_persist_kernel<T, C, false>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
+  if (bias != nullptr)
+    hipLaunchKernelGGL((conv_persist_kernel<T, C, true>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
                        (const T*)bias, (T*)y, gm);
   else
-    hipLaunchKernelGGL((conv_persist_kernel<T, C, true>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
+    hipLaunchKernelGGL((conv_persist_kernel<T, C, false>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
                        (const T*)bias, (T*)y, gm);
   return check_launch("conv_persist_kernel");
 }
@@ -382,8 +387,10 @@ int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const voi
                       void* partial, hipStream_t st) {
   // The persistent kernel pays off when the weight slab stays in registers for the whole launch, i.e. with a
   // single 32-channel reduction chunk; wider reductions run the brick-per-workgroup kernel. A brick (at most
-  // 10 x 10 input rows deep and high) must also span less than kRange bytes of the input.
-  if (a.cred != 32 || ((int64_t)10 * a.ih + 10) * a.iw * a.cred * 2 + 64 >= kRange)
+  // 10 x 10 input rows deep and high) must also span less than kRange bytes of the input, a tile (at most 8 x 8 output
+  // rows) less than kRange bytes of the output.
+  if (a.cred != 32 || ((int64_t)10 * a.ih + 10) * a.iw * a.cred * 2 + 64 >= kRange ||
+      ((int64_t)8 * a.oh + 8) * a.ow * a.cout * 2 + 64 >= kRange)
     return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st);
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st);
   return launch_typed<fp16_t>(a, x, packed, bias, y, st);
