@@ -38,6 +38,22 @@ template <> struct Mma<bf16_t> {
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 };
+// The same MFMA with the row operand held in an accumulation register (inline asm: the compiler would otherwise
+// copy such a fragment into a vector register before every use).
+typedef int sfh_i32x4_t __attribute__((ext_vector_type(4)));
+template <typename T> struct MmaAcc;
+template <> struct MmaAcc<bf16_t> {
+  static __device__ __forceinline__ void run(const sfh_i32x4_t& a, const uint4& b, f32x16_t& c) {
+    const sfh_i32x4_t bv = __builtin_bit_cast(sfh_i32x4_t, b);
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
+  }
+};
+template <> struct MmaAcc<fp16_t> {
+  static __device__ __forceinline__ void run(const sfh_i32x4_t& a, const uint4& b, f32x16_t& c) {
+    const sfh_i32x4_t bv = __builtin_bit_cast(sfh_i32x4_t, b);
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
+  }
+};
 template <> struct Mma<fp16_t> {
   static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
@@ -61,6 +77,7 @@ struct PTile {
   static constexpr int GPW = (NGROUP + 3) / 4;        // groups staged by each wavefront
   static constexpr int MS = TD * TH * TW / 128;       // 32-voxel sub-tiles per wavefront
   static constexpr int NIT = 27 * 2;                  // (tap, k-step) iterations per 32-channel chunk
+  static constexpr int NVEC = 27;                     // weight fragments kept in vector registers
   static constexpr int PIECES = BV * 4;
   static constexpr int PITER = (PIECES + 255) / 256;  // staging pieces per thread
   static_assert(TD * TH * TW == 512, "four wavefronts of four 32-voxel sub-tiles");
@@ -195,7 +212,8 @@ __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const 
 //     written over the ones this step has finished using.
 template <typename T, typename C>
 __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* cur, char* nxt, int wave, const LaneGeom<C>& lg,
-                                             const uint4 (&wq)[C::NIT], f32x16_t (&acc)[C::MS], const PendingStore<C>& ps,
+                                             const uint4 (&wq)[C::NVEC], const sfh_i32x4_t (&wa)[C::NIT - C::NVEC],
+                                             f32x16_t (&acc)[C::MS], const PendingStore<C>& ps,
                                              const T* fetch_origin, int (&voff)[C::GPW],
                                              __amdgpu_buffer_rsrc_t done_rsrc, int (&done_off)[C::MS],
                                              const TileCoord& plan_tc, bool plan_live, const TileCoord& tc) {
@@ -249,7 +267,10 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
       for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
     } else {
 #pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      for (int ms = 0; ms < C::MS; ++ms) {
+        if (it < C::NVEC) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+        else MmaAcc<T>::run(wa[it - C::NVEC], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -296,9 +317,14 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
 
   constexpr int FRAG = 512;
   const T* wblock = wp + (int64_t)nb * C::NIT * FRAG + lane * 8;
-  uint4 wq[C::NIT];
+  // The first NVEC fragments live in vector registers, the rest in accumulation registers (there are not 216 + the
+  // activation fragments' worth of vector registers; the MFMA reads its row operand from either file).
+  uint4 wq[C::NVEC];
+  sfh_i32x4_t wa[C::NIT - C::NVEC];
 #pragma unroll
-  for (int it = 0; it < C::NIT; ++it) wq[it] = *reinterpret_cast<const uint4*>(wblock + it * FRAG);
+  for (int it = 0; it < C::NVEC; ++it) wq[it] = *reinterpret_cast<const uint4*>(wblock + it * FRAG);
+#pragma unroll
+  for (int it = C::NVEC; it < C::NIT; ++it) wa[it - C::NVEC] = *reinterpret_cast<const sfh_i32x4_t*>(wblock + it * FRAG);
   float bias[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) bias[r] = BIAS ? to_float(bias_ptr[nb * 32 + 8 * (r / 4) + 4 * kg + (r % 4)]) : 0.f;
@@ -331,8 +357,9 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     const bool live2 = step + 2 < nsteps;
     const T* fetch_origin = brick_origin<T, C>(a, x, tc1);
     const __amdgpu_buffer_rsrc_t done_rsrc = __builtin_amdgcn_make_buffer_rsrc(done_origin, 0, kRange, 0x00020000);
-    if (step & 1) persist_step<T, C>(a, buf1, buf0, wave, lg, wq, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
-    else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
+    if (step & 1) persist_step<T, C>(a, buf1, buf0, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
+    else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
+    asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMAs are inline asm: the compiler does not know their result latency
     round_brick<T, C, BIAS>(acc, bias, ps);  // its stores ride along with the next step's MFMAs
     done_origin = tile_origin<T, C>(a, y, tc, nb);
     tc = tc1;
