@@ -182,7 +182,7 @@ def copy_calibration(device, mib=256, reps=4):
 
 def bench_unet_step(args, device):
     """Config 5: one Adam step of the base-32, 5-level U-Net on a 64x128x128 depth shard (zero halo),
-    bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0.
+    bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0 fused with the Adam update.
 
     Timed eagerly (how the reference's trainer runs) and, when the replay check passes, as a captured HIP graph
     of the whole step: the eager step is bound by ~600 Python-side launches, not by the GPU."""
@@ -195,7 +195,7 @@ def bench_unet_step(args, device):
     def make(shard_halo=True):
         torch.manual_seed(5001)
         model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(shard_halo)
-        opt = torch.optim.Adam(model.parameters(), lr=1e-3, fused=True, capturable=True)
+        opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0)  # clip_grad_norm_(1.0) + Adam, trainer.py:678-694
         return model, opt
 
     def step_fn(model, opt):
@@ -204,7 +204,6 @@ def bench_unet_step(args, device):
                 logits = model(occ)
             loss = sa.ce_dice_loss(logits, lab)
             loss.backward()
-            torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
             opt.step()
             opt.zero_grad(set_to_none=True)  # ScaFFold/utils/trainer.py:694
             return loss

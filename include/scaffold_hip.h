@@ -188,6 +188,32 @@ int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, 
 int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
                      void* grad_x, void* stream);
 
+/* ---- gradient clipping + Adam -----------------------------------------------------------
+ * The optimizer step of the trainer: torch.nn.utils.clip_grad_norm_(parameters, max_norm) followed by
+ * torch.optim.Adam.step() (ScaFFold/utils/trainer.py:678-694, optimizer built at trainer.py:268-274),
+ * over `ntensors` dense fp32 tensors given as HOST arrays of device pointers and element counts
+ * (every count >= 1). Pass 1 writes one fp32 slot per 8192-element chunk (sfh_adam_slots of them) and
+ * adds 1 to the device float `step`; pass 2 (which may cover a subset of the tensors, e.g. one
+ * hyperparameter group) folds all `nslots` slots in a fixed order, scales each gradient
+ * by min(1, max_norm / (norm + 1e-6)) on the fly (gradients are not modified; max_norm <= 0: no
+ * clipping) and applies Adam with torch's formulas (lerp first moment, bias corrections from
+ * `step`, denom = sqrt(v)/sqrt(1-beta2^step) + eps, weight_decay added to the gradient). `shadow`
+ * (NULL, or an array whose entries may be NULL) receives each updated parameter rounded to
+ * shadow_dtype (SFH_BF16 / SFH_FP16): the copy autocast would otherwise make in the next step.
+ * `grad_norm` (may be NULL) receives the unclipped total norm. Nothing synchronises; the pointers
+ * are passed to the kernels by value, so the two calls can be captured in a graph. */
+typedef struct sfh_adam_desc {
+  float lr, beta1, beta2, eps, weight_decay, max_norm;
+  int32_t shadow_dtype; /* SFH_BF16, SFH_FP16, or -1 for none */
+} sfh_adam_desc;
+int64_t sfh_adam_slots(int32_t ntensors, const int64_t* numel);
+int sfh_adam_grad_sumsq(int32_t ntensors, const float* const* grads, const int64_t* numel,
+                        float* slots, float* step, void* stream);
+int sfh_adam_clip_step(const sfh_adam_desc* d, int32_t ntensors, float* const* params,
+                       const float* const* grads, float* const* exp_avg, float* const* exp_avg_sq,
+                       void* const* shadow, const int64_t* numel, const float* slots,
+                       int64_t nslots, const float* step, float* grad_norm, void* stream);
+
 /* ---- measurement helper --------------------------------------------------------------
  * A plain streaming copy of `bytes` bytes (multiple of 16) used to calibrate achieved HBM
  * bandwidth and the scale of the FETCH_SIZE / WRITE_SIZE counters. Has no counterpart in the

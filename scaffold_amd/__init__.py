@@ -29,6 +29,8 @@ _EXPORTS = {
     "ce_dice_loss": "losses", "is_supported_loss": "losses",
     # pooling
     "max_pool3d_2x": "pooling", "is_supported_pool": "pooling", "FastMaxPool3d": "pooling",
+    # optimizer step
+    "FusedClipAdam": "optim",
     # modules / model
     "FastConv3d": "modules", "FastConvTranspose3d": "modules", "FastGroupNorm": "modules",
     "UNet": "unet",

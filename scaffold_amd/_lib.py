@@ -30,6 +30,7 @@ __all__ = [
     "GroupNormDesc",
     "LossDesc",
     "PoolDesc",
+    "AdamDesc",
     "dtype_code",
     "SUPPORTED_DTYPES",
     "EXPORTED_SYMBOLS",
@@ -66,6 +67,10 @@ class LossDesc(ctypes.Structure):
 
 class PoolDesc(ctypes.Structure):
     _fields_ = [(k, c_int32) for k in ("n", "c", "in_d", "in_h", "in_w")]
+
+
+class AdamDesc(ctypes.Structure):
+    _fields_ = [(k, c_float) for k in ("lr", "beta1", "beta2", "eps", "weight_decay", "max_norm")] + [("shadow_dtype", c_int32)]
 
 
 class GroupNormDesc(ctypes.Structure):
@@ -109,6 +114,10 @@ _SIGNATURES = {
     "sfh_ce_dice_bwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_fwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_bwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_adam_slots": (c_int64, [c_int32, POINTER(c_int64)]),
+    "sfh_adam_grad_sumsq": (c_int, [c_int32, POINTER(c_void_p), POINTER(c_int64), c_void_p, c_void_p, c_void_p]),
+    "sfh_adam_clip_step": (c_int, [POINTER(AdamDesc), c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                   POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "sfh_stream_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -9,6 +9,7 @@
 #include "conv_thin.hpp"
 #include "loss.hpp"
 #include "reduce.hpp"
+#include "optim.hpp"
 #include "pool.hpp"
 #include "wgrad_mfma.hpp"
 
@@ -540,6 +541,49 @@ extern "C" int sfh_ce_dice_bwd(const sfh_loss_desc* p, int dtype, const void* lo
   if (logits == nullptr || labels == nullptr || stats == nullptr || grad_loss == nullptr || dlogits == nullptr)
     return fail(SFH_ERR_INVALID, "ce_dice: null tensor");
   return loss_backward(*p, dtype, logits, labels, class_weight, stats, grad_loss, dlogits, (hipStream_t)stream);
+}
+
+// ---- gradient clipping + Adam ------------------------------------------------------------
+static int check_tensor_list(int32_t ntensors, const int64_t* numel, const char* what) {
+  if (ntensors < 1 || numel == nullptr) return fail(SFH_ERR_INVALID, "%s: need at least one tensor", what);
+  for (int i = 0; i < ntensors; ++i)
+    if (numel[i] < 1) return fail(SFH_ERR_INVALID, "%s: tensor %d has %lld elements", what, i, (long long)numel[i]);
+  return SFH_OK;
+}
+
+extern "C" int64_t sfh_adam_slots(int32_t ntensors, const int64_t* numel) {
+  if (ntensors < 1 || numel == nullptr) return 0;
+  return optim_chunks(ntensors, numel);
+}
+
+extern "C" int sfh_adam_grad_sumsq(int32_t ntensors, const float* const* grads, const int64_t* numel, float* slots, float* step,
+                                   void* stream) {
+  if (int rc = check_tensor_list(ntensors, numel, "adam sumsq")) return rc;
+  if (grads == nullptr || slots == nullptr || step == nullptr) return fail(SFH_ERR_INVALID, "adam sumsq: null argument");
+  for (int i = 0; i < ntensors; ++i)
+    if (grads[i] == nullptr) return fail(SFH_ERR_INVALID, "adam sumsq: gradient %d is null", i);
+  return optim_grad_sumsq(ntensors, grads, numel, slots, step, (hipStream_t)stream);
+}
+
+extern "C" int sfh_adam_clip_step(const sfh_adam_desc* d, int32_t ntensors, float* const* params, const float* const* grads,
+                                  float* const* exp_avg, float* const* exp_avg_sq, void* const* shadow, const int64_t* numel,
+                                  const float* slots, int64_t nslots, const float* step, float* grad_norm, void* stream) {
+  if (d == nullptr) return fail(SFH_ERR_INVALID, "adam: null descriptor");
+  if (nslots < 1 || nslots > 0x7fffffff) return fail(SFH_ERR_INVALID, "adam: bad slot count %lld", (long long)nslots);
+  if (int rc = check_tensor_list(ntensors, numel, "adam")) return rc;
+  if (params == nullptr || grads == nullptr || exp_avg == nullptr || exp_avg_sq == nullptr || slots == nullptr || step == nullptr)
+    return fail(SFH_ERR_INVALID, "adam: null argument");
+  if (!(d->lr >= 0.f) || !(d->beta1 >= 0.f && d->beta1 < 1.f) || !(d->beta2 >= 0.f && d->beta2 < 1.f) || !(d->eps >= 0.f) ||
+      !(d->weight_decay >= 0.f))
+    return fail(SFH_ERR_INVALID, "adam: bad hyperparameters lr=%g betas=(%g, %g) eps=%g weight_decay=%g", d->lr, d->beta1, d->beta2,
+                d->eps, d->weight_decay);
+  if (shadow != nullptr && d->shadow_dtype != SFH_BF16 && d->shadow_dtype != SFH_FP16)
+    return fail(SFH_ERR_INVALID, "adam: shadow copies need shadow_dtype bf16 or fp16, got %d", d->shadow_dtype);
+  for (int i = 0; i < ntensors; ++i)
+    if (params[i] == nullptr || grads[i] == nullptr || exp_avg[i] == nullptr || exp_avg_sq[i] == nullptr)
+      return fail(SFH_ERR_INVALID, "adam: tensor %d has a null pointer", i);
+  return optim_clip_adam(*d, ntensors, params, grads, exp_avg, exp_avg_sq, shadow, numel, slots, (int)nslots, step, grad_norm,
+                         (hipStream_t)stream);
 }
 
 // ---- measurement helper ----------------------------------------------------------------

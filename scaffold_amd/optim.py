@@ -1,0 +1,166 @@
+"""The optimizer step of the train loop in two kernel passes: gradient-norm clipping + Adam.
+
+Stands where the reference's trainer calls ``torch.nn.utils.clip_grad_norm_(model.parameters(), max_norm=1.0)``
+and then ``optimizer.step()`` on ``torch.optim.Adam(..., fused=True)`` (``ScaFFold/utils/trainer.py:678-694``,
+``:268-274``).  Same arithmetic (torch's Adam formulas, bias corrections from a step counter that lives on the
+device, the clipping factor ``min(1, max_norm / (norm + 1e-6))``), but the gradients are scaled on the fly instead
+of being rewritten, the norm is a fixed-order sum (bitwise reproducible), and the whole step is two launches per 48
+tensors with nothing that synchronises, so it can be captured in a graph.
+
+``state_dict()`` has the layout of ``torch.optim.Adam`` (``step``, ``exp_avg``, ``exp_avg_sq`` per parameter), so
+checkpoints move between the two.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import AdamDesc
+
+__all__ = ["FusedClipAdam"]
+
+
+def _ptr_array(tensors):
+    arr = (ctypes.c_void_p * len(tensors))()
+    for i, t in enumerate(tensors):
+        arr[i] = None if t is None else t.data_ptr()
+    return arr
+
+
+class FusedClipAdam(torch.optim.Optimizer):
+    """``clip_grad_norm_(params, max_norm)`` + ``Adam.step()`` fused. fp32 parameters on one GPU only.
+
+    ``max_norm=None`` disables clipping. ``shadow_dtype`` (``torch.bfloat16`` / ``torch.float16``) keeps a
+    half-precision copy of every parameter, refreshed by the update kernel itself, in ``self.shadow[param]``.
+    After ``step()``, ``self.grad_norm`` holds the unclipped total gradient norm (a 0-dim device tensor, what
+    ``clip_grad_norm_`` returns)."""
+
+    def __init__(self, params, lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8, weight_decay: float = 0.0,
+                 max_norm: Optional[float] = None, shadow_dtype: Optional[torch.dtype] = None):
+        if lr < 0.0 or eps < 0.0 or weight_decay < 0.0:
+            raise ValueError(f"invalid hyperparameter: lr={lr} eps={eps} weight_decay={weight_decay}")
+        if not (0.0 <= betas[0] < 1.0 and 0.0 <= betas[1] < 1.0):
+            raise ValueError(f"invalid betas {betas}")
+        if max_norm is not None and not max_norm > 0.0:
+            raise ValueError(f"max_norm must be positive or None, got {max_norm}")
+        if shadow_dtype not in (None, torch.bfloat16, torch.float16):
+            raise ValueError(f"shadow_dtype must be bfloat16, float16 or None, got {shadow_dtype}")
+        super().__init__(params, dict(lr=lr, betas=tuple(betas), eps=eps, weight_decay=weight_decay))
+        self.max_norm = max_norm
+        self.shadow_dtype = shadow_dtype
+        self.shadow = {}
+        self.grad_norm = None
+        self._slots = None
+        self._plans = {}
+
+    @staticmethod
+    def _dense(t):
+        return t.is_contiguous() or (t.dim() == 5 and t.is_contiguous(memory_format=torch.channels_last_3d))
+
+    def _check(self, p):
+        if not p.is_cuda or p.dtype is not torch.float32 or not self._dense(p):
+            raise NotImplementedError(f"FusedClipAdam: parameter must be a dense fp32 GPU tensor, got {p.dtype} on {p.device} "
+                                      f"with strides {tuple(p.stride())}")
+
+    def _state_of(self, p):
+        st = self.state[p]
+        if not st:
+            st["step"] = torch.zeros((), dtype=torch.float32, device=p.device)
+            st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+        return st
+
+    def _plan(self, active, device):
+        """Pointer tables of everything that does not move between steps (parameters, moments, shadow copies),
+        built once per set of active parameters."""
+        key = tuple(id(p) for _, p in active)
+        plan = self._plans.get(key)
+        if plan is not None:
+            return plan
+        L = _lib.lib()
+        params = [p for _, p in active]
+        for p in params:
+            if p.device != device:
+                raise NotImplementedError("FusedClipAdam: all parameters must live on one device")
+            self._check(p)
+        states = [self._state_of(p) for p in params]
+        numel = (ctypes.c_int64 * len(params))(*[p.numel() for p in params])
+        plan = {
+            "params": params, "states": states, "numel": numel, "nslots": int(L.sfh_adam_slots(len(params), numel)),
+            "others": [st["step"] for st in states[1:]], "groups": [],
+        }
+        for group in self.param_groups:
+            idx = [i for i, (g, _) in enumerate(active) if g is group]
+            if not idx:
+                continue
+            gp = [params[i] for i in idx]
+            shadows = None
+            if self.shadow_dtype is not None:
+                for p in gp:
+                    if p not in self.shadow:
+                        self.shadow[p] = torch.empty_like(p, dtype=self.shadow_dtype, memory_format=torch.preserve_format)
+                shadows = _ptr_array([self.shadow[p] for p in gp])
+            plan["groups"].append({
+                "group": group, "idx": idx, "n": len(gp), "p": _ptr_array(gp),
+                "m": _ptr_array([states[i]["exp_avg"] for i in idx]), "v": _ptr_array([states[i]["exp_avg_sq"] for i in idx]),
+                "shadow": shadows, "numel": (ctypes.c_int64 * len(gp))(*[p.numel() for p in gp]),
+            })
+        self._plans = {key: plan}  # keep the latest only: it holds references to every state tensor
+        return plan
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        active = [(g, p) for g in self.param_groups for p in g["params"] if p.grad is not None]
+        if not active:
+            return loss
+        device = active[0][1].device
+        plan = self._plan(active, device)
+        params, states = plan["params"], plan["states"]
+        grads = []
+        for p in params:
+            g = p.grad
+            if g.dtype is not torch.float32 or g.is_sparse or g.device != device or g.stride() != p.stride():
+                raise NotImplementedError(f"FusedClipAdam: gradient must be dense fp32 with the parameter's layout, got {g.dtype}, "
+                                          f"strides {tuple(g.stride())} vs {tuple(p.stride())}")
+            grads.append(g)
+        L = _lib.lib()
+        with torch.cuda.device(device):
+            stream = _lib.stream_ptr(device)
+            # The kernels keep one step counter (the first parameter's, advanced by the first pass); torch keeps one
+            # per parameter, all equal, and a checkpoint must hold them as separate tensors: the others are advanced
+            # by one multi-tensor add.
+            step = states[0]["step"]
+            if plan["others"]:
+                torch._foreach_add_(plan["others"], 1.0)
+            nslots = plan["nslots"]
+            if self._slots is None or self._slots.numel() < nslots or self._slots.device != device:
+                self._slots = torch.empty(nslots, dtype=torch.float32, device=device)
+            if self.grad_norm is None or self.grad_norm.device != device:
+                self.grad_norm = torch.zeros((), dtype=torch.float32, device=device)
+            # one squared-norm pass over every gradient (the norm is global, as in clip_grad_norm_)
+            g_all = _ptr_array(grads)
+            _lib.check(L.sfh_adam_grad_sumsq(len(params), g_all, plan["numel"], _lib.ptr(self._slots), _lib.ptr(step), stream),
+                       "FusedClipAdam (gradient norm)")
+            # one update per hyperparameter group (usually one); each folds ALL slots
+            for gpl in plan["groups"]:
+                group = gpl["group"]
+                desc = AdamDesc(group["lr"], group["betas"][0], group["betas"][1], group["eps"], group["weight_decay"],
+                                -1.0 if self.max_norm is None else float(self.max_norm),
+                                -1 if self.shadow_dtype is None else _lib.dtype_code(self.shadow_dtype))
+                g_arr = g_all if len(plan["groups"]) == 1 else _ptr_array([grads[i] for i in gpl["idx"]])
+                rc = L.sfh_adam_clip_step(ctypes.byref(desc), gpl["n"], gpl["p"], g_arr, gpl["m"], gpl["v"], gpl["shadow"], gpl["numel"],
+                                          _lib.ptr(self._slots), nslots, _lib.ptr(step), _lib.ptr(self.grad_norm), stream)
+                _lib.check(rc, "FusedClipAdam (update)")
+        return loss
+
+    def load_state_dict(self, state_dict):
+        super().load_state_dict(state_dict)
+        self._plans = {}  # the state tensors were replaced
