@@ -192,6 +192,60 @@ def ptr(t):
     return None if t is None else c_void_p(t.data_ptr())
 
 
+class _NoGuard:
+    __slots__ = ()
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """``torch.cuda.device(device)`` only when ``device`` is not already current (the common case costs one query)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
+def _meta(v):
+    """Everything a gate may look at, as a hashable value: tensors by their metadata, sequences as tuples."""
+    if isinstance(v, torch.Tensor):
+        return (torch.Tensor, v.shape, v.dtype, v.device, v.stride(), v.layout)
+    if isinstance(v, (list, tuple)):
+        return tuple(_meta(e) for e in v)
+    return (type(v), v)
+
+
+def memoized_gate(fn):
+    """Caches a gate's verdict by the metadata of its arguments and the autocast state (gates are pure functions of
+    those). Unhashable or exotic arguments simply take the uncached path."""
+    cache = {}
+
+    def wrapper(*args, **kwargs):
+        try:
+            key = (tuple(_meta(a) for a in args), tuple((k, _meta(v)) for k, v in kwargs.items()),
+                   torch.is_autocast_enabled("cuda"))
+            hit = cache.get(key)
+        except Exception:
+            return fn(*args, **kwargs)
+        if hit is None:
+            hit = fn(*args, **kwargs)
+            if len(cache) > 4096:
+                cache.clear()
+            cache[key] = hit
+        return hit
+
+    wrapper.__name__ = fn.__name__
+    wrapper.__doc__ = fn.__doc__
+    wrapper.__wrapped__ = fn
+    return wrapper
+
+
 def workspace(nbytes: int, device: torch.device):
     """A scratch buffer from torch's caching allocator (None when nothing is needed)."""
     if nbytes <= 0:

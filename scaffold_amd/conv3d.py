@@ -93,6 +93,7 @@ def _desc(n, cin, in_sp, cout, k, s, p, d) -> ConvDesc:
 # ---------------------------------------------------------------------------------------------
 # gates
 # ---------------------------------------------------------------------------------------------
+@_lib.memoized_gate
 def is_supported(x, w, bias=None, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
     """Whether :func:`conv3d_forward` serves this call.  Total: never raises."""
     try:
@@ -129,6 +130,7 @@ def is_supported(x, w, bias=None, stride=1, padding=0, dilation=1, groups: int =
         return False
 
 
+@_lib.memoized_gate
 def is_supported_bwd_data(grad_output, weight, input_shape, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
     """Whether :func:`conv3d_backward_data` serves this call: stride 1 and ``p <= dil*(k-1)`` only."""
     try:
@@ -162,6 +164,7 @@ def is_supported_bwd_data(grad_output, weight, input_shape, stride=1, padding=0,
         return False
 
 
+@_lib.memoized_gate
 def is_supported_bwd_weight(input, weight_shape, grad_output, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
     """Whether :func:`conv3d_backward_weight` serves this call (any stride)."""
     try:
@@ -194,6 +197,7 @@ def is_supported_bwd_weight(input, weight_shape, grad_output, stride=1, padding=
         return False
 
 
+@_lib.memoized_gate
 def is_supported_all(x, w, bias=None, stride=1, padding=0, dilation=1, groups: int = 1) -> bool:
     """Whether all three directions of this convolution are served (the gate for a caller
     that will differentiate): the forward accepts strides the data gradient refuses."""
@@ -292,7 +296,7 @@ def bias_grad(grad_output: torch.Tensor, dtype: Optional[torch.dtype] = None) ->
     if rows == 0:
         return gb.zero_()
     L = _lib.lib()
-    with torch.cuda.device(g.device):
+    with _lib.device_guard(g.device):
         ws = _lib.workspace(int(L.sfh_bias_grad_workspace_bytes(rows, c)), g.device)
         rc = L.sfh_bias_grad(_lib.dtype_code(g.dtype), _lib.dtype_code(out_dtype), _lib.ptr(g), rows, c, _lib.ptr(gb),
                              _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(g.device))
@@ -317,6 +321,7 @@ def conv3d_forward(
     weight_flip: bool = False,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    _checked: bool = False,
 ) -> torch.Tensor:
     """Forward 3-D convolution; input and output are ``channels_last_3d``.
 
@@ -325,7 +330,7 @@ def conv3d_forward(
     a host-side transform and give bitwise identical results.  ``weight_flip`` consumes the
     taps mirrored in all three axes (the data gradient's view of the weight).
     """
-    if not is_supported(x, w, bias, stride, padding, dilation, groups):
+    if not _checked and not is_supported(x, w, bias, stride, padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)} "
             f"w={tuple(getattr(w, 'shape', ()))} stride={stride} padding={padding} dilation={dilation} groups={groups}"
@@ -354,7 +359,7 @@ def conv3d_forward(
     L = _lib.lib()
     desc = _desc(n, cin, in_sp, cout, k, s, p, d)
     code = _lib.dtype_code(x.dtype)
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         ws = _lib.workspace(L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
         rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(bias),
                               _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
@@ -379,6 +384,7 @@ def conv3d_backward_data(
     weight_rsck: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    _checked: bool = False,
 ) -> torch.Tensor:
     """Gradient of a conv3d with respect to its input (stride 1 only).
 
@@ -386,7 +392,7 @@ def conv3d_backward_data(
     taps mirrored and padding ``dil*(k-1) - p``; the swap and the mirror happen while the library
     repacks the weight, so no transformed copy of the weight is made here.
     """
-    if not is_supported_bwd_data(grad_output, weight, input_shape, stride, padding, dilation, groups):
+    if not _checked and not is_supported_bwd_data(grad_output, weight, input_shape, stride, padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: grad_output={tuple(getattr(grad_output, 'shape', ()))}/{getattr(grad_output, 'dtype', None)} "
             f"w={tuple(getattr(weight, 'shape', ()))} input_shape={tuple(input_shape)} stride={stride} "
@@ -412,7 +418,7 @@ def conv3d_backward_data(
     L = _lib.lib()
     desc = _desc(n, cin, in_sp, cout, k, s, p, d)
     code = _lib.dtype_code(gy.dtype)
-    with torch.cuda.device(gy.device):
+    with _lib.device_guard(gy.device):
         ws = _lib.workspace(L.sfh_conv3d_dgrad_workspace_bytes(ctypes.byref(desc), code), gy.device)
         rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(gx),
                                 _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
@@ -455,6 +461,7 @@ def conv3d_backward_weight(
     workspace: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    _checked: bool = False,
 ) -> torch.Tensor:
     """Gradient of a conv3d with respect to its weight, returned ``channels_last_3d``.
 
@@ -462,7 +469,7 @@ def conv3d_backward_weight(
     ordered reduction; there is no atomic variant, so ``deterministic=False`` is refused rather
     than silently served by the deterministic path.
     """
-    if not is_supported_bwd_weight(input, weight_shape, grad_output, stride, padding, dilation, groups):
+    if not _checked and not is_supported_bwd_weight(input, weight_shape, grad_output, stride, padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: input={tuple(getattr(input, 'shape', ()))}/{getattr(input, 'dtype', None)} "
             f"weight_shape={tuple(weight_shape)} grad_output={tuple(getattr(grad_output, 'shape', ()))} "
@@ -488,7 +495,7 @@ def conv3d_backward_weight(
     code = _lib.dtype_code(x.dtype)
     if n == 0:
         return gw.zero_()
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         need = 0 if force_generic else int(L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(desc), code))
         if workspace is None:
             ws = _lib.workspace(need, x.device)

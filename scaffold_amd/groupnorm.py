@@ -85,17 +85,8 @@ def _desc(input, num_groups: int, eps: float, activation) -> GroupNormDesc:
     return GroupNormDesc(n, c, int(num_groups), 1 if activation == "relu" else 0, spatial, float(eps))
 
 
-@torch.library.custom_op("scaffold_gn::group_norm", mutates_args=(), device_types="cuda")
-def _group_norm_op(
-    input: torch.Tensor,
-    num_groups: int,
-    weight: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    eps: float,
-    activation: Optional[str],
-    out_dtype: Optional[torch.dtype],
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """Channels-last GroupNorm forward: ``(output, mean, rstd)``; mean/rstd are ``(N, G)`` fp32."""
+def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype):
+    """The forward launch: ``(output, mean, rstd)``; shared by the registered operator and the eager autograd node."""
     _validate(input, num_groups, weight, bias, activation)
     weight = None if weight is None else weight.contiguous()
     bias = None if bias is None else bias.contiguous()
@@ -111,7 +102,7 @@ def _group_norm_op(
     L = _lib.lib()
     desc = _desc(input, num_groups, eps, activation)
     xcode = _lib.dtype_code(input.dtype)
-    with torch.cuda.device(input.device):
+    with _lib.device_guard(input.device):
         ws = _lib.workspace(L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
         rc = L.sfh_groupnorm_fwd(
             ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
@@ -119,6 +110,20 @@ def _group_norm_op(
             _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
     _lib.check(rc, "group_norm")
     return out, mean, rstd
+
+
+@torch.library.custom_op("scaffold_gn::group_norm", mutates_args=(), device_types="cuda")
+def _group_norm_op(
+    input: torch.Tensor,
+    num_groups: int,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    eps: float,
+    activation: Optional[str],
+    out_dtype: Optional[torch.dtype],
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Channels-last GroupNorm forward: ``(output, mean, rstd)``; mean/rstd are ``(N, G)`` fp32."""
+    return _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype)
 
 
 @_group_norm_op.register_fake
@@ -129,19 +134,8 @@ def _(input, num_groups, weight, bias, eps, activation, out_dtype):
     return out, mean, rstd
 
 
-@torch.library.custom_op("scaffold_gn::group_norm_backward", mutates_args=(), device_types="cuda")
-def _group_norm_backward_op(
-    grad_out: torch.Tensor,
-    input: torch.Tensor,
-    weight: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    mean: torch.Tensor,
-    rstd: torch.Tensor,
-    num_groups: int,
-    activation: Optional[str],
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """``(d_input, d_weight, d_bias)``; the parameter gradients are empty when the parameter is None.
-    ``d_input`` has the input's dtype and is channels_last_3d."""
+def _backward_impl(grad_out, input, weight, bias, mean, rstd, num_groups, activation):
+    """The backward launch: ``(d_input, d_weight, d_bias)``."""
     if not grad_out.is_contiguous(memory_format=_CL3D):
         grad_out = grad_out.contiguous(memory_format=_CL3D)
     if not input.is_contiguous(memory_format=_CL3D):
@@ -160,7 +154,7 @@ def _group_norm_backward_op(
         L = _lib.lib()
         desc = _desc(input, num_groups, 0.0, activation)
         xcode = _lib.dtype_code(input.dtype)
-        with torch.cuda.device(input.device):
+        with _lib.device_guard(input.device):
             ws = _lib.workspace(L.sfh_groupnorm_bwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
             rc = L.sfh_groupnorm_bwd(
                 ctypes.byref(desc), xcode, _lib.dtype_code(grad_out.dtype),
@@ -176,6 +170,22 @@ def _group_norm_backward_op(
     d_weight = input.new_empty(0, dtype=torch.float32) if weight is None else dw32.to(weight.dtype)
     d_bias = input.new_empty(0, dtype=torch.float32) if bias is None else db32.to(bias.dtype)
     return d_input, d_weight, d_bias
+
+
+@torch.library.custom_op("scaffold_gn::group_norm_backward", mutates_args=(), device_types="cuda")
+def _group_norm_backward_op(
+    grad_out: torch.Tensor,
+    input: torch.Tensor,
+    weight: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    mean: torch.Tensor,
+    rstd: torch.Tensor,
+    num_groups: int,
+    activation: Optional[str],
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(d_input, d_weight, d_bias)``; the parameter gradients are empty when the parameter is None.
+    ``d_input`` has the input's dtype and is channels_last_3d."""
+    return _backward_impl(grad_out, input, weight, bias, mean, rstd, num_groups, activation)
 
 
 @_group_norm_backward_op.register_fake
@@ -213,6 +223,29 @@ def _autograd_backward(ctx, grad_out, grad_mean, grad_rstd):
 torch.library.register_autograd("scaffold_gn::group_norm", _autograd_backward, setup_context=_setup_context)
 
 
+class _EagerGroupNormFn(torch.autograd.Function):
+    """The same two launches as the registered operators, as a plain autograd node: outside ``torch.compile`` the
+    operator registry's dispatch costs more host time per call than both launches together."""
+
+    @staticmethod
+    def forward(ctx, input, num_groups, weight, bias, eps, activation, out_dtype):
+        out, mean, rstd = _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype)
+        ctx.save_for_backward(input, weight, bias, mean, rstd)
+        ctx.num_groups = num_groups
+        ctx.activation = activation
+        return out
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_out):
+        input, weight, bias, mean, rstd = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[2], ctx.needs_input_grad[3]
+        if not (need_x or need_w or need_b):
+            return None, None, None, None, None, None, None
+        d_input, d_weight, d_bias = _backward_impl(grad_out, input, weight, bias, mean, rstd, ctx.num_groups, ctx.activation)
+        return (d_input if need_x else None, None, d_weight if need_w else None, d_bias if need_b else None, None, None, None)
+
+
 # ---------------------------------------------------------------------------------------------
 # public API
 # ---------------------------------------------------------------------------------------------
@@ -242,6 +275,7 @@ def _resolve_out_dtype(input: torch.Tensor, out_dtype) -> Optional[torch.dtype]:
     return out_dtype
 
 
+@_lib.memoized_gate
 def is_supported(input, num_groups: int, weight=None, bias=None, activation: Optional[str] = None) -> bool:
     """Whether the HIP kernels serve this call: a 5-D CUDA tensor, ``channels_last_3d``-contiguous,
     fp32/bf16/fp16, C divisible by ``num_groups``, affine parameters of the input's dtype (or fp32 under
@@ -297,10 +331,12 @@ def group_norm(input, num_groups: int, weight=None, bias=None, eps: float = 1e-5
             f"unsupported group_norm call: input={tuple(getattr(input, 'shape', ()))}/{getattr(input, 'dtype', None)} on "
             f"{getattr(input, 'device', None)}, num_groups={num_groups}; needs a channels_last_3d CUDA tensor"
         )
-    out, _mean, _rstd = torch.ops.scaffold_gn.group_norm(
-        input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype)
-    )
-    return out
+    if torch.compiler.is_compiling():
+        out, _mean, _rstd = torch.ops.scaffold_gn.group_norm(
+            input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype)
+        )
+        return out
+    return _EagerGroupNormFn.apply(input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype))
 
 
 #: the reference's name for :func:`group_norm`

@@ -57,7 +57,7 @@ class _CeDiceFn(torch.autograd.Function):
         L = _lib.lib()
         loss = torch.empty((), dtype=torch.float32, device=x.device)
         stats = torch.empty((n * 3 * c + 2,), dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
+        with _lib.device_guard(x.device):
             ws = _lib.workspace(int(L.sfh_ce_dice_workspace_bytes(ctypes.byref(desc))), x.device)
             rc = L.sfh_ce_dice_fwd(ctypes.byref(desc), _lib.dtype_code(x.dtype), _lib.ptr(x), _lib.ptr(lab), _lib.ptr(cw),
                                    _lib.ptr(loss), _lib.ptr(stats), _lib.ptr(ws), 0 if ws is None else ws.numel(),
@@ -78,7 +78,7 @@ class _CeDiceFn(torch.autograd.Function):
         g = grad_loss.detach().to(device=x.device, dtype=torch.float32).reshape(1).contiguous()
         dx = torch.empty_like(x, memory_format=_CL3D)
         L = _lib.lib()
-        with torch.cuda.device(x.device):
+        with _lib.device_guard(x.device):
             rc = L.sfh_ce_dice_bwd(ctypes.byref(desc), _lib.dtype_code(x.dtype), _lib.ptr(x), _lib.ptr(lab), _lib.ptr(cw),
                                    _lib.ptr(stats), _lib.ptr(g), _lib.ptr(dx), _lib.stream_ptr(x.device))
         _lib.check(rc, "ce_dice_loss backward")

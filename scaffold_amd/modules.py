@@ -61,9 +61,12 @@ def cast_operand(tensor: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
 
 
 class _Conv3dFn(torch.autograd.Function):
+    """The caller (``FastConv3d.forward``) has passed the gate for all three directions with these very operands, and
+    autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
+
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, dilation):
-        y = _c3.conv3d_forward(x, weight, bias, stride, padding, dilation, 1)
+        y = _c3.conv3d_forward(x, weight, bias, stride, padding, dilation, 1, _checked=True)
         ctx.save_for_backward(x, weight)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype)
         return y
@@ -75,8 +78,8 @@ class _Conv3dFn(torch.autograd.Function):
         stride, padding, dilation, has_bias, bias_dtype = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
-        grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1) if needs_x else None
-        grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1) if needs_w else None
+        grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1, _checked=True) if needs_x else None
+        grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True) if needs_w else None
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
         return grad_x, grad_w, grad_b, None, None, None
 
@@ -125,6 +128,8 @@ class FastConv3d(nn.Conv3d):
             x = F.pad(x, (0, 0, 0, 0, padding[0], padding[0]))
             padding = (0, padding[1], padding[2])
         x = x.contiguous(memory_format=_CL3D)
+        # the node below skips its own gates on the strength of this one (a call that will be differentiated is
+        # gated for all three directions here)
         gate = _c3.is_supported_all if _wants_grad(x, w, b) else _c3.is_supported
         if not gate(x, w, b, self.stride, padding, self.dilation, self.groups):
             raise NotImplementedError(

@@ -132,7 +132,7 @@ class FusedClipAdam(torch.optim.Optimizer):
                                           f"strides {tuple(g.stride())} vs {tuple(p.stride())}")
             grads.append(g)
         L = _lib.lib()
-        with torch.cuda.device(device):
+        with _lib.device_guard(device):
             stream = _lib.stream_ptr(device)
             # The kernels keep one step counter (the first parameter's, advanced by the first pass); torch keeps one
             # per parameter, all equal, and a checkpoint must hold them as separate tensors: the others are advanced

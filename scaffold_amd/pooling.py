@@ -39,7 +39,7 @@ class _MaxPool2Fn(torch.autograd.Function):
         y = torch.empty((n, c, d // 2, h // 2, w // 2), dtype=x.dtype, device=x.device, memory_format=_CL3D)
         idx = torch.empty((n, d // 2, h // 2, w // 2, c), dtype=torch.uint8, device=x.device)
         desc = PoolDesc(n, c, d, h, w)
-        with torch.cuda.device(x.device):
+        with _lib.device_guard(x.device):
             rc = _lib.lib().sfh_maxpool2_fwd(ctypes.byref(desc), _lib.dtype_code(x.dtype), _lib.ptr(x), _lib.ptr(y), _lib.ptr(idx),
                                              _lib.stream_ptr(x.device))
         _lib.check(rc, "max_pool3d_2x")
@@ -55,7 +55,7 @@ class _MaxPool2Fn(torch.autograd.Function):
         gy = grad_y.contiguous(memory_format=_CL3D)
         gx = torch.empty((n, c, d, h, w), dtype=gy.dtype, device=gy.device, memory_format=_CL3D)
         desc = PoolDesc(n, c, d, h, w)
-        with torch.cuda.device(gy.device):
+        with _lib.device_guard(gy.device):
             rc = _lib.lib().sfh_maxpool2_bwd(ctypes.byref(desc), _lib.dtype_code(gy.dtype), _lib.ptr(gy), _lib.ptr(idx), _lib.ptr(gx),
                                              _lib.stream_ptr(gy.device))
         _lib.check(rc, "max_pool3d_2x backward")

@@ -68,6 +68,7 @@ def _kernel_if_tiling(x_dim: int, w, stride, padding, output_padding, dilation, 
         return None
 
 
+@_lib.memoized_gate
 def is_supported_transposed(x, w, bias=None, stride=1, padding=0, output_padding=0, dilation=1, groups: int = 1) -> bool:
     """Whether :func:`conv_transpose3d_forward` serves this call.  ``w`` is ``(Cin, Cout, kd, kh, kw)``."""
     try:
@@ -94,6 +95,7 @@ def is_supported_transposed(x, w, bias=None, stride=1, padding=0, output_padding
         return False
 
 
+@_lib.memoized_gate
 def is_supported_transposed_bwd_data(grad_output, w, input_shape, stride=1, padding=0, output_padding=0, dilation=1,
                                      groups: int = 1) -> bool:
     """Whether :func:`conv_transpose3d_backward_data` serves this call."""
@@ -118,6 +120,7 @@ def is_supported_transposed_bwd_data(grad_output, w, input_shape, stride=1, padd
         return False
 
 
+@_lib.memoized_gate
 def is_supported_transposed_bwd_weight(x, weight_shape, grad_output, stride=1, padding=0, output_padding=0, dilation=1,
                                        groups: int = 1) -> bool:
     """Whether :func:`conv_transpose3d_backward_weight` serves this call."""
@@ -132,6 +135,7 @@ def is_supported_transposed_bwd_weight(x, weight_shape, grad_output, stride=1, p
         return False
 
 
+@_lib.memoized_gate
 def is_supported_transposed_all(x, w, bias=None, stride=1, padding=0, output_padding=0, dilation=1, groups: int = 1) -> bool:
     """All three directions; asked for real rather than assumed to agree."""
     if not is_supported_transposed(x, w, bias, stride, padding, output_padding, dilation, groups):
@@ -189,7 +193,7 @@ def conv_transpose3d_forward(
     L = _lib.lib()
     desc = ConvTDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2])
     code = _lib.dtype_code(x.dtype)
-    with torch.cuda.device(x.device):
+    with _lib.device_guard(x.device):
         ws = _lib.workspace(L.sfh_convT3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
         rc = L.sfh_convT3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w), _lib.strides5(w), _lib.ptr(bias),
                                _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
