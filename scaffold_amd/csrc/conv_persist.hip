@@ -182,25 +182,37 @@ __device__ __forceinline__ T* tile_origin(const MfmaConvArgs& a, T* y, const Til
 }
 
 // Output of a finished brick, rounded, waiting to be stored during the next step. Accumulator register 4g+t of a
-// lane is output channel 8g + 4*kg + t of voxel j of the sub-tile: the two k-half lanes of a voxel write adjacent
-// 8-byte halves of a 16-byte piece.
+// lane is output channel 8g + 4*kg + t of voxel j of the sub-tile, so the two k-half lanes of a voxel (lanes j and
+// j + 32) hold interleaved runs of four channels. They trade runs (v_permlane32_swap) so that the kg = 0 lane ends
+// up with channels 0-7 and 16-23 and the kg = 1 lane with 8-15 and 24-31: each then stores two 16-byte pieces, and
+// one store instruction covers 32 contiguous bytes of every voxel instead of 16.
+typedef uint32_t sfh_u32x4_t __attribute__((ext_vector_type(4)));
 template <typename C>
 struct PendingStore {
-  sfh_u32x2_t data[C::MS][4];
+  sfh_u32x4_t data[C::MS][2];
 };
 
 template <typename T, typename C, bool BIAS>
 __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const float (&bias)[16], PendingStore<C>& ps) {
 #pragma unroll
-  for (int ms = 0; ms < C::MS; ++ms)
+  for (int ms = 0; ms < C::MS; ++ms) {
+    uint32_t run[4][2];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       float v[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) v[t] = BIAS ? acc[ms][4 * g + t] + bias[4 * g + t] : acc[ms][4 * g + t];
-      ps.data[ms][g][0] = Mma<T>::pack2(v[0], v[1]);
-      ps.data[ms][g][1] = Mma<T>::pack2(v[2], v[3]);
+      run[g][0] = Mma<T>::pack2(v[0], v[1]);
+      run[g][1] = Mma<T>::pack2(v[2], v[3]);
     }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // lanes 32-63 of run 2h <-> lanes 0-31 of run 2h+1
+      const auto lo = __builtin_amdgcn_permlane32_swap(run[2 * h][0], run[2 * h + 1][0], false, false);
+      const auto hi = __builtin_amdgcn_permlane32_swap(run[2 * h][1], run[2 * h + 1][1], false, false);
+      ps.data[ms][h] = sfh_u32x4_t{lo[0], hi[0], lo[1], hi[1]};
+    }
+  }
 }
 
 // One step = one output brick. While the 54 x MS MFMAs run over the brick in `cur`, the wavefront also issues, a
@@ -219,10 +231,11 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
                                              const TileCoord& plan_tc, bool plan_live, const TileCoord& tc) {
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(fetch_origin), 0, kRange, 0x00020000);
   constexpr int NLOAD = C::GPW * 4;
-  constexpr int NSTORE = C::MS * 4;
-  constexpr int PLAN0 = 2 * NSTORE + 1;             // first (odd) iteration that plans a group
+  constexpr int NSTORE = C::MS * 2;
+  // group k's offsets are overwritten in place, so its planning must come after its last load (iteration 8k + 6)
+  constexpr int PLAN0 = 6 * (C::GPW - 1) + 9;       // first (odd) iteration that plans a group
   constexpr int OFF0 = PLAN0 + 2 * C::GPW;          // first (odd) iteration that computes a store offset
-  static_assert(2 * NLOAD <= C::NIT && OFF0 + 2 * C::MS <= C::NIT + 1, "one piece of side work per iteration");
+  static_assert(2 * NLOAD <= C::NIT && OFF0 + 2 * C::MS <= C::NIT + 1 && PLAN0 > 2 * NSTORE, "one piece of side work per iteration");
   // activation fragments are requested ADEPTH iterations ahead of the MFMAs that consume them
   constexpr int ADEPTH = 2;
   uint4 aq[ADEPTH + 1][C::MS];
@@ -246,8 +259,8 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
                                                  16, voff[k] + p * 16, 0, 0, 0);
     }
     if (it % 2 == 1 && it / 2 < NSTORE) {
-      const int ms = (it / 2) / 4, g = (it / 2) % 4;
-      __builtin_amdgcn_raw_buffer_store_b64(ps.data[ms][g], done_rsrc, done_off[ms] + 16 * g, 0, 0);
+      const int ms = (it / 2) / 2, h = (it / 2) % 2;
+      __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
     }
     if (it % 2 == 1 && it >= PLAN0 && (it - PLAN0) / 2 < C::GPW) {
       const int k = (it - PLAN0) / 2;
@@ -303,7 +316,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
     lg.lbase[ms] = kg * C::PLANE + ((td * C::BH + th) * C::BW + tw) * 16;
     lg.vcoord[ms] = td | (th << 8) | (tw << 16);
-    lg.vrel[ms] = (((td * a.oh + th) * a.ow + tw) * a.cout + 4 * kg) * 2;
+    lg.vrel[ms] = (((td * a.oh + th) * a.ow + tw) * a.cout + 8 * kg) * 2;
   }
   // Staging role of this lane, fixed for the whole launch: wave w fills the 64-voxel groups w, w+4, ... of every
   // plane; the lane's voxel inside the brick and its byte offset from the brick origin in the input tensor.
@@ -346,7 +359,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) ps.data[ms][g] = sfh_u32x2_t{0u, 0u};
+    for (int h = 0; h < 2; ++h) ps.data[ms][h] = sfh_u32x4_t{0u, 0u, 0u, 0u};
   int done_off[C::MS];
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) done_off[ms] = kRange;  // nothing to store during the first step
@@ -372,7 +385,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) __builtin_amdgcn_raw_buffer_store_b64(ps.data[ms][g], done_rsrc, done_off[ms] + 16 * g, 0, 0);
+    for (int h = 0; h < 2; ++h) __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
 #endif
 }
 
