@@ -59,6 +59,19 @@ __device__ __forceinline__ uint32_t pack_fp16x2(float lo, float hi) {
 __device__ __forceinline__ float fp16_lo(uint32_t u) { union { uint32_t u; _Float16 h[2]; } r; r.u = u; return (float)r.h[0]; }
 __device__ __forceinline__ float fp16_hi(uint32_t u) { union { uint32_t u; _Float16 h[2]; } r; r.u = u; return (float)r.h[1]; }
 
+// Four packed runs of four 16-bit channels each, as an MFMA 32x32 result leaves them in the two lanes of a voxel
+// (lane kg holds channels 8g + 4kg .. + 3 as run g): the lanes l and l + 32 trade runs so that lane kg ends up with
+// the 16-byte pieces of channels 8kg .. 8kg + 7 (out[0]) and 16 + 8kg .. 16 + 8kg + 7 (out[1]). All 64 lanes must
+// call it.
+__device__ __forceinline__ void trade_channel_runs(const uint32_t (&run)[4][2], uint4 (&out)[2]) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const auto lo = __builtin_amdgcn_permlane32_swap(run[2 * h][0], run[2 * h + 1][0], false, false);
+    const auto hi = __builtin_amdgcn_permlane32_swap(run[2 * h][1], run[2 * h + 1][1], false, false);
+    out[h] = make_uint4(lo[0], hi[0], lo[1], hi[1]);
+  }
+}
+
 inline size_t dtype_size(int dtype) { return dtype == SFH_FP32 ? 4 : 2; }
 inline bool dtype_ok(int dtype) { return dtype == SFH_BF16 || dtype == SFH_FP16 || dtype == SFH_FP32; }
 

@@ -17,7 +17,8 @@
 //     wavefront fetches the fragment for (tap, k-step) as one contiguous 1 KiB global load that
 //     hits in L1/L2; it is reused across the wave's four 32-voxel sub-tiles.
 //   * v_mfma_f32_32x32x16 with the WEIGHT as the row operand: a lane then ends up holding, for
-//     one voxel, four runs of four consecutive output channels, which are stored as 8-byte pieces.
+//     one voxel, four runs of four consecutive output channels; the two lanes of a voxel trade runs and store
+//     16-byte pieces.
 //
 // The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
 // padding k-1-p (triton_conv3d/bwd_data.py:344-363).
@@ -191,15 +192,18 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   }
 
   // Epilogue. Accumulator register r of a lane is output channel 8*(r/4) + 4*kg + r%4 of the
-  // sub-tile's voxel j: four runs of four consecutive channels per 32-channel block.
+  // sub-tile's voxel j: four runs of four consecutive channels per 32-channel block. For the 16-bit output the two
+  // lanes of a voxel trade runs so that each stores two 16-byte pieces (32 contiguous bytes of a voxel per store
+  // instruction).
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     const int v = (wave * C::MS + ms) * 32 + j;
     const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
     const int od = od0 + td, oh = oh0 + th, ow = ow0 + tw;
-    if (od >= a.od || oh >= a.oh || ow >= a.ow) continue;
+    const bool inside = od < a.od && oh < a.oh && ow < a.ow;
     const int64_t vox = (((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow;
     if (ksplit > 1) {
+      if (!inside) continue;
       // fp32 slice of this reduction range; the slices are summed (and the bias added) by sum_slices_bias
       float* pp = partial + ((int64_t)ksp * a.n * a.od * a.oh * a.ow + vox) * a.cout + nb * C::NSUB * 32;
 #pragma unroll
@@ -213,6 +217,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     T* yp = y + vox * a.cout + nb * C::NSUB * 32;
 #pragma unroll
     for (int ns = 0; ns < C::NSUB; ++ns) {
+      uint32_t run[4][2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int co = ns * 32 + 8 * g + 4 * kg;
@@ -221,10 +226,14 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
           const T* bp = bias + nb * C::NSUB * 32 + co;
           b0 = to_float(bp[0]); b1 = to_float(bp[1]); b2 = to_float(bp[2]); b3 = to_float(bp[3]);
         }
-        uint2 o;
-        o.x = Mma<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
-        o.y = Mma<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
-        *reinterpret_cast<uint2*>(yp + co) = o;
+        run[g][0] = Mma<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
+        run[g][1] = Mma<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
+      }
+      uint4 piece[2];
+      trade_channel_runs(run, piece);  // all lanes take part, also those of voxels past the edge
+      if (inside) {
+        *reinterpret_cast<uint4*>(yp + ns * 32 + 8 * kg) = piece[0];
+        *reinterpret_cast<uint4*>(yp + ns * 32 + 16 + 8 * kg) = piece[1];
       }
     }
   }

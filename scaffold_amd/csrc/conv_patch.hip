@@ -47,19 +47,25 @@ template <typename T>
 __device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
 
 // Stores result block `acc` (32 produced channels x 32 voxels): this lane's voxel row starts at `row`
-// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given.
+// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given. The two lanes of a voxel trade
+// channel runs first, so each stores two 16-byte pieces. All 64 lanes must call it; `valid` masks the stores.
 template <typename T>
-__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg) {
+__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
+  uint32_t run[4][2];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     const int c = 8 * g + 4 * kg;
     float v[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = acc[4 * g + i] + (bias != nullptr ? to_float(bias[c0 + c + i]) : 0.f);
-    uint2 o;
-    o.x = Mma32<T>::pack2(v[0], v[1]);
-    o.y = Mma32<T>::pack2(v[2], v[3]);
-    *reinterpret_cast<uint2*>(row + c) = o;
+    run[g][0] = Mma32<T>::pack2(v[0], v[1]);
+    run[g][1] = Mma32<T>::pack2(v[2], v[3]);
+  }
+  uint4 piece[2];
+  trade_channel_runs(run, piece);
+  if (valid) {
+    *reinterpret_cast<uint4*>(row + 8 * kg) = piece[0];
+    *reinterpret_cast<uint4*>(row + 16 + 8 * kg) = piece[1];
   }
 }
 
@@ -97,9 +103,9 @@ __global__ void __launch_bounds__(256) patch_gather_kernel(PatchArgs a, const T*
         for (int b = 0; b < NB; ++b) acc[b] = Mma32<T>::run(wf[ks][b], bf[ks], acc[b]);
     }
   }
-  if (!valid) return;
+  const int64_t vs = valid ? v : total - 1;
 #pragma unroll
-  for (int b = 0; b < NB; ++b) store_block<T>(acc[b], small + v * a.csmall + (blk0 + b) * 32, bias, (blk0 + b) * 32, kg);
+  for (int b = 0; b < NB; ++b) store_block<T>(acc[b], small + vs * a.csmall + (blk0 + b) * 32, bias, (blk0 + b) * 32, kg, valid);
 }
 
 // ---- scatter: transposed convolution -----------------------------------------------------------
@@ -132,10 +138,9 @@ __global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T
       for (int t = 0; t < kTaps; ++t) acc[t] = Mma32<T>::run(wf[t], sf, acc[t]);
     }
   }
-  if (!valid) return;
-  const Voxel vx = decode_small(a, v);
+  const Voxel vx = decode_small(a, vc);
 #pragma unroll
-  for (int t = 0; t < kTaps; ++t) store_block<T>(acc[t], big + big_index(a, vx, t) * a.cbig + blk * 32, bias, blk * 32, kg);
+  for (int t = 0; t < kTaps; ++t) store_block<T>(acc[t], big + big_index(a, vx, t) * a.cbig + blk * 32, bias, blk * 32, kg, valid);
 }
 
 // ---- reduce: weight gradient -------------------------------------------------------------------
