@@ -180,7 +180,7 @@ def copy_calibration(device, mib=256, reps=4):
     return {"bytes_read": src.numel(), "bytes_written": src.numel(), "launches": reps}
 
 
-def bench_unet_step(args, device):
+def bench_unet_step(args, device, eager_only=False):
     """Config 5: one Adam step of the base-32, 5-level U-Net on a 64x128x128 depth shard (zero halo),
     bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0 fused with the Adam update.
 
@@ -213,6 +213,8 @@ def bench_unet_step(args, device):
     step = step_fn(model, opt)
     ms = event_time_ms(step, 10, warmup=3)
     out = {"ms_per_step": ms, "input": "1x1x64x128x128 occupancy (5% ones), zero depth halo, padding (0,1,1)"}
+    if eager_only:
+        return out
     # The same arithmetic without the halo emulation's copies (depth padding 1 inside the kernels; bitwise the same
     # result): what remains is the cost of the step itself, the difference is the bench's stand-in for DistConv's
     # halo exchange.
@@ -299,6 +301,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--skip-unet", action="store_true", help="omit the U-Net train step")
+    ap.add_argument("--unet-profile", action="store_true",
+                    help="run only 13 eager U-Net train steps (3 warm-up + 10) and print their time: the command to trace "
+                         "when a per-kernel breakdown of the step is wanted")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB (reference point for HBM counter runs)")
     args = ap.parse_args()
@@ -310,6 +315,9 @@ def main():
         print("bench.py needs a GPU (no CPU fallback exists for the hot path)", file=sys.stderr)
         sys.exit(2)
     device = torch.device("cuda:0")
+    if args.unet_profile:
+        print(json.dumps({"unet_step_cfg5": bench_unet_step(args, device, eager_only=True)}))
+        return
     conv = bench_conv(args, device)
     details = {"conv": conv}
     if args.copy_calibration:
