@@ -195,7 +195,9 @@ def bench_unet_step(args, device, eager_only=False):
     def make(shard_halo=True):
         torch.manual_seed(5001)
         model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(shard_halo)
-        opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0)  # clip_grad_norm_(1.0) + Adam, trainer.py:678-694
+        # clip_grad_norm_(1.0) + Adam (trainer.py:678-694); the update kernel also keeps the bf16 copies of the weights
+        # the convolutions read under autocast, and they return fp32 weight gradients: no per-step casts either way
+        opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
         return model, opt
 
     def step_fn(model, opt):
@@ -243,6 +245,7 @@ def bench_unet_step(args, device, eager_only=False):
             for k, v in st.items():
                 if torch.is_tensor(v):
                     v.zero_()
+        opt_g.refresh_shadows()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             static_loss = gstep()

@@ -41,6 +41,10 @@ extern "C" {
 
 /* Flags for the convolution entry points. */
 #define SFH_FLAG_FORCE_GENERIC 1u /* use the direct (non-MFMA) kernels whatever the shape */
+#define SFH_FLAG_GRAD_FP32 2u     /* sfh_conv3d_wgrad: write grad_w as fp32 (the master weight's dtype under
+                                     autocast) instead of the operands' dtype: the fp32 sum of the slices is
+                                     stored as it is, saving the rounding and the caller's up-cast. Served by
+                                     the tiled kernels; SFH_ERR_UNSUPPORTED where only the untiled one applies. */
 
 /* A convolution problem as torch.nn.functional.conv3d names it (groups == 1). */
 typedef struct sfh_conv3d_desc {

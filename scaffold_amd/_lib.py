@@ -38,6 +38,7 @@ __all__ = [
 
 SFH_OK, SFH_ERR_INVALID, SFH_ERR_UNSUPPORTED, SFH_ERR_WORKSPACE, SFH_ERR_LAUNCH = range(5)
 SFH_FLAG_FORCE_GENERIC = 1
+SFH_FLAG_GRAD_FP32 = 2
 
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 SUPPORTED_DTYPES = tuple(_DTYPE_CODE)

@@ -461,13 +461,16 @@ def conv3d_backward_weight(
     workspace: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    grad_dtype: Optional[torch.dtype] = None,
     _checked: bool = False,
 ) -> torch.Tensor:
     """Gradient of a conv3d with respect to its weight, returned ``channels_last_3d``.
 
     Split-K over the output voxels with fp32 partial slices at fixed workspace slots and an
     ordered reduction; there is no atomic variant, so ``deterministic=False`` is refused rather
-    than silently served by the deterministic path.
+    than silently served by the deterministic path.  ``grad_dtype=torch.float32`` with 16-bit operands returns
+    the fp32 sum of the slices unrounded (the gradient of an fp32 master weight under autocast, without the
+    rounding and the up-cast); shapes only the untiled kernel serves raise ``NotImplementedError`` for it.
     """
     if not _checked and not is_supported_bwd_weight(input, weight_shape, grad_output, stride, padding, dilation, groups):
         raise NotImplementedError(
@@ -483,11 +486,14 @@ def conv3d_backward_weight(
     x = input.contiguous(memory_format=_CL3D)
     gy = grad_output.contiguous(memory_format=_CL3D)
     n, _, *in_sp = (int(v) for v in x.shape)
+    gdt = x.dtype if grad_dtype is None else grad_dtype
+    if gdt is not x.dtype and gdt is not torch.float32:
+        raise ValueError(f"grad_dtype must be the operands' dtype or torch.float32, got {grad_dtype}")
     if out is None:
-        gw = grad_weight_empty(cout, cin, k, dtype=x.dtype, device=x.device)
+        gw = grad_weight_empty(cout, cin, k, dtype=gdt, device=x.device)
     else:
         gw = out
-        why = _validate_gw_out(gw, cout, cin, tuple(k), x.dtype, x.device)
+        why = _validate_gw_out(gw, cout, cin, tuple(k), gdt, x.device)
         if why is not None:
             raise ValueError(f"out= is not usable for this problem: {why}")
     L = _lib.lib()
@@ -511,7 +517,8 @@ def conv3d_backward_weight(
                     f"got {workspace.numel()} of {workspace.dtype}"
                 )
             ws, ws_bytes = workspace, have
+        flags = _flags(force_generic) | (_lib.SFH_FLAG_GRAD_FP32 if gdt is not x.dtype else 0)
         rc = L.sfh_conv3d_wgrad(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(ws), ws_bytes,
-                                _flags(force_generic), _lib.stream_ptr(x.device))
+                                flags, _lib.stream_ptr(x.device))
     _lib.check(rc, "conv3d_backward_weight")
     return gw

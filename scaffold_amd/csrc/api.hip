@@ -401,19 +401,20 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (x == nullptr || gy == nullptr || gw == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad: null tensor");
   hipStream_t st = (hipStream_t)stream;
+  const int gw_dtype = (flags & SFH_FLAG_GRAD_FP32) ? SFH_FP32 : dtype;
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_mfma(*p, dtype, out)) {
     const WgradArgs a = wgrad_args(*p, out);
     const size_t need = mfma_wgrad_workspace_bytes(a);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
-    return mfma_wgrad(a, dtype, x, gy, gw, workspace, st);
+    return mfma_wgrad(a, dtype, x, gy, gw, gw_dtype, workspace, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_patch(*p, dtype, out)) {
     const PatchArgs a = patch_args(*p, out);
     const size_t need = patch_reduce_workspace_bytes(a);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
-    return patch_reduce(a, dtype, gy, x, gw, workspace, st);
+    return patch_reduce(a, dtype, gy, x, gw, gw_dtype, workspace, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
     ThinArgs t;
@@ -422,9 +423,12 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
       const size_t need = thin_reduce_workspace_bytes(t);
       if (workspace == nullptr || workspace_bytes < need)
         return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
-      return thin_is_x ? thin_reduce(t, dtype, x, gy, gw, workspace, st) : thin_reduce(t, dtype, gy, x, gw, workspace, st);
+      return thin_is_x ? thin_reduce(t, dtype, x, gy, gw, gw_dtype, workspace, st)
+                       : thin_reduce(t, dtype, gy, x, gw, gw_dtype, workspace, st);
     }
   }
+  if (gw_dtype != dtype)
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad: the untiled kernel writes the gradient in the operands' dtype only");
   DirectConvArgs a{};
   a.n = p->n; a.cin = p->cin; a.id = p->in_d; a.ih = p->in_h; a.iw = p->in_w;
   a.cout = p->cout; a.od = out[0]; a.oh = out[1]; a.ow = out[2];

@@ -284,7 +284,7 @@ ReducePlan reduce_plan(const PatchArgs& a) {
 }
 
 template <typename T>
-int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* g, void* ws, hipStream_t st) {
+int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st) {
   const ReducePlan p = reduce_plan(a);
   const int64_t total = small_voxels(a);
   const dim3 grid((unsigned)p.splits, (unsigned)(a.csmall / kSmallTile), (unsigned)(a.cbig / 32));
@@ -292,7 +292,7 @@ int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* 
                      p.per_split);
   if (int rc = check_launch("patch_reduce_kernel")) return rc;
   const int64_t nelem = (int64_t)a.csmall * kTaps * a.cbig;
-  return sum_slices(__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16, (const float*)ws, g, nelem, p.splits, st);
+  return sum_slices(g_dtype, (const float*)ws, g, nelem, p.splits, st);
 }
 
 bool geometry_ok(const PatchArgs& a, int dtype) {
@@ -330,9 +330,9 @@ size_t patch_reduce_workspace_bytes(const PatchArgs& a) {
   return (size_t)reduce_plan(a).splits * a.csmall * kTaps * a.cbig * sizeof(float);
 }
 
-int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, void* ws, hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_reduce<bf16_t>(a, small, big, g, ws, st);
-  return launch_reduce<fp16_t>(a, small, big, g, ws, st);
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_reduce<bf16_t>(a, small, big, g, g_dtype, ws, st);
+  return launch_reduce<fp16_t>(a, small, big, g, g_dtype, ws, st);
 }
 
 }  // namespace sfh

@@ -25,6 +25,6 @@ int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* 
 int patch_reduce_splits(const PatchArgs& a);
 size_t patch_reduce_workspace_bytes(const PatchArgs& a);
 // g: dense [csmall][8][cbig] in the element type, from fp32 partial slices in ws summed in split order
-int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, void* ws, hipStream_t st);
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st);
 
 }  // namespace sfh

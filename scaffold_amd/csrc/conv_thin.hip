@@ -381,15 +381,14 @@ int launch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const v
 }
 
 template <typename T, int K, int J>
-int launch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, void* ws, hipStream_t st) {
+int launch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
   const int64_t total = (int64_t)a.n * a.od * a.oh * a.ow;
   const int nsplit = thin_reduce_splits(a);
   const int64_t per = cdiv(total, nsplit);
   hipLaunchKernelGGL((thin_reduce_kernel<T, K, J>), dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide,
                      (float*)ws, total, per);
   if (int rc = check_launch("thin_reduce_kernel")) return rc;
-  const int dtype = sizeof(T) == 4 ? SFH_FP32 : (__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16);
-  return sum_slices(dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+  return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
 }
 
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
@@ -413,7 +412,7 @@ int dispatch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const
   return launch_thin_out<T, 32>(a, wide, wt, bias, out, st);
 }
 template <typename T>
-int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, void* ws, hipStream_t st) {
+int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
   if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
     const int nsplit = thin_reduce_splits(a);
     const int ntiles = (int)stem_tiles(a);
@@ -421,14 +420,13 @@ int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void*
     hipLaunchKernelGGL(stem_wgrad_kernel<T>, dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws,
                        (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW), ntiles, per);
     if (int rc = check_launch("stem_wgrad_kernel")) return rc;
-    const int dtype = sizeof(T) == 4 ? SFH_FP32 : (__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16);
-    return sum_slices(dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+    return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
   }
-  if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, ws, st);
-  if (a.K == 2) return launch_reduce<T, 2, 8>(a, thin, wide, gw, ws, st);
-  if (a.J <= 4) return launch_reduce<T, 0, 4>(a, thin, wide, gw, ws, st);
-  if (a.J <= 16) return launch_reduce<T, 0, 16>(a, thin, wide, gw, ws, st);
-  return launch_reduce<T, 0, 32>(a, thin, wide, gw, ws, st);
+  if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, gw_dtype, ws, st);
+  if (a.K == 2) return launch_reduce<T, 2, 8>(a, thin, wide, gw, gw_dtype, ws, st);
+  if (a.J <= 4) return launch_reduce<T, 0, 4>(a, thin, wide, gw, gw_dtype, ws, st);
+  if (a.J <= 16) return launch_reduce<T, 0, 16>(a, thin, wide, gw, gw_dtype, ws, st);
+  return launch_reduce<T, 0, 32>(a, thin, wide, gw, gw_dtype, ws, st);
 }
 
 }  // namespace
@@ -464,8 +462,8 @@ int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt
 int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st) {
   SFH_THIN_BY_DTYPE(dispatch_thin_out, a, wide, wt, bias, out, st)
 }
-int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, void* ws, hipStream_t st) {
-  SFH_THIN_BY_DTYPE(dispatch_reduce, a, thin, wide, gw, ws, st)
+int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
+  SFH_THIN_BY_DTYPE(dispatch_reduce, a, thin, wide, gw, gw_dtype, ws, st)
 }
 
 }  // namespace sfh

@@ -29,6 +29,6 @@ int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, con
 // G[j][c] = sum_v s_j(v) * wide[v][c], through fp32 partial slices in `ws`
 int thin_reduce_splits(const ThinArgs& a);
 size_t thin_reduce_workspace_bytes(const ThinArgs& a);
-int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, void* ws, hipStream_t st);
+int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st);
 
 }  // namespace sfh

@@ -427,7 +427,7 @@ int launch_tile(const WgradArgs& a, const Plan& p, const void* x, const void* gy
 }
 
 template <typename T>
-int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, void* workspace, hipStream_t st) {
+int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace, hipStream_t st) {
   const Plan p = make_plan(a);
   float* ws = (float*)workspace;
   int rc;
@@ -436,7 +436,7 @@ int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, vo
   else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st);
   if (rc != SFH_OK) return rc;
   const int64_t nelem = (int64_t)a.cout * 27 * a.cin;
-  return sum_slices(__is_same(T, bf16_t) ? SFH_BF16 : SFH_FP16, ws, gw, nelem, p.splits, st);
+  return sum_slices(gw_dtype, ws, gw, nelem, p.splits, st);
 }
 
 }  // namespace
@@ -461,9 +461,10 @@ size_t mfma_wgrad_workspace_bytes(const WgradArgs& a) {
   return align_up((size_t)p.splits * a.cout * 27 * a.cin * sizeof(float), 256);
 }
 
-int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, void* workspace, hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, gy, gw, workspace, st);
-  return launch_typed<fp16_t>(a, x, gy, gw, workspace, st);
+int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace,
+               hipStream_t st) {
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, gy, gw, gw_dtype, workspace, st);
+  return launch_typed<fp16_t>(a, x, gy, gw, gw_dtype, workspace, st);
 }
 
 }  // namespace sfh

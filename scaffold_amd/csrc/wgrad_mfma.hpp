@@ -14,6 +14,8 @@ bool mfma_wgrad_supported(const WgradArgs& a, int dtype);
 // Number of fp32 partial slices [Cout][27][Cin]; a pure function of the shape.
 int mfma_wgrad_splits(const WgradArgs& a);
 size_t mfma_wgrad_workspace_bytes(const WgradArgs& a);
-int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, void* workspace, hipStream_t st);
+// gw is written in gw_dtype (the operands' dtype, or SFH_FP32 for a full-precision gradient).
+int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace,
+               hipStream_t st);
 
 }  // namespace sfh

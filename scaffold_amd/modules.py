@@ -38,7 +38,7 @@ from . import conv3d as _c3
 from . import groupnorm as _gn
 from . import transposed as _ct
 
-__all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand"]
+__all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand", "compute_copy"]
 
 _CL3D = torch.channels_last_3d
 
@@ -60,49 +60,88 @@ def cast_operand(tensor: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
     return tensor.to(dtype)
 
 
+def compute_copy(param: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
+    """A current half-precision copy of an fp32 parameter kept by the optimizer (``FusedClipAdam(shadow_dtype=...)``
+    refreshes it inside its update kernel), or ``None``.  It is used only while the parameter has not been written
+    by anything else since the copy was made (torch's version counter), so a stale copy is never read."""
+    if param is None or dtype is None or param.dtype is not torch.float32:
+        return None
+    copy = getattr(param, "_sfh_shadow", None)
+    if copy is None or copy.dtype is not dtype or getattr(param, "_sfh_shadow_version", None) != param._version:
+        return None
+    return copy
+
+
+def _fp32_weight_grad(fn, *args, **kwargs):
+    """Weight gradient straight in fp32 where the tiled kernels serve the shape, else in the operands' dtype and
+    widened afterwards (what autocast's cast node would have done)."""
+    try:
+        return fn(*args, grad_dtype=torch.float32, **kwargs)
+    except NotImplementedError:
+        return fn(*args, **kwargs).to(torch.float32)
+
+
 class _Conv3dFn(torch.autograd.Function):
     """The caller (``FastConv3d.forward``) has passed the gate for all three directions with these very operands, and
     autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, padding, dilation):
-        y = _c3.conv3d_forward(x, weight, bias, stride, padding, dilation, 1, _checked=True)
-        ctx.save_for_backward(x, weight)
-        ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype)
+    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None):
+        # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
+        # given, the kernels read those and the gradients are produced in the masters' dtype directly
+        wc = weight if weight_compute is None else weight_compute
+        bc = bias if bias_compute is None else bias_compute
+        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, _checked=True)
+        ctx.save_for_backward(x, wc)
+        ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
+                         weight.dtype is not wc.dtype)
         return y
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
         x, weight = ctx.saved_tensors
-        stride, padding, dilation, has_bias, bias_dtype = ctx.conv_args
+        stride, padding, dilation, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1, _checked=True) if needs_x else None
-        grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True) if needs_w else None
+        grad_w = None
+        if needs_w:
+            if master:
+                grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight, x, weight.shape, grad_output, stride, padding, dilation, 1,
+                                           _checked=True)
+            else:
+                grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, stride):
-        y = _ct.conv_transpose3d_forward(x, weight, bias, stride, 0, 0, 1, 1)
-        ctx.save_for_backward(x, weight)
-        ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype)
+    def forward(ctx, x, weight, bias, stride, weight_compute=None, bias_compute=None):
+        wc = weight if weight_compute is None else weight_compute
+        bc = bias if bias_compute is None else bias_compute
+        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1)
+        ctx.save_for_backward(x, wc)
+        ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype, weight.dtype is not wc.dtype)
         return y
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
         x, weight = ctx.saved_tensors
-        stride, has_bias, bias_dtype = ctx.conv_args
+        stride, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1) if needs_x else None
-        grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1) if needs_w else None
+        grad_w = None
+        if needs_w:
+            if master:
+                grad_w = _fp32_weight_grad(_ct.conv_transpose3d_backward_weight, x, weight.shape, grad_output, stride, 0, 0, 1, 1)
+            else:
+                grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None
+        return grad_x, grad_w, grad_b, None, None, None
 
 
 def _wants_grad(*tensors) -> bool:
@@ -120,8 +159,12 @@ class FastConv3d(nn.Conv3d):
             raise NotImplementedError(f"FastConv3d: padding_mode={self.padding_mode!r} padding={self.padding!r}")
         dt = autocast_dtype(x)
         x = cast_operand(x, dt)
-        w = cast_operand(self.weight, dt)
-        b = cast_operand(self.bias, dt)
+        # under autocast, an up-to-date half-precision copy kept by the optimizer replaces the per-call cast
+        wc = compute_copy(self.weight, dt)
+        bc = compute_copy(self.bias, dt) if wc is not None else None
+        master = wc is not None and (self.bias is None or bc is not None)
+        w = wc if master else cast_operand(self.weight, dt)
+        b = bc if master else cast_operand(self.bias, dt)
         padding = tuple(self.padding)
         if self.shard_halo and padding[0] > 0:
             # (N, C, D, H, W): extend D by the halo the neighbours would have sent
@@ -136,6 +179,8 @@ class FastConv3d(nn.Conv3d):
                 f"FastConv3d: not served: x={tuple(x.shape)}/{x.dtype} on {x.device}, weight={tuple(w.shape)}/{w.dtype}, "
                 f"stride={self.stride} padding={padding} dilation={self.dilation} groups={self.groups}"
             )
+        if master:
+            return _Conv3dFn.apply(x, self.weight, self.bias, tuple(self.stride), padding, tuple(self.dilation), w, b)
         return _Conv3dFn.apply(x, w, b, tuple(self.stride), padding, tuple(self.dilation))
 
 
@@ -147,8 +192,11 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
             raise NotImplementedError("FastConvTranspose3d: output_size is not supported")
         dt = autocast_dtype(x)
         x = cast_operand(x, dt)
-        w = cast_operand(self.weight, dt)
-        b = cast_operand(self.bias, dt)
+        wc = compute_copy(self.weight, dt)
+        bc = compute_copy(self.bias, dt) if wc is not None else None
+        master = wc is not None and (self.bias is None or bc is not None)
+        w = wc if master else cast_operand(self.weight, dt)
+        b = bc if master else cast_operand(self.bias, dt)
         x = x.contiguous(memory_format=_CL3D)
         gate = _ct.is_supported_transposed_all if _wants_grad(x, w, b) else _ct.is_supported_transposed
         if not gate(x, w, b, self.stride, self.padding, self.output_padding, self.dilation, self.groups):
@@ -157,6 +205,8 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
                 f"stride={self.stride} padding={self.padding} output_padding={self.output_padding} "
                 f"dilation={self.dilation} groups={self.groups}"
             )
+        if master:
+            return _ConvTranspose3dFn.apply(x, self.weight, self.bias, tuple(self.stride), w, b)
         return _ConvTranspose3dFn.apply(x, w, b, tuple(self.stride))
 
 

@@ -53,9 +53,30 @@ class FusedClipAdam(torch.optim.Optimizer):
         self.max_norm = max_norm
         self.shadow_dtype = shadow_dtype
         self.shadow = {}
+        if shadow_dtype is not None:
+            self.refresh_shadows()
         self.grad_norm = None
         self._slots = None
         self._plans = {}
+
+    @torch.no_grad()
+    def refresh_shadows(self):
+        """(Re)makes the half-precision copy of every parameter and publishes it on the parameter, where
+        ``FastConv3d`` / ``FastConvTranspose3d`` find it under autocast. Needed only after the parameters were
+        changed behind torch's back (``.data`` writes); ordinary in-place updates are noticed through the version
+        counter and simply fall back to the per-call cast until the next ``step()``."""
+        if self.shadow_dtype is None:
+            return
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.dtype is not torch.float32 or not p.is_cuda:
+                    continue
+                sh = self.shadow.get(p)
+                if sh is None:
+                    sh = self.shadow[p] = torch.empty_like(p, dtype=self.shadow_dtype, memory_format=torch.preserve_format)
+                sh.copy_(p)
+                p._sfh_shadow = sh
+                p._sfh_shadow_version = p._version
 
     @staticmethod
     def _dense(t):
@@ -159,6 +180,10 @@ class FusedClipAdam(torch.optim.Optimizer):
                 rc = L.sfh_adam_clip_step(ctypes.byref(desc), gpl["n"], gpl["p"], g_arr, gpl["m"], gpl["v"], gpl["shadow"], gpl["numel"],
                                           _lib.ptr(self._slots), nslots, _lib.ptr(step), _lib.ptr(self.grad_norm), stream)
                 _lib.check(rc, "FusedClipAdam (update)")
+            if self.shadow_dtype is not None:
+                for p in params:  # the kernel wrote parameter and copy together
+                    p._sfh_shadow = self.shadow[p]
+                    p._sfh_shadow_version = p._version
         return loss
 
     def load_state_dict(self, state_dict):

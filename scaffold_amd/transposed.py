@@ -242,6 +242,7 @@ def conv_transpose3d_backward_weight(
     out: Optional[torch.Tensor] = None,
     deterministic: bool = True,
     force_generic: bool = False,
+    grad_dtype: Optional[torch.dtype] = None,
 ) -> torch.Tensor:
     """Weight gradient ``(Cin, Cout, k, k, k)``, ``channels_last_3d``: the ordinary weight gradient of
     the stride-``k`` convolution whose input is ``grad_output`` and whose output gradient is ``x``."""
@@ -254,4 +255,4 @@ def conv_transpose3d_backward_weight(
         )
     ws = tuple(int(v) for v in weight_shape)
     return conv3d_backward_weight(grad_output, ws, x, ws[2:], 0, 1, 1, config=config, workspace=workspace, out=out,
-                                  deterministic=deterministic, force_generic=force_generic)
+                                  deterministic=deterministic, force_generic=force_generic, grad_dtype=grad_dtype)

@@ -210,3 +210,107 @@ def test_step_captured_in_a_graph_replays_to_the_eager_result(device):
         torch.cuda.synchronize()
         torch.randn(1 << 14, device=device).sum().item()
         assert all(torch.equal(p, q) for p, q in zip(eager, graphed)), step
+
+
+# ---- half-precision parameter copies feeding the modules, fp32 weight gradients ---------------------------------
+@pytest.mark.parametrize("shape", [
+    # cin, cout, spatial, kernel, stride, padding     (tiled MFMA, 2x2x2 stride-2, thin head, thin stem)
+    (32, 32, (8, 16, 32), 3, 1, 1),
+    (64, 128, (4, 8, 8), 3, 1, 1),
+    (32, 64, (8, 8, 16), 2, 2, 0),
+    (32, 11, (8, 8, 16), 1, 1, 0),
+    (1, 32, (8, 16, 32), 3, 1, 1),
+])
+def test_fp32_weight_gradient_is_the_unrounded_sum(device, shape):
+    """grad_dtype=float32 stores the fp32 slice sum the 16-bit path rounds: rounding it must give the 16-bit result
+    bit for bit."""
+    cin, cout, sp, k, stride, pad = shape
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn((1, cin, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    osp = tuple((s + 2 * pad - k) // stride + 1 for s in sp)
+    gy = torch.randn((1, cout, *osp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    wshape = (cout, cin, k, k, k)
+    g16 = sa.conv3d_backward_weight(x, wshape, gy, stride, pad, 1)
+    g32 = sa.conv3d_backward_weight(x, wshape, gy, stride, pad, 1, grad_dtype=torch.float32)
+    assert g32.dtype is torch.float32 and g32.stride() == g16.stride()
+    assert torch.equal(g32.to(torch.bfloat16), g16)
+    assert not torch.equal(g32, g16.float())  # it really carries more bits
+
+
+def test_fp32_weight_gradient_refused_where_only_the_untiled_kernel_applies(device):
+    x = torch.randn((1, 5, 6, 6, 6), device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    gy = torch.randn((1, 7, 6, 6, 6), device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    with pytest.raises(NotImplementedError):
+        sa.conv3d_backward_weight(x, (7, 5, 3, 3, 3), gy, 1, 1, 1, grad_dtype=torch.float32)
+    with pytest.raises(ValueError):
+        sa.conv3d_backward_weight(x, (7, 5, 3, 3, 3), gy, 1, 1, 1, grad_dtype=torch.float16)
+
+
+def _tiny_unet(device):
+    torch.manual_seed(31)
+    model = sa.UNet(1, 5, layers=2, base_width=32).to(device).to(memory_format=CL)
+    g = torch.Generator().manual_seed(32)
+    x = (torch.rand((1, 1, 16, 16, 32), generator=g) < 0.05).float().contiguous(memory_format=CL).to(device)
+    lab = torch.randint(0, 5, (1, 16, 16, 32), generator=g).to(device)
+    return model, x, lab
+
+
+def _train(model, opt, x, lab, steps):
+    losses, grads = [], None
+    for _ in range(steps):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(x)
+        loss = sa.ce_dice_loss(logits, lab)
+        loss.backward()
+        if grads is None:
+            grads = {k: p.grad.clone() for k, p in model.named_parameters()}
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        losses.append(loss.item())
+    return losses, grads
+
+
+def test_modules_read_the_optimizers_copies_and_get_fp32_gradients(device):
+    """Same model trained with and without the optimizer's bf16 copies: the first forward is bitwise the same (the
+    copy is the cast autocast would make), every parameter gradient is fp32 and equals the cast path's up to the one
+    bf16 rounding that path applies, and training stays together."""
+    plain, x, lab = _tiny_unet(device)
+    fused, _, _ = _tiny_unet(device)
+    opt_p = sa.FusedClipAdam(plain.parameters(), lr=1e-3, max_norm=1.0)
+    opt_f = sa.FusedClipAdam(fused.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+    from scaffold_amd.modules import compute_copy
+    convs = [m for m in fused.modules() if isinstance(m, (sa.FastConv3d, sa.FastConvTranspose3d))]
+    assert convs and all(compute_copy(m.weight, torch.bfloat16) is not None for m in convs)
+    lp, gp = _train(plain, opt_p, x, lab, 4)
+    lf, gf = _train(fused, opt_f, x, lab, 4)
+    assert lp[0] == lf[0]
+    for k in gp:
+        assert gf[k].dtype is torch.float32
+        # conv weights and biases: the cast path rounded to bf16 once; GroupNorm parameters: fp32 in both
+        assert torch.equal(gf[k].to(torch.bfloat16), gp[k].to(torch.bfloat16)) or \
+            torch.allclose(gf[k], gp[k], rtol=1e-5, atol=1e-7), k
+    assert all(abs(a - b) <= 2e-3 * abs(a) for a, b in zip(lp, lf))
+    # after the steps the copies are still current and equal to the rounded parameters
+    for m in convs:
+        c = compute_copy(m.weight, torch.bfloat16)
+        assert c is not None and torch.equal(c, m.weight.detach().to(torch.bfloat16))
+
+
+def test_a_parameter_written_by_someone_else_is_not_read_through_a_stale_copy(device):
+    model, x, lab = _tiny_unet(device)
+    opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+    from scaffold_amd.modules import compute_copy
+    conv = next(m for m in model.modules() if isinstance(m, sa.FastConv3d))
+    assert compute_copy(conv.weight, torch.bfloat16) is not None
+    with torch.no_grad():
+        conv.weight.mul_(0.5)  # version counter moves
+    assert compute_copy(conv.weight, torch.bfloat16) is None
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        y_after = model(x)
+    ref, _, _ = _tiny_unet(device)
+    with torch.no_grad():
+        next(m for m in ref.modules() if isinstance(m, sa.FastConv3d)).weight.mul_(0.5)
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        assert torch.equal(y_after, ref(x))
+    opt.refresh_shadows()
+    assert compute_copy(conv.weight, torch.bfloat16) is not None
