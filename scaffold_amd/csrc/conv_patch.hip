@@ -274,7 +274,7 @@ ReducePlan reduce_plan(const PatchArgs& a) {
   const int64_t total = small_voxels(a);
   const int64_t tiles = (int64_t)(a.csmall / kSmallTile) * (a.cbig / 32);
   const int64_t rounds = cdiv(total, kVx);
-  int64_t splits = cdiv(4 * kComputeUnits, tiles);
+  int64_t splits = cdiv(2 * kComputeUnits, tiles);  // every split writes a whole fp32 slice: more would be write-bound
   if (splits > rounds) splits = rounds;
   if (splits < 1) splits = 1;
   ReducePlan p;

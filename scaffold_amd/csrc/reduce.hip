@@ -2,6 +2,7 @@
 // channels-last tensor (the bias gradient, ScaFFold/unet/conv3d.py:1231,1786). No atomics: every
 // partial has a fixed slot and every sum a fixed order, so a call gives the same bits every time.
 #include "reduce.hpp"
+#include "vec_io.hpp"
 
 namespace sfh {
 namespace {
@@ -34,8 +35,18 @@ __global__ void __launch_bounds__(kBlock) sum_slices_grouped(const float* __rest
   const int el = threadIdx.x & 15, sl = threadIdx.x >> 4;
   const int64_t e = (int64_t)blockIdx.x * 16 + el;
   float s = 0.f;
-  if (e < nelem)
-    for (int sp = sl; sp < splits; sp += 16) s += part[(int64_t)sp * nelem + e];
+  if (e < nelem) {
+    // eight loads in flight per thread; the additions keep the slice order
+    int sp = sl;
+    for (; sp + 7 * 16 < splits; sp += 8 * 16) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] = part[(int64_t)(sp + 16 * k) * nelem + e];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) s += v[k];
+    }
+    for (; sp < splits; sp += 16) s += part[(int64_t)sp * nelem + e];
+  }
   buf[sl][el] = s;
   __syncthreads();
   if (sl == 0 && e < nelem) {
@@ -114,16 +125,76 @@ __global__ void __launch_bounds__(kBlock) channel_partial(const T* __restrict__ 
   }
 }
 
-int bias_blocks(int64_t rows) {
-  int64_t n = cdiv(rows, 1024);
-  if (n > kComputeUnits * 4) n = kComputeUnits * 4;
+// The same sums with 16-byte loads: thread = (row slot, vector of V channels), C a multiple of V, C / V <= 256.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) channel_partial_vec(const T* __restrict__ g, float* __restrict__ part, int64_t rows, int C,
+                                                              int64_t rows_per_block) {
+  constexpr int V = VecOf<T>::N;
+  extern __shared__ float vbuf[];  // V * kBlock
+  const int tpr = C / V;
+  const int rpp = kBlock / tpr;
+  const int tid = threadIdx.x;
+  const int r = tid / tpr, cv = tid - r * tpr;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_block;
+  int64_t end = begin + rows_per_block;
+  if (end > rows) end = rows;
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.f;
+  if (r < rpp) {
+    const T* p = g + cv * V;
+    int64_t row = begin + r;
+    for (; row + 3 * (int64_t)rpp < end; row += 4 * (int64_t)rpp) {
+      float f0[V], f1[V], f2[V], f3[V];
+      Ld<T, V>::run(p + row * C, f0);
+      Ld<T, V>::run(p + (row + rpp) * C, f1);
+      Ld<T, V>::run(p + (row + 2 * rpp) * C, f2);
+      Ld<T, V>::run(p + (row + 3 * rpp) * C, f3);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += (f0[e] + f1[e]) + (f2[e] + f3[e]);
+    }
+    for (; row < end; row += rpp) {
+      float f0[V];
+      Ld<T, V>::run(p + row * C, f0);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += f0[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) vbuf[e * kBlock + tid] = r < rpp ? acc[e] : 0.f;
+  __syncthreads();
+  for (int c = tid; c < C; c += kBlock) {
+    const int v = c / V, e = c - v * V;
+    float t = 0.f;
+    for (int i = 0; i < rpp; ++i) t += vbuf[e * kBlock + i * tpr + v];
+    part[(int64_t)blockIdx.x * C + c] = t;
+  }
+}
+
+template <typename T>
+bool bias_vector_form(const void* g, int C) {
+  constexpr int V = VecOf<T>::N;
+  return C % V == 0 && C / V <= kBlock && (reinterpret_cast<uintptr_t>(g) & 15) == 0;
+}
+
+// Workgroups of the partial pass: at most 1024, each at least one pass of rows (a pass is 4 KiB in the vector form).
+int bias_blocks(int64_t rows, int C) {
+  int64_t per = cdiv(rows, 1024);
+  const int64_t pass = C >= 8 && C <= 2048 ? (2048 / C < 1 ? 1 : 2048 / C) : 1;
+  if (per < pass) per = pass;
+  const int64_t n = cdiv(rows, per);
   return (int)(n < 1 ? 1 : n);
 }
 
 template <typename T>
 int launch_bias(const void* g, int64_t rows, int C, float* ws, hipStream_t st) {
-  const int nblk = bias_blocks(rows);
+  const int nblk = bias_blocks(rows, C);
   const int64_t per = cdiv(rows, nblk);
+  if (bias_vector_form<T>(g, C)) {
+    hipLaunchKernelGGL(channel_partial_vec<T>, dim3((unsigned)nblk), dim3(kBlock), VecOf<T>::N * kBlock * sizeof(float), st,
+                       (const T*)g, ws, rows, C, per);
+    return check_launch("channel_partial_vec");
+  }
   hipLaunchKernelGGL(channel_partial<T>, dim3((unsigned)nblk, (unsigned)cdiv(C, kBlock)), dim3(kBlock), 0, st, (const T*)g, ws, rows, C,
                      per);
   return check_launch("channel_partial");
@@ -156,7 +227,7 @@ int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, i
 }
 
 size_t bias_grad_workspace_bytes(int64_t rows, int channels) {
-  return (size_t)bias_blocks(rows) * channels * sizeof(float);
+  return (size_t)bias_blocks(rows, channels) * channels * sizeof(float);
 }
 
 int bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int channels, void* gb, void* ws, hipStream_t st) {
@@ -167,7 +238,7 @@ int bias_grad(int dtype, int out_dtype, const void* g, int64_t rows, int channel
     default: rc = launch_bias<float>(g, rows, channels, (float*)ws, st); break;
   }
   if (rc != SFH_OK) return rc;
-  return sum_slices(out_dtype, (const float*)ws, gb, channels, bias_blocks(rows), st);
+  return sum_slices(out_dtype, (const float*)ws, gb, channels, bias_blocks(rows, channels), st);
 }
 
 }  // namespace sfh
