@@ -163,6 +163,19 @@ def bench_groupnorm(args, device):
     }
 
 
+def gemm_reference(device):
+    """What the vendor's tuned dense GEMM (hipBLASLt through torch.matmul, 8192^3 bf16) reaches on this box in this
+    run: the practical ceiling of the matrix pipe under real data and the chip's power management, next to the
+    nominal 2.5 PFLOP/s the roofline fraction is quoted against."""
+    n = 8192
+    g = torch.Generator(device=device).manual_seed(4000)
+    a = torch.randn((n, n), generator=g, device=device, dtype=torch.bfloat16)
+    b = torch.randn((n, n), generator=g, device=device, dtype=torch.bfloat16)
+    ms = event_time_ms(lambda: torch.matmul(a, b), 20, warmup=5)
+    tflops = 2 * n ** 3 / (ms * 1e-3) / 1e12
+    return {"workload": "torch.matmul 8192x8192x8192 bf16", "ms": ms, "tflops": tflops, "frac_of_mfma_peak": tflops / MFMA_PEAK_TFLOPS}
+
+
 def copy_calibration(device, mib=256, reps=4):
     """Runs the library's plain copy kernel on a buffer of known size, so that a counter run of this script
     also holds FETCH_SIZE / WRITE_SIZE for a launch whose HBM traffic is known exactly."""
@@ -323,6 +336,10 @@ def main():
         return
     conv = bench_conv(args, device)
     details = {"conv": conv}
+    try:
+        details["vendor_gemm_reference"] = gemm_reference(device)
+    except Exception as exc:  # report, do not hide
+        details["vendor_gemm_reference"] = {"error": repr(exc)}
     if args.copy_calibration:
         details["copy_calibration"] = copy_calibration(device)
     try:
