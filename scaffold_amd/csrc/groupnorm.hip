@@ -10,8 +10,11 @@
 // (ScaFFold/unet/triton_group_norm.py:148-165,594-694).
 //
 // Launch chain (no atomics, partials at fixed scratch slots, fixed-order sums):
-//   forward : gn_stats_partial -> gn_stats_finalize -> gn_normalize          (3*B bytes streamed)
-//   backward: gn_bwd_partial   -> gn_bwd_finalize   -> gn_dx                 (5*B bytes streamed)
+//   forward : gn_stats_partial -> [gn_stats_finalize] -> gn_normalize        (3*B bytes streamed)
+//   backward: gn_bwd_partial   -> [gn_bwd_finalize]   -> gn_dx               (5*B bytes streamed)
+// The finalize launches run only when a sample has more than 16 Ki floats of group-level partials; below that the
+// consumer kernel folds the partials itself (every workgroup the same way, 64 KiB from L2 at most), which is
+// cheaper than a launch of its own.
 // The fused ReLU is spelled `y <= 0 ? 0 : y` and the backward gate `pre <= 0 ? 0 : dy` so that
 // NaN propagates exactly as F.relu / threshold_backward do (triton_group_norm.py:176-198), and
 // the gate is evaluated on the pre-activation recomputed with the forward's own expression.
@@ -240,24 +243,98 @@ __global__ void __launch_bounds__(64) gn_stats_finalize(const float* __restrict_
   }
 }
 
+// Sums the split partials of one sample inside a consumer kernel, the same way in every workgroup that calls it (so
+// all of them get the same bits). `rows` points at the sample's slots [split][quantity][group], 2 * G floats per
+// split, nsplit * 2 * G <= kFoldFloats in total and 2 * G a power of two <= 64. Thread t reads the 16-byte pieces
+// t, t + 256, ... (all loads in flight at once) and keeps one running sum per float of its piece's column; the
+// threads that share a column are then added in thread order through LDS. Thread c < 2 * G ends up holding the
+// total of column c (quantity c / G, group c % G) and passes it to emit(c, total).
+constexpr int kFoldFloats = 16384;
+
+__device__ __forceinline__ bool fold_in_consumer(int G, int nsplit) {
+  const int cols = 2 * G;
+  return cols >= 4 && cols <= 64 && (cols & (cols - 1)) == 0 && (int64_t)nsplit * cols <= kFoldFloats;
+}
+inline bool fold_in_consumer_host(int G, int nsplit) {
+  const int cols = 2 * G;
+  return cols >= 4 && cols <= 64 && (cols & (cols - 1)) == 0 && (int64_t)nsplit * cols <= kFoldFloats;
+}
+
+template <typename Emit>
+__device__ __forceinline__ void fold_split_partials(const float* __restrict__ rows, int G, int nsplit, float* lds /* 4 * kBlock */,
+                                                    Emit emit) {
+  const int tid = threadIdx.x;
+  const int cols = 2 * G, total = nsplit * cols;
+  constexpr int NB = kFoldFloats / (4 * kBlock);  // pieces per thread at most
+  float4 v[NB];
+#pragma unroll
+  for (int k = 0; k < NB; ++k) {
+    const int i = (tid + k * kBlock) * 4;
+    v[k] = i < total ? *reinterpret_cast<const float4*>(rows + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  // kBlock * 4 is a multiple of cols, so every piece of a thread lies in the same four columns
+  float4 s = v[0];
+#pragma unroll
+  for (int k = 1; k < NB; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+  *reinterpret_cast<float4*>(lds + tid * 4) = s;
+  __syncthreads();
+  if (tid < cols) {
+    // column tid appears in the pieces of threads tid / 4 + j * (cols / 4), at float tid % 4
+    const int per = cols / 4, nthr = kBlock / per;
+    float t = 0.f;
+    for (int j = 0; j < nthr; ++j) t += lds[(tid / 4 + j * per) * 4 + (tid & 3)];
+    emit(tid, t);
+  }
+}
+
 // ---- forward: normalise + affine (+ReLU) (vector path) ------------------------------------
+// When the sample's split partials are few (fold_in_consumer), every workgroup derives mean and rstd from them itself
+// (mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps)): 32 KiB from L2 cost less than a launch of their
+// own, and the first workgroup of a sample writes them out for the backward pass. Otherwise gn_stats_finalize has run.
 template <typename T, typename TO>
-__global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, TO* __restrict__ y, const float* __restrict__ mean,
-                                                       const float* __restrict__ rstd, const void* __restrict__ gamma,
+__global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, TO* __restrict__ y, const float* __restrict__ shift,
+                                                       const float* __restrict__ part, float* __restrict__ mean,
+                                                       float* __restrict__ rstd, const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
-                                                       int tpr, int rpp, int64_t rows_per_split, int relu) {
+                                                       int tpr, int rpp, int nsplit, int64_t rows_per_split, float m, float eps,
+                                                       int relu) {
   constexpr int V = VecOf<T>::N;
+  extern __shared__ float gstat[];  // sums[2 G] | mean[G] | rstd[G] | fold scratch (4 * kBlock)
   const int tid = threadIdx.x;
   const int n = blockIdx.y;
   const int cg = C / G;
   const int r = tid / tpr, cv = tid - r * tpr;
+  float* g_mean = gstat + 2 * G;
+  float* g_rstd = gstat + 3 * G;
+  if (fold_in_consumer(G, nsplit)) {
+    fold_split_partials(part + (int64_t)n * nsplit * 2 * G, G, nsplit, gstat + 4 * G, [&](int c, float t) { gstat[c] = t; });
+    __syncthreads();
+    if (tid < G) {
+      const float d = gstat[tid] / m;
+      float var = gstat[G + tid] / m - d * d;
+      var = var < 0.f ? 0.f : var;
+      const float mu_g = shift[n * G + tid] + d, rs_g = 1.f / sqrtf(var + eps);
+      g_mean[tid] = mu_g;
+      g_rstd[tid] = rs_g;
+      if (blockIdx.x == 0) {  // for the backward pass
+        mean[n * G + tid] = mu_g;
+        rstd[n * G + tid] = rs_g;
+      }
+    }
+  } else {
+    for (int g = tid; g < G; g += kBlock) {  // a finalize launch has filled mean / rstd
+      g_mean[g] = mean[n * G + g];
+      g_rstd[g] = rstd[n * G + g];
+    }
+  }
+  __syncthreads();
   if (r >= rpp) return;
   float mu[V], rs[V], ga[V], be[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = cv * V + e;
-    mu[e] = mean[n * G + c / cg];
-    rs[e] = rstd[n * G + c / cg];
+    mu[e] = g_mean[c / cg];
+    rs[e] = g_rstd[c / cg];
     ga[e] = load_param(gamma, param_dtype, c, 1.f);
     be[e] = load_param(beta, param_dtype, c, 0.f);
   }
@@ -304,8 +381,9 @@ template <typename T, typename TG>
 __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x, const TG* __restrict__ dy,
                                                          const float* __restrict__ mean, const float* __restrict__ rstd,
                                                          const void* __restrict__ gamma, const void* __restrict__ beta,
-                                                         int param_dtype, float* __restrict__ part, int64_t S, int C, int G,
-                                                         int tpr, int rpp, int nsplit, int64_t rows_per_split, int relu) {
+                                                         int param_dtype, float* __restrict__ part, float* __restrict__ gpart,
+                                                         int64_t S, int C, int G, int tpr, int rpp, int nsplit,
+                                                         int64_t rows_per_split, int relu) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float smem[];  // 2 * V * kBlock
   const int tid = threadIdx.x;
@@ -372,6 +450,20 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
   for (int i = tid; i < 2 * C; i += kBlock) {
     const int q = i / C, c = i - q * C;
     dst[i] = smem[(q * V + c % V) * kBlock + c / V];
+  }
+  // The same sums folded per group with the gamma weights (what dx needs): gpart[n][split][q][g]. Sixteen lanes share
+  // a (quantity, group) pair, lane s takes channels s, s + 16, ... of the group, then a fixed tree over the 16 lanes.
+  float* gdst = gpart + ((int64_t)n * nsplit + split) * 2 * G;
+  for (int pair = tid >> 4; pair < 2 * G; pair += kBlock >> 4) {
+    const int q = pair / G, g = pair - q * G;
+    float t = 0.f;
+    for (int cc = tid & 15; cc < cg; cc += 16) {
+      const int c = g * cg + cc;
+      t = fmaf(load_param(gamma, param_dtype, c, 1.f), smem[(q * V + c % V) * kBlock + c / V], t);
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) t += __shfl_down(t, off, 16);
+    if ((tid & 15) == 0) gdst[pair] = t;
   }
 }
 
@@ -443,18 +535,37 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_finalize(const float* __restric
 }
 
 // dx = rstd * (dy'*gamma - A - xhat*B)   (ScaFFold/unet/triton_group_norm.py:908-1043)
+// When the sample's group-level partials are few (fold_in_consumer) every workgroup derives the group coefficients
+// A = mean(dy'*gamma), B = mean(dy'*gamma*xhat) from them itself, and workgroups of sample 0 finish by summing the
+// per-channel partials of one channel each into dgamma / dbeta (samples and splits in index order): no finalize
+// launch. Otherwise gn_bwd_finalize has filled `coef` and the parameter gradients.
 template <typename T, typename TG>
 __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const TG* __restrict__ dy, T* __restrict__ dx,
                                                 const float* __restrict__ mean, const float* __restrict__ rstd,
                                                 const void* __restrict__ gamma, const void* __restrict__ beta, int param_dtype,
-                                                const float* __restrict__ coef, int64_t S, int C, int G, int tpr, int rpp,
-                                                int64_t rows_per_split, int relu) {
+                                                const float* __restrict__ coef, const float* __restrict__ part,
+                                                const float* __restrict__ gpart, float* __restrict__ dgamma,
+                                                float* __restrict__ dbeta, int N, int64_t S, int C, int G, int tpr, int rpp,
+                                                int nsplit, int64_t rows_per_split, float m, int relu) {
   constexpr int V = VecOf<T>::N;
+  extern __shared__ float gco[];  // sums[2 G] | fold scratch (4 * kBlock)
+  __shared__ float red4[4];
   const int tid = threadIdx.x;
   const int n = blockIdx.y;
   const int cg = C / G;
   const int r = tid / tpr, cv = tid - r * tpr;
-  if (r >= rpp) return;
+  const bool fused = fold_in_consumer(G, nsplit);
+  if (fused) {
+    // gpart quantity 0 = sum dy'*gamma*xhat (-> B), quantity 1 = sum dy'*gamma (-> A)
+    fold_split_partials(gpart + (int64_t)n * nsplit * 2 * G, G, nsplit, gco + 2 * G, [&](int c, float t) { gco[c] = t / m; });
+  } else {
+    for (int i = tid; i < 2 * G; i += kBlock) {
+      const int q = i / G, g = i - q * G;
+      gco[i] = coef[(n * G + g) * 2 + (1 - q)];  // coef holds (A, B) per group
+    }
+  }
+  __syncthreads();
+  if (r < rpp) {
   float mu[V], rs[V], ga[V], be[V], ca[V], cb[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
@@ -464,8 +575,8 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
     rs[e] = rstd[n * G + g];
     ga[e] = load_param(gamma, param_dtype, c, 1.f);
     be[e] = load_param(beta, param_dtype, c, 0.f);
-    ca[e] = coef[(n * G + g) * 2];
-    cb[e] = coef[(n * G + g) * 2 + 1];
+    ca[e] = gco[G + g];
+    cb[e] = gco[g];
   }
   const int64_t base = (int64_t)n * S * C + cv * V;
   const T* xs = x + base;
@@ -508,6 +619,24 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
       o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
     }
     St<T, V>::run(ds + row * C, o);
+  }
+  }
+  if (fused && n == 0 && (dgamma != nullptr || dbeta != nullptr)) {
+    const int total = N * nsplit;
+    for (int c = blockIdx.x; c < C; c += gridDim.x) {
+      float s1 = 0.f, s2 = 0.f;
+      for (int i = tid; i < total; i += kBlock) {
+        const float* p = part + (int64_t)i * 2 * C;
+        s1 += p[c];
+        s2 += p[C + c];
+      }
+      s1 = block_sum256(s1, red4);
+      s2 = block_sum256(s2, red4);
+      if (tid == 0) {
+        if (dgamma != nullptr) dgamma[c] = s1;
+        if (dbeta != nullptr) dbeta[c] = s2;
+      }
+    }
   }
 }
 
@@ -655,11 +784,14 @@ int check_desc(const sfh_groupnorm_desc* p, int x_dtype) {
 bool aligned16(const void* a) { return (reinterpret_cast<uintptr_t>(a) & 15u) == 0; }
 
 size_t fwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
-  return (size_t)p.n * p.groups + (size_t)p.n * pl.nsplit * 2 * p.groups;
+  // shift[N][G] (padded to 16 bytes so the slots can be read as float4) | part[N][nsplit][2][G]
+  return align_up((size_t)p.n * p.groups, 4) + (size_t)p.n * pl.nsplit * 2 * p.groups;
 }
 size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
-  // coef[N][G][2] | part[N][nsplit][2][C]   (scalar path: chan[N][2][C] in the part slot)
-  return (size_t)p.n * p.groups * 2 + (size_t)p.n * pl.nsplit * 2 * p.c;
+  // coef[N][G][2] | part[N][nsplit][2][C] | gpart[N][nsplit][2][G]; every section starts on 16 bytes
+  // (scalar path: chan[N][2][C] in the part slot)
+  return align_up((size_t)p.n * p.groups * 2, 4) + align_up((size_t)p.n * pl.nsplit * 2 * p.c, 4) +
+         (size_t)p.n * pl.nsplit * 2 * p.groups;
 }
 
 template <typename T, typename TO>
@@ -677,7 +809,7 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
     return check_launch("gn_scalar_normalize");
   }
   float* shift = ws;
-  float* part = ws + (size_t)p.n * G;
+  float* part = ws + align_up((size_t)p.n * G, 4);
   const size_t lds = (size_t)(2 * pl.slots * kBlock + 2 * G) * sizeof(float);
   const dim3 grid(pl.nsplit, p.n);
 #define SFH_GN_STATS(SL)                                                                                                   \
@@ -692,10 +824,12 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
 #undef SFH_GN_STATS
   if (int rc = check_launch("gn_stats_partial")) return rc;
   const float m = (float)S * (float)(C / G);
-  hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, pl.nsplit, m, p.eps);
-  if (int rc = check_launch("gn_stats_finalize")) return rc;
-  hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), 0, st, (const T*)x, (TO*)y, mean, rstd, gamma, beta,
-                     param_dtype, S, C, G, pl.tpr, pl.rpp, pl.rows_per_split, p.relu);
+  if (!fold_in_consumer_host(G, pl.nsplit)) {
+    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, pl.nsplit, m, p.eps);
+    if (int rc = check_launch("gn_stats_finalize")) return rc;
+  }
+  hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
+                     mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu);
   return check_launch("gn_normalize");
 }
 
@@ -706,7 +840,8 @@ int bwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
   float* coef = ws;
-  float* part = ws + (size_t)p.n * G * 2;
+  float* part = ws + align_up((size_t)p.n * G * 2, 4);
+  float* gpart = part + align_up((size_t)p.n * pl.nsplit * 2 * C, 4);
   if (!pl.vector) {
     hipLaunchKernelGGL((gn_scalar_bwd_sums<T, TG>), dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, (const TG*)dy, mean, rstd,
                        gamma, beta, param_dtype, part, coef, S, C, G, p.relu);
@@ -724,15 +859,18 @@ int bwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
   constexpr int V = VecOf<T>::N;
   const dim3 grid(pl.nsplit, p.n);
   hipLaunchKernelGGL((gn_bwd_partial<T, TG>), grid, dim3(kBlock), (size_t)2 * V * kBlock * sizeof(float), st, (const T*)x,
-                     (const TG*)dy, mean, rstd, gamma, beta, param_dtype, part, S, C, G, pl.tpr, pl.rpp, pl.nsplit,
+                     (const TG*)dy, mean, rstd, gamma, beta, param_dtype, part, gpart, S, C, G, pl.tpr, pl.rpp, pl.nsplit,
                      pl.rows_per_split, p.relu);
   if (int rc = check_launch("gn_bwd_partial")) return rc;
   const float m = (float)S * (float)(C / G);
-  hipLaunchKernelGGL(gn_bwd_finalize, dim3(p.n * G + C), dim3(kBlock), 0, st, part, gamma, param_dtype, coef, dgamma, dbeta, p.n, C,
-                     G, pl.nsplit, m);
-  if (int rc = check_launch("gn_bwd_finalize")) return rc;
-  hipLaunchKernelGGL((gn_dx<T, TG>), grid, dim3(kBlock), 0, st, (const T*)x, (const TG*)dy, (T*)dx, mean, rstd, gamma, beta,
-                     param_dtype, coef, S, C, G, pl.tpr, pl.rpp, pl.rows_per_split, p.relu);
+  if (!fold_in_consumer_host(G, pl.nsplit)) {
+    hipLaunchKernelGGL(gn_bwd_finalize, dim3(p.n * G + C), dim3(kBlock), 0, st, part, gamma, param_dtype, coef, dgamma, dbeta, p.n,
+                       C, G, pl.nsplit, m);
+    if (int rc = check_launch("gn_bwd_finalize")) return rc;
+  }
+  hipLaunchKernelGGL((gn_dx<T, TG>), grid, dim3(kBlock), (size_t)(2 * G + 4 * kBlock) * sizeof(float), st, (const T*)x,
+                     (const TG*)dy, (T*)dx, mean, rstd, gamma, beta, param_dtype, coef, part, gpart, dgamma, dbeta, p.n, S, C, G,
+                     pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.relu);
   return check_launch("gn_dx");
 }
 
