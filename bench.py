@@ -38,7 +38,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the forward kernel on the bench workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
 # counter runs of this script scaled by the same counters on the 256 MiB copy kernel (profiles/ holds the runs).
-CONV_FWD_HBM_TRAFFIC_BYTES = int((109557.0 * 2.000 + 131094.3) * 1024)
+CONV_FWD_HBM_TRAFFIC_BYTES = int((108952.6 * 2.000 + 131084.5) * 1024)
 CL = torch.channels_last_3d
 
 
