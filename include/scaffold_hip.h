@@ -192,6 +192,18 @@ int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, 
 int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
                      void* grad_x, void* stream);
 
+/* ---- halo slab assembly ------------------------------------------------------------------
+ * The local step of a depth shard's forward halo exchange: out = [lo | x | hi] along depth, where
+ * lo / hi are the `halo` boundary planes received from the lower / upper neighbour, or NULL for
+ * zeros (no neighbour) -- what ScaFFold/unet/conv3d.py:769-776 builds with three strided copies
+ * after its receives. x (N, D, H, W, C), lo / hi (N, halo, H, W, C), out (N, D + 2*halo, H, W, C),
+ * all dense channels-last of `dtype`. The convolution then runs on `out` at depth padding 0. */
+typedef struct sfh_halo_desc {
+  int32_t n, c, d, h, w, halo;
+} sfh_halo_desc;
+int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* x, const void* lo,
+                      const void* hi, void* out, void* stream);
+
 /* ---- gradient clipping + Adam -----------------------------------------------------------
  * The optimizer step of the trainer: torch.nn.utils.clip_grad_norm_(parameters, max_norm) followed by
  * torch.optim.Adam.step() (ScaFFold/utils/trainer.py:678-694, optimizer built at trainer.py:268-274),

@@ -29,6 +29,8 @@ _EXPORTS = {
     "ce_dice_loss": "losses", "is_supported_loss": "losses",
     # pooling
     "max_pool3d_2x": "pooling", "is_supported_pool": "pooling", "FastMaxPool3d": "pooling",
+    # halo slab of a depth shard
+    "halo_assemble": "halo", "is_supported_halo": "halo",
     # optimizer step
     "FusedClipAdam": "optim",
     # modules / model

@@ -31,6 +31,7 @@ __all__ = [
     "LossDesc",
     "PoolDesc",
     "AdamDesc",
+    "HaloDesc",
     "dtype_code",
     "SUPPORTED_DTYPES",
     "EXPORTED_SYMBOLS",
@@ -68,6 +69,10 @@ class LossDesc(ctypes.Structure):
 
 class PoolDesc(ctypes.Structure):
     _fields_ = [(k, c_int32) for k in ("n", "c", "in_d", "in_h", "in_w")]
+
+
+class HaloDesc(ctypes.Structure):
+    _fields_ = [(k, c_int32) for k in ("n", "c", "d", "h", "w", "halo")]
 
 
 class AdamDesc(ctypes.Structure):
@@ -115,6 +120,7 @@ _SIGNATURES = {
     "sfh_ce_dice_bwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_fwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_bwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_halo_assemble": (c_int, [POINTER(HaloDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_adam_slots": (c_int64, [c_int32, POINTER(c_int64)]),
     "sfh_adam_grad_sumsq": (c_int, [c_int32, POINTER(c_void_p), POINTER(c_int64), c_void_p, c_void_p, c_void_p]),
     "sfh_adam_clip_step": (c_int, [POINTER(AdamDesc), c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),

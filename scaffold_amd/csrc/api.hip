@@ -7,6 +7,7 @@
 #include "conv_mfma.hpp"
 #include "conv_patch.hpp"
 #include "conv_thin.hpp"
+#include "halo.hpp"
 #include "loss.hpp"
 #include "reduce.hpp"
 #include "optim.hpp"
@@ -545,6 +546,18 @@ extern "C" int sfh_ce_dice_bwd(const sfh_loss_desc* p, int dtype, const void* lo
   if (logits == nullptr || labels == nullptr || stats == nullptr || grad_loss == nullptr || dlogits == nullptr)
     return fail(SFH_ERR_INVALID, "ce_dice: null tensor");
   return loss_backward(*p, dtype, logits, labels, class_weight, stats, grad_loss, dlogits, (hipStream_t)stream);
+}
+
+// ---- halo slab assembly ------------------------------------------------------------------
+extern "C" int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* x, const void* lo, const void* hi, void* out,
+                                 void* stream) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "halo assemble: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "halo assemble: bad dtype %d", dtype);
+  if (p->n < 0 || p->c < 1 || p->d < 1 || p->h < 1 || p->w < 1 || p->halo < 0)
+    return fail(SFH_ERR_INVALID, "halo assemble: bad extents n=%d c=%d (%d,%d,%d) halo=%d", p->n, p->c, p->d, p->h, p->w, p->halo);
+  if (p->n == 0) return SFH_OK;
+  if (x == nullptr || out == nullptr) return fail(SFH_ERR_INVALID, "halo assemble: null tensor");
+  return halo_assemble(*p, dtype, x, lo, hi, out, (hipStream_t)stream);
 }
 
 // ---- gradient clipping + Adam ------------------------------------------------------------

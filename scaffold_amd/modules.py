@@ -36,6 +36,7 @@ from torch.autograd.function import once_differentiable
 
 from . import conv3d as _c3
 from . import groupnorm as _gn
+from . import halo as _halo
 from . import transposed as _ct
 
 __all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand", "compute_copy"]
@@ -167,8 +168,8 @@ class FastConv3d(nn.Conv3d):
         b = bc if master else cast_operand(self.bias, dt)
         padding = tuple(self.padding)
         if self.shard_halo and padding[0] > 0:
-            # (N, C, D, H, W): extend D by the halo the neighbours would have sent
-            x = F.pad(x, (0, 0, 0, 0, padding[0], padding[0]))
+            # (N, C, D, H, W): extend D by the halo the neighbours would have sent (none here: zeros)
+            x = _halo.halo_assemble(x, None, None, int(padding[0]))
             padding = (0, padding[1], padding[2])
         x = x.contiguous(memory_format=_CL3D)
         # the node below skips its own gates on the strength of this one (a call that will be differentiated is
