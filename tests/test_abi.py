@@ -104,3 +104,61 @@ def test_transposed_and_copy_entry_points_check_arguments():
     strides = (ctypes.c_int64 * 5)(512, 1, 256, 128, 64)
     assert L.sfh_convT3d_fwd(ctypes.byref(d), 0, None, None, strides, None, None, None, 0, 0, None) == _lib.SFH_ERR_INVALID
     assert L.sfh_stream_copy(None, None, 64, None) == _lib.SFH_ERR_INVALID
+
+
+def test_argument_checks_of_the_rows_beside_the_convolutions():
+    """Loss head, pooling, halo slab, bias gradient and optimizer entry points reject bad arguments with a message
+    before anything is launched (so this runs without a GPU)."""
+    from scaffold_amd._lib import AdamDesc, HaloDesc, LossDesc, PoolDesc
+
+    L = _lib.lib()
+    bf16 = 0
+    one = ctypes.c_void_p(16)  # never dereferenced: every call below fails its checks first
+
+    # loss head: classes in [2, 32], positive extents, non-null tensors
+    assert L.sfh_ce_dice_workspace_bytes(ctypes.byref(LossDesc(1, 11, 64, 1e-6))) > 0
+    assert L.sfh_ce_dice_workspace_bytes(ctypes.byref(LossDesc(1, 1, 64, 1e-6))) == 0
+    assert L.sfh_ce_dice_workspace_bytes(ctypes.byref(LossDesc(1, 33, 64, 1e-6))) == 0
+    assert L.sfh_ce_dice_fwd(ctypes.byref(LossDesc(1, 11, 64, 1e-6)), bf16, None, one, None, one, one, one, 1 << 20, None) \
+        == _lib.SFH_ERR_INVALID
+    assert L.sfh_ce_dice_fwd(ctypes.byref(LossDesc(1, 11, 64, 1e-6)), bf16, one, one, None, one, one, None, 0, None) \
+        == _lib.SFH_ERR_WORKSPACE
+    assert L.sfh_ce_dice_bwd(ctypes.byref(LossDesc(0, 11, 64, 1e-6)), bf16, one, one, None, one, one, one, None) != _lib.SFH_OK
+
+    # pooling
+    assert L.sfh_maxpool2_fwd(None, bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_maxpool2_fwd(ctypes.byref(PoolDesc(1, 0, 4, 4, 4)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_maxpool2_fwd(ctypes.byref(PoolDesc(1, 8, 4, 4, 4)), 7, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_maxpool2_fwd(ctypes.byref(PoolDesc(1, 8, 4, 4, 4)), bf16, None, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_maxpool2_fwd(ctypes.byref(PoolDesc(1, 8, 1, 4, 4)), bf16, None, None, None, None) == _lib.SFH_OK  # empty output
+    assert L.sfh_maxpool2_bwd(ctypes.byref(PoolDesc(1, 8, 4, 4, 4)), bf16, one, None, one, None) == _lib.SFH_ERR_INVALID
+
+    # halo slab
+    assert L.sfh_halo_assemble(None, bf16, one, None, None, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_halo_assemble(ctypes.byref(HaloDesc(1, 8, 4, 4, 4, -1)), bf16, one, None, None, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_halo_assemble(ctypes.byref(HaloDesc(1, 8, 4, 4, 4, 1)), bf16, None, None, None, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_halo_assemble(ctypes.byref(HaloDesc(0, 8, 4, 4, 4, 1)), bf16, None, None, None, None, None) == _lib.SFH_OK
+
+    # bias gradient
+    assert L.sfh_bias_grad_workspace_bytes(0, 32) == 0 and L.sfh_bias_grad_workspace_bytes(4096, 32) > 0
+    assert L.sfh_bias_grad(bf16, bf16, one, 0, 32, one, one, 1 << 20, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_bias_grad(bf16, bf16, one, 4096, 32, one, None, 0, None) == _lib.SFH_ERR_WORKSPACE
+
+    # optimizer: slot count = sum of ceil(numel / 8192); hyperparameter and pointer checks
+    numel = (ctypes.c_int64 * 3)(1, 8192, 8193)
+    assert L.sfh_adam_slots(3, numel) == 1 + 1 + 2
+    assert L.sfh_adam_slots(0, numel) == 0
+    ptrs = (ctypes.c_void_p * 3)(16, 16, 16)
+    nulls = (ctypes.c_void_p * 3)(16, None, 16)
+    assert L.sfh_adam_grad_sumsq(3, nulls, numel, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_adam_grad_sumsq(3, ptrs, (ctypes.c_int64 * 3)(1, 0, 1), one, one, None) == _lib.SFH_ERR_INVALID
+    good = AdamDesc(1e-3, 0.9, 0.999, 1e-8, 0.0, 1.0, -1)
+    assert L.sfh_adam_clip_step(ctypes.byref(good), 3, ptrs, ptrs, ptrs, nulls, None, numel, one, 4, one, None, None) \
+        == _lib.SFH_ERR_INVALID
+    bad_beta = AdamDesc(1e-3, 1.0, 0.999, 1e-8, 0.0, 1.0, -1)
+    assert L.sfh_adam_clip_step(ctypes.byref(bad_beta), 3, ptrs, ptrs, ptrs, ptrs, None, numel, one, 4, one, None, None) \
+        == _lib.SFH_ERR_INVALID
+    assert L.sfh_adam_clip_step(ctypes.byref(good), 3, ptrs, ptrs, ptrs, ptrs, ptrs, numel, one, 4, one, None, None) \
+        == _lib.SFH_ERR_INVALID  # shadow copies without a shadow dtype
+    assert L.sfh_adam_clip_step(ctypes.byref(good), 3, ptrs, ptrs, ptrs, ptrs, None, numel, one, 0, one, None, None) \
+        == _lib.SFH_ERR_INVALID  # no slots to fold
