@@ -41,6 +41,9 @@ extern "C" {
 
 /* Flags for the convolution entry points. */
 #define SFH_FLAG_FORCE_GENERIC 1u /* use the direct (non-MFMA) kernels whatever the shape */
+#define SFH_FLAG_WEIGHT_PACKED 4u /* sfh_conv3d_fwd / _dgrad: `w` is the weight already packed for that direction by
+                                     sfh_conv3d_pack_weights (same descriptor and dtype); w_stride is ignored and
+                                     the workspace only needs the bytes beyond sfh_conv3d_packed_weight_bytes. */
 #define SFH_FLAG_GRAD_FP32 2u     /* sfh_conv3d_wgrad: write grad_w as fp32 (the master weight's dtype under
                                      autocast) instead of the operands' dtype: the fp32 sum of the slices is
                                      stored as it is, saving the rounding and the caller's up-cast. Served by
@@ -99,6 +102,19 @@ size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
 int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w,
                      const int64_t w_stride[5], void* gx, void* workspace,
                      size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- packing a weight once for both directions ------------------------------------------
+ * The MFMA kernels read the weight in fragment order; sfh_conv3d_fwd / _dgrad repack it on every
+ * call (the reference transforms nothing, gather_gemm.py:894-942, and this keeps that contract by
+ * default). A caller that runs forward and data gradient with one weight (every training step)
+ * can pack both forms in ONE launch here and pass them with SFH_FLAG_WEIGHT_PACKED.
+ * sfh_conv3d_packed_weight_bytes: bytes of the packed form for direction 0 (forward) or
+ * 1 (data gradient), 0 when that direction of this problem does not read a packed weight.
+ * Either output of sfh_conv3d_pack_weights may be NULL. No counterpart in the reference. */
+size_t sfh_conv3d_packed_weight_bytes(const sfh_conv3d_desc* p, int dtype, int direction);
+int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w,
+                            const int64_t w_stride[5], void* packed_fwd, void* packed_dgrad,
+                            void* stream);
 
 /* ---- conv3d weight gradient ----------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_backward_weight (triton_conv3d/reduce_gemm.py:1177),

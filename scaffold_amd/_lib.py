@@ -40,6 +40,7 @@ __all__ = [
 SFH_OK, SFH_ERR_INVALID, SFH_ERR_UNSUPPORTED, SFH_ERR_WORKSPACE, SFH_ERR_LAUNCH = range(5)
 SFH_FLAG_FORCE_GENERIC = 1
 SFH_FLAG_GRAD_FP32 = 2
+SFH_FLAG_WEIGHT_PACKED = 4
 
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 SUPPORTED_DTYPES = tuple(_DTYPE_CODE)
@@ -99,6 +100,8 @@ _SIGNATURES = {
     "sfh_conv3d_dgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_dgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                  c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_packed_weight_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),
+    "sfh_conv3d_pack_weights": (c_int, [POINTER(ConvDesc), c_int, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_void_p]),
     "sfh_conv3d_wgrad_splits": (c_int, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_wgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_wgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,

@@ -49,6 +49,8 @@ __all__ = [
     "bwd_data_padding",
     "grad_weight_empty",
     "workspace_elements",
+    "pack_weights",
+    "packed_weight_bytes",
     "split_count",
     "uses_mfma",
     "output_shape",
@@ -304,6 +306,68 @@ def bias_grad(grad_output: torch.Tensor, dtype: Optional[torch.dtype] = None) ->
     return gb
 
 
+_PACKED_BYTES_CACHE: dict = {}
+
+
+def packed_weight_bytes(in_shape, weight_shape, stride, padding, dilation, dtype) -> tuple[int, int]:
+    """Bytes of the packed weight the forward and the data gradient of this problem read (0 where a direction does
+    not read one)."""
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    key = (tuple(int(v) for v in in_shape), tuple(int(v) for v in weight_shape), s, p, d, dtype)
+    hit = _PACKED_BYTES_CACHE.get(key)
+    if hit is None:
+        n, cin, *in_sp = key[0]
+        cout, _, *k = key[1]
+        desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+        L = _lib.lib()
+        try:
+            code = _lib.dtype_code(dtype)
+            hit = (int(L.sfh_conv3d_packed_weight_bytes(ctypes.byref(desc), code, 0)),
+                   int(L.sfh_conv3d_packed_weight_bytes(ctypes.byref(desc), code, 1)))
+        except NotImplementedError:
+            hit = (0, 0)
+        if len(_PACKED_BYTES_CACHE) > 4096:
+            _PACKED_BYTES_CACHE.clear()
+        _PACKED_BYTES_CACHE[key] = hit
+    return hit
+
+
+_PACK_PLAN_CACHE: dict = {}
+
+
+def pack_weights(w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1, *, forward: bool = True, backward_data: bool = True):
+    """Packs ``w`` once, in one launch, for the forward and / or the data gradient of the convolution of an input of
+    ``in_shape``: returns ``(packed_fwd, packed_dgrad)`` to pass as ``packed_weight=``; an entry is ``None`` when it
+    was not asked for or when that direction of the problem does not read a packed weight (it then takes ``w``).
+    The default entry points repack on every call; a train step that packs once here saves a launch per convolution."""
+    key = (in_shape, w.shape, stride, padding, dilation, w.dtype)
+    try:
+        plan = _PACK_PLAN_CACHE.get(key)
+    except TypeError:  # unhashable spelling of stride / padding / dilation
+        key, plan = None, None
+    if plan is None:
+        s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+        nbf, nbd = packed_weight_bytes(in_shape, w.shape, s, p, d, w.dtype)
+        n, cin, *in_sp = (int(v) for v in in_shape)
+        k = tuple(int(v) for v in w.shape[2:])
+        plan = (nbf, nbd, _desc(n, cin, in_sp, int(w.shape[0]), k, s, p, d), _lib.dtype_code(w.dtype) if (nbf or nbd) else -1)
+        if key is not None:
+            if len(_PACK_PLAN_CACHE) > 4096:
+                _PACK_PLAN_CACHE.clear()
+            _PACK_PLAN_CACHE[key] = plan
+    nbf, nbd, desc, code = plan
+    pf = torch.empty(nbf, dtype=torch.uint8, device=w.device) if (forward and nbf) else None
+    pd = torch.empty(nbd, dtype=torch.uint8, device=w.device) if (backward_data and nbd) else None
+    if pf is None and pd is None:
+        return None, None
+    with _lib.device_guard(w.device):
+        rc = _lib.lib().sfh_conv3d_pack_weights(ctypes.byref(desc), code, _lib.ptr(w), _lib.strides5(w), _lib.ptr(pf), _lib.ptr(pd),
+                                                _lib.stream_ptr(w.device))
+    if rc:
+        _lib.check(rc, "pack_weights")
+    return pf, pd
+
+
 # ---------------------------------------------------------------------------------------------
 # forward
 # ---------------------------------------------------------------------------------------------
@@ -321,6 +385,7 @@ def conv3d_forward(
     weight_flip: bool = False,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    packed_weight: Optional[torch.Tensor] = None,
     _checked: bool = False,
 ) -> torch.Tensor:
     """Forward 3-D convolution; input and output are ``channels_last_3d``.
@@ -360,10 +425,19 @@ def conv3d_forward(
     desc = _desc(n, cin, in_sp, cout, k, s, p, d)
     code = _lib.dtype_code(x.dtype)
     with _lib.device_guard(x.device):
-        ws = _lib.workspace(L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
-        rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(bias),
-                              _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
-                              _lib.stream_ptr(x.device))
+        need = int(L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(desc), code))
+        flags = _flags(force_generic)
+        if packed_weight is not None:
+            # ``packed_weight`` comes from pack_weights() for this very problem: the library reads it in place of w
+            if weight_rsck is not None or weight_flip or force_generic:
+                raise ValueError("packed_weight= cannot be combined with weight_rsck=, weight_flip= or force_generic=")
+            need -= packed_weight.numel()
+            flags |= _lib.SFH_FLAG_WEIGHT_PACKED
+            w_eff = packed_weight
+        ws = _lib.workspace(need, x.device)
+        rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
+                              None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                              _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(x.device))
     _lib.check(rc, "conv3d_forward")
     return y
 
@@ -384,6 +458,7 @@ def conv3d_backward_data(
     weight_rsck: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    packed_weight: Optional[torch.Tensor] = None,
     _checked: bool = False,
 ) -> torch.Tensor:
     """Gradient of a conv3d with respect to its input (stride 1 only).
@@ -419,10 +494,18 @@ def conv3d_backward_data(
     desc = _desc(n, cin, in_sp, cout, k, s, p, d)
     code = _lib.dtype_code(gy.dtype)
     with _lib.device_guard(gy.device):
-        ws = _lib.workspace(L.sfh_conv3d_dgrad_workspace_bytes(ctypes.byref(desc), code), gy.device)
-        rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff), _lib.strides5(w_eff), _lib.ptr(gx),
-                                _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
-                                _lib.stream_ptr(gy.device))
+        need = int(L.sfh_conv3d_dgrad_workspace_bytes(ctypes.byref(desc), code))
+        flags = _flags(force_generic)
+        if packed_weight is not None:
+            if weight_rsck is not None or force_generic:
+                raise ValueError("packed_weight= cannot be combined with weight_rsck= or force_generic=")
+            need -= packed_weight.numel()
+            flags |= _lib.SFH_FLAG_WEIGHT_PACKED
+            w_eff = packed_weight
+        ws = _lib.workspace(need, gy.device)
+        rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff),
+                                None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(gx),
+                                _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(gy.device))
     _lib.check(rc, "conv3d_backward_data")
     return gx
 

@@ -277,12 +277,18 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
                               const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
-  if (x == nullptr || w == nullptr || y == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d fwd: null tensor");
+  if (x == nullptr || w == nullptr || y == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
+    return fail(SFH_ERR_INVALID, "conv3d fwd: null tensor");
   if (p->n == 0) return SFH_OK;
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_mfma(*p, dtype, out)) {
     const MfmaConvArgs a = fwd_mfma_args(*p, out);
     const size_t packed_bytes = mfma_conv_packed_weight_bytes(a), partial_bytes = mfma_conv_partial_bytes(a);
+    if (flags & SFH_FLAG_WEIGHT_PACKED) {  // w is the packed weight; the workspace only holds the partial slices
+      if (partial_bytes && (workspace == nullptr || workspace_bytes < partial_bytes))
+        return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", partial_bytes, workspace_bytes);
+      return mfma_conv_persist(a, dtype, x, w, bias, y, partial_bytes ? workspace : nullptr, st);
+    }
     const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
@@ -291,6 +297,7 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st);
   }
+  if (flags & SFH_FLAG_WEIGHT_PACKED) return fail(SFH_ERR_INVALID, "conv3d fwd: this problem does not read a packed weight");
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_patch(*p, dtype, out)) {
     const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);
     const size_t need = mfma_conv_packed_weight_bytes(pk);
@@ -323,6 +330,31 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
   return direct_conv_gather(a, dtype, x, w, bias, y, st);
 }
 
+// ---- packing a weight once for both directions ------------------------------------------------
+extern "C" size_t sfh_conv3d_packed_weight_bytes(const sfh_conv3d_desc* p, int dtype, int direction) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK) return 0;
+  if (direction == 0) return fwd_uses_mfma(*p, dtype, out) ? mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out)) : 0;
+  if (direction == 1)
+    return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)) ? mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out)) : 0;
+  return 0;
+}
+
+extern "C" int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t w_stride[5], void* packed_fwd,
+                                       void* packed_dgrad, void* stream) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (w == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack: null weight");
+  if (packed_fwd != nullptr && !fwd_uses_mfma(*p, dtype, out))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the forward of this problem does not read a packed weight");
+  if (packed_dgrad != nullptr && !(check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the data gradient of this problem does not read a packed weight");
+  if (packed_fwd == nullptr && packed_dgrad == nullptr) return SFH_OK;
+  const MfmaConvArgs fa = packed_fwd != nullptr ? fwd_mfma_args(*p, out) : MfmaConvArgs{};
+  const MfmaConvArgs da = packed_dgrad != nullptr ? dgrad_mfma_args(*p, out) : MfmaConvArgs{};
+  return mfma_pack_weight_pair(fa, da, dtype, w, w_stride, packed_fwd, packed_dgrad, (hipStream_t)stream);
+}
+
 // ---- data gradient ---------------------------------------------------------------------
 extern "C" size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
@@ -336,11 +368,17 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (int rc = check_dgrad(*p)) return rc;
-  if (gy == nullptr || w == nullptr || gx == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d dgrad: null tensor");
+  if (gy == nullptr || w == nullptr || gx == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
+    return fail(SFH_ERR_INVALID, "conv3d dgrad: null tensor");
   hipStream_t st = (hipStream_t)stream;
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && dgrad_uses_mfma(*p, dtype, out)) {
     const MfmaConvArgs a = dgrad_mfma_args(*p, out);
     const size_t packed_bytes = mfma_conv_packed_weight_bytes(a), partial_bytes = mfma_conv_partial_bytes(a);
+    if (flags & SFH_FLAG_WEIGHT_PACKED) {
+      if (partial_bytes && (workspace == nullptr || workspace_bytes < partial_bytes))
+        return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", partial_bytes, workspace_bytes);
+      return mfma_conv_persist(a, dtype, gy, w, nullptr, gx, partial_bytes ? workspace : nullptr, st);
+    }
     const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
@@ -350,6 +388,7 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st);
   }
+  if (flags & SFH_FLAG_WEIGHT_PACKED) return fail(SFH_ERR_INVALID, "conv3d dgrad: this problem does not read a packed weight");
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
     ThinArgs t;
     const ThinKind kind = thin_dgrad_plan(*p, dtype, out, t);

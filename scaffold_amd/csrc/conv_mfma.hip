@@ -242,36 +242,50 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 // One thread per packed 16-byte piece: the 8 consecutive reduction channels of one (output channel, tap, k-half).
 // With the reduction channel innermost in memory (forward, channels-last weight) that is one 16-byte load;
 // otherwise eight 2-byte loads, each coalesced across the wavefront's 32 consecutive output channels.
+struct PackJob {
+  const void* w;
+  void* packed;
+  int cout, cred, kd, kh, kw, flip;
+  int64_t s_out, s_red, s_kd, s_kh, s_kw;
+  int64_t pieces;
+};
+
 template <typename T>
-__global__ void __launch_bounds__(256) pack_weight_kernel(const T* __restrict__ w, T* __restrict__ packed, int cout, int cred,
-                                                          int kd, int kh, int kw, int64_t s_out, int64_t s_red, int64_t s_kd,
-                                                          int64_t s_kh, int64_t s_kw, int flip, int64_t pieces) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= pieces) return;
-  const int taps = kd * kh * kw;
+__device__ __forceinline__ void pack_piece(const PackJob& j, int64_t idx) {
+  const T* w = static_cast<const T*>(j.w);
+  T* packed = static_cast<T*>(j.packed);
+  const int taps = j.kd * j.kh * j.kw;
   int64_t r = idx;
   const int lane = (int)(r % 64); r /= 64;
   const int ks = (int)(r % 2); r /= 2;
   int tap = (int)(r % taps); r /= taps;
-  const int ncc = cred / kChunk;
+  const int ncc = j.cred / kChunk;
   const int cc = (int)(r % ncc);
   const int nblk = (int)(r / ncc);
   const int co = nblk * 32 + (lane & 31);
   const int ci = cc * kChunk + ks * 16 + (lane >> 5) * 8;
-  if (flip) tap = taps - 1 - tap;
-  const int tkw = tap % kw, tkh = (tap / kw) % kh, tkd = tap / (kw * kh);
-  const T* src = w + co * s_out + ci * s_red + tkd * s_kd + tkh * s_kh + tkw * s_kw;
+  if (j.flip) tap = taps - 1 - tap;
+  const int tkw = tap % j.kw, tkh = (tap / j.kw) % j.kh, tkd = tap / (j.kw * j.kh);
+  const T* src = w + co * j.s_out + ci * j.s_red + tkd * j.s_kd + tkh * j.s_kh + tkw * j.s_kw;
   uint4 v;
-  if (s_red == 1 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
+  if (j.s_red == 1 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
     v = *reinterpret_cast<const uint4*>(src);
   } else {
     uint16_t h[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) h[e] = *reinterpret_cast<const uint16_t*>(src + e * s_red);
+    for (int e = 0; e < 8; ++e) h[e] = *reinterpret_cast<const uint16_t*>(src + e * j.s_red);
     v.x = h[0] | ((uint32_t)h[1] << 16); v.y = h[2] | ((uint32_t)h[3] << 16);
     v.z = h[4] | ((uint32_t)h[5] << 16); v.w = h[6] | ((uint32_t)h[7] << 16);
   }
   *reinterpret_cast<uint4*>(packed + idx * 8) = v;
+}
+
+// Up to two packings of one weight (the forward's and the data gradient's) in one launch.
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_kernel(PackJob first, PackJob second) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx < first.pieces) pack_piece<T>(first, idx);
+  else if (idx - first.pieces < second.pieces) pack_piece<T>(second, idx - first.pieces);
 }
 
 struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
@@ -345,17 +359,40 @@ size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a) {
   return align_up((size_t)a.cout * a.cred * a.kd * a.kh * a.kw * 2, 256);
 }
 
+namespace {
+PackJob pack_job(const MfmaConvArgs& a, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd, int64_t s_kh, int64_t s_kw, int flip,
+                 void* packed) {
+  PackJob j{};
+  j.w = w; j.packed = packed;
+  j.cout = a.cout; j.cred = a.cred; j.kd = a.kd; j.kh = a.kh; j.kw = a.kw; j.flip = flip;
+  j.s_out = s_out; j.s_red = s_red; j.s_kd = s_kd; j.s_kh = s_kh; j.s_kw = s_kw;
+  j.pieces = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw / 8;  // 16-byte pieces
+  return j;
+}
+int launch_pack(int dtype, const PackJob& first, const PackJob& second, hipStream_t st) {
+  const int64_t total = first.pieces + second.pieces;
+  if (total <= 0) return SFH_OK;
+  const unsigned blocks = (unsigned)cdiv(total, 256);
+  if (dtype == SFH_BF16) hipLaunchKernelGGL(pack_weight_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, first, second);
+  else hipLaunchKernelGGL(pack_weight_kernel<fp16_t>, dim3(blocks), dim3(256), 0, st, first, second);
+  return check_launch("pack_weight_kernel");
+}
+}  // namespace
+
 int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd, int64_t s_kh,
                      int64_t s_kw, int flip, void* packed, hipStream_t st) {
-  const int64_t total = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw / 8;  // 16-byte pieces
-  const unsigned blocks = (unsigned)cdiv(total, 256);
-  if (dtype == SFH_BF16)
-    hipLaunchKernelGGL(pack_weight_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)w, (bf16_t*)packed, a.cout,
-                       a.cred, a.kd, a.kh, a.kw, s_out, s_red, s_kd, s_kh, s_kw, flip, total);
-  else
-    hipLaunchKernelGGL(pack_weight_kernel<fp16_t>, dim3(blocks), dim3(256), 0, st, (const fp16_t*)w, (fp16_t*)packed, a.cout,
-                       a.cred, a.kd, a.kh, a.kw, s_out, s_red, s_kd, s_kh, s_kw, flip, total);
-  return check_launch("pack_weight_kernel");
+  PackJob none{};
+  return launch_pack(dtype, pack_job(a, w, s_out, s_red, s_kd, s_kh, s_kw, flip, packed), none, st);
+}
+
+int mfma_pack_weight_pair(const MfmaConvArgs& fwd, const MfmaConvArgs& dgrad, int dtype, const void* w, const int64_t w_stride[5],
+                          void* packed_fwd, void* packed_dgrad, hipStream_t st) {
+  PackJob first{}, second{};
+  // forward: produced channel = Cout (w_stride[0]), reduced = Cin; data gradient: produced = Cin, reduced = Cout, taps flipped
+  if (packed_fwd != nullptr) first = pack_job(fwd, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, packed_fwd);
+  if (packed_dgrad != nullptr)
+    second = pack_job(dgrad, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, packed_dgrad);
+  return launch_pack(dtype, first, second, st);
 }
 
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {

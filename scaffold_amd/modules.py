@@ -43,6 +43,9 @@ __all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype
 
 _CL3D = torch.channels_last_3d
 
+#: pack each convolution weight once per step for forward and data gradient also outside graph capture
+PACK_WEIGHTS_ONCE = False
+
 
 def autocast_dtype(tensor: torch.Tensor) -> Optional[torch.dtype]:
     """The dtype autocast would cast a convolution's operands to on this device, or ``None``."""
@@ -92,8 +95,14 @@ class _Conv3dFn(torch.autograd.Function):
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
         bc = bias if bias_compute is None else bias_compute
-        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, _checked=True)
-        ctx.save_for_backward(x, wc)
+        # When the data gradient will be wanted too, the weight can be packed for both directions in one launch. That
+        # saves a launch per convolution on the GPU and costs a little more host time, so it is done where host time
+        # is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
+        pf = pd = None
+        if ctx.needs_input_grad[0] and (PACK_WEIGHTS_ONCE or torch.cuda.is_current_stream_capturing()):
+            pf, pd = _c3.pack_weights(wc, x.shape, stride, padding, dilation)
+        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, _checked=True)
+        ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
         return y
@@ -101,11 +110,12 @@ class _Conv3dFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
-        x, weight = ctx.saved_tensors
+        x, weight, *packed = ctx.saved_tensors
         stride, padding, dilation, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
-        grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1, _checked=True) if needs_x else None
+        grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1,
+                                          packed_weight=packed[0] if packed else None, _checked=True) if needs_x else None
         grad_w = None
         if needs_w:
             if master:

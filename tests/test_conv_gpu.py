@@ -425,3 +425,40 @@ def test_bias_grad_matches_sum(device, dtype, shape):
     assert torch.equal(sa.bias_grad(gauss.contiguous().to(device), torch.float32).cpu().double(), got)
     # same call, same bits
     assert torch.equal(sa.bias_grad(gauss.to(device), torch.float32).cpu().double(), got)
+
+
+# ---- packing a weight once for both directions -------------------------------------------------------------------
+CL = torch.channels_last_3d
+
+@pytest.mark.parametrize("cin,cout,sp,pad", [
+    (32, 32, (8, 16, 32), (1, 1, 1)),      # persistent kernel
+    (32, 64, (6, 16, 32), (0, 1, 1)),      # shard form
+    (64, 32, (8, 16, 32), (1, 1, 1)),      # brick-per-workgroup kernel
+    (256, 256, (4, 8, 8), (1, 1, 1)),      # reduction channels cut into slices (partial workspace beside the weight)
+])
+def test_prepacked_weight_gives_the_same_bits(device, cin, cout, sp, pad):
+    g = torch.Generator().manual_seed(61)
+    x = torch.randn((1, cin, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    w = (torch.randn((cout, cin, 3, 3, 3), generator=g) * 0.05).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    y = sa.conv3d_forward(x, w, None, 1, pad, 1)
+    gy = torch.randn(y.shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    gx = sa.conv3d_backward_data(gy, w, x.shape, 1, pad, 1)
+    pf, pd = sa.pack_weights(w, x.shape, 1, pad, 1)
+    assert pf is not None and pd is not None
+    assert (pf.numel(), pd.numel()) == sa.packed_weight_bytes(x.shape, w.shape, 1, pad, 1, w.dtype)
+    assert torch.equal(sa.conv3d_forward(x, w, None, 1, pad, 1, packed_weight=pf), y)
+    assert torch.equal(sa.conv3d_backward_data(gy, w, x.shape, 1, pad, 1, packed_weight=pd), gx)
+    only_f, none_d = sa.pack_weights(w, x.shape, 1, pad, 1, backward_data=False)
+    assert none_d is None and torch.equal(only_f, pf)
+
+
+def test_pack_weights_declines_problems_that_read_the_weight_where_it_lies(device):
+    w5 = torch.randn((7, 5, 3, 3, 3), device=device).to(torch.bfloat16)
+    assert sa.pack_weights(w5, (1, 5, 8, 8, 8), 1, 1, 1) == (None, None)
+    w32 = torch.randn((32, 32, 3, 3, 3), device=device)           # fp32: true fp32 kernels, no MFMA packing
+    assert sa.pack_weights(w32, (1, 32, 8, 8, 8), 1, 1, 1) == (None, None)
+    wb = w32.to(torch.bfloat16).contiguous(memory_format=CL)
+    x = torch.randn((1, 32, 8, 8, 8), device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    pf, _ = sa.pack_weights(wb, x.shape, 1, 1, 1)
+    with pytest.raises(ValueError):
+        sa.conv3d_forward(x, wb, None, 1, 1, 1, packed_weight=pf, force_generic=True)

@@ -252,3 +252,19 @@ def test_train_step_as_a_hip_graph_replays_to_the_eager_result(device):
         torch.randn(1 << 16, device=device).sum().item()
     assert got == want
     assert want[0] != want[1]
+
+
+def test_packing_the_weight_once_per_step_changes_no_bits(device):
+    import scaffold_amd.modules as mods
+
+    def grads(flag):
+        mods.PACK_WEIGHTS_ONCE = flag
+        try:
+            _, ours, x, lab = _two_arms(device, torch.bfloat16, shard=True)
+            _step(ours, x.to(device).contiguous(memory_format=CL), lab.to(device), "cuda")
+            return [p.grad.clone() for p in ours.parameters()]
+        finally:
+            mods.PACK_WEIGHTS_ONCE = False
+
+    a, b = grads(False), grads(True)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
