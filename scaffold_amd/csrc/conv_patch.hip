@@ -43,31 +43,6 @@ __device__ __forceinline__ int64_t big_index(const PatchArgs& a, const Voxel& v,
   return (((int64_t)v.nn * a.bd + 2 * v.d + (tap >> 2)) * a.bh + 2 * v.h + ((tap >> 1) & 1)) * a.bw + 2 * v.w + (tap & 1);
 }
 
-template <typename T>
-__device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
-
-// Stores result block `acc` (32 produced channels x 32 voxels): this lane's voxel row starts at `row`
-// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given. The two lanes of a voxel trade
-// channel runs first, so each stores two 16-byte pieces. All 64 lanes must call it; `valid` masks the stores.
-template <typename T>
-__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
-  uint32_t run[4][2];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const int c = 8 * g + 4 * kg;
-    float v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = acc[4 * g + i] + (bias != nullptr ? to_float(bias[c0 + c + i]) : 0.f);
-    run[g][0] = Mma32<T>::pack2(v[0], v[1]);
-    run[g][1] = Mma32<T>::pack2(v[2], v[3]);
-  }
-  uint4 piece[2];
-  trade_channel_runs(run, piece);
-  if (valid) {
-    *reinterpret_cast<uint4*>(row + 8 * kg) = piece[0];
-    *reinterpret_cast<uint4*>(row + 16 + 8 * kg) = piece[1];
-  }
-}
 
 // ---- gather: stride-2 convolution --------------------------------------------------------------
 // A wavefront owns 32 small voxels x NB blocks of 32 produced channels. grid = (voxel tiles of 128, groups of NB blocks).

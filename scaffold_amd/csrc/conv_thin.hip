@@ -13,6 +13,7 @@
 // The reference serves these shapes with the same implicit-GEMM kernels at small tile sizes
 // (triton_conv3d/gather_gemm.py:493-560, reduce_gemm.py:655-700).
 #include "conv_thin.hpp"
+#include "mma.hpp"
 #include "reduce.hpp"
 #include "vec_io.hpp"
 
@@ -138,6 +139,213 @@ __global__ void __launch_bounds__(kBlock) thin_out_kernel(ThinArgs a, const T* _
 #pragma unroll
     for (int j = 0; j < J; ++j)
       if (j < a.J) o[j] = elem<T>::from_float(acc[j]);
+  }
+}
+
+// ---- pointwise head on the matrix cores -----------------------------------------------------------
+// 16-bit types, K == 0 and a wide side of 32, 64 or 128 channels. A workgroup owns 128 consecutive voxels per
+// round, a wavefront 32 of them; the thin side (at most 32 channels, e.g. the 11 classes) is zero-padded to one
+// MFMA tile. The thin rows of a round are one contiguous byte range of the thin tensor, which moves between
+// global memory and LDS in 16-byte pieces whatever the channel count.
+constexpr int kHeadVoxels = 128;
+constexpr int kHeadThinMax = 32;
+
+// 8 consecutive wide channels from c0 of thin channel j (zero at and beyond J) as a packed MFMA operand piece.
+template <typename T>
+__device__ __forceinline__ uint4 head_weight_wide_run(const ThinArgs& a, const T* __restrict__ wt, int j, int c0) {
+  uint16_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    h[e] = j < a.J ? reinterpret_cast<const uint16_t*>(wt)[(int64_t)(c0 + e) * a.ws_wide + (int64_t)j * a.ws_thin] : (uint16_t)0;
+  return make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
+}
+// 8 consecutive thin channels from j0 of wide channel c.
+template <typename T>
+__device__ __forceinline__ uint4 head_weight_thin_run(const ThinArgs& a, const T* __restrict__ wt, int c, int j0) {
+  uint16_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    h[e] = j0 + e < a.J ? reinterpret_cast<const uint16_t*>(wt)[(int64_t)c * a.ws_wide + (int64_t)(j0 + e) * a.ws_thin] : (uint16_t)0;
+  return make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
+}
+
+// thin-out: out[v][j] = bias[j] + sum_c wide[v][c] * W[j][c]. Result tile: rows = thin channels, columns = voxels.
+template <typename T, int NC>
+__global__ void __launch_bounds__(kBlock) head_thin_out_kernel(ThinArgs a, const T* __restrict__ wide, const T* __restrict__ wt,
+                                                               const T* __restrict__ bias, T* __restrict__ out, int64_t total) {
+  __shared__ __align__(16) T rows[kHeadVoxels * kHeadThinMax];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, kg = lane >> 5;
+  const int J = a.J;
+  uint4 wf[NC][2];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) wf[cc][ks] = head_weight_wide_run<T>(a, wt, col, cc * 32 + ks * 16 + kg * 8);
+  float bv[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int j = 8 * (r / 4) + 4 * kg + r % 4;
+    bv[r] = (bias != nullptr && j < J) ? to_float(bias[j]) : 0.f;
+  }
+  for (int64_t base = (int64_t)blockIdx.x * kHeadVoxels; base < total; base += (int64_t)gridDim.x * kHeadVoxels) {
+    const int64_t v = base + wave * 32 + col;
+    const T* src = wide + (v < total ? v : total - 1) * a.cw + kg * 8;
+    uint4 xf[NC][2];
+#pragma unroll
+    for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) xf[cc][ks] = load16(src + cc * 32 + ks * 16);
+    f32x16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[cc][ks], acc);
+    T* mine = rows + (wave * 32 + col) * J;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 8 * (r / 4) + 4 * kg + r % 4;
+      if (j < J) mine[j] = elem<T>::from_float(acc[r] + bv[r]);
+    }
+    __syncthreads();
+    const int64_t left = total - base;
+    const int nv = left < kHeadVoxels ? (int)left : kHeadVoxels;
+    const int nelem = nv * J, npiece = nelem / 8;
+    T* dst = out + base * J;
+    for (int i = tid; i < npiece; i += kBlock) reinterpret_cast<uint4*>(dst)[i] = reinterpret_cast<const uint4*>(rows)[i];
+    for (int i = npiece * 8 + tid; i < nelem; i += kBlock) dst[i] = rows[i];
+    __syncthreads();
+  }
+}
+
+// wide-out: out[v][c] = bias[c] + sum_j thin[v][j] * W[j][c]. Result tile: rows = wide channels, columns = voxels.
+// NK = MFMA steps of 16 thin channels.
+template <typename T, int NC, int NK>
+__global__ void __launch_bounds__(kBlock) head_wide_out_kernel(ThinArgs a, const T* __restrict__ thin, const T* __restrict__ wt,
+                                                               const T* __restrict__ bias, T* __restrict__ out, int64_t total) {
+  // one row of slack: the operand read of the last voxel runs up to 16 * NK channels
+  __shared__ __align__(16) uint16_t rows[(kHeadVoxels + 1) * kHeadThinMax];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, kg = lane >> 5;
+  const int J = a.J;
+  uint4 wf[NC][NK];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) wf[cc][ks] = head_weight_thin_run<T>(a, wt, cc * 32 + col, ks * 16 + kg * 8);
+  for (int64_t base = (int64_t)blockIdx.x * kHeadVoxels; base < total; base += (int64_t)gridDim.x * kHeadVoxels) {
+    const int64_t left = total - base;
+    const int nv = left < kHeadVoxels ? (int)left : kHeadVoxels;
+    const int nelem = nv * J, npiece = nelem / 8;
+    const uint16_t* src = reinterpret_cast<const uint16_t*>(thin) + base * J;
+    for (int i = tid; i < npiece; i += kBlock) reinterpret_cast<uint4*>(rows)[i] = reinterpret_cast<const uint4*>(src)[i];
+    for (int i = npiece * 8 + tid; i < nelem; i += kBlock) rows[i] = src[i];
+    __syncthreads();
+    const int lv = wave * 32 + col;
+    const bool valid = lv < nv;
+    const uint16_t* mine = rows + (valid ? lv : 0) * J;
+    uint4 xf[NK];
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) {
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = ks * 16 + kg * 8 + e;
+        const uint32_t bits = mine[j];
+        h[e] = j < J ? bits : 0u;
+      }
+      xf[ks] = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+    }
+    T* dst = out + (base + (valid ? lv : 0)) * a.cw;
+#pragma unroll
+    for (int cc = 0; cc < NC; ++cc) {
+      f32x16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[ks], acc);
+      store_block<T>(acc, dst + cc * 32, bias, cc * 32, kg, valid);
+    }
+    __syncthreads();
+  }
+}
+
+// reduce: G[j][c] = sum_v thin[v][j] * wide[v][c]. The contraction runs over voxels, so both operands are read from
+// LDS against their storage order (8 voxels of one channel per lane). A workgroup owns a contiguous voxel range in
+// rounds of 128, its four wavefronts a quarter of each round; their tiles are folded in wave order into one fp32
+// partial slice, already in the layout of the weight gradient. Tile rows at and beyond J carry garbage that is
+// never written out; voxels beyond the range are zero on both sides.
+template <typename T, int NC>
+__global__ void __launch_bounds__(kBlock) head_reduce_kernel(ThinArgs a, const T* __restrict__ thin, const T* __restrict__ wide,
+                                                             float* __restrict__ part, int64_t total, int64_t per_split) {
+  constexpr int CW = NC * 32;
+  __shared__ __align__(16) uint16_t trows[(kHeadVoxels + 1) * kHeadThinMax];
+  constexpr int kFoldHalves = 4 * 32 * 33 * 2;  // the fold at the end reuses the wide rows
+  __shared__ __align__(16) uint16_t wrows[kHeadVoxels * CW > kFoldHalves ? kHeadVoxels * CW : kFoldHalves];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, kg = lane >> 5;
+  const int J = a.J;
+  f32x16_t acc[NC];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[cc][r] = 0.f;
+  const int64_t begin = (int64_t)blockIdx.x * per_split;
+  int64_t end = begin + per_split;
+  if (end > total) end = total;
+  for (int64_t base = begin; base < end; base += kHeadVoxels) {
+    const int64_t left = end - base;
+    const int nv = left < kHeadVoxels ? (int)left : kHeadVoxels;
+    {
+      const int nelem = nv * J, npiece = nelem / 8;
+      const uint16_t* src = reinterpret_cast<const uint16_t*>(thin) + base * J;
+      for (int i = tid; i < npiece; i += kBlock) reinterpret_cast<uint4*>(trows)[i] = reinterpret_cast<const uint4*>(src)[i];
+      for (int i = npiece * 8 + tid; i < nelem; i += kBlock) trows[i] = src[i];
+      if (nv < kHeadVoxels)
+        for (int i = nelem + tid; i < kHeadVoxels * J; i += kBlock) trows[i] = 0;
+      const uint4* wsrc = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(wide) + base * CW);
+      for (int i = tid; i < kHeadVoxels * CW / 8; i += kBlock)
+        reinterpret_cast<uint4*>(wrows)[i] = i < nv * CW / 8 ? wsrc[i] : make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int v0 = wave * 32 + ks * 16 + kg * 8;
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) h[e] = trows[(v0 + e) * J + col];
+      const uint4 tf = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+#pragma unroll
+      for (int cc = 0; cc < NC; ++cc) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] = wrows[(v0 + e) * CW + cc * 32 + col];
+        const uint4 xf = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+        acc[cc] = Mma32<T>::run(tf, xf, acc[cc]);
+      }
+    }
+    __syncthreads();
+  }
+  // Fold the four wavefronts: tile element (j, c) of wave w sits at fold[w][j][c] (rows padded to 33 floats).
+  float* fold = reinterpret_cast<float*>(wrows);
+  float* dst = part + (int64_t)blockIdx.x * J * CW;
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 8 * (r / 4) + 4 * kg + r % 4;
+      fold[(wave * 32 + j) * 33 + col] = acc[cc][r];
+    }
+    __syncthreads();
+    for (int i = tid; i < J * 32; i += kBlock) {
+      const int j = i >> 5, c = i & 31;
+      float sum = fold[j * 33 + c];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += fold[(w * 32 + j) * 33 + c];
+      dst[(int64_t)(cc * 32 + c) * a.so_wide + (int64_t)j * a.so_thin] = sum;
+    }
+    __syncthreads();
   }
 }
 
@@ -391,6 +599,20 @@ int launch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* g
   return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
 }
 
+template <typename T, int NK>
+int launch_head_wide_out_nk(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
+  const int64_t total = (int64_t)a.n * a.od * a.oh * a.ow;
+  const dim3 grid(grid_for(total, kHeadVoxels));
+  if (a.cw == 32) hipLaunchKernelGGL((head_wide_out_kernel<T, 1, NK>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, total);
+  else if (a.cw == 64) hipLaunchKernelGGL((head_wide_out_kernel<T, 2, NK>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, total);
+  else hipLaunchKernelGGL((head_wide_out_kernel<T, 4, NK>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, total);
+  return check_launch("head_wide_out_kernel");
+}
+template <typename T>
+int launch_head_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
+  return a.J <= 16 ? launch_head_wide_out_nk<T, 1>(a, thin, wt, bias, out, st) : launch_head_wide_out_nk<T, 2>(a, thin, wt, bias, out, st);
+}
+
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
 template <typename T>
 int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
@@ -398,6 +620,9 @@ int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const
     hipLaunchKernelGGL(stem_fwd_kernel<T>, dim3((unsigned)stem_tiles(a)), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt,
                        (const T*)bias, (T*)out, (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW));
     return check_launch("stem_fwd_kernel");
+  }
+  if constexpr (sizeof(T) == 2) {
+    if (a.K == 0 && (a.cw == 32 || a.cw == 64 || a.cw == 128) && ((uintptr_t)thin | (uintptr_t)out) % 16 == 0) return launch_head_wide_out<T>(a, thin, wt, bias, out, st);
   }
   if (a.K == 3) return launch_wide_out<T, 3, 27>(a, thin, wt, bias, out, st);
   if (a.K == 2) return launch_wide_out<T, 2, 8>(a, thin, wt, bias, out, st);
@@ -407,6 +632,16 @@ int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const
 }
 template <typename T>
 int dispatch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
+    const int64_t total = (int64_t)a.n * a.od * a.oh * a.ow;
+    const dim3 grid(grid_for(total, kHeadVoxels));
+    if ((a.cw == 32 || a.cw == 64 || a.cw == 128) && ((uintptr_t)wide | (uintptr_t)out) % 16 == 0) {
+      if (a.cw == 32) hipLaunchKernelGGL((head_thin_out_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)wide, (const T*)wt, (const T*)bias, (T*)out, total);
+      else if (a.cw == 64) hipLaunchKernelGGL((head_thin_out_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)wide, (const T*)wt, (const T*)bias, (T*)out, total);
+      else hipLaunchKernelGGL((head_thin_out_kernel<T, 4>), grid, dim3(kBlock), 0, st, a, (const T*)wide, (const T*)wt, (const T*)bias, (T*)out, total);
+      return check_launch("head_thin_out_kernel");
+    }
+  }
   if (a.J <= 4) return launch_thin_out<T, 4>(a, wide, wt, bias, out, st);
   if (a.J <= 16) return launch_thin_out<T, 16>(a, wide, wt, bias, out, st);
   return launch_thin_out<T, 32>(a, wide, wt, bias, out, st);
@@ -421,6 +656,19 @@ int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void*
                        (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW), ntiles, per);
     if (int rc = check_launch("stem_wgrad_kernel")) return rc;
     return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+  }
+  if constexpr (sizeof(T) == 2) {
+    if (a.K == 0 && (a.cw == 32 || a.cw == 64 || a.cw == 128) && ((uintptr_t)thin | (uintptr_t)wide) % 16 == 0) {
+      const int64_t total = (int64_t)a.n * a.od * a.oh * a.ow;
+      const int nsplit = thin_reduce_splits(a);
+      const int64_t per = cdiv(cdiv(total, nsplit), kHeadVoxels) * kHeadVoxels;  // keeps every range 16-byte aligned
+      const dim3 grid(nsplit);
+      if (a.cw == 32) hipLaunchKernelGGL((head_reduce_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
+      else if (a.cw == 64) hipLaunchKernelGGL((head_reduce_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
+      else hipLaunchKernelGGL((head_reduce_kernel<T, 4>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
+      if (int rc = check_launch("head_reduce_kernel")) return rc;
+      return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+    }
   }
   if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, gw_dtype, ws, st);
   if (a.K == 2) return launch_reduce<T, 2, 8>(a, thin, wide, gw, gw_dtype, ws, st);

@@ -26,4 +26,30 @@ template <> struct Mma32<fp16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_fp16x2(lo, hi); }
 };
 
+template <typename T>
+__device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
+
+// Stores result block `acc` (32 produced channels x 32 voxels): this lane's voxel row starts at `row`
+// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given. The two lanes of a voxel trade
+// channel runs first, so each stores two 16-byte pieces. All 64 lanes must call it; `valid` masks the stores.
+template <typename T>
+__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
+  uint32_t run[4][2];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int c = 8 * g + 4 * kg;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = acc[4 * g + i] + (bias != nullptr ? to_float(bias[c0 + c + i]) : 0.f);
+    run[g][0] = Mma32<T>::pack2(v[0], v[1]);
+    run[g][1] = Mma32<T>::pack2(v[2], v[3]);
+  }
+  uint4 piece[2];
+  trade_channel_runs(run, piece);
+  if (valid) {
+    *reinterpret_cast<uint4*>(row + 8 * kg) = piece[0];
+    *reinterpret_cast<uint4*>(row + 16 + 8 * kg) = piece[1];
+  }
+}
+
 }  // namespace sfh

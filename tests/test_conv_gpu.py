@@ -134,6 +134,9 @@ THIN_SHAPES = [
     (1, 11, 32, (5, 6, 7), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),      # thin input, wide output
     (1, 32, 32, (4, 4, 9), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),
     (1, 2, 8, (30, 30, 30), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),    # several splits in the weight gradient
+    (1, 128, 20, (3, 7, 11), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),    # two 16-channel steps on the thin side
+    (2, 20, 64, (6, 5, 9), (1, 1, 1), (1, 1, 1), (0, 0, 0), True),
+    (1, 32, 11, (3, 43, 1), (1, 1, 1), (1, 1, 1), (0, 0, 0), False),    # 129 voxels: a round of one voxel
 ]
 
 
