@@ -156,7 +156,10 @@ __device__ __forceinline__ uint4 head_weight_wide_run(const ThinArgs& a, const T
   uint16_t h[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e)
-    h[e] = j < a.J ? reinterpret_cast<const uint16_t*>(wt)[(int64_t)(c0 + e) * a.ws_wide + (int64_t)j * a.ws_thin] : (uint16_t)0;
+    h[e] = reinterpret_cast<const uint16_t*>(wt)[(int64_t)(c0 + e) * a.ws_wide + (int64_t)(j < a.J ? j : 0) * a.ws_thin];
+  if (j >= a.J)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = 0;
   return make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
 }
 // 8 consecutive thin channels from j0 of wide channel c.
@@ -165,7 +168,11 @@ __device__ __forceinline__ uint4 head_weight_thin_run(const ThinArgs& a, const T
   uint16_t h[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e)
-    h[e] = j0 + e < a.J ? reinterpret_cast<const uint16_t*>(wt)[(int64_t)c * a.ws_wide + (int64_t)(j0 + e) * a.ws_thin] : (uint16_t)0;
+  {
+    const int j = j0 + e < a.J ? j0 + e : 0;
+    const uint16_t bits = reinterpret_cast<const uint16_t*>(wt)[(int64_t)c * a.ws_wide + (int64_t)j * a.ws_thin];
+    h[e] = j0 + e < a.J ? bits : (uint16_t)0;
+  }
   return make_uint4(h[0] | (uint32_t)h[1] << 16, h[2] | (uint32_t)h[3] << 16, h[4] | (uint32_t)h[5] << 16, h[6] | (uint32_t)h[7] << 16);
 }
 
@@ -186,7 +193,8 @@ __global__ void __launch_bounds__(kBlock) head_thin_out_kernel(ThinArgs a, const
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int j = 8 * (r / 4) + 4 * kg + r % 4;
-    bv[r] = (bias != nullptr && j < J) ? to_float(bias[j]) : 0.f;
+    const float b = bias != nullptr ? to_float(bias[j < J ? j : 0]) : 0.f;
+    bv[r] = j < J ? b : 0.f;
   }
   for (int64_t base = (int64_t)blockIdx.x * kHeadVoxels; base < total; base += (int64_t)gridDim.x * kHeadVoxels) {
     const int64_t v = base + wave * 32 + col;
@@ -235,6 +243,9 @@ __global__ void __launch_bounds__(kBlock) head_wide_out_kernel(ThinArgs a, const
   for (int cc = 0; cc < NC; ++cc)
 #pragma unroll
     for (int ks = 0; ks < NK; ++ks) wf[cc][ks] = head_weight_thin_run<T>(a, wt, cc * 32 + col, ks * 16 + kg * 8);
+  float bv[NC][16];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc) load_block_bias<T>(bias, cc * 32, kg, bv[cc]);
   for (int64_t base = (int64_t)blockIdx.x * kHeadVoxels; base < total; base += (int64_t)gridDim.x * kHeadVoxels) {
     const int64_t left = total - base;
     const int nv = left < kHeadVoxels ? (int)left : kHeadVoxels;
@@ -266,7 +277,7 @@ __global__ void __launch_bounds__(kBlock) head_wide_out_kernel(ThinArgs a, const
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < NK; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[ks], acc);
-      store_block<T>(acc, dst + cc * 32, bias, cc * 32, kg, valid);
+      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid);
     }
     __syncthreads();
   }
@@ -550,6 +561,197 @@ __global__ void __launch_bounds__(kBlock) stem_wgrad_kernel(ThinArgs a, const T*
   }
 }
 
+// ---- the same stem on the matrix cores (16-bit types, 32 or 64 output channels) ---------------------------------
+// The 27 taps are the contraction (padded to 32 with zeros), the brick sits in LDS in the storage type, and a
+// wavefront owns 32 voxels along w at a time: 4 of the tile's 16 such runs.
+template <typename T>
+__device__ __forceinline__ void stem_stage_bits(const ThinArgs& a, const T* __restrict__ x, const StemTile& t, uint16_t* brick) {
+  const int id0 = t.d0 - a.pd, ih0 = t.h0 - a.ph, iw0 = t.w0 - a.pw;
+  const uint16_t* xb = reinterpret_cast<const uint16_t*>(x);
+  constexpr int kRounds = (kSBV + kBlock - 1) / kBlock;
+  // all loads of a thread are issued before the first LDS write, so their latencies overlap
+  uint16_t v[kRounds];
+#pragma unroll
+  for (int k = 0; k < kRounds; ++k) {
+    const int i = threadIdx.x + k * kBlock;
+    const int bw = i % kSBW, bh = (i / kSBW) % kSBH, bd = i / (kSBW * kSBH);
+    const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
+    // unconditional loads from a clamped address: a load under a branch would wait for the one before it
+    const bool in = i < kSBV && (unsigned)id < (unsigned)a.td && (unsigned)ih < (unsigned)a.th && (unsigned)iw < (unsigned)a.tw;
+    const uint16_t bits = xb[in ? (((int64_t)t.n * a.td + id) * a.th + ih) * a.tw + iw : 0];
+    v[k] = in ? bits : (uint16_t)0;
+  }
+#pragma unroll
+  for (int k = 0; k < kRounds; ++k) {
+    const int i = threadIdx.x + k * kBlock;
+    if (i < kSBV) brick[i] = v[k];
+  }
+}
+
+__device__ __forceinline__ uint4 pack_halves(const uint32_t (&h)[8]) {
+  return make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+}
+
+// brick offset of tap j relative to the voxel's own brick position
+__device__ __forceinline__ int stem_tap_offset(int j) { return ((j / 9) * kSBH + (j / 3) % 3) * kSBW + j % 3; }
+
+template <typename T, int NC>
+__global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const T* __restrict__ x, const T* __restrict__ wt,
+                                                               const T* __restrict__ bias, T* __restrict__ out, int tiles_d,
+                                                               int tiles_h, int tiles_w) {
+  __shared__ uint16_t brick[kSBV];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, kg = lane >> 5;
+  // result tile: rows = output channels (weights), columns = voxels (taps of the voxel)
+  uint4 wf[NC][2];
+  int off[2][8];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = ks * 16 + kg * 8 + e;
+      off[ks][e] = j < 27 ? stem_tap_offset(j) : -1;
+    }
+#pragma unroll
+    for (int cc = 0; cc < NC; ++cc) {
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = ks * 16 + kg * 8 + e;
+        const int jc = j < 27 ? j : 0;
+        const int64_t at = (int64_t)(cc * 32 + col) * a.ws_wide + (jc / 9) * a.ws_kd + ((jc / 3) % 3) * a.ws_kh + (jc % 3) * a.ws_kw;
+        const uint32_t bits = reinterpret_cast<const uint16_t*>(wt)[at];
+        h[e] = j < 27 ? bits : 0u;
+      }
+      wf[cc][ks] = pack_halves(h);
+    }
+  }
+  float bv[NC][16];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc) load_block_bias<T>(bias, cc * 32, kg, bv[cc]);
+  const StemTile t = stem_tile(a, blockIdx.x, tiles_h, tiles_w, tiles_d);
+  stem_stage_bits<T>(a, x, t, brick);
+  __syncthreads();
+#pragma unroll 1
+  for (int i = 0; i < 4; ++i) {
+    const int run = wave * 4 + i, row = run >> 1;
+    const int td = row / kSTH, th = row % kSTH, tw = (run & 1) * 32 + col;
+    const uint16_t* src = brick + (td * kSBH + th) * kSBW + tw;
+    uint4 xf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      uint32_t h[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int o = off[ks][e];
+        const uint32_t bits = src[o < 0 ? 0 : o];
+        h[e] = o < 0 ? 0u : bits;
+      }
+      xf[ks] = pack_halves(h);
+    }
+    const int od = t.d0 + td, oh = t.h0 + th, ow = t.w0 + tw;
+    const bool valid = od < a.od && oh < a.oh && ow < a.ow;
+    T* dst = out + (valid ? ((((int64_t)t.n * a.od + od) * a.oh + oh) * a.ow + ow) * a.cw : 0);
+#pragma unroll
+    for (int cc = 0; cc < NC; ++cc) {
+      f32x16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[ks], acc);
+      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid);
+    }
+  }
+}
+
+// G[c][tap] = sum_v gy[v][c] * x[v (+) tap] with the voxels as the contraction: result rows = channels (gy read
+// against its storage order from an LDS copy of the tile's rows), columns = taps (8 consecutive brick cells per lane).
+template <typename T, int NC>
+__global__ void __launch_bounds__(kBlock) stem_wgrad_mfma_kernel(ThinArgs a, const T* __restrict__ x, const T* __restrict__ gy,
+                                                                 float* __restrict__ part, int tiles_d, int tiles_h, int tiles_w,
+                                                                 int ntiles, int tiles_per_wg) {
+  constexpr int CW = NC * 32;
+  constexpr int kTileVoxels = kSTD * kSTH * kSTW;
+  constexpr int kRowPieces = kSTW * CW / 8;  // 16-byte pieces of one w-row of the tile
+  __shared__ uint16_t brick[kSBV];
+  __shared__ __align__(16) uint16_t grows[kTileVoxels * CW];
+  static_assert(sizeof(grows) >= 4 * 32 * 33 * sizeof(float), "the fold at the end reuses the gradient rows");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 31, kg = lane >> 5;
+  const int tap = stem_tap_offset(col < 27 ? col : 26);
+  f32x16_t acc[NC];
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[cc][r] = 0.f;
+  const int t_begin = blockIdx.x * tiles_per_wg;
+  int t_end = t_begin + tiles_per_wg;
+  if (t_end > ntiles) t_end = ntiles;
+  for (int tile = t_begin; tile < t_end; ++tile) {
+    const StemTile t = stem_tile(a, tile, tiles_h, tiles_w, tiles_d);
+    __syncthreads();  // the previous tile is consumed
+    stem_stage_bits<T>(a, x, t, brick);
+    constexpr int kPieceRounds = kSTD * kSTH * kRowPieces / kBlock;
+    static_assert(kSTD * kSTH * kRowPieces % (8 * kBlock) == 0, "piece rounds come in groups of 8");
+#pragma unroll 1
+    for (int k0 = 0; k0 < kPieceRounds; k0 += 8) {
+      uint4 v[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int i = tid + (k0 + k) * kBlock;
+        const int row = i / kRowPieces, p = i - row * kRowPieces;
+        const int od = t.d0 + row / kSTH, oh = t.h0 + row % kSTH, ow = t.w0 + p / (CW / 8);
+        const bool in = od < a.od && oh < a.oh && ow < a.ow;
+        const uint4 u = *reinterpret_cast<const uint4*>(
+            gy + (in ? ((((int64_t)t.n * a.od + od) * a.oh + oh) * a.ow + ow) * CW + (p % (CW / 8)) * 8 : 0));
+        v[k] = in ? u : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) reinterpret_cast<uint4*>(grows)[tid + (k0 + k) * kBlock] = v[k];
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int i = 0; i < 4; ++i) {
+      const int run = wave * 4 + i, row = run >> 1;
+      const int td = row / kSTH, th = row % kSTH;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int tw = (run & 1) * 32 + ks * 16 + kg * 8;
+        const uint16_t* xs = brick + (td * kSBH + th) * kSBW + tw + tap;
+        uint32_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] = xs[e];
+        const uint4 xf = pack_halves(h);
+        const uint16_t* gs = grows + (row * kSTW + tw) * CW + col;
+#pragma unroll
+        for (int cc = 0; cc < NC; ++cc) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = gs[e * CW + cc * 32];
+          acc[cc] = Mma32<T>::run(pack_halves(h), xf, acc[cc]);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  float* fold = reinterpret_cast<float*>(grows);
+  float* dst = part + (int64_t)blockIdx.x * 27 * CW;
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc) {
+    // result register r of this lane: channel 8 * (r / 4) + 4 * kg + r % 4, tap col
+#pragma unroll
+    for (int r = 0; r < 16; ++r) fold[(wave * 32 + 8 * (r / 4) + 4 * kg + r % 4) * 33 + col] = acc[cc][r];
+    __syncthreads();
+    for (int i = tid; i < 32 * 27; i += kBlock) {
+      const int c = i / 27, j = i - c * 27;
+      float sum = fold[c * 33 + j];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += fold[(w * 32 + c) * 33 + j];
+      dst[(int64_t)(cc * 32 + c) * a.so_wide + (int64_t)j * a.so_thin] = sum;
+    }
+    __syncthreads();
+  }
+}
+
 bool stem_brick_ok(const ThinArgs& a) {
   return a.K == 3 && a.sd == 1 && a.sh == 1 && a.sw == 1 && a.dd == 1 && a.dh == 1 && a.dw == 1 && a.pd <= 2 && a.ph <= 2 &&
          a.pw <= 2;
@@ -616,6 +818,15 @@ int launch_head_wide_out(const ThinArgs& a, const void* thin, const void* wt, co
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
 template <typename T>
 int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
+    if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL && (a.cw == 32 || a.cw == 64) && (uintptr_t)out % 16 == 0) {
+      const dim3 grid((unsigned)stem_tiles(a));
+      const int td = (int)cdiv(a.od, kSTD), th = (int)cdiv(a.oh, kSTH), tw = (int)cdiv(a.ow, kSTW);
+      if (a.cw == 32) hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw);
+      else hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw);
+      return check_launch("stem_fwd_mfma_kernel");
+    }
+  }
   if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
     hipLaunchKernelGGL(stem_fwd_kernel<T>, dim3((unsigned)stem_tiles(a)), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt,
                        (const T*)bias, (T*)out, (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW));
@@ -648,6 +859,18 @@ int dispatch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const
 }
 template <typename T>
 int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
+    if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL && (a.cw == 32 || a.cw == 64) && (uintptr_t)wide % 16 == 0) {
+      const int nsplit = thin_reduce_splits(a);
+      const int ntiles = (int)stem_tiles(a);
+      const int per = (int)cdiv(ntiles, nsplit);
+      const int td = (int)cdiv(a.od, kSTD), th = (int)cdiv(a.oh, kSTH), tw = (int)cdiv(a.ow, kSTW);
+      if (a.cw == 32) hipLaunchKernelGGL((stem_wgrad_mfma_kernel<T, 1>), dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, td, th, tw, ntiles, per);
+      else hipLaunchKernelGGL((stem_wgrad_mfma_kernel<T, 2>), dim3(nsplit), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, td, th, tw, ntiles, per);
+      if (int rc = check_launch("stem_wgrad_mfma_kernel")) return rc;
+      return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+    }
+  }
   if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
     const int nsplit = thin_reduce_splits(a);
     const int ntiles = (int)stem_tiles(a);

@@ -29,20 +29,17 @@ template <> struct Mma32<fp16_t> {
 template <typename T>
 __device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
 
-// Stores result block `acc` (32 produced channels x 32 voxels): this lane's voxel row starts at `row`
-// (element pointer at channel 0 of the block); adds bias[c0 + channel] when given. The two lanes of a voxel trade
-// channel runs first, so each stores two 16-byte pieces. All 64 lanes must call it; `valid` masks the stores.
+// Stores result block `acc` (32 produced channels x 32 voxels) plus `add` (same register layout: register r of
+// this lane is channel 8 * (r / 4) + 4 * kg + r % 4): this lane's voxel row starts at `row` (element pointer at
+// channel 0 of the block). The two lanes of a voxel trade channel runs first, so each stores two 16-byte pieces.
+// All 64 lanes must call it; `valid` masks the stores.
 template <typename T>
-__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
+__device__ __forceinline__ void store_block_plus(const f32x16_t& acc, T* row, const float (&add)[16], int kg, bool valid) {
   uint32_t run[4][2];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const int c = 8 * g + 4 * kg;
-    float v[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = acc[4 * g + i] + (bias != nullptr ? to_float(bias[c0 + c + i]) : 0.f);
-    run[g][0] = Mma32<T>::pack2(v[0], v[1]);
-    run[g][1] = Mma32<T>::pack2(v[2], v[3]);
+    run[g][0] = Mma32<T>::pack2(acc[4 * g] + add[4 * g], acc[4 * g + 1] + add[4 * g + 1]);
+    run[g][1] = Mma32<T>::pack2(acc[4 * g + 2] + add[4 * g + 2], acc[4 * g + 3] + add[4 * g + 3]);
   }
   uint4 piece[2];
   trade_channel_runs(run, piece);
@@ -50,6 +47,28 @@ __device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T
     *reinterpret_cast<uint4*>(row + 8 * kg) = piece[0];
     *reinterpret_cast<uint4*>(row + 16 + 8 * kg) = piece[1];
   }
+}
+
+// This lane's 16 bias values of the channel block from c0 (zeros without a bias), in result-register order.
+template <typename T>
+__device__ __forceinline__ void load_block_bias(const T* bias, int c0, int kg, float (&add)[16]) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) add[r] = 0.f;
+  if (bias != nullptr) {
+    T b[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) b[r] = bias[c0 + 8 * (r / 4) + 4 * kg + r % 4];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) add[r] = to_float(b[r]);
+  }
+}
+
+// As store_block_plus with bias[c0 + channel] (when given) as the addend.
+template <typename T>
+__device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
+  float add[16];
+  load_block_bias<T>(bias, c0, kg, add);
+  store_block_plus<T>(acc, row, add, kg, valid);
 }
 
 }  // namespace sfh
