@@ -116,6 +116,19 @@ int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w,
                             const int64_t w_stride[5], void* packed_fwd, void* packed_dgrad,
                             void* stream);
 
+/* The packings of many weights in as few launches as possible (a training loop repacks every
+ * convolution weight once per optimizer step). Each item is one sfh_conv3d_pack_weights call;
+ * all weights share `dtype`. No counterpart in the reference. */
+typedef struct sfh_pack_item {
+  sfh_conv3d_desc desc;
+  const void* w;
+  int64_t w_stride[5];
+  void* packed_fwd;   /* may be NULL */
+  void* packed_dgrad; /* may be NULL */
+} sfh_pack_item;
+int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t nitems, int dtype,
+                                  void* stream);
+
 /* ---- conv3d weight gradient ----------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_backward_weight (triton_conv3d/reduce_gemm.py:1177),
  * _conv3d_bwd_weight_kernel (:137) and _reduce_partials_kernel (:396).

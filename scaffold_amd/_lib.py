@@ -60,6 +60,11 @@ class ConvDesc(ctypes.Structure):
         "sd", "sh", "sw", "pd", "ph", "pw", "dd", "dh", "dw")]
 
 
+class PackItem(ctypes.Structure):
+    _fields_ = [("desc", ConvDesc), ("w", c_void_p), ("w_stride", c_int64 * 5), ("packed_fwd", c_void_p),
+                ("packed_dgrad", c_void_p)]
+
+
 class ConvTDesc(ctypes.Structure):
     _fields_ = [(k, c_int32) for k in ("n", "cin", "in_d", "in_h", "in_w", "cout", "kd", "kh", "kw")]
 
@@ -102,6 +107,7 @@ _SIGNATURES = {
                                  c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_packed_weight_bytes": (c_size_t, [POINTER(ConvDesc), c_int, c_int]),
     "sfh_conv3d_pack_weights": (c_int, [POINTER(ConvDesc), c_int, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_void_p]),
+    "sfh_conv3d_pack_weights_batch": (c_int, [POINTER(PackItem), c_int32, c_int, c_void_p]),
     "sfh_conv3d_wgrad_splits": (c_int, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_wgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_wgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,

@@ -49,7 +49,7 @@ __all__ = [
     "bwd_data_padding",
     "grad_weight_empty",
     "workspace_elements",
-    "pack_weights",
+    "pack_weights", "pack_weights_batch", "PackedWeights",
     "packed_weight_bytes",
     "split_count",
     "uses_mfma",
@@ -335,11 +335,7 @@ def packed_weight_bytes(in_shape, weight_shape, stride, padding, dilation, dtype
 _PACK_PLAN_CACHE: dict = {}
 
 
-def pack_weights(w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1, *, forward: bool = True, backward_data: bool = True):
-    """Packs ``w`` once, in one launch, for the forward and / or the data gradient of the convolution of an input of
-    ``in_shape``: returns ``(packed_fwd, packed_dgrad)`` to pass as ``packed_weight=``; an entry is ``None`` when it
-    was not asked for or when that direction of the problem does not read a packed weight (it then takes ``w``).
-    The default entry points repack on every call; a train step that packs once here saves a launch per convolution."""
+def _pack_plan(w, in_shape, stride, padding, dilation):
     key = (in_shape, w.shape, stride, padding, dilation, w.dtype)
     try:
         plan = _PACK_PLAN_CACHE.get(key)
@@ -355,9 +351,24 @@ def pack_weights(w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1, *, 
             if len(_PACK_PLAN_CACHE) > 4096:
                 _PACK_PLAN_CACHE.clear()
             _PACK_PLAN_CACHE[key] = plan
-    nbf, nbd, desc, code = plan
-    pf = torch.empty(nbf, dtype=torch.uint8, device=w.device) if (forward and nbf) else None
-    pd = torch.empty(nbd, dtype=torch.uint8, device=w.device) if (backward_data and nbd) else None
+    return plan
+
+
+def pack_weights(w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1, *, forward: bool = True, backward_data: bool = True,
+                 out=None):
+    """Packs ``w`` once, in one launch, for the forward and / or the data gradient of the convolution of an input of
+    ``in_shape``: returns ``(packed_fwd, packed_dgrad)`` to pass as ``packed_weight=``; an entry is ``None`` when it
+    was not asked for or when that direction of the problem does not read a packed weight (it then takes ``w``).
+    ``out=(packed_fwd, packed_dgrad)`` reuses the buffers of an earlier call for the same problem.
+    The default entry points repack on every call; a train step that packs once here saves a launch per convolution."""
+    nbf, nbd, desc, code = _pack_plan(w, in_shape, stride, padding, dilation)
+    if out is not None:
+        pf, pd = out
+        if (pf is not None and pf.numel() != nbf) or (pd is not None and pd.numel() != nbd):
+            raise ValueError("pack_weights: out= buffers are not those of this problem")
+    else:
+        pf = torch.empty(nbf, dtype=torch.uint8, device=w.device) if (forward and nbf) else None
+        pd = torch.empty(nbd, dtype=torch.uint8, device=w.device) if (backward_data and nbd) else None
     if pf is None and pd is None:
         return None, None
     with _lib.device_guard(w.device):
@@ -366,6 +377,82 @@ def pack_weights(w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1, *, 
     if rc:
         _lib.check(rc, "pack_weights")
     return pf, pd
+
+
+class PackedWeights:
+    """Both packed forms of one convolution weight for one problem, in buffers that live as long as this object, so
+    that whoever changes the weight can refresh them in place (``repack`` / ``pack_weights_batch``).
+
+    ``source`` is the tensor the forms were packed from; ``version`` is a stamp for the caller's own validity rule
+    (``FastConv3d`` stores the version counter of the parameter there); ``maintained`` says that the writer of the
+    weight refreshes the forms itself after every change."""
+
+    __slots__ = ("source", "problem", "fwd", "dgrad", "version", "maintained")
+
+    #: bumped whenever an instance is created or packs from another source: holders of batch plans rebuild on change
+    generation = 0
+
+    def __init__(self, w: torch.Tensor, in_shape, stride=1, padding=0, dilation=1):
+        self.problem = (tuple(int(v) for v in in_shape), stride, padding, dilation)
+        self.source = None
+        self.version = None
+        self.maintained = False
+        self.fwd, self.dgrad = pack_weights(w, self.problem[0], stride, padding, dilation)
+        self.source = w
+        PackedWeights.generation += 1
+
+    def __bool__(self):
+        return self.fwd is not None or self.dgrad is not None
+
+    def repack(self, w: Optional[torch.Tensor] = None) -> None:
+        """Packs again from ``w`` (default: the same source) into the same buffers."""
+        if w is not None and w is not self.source:
+            if w.shape != self.source.shape or w.dtype is not self.source.dtype or w.device != self.source.device:
+                raise ValueError("PackedWeights.repack: the new source is a different problem")
+            self.source = w
+            PackedWeights.generation += 1
+        if self:
+            pack_weights(self.source, self.problem[0], *self.problem[1:], out=(self.fwd, self.dgrad))
+
+
+def pack_weights_batch(packs):
+    """Refreshes many ``PackedWeights`` in as few launches as possible.  Returns a plan to pass back as ``packs`` the
+    next time (it holds the prepared argument list; valid while no source tensor is replaced)."""
+    if not isinstance(packs, _PackBatchPlan):
+        packs = _PackBatchPlan(packs)
+    packs.run()
+    return packs
+
+
+class _PackBatchPlan:
+    def __init__(self, packs):
+        self.generation = PackedWeights.generation
+        groups = {}
+        for e in packs:
+            if e:
+                groups.setdefault((e.source.device, e.source.dtype), []).append(e)
+        self.groups = []
+        for (device, dtype), entries in groups.items():
+            items = (_lib.PackItem * len(entries))()
+            for it, e in zip(items, entries):
+                w = e.source
+                _, _, desc, _ = _pack_plan(w, e.problem[0], *e.problem[1:])
+                it.desc = desc
+                it.w = w.data_ptr()
+                for i, v in enumerate(_lib.strides5(w)):
+                    it.w_stride[i] = v
+                it.packed_fwd = None if e.fwd is None else e.fwd.data_ptr()
+                it.packed_dgrad = None if e.dgrad is None else e.dgrad.data_ptr()
+            # the entries are held so that the addresses in `items` stay valid
+            self.groups.append((device, _lib.dtype_code(dtype), items, len(entries), entries))
+
+    def run(self):
+        L = _lib.lib()
+        for device, code, items, n, _ in self.groups:
+            with _lib.device_guard(device):
+                rc = L.sfh_conv3d_pack_weights_batch(items, n, code, _lib.stream_ptr(device))
+            if rc:
+                _lib.check(rc, "pack_weights_batch")
 
 
 # ---------------------------------------------------------------------------------------------

@@ -2,6 +2,7 @@
 // function of descriptor and dtype), workspace carving. No allocation, no synchronisation.
 #include <string.h>
 
+#include <vector>
 #include "common.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
@@ -353,6 +354,32 @@ extern "C" int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, cons
   const MfmaConvArgs fa = packed_fwd != nullptr ? fwd_mfma_args(*p, out) : MfmaConvArgs{};
   const MfmaConvArgs da = packed_dgrad != nullptr ? dgrad_mfma_args(*p, out) : MfmaConvArgs{};
   return mfma_pack_weight_pair(fa, da, dtype, w, w_stride, packed_fwd, packed_dgrad, (hipStream_t)stream);
+}
+
+extern "C" int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t nitems, int dtype, void* stream) {
+  if (nitems < 0 || (nitems > 0 && items == nullptr)) return fail(SFH_ERR_INVALID, "conv3d pack batch: bad item list");
+  std::vector<MfmaPackItem> jobs;
+  jobs.reserve((size_t)nitems * 2);
+  for (int i = 0; i < nitems; ++i) {
+    const sfh_pack_item& it = items[i];
+    int32_t out[3];
+    if (int rc = check_conv(&it.desc, dtype, out)) return rc;
+    if (it.w == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack batch: item %d has a null weight", i);
+    if (it.packed_fwd != nullptr) {
+      if (!fwd_uses_mfma(it.desc, dtype, out))
+        return fail(SFH_ERR_UNSUPPORTED, "conv3d pack batch: the forward of item %d does not read a packed weight", i);
+      jobs.push_back(MfmaPackItem{fwd_mfma_args(it.desc, out), it.w, it.w_stride[0], it.w_stride[1], it.w_stride[2], it.w_stride[3],
+                                  it.w_stride[4], 0, it.packed_fwd});
+    }
+    if (it.packed_dgrad != nullptr) {
+      if (!(check_dgrad(it.desc) == SFH_OK && dgrad_uses_mfma(it.desc, dtype, out)))
+        return fail(SFH_ERR_UNSUPPORTED, "conv3d pack batch: the data gradient of item %d does not read a packed weight", i);
+      jobs.push_back(MfmaPackItem{dgrad_mfma_args(it.desc, out), it.w, it.w_stride[1], it.w_stride[0], it.w_stride[2], it.w_stride[3],
+                                  it.w_stride[4], 1, it.packed_dgrad});
+    }
+  }
+  if (jobs.empty()) return SFH_OK;
+  return mfma_pack_weight_batch(jobs.data(), (int)jobs.size(), dtype, (hipStream_t)stream);
 }
 
 // ---- data gradient ---------------------------------------------------------------------

@@ -288,6 +288,22 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(PackJob first, PackJob
   else if (idx - first.pieces < second.pieces) pack_piece<T>(second, idx - first.pieces);
 }
 
+// Many packings in one launch: a workgroup finds its job from the table of first workgroups.
+constexpr int kPackBatch = 16;
+struct PackBatch {
+  PackJob job[kPackBatch];
+  int first_block[kPackBatch + 1];
+  int njobs;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) pack_weight_batch_kernel(PackBatch b) {
+  int j = 0;
+  while (j + 1 < b.njobs && (int)blockIdx.x >= b.first_block[j + 1]) ++j;
+  const int64_t idx = (int64_t)((int)blockIdx.x - b.first_block[j]) * 256 + threadIdx.x;
+  if (idx < b.job[j].pieces) pack_piece<T>(b.job[j], idx);
+}
+
 struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
 
 // Launch geometry, a pure function of the problem: brick shape by row length; two output blocks per workgroup
@@ -393,6 +409,29 @@ int mfma_pack_weight_pair(const MfmaConvArgs& fwd, const MfmaConvArgs& dgrad, in
   if (packed_dgrad != nullptr)
     second = pack_job(dgrad, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, packed_dgrad);
   return launch_pack(dtype, first, second, st);
+}
+
+int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStream_t st) {
+  for (int i0 = 0; i0 < n; i0 += kPackBatch) {
+    PackBatch b{};
+    int64_t blocks = 0;
+    for (int i = i0; i < n && i < i0 + kPackBatch; ++i) {
+      const MfmaPackItem& it = items[i];
+      const PackJob job = pack_job(it.a, it.w, it.s_out, it.s_red, it.s_kd, it.s_kh, it.s_kw, it.flip, it.packed);
+      if (job.pieces <= 0) continue;
+      b.job[b.njobs] = job;
+      b.first_block[b.njobs] = (int)blocks;
+      blocks += cdiv(job.pieces, 256);
+      ++b.njobs;
+      if (blocks > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: batch too large");
+    }
+    b.first_block[b.njobs] = (int)blocks;
+    if (b.njobs == 0) continue;
+    if (dtype == SFH_BF16) hipLaunchKernelGGL(pack_weight_batch_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, st, b);
+    else hipLaunchKernelGGL(pack_weight_batch_kernel<fp16_t>, dim3((unsigned)blocks), dim3(256), 0, st, b);
+    if (int rc = check_launch("pack_weight_batch_kernel")) return rc;
+  }
+  return SFH_OK;
 }
 
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {

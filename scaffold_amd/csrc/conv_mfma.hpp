@@ -22,6 +22,15 @@ size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a);
 // strides of the source for the produced channel, the reduction channel and the taps.
 int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_out, int64_t s_red, int64_t s_kd,
                      int64_t s_kh, int64_t s_kw, int flip, void* packed, hipStream_t st);
+// Any number of packings (of any weights) in as few launches as the kernel argument space allows.
+struct MfmaPackItem {
+  MfmaConvArgs a;
+  const void* w;
+  int64_t s_out, s_red, s_kd, s_kh, s_kw;
+  int flip;
+  void* packed;
+};
+int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStream_t st);
 // Both packings of one weight (either output may be null) in one launch: the forward's and the data gradient's.
 int mfma_pack_weight_pair(const MfmaConvArgs& fwd, const MfmaConvArgs& dgrad, int dtype, const void* w, const int64_t w_stride[5],
                           void* packed_fwd, void* packed_dgrad, hipStream_t st);

@@ -76,6 +76,34 @@ def compute_copy(param: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
     return copy
 
 
+def _current_packs(owner: torch.Tensor, source: torch.Tensor, x: torch.Tensor, stride, padding, dilation):
+    """The packed forms of a parameter's weight for this problem, or ``None`` when the problem reads no packed weight.
+
+    They are kept on the parameter (``owner._sfh_packs``) and trusted without a launch only under the rule that also
+    guards the optimizer's half-precision copies: the optimizer that writes the parameter refreshes them inside its
+    step (``maintained``) and nothing else has written the parameter since (torch's version counter).  Otherwise they
+    are packed again here, in one launch for both directions."""
+    if source.dtype is torch.float32:
+        return None
+    table = owner.__dict__.get("_sfh_packs")
+    if table is None:
+        table = owner._sfh_packs = {}
+    key = (x.shape, padding)
+    e = table.get(key)
+    if e is None:
+        if len(table) >= 8:  # a parameter meets few problems; shapes that keep changing are not worth the buffers
+            table.clear()
+        e = table[key] = _c3.PackedWeights(source, x.shape, stride, padding, dilation)
+        e.version = owner._version
+        return e if e else None
+    if not e:
+        return None
+    if not (e.maintained and e.version == owner._version and e.source is source):
+        e.repack(source)
+        e.version = owner._version
+    return e
+
+
 def _fp32_weight_grad(fn, *args, **kwargs):
     """Weight gradient straight in fp32 where the tiled kernels serve the shape, else in the operands' dtype and
     widened afterwards (what autocast's cast node would have done)."""
@@ -90,16 +118,19 @@ class _Conv3dFn(torch.autograd.Function):
     autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None):
+    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
         bc = bias if bias_compute is None else bias_compute
-        # When the data gradient will be wanted too, the weight can be packed for both directions in one launch. That
-        # saves a launch per convolution on the GPU and costs a little more host time, so it is done where host time
-        # is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
         pf = pd = None
-        if ctx.needs_input_grad[0] and (PACK_WEIGHTS_ONCE or torch.cuda.is_current_stream_capturing()):
+        if packs is not None:
+            # packed forms that are current (kept by the module, refreshed by whoever writes the weight)
+            pf, pd = packs.fwd, packs.dgrad
+        elif ctx.needs_input_grad[0] and (PACK_WEIGHTS_ONCE or torch.cuda.is_current_stream_capturing()):
+            # When the data gradient will be wanted too, the weight can be packed for both directions in one launch.
+            # That saves a launch per convolution on the GPU and costs a little more host time, so it is done where
+            # host time is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
             pf, pd = _c3.pack_weights(wc, x.shape, stride, padding, dilation)
         y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, _checked=True)
         ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
@@ -124,7 +155,7 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
@@ -190,9 +221,13 @@ class FastConv3d(nn.Conv3d):
                 f"FastConv3d: not served: x={tuple(x.shape)}/{x.dtype} on {x.device}, weight={tuple(w.shape)}/{w.dtype}, "
                 f"stride={self.stride} padding={padding} dilation={self.dilation} groups={self.groups}"
             )
+        stride, dilation = tuple(self.stride), tuple(self.dilation)
         if master:
-            return _Conv3dFn.apply(x, self.weight, self.bias, tuple(self.stride), padding, tuple(self.dilation), w, b)
-        return _Conv3dFn.apply(x, w, b, tuple(self.stride), padding, tuple(self.dilation))
+            return _Conv3dFn.apply(x, self.weight, self.bias, stride, padding, dilation, w, b,
+                                   _current_packs(self.weight, w, x, stride, padding, dilation))
+        if w is self.weight:
+            return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, _current_packs(w, w, x, stride, padding, dilation))
+        return _Conv3dFn.apply(x, w, b, stride, padding, dilation)
 
 
 class FastConvTranspose3d(nn.ConvTranspose3d):

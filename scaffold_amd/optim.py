@@ -58,6 +58,7 @@ class FusedClipAdam(torch.optim.Optimizer):
         self.grad_norm = None
         self._slots = None
         self._plans = {}
+        self._pack_plan = None
 
     @torch.no_grad()
     def refresh_shadows(self):
@@ -184,7 +185,29 @@ class FusedClipAdam(torch.optim.Optimizer):
                 for p in params:  # the kernel wrote parameter and copy together
                     p._sfh_shadow = self.shadow[p]
                     p._sfh_shadow_version = p._version
+            self._refresh_packs(params)
         return loss
+
+    def _refresh_packs(self, params):
+        """Packed forms of convolution weights that the modules keep on the parameters (``p._sfh_packs``) are derived
+        from what this step just wrote: they are packed again here, all in one batch, and stamped as current."""
+        from . import conv3d as _c3
+        plan = self._pack_plan
+        if plan is None or plan[0] != _c3.PackedWeights.generation or plan[1] is not params:
+            pairs = []
+            for p in params:
+                table = p.__dict__.get("_sfh_packs")
+                if table:
+                    src = self.shadow.get(p) if self.shadow_dtype is not None else p
+                    pairs.extend((p, e) for e in table.values() if e and e.source is src)
+            batch = _c3._PackBatchPlan([e for _, e in pairs]) if pairs else None
+            plan = self._pack_plan = (_c3.PackedWeights.generation, params, pairs, batch)
+        _, _, pairs, batch = plan
+        if batch is not None:
+            batch.run()
+            for p, e in pairs:
+                e.version = p._version
+                e.maintained = True
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)

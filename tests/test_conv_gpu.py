@@ -455,6 +455,33 @@ def test_prepacked_weight_gives_the_same_bits(device, cin, cout, sp, pad):
     assert none_d is None and torch.equal(only_f, pf)
 
 
+def test_batch_packing_gives_the_same_bits(device):
+    """Many weights packed in a few launches (more jobs than one launch's table holds), also on a second run of the
+    same plan after the weights changed in place, and with layouts and dtypes mixed."""
+    from scaffold_amd import conv3d as C
+    g = torch.Generator().manual_seed(67)
+    packs = []
+    for i in range(11):
+        cin, cout = (32, 64, 96)[i % 3], (64, 32, 128)[i % 3]
+        dtype = torch.float16 if i % 4 == 3 else torch.bfloat16
+        w = (torch.randn((cout, cin, 3, 3, 3), generator=g) * 0.05).to(dtype).to(device)
+        if i % 2 == 0:
+            w = w.contiguous(memory_format=CL)
+        packs.append(C.PackedWeights(w, (1, cin, 4 + i, 8, 16), 1, 1, 1))
+    packs.append(C.PackedWeights(torch.randn((7, 5, 3, 3, 3), device=device).to(torch.bfloat16), (1, 5, 8, 8, 8), 1, 1, 1))
+    assert not packs[-1] and all(packs[:-1])
+    plan = None
+    for round_ in range(2):
+        want = [sa.pack_weights(e.source, e.problem[0], 1, 1, 1) for e in packs[:-1]]
+        for e in packs[:-1]:
+            e.fwd.zero_(), e.dgrad.zero_()
+        plan = C.pack_weights_batch(packs if plan is None else plan)
+        for e, (pf, pd) in zip(packs, want):
+            assert torch.equal(e.fwd, pf) and torch.equal(e.dgrad, pd)
+        for e in packs[:-1]:
+            e.source.mul_(-0.5)
+
+
 def test_pack_weights_declines_problems_that_read_the_weight_where_it_lies(device):
     w5 = torch.randn((7, 5, 3, 3, 3), device=device).to(torch.bfloat16)
     assert sa.pack_weights(w5, (1, 5, 8, 8, 8), 1, 1, 1) == (None, None)

@@ -268,3 +268,64 @@ def test_packing_the_weight_once_per_step_changes_no_bits(device):
 
     a, b = grads(False), grads(True)
     assert all(torch.equal(p, q) for p, q in zip(a, b))
+
+
+def _fused_adam_run(device, steps):
+    _, ours, x, lab = _two_arms(device, torch.bfloat16, shard=True)
+    opt = sa.FusedClipAdam(ours.parameters(), lr=1e-2, max_norm=1.0, shadow_dtype=torch.bfloat16)
+    xd, labd = x.to(device).contiguous(memory_format=CL), lab.to(device)
+    losses = []
+    for _ in range(steps):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = ours(xd)
+        loss = sa.ce_dice_loss(logits, labd)
+        loss.backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        losses.append(loss.item())
+    return ours, losses
+
+
+def test_packed_weights_kept_by_the_optimizer_change_no_bits(device, monkeypatch):
+    """FusedClipAdam repacks the convolution weights inside its step and the modules then launch no packing of their
+    own: the run must equal, bit for bit, one in which every call packs for itself."""
+    import scaffold_amd.modules as mods
+    kept, a = _fused_adam_run(device, 4)
+    entries = [e for p in kept.parameters() for e in getattr(p, "_sfh_packs", {}).values() if e]
+    assert entries and all(e.maintained for e in entries)
+    assert all(e.version == p._version for p in kept.parameters() for e in getattr(p, "_sfh_packs", {}).values() if e)
+    monkeypatch.setattr(mods, "_current_packs", lambda *args, **kwargs: None)
+    plain, b = _fused_adam_run(device, 4)
+    assert not any(hasattr(p, "_sfh_packs") for p in plain.parameters())
+    assert a == b and a[0] != a[-1]
+    assert all(torch.equal(p, q) for p, q in zip(kept.parameters(), plain.parameters()))
+
+
+def test_kept_packed_weights_are_not_trusted_after_a_foreign_write(device):
+    torch.manual_seed(3)
+    conv = sa.FastConv3d(32, 32, 3, padding=1, bias=False).to(device).to(memory_format=CL)
+    opt = sa.FusedClipAdam(conv.parameters(), lr=1e-2, shadow_dtype=torch.bfloat16)
+    x = torch.randn(1, 32, 8, 16, 16, device=device).to(torch.bfloat16).contiguous(memory_format=CL).requires_grad_()
+    for _ in range(2):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = conv(x)
+        y.float().square().mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    (entry,) = conv.weight._sfh_packs.values()
+    assert entry.maintained and entry.version == conv.weight._version
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(conv(x), sa.conv3d_forward(x.detach(), conv.weight.detach().to(torch.bfloat16), None, 1, 1, 1))
+    with torch.no_grad():
+        conv.weight.mul_(-0.5)                    # not the optimizer: the copies and packed forms are stale now
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = conv(x)                               # the per-call cast path
+    want = sa.conv3d_forward(x.detach(), conv.weight.detach().to(torch.bfloat16), None, 1, 1, 1)
+    assert torch.equal(y, want)
+    opt.refresh_shadows()                         # the copies are current again, the packed forms are repacked on use
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = conv(x)
+    assert torch.equal(y, want)
+    x.grad = None
+    y.float().sum().backward()
+    assert torch.equal(x.grad, sa.conv3d_backward_data(torch.ones_like(want), conv.weight.detach().to(torch.bfloat16), x.shape, 1, 1, 1))
