@@ -169,6 +169,16 @@ size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtyp
 int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
                       const void* x, const void* gamma, const void* beta, void* y, float* mean,
                       float* rstd, void* workspace, size_t workspace_bytes, void* stream);
+/* The same with the result written into the interior of a slab: y_slab is
+ * (N, halo_rows + S + halo_rows, C) and its two faces of halo_rows rows per sample are set to
+ * zero. With S = D*H*W and halo_rows = h*H*W that is the input a depth shard's convolution reads
+ * after the halo exchange (ScaFFold/unet/conv3d.py:648-677), produced without a copy of the
+ * interior; a neighbour's planes, where there is one, overwrite the zero faces. The output must
+ * have the input's element width. Same workspace as sfh_groupnorm_fwd. */
+int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
+                           const void* x, const void* gamma, const void* beta, void* y_slab,
+                           int64_t halo_rows, float* mean, float* rstd, void* workspace,
+                           size_t workspace_bytes, void* stream);
 
 /* ---- GroupNorm backward --------------------------------------------------------------
  * Stands in for torch.ops.scaffold_gn.group_norm_backward (triton_group_norm.py:1394) and
@@ -232,6 +242,23 @@ typedef struct sfh_halo_desc {
 } sfh_halo_desc;
 int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* x, const void* lo,
                       const void* hi, void* out, void* stream);
+
+/* ---- skip connection concat ---------------------------------------------------------------
+ * torch.cat([skip, upsampled], dim=1) of the decoder (ScaFFold/unet/unet_parts.py:107-120) on
+ * channels-last tensors, one streaming pass: out (N, halo_rows + rows + halo_rows, c_a + c_b) gets
+ * [a (N, rows, c_a) | b (N, rows, c_b)] in its interior and zeros in its faces. With rows = D*H*W
+ * and halo_rows = h*H*W the result is the slab a depth shard's convolution reads (see
+ * sfh_halo_assemble); halo_rows = 0 is the plain concatenation. The backward copies the two channel
+ * ranges of the interior of g (laid out like out) into ga and gb. Both channel counts must fill
+ * whole 16-byte pieces of `dtype`; pointers 16-byte aligned. */
+typedef struct sfh_concat_desc {
+  int32_t n, c_a, c_b;
+  int64_t rows, halo_rows;
+} sfh_concat_desc;
+int sfh_skip_concat_fwd(const sfh_concat_desc* p, int dtype, const void* a, const void* b, void* out,
+                        void* stream);
+int sfh_skip_concat_bwd(const sfh_concat_desc* p, int dtype, const void* g, void* ga, void* gb,
+                        void* stream);
 
 /* ---- gradient clipping + Adam -----------------------------------------------------------
  * The optimizer step of the trainer: torch.nn.utils.clip_grad_norm_(parameters, max_norm) followed by

@@ -4,6 +4,7 @@
 
 #include <vector>
 #include "common.hpp"
+#include "concat.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
 #include "conv_patch.hpp"
@@ -624,6 +625,32 @@ extern "C" int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* 
   if (p->n == 0) return SFH_OK;
   if (x == nullptr || out == nullptr) return fail(SFH_ERR_INVALID, "halo assemble: null tensor");
   return halo_assemble(*p, dtype, x, lo, hi, out, (hipStream_t)stream);
+}
+
+// ---- skip connection concat ------------------------------------------------------------------
+static int check_concat(const sfh_concat_desc* p, int dtype) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "skip concat: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "skip concat: bad dtype %d", dtype);
+  if (p->n < 0 || p->c_a < 1 || p->c_b < 1 || p->rows < 1 || p->halo_rows < 0)
+    return fail(SFH_ERR_INVALID, "skip concat: bad extents n=%d channels=(%d, %d) rows=%lld halo_rows=%lld", p->n, p->c_a, p->c_b,
+                (long long)p->rows, (long long)p->halo_rows);
+  if (p->n > 0 && !concat_supported(*p, dtype))
+    return fail(SFH_ERR_UNSUPPORTED, "skip concat: channel counts (%d, %d) do not fill 16-byte pieces", p->c_a, p->c_b);
+  return SFH_OK;
+}
+
+extern "C" int sfh_skip_concat_fwd(const sfh_concat_desc* p, int dtype, const void* a, const void* b, void* out, void* stream) {
+  if (int rc = check_concat(p, dtype)) return rc;
+  if (p->n == 0) return SFH_OK;
+  if (a == nullptr || b == nullptr || out == nullptr) return fail(SFH_ERR_INVALID, "skip concat: null tensor");
+  return concat_forward(*p, dtype, a, b, out, (hipStream_t)stream);
+}
+
+extern "C" int sfh_skip_concat_bwd(const sfh_concat_desc* p, int dtype, const void* g, void* ga, void* gb, void* stream) {
+  if (int rc = check_concat(p, dtype)) return rc;
+  if (p->n == 0) return SFH_OK;
+  if (g == nullptr || ga == nullptr || gb == nullptr) return fail(SFH_ERR_INVALID, "skip concat: null tensor");
+  return concat_backward(*p, dtype, g, ga, gb, (hipStream_t)stream);
 }
 
 // ---- gradient clipping + Adam ------------------------------------------------------------

@@ -297,7 +297,7 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
                                                        float* __restrict__ rstd, const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
                                                        int tpr, int rpp, int nsplit, int64_t rows_per_split, float m, float eps,
-                                                       int relu) {
+                                                       int relu, int64_t y_halo) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float gstat[];  // sums[2 G] | mean[G] | rstd[G] | fold scratch (4 * kBlock)
   const int tid = threadIdx.x;
@@ -328,6 +328,17 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
     }
   }
   __syncthreads();
+  // y is a slab of y_halo + S + y_halo rows per sample: the sample's workgroups zero the two faces between them
+  const int64_t y_sample = (int64_t)n * (S + 2 * y_halo) * C;
+  if (y_halo > 0) {
+    const int64_t face_pieces = y_halo * C * (int64_t)sizeof(TO) / 16;
+    uint4* lo = reinterpret_cast<uint4*>(y + y_sample);
+    uint4* hi = reinterpret_cast<uint4*>(y + y_sample + (y_halo + S) * C);
+    for (int64_t u = (int64_t)blockIdx.x * kBlock + tid; u < face_pieces; u += (int64_t)gridDim.x * kBlock) {
+      lo[u] = make_uint4(0, 0, 0, 0);
+      hi[u] = make_uint4(0, 0, 0, 0);
+    }
+  }
   if (r >= rpp) return;
   float mu[V], rs[V], ga[V], be[V];
 #pragma unroll
@@ -338,9 +349,8 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
     ga[e] = load_param(gamma, param_dtype, c, 1.f);
     be[e] = load_param(beta, param_dtype, c, 0.f);
   }
-  const int64_t base = (int64_t)n * S * C + cv * V;
-  const T* xs = x + base;
-  TO* ys = y + base;
+  const T* xs = x + (int64_t)n * S * C + cv * V;
+  TO* ys = y + y_sample + y_halo * C + cv * V;
   const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
   int64_t end = begin + rows_per_split;
   if (end > S) end = S;
@@ -796,9 +806,11 @@ size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
 
 template <typename T, typename TO>
 int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
-              void* y, float* mean, float* rstd, float* ws, hipStream_t st) {
+              void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st) {
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
+  if (y_halo > 0 && (!pl.vector || sizeof(T) != sizeof(TO) || (y_halo * C * sizeof(TO)) % 16 != 0))
+    return fail(SFH_ERR_UNSUPPORTED, "groupnorm: the slab output needs the vector path and an output of the input's width");
   if (!pl.vector) {
     hipLaunchKernelGGL(gn_scalar_stats<T>, dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, mean, rstd, S, C, G, p.eps);
     if (int rc = check_launch("gn_scalar_stats")) return rc;
@@ -829,7 +841,7 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
     if (int rc = check_launch("gn_stats_finalize")) return rc;
   }
   hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
-                     mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu);
+                     mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu, y_halo);
   return check_launch("gn_normalize");
 }
 
@@ -886,12 +898,13 @@ extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p,
   return align_up(fwd_ws_floats(*p, pl) * sizeof(float), 256);
 }
 
-extern "C" int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
-                                 const void* gamma, const void* beta, void* y, float* mean, float* rstd, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
+static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x, const void* gamma,
+                             const void* beta, void* y, int64_t y_halo, float* mean, float* rstd, void* workspace,
+                             size_t workspace_bytes, void* stream) {
   if (int rc = check_desc(p, x_dtype)) return rc;
   if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
   if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
+  if (y_halo < 0) return fail(SFH_ERR_INVALID, "groupnorm: negative halo");
   const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(y));
   if (pl.vector) {
     const size_t need = fwd_ws_floats(*p, pl) * sizeof(float);
@@ -900,7 +913,7 @@ extern "C" int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y
   }
   hipStream_t st = (hipStream_t)stream;
   float* ws = (float*)workspace;
-#define SFH_GN_FWD(TX, TY) return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, mean, rstd, ws, st)
+#define SFH_GN_FWD(TX, TY) return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st)
   if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
@@ -911,6 +924,19 @@ extern "C" int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y
   if (x_dtype == SFH_FP32 && y_dtype == SFH_BF16) SFH_GN_FWD(float, bf16_t);
   SFH_GN_FWD(float, fp16_t);
 #undef SFH_GN_FWD
+}
+
+extern "C" int sfh_groupnorm_fwd(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
+                                 const void* gamma, const void* beta, void* y, float* mean, float* rstd, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y, 0, mean, rstd, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
+                                      const void* gamma, const void* beta, void* y_slab, int64_t halo_rows, float* mean, float* rstd,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, workspace,
+                           workspace_bytes, stream);
 }
 
 extern "C" size_t sfh_groupnorm_bwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype) {

@@ -85,8 +85,12 @@ def _desc(input, num_groups: int, eps: float, activation) -> GroupNormDesc:
     return GroupNormDesc(n, c, int(num_groups), 1 if activation == "relu" else 0, spatial, float(eps))
 
 
-def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype):
-    """The forward launch: ``(output, mean, rstd)``; shared by the registered operator and the eager autograd node."""
+def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, out_halo: int = 0):
+    """The forward launch: ``(output, mean, rstd)``; shared by the registered operator and the eager autograd node.
+
+    ``out_halo > 0`` (one sample, output of the input's element width): the output is the interior view of a slab with
+    ``out_halo`` zero depth planes on each face, which rides along as ``output._sfh_slab = (slab, out_halo)`` for a
+    consumer that wants the extended tensor (a depth shard's convolution) without copying the interior."""
     _validate(input, num_groups, weight, bias, activation)
     weight = None if weight is None else weight.contiguous()
     bias = None if bias is None else bias.contiguous()
@@ -94,7 +98,14 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype):
         bias = bias.to(weight.dtype)
     odt = out_dtype or input.dtype
     n = int(input.shape[0])
-    out = torch.empty_like(input, dtype=odt)  # keeps the channels_last_3d strides
+    slab = None
+    if out_halo > 0 and n == 1 and odt.itemsize == input.dtype.itemsize and input.numel() > 0:
+        c, d, h, w = (int(v) for v in input.shape[1:])
+        slab = torch.empty((1, c, d + 2 * out_halo, h, w), dtype=odt, device=input.device, memory_format=_CL3D)
+        out = slab[:, :, out_halo:out_halo + d]
+        out._sfh_slab = (slab, out_halo)
+    else:
+        out = torch.empty_like(input, dtype=odt)  # keeps the channels_last_3d strides
     mean = torch.empty((n, num_groups), dtype=torch.float32, device=input.device)
     rstd = torch.empty((n, num_groups), dtype=torch.float32, device=input.device)
     if input.numel() == 0:
@@ -104,10 +115,22 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype):
     xcode = _lib.dtype_code(input.dtype)
     with _lib.device_guard(input.device):
         ws = _lib.workspace(L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
-        rc = L.sfh_groupnorm_fwd(
-            ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
-            _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
-            _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+        if slab is None:
+            rc = L.sfh_groupnorm_fwd(
+                ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+                _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
+                _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+        else:
+            rc = L.sfh_groupnorm_fwd_slab(
+                ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+                _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(slab), out_halo * int(input.shape[3]) * int(input.shape[4]),
+                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+            if rc == _lib.SFH_ERR_UNSUPPORTED:  # channel counts off the vector path: the plain form
+                out = torch.empty_like(input, dtype=odt)
+                rc = L.sfh_groupnorm_fwd(
+                    ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+                    _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
+                    _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
     _lib.check(rc, "group_norm")
     return out, mean, rstd
 
@@ -228,8 +251,8 @@ class _EagerGroupNormFn(torch.autograd.Function):
     operator registry's dispatch costs more host time per call than both launches together."""
 
     @staticmethod
-    def forward(ctx, input, num_groups, weight, bias, eps, activation, out_dtype):
-        out, mean, rstd = _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype)
+    def forward(ctx, input, num_groups, weight, bias, eps, activation, out_dtype, out_halo=0):
+        out, mean, rstd = _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, out_halo)
         ctx.save_for_backward(input, weight, bias, mean, rstd)
         ctx.num_groups = num_groups
         ctx.activation = activation
@@ -241,9 +264,9 @@ class _EagerGroupNormFn(torch.autograd.Function):
         input, weight, bias, mean, rstd = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad[0], ctx.needs_input_grad[2], ctx.needs_input_grad[3]
         if not (need_x or need_w or need_b):
-            return None, None, None, None, None, None, None
+            return None, None, None, None, None, None, None, None
         d_input, d_weight, d_bias = _backward_impl(grad_out, input, weight, bias, mean, rstd, ctx.num_groups, ctx.activation)
-        return (d_input if need_x else None, None, d_weight if need_w else None, d_bias if need_b else None, None, None, None)
+        return (d_input if need_x else None, None, d_weight if need_w else None, d_bias if need_b else None, None, None, None, None)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -310,9 +333,12 @@ def is_supported(input, num_groups: int, weight=None, bias=None, activation: Opt
 
 
 def group_norm(input, num_groups: int, weight=None, bias=None, eps: float = 1e-5, activation: Optional[str] = None, *,
-               out_dtype=MATCH_STOCK_DTYPE):
+               out_dtype=MATCH_STOCK_DTYPE, out_halo: int = 0):
     """``F.group_norm(input, num_groups, weight, bias, eps)`` (then ``F.relu`` when ``activation="relu"``)
-    on a channels_last_3d CUDA tensor.  Raises ``NotImplementedError`` for calls :func:`is_supported` refuses."""
+    on a channels_last_3d CUDA tensor.  Raises ``NotImplementedError`` for calls :func:`is_supported` refuses.
+
+    ``out_halo`` (eager calls on one sample) asks for the result as the interior of a depth slab with that many zero
+    planes on each face (``result._sfh_slab``), for ``FastConv3d.shard_halo``; values and gradients are unchanged."""
     if activation not in SUPPORTED_ACTIVATIONS:
         raise ValueError(f"activation must be one of {SUPPORTED_ACTIVATIONS}, got {activation!r}")
     if not (out_dtype is MATCH_STOCK_DTYPE or out_dtype is None or out_dtype in SUPPORTED_DTYPES):
@@ -336,7 +362,8 @@ def group_norm(input, num_groups: int, weight=None, bias=None, eps: float = 1e-5
             input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype)
         )
         return out
-    return _EagerGroupNormFn.apply(input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype))
+    return _EagerGroupNormFn.apply(input, num_groups, weight, bias, float(eps), activation, _resolve_out_dtype(input, out_dtype),
+                                   int(out_halo))
 
 
 #: the reference's name for :func:`group_norm`

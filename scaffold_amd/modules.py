@@ -118,11 +118,17 @@ class _Conv3dFn(torch.autograd.Function):
     autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None):
+    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
         bc = bias if bias_compute is None else bias_compute
+        # `slab` = (tensor, halo): x is the depth interior of that tensor, whose faces already hold the halo; the
+        # kernels read the whole of it and the data gradient of its interior is x's
+        ctx.halo = 0
+        if slab is not None:
+            ctx.halo, ctx.depth = slab[1], x.shape[2]
+            x = slab[0]
         pf = pd = None
         if packs is not None:
             # packed forms that are current (kept by the module, refreshed by whoever writes the weight)
@@ -147,6 +153,8 @@ class _Conv3dFn(torch.autograd.Function):
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1,
                                           packed_weight=packed[0] if packed else None, _checked=True) if needs_x else None
+        if ctx.halo and grad_x is not None:
+            grad_x = grad_x[:, :, ctx.halo:ctx.halo + ctx.depth]
         grad_w = None
         if needs_w:
             if master:
@@ -155,7 +163,7 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
@@ -208,26 +216,36 @@ class FastConv3d(nn.Conv3d):
         w = wc if master else cast_operand(self.weight, dt)
         b = bc if master else cast_operand(self.bias, dt)
         padding = tuple(self.padding)
+        inner, slab = x, None
         if self.shard_halo and padding[0] > 0:
-            # (N, C, D, H, W): extend D by the halo the neighbours would have sent (none here: zeros)
-            x = _halo.halo_assemble(x, None, None, int(padding[0]))
+            # (N, C, D, H, W): extend D by the halo the neighbours would have sent (none here: zeros). A producer that
+            # already wrote x into the interior of such a slab (zero faces) has left it on the tensor.
+            slab = getattr(x, "_sfh_slab", None)
+            if slab is not None and slab[1] == padding[0] and slab[0].dtype is x.dtype:
+                x = slab[0]
+            else:
+                slab = None
+                x = inner = _halo.halo_assemble(x, None, None, int(padding[0]))
             padding = (0, padding[1], padding[2])
         x = x.contiguous(memory_format=_CL3D)
         # the node below skips its own gates on the strength of this one (a call that will be differentiated is
         # gated for all three directions here)
-        gate = _c3.is_supported_all if _wants_grad(x, w, b) else _c3.is_supported
+        gate = _c3.is_supported_all if _wants_grad(inner, w, b) else _c3.is_supported
         if not gate(x, w, b, self.stride, padding, self.dilation, self.groups):
             raise NotImplementedError(
                 f"FastConv3d: not served: x={tuple(x.shape)}/{x.dtype} on {x.device}, weight={tuple(w.shape)}/{w.dtype}, "
                 f"stride={self.stride} padding={padding} dilation={self.dilation} groups={self.groups}"
             )
         stride, dilation = tuple(self.stride), tuple(self.dilation)
+        if slab is None:
+            inner = x
         if master:
-            return _Conv3dFn.apply(x, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, x, stride, padding, dilation))
+            return _Conv3dFn.apply(inner, self.weight, self.bias, stride, padding, dilation, w, b,
+                                   _current_packs(self.weight, w, x, stride, padding, dilation), slab)
         if w is self.weight:
-            return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, _current_packs(w, w, x, stride, padding, dilation))
-        return _Conv3dFn.apply(x, w, b, stride, padding, dilation)
+            return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
+                                   _current_packs(w, w, x, stride, padding, dilation), slab)
+        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab)
 
 
 class FastConvTranspose3d(nn.ConvTranspose3d):
@@ -260,6 +278,8 @@ class FastGroupNorm(nn.GroupNorm):
     """``nn.GroupNorm`` (+ optional fused ReLU) served by the HIP kernels; output dtype = input dtype."""
 
     activation = None  # class-level default: not a parameter, buffer or state-dict key
+    #: depth planes of zero halo to leave around the output for a following ``FastConv3d.shard_halo`` (0: none)
+    out_halo = 0
 
     def __init__(self, num_groups, num_channels, eps=1e-5, affine=True, device=None, dtype=None, activation=None):
         super().__init__(num_groups, num_channels, eps=eps, affine=affine, device=device, dtype=dtype)
@@ -274,4 +294,5 @@ class FastGroupNorm(nn.GroupNorm):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dim() == 5 and not x.is_contiguous(memory_format=_CL3D):
             x = x.contiguous(memory_format=_CL3D)
-        return _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None)
+        return _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
+                              out_halo=self.out_halo)

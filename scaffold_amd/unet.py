@@ -20,6 +20,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 import torch.utils.checkpoint
 
+from . import concat as _cat
 from .modules import FastConv3d, FastConvTranspose3d, FastGroupNorm, autocast_dtype
 from .pooling import FastMaxPool3d
 
@@ -72,10 +73,14 @@ def _consumer_dtype(*tensors):
     return ac
 
 
-def skip_concat(skip, upsampled):
-    """``torch.cat([skip, upsampled], 1)`` at the consumer's dtype (``unet_parts.py:107-120``)."""
+def skip_concat(skip, upsampled, out_halo=0):
+    """``torch.cat([skip, upsampled], 1)`` at the consumer's dtype (``unet_parts.py:107-120``): the one-pass kernel
+    where it serves the tensors (``out_halo``: into the slab of a following depth-shard convolution), else ``torch.cat``."""
     dtype = _consumer_dtype(skip, upsampled)
-    return torch.cat([skip.to(dtype), upsampled.to(dtype)], dim=1)
+    skip, upsampled = skip.to(dtype), upsampled.to(dtype)
+    if _cat.is_supported_concat(skip, upsampled):
+        return _cat.skip_concat(skip, upsampled, out_halo)
+    return torch.cat([skip, upsampled], dim=1)
 
 
 class DoubleConv(nn.Module):
@@ -115,7 +120,9 @@ class Up(nn.Module):
         dz, dy, dx = (x2.size(i) - x1.size(i) for i in (2, 3, 4))
         if dx or dy or dz:
             x1 = F.pad(x1, [dx // 2, dx - dx // 2, dy // 2, dy - dy // 2, dz // 2, dz - dz // 2])
-        return self.conv(skip_concat(x2, x1))
+        first = self.conv.double_conv[0]
+        halo = int(first.padding[0]) if getattr(first, "shard_halo", False) else 0
+        return self.conv(skip_concat(x2, x1, halo))
 
 
 class OutConv(nn.Module):
@@ -157,6 +164,11 @@ class UNet(nn.Module):
         for m in self.modules():
             if isinstance(m, FastConv3d):
                 m.shard_halo = bool(enabled)
+            if isinstance(m, DoubleConv):
+                # the first GroupNorm writes straight into the slab the second convolution reads
+                norm, conv = m.double_conv[1], m.double_conv[3]
+                if isinstance(norm, FastGroupNorm) and isinstance(conv, FastConv3d):
+                    norm.out_halo = int(conv.padding[0]) if enabled else 0
         return self
 
     def _run(self, block, *inputs):

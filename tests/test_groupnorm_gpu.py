@@ -234,3 +234,34 @@ def test_same_call_same_bits_with_poisoned_scratch(device):
             ref = got
         else:
             assert all(torch.equal(a, b) for a, b in zip(ref, got))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape,halo", [((1, 64, 6, 7, 8), 1), ((1, 32, 3, 5, 4), 2), ((1, 48, 40, 16, 16), 1)])
+def test_output_into_a_depth_slab_is_bitwise_the_plain_output(device, dtype, shape, halo):
+    """``out_halo``: the result lands in the interior of a slab whose faces are zero; values, statistics and all
+    gradients are those of the plain call."""
+    x, gamma, beta, dy = make(shape, dtype, 5)
+    outs = []
+    for h in (0, halo):
+        xd = x.to(device).requires_grad_(True)
+        gd, bd = gamma.to(device).requires_grad_(True), beta.to(device).requires_grad_(True)
+        y = sa.group_norm(xd, 8, gd, bd, 1e-5, "relu", out_dtype=None, out_halo=h)
+        y.backward(dy.to(device))
+        outs.append((y, xd.grad, gd.grad, bd.grad))
+    (y0, *g0), (y1, *g1) = outs
+    assert not hasattr(y0, "_sfh_slab")
+    if shape[1] == 48:   # 6 sixteen-byte pieces per row do not divide the workgroup: plain form, same values
+        assert not hasattr(y1, "_sfh_slab") and torch.equal(y0, y1)
+        return
+    slab, h = y1._sfh_slab
+    assert h == halo and slab.shape == (1, shape[1], shape[2] + 2 * halo, shape[3], shape[4])
+    assert slab.is_contiguous(memory_format=CL) and y1.is_contiguous(memory_format=CL)
+    assert y1.data_ptr() == slab[:, :, halo:].data_ptr()
+    assert torch.equal(y0, y1) and all(torch.equal(a, b) for a, b in zip(g0, g1))
+    assert not slab[:, :, :halo].any() and not slab[:, :, -halo:].any()
+    # batches and outputs of another width keep the plain form
+    xb = torch.cat([x, x]).contiguous(memory_format=CL).to(device)
+    assert not hasattr(sa.group_norm(xb, 8, None, None, 1e-5, None, out_dtype=None, out_halo=halo), "_sfh_slab")
+    if dtype is torch.bfloat16:
+        assert not hasattr(sa.group_norm(x.to(device), 8, None, None, 1e-5, None, out_dtype=torch.float32, out_halo=halo), "_sfh_slab")

@@ -329,3 +329,25 @@ def test_kept_packed_weights_are_not_trusted_after_a_foreign_write(device):
     x.grad = None
     y.float().sum().backward()
     assert torch.equal(x.grad, sa.conv3d_backward_data(torch.ones_like(want), conv.weight.detach().to(torch.bfloat16), x.shape, 1, 1, 1))
+
+
+def test_conv_reading_the_producers_slab_is_bitwise_the_assembled_form(device):
+    """GroupNorm -> FastConv3d(shard_halo): with ``out_halo`` the norm writes into the slab the convolution reads; the
+    result and every gradient equal the form that assembles the slab with a copy."""
+    torch.manual_seed(11)
+    x0 = torch.randn(1, 32, 6, 12, 20, device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    gy = torch.randn(1, 64, 6, 12, 20, device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    results = []
+    for out_halo in (0, 1):
+        torch.manual_seed(12)
+        norm = FastGroupNorm(8, 32, activation="relu").to(device).to(torch.bfloat16)
+        conv = FastConv3d(32, 64, 3, padding=1, bias=False).to(device).to(torch.bfloat16).to(memory_format=CL)
+        conv.shard_halo = True
+        norm.out_halo = out_halo
+        x = x0.clone().requires_grad_(True)
+        h = norm(x)
+        assert hasattr(h, "_sfh_slab") == bool(out_halo)
+        y = conv(h)
+        y.backward(gy)
+        results.append((y.detach(), x.grad, conv.weight.grad, norm.weight.grad, norm.bias.grad))
+    assert all(torch.equal(a, b) for a, b in zip(*results))
