@@ -162,3 +162,46 @@ def test_argument_checks_of_the_rows_beside_the_convolutions():
         == _lib.SFH_ERR_INVALID  # shadow copies without a shadow dtype
     assert L.sfh_adam_clip_step(ctypes.byref(good), 3, ptrs, ptrs, ptrs, ptrs, None, numel, one, 0, one, None, None) \
         == _lib.SFH_ERR_INVALID  # no slots to fold
+
+
+def test_argument_checks_of_the_slab_concat_and_batch_packing_entry_points():
+    """Rejected before anything is launched, so this runs without a GPU."""
+    from scaffold_amd._lib import ConcatDesc, GroupNormDesc, PackItem
+
+    L = _lib.lib()
+    bf16 = 0
+    one = ctypes.c_void_p(16)  # never dereferenced: every call below fails its checks first
+
+    # skip concat: both channel counts must fill 16-byte pieces; extents positive; tensors non-null
+    assert L.sfh_skip_concat_fwd(None, bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_skip_concat_fwd(ctypes.byref(ConcatDesc(1, 32, 0, 64, 0)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_skip_concat_fwd(ctypes.byref(ConcatDesc(1, 32, 32, 64, -1)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_skip_concat_fwd(ctypes.byref(ConcatDesc(1, 32, 4, 64, 0)), bf16, one, one, one, None) == _lib.SFH_ERR_UNSUPPORTED
+    assert b"16-byte" in L.sfh_last_error()
+    assert L.sfh_skip_concat_fwd(ctypes.byref(ConcatDesc(1, 32, 32, 64, 8)), bf16, one, None, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_skip_concat_bwd(ctypes.byref(ConcatDesc(1, 32, 32, 64, 8)), bf16, None, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_skip_concat_bwd(ctypes.byref(ConcatDesc(0, 32, 32, 64, 8)), bf16, None, None, None, None) == _lib.SFH_OK  # empty batch
+
+    # GroupNorm into a slab: same checks as the plain forward, plus the halo
+    gd = GroupNormDesc(1, 64, 8, 1, 512, 1e-5)
+    assert L.sfh_groupnorm_fwd_slab(ctypes.byref(gd), bf16, bf16, bf16, one, None, None, one, -1, one, one, one, 1 << 20, None) \
+        == _lib.SFH_ERR_INVALID
+    assert L.sfh_groupnorm_fwd_slab(ctypes.byref(gd), bf16, bf16, bf16, one, None, None, None, 64, one, one, one, 1 << 20, None) \
+        == _lib.SFH_ERR_INVALID
+    assert L.sfh_groupnorm_fwd_slab(None, bf16, bf16, bf16, one, None, None, one, 64, one, one, one, 1 << 20, None) == _lib.SFH_ERR_INVALID
+
+    # batch packing: an empty batch is fine, a bad list or a problem that reads no packed weight is not
+    assert L.sfh_conv3d_pack_weights_batch(None, 0, bf16, None) == _lib.SFH_OK
+    assert L.sfh_conv3d_pack_weights_batch(None, 2, bf16, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_conv3d_pack_weights_batch(None, -1, bf16, None) == _lib.SFH_ERR_INVALID
+    items = (PackItem * 1)()
+    items[0].desc = conv_desc(cin=3)
+    items[0].w = 16
+    items[0].packed_fwd = 16
+    assert L.sfh_conv3d_pack_weights_batch(items, 1, bf16, None) == _lib.SFH_ERR_UNSUPPORTED
+    items[0].desc = conv_desc()
+    items[0].w = None
+    assert L.sfh_conv3d_pack_weights_batch(items, 1, bf16, None) == _lib.SFH_ERR_INVALID
+    items[0].w = 16
+    items[0].packed_fwd = None                      # nothing asked for: nothing launched
+    assert L.sfh_conv3d_pack_weights_batch(items, 1, bf16, None) == _lib.SFH_OK
