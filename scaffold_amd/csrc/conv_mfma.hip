@@ -133,14 +133,23 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 #pragma unroll
         for (int u = 0; u < BATCH; ++u) {
           if (it0 + u < ITERS) {
-            const int p = (it0 + u) * 256 + tid;
-            v[u] = make_uint4(0, 0, 0, 0);
-            if (p < PIECES) {
-              const int vox = p >> 2, piece = p & 3;
-              const int bw = vox % C::BW, bh = (vox / C::BW) % C::BH, bd = vox / (C::BW * C::BH);
-              const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
-              if ((unsigned)id < (unsigned)a.id && (unsigned)ih < (unsigned)a.ih && (unsigned)iw < (unsigned)a.iw)
-                v[u] = *reinterpret_cast<const uint4*>(xn + (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8);
+            // With two output blocks per workgroup registers are short: the brick position is worked out again for
+            // every chunk (the empty asm keeps the compiler from hoisting 64-bit addresses out of the chunk loop, where
+            // they were spilled and every load waited for the reload of its address), and the load is unconditional
+            // from a clamped address, masked afterwards.
+            int p = (it0 + u) * 256 + tid;
+            if constexpr (C::NSUB > 1) asm volatile("" : "+v"(p));
+            const int vox = p >> 2, piece = p & 3;
+            const int bw = vox % C::BW, bh = (vox / C::BW) % C::BH, bd = vox / (C::BW * C::BH);
+            const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
+            const bool in = p < PIECES && (unsigned)id < (unsigned)a.id && (unsigned)ih < (unsigned)a.ih && (unsigned)iw < (unsigned)a.iw;
+            if constexpr (C::NSUB > 1) {
+              const int64_t at = in ? (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8 : 0;
+              const uint4 got = *reinterpret_cast<const uint4*>(xn + at);
+              v[u] = in ? got : make_uint4(0, 0, 0, 0);
+            } else {  // registers to spare: the compiler keeps the addresses across chunks and batches every load
+              v[u] = make_uint4(0, 0, 0, 0);
+              if (in) v[u] = *reinterpret_cast<const uint4*>(xn + (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8);
             }
           }
         }
@@ -161,7 +170,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
     const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
     constexpr int NIT = C::TAPS * 2;
-    constexpr int WDEPTH = NIT < 6 ? NIT : 6;
+    constexpr int WDEPTH = NIT < 6 ? NIT : (C::NSUB > 1 ? 4 : 6);
     uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
     uint4 aq[2][C::MS];
 #pragma unroll
@@ -308,7 +317,8 @@ struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
 
 // Launch geometry, a pure function of the problem: brick shape by row length; two output blocks per workgroup
 // when that still fills the chip, else one; and when even that leaves CUs idle (the deep, small-volume levels)
-// the reduction channels are cut into slices that are summed afterwards.
+// the reduction channels are cut into slices that are summed afterwards (one workgroup per CU: more slices cost more
+// in fp32 partials than the second resident workgroup gains).
 GatherPlan gather_plan(const MfmaConvArgs& a) {
   GatherPlan p{};
   int td, th, tw;
@@ -321,7 +331,7 @@ GatherPlan gather_plan(const MfmaConvArgs& a) {
   const int64_t wgs = p.tiles * (a.cout / (32 * p.nsub));
   const int ncc = a.cred / kChunk;
   if (wgs < kComputeUnits && ncc > 1) {
-    int64_t k = cdiv(2 * kComputeUnits, wgs);
+    int64_t k = cdiv(kComputeUnits, wgs);
     p.ksplit = (int)(k < ncc ? k : ncc);
   }
   return p;
