@@ -92,6 +92,49 @@ def _desc(n, cin, in_sp, cout, k, s, p, d) -> ConvDesc:
                     p[0], p[1], p[2], d[0], d[1], d[2])
 
 
+class _Problem:
+    """Everything about one convolution problem that does not depend on the tensors: parsed geometry, the descriptor
+    the library takes, and (filled on first use) the workspace bytes of each direction."""
+
+    __slots__ = ("s", "p", "d", "k", "n", "cin", "in_sp", "cout", "y_shape", "desc", "code", "need")
+
+    def __init__(self, in_shape, w_shape, stride, padding, dilation, dtype):
+        self.s, self.p, self.d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+        self.n, self.cin, *in_sp = (int(v) for v in in_shape)
+        self.in_sp = tuple(in_sp)
+        self.cout = int(w_shape[0])
+        self.k = tuple(int(v) for v in w_shape[2:])
+        self.y_shape = output_shape(in_shape, w_shape, self.s, self.p, self.d)
+        self.desc = _desc(self.n, self.cin, self.in_sp, self.cout, self.k, self.s, self.p, self.d)
+        self.code = _lib.dtype_code(dtype)
+        self.need = {}
+
+    def workspace_bytes(self, direction: str) -> int:
+        need = self.need.get(direction)
+        if need is None:
+            fn = getattr(_lib.lib(), f"sfh_conv3d_{direction}_workspace_bytes")
+            need = self.need[direction] = int(fn(ctypes.byref(self.desc), self.code))
+        return need
+
+
+_PROBLEMS: dict = {}
+
+
+def _problem(in_shape, w_shape, stride, padding, dilation, dtype) -> _Problem:
+    """The cached :class:`_Problem` of a call (one dictionary lookup per call once a shape has been seen)."""
+    key = (in_shape, w_shape, stride, padding, dilation, dtype)
+    try:
+        prob = _PROBLEMS.get(key)
+    except TypeError:  # unhashable spelling of a shape, stride, padding or dilation
+        return _Problem(in_shape, w_shape, stride, padding, dilation, dtype)
+    if prob is None:
+        prob = _Problem(in_shape, w_shape, stride, padding, dilation, dtype)
+        if len(_PROBLEMS) > 4096:
+            _PROBLEMS.clear()
+        _PROBLEMS[key] = prob
+    return prob
+
+
 # ---------------------------------------------------------------------------------------------
 # gates
 # ---------------------------------------------------------------------------------------------
@@ -488,31 +531,26 @@ def conv3d_forward(
             f"w={tuple(getattr(w, 'shape', ()))} stride={stride} padding={padding} dilation={dilation} groups={groups}"
         )
     _no_config(config)
-    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
-    k = tuple(int(v) for v in w.shape[2:])
     x = x.contiguous(memory_format=_CL3D)
-    n, cin, *in_sp = (int(v) for v in x.shape)
-    cout = int(w.shape[0])
-    y_shape = output_shape(x.shape, w.shape, s, p, d)
+    prob = _problem(x.shape, w.shape, stride, padding, dilation, x.dtype)
     if out is None:
-        y = torch.empty(y_shape, device=x.device, dtype=x.dtype, memory_format=_CL3D)
+        y = torch.empty(prob.y_shape, device=x.device, dtype=x.dtype, memory_format=_CL3D)
     else:
         y = out
-        _check_out(y, y_shape, x)
+        _check_out(y, prob.y_shape, x)
     if weight_rsck is not None:
-        _check_weight_rsck(weight_rsck, (*k, cin, cout), x)
+        _check_weight_rsck(weight_rsck, (*prob.k, prob.cin, prob.cout), x)
         w_eff = weight_rsck.permute(4, 3, 0, 1, 2)  # (Cout, Cin, kd, kh, kw) view of the RSCK buffer
     else:
         w_eff = w
     if weight_flip:
         w_eff = w_eff.flip(2, 3, 4)  # small copy; the data-gradient entry point flips inside the library instead
-    if n == 0:
+    if prob.n == 0:
         return y
     L = _lib.lib()
-    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
-    code = _lib.dtype_code(x.dtype)
+    desc, code = prob.desc, prob.code
     with _lib.device_guard(x.device):
-        need = int(L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(desc), code))
+        need = prob.workspace_bytes("fwd")
         flags = _flags(force_generic)
         if packed_weight is not None:
             # ``packed_weight`` comes from pack_weights() for this very problem: the library reads it in place of w
@@ -561,27 +599,24 @@ def conv3d_backward_data(
             f"padding={padding} dilation={dilation} groups={groups}"
         )
     _no_config(config)
-    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
-    k = tuple(int(v) for v in weight.shape[2:])
-    n, cin, *in_sp = (int(v) for v in input_shape)
-    cout = int(weight.shape[0])
     gy = grad_output.contiguous(memory_format=_CL3D)
-    gx_shape = (n, cin, *in_sp)
+    prob = _problem(input_shape if isinstance(input_shape, torch.Size) else tuple(input_shape), weight.shape, stride, padding,
+                    dilation, gy.dtype)
+    gx_shape = (prob.n, prob.cin, *prob.in_sp)
     if out is None:
         gx = torch.empty(gx_shape, device=gy.device, dtype=gy.dtype, memory_format=_CL3D)
     else:
         gx = out
         _check_out(gx, gx_shape, gy)
     if weight_rsck is not None:
-        _check_weight_rsck(weight_rsck, (*k, cin, cout), gy)
+        _check_weight_rsck(weight_rsck, (*prob.k, prob.cin, prob.cout), gy)
         w_eff = weight_rsck.permute(4, 3, 0, 1, 2)
     else:
         w_eff = weight
     L = _lib.lib()
-    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
-    code = _lib.dtype_code(gy.dtype)
+    desc, code = prob.desc, prob.code
     with _lib.device_guard(gy.device):
-        need = int(L.sfh_conv3d_dgrad_workspace_bytes(ctypes.byref(desc), code))
+        need = prob.workspace_bytes("dgrad")
         flags = _flags(force_generic)
         if packed_weight is not None:
             if weight_rsck is not None or force_generic:
@@ -651,28 +686,27 @@ def conv3d_backward_weight(
     _no_config(config)
     if not deterministic:
         raise NotImplementedError("deterministic=False: this library has no atomic weight-gradient path")
-    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
-    cout, cin, *k = (int(v) for v in weight_shape)
     x = input.contiguous(memory_format=_CL3D)
     gy = grad_output.contiguous(memory_format=_CL3D)
-    n, _, *in_sp = (int(v) for v in x.shape)
+    prob = _problem(x.shape, weight_shape if isinstance(weight_shape, torch.Size) else tuple(weight_shape), stride, padding,
+                    dilation, x.dtype)
+    cout, cin, k, n = prob.cout, prob.cin, prob.k, prob.n
     gdt = x.dtype if grad_dtype is None else grad_dtype
     if gdt is not x.dtype and gdt is not torch.float32:
         raise ValueError(f"grad_dtype must be the operands' dtype or torch.float32, got {grad_dtype}")
     if out is None:
-        gw = grad_weight_empty(cout, cin, k, dtype=gdt, device=x.device)
+        gw = torch.empty((cout, cin, *k), dtype=gdt, device=x.device, memory_format=_CL3D)
     else:
         gw = out
         why = _validate_gw_out(gw, cout, cin, tuple(k), gdt, x.device)
         if why is not None:
             raise ValueError(f"out= is not usable for this problem: {why}")
     L = _lib.lib()
-    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
-    code = _lib.dtype_code(x.dtype)
+    desc, code = prob.desc, prob.code
     if n == 0:
         return gw.zero_()
     with _lib.device_guard(x.device):
-        need = 0 if force_generic else int(L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(desc), code))
+        need = 0 if force_generic else prob.workspace_bytes("wgrad")
         if workspace is None:
             ws = _lib.workspace(need, x.device)
             ws_bytes = 0 if ws is None else ws.numel()

@@ -85,6 +85,24 @@ def _desc(input, num_groups: int, eps: float, activation) -> GroupNormDesc:
     return GroupNormDesc(n, c, int(num_groups), 1 if activation == "relu" else 0, spatial, float(eps))
 
 
+_PLANS: dict = {}
+
+
+def _plan(input, num_groups: int, eps: float, activation, backward: bool):
+    """``(descriptor, dtype code, workspace bytes)`` of a call, cached by shape: one dictionary lookup per call."""
+    key = (input.shape, input.dtype, num_groups, eps, activation, backward)
+    plan = _PLANS.get(key)
+    if plan is None:
+        desc = _desc(input, num_groups, eps, activation)
+        code = _lib.dtype_code(input.dtype)
+        L = _lib.lib()
+        need = (L.sfh_groupnorm_bwd_workspace_bytes if backward else L.sfh_groupnorm_fwd_workspace_bytes)(ctypes.byref(desc), code)
+        if len(_PLANS) > 4096:
+            _PLANS.clear()
+        plan = _PLANS[key] = (desc, code, int(need))
+    return plan
+
+
 def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, out_halo: int = 0):
     """The forward launch: ``(output, mean, rstd)``; shared by the registered operator and the eager autograd node.
 
@@ -111,10 +129,9 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, o
     if input.numel() == 0:
         return out, mean, rstd
     L = _lib.lib()
-    desc = _desc(input, num_groups, eps, activation)
-    xcode = _lib.dtype_code(input.dtype)
+    desc, xcode, need = _plan(input, num_groups, eps, activation, False)
     with _lib.device_guard(input.device):
-        ws = _lib.workspace(L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
+        ws = _lib.workspace(need, input.device)
         if slab is None:
             rc = L.sfh_groupnorm_fwd(
                 ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
@@ -175,10 +192,9 @@ def _backward_impl(grad_out, input, weight, bias, mean, rstd, num_groups, activa
     db32 = torch.empty(channels, dtype=torch.float32, device=input.device) if bias is not None else None
     if input.numel() > 0:
         L = _lib.lib()
-        desc = _desc(input, num_groups, 0.0, activation)
-        xcode = _lib.dtype_code(input.dtype)
+        desc, xcode, need = _plan(input, num_groups, 0.0, activation, True)
         with _lib.device_guard(input.device):
-            ws = _lib.workspace(L.sfh_groupnorm_bwd_workspace_bytes(ctypes.byref(desc), xcode), input.device)
+            ws = _lib.workspace(need, input.device)
             rc = L.sfh_groupnorm_bwd(
                 ctypes.byref(desc), xcode, _lib.dtype_code(grad_out.dtype),
                 _lib.dtype_code(_param_dtype(weight, bias, input)), _lib.ptr(grad_out), _lib.ptr(input), _lib.ptr(weight),
