@@ -23,14 +23,40 @@ __device__ __forceinline__ float wave_sum_all(float v) {
   return v;  // lane 0 holds the sum
 }
 
+// A tile's logits are one contiguous byte range whatever the class count (11 classes: 22-byte rows): it moves between
+// global memory and LDS in 16-byte pieces when the range starts on a 16-byte boundary (`vec`), element by element else.
+template <typename T>
+__device__ __forceinline__ void tile_in(T* tile, const T* __restrict__ src, int nelem, bool vec) {
+  const int tid = threadIdx.x;
+  if (vec) {
+    constexpr int E = 16 / (int)sizeof(T);
+    const int npiece = nelem / E;
+    for (int i = tid; i < npiece; i += kBlock) reinterpret_cast<uint4*>(tile)[i] = reinterpret_cast<const uint4*>(src)[i];
+    for (int i = npiece * E + tid; i < nelem; i += kBlock) tile[i] = src[i];
+  } else {
+    for (int i = tid; i < nelem; i += kBlock) tile[i] = src[i];
+  }
+}
+template <typename T>
+__device__ __forceinline__ void tile_out(T* __restrict__ dst, const T* tile, int nelem, bool vec) {
+  const int tid = threadIdx.x;
+  if (vec) {
+    constexpr int E = 16 / (int)sizeof(T);
+    const int npiece = nelem / E;
+    for (int i = tid; i < npiece; i += kBlock) reinterpret_cast<uint4*>(dst)[i] = reinterpret_cast<const uint4*>(tile)[i];
+    for (int i = npiece * E + tid; i < nelem; i += kBlock) dst[i] = tile[i];
+  } else {
+    for (int i = tid; i < nelem; i += kBlock) dst[i] = tile[i];
+  }
+}
+
 // Quantities per sample: inter[c], psum[c], tsum[c] (3 * C), then the two launch-wide ones: ce_sum, normaliser.
 template <typename T, int CMAX>
 __global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ logits, const int64_t* __restrict__ labels,
                                                           const float* __restrict__ cw, float* __restrict__ part, int64_t S, int C,
-                                                          int nsplit, int64_t per_split) {
-  extern __shared__ char smem_raw[];
+                                                          int nsplit, int64_t per_split, int vec) {
+  extern __shared__ __align__(16) char smem_raw[];
   T* tile = reinterpret_cast<T*>(smem_raw);  // kBlock voxels x C logits
-  __shared__ float red[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = blockIdx.y, split = blockIdx.x;
   const T* src = logits + (int64_t)n * S * C;
@@ -44,7 +70,7 @@ __global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ 
   for (int64_t v0 = begin; v0 < end; v0 += kBlock) {
     const int nv = (int)((end - v0) < kBlock ? (end - v0) : kBlock);
     __syncthreads();
-    for (int i = tid; i < nv * C; i += kBlock) tile[i] = src[v0 * C + i];
+    tile_in<T>(tile, src + v0 * C, nv * C, vec != 0);
     __syncthreads();
     if (tid < nv) {
       float x[CMAX];
@@ -79,25 +105,32 @@ __global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ 
       }
     }
   }
-  // workgroup totals: wavefront trees, then the four wave totals in order
+  // workgroup totals: every quantity through the wavefront tree, the wave totals parked in LDS, then one thread per
+  // quantity adds the four wave totals in order (one barrier for all 3 C + 2 quantities)
   float* dst = part + ((int64_t)n * nsplit + split) * (3 * C + 2);
-  auto fold = [&](float v, int slot) {
+  __syncthreads();  // the tile is consumed: its LDS holds the wave totals now
+  float* wave_tot = reinterpret_cast<float*>(smem_raw);  // [4][3 * CMAX + 2]
+  constexpr int Q = 3 * CMAX + 2;
+  auto park = [&](float v, int slot) {
     v = wave_sum_all(v);
-    __syncthreads();
-    if (lane == 0) red[wave] = v;
-    __syncthreads();
-    if (tid == 0) dst[slot] = (red[0] + red[1]) + (red[2] + red[3]);
+    if (lane == 0) wave_tot[wave * Q + slot] = v;
   };
 #pragma unroll
   for (int c = 0; c < CMAX; ++c) {
-    if (c < C) {
-      fold(inter[c], c);
-      fold(psum[c], C + c);
-      fold(tsum[c], 2 * C + c);
+    park(inter[c], c);
+    park(psum[c], CMAX + c);
+    park(tsum[c], 2 * CMAX + c);
+  }
+  park(ce, 3 * CMAX);
+  park(norm, 3 * CMAX + 1);
+  __syncthreads();
+  if (tid < Q) {
+    const int q = tid < 3 * CMAX ? tid / CMAX : 3, c = tid < 3 * CMAX ? tid % CMAX : tid - 3 * CMAX;
+    if (q == 3 || c < C) {
+      const float t = (wave_tot[tid] + wave_tot[Q + tid]) + (wave_tot[2 * Q + tid] + wave_tot[3 * Q + tid]);
+      dst[q == 3 ? 3 * C + c : q * C + c] = t;
     }
   }
-  fold(ce, 3 * C);
-  fold(norm, 3 * C + 1);
 }
 
 // One 64-lane workgroup per quantity: lane l adds slots l, l + 64, ... and the lane totals meet in a fixed tree.
@@ -154,8 +187,8 @@ template <typename T, int CMAX>
 __global__ void __launch_bounds__(kBlock) ce_dice_backward(const T* __restrict__ logits, const int64_t* __restrict__ labels,
                                                            const float* __restrict__ cw, const float* __restrict__ stats,
                                                            const float* __restrict__ grad_loss, T* __restrict__ dlogits, int64_t S,
-                                                           int N, int C, float eps, int64_t per_split) {
-  extern __shared__ char smem_raw[];
+                                                           int N, int C, float eps, int64_t per_split, int vec) {
+  extern __shared__ __align__(16) char smem_raw[];
   T* tile = reinterpret_cast<T*>(smem_raw);
   __shared__ float ca[CMAX], cb[CMAX];
   const int tid = threadIdx.x;
@@ -184,7 +217,7 @@ __global__ void __launch_bounds__(kBlock) ce_dice_backward(const T* __restrict__
   for (int64_t v0 = begin; v0 < end; v0 += kBlock) {
     const int nv = (int)((end - v0) < kBlock ? (end - v0) : kBlock);
     __syncthreads();
-    for (int i = tid; i < nv * C; i += kBlock) tile[i] = src[v0 * C + i];
+    tile_in<T>(tile, src + v0 * C, nv * C, vec != 0);
     __syncthreads();
     if (tid < nv) {
       float p[CMAX];
@@ -223,7 +256,7 @@ __global__ void __launch_bounds__(kBlock) ce_dice_backward(const T* __restrict__
       }
     }
     __syncthreads();
-    for (int i = tid; i < nv * C; i += kBlock) dst[v0 * C + i] = tile[i];
+    tile_out<T>(dst + v0 * C, tile, nv * C, vec != 0);
   }
 }
 
@@ -240,13 +273,23 @@ LossPlan loss_plan(const sfh_loss_desc& p) {
   return pl;
 }
 
+// Every tile starts kBlock * classes elements after the previous one and every sample spatial * classes elements after
+// the previous one: all tiles start on 16-byte boundaries when those two strides and the base pointers do.
+template <typename T>
+int tiles_on_16_bytes(const sfh_loss_desc& p, const void* a, const void* b) {
+  const bool ok = (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(b) & 15) == 0 &&
+                  ((size_t)kBlock * p.classes * sizeof(T)) % 16 == 0 && (p.n == 1 || ((size_t)p.spatial * p.classes * sizeof(T)) % 16 == 0);
+  return ok ? 1 : 0;
+}
+
 template <typename T, int CMAX>
 int fwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels, const float* cw, float* loss, float* stats,
               float* ws, hipStream_t st) {
   const LossPlan pl = loss_plan(p);
-  const size_t lds = (size_t)kBlock * p.classes * sizeof(T);
+  size_t lds = (size_t)kBlock * p.classes * sizeof(T);
+  if (lds < 4 * (3 * CMAX + 2) * sizeof(float)) lds = 4 * (3 * CMAX + 2) * sizeof(float);  // the fold at the end reuses the tile
   hipLaunchKernelGGL((ce_dice_partial<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, ws,
-                     p.spatial, p.classes, pl.nsplit, pl.per_split);
+                     p.spatial, p.classes, pl.nsplit, pl.per_split, tiles_on_16_bytes<T>(p, logits, nullptr));
   if (int rc = check_launch("ce_dice_partial")) return rc;
   hipLaunchKernelGGL(ce_dice_sum, dim3(p.n * 3 * p.classes + 2), dim3(64), 0, st, ws, stats, p.n, p.classes, pl.nsplit,
                      cw == nullptr ? 1 : 0, (float)p.n * (float)p.spatial);
@@ -261,7 +304,7 @@ int bwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels,
   const LossPlan pl = loss_plan(p);
   const size_t lds = (size_t)kBlock * p.classes * sizeof(T);
   hipLaunchKernelGGL((ce_dice_backward<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, stats,
-                     grad_loss, (T*)dlogits, p.spatial, p.n, p.classes, p.eps, pl.per_split);
+                     grad_loss, (T*)dlogits, p.spatial, p.n, p.classes, p.eps, pl.per_split, tiles_on_16_bytes<T>(p, logits, dlogits));
   return check_launch("ce_dice_backward");
 }
 
@@ -276,6 +319,11 @@ size_t loss_workspace_bytes(const sfh_loss_desc& p) {
 }
 
 #define SFH_LOSS_DISPATCH(fn, ...)                                               \
+  if (p.classes <= 12) {                                                         \
+    if (dtype == SFH_BF16) return fn<bf16_t, 12>(__VA_ARGS__);                   \
+    if (dtype == SFH_FP16) return fn<fp16_t, 12>(__VA_ARGS__);                   \
+    return fn<float, 12>(__VA_ARGS__);                                           \
+  }                                                                              \
   if (p.classes <= 16) {                                                         \
     if (dtype == SFH_BF16) return fn<bf16_t, 16>(__VA_ARGS__);                   \
     if (dtype == SFH_FP16) return fn<fp16_t, 16>(__VA_ARGS__);                   \

@@ -23,7 +23,8 @@ def reference(logits, labels, cw, grad=True):
 
 @pytest.mark.parametrize("weighted", [False, True])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(1, 11, 6, 9, 13), (2, 11, 4, 5, 70), (1, 2, 3, 3, 3), (3, 17, 2, 8, 9), (1, 32, 5, 5, 5)])
+@pytest.mark.parametrize("shape", [(1, 11, 6, 9, 13), (2, 11, 4, 5, 70), (1, 2, 3, 3, 3), (3, 17, 2, 8, 9), (1, 32, 5, 5, 5),
+                                   (2, 11, 3, 3, 3)])  # the last: samples that do not start on 16-byte boundaries
 def test_loss_and_gradient_match_oracle(device, dtype, shape, weighted):
     g = torch.Generator().manual_seed(31)
     n, c = shape[:2]
