@@ -429,12 +429,15 @@ int launch_tile(const WgradArgs& a, const Plan& p, const void* x, const void* gy
 template <typename T>
 int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace, hipStream_t st) {
   const Plan p = make_plan(a);
-  float* ws = (float*)workspace;
+  // One slice and an fp32 gradient (the deepest levels under fp32 master weights): the kernel's slice IS the
+  // gradient, so it is written in place and no sum pass follows.
+  const bool direct = p.splits == 1 && gw_dtype == SFH_FP32;
+  float* ws = direct ? (float*)gw : (float*)workspace;
   int rc;
   if (p.tw == 32) rc = launch_tile<T, WTile<2, 4, 32>>(a, p, x, gy, ws, st);
   else if (p.tw == 16) rc = launch_tile<T, WTile<2, 8, 16>>(a, p, x, gy, ws, st);
   else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st);
-  if (rc != SFH_OK) return rc;
+  if (rc != SFH_OK || direct) return rc;
   const int64_t nelem = (int64_t)a.cout * 27 * a.cin;
   return sum_slices(gw_dtype, ws, gw, nelem, p.splits, st);
 }

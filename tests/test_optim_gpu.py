@@ -217,6 +217,7 @@ def test_step_captured_in_a_graph_replays_to_the_eager_result(device):
     # cin, cout, spatial, kernel, stride, padding     (tiled MFMA, 2x2x2 stride-2, thin head, thin stem)
     (32, 32, (8, 16, 32), 3, 1, 1),
     (64, 128, (4, 8, 8), 3, 1, 1),
+    (256, 512, (4, 8, 8), 3, 1, 1),   # one voxel slice: the fp32 gradient is written in place, no sum pass
     (32, 64, (8, 8, 16), 2, 2, 0),
     (32, 11, (8, 8, 16), 1, 1, 0),
     (1, 32, (8, 16, 32), 3, 1, 1),
