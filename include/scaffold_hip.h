@@ -230,6 +230,11 @@ int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, 
                      void* stream);
 int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
                      void* grad_x, void* stream);
+/* grad_x = (the pooling gradient) + add, summed in fp32 and rounded once; `add` has the input's
+ * shape. In the U-Net the pooled tensor is also the skip connection (unet_model.py:141-155): its
+ * two gradients meet here instead of in a separate addition. */
+int sfh_maxpool2_bwd_add(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
+                         const void* add, void* grad_x, void* stream);
 
 /* ---- halo slab assembly ------------------------------------------------------------------
  * The local step of a depth shard's forward halo exchange: out = [lo | x | hi] along depth, where

@@ -545,7 +545,17 @@ extern "C" int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* g
   const bool empty_out = p->in_d < 2 || p->in_h < 2 || p->in_w < 2;
   if (grad_x == nullptr || (!empty_out && (grad_y == nullptr || idx == nullptr)))
     return fail(SFH_ERR_INVALID, "maxpool bwd: null tensor");
-  return maxpool2_bwd(*p, dtype, grad_y, idx, grad_x, (hipStream_t)stream);
+  return maxpool2_bwd(*p, dtype, grad_y, idx, nullptr, grad_x, (hipStream_t)stream);
+}
+
+extern "C" int sfh_maxpool2_bwd_add(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx, const void* add,
+                                    void* grad_x, void* stream) {
+  if (int rc = check_pool(p, dtype, "maxpool bwd")) return rc;
+  if (p->n == 0) return SFH_OK;
+  const bool empty_out = p->in_d < 2 || p->in_h < 2 || p->in_w < 2;
+  if (grad_x == nullptr || add == nullptr || (!empty_out && (grad_y == nullptr || idx == nullptr)))
+    return fail(SFH_ERR_INVALID, "maxpool bwd: null tensor");
+  return maxpool2_bwd(*p, dtype, grad_y, idx, add, grad_x, (hipStream_t)stream);
 }
 
 // ---- transposed convolution ------------------------------------------------------------

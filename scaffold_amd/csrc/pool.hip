@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(kBlock) maxpool2_fwd_kernel(PoolGeom g, int64_
 template <typename T, int V>
 __global__ void __launch_bounds__(kBlock) maxpool2_bwd_kernel(PoolGeom g, int cd, int ch, int cw, int64_t total,
                                                               const T* __restrict__ gy, const uint8_t* __restrict__ idx,
-                                                              T* __restrict__ gx) {
+                                                              const T* __restrict__ add, T* __restrict__ gx) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= total) return;
   const int64_t cv = i % g.cvec;
@@ -111,15 +111,23 @@ __global__ void __launch_bounds__(kBlock) maxpool2_bwd_kernel(PoolGeom g, int cd
       which[0] = idx[o];
     }
   }
-  T* dst = gx + ((((n * g.d + 2 * od) * g.h + 2 * oh) * g.w + 2 * ow) * (int64_t)g.c + cv * V);
+  const int64_t cell = (((n * g.d + 2 * od) * g.h + 2 * oh) * g.w + 2 * ow) * (int64_t)g.c + cv * V;
+  T* dst = gx + cell;
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     const int kd = k >> 2, kh = (k >> 1) & 1, kw = k & 1;
     if ((2 * od + kd < g.d) & (2 * oh + kh < g.h) & (2 * ow + kw < g.w)) {
+      const int64_t at = (((int64_t)kd * g.h + kh) * g.w + kw) * g.c;
       float out[V];
 #pragma unroll
       for (int e = 0; e < V; ++e) out[e] = which[e] == k ? grad[e] : 0.f;
-      StN<T, V>::run(dst + (((int64_t)kd * g.h + kh) * g.w + kw) * g.c, out);
+      if (add != nullptr) {  // a second gradient of the pooled tensor (its use as a skip connection), summed in fp32
+        float more[V];
+        LdN<T, V>::run(add + cell + at, more);
+#pragma unroll
+        for (int e = 0; e < V; ++e) out[e] += more[e];
+      }
+      StN<T, V>::run(dst + at, out);
     }
   }
 }
@@ -153,9 +161,9 @@ int fwd_typed(const sfh_pool_desc& p, const void* x, void* y, uint8_t* idx, hipS
 }
 
 template <typename T>
-int bwd_typed(const sfh_pool_desc& p, const void* gy, const uint8_t* idx, void* gx, hipStream_t st) {
+int bwd_typed(const sfh_pool_desc& p, const void* gy, const uint8_t* idx, const void* add, void* gx, hipStream_t st) {
   constexpr int V = VecOf<T>::N;
-  const bool vec = p.c % V == 0 && aligned16(gy) && aligned16(gx) && (reinterpret_cast<uintptr_t>(idx) & 7) == 0;
+  const bool vec = p.c % V == 0 && aligned16(gy) && aligned16(gx) && aligned16(add) && (reinterpret_cast<uintptr_t>(idx) & 7) == 0;
   const PoolGeom g = geom(p, vec ? V : 1);
   const int cd = (p.in_d + 1) / 2, ch = (p.in_h + 1) / 2, cw = (p.in_w + 1) / 2;
   const int64_t total = (int64_t)p.n * cd * ch * cw * g.cvec;
@@ -164,10 +172,10 @@ int bwd_typed(const sfh_pool_desc& p, const void* gy, const uint8_t* idx, void* 
   if (blocks > 0x7fffffff) return fail(SFH_ERR_UNSUPPORTED, "maxpool bwd: %lld workgroups exceed the grid limit", (long long)blocks);
   if (vec)
     hipLaunchKernelGGL((maxpool2_bwd_kernel<T, V>), dim3((unsigned)blocks), dim3(kBlock), 0, st, g, cd, ch, cw, total,
-                       static_cast<const T*>(gy), idx, static_cast<T*>(gx));
+                       static_cast<const T*>(gy), idx, static_cast<const T*>(add), static_cast<T*>(gx));
   else
     hipLaunchKernelGGL((maxpool2_bwd_kernel<T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, st, g, cd, ch, cw, total,
-                       static_cast<const T*>(gy), idx, static_cast<T*>(gx));
+                       static_cast<const T*>(gy), idx, static_cast<const T*>(add), static_cast<T*>(gx));
   return check_launch("maxpool2_bwd_kernel");
 }
 
@@ -179,10 +187,10 @@ int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint
   return fwd_typed<float>(p, x, y, idx, st);
 }
 
-int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, void* gx, hipStream_t st) {
-  if (dtype == SFH_BF16) return bwd_typed<bf16_t>(p, gy, idx, gx, st);
-  if (dtype == SFH_FP16) return bwd_typed<fp16_t>(p, gy, idx, gx, st);
-  return bwd_typed<float>(p, gy, idx, gx, st);
+int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, const void* add, void* gx, hipStream_t st) {
+  if (dtype == SFH_BF16) return bwd_typed<bf16_t>(p, gy, idx, add, gx, st);
+  if (dtype == SFH_FP16) return bwd_typed<fp16_t>(p, gy, idx, add, gx, st);
+  return bwd_typed<float>(p, gy, idx, add, gx, st);
 }
 
 }  // namespace sfh

@@ -9,6 +9,7 @@ namespace sfh {
 int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st);
 
 // gx = gy routed to the voxel idx names, zero elsewhere (including dropped odd planes). Writes all of gx.
-int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, void* gx, hipStream_t st);
+// gx = the pooling gradient (+ `add`, a tensor of the input's shape, when given)
+int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, const void* add, void* gx, hipStream_t st);
 
 }  // namespace sfh

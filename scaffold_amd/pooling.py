@@ -17,7 +17,7 @@ from torch.autograd.function import once_differentiable
 from . import _lib
 from ._lib import PoolDesc
 
-__all__ = ["max_pool3d_2x", "is_supported_pool", "FastMaxPool3d"]
+__all__ = ["max_pool3d_2x_with_skip", "max_pool3d_2x", "is_supported_pool", "FastMaxPool3d"]
 
 _CL3D = torch.channels_last_3d
 
@@ -62,6 +62,48 @@ class _MaxPool2Fn(torch.autograd.Function):
         return gx
 
 
+class _MaxPool2SkipFn(torch.autograd.Function):
+    """Pooling of a tensor that is also carried on as a skip connection: returns ``(pooled, x)``; the two gradients
+    of ``x`` (through the pooling and through the skip) are summed inside the pooling-gradient kernel instead of by a
+    separate addition over the full-size tensor."""
+
+    @staticmethod
+    def forward(ctx, x):
+        y = _MaxPool2Fn.forward(ctx, x)
+        return y, x  # autograd hands out an alias of x with this node as its history
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_y, grad_skip):
+        if grad_skip is None:
+            return _MaxPool2Fn.backward(ctx, grad_y)
+        if grad_y is None:
+            return grad_skip
+        (idx,) = ctx.saved_tensors
+        n, c, d, h, w = ctx.pool_shape
+        gy = grad_y.contiguous(memory_format=_CL3D)
+        gs = grad_skip.contiguous(memory_format=_CL3D)
+        if gs.dtype is not gy.dtype:
+            gs = gs.to(gy.dtype)
+        gx = torch.empty((n, c, d, h, w), dtype=gy.dtype, device=gy.device, memory_format=_CL3D)
+        desc = PoolDesc(n, c, d, h, w)
+        with _lib.device_guard(gy.device):
+            rc = _lib.lib().sfh_maxpool2_bwd_add(ctypes.byref(desc), _lib.dtype_code(gy.dtype), _lib.ptr(gy), _lib.ptr(idx),
+                                                 _lib.ptr(gs), _lib.ptr(gx), _lib.stream_ptr(gy.device))
+        _lib.check(rc, "max_pool3d_2x backward")
+        return gx
+
+
+def max_pool3d_2x_with_skip(x: torch.Tensor):
+    """``(F.max_pool3d(x, 2), x)``: use the returned ``x`` for the skip connection and the gradients of both uses are
+    combined in one kernel (same values as autograd's own addition: one fp32 sum, one rounding)."""
+    if not is_supported_pool(x):
+        raise NotImplementedError(f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)}")
+    if not x.is_contiguous(memory_format=_CL3D):
+        return _MaxPool2Fn.apply(x), x
+    return _MaxPool2SkipFn.apply(x)
+
+
 def max_pool3d_2x(x: torch.Tensor) -> torch.Tensor:
     """``F.max_pool3d(x, 2)`` for a 5-D GPU tensor; the result is channels-last."""
     if not is_supported_pool(x):
@@ -80,10 +122,24 @@ class FastMaxPool3d(nn.MaxPool3d):
     ``kernel_size == stride == 2``, no padding, no dilation, floor mode, no returned indices; anything else
     raises ``NotImplementedError`` at call time."""
 
-    def forward(self, input):
+    def _is_pool2(self) -> bool:
         stride = self.kernel_size if self.stride is None else self.stride
-        if not (_all_equal(self.kernel_size, 2) and _all_equal(stride, 2) and _all_equal(self.padding, 0)
-                and _all_equal(self.dilation, 1) and not self.ceil_mode and not self.return_indices):
+        return (_all_equal(self.kernel_size, 2) and _all_equal(stride, 2) and _all_equal(self.padding, 0)
+                and _all_equal(self.dilation, 1) and not self.ceil_mode and not self.return_indices)
+
+    def serves(self, input) -> bool:
+        """Whether :meth:`with_skip` applies to this module and tensor."""
+        return self._is_pool2() and is_supported_pool(input) and input.is_contiguous(memory_format=_CL3D)
+
+    def with_skip(self, input):
+        """``(self(input), input)`` for an input that is also used elsewhere (the U-Net's skip connection): use the
+        returned pair and the two gradients of ``input`` are summed inside the pooling-gradient kernel."""
+        if not self._is_pool2():
+            raise NotImplementedError("FastMaxPool3d.with_skip supports MaxPool3d(2) only")
+        return max_pool3d_2x_with_skip(input)
+
+    def forward(self, input):
+        if not self._is_pool2():
             raise NotImplementedError(
                 f"FastMaxPool3d supports MaxPool3d(2) only, got kernel_size={self.kernel_size} stride={self.stride} "
                 f"padding={self.padding} dilation={self.dilation} ceil_mode={self.ceil_mode} "

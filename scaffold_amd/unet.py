@@ -179,7 +179,13 @@ class UNet(nn.Module):
     def forward(self, x):
         feats = [self._run(self.down_list[0], x)]
         for i in range(1, self.layers + 1):
-            feats.append(self._run(self.down_list[i], feats[-1]))
+            pool, block = self.down_list[i].maxpool_conv
+            if isinstance(pool, FastMaxPool3d) and not self.checkpointing and pool.serves(feats[-1]):
+                # the tensor that is pooled is also the skip connection: both gradients meet in the pooling kernel
+                pooled, feats[-1] = pool.with_skip(feats[-1])
+                feats.append(block(pooled))
+            else:
+                feats.append(self._run(self.down_list[i], feats[-1]))
         feats.reverse()
         out = feats[0]
         for i in range(self.layers):

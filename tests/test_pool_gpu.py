@@ -144,3 +144,35 @@ def test_full_size_level0_properties(device):
     picked = (gx.float() * x.float()).reshape(1, 32, 32, 2, 64, 2, 64, 2).sum(dim=(3, 5, 7))
     assert torch.equal(picked, y.detach().float())
     assert torch.equal(y.detach(), F.max_pool3d(x, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(1, 32, 6, 8, 10), (2, 16, 5, 7, 9), (1, 3, 4, 4, 6)])
+def test_pool_with_skip_sums_both_gradients_in_one_kernel(device, dtype, shape):
+    """``max_pool3d_2x_with_skip``: the pooled tensor and an alias of the input for the skip connection; the input's
+    gradient is the bits autograd's own accumulation gives (one fp32 sum, one rounding)."""
+    from scaffold_amd.pooling import max_pool3d_2x_with_skip
+
+    g = torch.Generator().manual_seed(17)
+    x0 = torch.randn(shape, generator=g).to(dtype).contiguous(memory_format=CL).to(device)
+    n, c, d, h, w = shape
+    gy = torch.randn((n, c, d // 2, h // 2, w // 2), generator=g).to(dtype).contiguous(memory_format=CL).to(device)
+    gs = torch.randn(shape, generator=g).to(dtype).contiguous(memory_format=CL).to(device)
+    a = x0.clone().requires_grad_(True)
+    pooled, skip = max_pool3d_2x_with_skip(a)
+    assert skip is not a and skip.data_ptr() == a.data_ptr() and torch.equal(pooled, F.max_pool3d(x0, 2))
+    torch.autograd.backward([pooled, skip], [gy, gs])
+    b = x0.clone().requires_grad_(True)
+    torch.autograd.backward([sa.max_pool3d_2x(b), b * 1], [gy, gs])
+    assert torch.equal(a.grad, b.grad)
+    # only one of the two uses differentiated
+    c1 = x0.clone().requires_grad_(True)
+    p1, s1 = max_pool3d_2x_with_skip(c1)
+    p1.backward(gy)
+    d1 = x0.clone().requires_grad_(True)
+    sa.max_pool3d_2x(d1).backward(gy)
+    assert torch.equal(c1.grad, d1.grad)
+    c2 = x0.clone().requires_grad_(True)
+    _, s2 = max_pool3d_2x_with_skip(c2)
+    s2.backward(gs)
+    assert torch.equal(c2.grad, gs)
