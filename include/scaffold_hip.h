@@ -110,7 +110,12 @@ int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const 
  * can pack both forms in ONE launch here and pass them with SFH_FLAG_WEIGHT_PACKED.
  * sfh_conv3d_packed_weight_bytes: bytes of the packed form for direction 0 (forward) or
  * 1 (data gradient), 0 when that direction of this problem does not read a packed weight.
- * Either output of sfh_conv3d_pack_weights may be NULL. No counterpart in the reference. */
+ * Either output of sfh_conv3d_pack_weights may be NULL. For a 2x2x2 stride-2 problem the forward
+ * form is what sfh_conv3d_fwd reads, and the data-gradient form is what sfh_convT3d_fwd -- the
+ * transposed convolution, which IS that data gradient -- reads under SFH_FLAG_WEIGHT_PACKED
+ * (describe the up-convolution's weight (Cin_T, Cout_T, 2,2,2) as the stride-2 convolution with
+ * cout = Cin_T, cin = Cout_T over the up-convolution's output extents). No counterpart in the
+ * reference. */
 size_t sfh_conv3d_packed_weight_bytes(const sfh_conv3d_desc* p, int dtype, int direction);
 int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w,
                             const int64_t w_stride[5], void* packed_fwd, void* packed_dgrad,

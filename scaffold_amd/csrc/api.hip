@@ -156,6 +156,37 @@ bool convT_uses_patch(const sfh_convT3d_desc& p, int dtype) {
   return p.kd == 2 && p.kh == 2 && p.kw == 2 && p.n >= 1 && patch_supported(convT_patch_args(p), dtype);
 }
 
+// The transposed convolution that is the data gradient of the kernel == stride convolution `p` (its input is p's output).
+sfh_convT3d_desc transposed_of(const sfh_conv3d_desc& p, const int32_t out[3]) {
+  sfh_convT3d_desc t{};
+  t.n = p.n; t.cin = p.cout; t.in_d = out[0]; t.in_h = out[1]; t.in_w = out[2];
+  t.cout = p.cin; t.kd = p.kd; t.kh = p.kh; t.kw = p.kw;
+  return t;
+}
+
+// One packing job of a weight (Cout, Cin, k, k, k) with element strides ws[5].
+struct PackSpec {
+  bool any;
+  MfmaConvArgs a;
+  int64_t s_out, s_red;
+  int flip;
+};
+
+// What the forward of `p` reads: the tiled 3x3x3 kernels' form, or the 2x2x2 stride-2 gather's.
+PackSpec fwd_pack_spec(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], const int64_t ws[5]) {
+  if (fwd_uses_mfma(p, dtype, out)) return {true, fwd_mfma_args(p, out), ws[0], ws[1], 0};
+  if (fwd_uses_patch(p, dtype, out)) return {true, patch_pack_args(p.cout, p.cin), ws[0], ws[1], 0};
+  return {false, MfmaConvArgs{}, 0, 0, 0};
+}
+
+// What the data gradient of `p` reads: the tiled kernels' transposed, tap-flipped form, or -- for a 2x2x2 stride-2
+// problem, whose data gradient is the transposed convolution -- the scatter's (produced = Cin, reduced = Cout).
+PackSpec dgrad_pack_spec(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], const int64_t ws[5]) {
+  if (check_dgrad(p) == SFH_OK && dgrad_uses_mfma(p, dtype, out)) return {true, dgrad_mfma_args(p, out), ws[1], ws[0], 1};
+  if (is_patch(p) && convT_uses_patch(transposed_of(p, out), dtype)) return {true, patch_pack_args(p.cin, p.cout), ws[1], ws[0], 0};
+  return {false, MfmaConvArgs{}, 0, 0, 0};
+}
+
 // ---- thin-channel problems (Cin == 1 stems, 1x1x1 heads) ---------------------------------------
 bool is_pointwise(const sfh_conv3d_desc& p) {
   return p.kd == 1 && p.kh == 1 && p.kw == 1 && p.sd == 1 && p.sh == 1 && p.sw == 1 && p.pd == 0 && p.ph == 0 && p.pw == 0;
@@ -299,6 +330,8 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st);
   }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && (flags & SFH_FLAG_WEIGHT_PACKED) && fwd_uses_patch(*p, dtype, out))
+    return patch_gather(patch_args(*p, out), dtype, x, w, bias, y, st);
   if (flags & SFH_FLAG_WEIGHT_PACKED) return fail(SFH_ERR_INVALID, "conv3d fwd: this problem does not read a packed weight");
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && fwd_uses_patch(*p, dtype, out)) {
     const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);
@@ -336,49 +369,46 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
 extern "C" size_t sfh_conv3d_packed_weight_bytes(const sfh_conv3d_desc* p, int dtype, int direction) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (direction == 0) return fwd_uses_mfma(*p, dtype, out) ? mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out)) : 0;
-  if (direction == 1)
-    return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)) ? mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out)) : 0;
-  return 0;
+  const int64_t unit[5] = {1, 1, 1, 1, 1};
+  const PackSpec spec = direction == 0 ? fwd_pack_spec(*p, dtype, out, unit)
+                                       : direction == 1 ? dgrad_pack_spec(*p, dtype, out, unit) : PackSpec{false, MfmaConvArgs{}, 0, 0, 0};
+  return spec.any ? mfma_conv_packed_weight_bytes(spec.a) : 0;
+}
+
+static int collect_pack_jobs(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t w_stride[5], void* packed_fwd,
+                             void* packed_dgrad, std::vector<MfmaPackItem>& jobs) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (w == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack: null weight");
+  if (packed_fwd != nullptr) {
+    const PackSpec spec = fwd_pack_spec(*p, dtype, out, w_stride);
+    if (!spec.any) return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the forward of this problem does not read a packed weight");
+    jobs.push_back(MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_fwd});
+  }
+  if (packed_dgrad != nullptr) {
+    const PackSpec spec = dgrad_pack_spec(*p, dtype, out, w_stride);
+    if (!spec.any) return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the data gradient of this problem does not read a packed weight");
+    jobs.push_back(MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_dgrad});
+  }
+  return SFH_OK;
 }
 
 extern "C" int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t w_stride[5], void* packed_fwd,
                                        void* packed_dgrad, void* stream) {
-  int32_t out[3];
-  if (int rc = check_conv(p, dtype, out)) return rc;
-  if (w == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack: null weight");
-  if (packed_fwd != nullptr && !fwd_uses_mfma(*p, dtype, out))
-    return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the forward of this problem does not read a packed weight");
-  if (packed_dgrad != nullptr && !(check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)))
-    return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the data gradient of this problem does not read a packed weight");
-  if (packed_fwd == nullptr && packed_dgrad == nullptr) return SFH_OK;
-  const MfmaConvArgs fa = packed_fwd != nullptr ? fwd_mfma_args(*p, out) : MfmaConvArgs{};
-  const MfmaConvArgs da = packed_dgrad != nullptr ? dgrad_mfma_args(*p, out) : MfmaConvArgs{};
-  return mfma_pack_weight_pair(fa, da, dtype, w, w_stride, packed_fwd, packed_dgrad, (hipStream_t)stream);
+  std::vector<MfmaPackItem> jobs;
+  if (int rc = collect_pack_jobs(p, dtype, w, w_stride, packed_fwd, packed_dgrad, jobs)) return rc;
+  if (jobs.empty()) return SFH_OK;
+  return mfma_pack_weight_batch(jobs.data(), (int)jobs.size(), dtype, (hipStream_t)stream);
 }
 
 extern "C" int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t nitems, int dtype, void* stream) {
   if (nitems < 0 || (nitems > 0 && items == nullptr)) return fail(SFH_ERR_INVALID, "conv3d pack batch: bad item list");
   std::vector<MfmaPackItem> jobs;
   jobs.reserve((size_t)nitems * 2);
-  for (int i = 0; i < nitems; ++i) {
-    const sfh_pack_item& it = items[i];
-    int32_t out[3];
-    if (int rc = check_conv(&it.desc, dtype, out)) return rc;
-    if (it.w == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack batch: item %d has a null weight", i);
-    if (it.packed_fwd != nullptr) {
-      if (!fwd_uses_mfma(it.desc, dtype, out))
-        return fail(SFH_ERR_UNSUPPORTED, "conv3d pack batch: the forward of item %d does not read a packed weight", i);
-      jobs.push_back(MfmaPackItem{fwd_mfma_args(it.desc, out), it.w, it.w_stride[0], it.w_stride[1], it.w_stride[2], it.w_stride[3],
-                                  it.w_stride[4], 0, it.packed_fwd});
-    }
-    if (it.packed_dgrad != nullptr) {
-      if (!(check_dgrad(it.desc) == SFH_OK && dgrad_uses_mfma(it.desc, dtype, out)))
-        return fail(SFH_ERR_UNSUPPORTED, "conv3d pack batch: the data gradient of item %d does not read a packed weight", i);
-      jobs.push_back(MfmaPackItem{dgrad_mfma_args(it.desc, out), it.w, it.w_stride[1], it.w_stride[0], it.w_stride[2], it.w_stride[3],
-                                  it.w_stride[4], 1, it.packed_dgrad});
-    }
-  }
+  for (int i = 0; i < nitems; ++i)
+    if (int rc = collect_pack_jobs(&items[i].desc, dtype, items[i].w, items[i].w_stride, items[i].packed_fwd, items[i].packed_dgrad,
+                                   jobs))
+      return rc;
   if (jobs.empty()) return SFH_OK;
   return mfma_pack_weight_batch(jobs.data(), (int)jobs.size(), dtype, (hipStream_t)stream);
 }
@@ -576,8 +606,15 @@ extern "C" size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int
 extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
                                const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
   if (int rc = check_convT(p, dtype)) return rc;
-  if (x == nullptr || w == nullptr || y == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
+  if (x == nullptr || w == nullptr || y == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
+    return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
   if (p->n == 0) return SFH_OK;
+  if (flags & SFH_FLAG_WEIGHT_PACKED) {
+    // w is the packed form: the data-gradient packing of the kernel == stride convolution this one transposes
+    if ((flags & SFH_FLAG_FORCE_GENERIC) || !convT_uses_patch(*p, dtype))
+      return fail(SFH_ERR_INVALID, "convT3d fwd: this problem does not read a packed weight");
+    return patch_scatter(convT_patch_args(*p), dtype, x, w, bias, y, (hipStream_t)stream);
+  }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && convT_uses_patch(*p, dtype)) {
     // produced channel = Cout (w_stride[1]), reduced channel = Cin (w_stride[0])
     const MfmaConvArgs pk = patch_pack_args(p->cout, p->cin);

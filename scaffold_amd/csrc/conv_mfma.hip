@@ -411,16 +411,6 @@ int mfma_pack_weight(const MfmaConvArgs& a, int dtype, const void* w, int64_t s_
   return launch_pack(dtype, pack_job(a, w, s_out, s_red, s_kd, s_kh, s_kw, flip, packed), none, st);
 }
 
-int mfma_pack_weight_pair(const MfmaConvArgs& fwd, const MfmaConvArgs& dgrad, int dtype, const void* w, const int64_t w_stride[5],
-                          void* packed_fwd, void* packed_dgrad, hipStream_t st) {
-  PackJob first{}, second{};
-  // forward: produced channel = Cout (w_stride[0]), reduced = Cin; data gradient: produced = Cin, reduced = Cout, taps flipped
-  if (packed_fwd != nullptr) first = pack_job(fwd, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, packed_fwd);
-  if (packed_dgrad != nullptr)
-    second = pack_job(dgrad, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, packed_dgrad);
-  return launch_pack(dtype, first, second, st);
-}
-
 int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStream_t st) {
   for (int i0 = 0; i0 < n; i0 += kPackBatch) {
     PackBatch b{};

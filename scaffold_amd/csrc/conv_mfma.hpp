@@ -31,9 +31,6 @@ struct MfmaPackItem {
   void* packed;
 };
 int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStream_t st);
-// Both packings of one weight (either output may be null) in one launch: the forward's and the data gradient's.
-int mfma_pack_weight_pair(const MfmaConvArgs& fwd, const MfmaConvArgs& dgrad, int dtype, const void* w, const int64_t w_stride[5],
-                          void* packed_fwd, void* packed_dgrad, hipStream_t st);
 // Bytes of fp32 slices the kernel needs when it cuts the reduction channels to fill the chip (0 when it does not).
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a);
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,

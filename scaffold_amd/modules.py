@@ -76,7 +76,7 @@ def compute_copy(param: Optional[torch.Tensor], dtype: Optional[torch.dtype]):
     return copy
 
 
-def _current_packs(owner: torch.Tensor, source: torch.Tensor, x: torch.Tensor, stride, padding, dilation):
+def _current_packs(owner: torch.Tensor, source: torch.Tensor, in_shape, stride, padding, dilation):
     """The packed forms of a parameter's weight for this problem, or ``None`` when the problem reads no packed weight.
 
     They are kept on the parameter (``owner._sfh_packs``) and trusted without a launch only under the rule that also
@@ -88,12 +88,12 @@ def _current_packs(owner: torch.Tensor, source: torch.Tensor, x: torch.Tensor, s
     table = owner.__dict__.get("_sfh_packs")
     if table is None:
         table = owner._sfh_packs = {}
-    key = (x.shape, padding)
+    key = (in_shape, padding)
     e = table.get(key)
     if e is None:
         if len(table) >= 8:  # a parameter meets few problems; shapes that keep changing are not worth the buffers
             table.clear()
-        e = table[key] = _c3.PackedWeights(source, x.shape, stride, padding, dilation)
+        e = table[key] = _c3.PackedWeights(source, in_shape, stride, padding, dilation)
         e.version = owner._version
         return e if e else None
     if not e:
@@ -168,22 +168,26 @@ class _Conv3dFn(torch.autograd.Function):
 
 class _ConvTranspose3dFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, weight_compute=None, bias_compute=None):
+    def forward(ctx, x, weight, bias, stride, weight_compute=None, bias_compute=None, packs=None):
         wc = weight if weight_compute is None else weight_compute
         bc = bias if bias_compute is None else bias_compute
-        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1)
-        ctx.save_for_backward(x, wc)
+        # `packs`: kept packed forms of the kernel == stride convolution this op transposes; its data-gradient form is
+        # what this forward reads, its forward form what the data gradient below reads
+        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad)
+        pf = None if packs is None else packs.fwd
+        ctx.save_for_backward(x, wc) if pf is None else ctx.save_for_backward(x, wc, pf)
         ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype, weight.dtype is not wc.dtype)
         return y
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
-        x, weight = ctx.saved_tensors
+        x, weight, *packed = ctx.saved_tensors
         stride, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
-        grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1) if needs_x else None
+        grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1,
+                                                    packed_weight=packed[0] if packed else None) if needs_x else None
         grad_w = None
         if needs_w:
             if master:
@@ -191,7 +195,7 @@ class _ConvTranspose3dFn(torch.autograd.Function):
             else:
                 grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None
 
 
 def _wants_grad(*tensors) -> bool:
@@ -241,10 +245,10 @@ class FastConv3d(nn.Conv3d):
             inner = x
         if master:
             return _Conv3dFn.apply(inner, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, x, stride, padding, dilation), slab)
+                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab)
         if w is self.weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
-                                   _current_packs(w, w, x, stride, padding, dilation), slab)
+                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab)
         return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab)
 
 
@@ -269,9 +273,18 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
                 f"stride={self.stride} padding={self.padding} output_padding={self.output_padding} "
                 f"dilation={self.dilation} groups={self.groups}"
             )
-        if master:
-            return _ConvTranspose3dFn.apply(x, self.weight, self.bias, tuple(self.stride), w, b)
-        return _ConvTranspose3dFn.apply(x, w, b, tuple(self.stride))
+        stride = tuple(self.stride)
+        if master or w is self.weight:
+            # the problem the packed forms belong to: the stride-k convolution over this op's output
+            n, _, d, h, wd = x.shape
+            big = torch.Size((n, w.shape[1], d * stride[0], h * stride[1], wd * stride[2]))
+            packs = _current_packs(self.weight, w, big, stride, (0, 0, 0), (1, 1, 1))
+            if packs is not None and (packs.fwd is None or packs.dgrad is None):
+                packs = None
+            if master:
+                return _ConvTranspose3dFn.apply(x, self.weight, self.bias, stride, w, b, packs)
+            return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, packs)
+        return _ConvTranspose3dFn.apply(x, w, b, stride)
 
 
 class FastGroupNorm(nn.GroupNorm):

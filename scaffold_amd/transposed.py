@@ -169,9 +169,11 @@ def conv_transpose3d_forward(
     config=None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    packed_weight: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Transposed 3-D convolution at ``kernel == stride``; NDHWC in and out; the bias is per
-    output channel (not per tap column)."""
+    output channel (not per tap column).  ``packed_weight``: the data-gradient form from
+    ``pack_weights(w, output_shape, stride=kernel, padding=0)`` -- this op is the data gradient of that convolution."""
     if not is_supported_transposed(x, w, bias, stride, padding, output_padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)} w={tuple(getattr(w, 'shape', ()))} "
@@ -194,10 +196,16 @@ def conv_transpose3d_forward(
     desc = ConvTDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2])
     code = _lib.dtype_code(x.dtype)
     with _lib.device_guard(x.device):
-        ws = _lib.workspace(L.sfh_convT3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
-        rc = L.sfh_convT3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w), _lib.strides5(w), _lib.ptr(bias),
-                               _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
-                               _lib.stream_ptr(x.device))
+        if packed_weight is not None:
+            if force_generic:
+                raise ValueError("packed_weight= cannot be combined with force_generic=")
+            rc = L.sfh_convT3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(packed_weight), None, _lib.ptr(bias),
+                                   _lib.ptr(y), None, 0, _lib.SFH_FLAG_WEIGHT_PACKED, _lib.stream_ptr(x.device))
+        else:
+            ws = _lib.workspace(L.sfh_convT3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
+            rc = L.sfh_convT3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w), _lib.strides5(w), _lib.ptr(bias),
+                                   _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
+                                   _lib.stream_ptr(x.device))
     _lib.check(rc, "conv_transpose3d_forward")
     return y
 
@@ -215,8 +223,10 @@ def conv_transpose3d_backward_data(
     config=None,
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
+    packed_weight: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """``grad_input = conv3d(grad_output, w, stride=k)`` with ``w`` unpermuted."""
+    """``grad_input = conv3d(grad_output, w, stride=k)`` with ``w`` unpermuted (``packed_weight``: that convolution's
+    forward form from ``pack_weights``)."""
     if not is_supported_transposed_bwd_data(grad_output, w, input_shape, stride, padding, output_padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: grad_output={tuple(getattr(grad_output, 'shape', ()))} w={tuple(getattr(w, 'shape', ()))} "
@@ -224,7 +234,8 @@ def conv_transpose3d_backward_data(
             f"dilation={dilation} groups={groups}"
         )
     k = tuple(int(v) for v in w.shape[2:])
-    return conv3d_forward(grad_output, w, None, k, 0, 1, 1, config=config, out=out, force_generic=force_generic)
+    return conv3d_forward(grad_output, w, None, k, 0, 1, 1, config=config, out=out, force_generic=force_generic,
+                          packed_weight=packed_weight)
 
 
 def conv_transpose3d_backward_weight(

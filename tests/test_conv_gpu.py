@@ -455,6 +455,24 @@ def test_prepacked_weight_gives_the_same_bits(device, cin, cout, sp, pad):
     assert none_d is None and torch.equal(only_f, pf)
 
 
+@pytest.mark.parametrize("cin_t,cout_t,sp", [(64, 32, (4, 6, 8)), (128, 64, (3, 4, 5)), (32, 32, (2, 2, 16))])
+def test_prepacked_weight_of_the_up_convolution_gives_the_same_bits(device, cin_t, cout_t, sp):
+    """The 2x2x2 stride-2 pair: the transposed convolution reads the data-gradient form, its own data gradient (a
+    stride-2 convolution) the forward form, of ``pack_weights`` for the stride-2 problem over the up-convolution's output."""
+    g = torch.Generator().manual_seed(71)
+    x = torch.randn((1, cin_t, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    w = (torch.randn((cin_t, cout_t, 2, 2, 2), generator=g) * 0.1).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    b = torch.randn(cout_t, generator=g).to(torch.bfloat16).to(device)
+    y = sa.conv_transpose3d_forward(x, w, b, 2)
+    gy = torch.randn(y.shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    gx = sa.conv_transpose3d_backward_data(gy, w, x.shape, 2)
+    pf, pd = sa.pack_weights(w, y.shape, 2, 0, 1)
+    assert pf is not None and pd is not None
+    assert torch.equal(sa.conv_transpose3d_forward(x, w, b, 2, packed_weight=pd), y)
+    assert torch.equal(sa.conv_transpose3d_backward_data(gy, w, x.shape, 2, packed_weight=pf), gx)
+    assert torch.equal(sa.conv3d_forward(gy, w, None, 2, 0, 1, packed_weight=pf), gx)
+
+
 def test_batch_packing_gives_the_same_bits(device):
     """Many weights packed in a few launches (more jobs than one launch's table holds), also on a second run of the
     same plan after the weights changed in place, and with layouts and dtypes mixed."""
