@@ -97,10 +97,26 @@ struct TileCoord { int n, d, h, w; };
 struct PersistGeom {
   int tiles_d, tiles_h, tiles_w, ntiles;  // bricks per output block (batch folded in)
   int nblocks, wgs_per_block, items_per_wg;
+  int blocked;  // brick order, see decode_tile
 };
 
+// Brick order. Plain: (n, d, h, w), w fastest. Blocked (brick counts along d and h divisible by 4): 4 x 4 groups of
+// bricks in (d, h), d fastest inside a group, then the groups along d, along h, then w, then n -- a workgroup's run of
+// 16 bricks is then a compact 16 x 16 rows region of one w column instead of a 4-row slab across the whole width, and
+// consecutive bricks share two of their six input planes: fewer halo voxels are fetched twice (1.34x against 1.7x
+// of the input at 128^3) and the re-fetched ones were read one step ago.
 __device__ __forceinline__ TileCoord decode_tile(int tile, const PersistGeom& gm) {
   TileCoord tc;
+  if (gm.blocked) {
+    const int din = tile & 3, hin = (tile >> 2) & 3;
+    tile >>= 4;
+    const int gd = gm.tiles_d >> 2, gh = gm.tiles_h >> 2;
+    tc.d = (tile % gd) * 4 + din; tile /= gd;
+    tc.h = (tile % gh) * 4 + hin; tile /= gh;
+    tc.w = tile % gm.tiles_w;
+    tc.n = tile / gm.tiles_w;
+    return tc;
+  }
   tc.w = tile % gm.tiles_w; tile /= gm.tiles_w;
   tc.h = tile % gm.tiles_h; tile /= gm.tiles_h;
   tc.d = tile % gm.tiles_d;
@@ -108,8 +124,22 @@ __device__ __forceinline__ TileCoord decode_tile(int tile, const PersistGeom& gm
   return tc;
 }
 
-// The brick after `tc` in (n, d, h, w) order, w fastest: increments with carries, no divisions.
+// The brick after `tc` in the order of decode_tile: increments with carries, no divisions.
 __device__ __forceinline__ TileCoord next_tile(TileCoord tc, const PersistGeom& gm) {
+  if (gm.blocked) {
+    if ((++tc.d & 3) != 0) return tc;
+    tc.d -= 4;
+    if ((++tc.h & 3) != 0) return tc;
+    tc.h -= 4;
+    tc.d += 4;  // next group along d
+    if (tc.d != gm.tiles_d) return tc;
+    tc.d = 0;
+    tc.h += 4;  // next group along h
+    if (tc.h != gm.tiles_h) return tc;
+    tc.h = 0;
+    if (++tc.w == gm.tiles_w) { tc.w = 0; ++tc.n; }
+    return tc;
+  }
   if (++tc.w == gm.tiles_w) {
     tc.w = 0;
     if (++tc.h == gm.tiles_h) {
@@ -398,6 +428,7 @@ int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const 
   const int64_t ntiles = (int64_t)a.n * gm.tiles_d * gm.tiles_h * gm.tiles_w;
   if (ntiles > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: too many bricks");
   gm.ntiles = (int)ntiles;
+  gm.blocked = (gm.tiles_d % 4 == 0 && gm.tiles_h % 4 == 0) ? 1 : 0;
   gm.nblocks = a.cout / 32;
   int per_block = kComputeUnits / gm.nblocks;
   if (per_block < 1) per_block = 1;
