@@ -351,3 +351,29 @@ def test_conv_reading_the_producers_slab_is_bitwise_the_assembled_form(device):
         y.backward(gy)
         results.append((y.detach(), x.grad, conv.weight.grad, norm.weight.grad, norm.bias.grad))
     assert all(torch.equal(a, b) for a, b in zip(*results))
+
+
+@pytest.mark.parametrize("batch,size,checkpoint", [(1, (12, 20, 36), False), (2, (8, 12, 20), False), (1, (8, 16, 32), True)])
+def test_shard_form_gradients_equal_the_padded_form(device, batch, size, checkpoint):
+    """Every route of the depth-shard form -- slabs written by GroupNorm and by the fused concat (one sample), assembled
+    slabs (a batch), sizes that make the decoder pad, activation checkpointing -- gives the padded form's loss and
+    parameter gradients bit for bit."""
+    torch.manual_seed(5)
+    model = UNet(1, 5, layers=2, base_width=32).to(device).to(memory_format=CL)
+    if checkpoint:
+        model.use_checkpointing()
+    g0 = torch.Generator().manual_seed(6)
+    x = (torch.rand((batch, 1, *size), generator=g0) < 0.1).float().contiguous(memory_format=CL).to(device)
+    lab = torch.randint(0, 5, (batch, *size), generator=g0).to(device)
+
+    def grads(shard):
+        model.set_shard_halo(shard)
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(x)
+        loss = sa.ce_dice_loss(logits, lab)
+        loss.backward()
+        return [loss.detach().clone()] + [p.grad.clone() for p in model.parameters()]
+
+    a, b = grads(False), grads(True)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
