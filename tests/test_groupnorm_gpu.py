@@ -75,6 +75,13 @@ SHAPES = [
     ((1, 64, 1, 1, 257), 8),
     ((1, 2048, 1, 1, 2), 8),
     ((1, 1024, 2, 2, 2), 32),
+    # the deep U-Net levels and their neighbours: many channels, few voxels (the fold of many small splits)
+    ((1, 256, 8, 16, 16), 8),
+    ((1, 256, 8, 16, 17), 8),
+    ((1, 512, 4, 8, 8), 8),
+    ((1, 1024, 2, 4, 4), 8),
+    ((1, 2048, 1, 2, 2), 8),
+    ((2, 256, 4, 8, 8), 8),
 ]
 
 
