@@ -189,6 +189,48 @@ def bench_groupnorm(args, device):
     }
 
 
+def bench_ingest(args, device, iters=20):
+    """One rank's share of a 128-cube sample as the dataset stores it (float32 (3, 64, 128, 128) + 16-bit mask) into the
+    bf16 channels-last slab of the first convolution and int64 labels, through the C ABI with outputs allocated once.
+    Algorithmic bytes per voxel: 4 C read + 2 C written + 2 + 8 for the label; beside it the three torch passes the
+    trainer runs (ScaFFold/utils/trainer.py:572-589 and autocast's cast)."""
+    import ctypes
+
+    from scaffold_amd import _lib
+
+    n, c, d, h, w, halo = 1, 3, 64, 128, 128, 1
+    g = torch.Generator().manual_seed(5002)
+    volume = torch.rand((n, c, d, h, w), generator=g).to(device)
+    mask = torch.randint(0, 11, (n, d, h, w), generator=g, dtype=torch.int16).to(device)
+    slab = torch.empty((n, c, d + 2 * halo, h, w), dtype=torch.bfloat16, device=device, memory_format=CL)
+    labels = torch.empty((n, d, h, w), dtype=torch.long, device=device)
+    L = _lib.lib()
+    desc = _lib.IngestDesc(n, c, 1, d * h * w, halo * h * w)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+
+    def abi():
+        _lib.check(L.sfh_shard_ingest(ctypes.byref(desc), _lib.dtype_code(torch.bfloat16), P(volume), P(mask), P(slab), P(labels),
+                                      torch.cuda.current_stream().cuda_stream), "sfh_shard_ingest")
+
+    def torch_passes():
+        x = volume.to(dtype=torch.float32, memory_format=CL).to(torch.bfloat16)
+        return x, mask.to(torch.long)
+
+    # a 7 us kernel: replayed from a graph of `chunk` launches so that the figure is kernel time, not the launcher's
+    chunk = 20
+    abi()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(chunk):
+            abi()
+    ms = event_time_ms(graph.replay, max(1, iters // chunk) * 2) / chunk
+    nbytes = n * d * h * w * (4 * c + 2 * c + 2 + 8)
+    return {"input": "1x3x64x128x128 float32 + int16 mask -> bf16 slab (halo 1) + int64 labels", "ms": ms, "algorithmic_bytes": nbytes,
+            "gbs": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "launched_from_python_ms": event_time_ms(abi, iters), "torch_three_passes_ms": event_time_ms(torch_passes, iters)}
+
+
 def gemm_reference(device):
     """What the vendor's tuned dense GEMM (hipBLASLt through torch.matmul, 8192^3 bf16) reaches on this box in this
     run: the practical ceiling of the matrix pipe under real data and the chip's power management, next to the
@@ -348,6 +390,8 @@ def main():
     ap.add_argument("--unet-profile", action="store_true",
                     help="run only 13 eager U-Net train steps (3 warm-up + 10) and print their time: the command to trace "
                          "when a per-kernel breakdown of the step is wanted")
+    ap.add_argument("--ingest-profile", action="store_true",
+                    help="run only the shard ingest kernel (200 launches) and print its time: the command to trace for it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB (reference point for HBM counter runs)")
     args = ap.parse_args()
@@ -359,6 +403,9 @@ def main():
         print("bench.py needs a GPU (no CPU fallback exists for the hot path)", file=sys.stderr)
         sys.exit(2)
     device = torch.device("cuda:0")
+    if args.ingest_profile:
+        print(json.dumps({"shard_ingest": bench_ingest(args, device, iters=200)}))
+        return
     if args.unet_profile:
         print(json.dumps({"unet_step_cfg5": bench_unet_step(args, device, eager_only=True)}))
         return
@@ -374,6 +421,10 @@ def main():
         details["groupnorm_cfg2"] = bench_groupnorm(args, device)
     except Exception as exc:  # report, do not hide
         details["groupnorm_cfg2"] = {"error": repr(exc)}
+    try:
+        details["shard_ingest"] = bench_ingest(args, device)
+    except Exception as exc:  # report, do not hide
+        details["shard_ingest"] = {"error": repr(exc)}
     if not args.skip_unet:
         try:
             details["unet_step_cfg5"] = bench_unet_step(args, device)

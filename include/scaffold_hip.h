@@ -270,6 +270,30 @@ int sfh_skip_concat_fwd(const sfh_concat_desc* p, int dtype, const void* a, cons
 int sfh_skip_concat_bwd(const sfh_concat_desc* p, int dtype, const void* g, void* ga, void* gb,
                         void* stream);
 
+/* ---- shard ingest ---------------------------------------------------------------------------
+ * From a dataset shard as stored on disk to the tensors the step reads. The generator writes a
+ * volume as float32 (C, D, H, W) and its mask as uint16 (D, H, W), one pair of .npy files per
+ * physical shard (ScaFFold/datagen/volumegen.py:259-292; file names `{id}_shard{k:06d}.npy` and
+ * `{id}_shard{k:06d}_mask.npy`, ScaFFold/utils/spatial_sharding.py:130-133,
+ * ScaFFold/utils/data_loading.py:308-317). The trainer then does, on the device,
+ * images.to(float32, memory_format=channels_last_3d) and masks.to(torch.long)
+ * (ScaFFold/utils/trainer.py:572-589), and autocast rounds the volume to the compute type before the
+ * first convolution. This entry point is those three steps in one pass over a batch already in
+ * device memory: x (N, halo_rows + rows + halo_rows, c) of `dtype` gets the channels-last volume in
+ * its interior (bit copy for SFH_FP32, one round-to-nearest-even otherwise) and zeros in its faces;
+ * labels (N, rows) int64 gets the widened mask. rows = D*H*W; halo_rows = h*H*W makes x the slab a
+ * depth shard's first convolution reads (see sfh_halo_assemble), 0 the plain tensor. `mask` holds
+ * 16-bit integers: unsigned as in the file (mask_signed = 0) or the loader's signed carrier
+ * (mask_signed = 1; ScaFFold/utils/data_loading.py:540-545); mask and labels may both be NULL.
+ * c is 1..4. Any alignment is accepted; 16-byte aligned pointers with rows % 4 == 0 take the
+ * vector path. */
+typedef struct sfh_ingest_desc {
+  int32_t n, c, mask_signed;
+  int64_t rows, halo_rows;
+} sfh_ingest_desc;
+int sfh_shard_ingest(const sfh_ingest_desc* p, int dtype, const void* volume, const void* mask, void* x,
+                     void* labels, void* stream);
+
 /* ---- gradient clipping + Adam -----------------------------------------------------------
  * The optimizer step of the trainer: torch.nn.utils.clip_grad_norm_(parameters, max_norm) followed by
  * torch.optim.Adam.step() (ScaFFold/utils/trainer.py:678-694, optimizer built at trainer.py:268-274),

@@ -23,6 +23,9 @@ function                reference it follows                                    
                                                                                      zero-variance / one-element-group cases
 ``train_step_loss``     ``ScaFFold/utils/trainer.py:640-663`` (fp32 log-softmax,      closed form on a two-voxel example
                         CE + 1 - mean foreground Dice, eps 1e-6)
+``shard_ingest``        ``ScaFFold/utils/trainer.py:572-589`` (``.to(float32,          the calls are the reference's own library
+                        channels_last_3d)``, ``.to(long)``) + autocast's cast;        routines; index-by-index loops on a small
+                        file layout ``ScaFFold/datagen/volumegen.py:259-292``         case and the round trip through ``.npy``
 ======================  =========================================================  =====================================
 
 The reference's own oracle *is* a library routine (torch in fp64), so this file calls the same
@@ -390,3 +393,24 @@ def ifs_volume(size: Sequence[int], *, n_fractals: int = 3, n_classes: int = 10,
     lab = torch.from_numpy(labels)[None]
     occ = (lab > 0).to(torch.float32)[:, None]
     return occ, lab
+
+
+# ---------------------------------------------------------------------------------------------
+# dataset shard -> step inputs
+# ---------------------------------------------------------------------------------------------
+def shard_ingest(volume: torch.Tensor, mask: Optional[torch.Tensor] = None, *, dtype=torch.float32, halo: int = 0):
+    """What the trainer does with a batch before the first convolution, on the CPU with the library calls it uses:
+    ``volume (N, C, D, H, W)`` float32 -> channels-last ``dtype`` (``ScaFFold/utils/trainer.py:575-580``; the rounding to
+    a 16-bit ``dtype`` is autocast's cast of the convolution input), ``mask (N, D, H, W)`` 16-bit -> int64
+    (``trainer.py:581-583``).  ``halo`` > 0 returns the depth slab instead: ``halo`` zero planes on each face, the
+    zero-filled form of the halo exchange (``ScaFFold/unet/conv3d.py:769-776``).  Returns ``(x, labels)``."""
+    x = volume.to(dtype=torch.float32, memory_format=torch.channels_last_3d).to(dtype)
+    if halo:
+        x = F.pad(x, (0, 0, 0, 0, halo, halo)).contiguous(memory_format=torch.channels_last_3d)
+    labels = None
+    if mask is not None:
+        if mask.dtype is torch.uint16:   # the file's type: widen through numpy, which has the conversion on every build
+            labels = torch.from_numpy(mask.numpy().astype("int64"))
+        else:
+            labels = mask.to(torch.long)
+    return x, labels

@@ -34,6 +34,8 @@ _EXPORTS = {
     "halo_assemble": "halo", "is_supported_halo": "halo",
     # skip connection concat
     "skip_concat": "concat", "is_supported_concat": "concat",
+    # dataset shards: file layout, reader, device ingest
+    "ingest": "shards", "is_supported_ingest": "shards", "ShardReader": "shards",
     # optimizer step
     "FusedClipAdam": "optim",
     # modules / model

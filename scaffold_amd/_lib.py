@@ -73,6 +73,10 @@ class ConcatDesc(ctypes.Structure):
     _fields_ = [("n", c_int32), ("c_a", c_int32), ("c_b", c_int32), ("rows", c_int64), ("halo_rows", c_int64)]
 
 
+class IngestDesc(ctypes.Structure):
+    _fields_ = [("n", c_int32), ("c", c_int32), ("mask_signed", c_int32), ("rows", c_int64), ("halo_rows", c_int64)]
+
+
 class LossDesc(ctypes.Structure):
     _fields_ = [("n", c_int32), ("classes", c_int32), ("spatial", c_int64), ("eps", c_float)]
 
@@ -122,6 +126,7 @@ _SIGNATURES = {
     "sfh_groupnorm_fwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
     "sfh_groupnorm_fwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_shard_ingest": (c_int, [POINTER(IngestDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_skip_concat_fwd": (c_int, [POINTER(ConcatDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_skip_concat_bwd": (c_int, [POINTER(ConcatDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_groupnorm_fwd_slab": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,

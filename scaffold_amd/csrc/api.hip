@@ -5,6 +5,7 @@
 #include <vector>
 #include "common.hpp"
 #include "concat.hpp"
+#include "ingest.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
 #include "conv_patch.hpp"
@@ -698,6 +699,24 @@ extern "C" int sfh_skip_concat_bwd(const sfh_concat_desc* p, int dtype, const vo
   if (p->n == 0) return SFH_OK;
   if (g == nullptr || ga == nullptr || gb == nullptr) return fail(SFH_ERR_INVALID, "skip concat: null tensor");
   return concat_backward(*p, dtype, g, ga, gb, (hipStream_t)stream);
+}
+
+// ---- shard ingest -----------------------------------------------------------------------------
+extern "C" int sfh_shard_ingest(const sfh_ingest_desc* p, int dtype, const void* volume, const void* mask, void* x, void* labels,
+                                void* stream) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "shard ingest: null descriptor");
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "shard ingest: bad dtype %d", dtype);
+  if (p->n < 0 || p->c < 1 || p->rows < 1 || p->halo_rows < 0)
+    return fail(SFH_ERR_INVALID, "shard ingest: bad extents n=%d c=%d rows=%lld halo_rows=%lld", p->n, p->c, (long long)p->rows,
+                (long long)p->halo_rows);
+  if (p->c > kIngestMaxChannels) return fail(SFH_ERR_UNSUPPORTED, "shard ingest: %d channels (1..%d supported)", p->c, kIngestMaxChannels);
+  if ((mask == nullptr) != (labels == nullptr)) return fail(SFH_ERR_INVALID, "shard ingest: mask and labels go together");
+  if (p->n == 0) return SFH_OK;
+  if (volume == nullptr || x == nullptr) return fail(SFH_ERR_INVALID, "shard ingest: null tensor");
+  if ((reinterpret_cast<uintptr_t>(volume) & 3) || (reinterpret_cast<uintptr_t>(mask) & 1) || (reinterpret_cast<uintptr_t>(labels) & 7) ||
+      (reinterpret_cast<uintptr_t>(x) & (dtype_size(dtype) - 1)))
+    return fail(SFH_ERR_INVALID, "shard ingest: a pointer is not aligned to its element size");
+  return shard_ingest(*p, dtype, (const float*)volume, mask, x, (int64_t*)labels, (hipStream_t)stream);
 }
 
 // ---- gradient clipping + Adam ------------------------------------------------------------
