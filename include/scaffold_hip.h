@@ -252,6 +252,19 @@ typedef struct sfh_halo_desc {
 } sfh_halo_desc;
 int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* x, const void* lo,
                       const void* hi, void* out, void* stream);
+/* The sending side of the same exchange, and its backward. sfh_halo_pack gathers the boundary planes a
+ * shard sends into plain dense buffers (the wire format of ScaFFold/unet/conv3d.py:710-731,757-768):
+ * lo_out (N, halo, H, W, C) = x[:, :halo] for the lower neighbour, hi_out = x[:, D - halo:] for the
+ * upper one; either may be NULL (no such neighbour). In the backward exchange (conv3d.py:795-841) the
+ * same call on the slab's gradient (depth D + 2*halo) packs the outer planes that go back to their
+ * owners, and sfh_halo_accumulate adds what came back into the shard's own boundary planes, in place:
+ * g[:, :halo] += lo_in, g[:, D - halo:] += hi_in (fp32 sum, one rounding; NULL = nothing received),
+ * g (N, D, H, W, C) being the interior of that gradient. D >= 2*halo is required so the two ranges
+ * stay disjoint (the reference requires a shard at least two voxels thick, conv3d.py:669). */
+int sfh_halo_pack(const sfh_halo_desc* p, int dtype, const void* x, void* lo_out, void* hi_out,
+                  void* stream);
+int sfh_halo_accumulate(const sfh_halo_desc* p, int dtype, void* g, const void* lo_in,
+                        const void* hi_in, void* stream);
 
 /* ---- skip connection concat ---------------------------------------------------------------
  * torch.cat([skip, upsampled], dim=1) of the decoder (ScaFFold/unet/unet_parts.py:107-120) on

@@ -258,7 +258,7 @@ def assert_close(actual, expected, problem: ConvProblem, direction: str = "fwd",
 
 
 def assert_baseline_tolerance(actual, expected, dtype: torch.dtype, what: str = "") -> ErrorReport:
-    """BASELINE.json's bar: fp32 within 1e-5 relative (to the RMS of the expected tensor);
+    """The parity bar of the hot path: fp32 within 1e-5 relative (to the RMS of the expected tensor);
     bf16/fp16 within 2e-2 relative + 1e-2 absolute, elementwise."""
     report = compare(actual, expected)
     a = actual.detach().to(device="cpu", dtype=torch.float64)
@@ -268,7 +268,7 @@ def assert_baseline_tolerance(actual, expected, dtype: torch.dtype, what: str = 
     else:
         ok = bool(((a - e).abs() <= 1e-2 + 2e-2 * e.abs()).all())
     if not ok:
-        raise AssertionError(f"{what}: outside BASELINE tolerance for {dtype}: {report}")
+        raise AssertionError(f"{what}: outside the parity tolerance for {dtype}: {report}")
     return report
 
 

@@ -31,7 +31,8 @@ _EXPORTS = {
     # pooling
     "max_pool3d_2x": "pooling", "is_supported_pool": "pooling", "FastMaxPool3d": "pooling",
     # halo slab of a depth shard
-    "halo_assemble": "halo", "is_supported_halo": "halo",
+    "halo_assemble": "halo", "is_supported_halo": "halo", "halo_pack": "halo", "halo_accumulate_": "halo",
+    "halo_exchange": "halo",
     # skip connection concat
     "skip_concat": "concat", "is_supported_concat": "concat",
     # dataset shards: file layout, reader, device ingest

@@ -144,6 +144,8 @@ _SIGNATURES = {
     "sfh_maxpool2_bwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_bwd_add": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_halo_assemble": (c_int, [POINTER(HaloDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_halo_pack": (c_int, [POINTER(HaloDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_halo_accumulate": (c_int, [POINTER(HaloDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_adam_slots": (c_int64, [c_int32, POINTER(c_int64)]),
     "sfh_adam_grad_sumsq": (c_int, [c_int32, POINTER(c_void_p), POINTER(c_int64), c_void_p, c_void_p, c_void_p]),
     "sfh_adam_clip_step": (c_int, [POINTER(AdamDesc), c_int32, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),

@@ -675,6 +675,31 @@ extern "C" int sfh_halo_assemble(const sfh_halo_desc* p, int dtype, const void* 
   return halo_assemble(*p, dtype, x, lo, hi, out, (hipStream_t)stream);
 }
 
+static int check_halo_faces(const sfh_halo_desc* p, int dtype, const char* what) {
+  if (p == nullptr) return fail(SFH_ERR_INVALID, "%s: null descriptor", what);
+  if (!dtype_ok(dtype)) return fail(SFH_ERR_INVALID, "%s: bad dtype %d", what, dtype);
+  if (p->n < 0 || p->c < 1 || p->d < 1 || p->h < 1 || p->w < 1 || p->halo < 0)
+    return fail(SFH_ERR_INVALID, "%s: bad extents n=%d c=%d (%d,%d,%d) halo=%d", what, p->n, p->c, p->d, p->h, p->w, p->halo);
+  return SFH_OK;
+}
+
+extern "C" int sfh_halo_pack(const sfh_halo_desc* p, int dtype, const void* x, void* lo_out, void* hi_out, void* stream) {
+  if (int rc = check_halo_faces(p, dtype, "halo pack")) return rc;
+  if (p->halo > p->d) return fail(SFH_ERR_INVALID, "halo pack: halo %d exceeds the depth %d", p->halo, p->d);
+  if (p->n == 0 || p->halo == 0) return SFH_OK;
+  if (x == nullptr) return fail(SFH_ERR_INVALID, "halo pack: null tensor");
+  return halo_pack(*p, dtype, x, lo_out, hi_out, (hipStream_t)stream);
+}
+
+extern "C" int sfh_halo_accumulate(const sfh_halo_desc* p, int dtype, void* g, const void* lo_in, const void* hi_in, void* stream) {
+  if (int rc = check_halo_faces(p, dtype, "halo accumulate")) return rc;
+  if (2 * (int64_t)p->halo > p->d)
+    return fail(SFH_ERR_UNSUPPORTED, "halo accumulate: depth %d is thinner than two halos of %d (the faces would overlap)", p->d, p->halo);
+  if (p->n == 0 || p->halo == 0) return SFH_OK;
+  if (g == nullptr) return fail(SFH_ERR_INVALID, "halo accumulate: null tensor");
+  return halo_accumulate(*p, dtype, g, lo_in, hi_in, (hipStream_t)stream);
+}
+
 // ---- skip connection concat ------------------------------------------------------------------
 static int check_concat(const sfh_concat_desc* p, int dtype) {
   if (p == nullptr) return fail(SFH_ERR_INVALID, "skip concat: null descriptor");

@@ -1,4 +1,4 @@
-"""The ScaFFold 3D U-Net over the HIP ops, with the widths BASELINE's configs need as arguments.
+"""The ScaFFold 3D U-Net over the HIP ops, with the widths of the benchmark configurations as arguments.
 
 Structure, child names and therefore ``state_dict`` keys follow the reference model
 (``ScaFFold/unet/unet_model.py:27-162``, ``ScaFFold/unet/unet_parts.py:107-240``):

@@ -205,3 +205,24 @@ def test_argument_checks_of_the_slab_concat_and_batch_packing_entry_points():
     items[0].w = 16
     items[0].packed_fwd = None                      # nothing asked for: nothing launched
     assert L.sfh_conv3d_pack_weights_batch(items, 1, bf16, None) == _lib.SFH_OK
+
+
+def test_argument_checks_of_the_halo_pack_and_accumulate_entry_points():
+    """Rejected (or accepted as empty) before anything is launched, so this runs without a GPU."""
+    from scaffold_amd._lib import HaloDesc
+
+    L = _lib.lib()
+    bf16 = 0
+    one = ctypes.c_void_p(16)  # never dereferenced
+    good = HaloDesc(1, 32, 8, 4, 4, 1)
+    for fn in (L.sfh_halo_pack, L.sfh_halo_accumulate):
+        assert fn(None, bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+        assert fn(ctypes.byref(good), 7, one, one, one, None) == _lib.SFH_ERR_INVALID
+        assert fn(ctypes.byref(HaloDesc(1, 0, 8, 4, 4, 1)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+        assert fn(ctypes.byref(HaloDesc(1, 32, 8, 4, 4, -1)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+        assert fn(ctypes.byref(good), bf16, None, one, one, None) == _lib.SFH_ERR_INVALID
+        assert fn(ctypes.byref(HaloDesc(0, 32, 8, 4, 4, 1)), bf16, None, None, None, None) == _lib.SFH_OK   # empty batch
+        assert fn(ctypes.byref(HaloDesc(1, 32, 8, 4, 4, 0)), bf16, None, None, None, None) == _lib.SFH_OK   # no halo
+    assert L.sfh_halo_pack(ctypes.byref(HaloDesc(1, 32, 2, 4, 4, 3)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
+    assert L.sfh_halo_accumulate(ctypes.byref(HaloDesc(1, 32, 3, 4, 4, 2)), bf16, one, one, one, None) == _lib.SFH_ERR_UNSUPPORTED
+    assert b"overlap" in L.sfh_last_error()

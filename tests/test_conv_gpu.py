@@ -3,7 +3,7 @@
 Standards, as in the reference's kernel suite (``triton_conv3d/reference.py:4-18``):
 1. bitwise on {-1,0,1} operands whose sums are exactly representable (catches a wrong voxel / tap /
    channel, which a tolerance hides), each with the shapes that exercise partial tiles and padding forms;
-2. the K/dtype-derived ``error_bound`` on Gaussian operands, plus BASELINE.json's tolerance
+2. the K/dtype-derived ``error_bound`` on Gaussian operands, plus the stated tolerance
    (fp32 1e-5 relative, bf16 2e-2 relative + 1e-2 absolute);
 3. fp32 must really accumulate in fp32 (``max_abs < 1e-4 * peak``).
 """
@@ -189,7 +189,7 @@ def test_mfma_gaussian_tolerance(device, dtype, direction):
 
 @pytest.mark.parametrize("direction", DIRS)
 def test_fp32_is_true_fp32(device, direction):
-    """Config 1 of BASELINE.json: 32->32 at 32^3 in fp32, fwd + dgrad + wgrad."""
+    """Benchmark configuration 1: 32->32 at 32^3 in fp32, fwd + dgrad + wgrad."""
     prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(32, 32, 32), dtype=torch.float32)
     g = torch.Generator().manual_seed(1000)
     x = torch.randn(prob.input_shape, generator=g).contiguous(memory_format=torch.channels_last_3d)
@@ -358,7 +358,7 @@ def test_depth_shard_with_halo_equals_slice_of_full_volume(device):
 
 # --- full size: properties that do not need the CPU oracle --------------------------------------
 def test_full_size_128cube_properties(device):
-    """BASELINE's headline conv (32 -> 32, 3x3x3, 128^3, bf16) on the exact standard: the fp64 oracle would
+    """The headline conv (32 -> 32, 3x3x3, 128^3, bf16) on the exact standard: the fp64 oracle would
     take minutes on the host, so the full-size launch is pinned by size-independent properties.  Operands are
     in {-1,0,1}, thinned so every partial sum is an integer below 2^8 and the results are exact in bf16:
     (1) the tiled MFMA kernels agree bitwise with the untiled direct kernels (two independent index paths,

@@ -93,7 +93,7 @@ def test_parity(device, dtype, shape, groups, relu):
 
 
 def test_config2_full_size(device):
-    """BASELINE.json config 2: N=2, C=64, 64^3, 8 groups, bf16; statistics vs fp64 and the elementwise
+    """Benchmark configuration 2: N=2, C=64, 64^3, 8 groups, bf16; statistics vs fp64 and the elementwise
     results through sampled slices (the fp64 reference of the full tensor would take minutes)."""
     shape = (2, 64, 64, 64, 64)
     g = torch.Generator().manual_seed(2000)
