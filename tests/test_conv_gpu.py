@@ -510,3 +510,31 @@ def test_pack_weights_declines_problems_that_read_the_weight_where_it_lies(devic
     pf, _ = sa.pack_weights(wb, x.shape, 1, 1, 1)
     with pytest.raises(ValueError):
         sa.conv3d_forward(x, wb, None, 1, 1, 1, packed_weight=pf, force_generic=True)
+
+
+# --- allocation contract ------------------------------------------------------------------------
+def test_outputs_are_allocated_once_in_their_final_layout(device):
+    """The forward output is allocated once, directly channels-last: peak memory of the call stays below 1.5 x the output
+    (triton_conv3d/tests/test_gather_gemm.py:796-822); the weight gradient comes back channels-last, [Cout][tap][Cin] in
+    memory (tests/test_bwd_weight.py:1276-1296); results of no_grad / inference_mode calls carry no graph."""
+    x = torch.randn((1, 32, 32, 32, 64), device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    w = (torch.randn((32, 32, 3, 3, 3), device=device) * 0.05).to(torch.bfloat16).contiguous(memory_format=CL)
+    gy = torch.randn_like(x)
+    sa.conv3d_forward(x, w, None, 1, 1)                         # first call: library load, workspace cache
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    y = sa.conv3d_forward(x, w, None, 1, 1)
+    torch.cuda.synchronize()
+    grown = torch.cuda.max_memory_allocated() - before
+    assert y.is_contiguous(memory_format=CL)
+    assert grown < 1.5 * y.numel() * y.element_size(), (grown, y.numel() * y.element_size())
+    gw = sa.conv3d_backward_weight(x, w.shape, gy, 1, 1)
+    assert gw.shape == w.shape and gw.stride(1) == 1 and gw.is_contiguous(memory_format=CL)
+    gx = sa.conv3d_backward_data(gy, w, x.shape, 1, 1)
+    assert gx.shape == x.shape and gx.is_contiguous(memory_format=CL)
+    conv = sa.FastConv3d(32, 32, 3, padding=1).to(device).to(torch.bfloat16)
+    with torch.no_grad():
+        assert not conv(x).requires_grad
+    with torch.inference_mode():
+        assert conv(x).is_inference()

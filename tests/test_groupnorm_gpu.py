@@ -272,3 +272,78 @@ def test_output_into_a_depth_slab_is_bitwise_the_plain_output(device, dtype, sha
     assert not hasattr(sa.group_norm(xb, 8, None, None, 1e-5, None, out_dtype=None, out_halo=halo), "_sfh_slab")
     if dtype is torch.bfloat16:
         assert not hasattr(sa.group_norm(x.to(device), 8, None, None, 1e-5, None, out_dtype=torch.float32, out_halo=halo), "_sfh_slab")
+
+
+# ---- argument layouts and partial gradients (the reference's edge suite: tests/test_triton_group_norm.py:402-425,661-684,
+# ---- tests/test_triton_group_norm_edge.py:437-535) -------------------------------------------------------------------
+def test_gradient_dtypes_under_autocast(device):
+    x, gamma, beta, dy = make((2, 32, 4, 5, 6), torch.bfloat16, seed=31)
+    xd = x.to(device).requires_grad_(True)
+    gd, bd = gamma.float().to(device).requires_grad_(True), beta.float().to(device).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = sa.group_norm(xd, 8, gd, bd, 1e-5, "relu")
+    assert y.dtype is torch.float32                   # the stock operator's dtype under autocast
+    y.backward(dy.to(device).float())
+    assert xd.grad.dtype is torch.bfloat16 and gd.grad.dtype is torch.float32 and bd.grad.dtype is torch.float32
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y2 = sa.group_norm(xd, 8, gd, bd, 1e-5, "relu", out_dtype=None)
+    assert y2.dtype is torch.bfloat16 and torch.equal(y2, y.to(torch.bfloat16))   # the narrow result is the wide one rounded once
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_partial_requires_grad_changes_no_other_gradient(device, dtype):
+    x, gamma, beta, dy = make((2, 32, 4, 5, 6), dtype, seed=32)
+    full = run_ours(x, 8, gamma, beta, dy, True, device)
+    for need in [(True, False, False), (False, True, False), (False, False, True), (True, True, False), (False, True, True)]:
+        xd = x.to(device).requires_grad_(need[0])
+        gd, bd = gamma.to(device).requires_grad_(need[1]), beta.to(device).requires_grad_(need[2])
+        y = sa.group_norm(xd, 8, gd, bd, 1e-5, "relu")
+        y.backward(dy.to(device))
+        assert torch.equal(y.detach(), full[0])
+        for got, want, needed in ((xd.grad, full[1], need[0]), (gd.grad, full[2], need[1]), (bd.grad, full[3], need[2])):
+            assert (got is None) == (not needed)
+            if needed:
+                assert torch.equal(got, want)
+
+
+def test_parameter_views_and_offset_inputs_are_accepted(device):
+    x, gamma, beta, dy = make((2, 16, 3, 5, 7), torch.float32, seed=33)
+    want = run_ours(x, 4, gamma, beta, dy, False, device)
+    # gamma / beta as every second element of a longer vector; x as a channels-last view with a storage offset
+    wide_g, wide_b = torch.zeros(32, device=device), torch.zeros(32, device=device)
+    wide_g[::2], wide_b[::2] = gamma.to(device), beta.to(device)
+    gv, bv = wide_g[::2].requires_grad_(True), wide_b[::2].requires_grad_(True)
+    assert not gv.is_contiguous()
+    big = torch.zeros((3, 16, 3, 5, 7), device=device).contiguous(memory_format=CL)
+    big[1:] = x.to(device)
+    xv = big[1:].requires_grad_(True)
+    assert xv.storage_offset() > 0 and xv.is_contiguous(memory_format=CL)
+    y = sa.group_norm(xv, 4, gv, bv, 1e-5, None)
+    y.backward(dy.to(device))
+    for got, ref in zip((y.detach(), xv.grad, gv.grad, bv.grad), want):
+        assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("layout", ["ncdhw", "sliced", "expanded", "transposed"])
+def test_cotangent_layouts_are_relaid_out_not_misread(device, layout):
+    x, gamma, beta, dy = make((2, 16, 4, 6, 6), torch.float32, seed=34)
+    if layout == "ncdhw":
+        cot = dy.to(device).contiguous()                                  # plain contiguous instead of channels-last
+    elif layout == "sliced":
+        wide = torch.randn((2, 16, 4, 6, 12), device=device)
+        wide[..., ::2] = dy.to(device)
+        cot = wide[..., ::2]
+    elif layout == "expanded":
+        dy = dy[:, :, :1].expand(-1, -1, 4, -1, -1)                      # stride 0 along depth
+        cot = dy.to(device)[:, :, :1].expand(-1, -1, 4, -1, -1)
+    else:
+        dy = dy.transpose(3, 4).contiguous().transpose(3, 4)             # H and W swapped in memory
+        cot = dy.to(device)
+        assert not cot.is_contiguous() and not cot.is_contiguous(memory_format=CL)
+    want = orc.group_norm_reference(x, 4, gamma, beta, 1e-5, True, dy.contiguous())
+    xd = x.to(device).requires_grad_(True)
+    gd, bd = gamma.to(device).requires_grad_(True), beta.to(device).requires_grad_(True)
+    y = sa.group_norm(xd, 4, gd, bd, 1e-5, "relu")
+    y.backward(cot)
+    for got, ref in zip((y.detach(), xd.grad, gd.grad, bd.grad), want):
+        assert orc.gn_rel_error(got, ref) <= orc.GN_TOLERANCE[torch.float32]
