@@ -258,6 +258,28 @@ class ShardReader:
             raise ValueError(f"{mask_path}: mask extent {mask.shape} does not match the volume's {volume.shape[1:]}")
         return volume, mask
 
+    # -- the reference dataset's host-side protocol (``BasicDataset``, data_loading.py:535-576) --------------------
+    @staticmethod
+    def _mask_carrier(mask) -> torch.Tensor:
+        # class ids travel as int16 and are widened on the device (data_loading.py:540-545)
+        return torch.from_numpy(np.array(mask, dtype=MASK_DTYPE, order="C").astype(np.int16, copy=False)).contiguous()
+
+    def load_mask_only(self, idx: int) -> torch.Tensor:
+        """The int16 mask of sample ``idx`` without touching its volume (what the class-weight estimate reads,
+        ``ScaFFold/utils/losses.py:76-85``)."""
+        _, mask_path = self.paths(self.ids[idx])
+        mask = np.load(mask_path, mmap_mode="r", allow_pickle=False)
+        if mask.dtype != MASK_DTYPE or mask.ndim != 3:
+            raise ValueError(f"{mask_path}: expected a uint16 (D, H, W) mask, found {mask.dtype} {mask.shape}")
+        return self._mask_carrier(mask)
+
+    def __getitem__(self, idx: int):
+        """``{"image": float32 (C, d, h, w), "mask": int16 (d, h, w)}`` on the host, as the reference's dataset returns
+        it to a ``DataLoader`` (``data_loading.py:560-576``)."""
+        volume, mask = self.read(self.ids[idx])
+        return {"image": torch.from_numpy(np.array(volume, dtype=VOLUME_DTYPE, order="C")).contiguous().float(),
+                "mask": self._mask_carrier(mask)}
+
     def _pinned(self, key, shape, dtype) -> torch.Tensor:
         buf = self._staging.get(key)
         if buf is None or tuple(buf.shape) != tuple(shape):

@@ -110,6 +110,28 @@ def test_reader_indexes_one_shard_of_every_sample(tmp_path):
         shards.ShardReader(images, masks, shard_id=9)
 
 
+def test_reader_speaks_the_reference_datasets_protocol(tmp_path):
+    """Indexable like the reference's dataset (a DataLoader and the class-weight estimate of ScaFFold/utils/losses.py:42-114
+    can be pointed at it): float32 image + int16 mask carrier per item, masks alone on request."""
+    images, masks, data = _write_dataset(str(tmp_path), ["0", "1", "2"], [0, 1])
+    r = shards.ShardReader(images, masks, shard_id=1)
+    counts = torch.zeros(12, dtype=torch.long)
+    for idx in range(len(r)):
+        item = r[idx]
+        v, m = data[r.ids[idx], 1]
+        assert item["image"].dtype is torch.float32 and item["mask"].dtype is torch.int16
+        assert item["image"].is_contiguous() and item["mask"].is_contiguous()
+        np.testing.assert_array_equal(item["image"].numpy(), v)
+        np.testing.assert_array_equal(item["mask"].numpy(), m.astype(np.int16))
+        only = r.load_mask_only(idx)
+        assert torch.equal(only, item["mask"])
+        counts += torch.bincount(only.reshape(-1).long(), minlength=12)      # losses.py:83-85
+    want = sum(np.bincount(data[s, 1][1].reshape(-1), minlength=12) for s in r.ids)
+    np.testing.assert_array_equal(counts.numpy(), want)
+    batch = next(iter(torch.utils.data.DataLoader(r, batch_size=2)))
+    assert batch["image"].shape == (2, 3, 4, 5, 6) and batch["mask"].shape == (2, 4, 5, 6) and batch["mask"].dtype is torch.int16
+
+
 def test_reader_refuses_files_of_another_type(tmp_path):
     images, masks, _ = _write_dataset(str(tmp_path), ["s"], [0])
     np.save(os.path.join(images, "d_shard000000.npy"), np.zeros((3, 4, 5, 6), dtype=np.float64))
