@@ -10,6 +10,7 @@
 // [voxel][channel] layout and read with ds_read_b64_tr_b16, which hands each lane four consecutive
 // voxels of one channel.
 #include "conv_patch.hpp"
+#include <type_traits>
 #include "mma.hpp"
 #include "reduce.hpp"
 
@@ -83,9 +84,69 @@ __global__ void __launch_bounds__(256) patch_gather_kernel(PatchArgs a, const T*
   for (int b = 0; b < NB; ++b) store_block<T>(acc[b], small + vs * a.csmall + (blk0 + b) * 32, bias, (blk0 + b) * 32, kg, valid);
 }
 
-// ---- scatter: transposed convolution -----------------------------------------------------------
-// A wavefront owns 32 small voxels x one block of 32 big channels x all 8 taps. grid = (voxel tiles of 128, cbig / 32).
+// The same for launches that would leave most of the chip idle (the U-Net's deepest levels: a few hundred voxels, hundreds
+// of channels, where one wavefront's chain of dependent loads sets the time). A workgroup owns 32 small voxels x one block of
+// 32 produced channels; its four wavefronts take two taps each, keep the loads of four chunks in flight, and their partial
+// blocks are added in wavefront order through LDS. grid = (voxel tiles of 32, csmall / 32).
 template <typename T>
+__global__ void __launch_bounds__(256) patch_gather_deep_kernel(PatchArgs a, const T* __restrict__ big, const T* __restrict__ packed,
+                                                                const T* __restrict__ bias, T* __restrict__ small, int64_t total) {
+  __shared__ float part[3][16][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kg = lane >> 5;
+  const int64_t v = (int64_t)blockIdx.x * 32 + (lane & 31);
+  const bool valid = v < total;
+  const int64_t vs = valid ? v : total - 1;
+  const Voxel vx = decode_small(a, vs);
+  const int nchunks = a.cbig / 32;
+  const int blk = blockIdx.y;
+  f32x16_t acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int tap = 2 * wave; tap < 2 * wave + 2; ++tap) {
+    const T* src = big + big_index(a, vx, tap) * a.cbig + kg * 8;
+    const T* wsrc = packed + ((((int64_t)blk * nchunks) * kTaps + tap) * 2 * 64 + lane) * 8;
+    const int64_t wstep = (int64_t)kTaps * 2 * 64 * 8;  // elements between the fragments of consecutive chunks
+    // U chunks per step: all their loads are issued before the first MFMA
+    auto step = [&](int cc, auto width) {
+      constexpr int U = decltype(width)::value;
+      uint4 bf[U][2], wf[U][2];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          bf[u][ks] = load16(src + (cc + u) * 32 + ks * 16);
+          wf[u][ks] = load16(wsrc + (cc + u) * wstep + ks * 64 * 8);
+        }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) acc = Mma32<T>::run(wf[u][ks], bf[u][ks], acc);
+    };
+    int cc = 0;
+    for (; cc + 4 <= nchunks; cc += 4) step(cc, std::integral_constant<int, 4>{});
+    for (; cc < nchunks; ++cc) step(cc, std::integral_constant<int, 1>{});
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[wave - 1][r][lane] = acc[r];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] += part[w][r][lane];
+    store_block<T>(acc, small + vs * a.csmall + blk * 32, bias, blk * 32, kg, valid);
+  }
+}
+
+// ---- scatter: transposed convolution -----------------------------------------------------------
+// A wavefront owns 32 small voxels x one block of 32 big channels x TS of the 8 taps.
+// grid = (voxel tiles of 128, cbig / 32, 8 / TS). TS = 8 reads the small tensor once; TS = 1 and 2 are for launches that
+// would otherwise leave most of the chip idle or give a CU a single long chain of dependent loads (the deeper levels):
+// more workgroups, each with a shorter chain, and the loads of several k-steps in flight per lane.
+template <typename T, int TS>
 __global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T* __restrict__ small, const T* __restrict__ packed,
                                                             const T* __restrict__ bias, T* __restrict__ big, int64_t total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -95,27 +156,40 @@ __global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T
   const int64_t vc = valid ? v : total - 1;
   const int nchunks = a.csmall / 32;
   const int blk = blockIdx.y;
-  f32x16_t acc[kTaps];
+  const int tap0 = blockIdx.z * TS;
+  f32x16_t acc[TS];
 #pragma unroll
-  for (int t = 0; t < kTaps; ++t)
+  for (int t = 0; t < TS; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
   const T* src = small + vc * a.csmall + kg * 8;
-  for (int cc = 0; cc < nchunks; ++cc) {
+  // U half-chunks (k-steps of 16 channels) per step: all their loads are issued before the first MFMA
+  auto step = [&](int k, auto width) {
+    constexpr int U = decltype(width)::value;
+    uint4 sf[U], wf[U][TS];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const uint4 sf = load16(src + cc * 32 + ks * 16);
-      uint4 wf[kTaps];
+    for (int u = 0; u < U; ++u) {
+      const int cc = (k + u) >> 1, ks = (k + u) & 1;
+      sf[u] = load16(src + cc * 32 + ks * 16);
 #pragma unroll
-      for (int t = 0; t < kTaps; ++t)
-        wf[t] = load16(packed + (((((int64_t)blk * nchunks + cc) * kTaps + t) * 2 + ks) * 64 + lane) * 8);
-#pragma unroll
-      for (int t = 0; t < kTaps; ++t) acc[t] = Mma32<T>::run(wf[t], sf, acc[t]);
+      for (int t = 0; t < TS; ++t)
+        wf[u][t] = load16(packed + (((((int64_t)blk * nchunks + cc) * kTaps + tap0 + t) * 2 + ks) * 64 + lane) * 8);
     }
-  }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < TS; ++t) acc[t] = Mma32<T>::run(wf[u][t], sf[u], acc[t]);
+  };
+  int k = 0;
+  if constexpr (TS == 1)
+    for (; k + 8 <= 2 * nchunks; k += 8) step(k, std::integral_constant<int, 8>{});
+  if constexpr (TS == 2)
+    for (; k + 4 <= 2 * nchunks; k += 4) step(k, std::integral_constant<int, 4>{});
+  for (; k < 2 * nchunks; ++k) step(k, std::integral_constant<int, 1>{});
   const Voxel vx = decode_small(a, vc);
 #pragma unroll
-  for (int t = 0; t < kTaps; ++t) store_block<T>(acc[t], big + big_index(a, vx, t) * a.cbig + blk * 32, bias, blk * 32, kg, valid);
+  for (int t = 0; t < TS; ++t)
+    store_block<T>(acc[t], big + big_index(a, vx, tap0 + t) * a.cbig + blk * 32, bias, blk * 32, kg, valid);
 }
 
 // ---- reduce: weight gradient -------------------------------------------------------------------
@@ -223,6 +297,11 @@ int launch_gather(const PatchArgs& a, const void* big, const void* packed, const
   const int64_t total = small_voxels(a);
   const int nb = gather_blocks(a);
   const dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.csmall / 32 / nb));
+  if (nb == 1 && (int64_t)grid.x * grid.y < kComputeUnits) {  // under one workgroup per CU (no gain measured above that)
+    hipLaunchKernelGGL((patch_gather_deep_kernel<T>), dim3((unsigned)cdiv(total, 32), (unsigned)(a.csmall / 32)), dim3(256), 0, st, a,
+                       (const T*)big, (const T*)packed, (const T*)bias, (T*)small, total);
+    return check_launch("patch_gather_deep_kernel");
+  }
 #define SFH_PATCH_GATHER(NB)                                                                                              \
   hipLaunchKernelGGL((patch_gather_kernel<T, NB>), grid, dim3(256), 0, st, a, (const T*)big, (const T*)packed, (const T*)bias, \
                      (T*)small, total)
@@ -237,9 +316,20 @@ int launch_gather(const PatchArgs& a, const void* big, const void* packed, const
 template <typename T>
 int launch_scatter(const PatchArgs& a, const void* small, const void* packed, const void* bias, void* big, hipStream_t st) {
   const int64_t total = small_voxels(a);
-  const dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
-  hipLaunchKernelGGL((patch_scatter_kernel<T>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
-                     (T*)big, total);
+  dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
+  const int64_t wgs = (int64_t)grid.x * grid.y;
+  if (wgs < kComputeUnits) {  // under one workgroup per CU: one tap per workgroup
+    grid.z = kTaps;
+    hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
+                       (T*)big, total);
+  } else if (wgs <= 2 * kComputeUnits) {  // one or two per CU: two taps (the big voxels next to each other along W)
+    grid.z = kTaps / 2;
+    hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
+                       (T*)big, total);
+  } else {
+    hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
+                       (const T*)bias, (T*)big, total);
+  }
   return check_launch("patch_scatter_kernel");
 }
 

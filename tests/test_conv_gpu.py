@@ -218,6 +218,9 @@ CONVT_SHAPES = [
     (1, 64, 32, (9, 6, 11), (2, 2, 2), True),
     (2, 64, 96, (4, 4, 5), (2, 2, 2), False),
     (1, 32, 32, (1, 1, 1), (2, 2, 2), True),
+    # launches of a few workgroups take the one-tap-per-workgroup / unrolled forms: chunk counts that are not a multiple of the unroll
+    (1, 160, 96, (2, 2, 3), (2, 2, 2), True),
+    (1, 96, 160, (2, 3, 2), (2, 2, 2), False),
 ]
 
 
