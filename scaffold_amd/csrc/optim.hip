@@ -90,9 +90,16 @@ template <int SHADOW>  // 0 none, 1 bf16, 2 fp16
 __global__ void __launch_bounds__(kBlock) clip_adam_kernel(AdamTable t, AdamCoef c, const float* __restrict__ slots, int nslots,
                                                            int slot_base, const float* __restrict__ step_ptr, float* grad_norm) {
   __shared__ float red4[4];
-  float total = 0.f;
-  for (int i = threadIdx.x; i < nslots; i += kBlock) total += slots[i];
-  total = block_sum(total, red4);
+  // every workgroup folds all slots, the same way: four loads in flight per lane (one after the other they were a chain
+  // of a dozen dependent trips to L2 in front of every workgroup's own work), combined in a fixed order
+  float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+  int i = threadIdx.x;
+  for (; i + 3 * kBlock < nslots; i += 4 * kBlock) {
+    const float a0 = slots[i], a1 = slots[i + kBlock], a2 = slots[i + 2 * kBlock], a3 = slots[i + 3 * kBlock];
+    t0 += a0; t1 += a1; t2 += a2; t3 += a3;
+  }
+  for (; i < nslots; i += kBlock) t0 += slots[i];
+  float total = block_sum((t0 + t1) + (t2 + t3), red4);
   const float norm = sqrtf(total);
   float scale = 1.f;
   if (c.max_norm > 0.f) scale = fminf(c.max_norm / (norm + 1e-6f), 1.f);
