@@ -322,7 +322,7 @@ int launch_scatter(const PatchArgs& a, const void* small, const void* packed, co
     grid.z = kTaps;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total);
-  } else if (wgs <= 2 * kComputeUnits) {  // one or two per CU: two taps (the big voxels next to each other along W)
+  } else if (wgs <= 4 * kComputeUnits) {  // up to four per CU: two taps (the big voxels next to each other along W)
     grid.z = kTaps / 2;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total);
