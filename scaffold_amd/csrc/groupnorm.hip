@@ -632,17 +632,44 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   }
   }
   if (fused && n == 0 && (dgamma != nullptr || dbeta != nullptr)) {
+    // More channels than workgroups (the deepest levels): eight at a time, one per group of 32 lanes (workgroup b takes
+    // channels b, b + gridDim.x, ...): each lane
+    // adds every 32nd split partial of its channel, the 32 lanes meet in a butterfly; no LDS and no barrier. (One channel
+    // at a time over all 256 threads cost the deepest level, 512 channels over 64 workgroups, 6 us of serial rounds.)
     const int total = N * nsplit;
-    for (int c = blockIdx.x; c < C; c += gridDim.x) {
-      float s1 = 0.f, s2 = 0.f;
-      for (int i = tid; i < total; i += kBlock) {
-        const float* p = part + (int64_t)i * 2 * C;
-        s1 += p[c];
-        s2 += p[C + c];
+    const int grp = tid >> 5, li = tid & 31;
+    if (C <= (int)gridDim.x) {  // at most one channel per workgroup: all 256 threads on it
+      for (int c = blockIdx.x; c < C; c += gridDim.x) {
+        float s1 = 0.f, s2 = 0.f;
+        for (int i = tid; i < total; i += kBlock) {
+          const float* p = part + (int64_t)i * 2 * C;
+          s1 += p[c];
+          s2 += p[C + c];
+        }
+        s1 = block_sum256(s1, red4);
+        s2 = block_sum256(s2, red4);
+        if (tid == 0) {
+          if (dgamma != nullptr) dgamma[c] = s1;
+          if (dbeta != nullptr) dbeta[c] = s2;
+        }
       }
-      s1 = block_sum256(s1, red4);
-      s2 = block_sum256(s2, red4);
-      if (tid == 0) {
+    } else
+    for (int c0 = blockIdx.x; c0 < C; c0 += 8 * gridDim.x) {  // c0: the channel of group 0, uniform over the workgroup
+      const int c = c0 + grp * gridDim.x;
+      float s1 = 0.f, s2 = 0.f;
+      if (c < C) {
+        for (int i = li; i < total; i += 32) {
+          const float* p = part + (int64_t)i * 2 * C;
+          s1 += p[c];
+          s2 += p[C + c];
+        }
+      }
+#pragma unroll
+      for (int off = 16; off >= 1; off >>= 1) {
+        s1 += __shfl_xor(s1, off, 32);
+        s2 += __shfl_xor(s2, off, 32);
+      }
+      if (li == 0 && c < C) {
         if (dgamma != nullptr) dgamma[c] = s1;
         if (dbeta != nullptr) dbeta[c] = s2;
       }
