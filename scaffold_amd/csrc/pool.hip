@@ -92,6 +92,8 @@ __global__ void __launch_bounds__(kBlock) maxpool2_bwd_kernel(PoolGeom g, int cd
   const int od = (int)(v % cd);
   const int64_t n = v / cd;
   const bool pooled = (od < g.od) & (oh < g.oh) & (ow < g.ow);
+  // gy and idx are read only where a pooled cell exists: with an odd or unit extent some lanes have none, and when the
+  // pooled tensor is empty the pointers themselves are not valid, so there is no address to clamp to.
   float grad[V];
   uint8_t which[V];
 #pragma unroll
@@ -113,22 +115,31 @@ __global__ void __launch_bounds__(kBlock) maxpool2_bwd_kernel(PoolGeom g, int cd
   }
   const int64_t cell = (((n * g.d + 2 * od) * g.h + 2 * oh) * g.w + 2 * ow) * (int64_t)g.c + cv * V;
   T* dst = gx + cell;
+  bool inside[8];
+  int64_t at[8];
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
     const int kd = k >> 2, kh = (k >> 1) & 1, kw = k & 1;
-    if ((2 * od + kd < g.d) & (2 * oh + kh < g.h) & (2 * ow + kw < g.w)) {
-      const int64_t at = (((int64_t)kd * g.h + kh) * g.w + kw) * g.c;
-      float out[V];
+    inside[k] = (2 * od + kd < g.d) & (2 * oh + kh < g.h) & (2 * ow + kw < g.w);
+    at[k] = inside[k] ? (((int64_t)kd * g.h + kh) * g.w + kw) * g.c : 0;  // voxel 0 of the cell always exists
+  }
+  // The eight reads of `add` are issued together, from voxel 0 of the cell where a voxel lies outside the tensor
+  // (under per-lane conditions they wait for one another: eight trips to memory in a row on the small tensors).
+  float more[8][V];
+  if (add != nullptr) {  // a second gradient of the pooled tensor (its use as a skip connection), summed in fp32
 #pragma unroll
-      for (int e = 0; e < V; ++e) out[e] = which[e] == k ? grad[e] : 0.f;
-      if (add != nullptr) {  // a second gradient of the pooled tensor (its use as a skip connection), summed in fp32
-        float more[V];
-        LdN<T, V>::run(add + cell + at, more);
+    for (int k = 0; k < 8; ++k) LdN<T, V>::run(add + cell + at[k], more[k]);
+  }
 #pragma unroll
-        for (int e = 0; e < V; ++e) out[e] += more[e];
-      }
-      StN<T, V>::run(dst + at, out);
+  for (int k = 0; k < 8; ++k) {
+    float out[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) out[e] = which[e] == k ? grad[e] : 0.f;
+    if (add != nullptr) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] += more[k][e];
     }
+    if (inside[k]) StN<T, V>::run(dst + at[k], out);
   }
 }
 
