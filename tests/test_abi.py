@@ -226,3 +226,36 @@ def test_argument_checks_of_the_halo_pack_and_accumulate_entry_points():
     assert L.sfh_halo_pack(ctypes.byref(HaloDesc(1, 32, 2, 4, 4, 3)), bf16, one, one, one, None) == _lib.SFH_ERR_INVALID
     assert L.sfh_halo_accumulate(ctypes.byref(HaloDesc(1, 32, 3, 4, 4, 2)), bf16, one, one, one, None) == _lib.SFH_ERR_UNSUPPORTED
     assert b"overlap" in L.sfh_last_error()
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 and as C++, and a C caller links and runs -- here only calls
+    that need no GPU (version, an argument check, the error string)."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler here")
+    include = os.path.join(ROOT, "include")
+    libdir = os.path.dirname(_lib.lib_path())
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "scaffold_hip.h"\n'
+        "int main(void) {\n"
+        "  sfh_ingest_desc d = {1, 9, 0, 64, 0};  /* nine channels: refused before any launch */\n"
+        "  char one[16] = {0};\n"
+        "  int rc = sfh_shard_ingest(&d, SFH_BF16, one, NULL, one, NULL, NULL);\n"
+        '  printf("%d %d %s\\n", sfh_version(), rc, sfh_last_error());\n'
+        "  return rc == SFH_ERR_UNSUPPORTED && strstr(sfh_last_error(), \"channels\") != NULL ? 0 : 1;\n"
+        "}\n")
+    exe = tmp_path / "caller"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", f"-I{include}", str(src), "-o", str(exe), f"-L{libdir}",
+                    "-lscaffold_hip", f"-Wl,-rpath,{libdir}"], check=True, capture_output=True, text=True)
+    if shutil.which("g++") is not None:
+        cpp = tmp_path / "caller.cpp"
+        cpp.write_text('#include "scaffold_hip.h"\nint main() { return sfh_version() > 0 ? 0 : 1; }\n')
+        subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", f"-I{include}", str(cpp)], check=True,
+                       capture_output=True, text=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, (out.stdout, out.stderr)
+    assert out.stdout.split()[0] == str(_lib.lib().sfh_version())
