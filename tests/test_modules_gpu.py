@@ -377,3 +377,57 @@ def test_shard_form_gradients_equal_the_padded_form(device, batch, size, checkpo
 
     a, b = grads(False), grads(True)
     assert all(torch.equal(p, q) for p, q in zip(a, b))
+
+
+def test_from_shard_files_to_updated_weights(device, tmp_path):
+    """The whole path on one rank's share: a volume / mask pair as the generator writes it (float32 (3, d, h, w) + uint16),
+    read and ingested into the stem's slab, the 3-channel U-Net in shard form under bf16 autocast, the fused loss head and
+    one clipped Adam step -- against stock modules in fp32 on the host, fed the reference's way
+    (ScaFFold/utils/trainer.py:572-694)."""
+    import numpy as np
+
+    from scaffold_amd import shards
+
+    size = (8, 16, 32)
+    rng = np.random.default_rng(12)
+    volume = (rng.random((3,) + size, dtype=np.float32) * (rng.random(size) < 0.1)).astype(np.float32)   # sparse, coloured
+    mask = (rng.integers(1, 5, size=size) * (volume.sum(0) > 0)).astype(np.uint16)
+    images, masks = tmp_path / "volumes", tmp_path / "masks"
+    images.mkdir(), masks.mkdir()
+    np.save(images / "0_shard000000.npy", volume)
+    np.save(masks / "0_shard000000_mask.npy", mask)
+
+    torch.manual_seed(9)
+    stock = UNet(3, 5, layers=2, base_width=32, stock=True)
+    ours = UNet(3, 5, layers=2, base_width=32).to(device).to(memory_format=CL)
+    ours.load_state_dict(stock.state_dict())
+    ours.set_shard_halo(True)
+    init = torch.cat([p.detach().flatten().double() for p in stock.parameters()])
+
+    # the reference's arm: host tensors, channels_last_3d float32 image, long mask, torch loss recipe, clip + Adam
+    x0 = torch.from_numpy(volume)[None].contiguous(memory_format=CL)
+    lab0 = torch.from_numpy(mask.astype(np.int16))[None].long()
+    opt0 = torch.optim.Adam(stock.parameters(), lr=1e-3)
+    l0, _ = _step(stock, x0, lab0)          # in fp32: the host's bf16 kernels are not the oracle here
+    g0 = torch.cat([p.grad.flatten().double() for p in stock.parameters()])     # before the clipping scales them in place
+    torch.nn.utils.clip_grad_norm_(stock.parameters(), 1.0)
+    opt0.step()
+
+    # this build's arm: files -> pinned staging -> one ingest kernel (bf16 slab + int64 labels) -> HIP ops
+    reader = shards.ShardReader(images, masks, shard_id=0)
+    x1, lab1 = reader.load("0", device, dtype=torch.bfloat16, out_halo=1)
+    assert x1._sfh_slab[1] == 1 and torch.equal(lab1.cpu(), lab0)
+    opt1 = sa.FusedClipAdam(ours.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        logits = ours(x1)
+    l1 = sa.ce_dice_loss(logits, lab1)
+    l1.backward()
+    g1 = torch.cat([p.grad.flatten().cpu().double() for p in ours.parameters()])
+    opt1.step()
+
+    assert abs(l0.item() - l1.item()) <= 2e-2 * abs(l0.item())
+    assert ((g1 - g0).norm() / g0.norm()).item() < 5e-2          # aggregate bf16 tolerance of the reference's own suite
+    u0 = torch.cat([p.detach().flatten().double() for p in stock.parameters()]) - init
+    u1 = torch.cat([p.detach().flatten().cpu().double() for p in ours.parameters()]) - init
+    assert u0.abs().max() <= 1.001e-3 and u1.abs().max() <= 1.001e-3
+    assert (torch.dot(u0, u1) / (u0.norm() * u1.norm())).item() > 0.9
