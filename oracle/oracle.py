@@ -23,6 +23,15 @@ function                reference it follows                                    
                                                                                      zero-variance / one-element-group cases
 ``train_step_loss``     ``ScaFFold/utils/trainer.py:640-663`` (fp32 log-softmax,      closed form on a two-voxel example
                         CE + 1 - mean foreground Dice, eps 1e-6)
+``assert_baseline_...``  the parity bar itself: fp32 1e-5 relative, 16-bit          hand-computed tensors just inside and just
+                        2e-2 relative + 1e-2 absolute, elementwise                    outside each limit, NaN, one bad element
+``gn_rel_error``        ``tests/test_triton_group_norm.py:57-78`` (max error over     hand-computed three-element case
+                        max |reference|)
+``chaos_game``          ``ScaFFold/datagen/generate_fractal_points.py:62-104``        fixed point (I - M)^-1 o of one map; dyadic
+                                                                                     orbit of x/2, x/2 + 1/2 by hand
+``points_to_voxel_...``  ``ScaFFold/datagen/volumegen.py:103-160``                    hand-computed indices (scale, centring, clip)
+``ifs_volume``          ``volumegen.py:259-292`` (mask = class id + 1, painted in     one contraction -> one centre voxel; the
+                        turn)                                                         segment and Sierpinski attractors' voxel sets
 ``shard_ingest``        ``ScaFFold/utils/trainer.py:572-589`` (``.to(float32,          the calls are the reference's own library
                         channels_last_3d)``, ``.to(long)``) + autocast's cast;        routines; index-by-index loops on a small
                         file layout ``ScaFFold/datagen/volumegen.py:259-292``         case and the round trip through ``.npy``
@@ -189,20 +198,6 @@ def conv_reference(problem: ConvProblem, operands: dict, direction: str = "fwd",
     return grad
 
 
-def conv_working_dtype(problem: ConvProblem, operands: dict, direction: str = "fwd") -> torch.Tensor:
-    """The same convolution computed by torch's CPU kernels in the operands' own dtype (the
-    reference's CPU path: its ladders fall to stock ``nn.Conv3d`` off-GPU, ``ScaFFold/unet/conv3d.py:1371-1378``)."""
-    x, w, b = operands["input"], operands["weight"], operands.get("bias")
-    if direction == "fwd":
-        return _conv(problem, x, w, b)
-    gy = operands["grad_output"]
-    x = x.detach().requires_grad_(True)
-    w = w.detach().requires_grad_(True)
-    y = _conv(problem, x, w, b)
-    gx, gw = torch.autograd.grad(y, (x, w), gy)
-    return gx if direction == "bwd-data" else gw
-
-
 # ---------------------------------------------------------------------------------------------
 # comparison / tolerance policy
 # ---------------------------------------------------------------------------------------------
@@ -361,35 +356,69 @@ def train_step_loss(logits: torch.Tensor, labels: torch.Tensor, n_classes: int, 
     return ce + (1.0 - dice[:, 1:].mean())
 
 
-def ifs_volume(size: Sequence[int], *, n_fractals: int = 3, n_classes: int = 10, n_maps: int = 4, iterations: int = 200_000,
-               seed: int = 5000):
-    """Config 5's synthetic sample: voxelised points of random 3-D iterated function systems
-    (``n_maps`` affine maps each, contraction factors U(0.3, 0.7)); returns (occupancy float32
-    (1, 1, D, H, W), labels int64 (1, D, H, W)) with label = class id in 1..n_classes, 0 = background."""
+def chaos_game(mats, offs, choice):
+    """Orbit of an iterated function system: p_0 = origin, p_n = mats[choice[n]] @ p_{n-1} + offs[choice[n]] for
+    n = 1 .. len(choice) - 1 (``ScaFFold/datagen/generate_fractal_points.py:62-104``: the first point is the origin and
+    every later one is the chosen affine map of its predecessor).  Returns the (len(choice), 3) float64 points."""
+    import numpy as np
+
+    mats = np.asarray(mats, dtype=np.float64)
+    offs = np.asarray(offs, dtype=np.float64)
+    pts = np.zeros((len(choice), 3))
+    p = np.zeros(3)
+    for i in range(1, len(choice)):
+        t = choice[i]
+        p = mats[t] @ p + offs[t]
+        pts[i] = p
+    return pts
+
+
+def points_to_voxel_indices(points, grid_size: int, eps: float = 1e-6):
+    """The voxels a point cloud occupies on a ``grid_size``-cube (``ScaFFold/datagen/volumegen.py:103-160``): one
+    isotropic voxel size ``(largest extent + eps) / grid_size`` for all axes, the cloud's bounding box centred in the
+    grid (offset ``(grid_size - span) / 2`` per axis, span in voxels), floor, clip to the grid, duplicates removed.
+    Non-finite coordinates are refused.  Returns a (K, 3) int64 array sorted lexicographically."""
+    import numpy as np
+
+    points = np.asarray(points, dtype=np.float64)
+    if not np.isfinite(points).all():
+        raise ValueError("non-finite coordinates in the point cloud")
+    mins = points.min(axis=0)
+    voxel = (float((points.max(axis=0) - mins).max()) + eps) / grid_size
+    scaled = (points - mins) / voxel
+    offset = (grid_size - scaled.max(axis=0)) / 2.0
+    idx = np.clip(np.floor(scaled + offset).astype(np.int64), 0, grid_size - 1)
+    return np.unique(idx, axis=0)
+
+
+def ifs_volume(grid_size: int, *, n_fractals: int = 3, n_classes: int = 10, n_maps: int = 4, iterations: int = 200_000,
+               seed: int = 5000, systems=None, burn_in: int = 100):
+    """Config 5's synthetic sample on a ``grid_size``-cube: the voxelised orbits of ``n_fractals`` random 3-D iterated
+    function systems (``n_maps`` affine maps each: a random rotation scaled by a contraction factor U(0.3, 0.7), offset
+    U(-1, 1)^3, maps chosen uniformly), painted in turn with mask value ``class id + 1`` as the generator does
+    (``ScaFFold/datagen/volumegen.py:259-292``: later fractals overwrite earlier ones; background stays 0).
+    ``systems`` replaces the random draw by explicit ``(class_id, mats, offs)`` triples (orbit choices still come from
+    ``seed``).  The first ``burn_in`` points of an orbit are dropped (they are not yet on the attractor).
+    Returns (occupancy float32 (1, 1, G, G, G), labels int64 (1, G, G, G)); a depth shard is a slice of both."""
     import numpy as np
 
     rng = np.random.default_rng(seed)
-    d, h, w = (int(v) for v in size)
-    labels = np.zeros((d, h, w), dtype=np.int64)
-    for _ in range(n_fractals):
-        cls = int(rng.integers(1, n_classes + 1))
-        mats, offs = [], []
-        for _ in range(n_maps):
-            q, _r = np.linalg.qr(rng.standard_normal((3, 3)))
-            mats.append(q * rng.uniform(0.3, 0.7))
-            offs.append(rng.uniform(-1.0, 1.0, size=3))
-        mats, offs = np.stack(mats), np.stack(offs)
-        choice = rng.integers(0, n_maps, size=iterations)
-        pts = np.empty((iterations, 3))
-        p = np.zeros(3)
-        for i in range(iterations):
-            p = mats[choice[i]] @ p + offs[choice[i]]
-            pts[i] = p
-        pts = pts[100:]
-        lo, hi = pts.min(0), pts.max(0)
-        scale = (np.array([d, h, w]) - 1) / np.maximum(hi - lo, 1e-9).max()
-        idx = np.clip(np.floor((pts - lo) * scale).astype(np.int64), 0, [d - 1, h - 1, w - 1])
-        labels[idx[:, 0], idx[:, 1], idx[:, 2]] = cls
+    g = int(grid_size)
+    labels = np.zeros((g, g, g), dtype=np.int64)
+    if systems is None:
+        systems = []
+        for _ in range(n_fractals):
+            cls = int(rng.integers(0, n_classes))
+            mats, offs = [], []
+            for _ in range(n_maps):
+                q, _r = np.linalg.qr(rng.standard_normal((3, 3)))
+                mats.append(q * rng.uniform(0.3, 0.7))
+                offs.append(rng.uniform(-1.0, 1.0, size=3))
+            systems.append((cls, np.stack(mats), np.stack(offs)))
+    for cls, mats, offs in systems:
+        choice = rng.integers(0, len(mats), size=iterations)
+        idx = points_to_voxel_indices(chaos_game(mats, offs, choice)[burn_in:], g)
+        labels[idx[:, 0], idx[:, 1], idx[:, 2]] = cls + 1
     lab = torch.from_numpy(labels)[None]
     occ = (lab > 0).to(torch.float32)[:, None]
     return occ, lab

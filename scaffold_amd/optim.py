@@ -94,6 +94,7 @@ class FusedClipAdam(torch.optim.Optimizer):
             st["step"] = torch.zeros((), dtype=torch.float32, device=p.device)
             st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
             st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+        self._check_state(p, st)
         return st
 
     def _plan(self, active, device):
@@ -210,5 +211,55 @@ class FusedClipAdam(torch.optim.Optimizer):
                 e.maintained = True
 
     def load_state_dict(self, state_dict):
+        """As ``torch.optim.Optimizer.load_state_dict``, then the state is brought into the form the kernels read.
+
+        torch leaves ``step`` wherever the checkpoint held it (a host tensor after the reference's restore path,
+        ``ScaFFold/utils/checkpointing.py:309-340``, and in every checkpoint of a non-fused ``torch.optim.Adam``) and keeps
+        the strides the moments were saved with. The kernels dereference ``step`` on the device and walk parameter,
+        gradient and both moments as one flat array, so here ``step`` becomes a 0-dim fp32 tensor on the parameter's
+        device and the moments are re-laid out to the parameter's own strides (values follow their logical index)."""
         super().load_state_dict(state_dict)
         self._plans = {}  # the state tensors were replaced
+        self._pack_plan = None
+        steps = set()
+        for group in self.param_groups:
+            for p in group["params"]:
+                st = self.state.get(p)
+                if not st:
+                    continue
+                missing = [k for k in ("step", "exp_avg", "exp_avg_sq") if k not in st]
+                if missing:
+                    raise NotImplementedError(f"FusedClipAdam: loaded state lacks {missing} (amsgrad / foreign optimizers are not served)")
+                step = st["step"]
+                step = step.detach() if torch.is_tensor(step) else torch.tensor(float(step))
+                steps.add(float(step))  # a load is not the hot loop: one host read per parameter
+                st["step"] = step.to(device=p.device, dtype=torch.float32).reshape(()).clone()
+                for k in ("exp_avg", "exp_avg_sq"):
+                    st[k] = self._like_param(p, st[k], k)
+        if len(steps) > 1:
+            raise NotImplementedError(f"FusedClipAdam: the kernels keep one step counter for all parameters, the loaded state has {sorted(steps)}")
+
+    @staticmethod
+    def _like_param(p, t, what):
+        """``t`` as an fp32 tensor on ``p``'s device with ``p``'s strides (no copy when it already is)."""
+        if not torch.is_tensor(t) or t.shape != p.shape:
+            raise ValueError(f"FusedClipAdam: loaded {what} has shape {tuple(getattr(t, 'shape', ()))}, the parameter {tuple(p.shape)}")
+        if t.device == p.device and t.dtype is torch.float32 and t.stride() == p.stride():
+            return t
+        out = torch.empty_like(p, dtype=torch.float32, memory_format=torch.preserve_format)
+        out.copy_(t)
+        return out
+
+    def _check_state(self, p, st):
+        """What the kernels assume about a parameter's state; raises rather than hand the device a host address or a
+        permuted moment."""
+        step = st["step"]
+        if not torch.is_tensor(step) or step.device != p.device or step.dtype is not torch.float32 or step.numel() != 1:
+            raise NotImplementedError(f"FusedClipAdam: step must be a one-element fp32 tensor on {p.device}, got "
+                                      f"{getattr(step, 'dtype', type(step))} on {getattr(step, 'device', 'the host')}; "
+                                      "load checkpoints through load_state_dict")
+        for k in ("exp_avg", "exp_avg_sq"):
+            t = st[k]
+            if t.device != p.device or t.dtype is not torch.float32 or t.shape != p.shape or t.stride() != p.stride():
+                raise NotImplementedError(f"FusedClipAdam: {k} must be fp32 on {p.device} with the parameter's strides {tuple(p.stride())}, "
+                                          f"got {t.dtype} on {t.device} with strides {tuple(t.stride())}")

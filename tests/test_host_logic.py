@@ -140,3 +140,61 @@ def test_lazy_package_exports():
     assert sa.triton_group_norm is sa.group_norm
     with pytest.raises(AttributeError):
         sa.no_such_symbol
+
+
+# ---- optimizer state as the kernels read it (host logic; the kernels themselves need the GPU) ------------------
+def _stock_adam_checkpoint(params, steps=2):
+    """A checkpoint as a non-fused torch.optim.Adam writes it: one host `step` tensor per parameter."""
+    opt = torch.optim.Adam(params, lr=1e-2, foreach=False, fused=False)
+    gen = torch.Generator().manual_seed(7)
+    for _ in range(steps):
+        for p in params:
+            p.grad = torch.randn(p.shape, generator=gen).contiguous(memory_format=torch.channels_last_3d if p.dim() == 5 else torch.contiguous_format)
+        opt.step()
+    return opt.state_dict()
+
+
+def test_loaded_optimizer_state_is_brought_to_the_parameters_device_dtype_and_strides():
+    from scaffold_amd.optim import FusedClipAdam
+    CL = torch.channels_last_3d
+    src = [torch.randn(4, 3, 2, 2, 2).requires_grad_(True), torch.randn(5).requires_grad_(True)]   # contiguous weight
+    sd = _stock_adam_checkpoint(src)
+    assert sd["state"][0]["step"].device.type == "cpu" and sd["state"][0]["exp_avg"].is_contiguous()
+    sd["state"][1]["step"] = sd["state"][1]["step"].double()          # a foreign dtype
+    mine = [src[0].detach().clone().contiguous(memory_format=CL).requires_grad_(True), src[1].detach().clone().requires_grad_(True)]
+    opt = FusedClipAdam(mine, lr=1e-2, max_norm=1.0)
+    opt.load_state_dict(sd)
+    for i, p in enumerate(mine):
+        st = opt.state[p]
+        assert st["step"].device == p.device and st["step"].dtype is torch.float32 and st["step"].shape == () and st["step"].item() == 2.0
+        for k in ("exp_avg", "exp_avg_sq"):
+            assert st[k].dtype is torch.float32 and st[k].device == p.device and st[k].stride() == p.stride()
+            assert torch.equal(st[k], sd["state"][i][k])              # same values at the same logical index
+        opt._check_state(p, st)                                       # what step() verifies before the first launch
+    # python-number steps (old checkpoints) are accepted too
+    sd2 = _stock_adam_checkpoint([torch.randn(5).requires_grad_(True)])
+    sd2["state"][0]["step"] = 2
+    o2 = FusedClipAdam([torch.zeros(5, requires_grad=True)])
+    o2.load_state_dict(sd2)
+    assert o2.state[o2.param_groups[0]["params"][0]]["step"].item() == 2.0
+
+
+def test_optimizer_state_the_kernels_cannot_read_raises_before_any_launch():
+    from scaffold_amd.optim import FusedClipAdam
+    a, b = torch.zeros(5, requires_grad=True), torch.zeros(3, requires_grad=True)
+    sd = _stock_adam_checkpoint([torch.randn(5).requires_grad_(True), torch.randn(3).requires_grad_(True)])
+    sd["state"][1]["step"] = sd["state"][1]["step"] + 1                # torch allows per-parameter counters; the kernels keep one
+    with pytest.raises(NotImplementedError, match="one step counter"):
+        FusedClipAdam([a, b]).load_state_dict(sd)
+    sd = _stock_adam_checkpoint([torch.randn(5).requires_grad_(True), torch.randn(3).requires_grad_(True)])
+    del sd["state"][0]["exp_avg_sq"]
+    with pytest.raises(NotImplementedError, match="lacks"):
+        FusedClipAdam([a, b]).load_state_dict(sd)
+    # state put there behind load_state_dict's back: a step counter on another device, a moment with other strides
+    opt = FusedClipAdam([a])
+    good = {"step": torch.zeros(()), "exp_avg": torch.zeros(5), "exp_avg_sq": torch.zeros(5)}
+    opt._check_state(a, good)
+    for key, bad in (("step", torch.zeros((), device="meta")), ("step", torch.zeros((), dtype=torch.float64)), ("step", 3.0),
+                     ("exp_avg", torch.zeros(10)[::2]), ("exp_avg_sq", torch.zeros(5, dtype=torch.bfloat16))):
+        with pytest.raises(NotImplementedError):
+            opt._check_state(a, {**good, key: bad})

@@ -315,3 +315,65 @@ def test_a_parameter_written_by_someone_else_is_not_read_through_a_stale_copy(de
         assert torch.equal(y_after, ref(x))
     opt.refresh_shadows()
     assert compute_copy(conv.weight, torch.bfloat16) is not None
+
+
+def _to_host(obj):
+    """The reference's restore path: every tensor of the optimizer state dict moved to the host before it is loaded
+    back (`ScaFFold/utils/checkpointing.py:309-340`)."""
+    if torch.is_tensor(obj):
+        return obj.detach().cpu()
+    if isinstance(obj, dict):
+        return {k: _to_host(v) for k, v in obj.items()}
+    if isinstance(obj, (list, tuple)):
+        return type(obj)(_to_host(v) for v in obj)
+    return obj
+
+
+def _assign_grads(params, values):
+    """The same logical gradient values for every arm, each in its parameter's own memory layout."""
+    for p, v in zip(params, values):
+        fmt = CL if p.dim() == 5 and not p.is_contiguous() else torch.contiguous_format
+        p.grad = v.to(p.device).contiguous(memory_format=fmt)
+
+
+@pytest.mark.parametrize("source", ["stock_adam", "ours_through_the_host"])
+def test_resume_from_a_checkpoint_whose_step_counters_live_on_the_host(device, source):
+    """A checkpoint of a non-fused torch.optim.Adam (host `step`, contiguous moments for a weight we keep channels-last) or
+    our own state dict after a round trip through host memory: the resumed run must continue like stock clip + Adam."""
+    sizes = [(8, 4, 3, 3, 3), (33,), (8193,)]
+    gen = torch.Generator().manual_seed(5)
+    a = _make(device, sizes, channels_last=source != "stock_adam")   # the stock run keeps its 5-d weight contiguous
+    stock = [p.detach().clone().requires_grad_(True) for p in a]
+    opt_a = torch.optim.Adam(a, lr=1e-2, foreach=False, fused=False) if source == "stock_adam" else sa.FusedClipAdam(a, lr=1e-2, max_norm=1.0)
+    opt_s = torch.optim.Adam(stock, lr=1e-2, foreach=False, fused=False)
+    for _ in range(3):
+        values = [torch.randn(s, generator=gen) for s in sizes]
+        _assign_grads(stock, values)
+        _assign_grads(a, values)
+        torch.nn.utils.clip_grad_norm_(stock, 1.0)
+        opt_s.step()
+        if source == "stock_adam":
+            torch.nn.utils.clip_grad_norm_(a, 1.0)
+        opt_a.step()
+    sd = _to_host(copy.deepcopy(opt_a.state_dict()))
+    assert sd["state"][0]["step"].device.type == "cpu"
+    # resume into our optimizer with the 5-d weight channels-last
+    mine = [p.detach().clone().contiguous(memory_format=CL).requires_grad_(True) if p.dim() == 5 else p.detach().clone().requires_grad_(True)
+            for p in a]
+    opt_m = sa.FusedClipAdam(mine, lr=1e-2, max_norm=1.0)
+    opt_m.load_state_dict(sd)
+    for p in mine:
+        st = opt_m.state[p]
+        assert st["step"].is_cuda and st["step"].dtype is torch.float32 and st["exp_avg"].stride() == p.stride()
+    for _ in range(2):
+        values = [torch.randn(s, generator=gen) for s in sizes]
+        _assign_grads(stock, values)
+        _assign_grads(mine, values)
+        torch.nn.utils.clip_grad_norm_(stock, 1.0)
+        opt_s.step()
+        opt_m.step()
+    for p, q in zip(mine, stock):
+        assert torch.allclose(p, q, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(opt_m.state[p]["exp_avg"], opt_s.state[q]["exp_avg"], rtol=1e-5, atol=1e-7)
+        assert torch.allclose(opt_m.state[p]["exp_avg_sq"], opt_s.state[q]["exp_avg_sq"], rtol=1e-5, atol=1e-9)
+        assert opt_m.state[p]["step"].item() == 5.0

@@ -235,11 +235,108 @@ def test_train_step_loss_closed_form():
     assert math.isclose(orc.train_step_loss(logits, labels, 2).item(), want, rel_tol=1e-6)
 
 
-def test_ifs_volume_is_seeded_and_labelled():
-    occ, lab = orc.ifs_volume((16, 16, 16), iterations=4000, seed=1)
-    occ2, lab2 = orc.ifs_volume((16, 16, 16), iterations=4000, seed=1)
-    assert torch.equal(lab, lab2) and occ.shape == (1, 1, 16, 16, 16) and lab.shape == (1, 16, 16, 16)
-    assert 0 < occ.mean() < 0.5 and lab.max() <= 10 and torch.equal(occ[0, 0] > 0, lab[0] > 0)
+def test_chaos_game_by_hand_and_fixed_point():
+    # x -> x/2 and x -> x/2 + 1/2 on the first axis, choices (., 1, 0, 1): 0 -> 1/2 -> 1/4 -> 5/8
+    half = np.diag([0.5, 0.0, 0.0])
+    pts = orc.chaos_game([half, half], [[0, 0, 0], [0.5, 0, 0]], [0, 1, 0, 1])
+    assert np.array_equal(pts, [[0, 0, 0], [0.5, 0, 0], [0.25, 0, 0], [0.625, 0, 0]])
+    # one non-symmetric contraction: the orbit converges to (I - M)^-1 o; applying the transposed map would not
+    m = np.array([[0.3, 0.2, 0.0], [-0.1, 0.4, 0.1], [0.25, 0.0, -0.35]])
+    o = np.array([0.5, -1.0, 2.0])
+    pts = orc.chaos_game([m], [o], np.zeros(200, dtype=int))
+    want = np.linalg.solve(np.eye(3) - m, o)
+    assert np.allclose(pts[-1], want, rtol=0, atol=1e-13) and not np.allclose(want, np.linalg.solve(np.eye(3) - m.T, o), atol=1e-3)
+
+
+def test_voxelisation_rule_by_hand():
+    """grid 4, extents (1, 0.25, 0): voxel size (1 + 1e-6) / 4 for ALL axes; scaled spans (3.999996, 0.999999, 0) are centred
+    with offsets (2e-6, 1.5000005, 2); then floor."""
+    idx = orc.points_to_voxel_indices([[0, 0, 0], [1, 0, 0], [0.6, 0.25, 0], [0.6, 0.25, 0]], 4)
+    assert idx.tolist() == [[0, 1, 2], [2, 2, 2], [3, 1, 2]]
+    # a shifted and uniformly scaled cloud occupies the same voxels
+    idx2 = orc.points_to_voxel_indices(np.array([[0, 0, 0], [1, 0, 0], [0.6, 0.25, 0]]) * 7.0 + [3.0, -2.0, 11.0], 4)
+    assert idx2.tolist() == idx.tolist()
+    with pytest.raises(ValueError):
+        orc.points_to_voxel_indices([[0, 0, 0], [np.nan, 0, 0]], 4)
+
+
+def test_ifs_volume_closed_forms():
+    # one contraction map: every point past the burn-in is its fixed point -> one voxel, the centre of the grid
+    m = np.array([[0.3, 0.2, 0.0], [-0.1, 0.4, 0.1], [0.25, 0.0, -0.35]])
+    occ, lab = orc.ifs_volume(8, systems=[(6, [m], [[0.5, -1.0, 2.0]])], iterations=400, seed=1)
+    assert occ.shape == (1, 1, 8, 8, 8) and lab.shape == (1, 8, 8, 8) and lab.dtype == torch.int64
+    assert int(occ.sum()) == 1 and lab[0, 4, 4, 4] == 7 and torch.equal(occ[0, 0] > 0, lab[0] > 0)
+    # x/2, x/2 + 1/2: the attractor is the unit segment of the first axis -> the whole centre line, nothing else
+    half = np.diag([0.5, 0.0, 0.0])
+    occ, lab = orc.ifs_volume(8, systems=[(0, [half, half], [[0, 0, 0], [0.5, 0, 0]])], iterations=4000, seed=2)
+    want = torch.zeros(8, 8, 8, dtype=torch.int64)
+    want[:, 4, 4] = 1
+    assert torch.equal(lab[0], want)
+    # Cantor dust of ratio 1/5 (8 maps p/5 + 4c/5, c a cube corner): coordinates lie in [0,.04] [.16,.2] [.8,.84] [.96,1], i.e.
+    # voxels {0, 1, 6, 7} of 8 per axis with margins of a quarter voxel; a second system painted later overwrites the first
+    corners = np.array([[i, j, k] for i in (0, 1) for j in (0, 1) for k in (0, 1)], dtype=float)
+    dust = (3, [np.eye(3) / 5] * 8, corners * 0.8)
+    occ, lab = orc.ifs_volume(8, systems=[dust, (8, [m], [[0.5, -1.0, 2.0]])], iterations=20000, seed=3)
+    want = torch.zeros(8, 8, 8, dtype=torch.int64)
+    on = torch.tensor([0, 1, 6, 7])
+    want[on[:, None, None], on[None, :, None], on[None, None, :]] = 4
+    want[4, 4, 4] = 9
+    assert torch.equal(lab[0], want)
+    occ, lab = orc.ifs_volume(8, systems=[(8, [m], [[4.0, 4.0, 4.0]]), (3, [np.eye(3) / 5] * 8, corners * 0.8 + 7.0)], iterations=20000, seed=3)
+    assert lab[0, 4, 4, 4] == 9 and int((lab == 4).sum()) == 64      # the dust does not reach the centre voxel
+
+
+def test_ifs_volume_random_systems_are_seeded_and_labelled():
+    occ, lab = orc.ifs_volume(16, iterations=4000, seed=1)
+    occ2, lab2 = orc.ifs_volume(16, iterations=4000, seed=1)
+    assert torch.equal(lab, lab2) and not torch.equal(lab, orc.ifs_volume(16, iterations=4000, seed=2)[1])
+    assert 0 < occ.mean() < 0.5 and 1 <= lab.max() <= 10 and torch.equal(occ[0, 0] > 0, lab[0] > 0)
+
+
+# ---- the tolerance gates themselves ---------------------------------------------------------------------------
+def test_parity_gate_fp32_is_1e5_of_the_rms():
+    e = torch.tensor([3.0, -4.0, 0.0, 0.0], dtype=torch.float64)           # rms 2.5
+    inside = e.clone(); inside[2] += 0.9e-5 * 2.5
+    outside = e.clone(); outside[2] -= 2e-5 * 2.5
+    rep = orc.assert_baseline_tolerance(inside, e, torch.float32)
+    assert math.isclose(rep.max_rel, 0.9e-5, rel_tol=1e-9)
+    with pytest.raises(AssertionError):
+        orc.assert_baseline_tolerance(outside, e, torch.float32)
+    barely = e.clone(); barely[0] += 1.01e-5 * 2.5
+    with pytest.raises(AssertionError):
+        orc.assert_baseline_tolerance(barely, e, torch.float32)
+    with pytest.raises(AssertionError):
+        orc.assert_baseline_tolerance(torch.tensor([3.0, float("nan"), 0.0, 0.0], dtype=torch.float64), e, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_parity_gate_16bit_is_elementwise_2e2_relative_plus_1e2_absolute(dtype):
+    e = torch.tensor([2.0, -10.0, 0.0, 100.0], dtype=torch.float64)        # limits 0.05, 0.21, 0.01, 2.01
+    limit = torch.tensor([0.05, 0.21, 0.01, 2.01], dtype=torch.float64)
+    sign = torch.tensor([1.0, -1.0, -1.0, 1.0], dtype=torch.float64)
+    orc.assert_baseline_tolerance(e + sign * limit * 0.999, e, dtype)      # every element just inside
+    for k in range(4):                                                     # ONE element just outside must fail
+        a = e + sign * limit * 0.999
+        a[k] = e[k] + sign[k] * limit[k] * 1.001
+        with pytest.raises(AssertionError):
+            orc.assert_baseline_tolerance(a, e, dtype)
+    # the bar is per element, not relative to the tensor's scale: 0.02 off at an exact zero fails beside a value of 100
+    with pytest.raises(AssertionError):
+        orc.assert_baseline_tolerance(torch.tensor([2.0, -10.0, 0.02, 100.0], dtype=torch.float64), e, dtype)
+    with pytest.raises(AssertionError):
+        orc.assert_baseline_tolerance(torch.tensor([2.0, float("nan"), 0.0, 100.0], dtype=torch.float64), e, dtype)
+    with pytest.raises(ValueError):
+        orc.assert_baseline_tolerance(e[:3], e, dtype)
+
+
+def test_groupnorm_error_measure_by_hand():
+    e = torch.tensor([1.0, -4.0, 2.0])
+    assert orc.gn_rel_error(torch.tensor([1.5, -4.0, 2.0]), e) == 0.125          # 0.5 / max|e| = 0.5 / 4
+    assert orc.gn_rel_error(torch.tensor([1.0, -4.0, 1.0]), e) == 0.25
+    assert orc.gn_rel_error(e, e) == 0.0
+    poisoned = orc.gn_rel_error(torch.tensor([1.0, float("nan"), 2.0]), e)
+    assert math.isnan(poisoned) and not poisoned <= 1.0                          # a NaN fails every `<= tol` check
+    assert orc.GN_TOLERANCE == {torch.float32: 1e-4, torch.bfloat16: 2e-2, torch.float16: 3e-3}
 
 
 def test_train_step_loss_weighted_ce_closed_form():
