@@ -96,7 +96,7 @@ class _Problem:
     """Everything about one convolution problem that does not depend on the tensors: parsed geometry, the descriptor
     the library takes, and (filled on first use) the workspace bytes of each direction."""
 
-    __slots__ = ("s", "p", "d", "k", "n", "cin", "in_sp", "cout", "y_shape", "desc", "code", "need")
+    __slots__ = ("s", "p", "d", "k", "n", "cin", "in_sp", "cout", "y_shape", "desc", "code", "need", "packed")
 
     def __init__(self, in_shape, w_shape, stride, padding, dilation, dtype):
         self.s, self.p, self.d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
@@ -108,6 +108,32 @@ class _Problem:
         self.desc = _desc(self.n, self.cin, self.in_sp, self.cout, self.k, self.s, self.p, self.d)
         self.code = _lib.dtype_code(dtype)
         self.need = {}
+        self.packed = None
+
+    def packed_bytes(self, backward_data: bool) -> int:
+        """Bytes of the packed weight this direction of the problem reads (0: it reads the weight where it lies)."""
+        if self.packed is None:
+            L = _lib.lib()
+            self.packed = (int(L.sfh_conv3d_packed_weight_bytes(ctypes.byref(self.desc), self.code, 0)),
+                           int(L.sfh_conv3d_packed_weight_bytes(ctypes.byref(self.desc), self.code, 1)))
+        return self.packed[1 if backward_data else 0]
+
+    def check_packed(self, packed, backward_data: bool, like: torch.Tensor) -> int:
+        """A caller's ``packed_weight=`` is validated, not trusted: the MFMA kernels index it by fragment, so a pack made for
+        another shape, direction or dtype would be read out of bounds.  Returns its size in bytes."""
+        want = self.packed_bytes(backward_data)
+        what = "data-gradient" if backward_data else "forward"
+        if want == 0:
+            raise ValueError(f"packed_weight=: the {what} direction of this problem does not read a packed weight")
+        if not isinstance(packed, torch.Tensor) or packed.dtype is not torch.uint8 or packed.dim() != 1 or not packed.is_contiguous():
+            raise ValueError(f"packed_weight= must be the contiguous uint8 buffer pack_weights() returned, got "
+                             f"{getattr(packed, 'dtype', type(packed))} of shape {tuple(getattr(packed, 'shape', ()))}")
+        if packed.device != like.device:
+            raise ValueError(f"packed_weight= is on {packed.device}, the operands on {like.device}")
+        if packed.numel() != want:
+            raise ValueError(f"packed_weight= holds {packed.numel()} bytes, the {what} form of this problem has {want}: "
+                             "it was packed for another shape, direction or dtype")
+        return want
 
     def workspace_bytes(self, direction: str) -> int:
         need = self.need.get(direction)
@@ -556,7 +582,7 @@ def conv3d_forward(
             # ``packed_weight`` comes from pack_weights() for this very problem: the library reads it in place of w
             if weight_rsck is not None or weight_flip or force_generic:
                 raise ValueError("packed_weight= cannot be combined with weight_rsck=, weight_flip= or force_generic=")
-            need -= packed_weight.numel()
+            need -= prob.check_packed(packed_weight, False, x)
             flags |= _lib.SFH_FLAG_WEIGHT_PACKED
             w_eff = packed_weight
         ws = _lib.workspace(need, x.device)
@@ -621,7 +647,7 @@ def conv3d_backward_data(
         if packed_weight is not None:
             if weight_rsck is not None or force_generic:
                 raise ValueError("packed_weight= cannot be combined with weight_rsck= or force_generic=")
-            need -= packed_weight.numel()
+            need -= prob.check_packed(packed_weight, True, gy)
             flags |= _lib.SFH_FLAG_WEIGHT_PACKED
             w_eff = packed_weight
         ws = _lib.workspace(need, gy.device)

@@ -2,7 +2,6 @@
 // function of descriptor and dtype), workspace carving. No allocation, no synchronisation.
 #include <string.h>
 
-#include <vector>
 #include "common.hpp"
 #include "concat.hpp"
 #include "ingest.hpp"
@@ -376,42 +375,60 @@ extern "C" size_t sfh_conv3d_packed_weight_bytes(const sfh_conv3d_desc* p, int d
   return spec.any ? mfma_conv_packed_weight_bytes(spec.a) : 0;
 }
 
-static int collect_pack_jobs(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t w_stride[5], void* packed_fwd,
-                             void* packed_dgrad, std::vector<MfmaPackItem>& jobs) {
+// Appends the packings one weight asks for (its forward form and / or its data-gradient form) to jobs[njobs...]; the
+// caller leaves room for two.
+static int collect_pack_jobs(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t* w_stride, void* packed_fwd,
+                             void* packed_dgrad, MfmaPackItem* jobs, int* njobs) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (w == nullptr || w_stride == nullptr) return fail(SFH_ERR_INVALID, "conv3d pack: null weight");
   if (packed_fwd != nullptr) {
     const PackSpec spec = fwd_pack_spec(*p, dtype, out, w_stride);
     if (!spec.any) return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the forward of this problem does not read a packed weight");
-    jobs.push_back(MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_fwd});
+    jobs[(*njobs)++] = MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_fwd};
   }
   if (packed_dgrad != nullptr) {
     const PackSpec spec = dgrad_pack_spec(*p, dtype, out, w_stride);
     if (!spec.any) return fail(SFH_ERR_UNSUPPORTED, "conv3d pack: the data gradient of this problem does not read a packed weight");
-    jobs.push_back(MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_dgrad});
+    jobs[(*njobs)++] = MfmaPackItem{spec.a, w, spec.s_out, spec.s_red, w_stride[2], w_stride[3], w_stride[4], spec.flip, packed_dgrad};
   }
   return SFH_OK;
 }
 
 extern "C" int sfh_conv3d_pack_weights(const sfh_conv3d_desc* p, int dtype, const void* w, const int64_t w_stride[5], void* packed_fwd,
                                        void* packed_dgrad, void* stream) {
-  std::vector<MfmaPackItem> jobs;
-  if (int rc = collect_pack_jobs(p, dtype, w, w_stride, packed_fwd, packed_dgrad, jobs)) return rc;
-  if (jobs.empty()) return SFH_OK;
-  return mfma_pack_weight_batch(jobs.data(), (int)jobs.size(), dtype, (hipStream_t)stream);
+  MfmaPackItem jobs[2];
+  int njobs = 0;
+  if (int rc = collect_pack_jobs(p, dtype, w, w_stride, packed_fwd, packed_dgrad, jobs, &njobs)) return rc;
+  if (njobs == 0) return SFH_OK;
+  return mfma_pack_weight_batch(jobs, njobs, dtype, (hipStream_t)stream);
 }
 
 extern "C" int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t nitems, int dtype, void* stream) {
   if (nitems < 0 || (nitems > 0 && items == nullptr)) return fail(SFH_ERR_INVALID, "conv3d pack batch: bad item list");
-  std::vector<MfmaPackItem> jobs;
-  jobs.reserve((size_t)nitems * 2);
-  for (int i = 0; i < nitems; ++i)
-    if (int rc = collect_pack_jobs(&items[i].desc, dtype, items[i].w, items[i].w_stride, items[i].packed_fwd, items[i].packed_dgrad,
-                                   jobs))
-      return rc;
-  if (jobs.empty()) return SFH_OK;
-  return mfma_pack_weight_batch(jobs.data(), (int)jobs.size(), dtype, (hipStream_t)stream);
+  // Every item is validated before the first launch (a bad item must leave nothing half done), then the jobs go out in
+  // groups of a fixed-size array on the stack: nothing on this path touches the heap.
+  {
+    MfmaPackItem probe[2];
+    for (int i = 0; i < nitems; ++i) {
+      int n = 0;
+      if (int rc = collect_pack_jobs(&items[i].desc, dtype, items[i].w, items[i].w_stride, items[i].packed_fwd, items[i].packed_dgrad,
+                                     probe, &n))
+        return rc;
+    }
+  }
+  constexpr int kGroup = 32;
+  MfmaPackItem jobs[kGroup + 2];
+  int njobs = 0;
+  for (int i = 0; i < nitems; ++i) {
+    collect_pack_jobs(&items[i].desc, dtype, items[i].w, items[i].w_stride, items[i].packed_fwd, items[i].packed_dgrad, jobs, &njobs);
+    if (njobs >= kGroup || i + 1 == nitems) {
+      if (njobs > 0)
+        if (int rc = mfma_pack_weight_batch(jobs, njobs, dtype, (hipStream_t)stream)) return rc;
+      njobs = 0;
+    }
+  }
+  return SFH_OK;
 }
 
 // ---- data gradient ---------------------------------------------------------------------

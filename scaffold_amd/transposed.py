@@ -21,6 +21,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
+from . import conv3d as _c3
 from ._lib import ConvTDesc, SUPPORTED_DTYPES
 from .conv3d import (
     _CL3D,
@@ -199,6 +200,8 @@ def conv_transpose3d_forward(
         if packed_weight is not None:
             if force_generic:
                 raise ValueError("packed_weight= cannot be combined with force_generic=")
+            # the up-convolution is the data gradient of the stride-k convolution of its OUTPUT: that problem's form
+            _c3._problem(torch.Size(y_shape), torch.Size((cin, cout, *k)), k, 0, 1, x.dtype).check_packed(packed_weight, True, x)
             rc = L.sfh_convT3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(packed_weight), None, _lib.ptr(bias),
                                    _lib.ptr(y), None, 0, _lib.SFH_FLAG_WEIGHT_PACKED, _lib.stream_ptr(x.device))
         else:

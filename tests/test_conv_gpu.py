@@ -10,6 +10,7 @@ Standards, as in the reference's kernel suite (``triton_conv3d/reference.py:4-18
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 import scaffold_amd as sa
 from oracle import oracle as orc
@@ -395,12 +396,28 @@ def test_full_size_128cube_properties(device):
     assert torch.equal(y, y_d)
     assert torch.equal(gx, gx_d)
 
+    # The weight gradient the same way: every product is in {-1, 0, 1} and a sum over the 2M voxels stays far below 2^24,
+    # so fp32 accumulation is exact in ANY order -- the split-K MFMA kernel + ordered slice sum and the untiled kernel
+    # (a workgroup per (output channel, tap), LDS tree) must round the same integer and agree in all 27,648 elements.
+    gw_d = sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, force_generic=True)
+    assert torch.equal(gw, gw_d)
+    # ... and the unrounded fp32 form (what an fp32 master weight receives) is that integer itself
+    gw32 = sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, grad_dtype=torch.float32)
+    assert gw32.dtype is torch.float32 and torch.equal(gw32, gw32.round()) and torch.equal(gw32.to(torch.bfloat16), gw)
+    # a sub-volume against the fp64 oracle: the gradient of the first 8 x 16 x 128 output rows alone (gy zero elsewhere)
+    gy_sub = torch.zeros_like(gy)
+    gy_sub[:, :, :8, :16, :] = gy[:, :, :8, :16, :]
+    gw_sub = sa.conv3d_backward_weight(x, w.shape, gy_sub, 1, 1, grad_dtype=torch.float32)
+    sub = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(10, 18, 128), padding=(0, 0, 1), dtype=torch.bfloat16)
+    xs = F.pad(x[:, :, :9, :17, :].cpu().float(), (0, 0, 1, 0, 1, 0)).contiguous(memory_format=cl)   # the volume's zero padding at d = h = -1
+    ref = orc.conv_reference(sub, {"input": xs, "weight": w.cpu(), "bias": None,
+                                   "grad_output": gy[:, :, :8, :16, :].cpu().contiguous(memory_format=cl)}, "bwd-weight")
+    assert torch.equal(gw_sub.cpu().double(), ref)
+
     lhs = (y.double() * gy.double()).sum().item()
     mid = (x.double() * gx.double()).sum().item()
-    assert lhs == mid
-    if gw.abs().max() < 256:
-        rhs = (w.double() * gw.double()).sum().item()
-        assert lhs == rhs
+    rhs = (w.double() * gw32.double()).sum().item()
+    assert lhs == mid == rhs
 
     corner = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(10, 10, 40), dtype=torch.bfloat16)
     xc = x[:, :, :10, :10, :40].cpu().contiguous(memory_format=cl)

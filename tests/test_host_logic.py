@@ -198,3 +198,22 @@ def test_optimizer_state_the_kernels_cannot_read_raises_before_any_launch():
                      ("exp_avg", torch.zeros(10)[::2]), ("exp_avg_sq", torch.zeros(5, dtype=torch.bfloat16))):
         with pytest.raises(NotImplementedError):
             opt._check_state(a, {**good, key: bad})
+
+
+def test_a_callers_packed_weight_is_validated_not_trusted(monkeypatch):
+    """`packed_weight=` must be the uint8 buffer of exactly this problem's and direction's packed size, on the operands'
+    device: anything else raises before the library is called (the MFMA kernels would index it out of bounds)."""
+    prob = c3._Problem((1, 32, 8, 8, 8), (64, 32, 3, 3, 3), 1, 1, 1, torch.bfloat16)
+    prob.packed = (4096, 8192)                     # what the library would report (forward, data gradient)
+    like = torch.empty(1)
+    assert prob.check_packed(torch.empty(4096, dtype=torch.uint8), False, like) == 4096
+    assert prob.check_packed(torch.empty(8192, dtype=torch.uint8), True, like) == 8192
+    for bad in (torch.empty(8192, dtype=torch.uint8),             # the other direction's form
+                torch.empty(4095, dtype=torch.uint8), torch.empty(2048, dtype=torch.bfloat16),
+                torch.empty(8192, dtype=torch.uint8)[::2], torch.empty(64, 64, dtype=torch.uint8),
+                torch.empty(4096, dtype=torch.uint8, device="meta"), None, 4096):
+        with pytest.raises(ValueError):
+            prob.check_packed(bad, False, like)
+    prob.packed = (0, 0)                            # a problem whose kernels read the weight where it lies
+    with pytest.raises(ValueError, match="does not read a packed weight"):
+        prob.check_packed(torch.empty(0, dtype=torch.uint8), False, like)

@@ -185,6 +185,74 @@ def test_unet_bf16_autocast_train_step_matches_stock(device):
     assert (torch.dot(u0, u1) / (u0.norm() * u1.norm())).item() > 0.9
 
 
+# ---- config 5's architecture: 5 levels, base width 32 doubling to 512, 11 classes, depth-shard form ------------------
+def _cfg5_arms(device, grid, iterations):
+    """Stock-module arm on the host and ours on the GPU in shard form (zero depth halo, padding (0, 1, 1)), the same seeded
+    weights; input = the first half along depth of an IFS sample (occupancy in, class ids 0..10 as labels)."""
+    torch.manual_seed(5001)
+    stock = UNet(1, 11, layers=4, base_width=32, stock=True)
+    ours = UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
+    ours.load_state_dict(stock.state_dict())
+    occ, lab = orc.ifs_volume(grid, iterations=iterations, seed=5000)
+    x, lab = occ[:, :, : grid // 2].contiguous(), lab[:, : grid // 2].contiguous()
+    assert 0.01 < x.mean() < 0.5 and lab.unique().numel() >= 3
+    return stock, ours, x, lab
+
+
+def test_cfg5_architecture_fp32_gradients_match_stock_per_parameter(device):
+    """The reference's fp32 arm (`tests/test_groupnorm.py:1174-1228`: worst per-parameter relative L2 < 1e-4) on the
+    5-level / 11-class network: every kernel family of the step chained at widths 32..512, fp64 stock modules as truth,
+    the fused loss head against the loss recipe."""
+    stock, ours, x, lab = _cfg5_arms(device, 32, 20000)
+    assert sum(isinstance(m, FastConv3d) for m in ours.modules()) == 19 and sum(isinstance(m, FastGroupNorm) for m in ours.modules()) == 18
+    stock = stock.double()
+    l0 = orc.train_step_loss(stock(x.double()), lab, 11, dtype=torch.float64)
+    l0.backward()
+    l1 = sa.ce_dice_loss(ours(x.to(device).contiguous(memory_format=CL)), lab.to(device))
+    l1.backward()
+    assert abs(l0.item() - l1.item()) <= 1e-5 * abs(l0.item())
+    for (k, p0), (_, p1) in zip(stock.named_parameters(), ours.named_parameters()):
+        rel = (p1.grad.cpu().double() - p0.grad).norm() / p0.grad.norm().clamp_min(1e-30)
+        assert rel < 1e-4, (k, rel.item())
+
+
+@pytest.mark.parametrize("grid,iterations", [(32, 20000), (64, 60000)])
+def test_cfg5_architecture_bf16_train_step_matches_stock(device, grid, iterations):
+    """The reference's bf16 arm (aggregate relative L2 of the concatenated gradient < 5e-2) plus the loss within 2e-2 and the
+    clipped Adam step, for the step exactly as the bench runs it: bf16 autocast over fp32 master weights, every convolution
+    reading a depth slab, fused CE + Dice, `FusedClipAdam` with bf16 shadow weights.  Truth is the stock-module arm in
+    fp32 on the host (no autocast), with `clip_grad_norm_(1.0)` + `torch.optim.Adam` (`ScaFFold/utils/trainer.py:640-694`)."""
+    stock, ours, x, lab = _cfg5_arms(device, grid, iterations)
+    opt0 = torch.optim.Adam(stock.parameters(), lr=1e-3)
+    opt1 = sa.FusedClipAdam(ours.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+    l0 = orc.train_step_loss(stock(x), lab, 11)
+    l0.backward()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        logits = ours(x.to(device).contiguous(memory_format=CL))
+    assert logits.dtype is torch.bfloat16 and logits.shape == (1, 11, grid // 2, grid, grid)
+    l1 = sa.ce_dice_loss(logits, lab.to(device))
+    l1.backward()
+    assert abs(l0.item() - l1.item()) <= 2e-2 * abs(l0.item()), (l0.item(), l1.item())
+    assert all(p.grad.dtype is torch.float32 for p in ours.parameters())
+    g0 = torch.cat([p.grad.flatten().double() for p in stock.parameters()])
+    g1 = torch.cat([p.grad.flatten().cpu().double() for p in ours.parameters()])
+    assert ((g1 - g0).norm() / g0.norm()).item() < 5e-2
+    init = torch.cat([p.detach().flatten().double() for p in stock.parameters()])
+    want_norm = torch.nn.utils.clip_grad_norm_(stock.parameters(), 1.0)
+    opt0.step()
+    opt1.step()
+    assert abs(opt1.grad_norm.item() - want_norm.item()) <= 5e-2 * want_norm.item()
+    u0 = torch.cat([p.detach().flatten().double() for p in stock.parameters()]) - init
+    u1 = torch.cat([p.detach().flatten().cpu().double() for p in ours.parameters()]) - init
+    # Adam's first update is lr * sign(g) (amplifying the sign of gradients that are noise in bf16): bounded are the step
+    # size and the agreement of the two update directions
+    assert u0.abs().max() <= 1.001e-3 and u1.abs().max() <= 1.001e-3
+    assert (torch.dot(u0, u1) / (u0.norm() * u1.norm())).item() > 0.9
+    # the bf16 copies the next step's convolutions read are the rounded new weights
+    for p in ours.parameters():
+        assert torch.equal(opt1.shadow[p], p.detach().to(torch.bfloat16))
+
+
 def test_shard_halo_form_is_bitwise_the_padded_form(device):
     """Zero depth halo + depth padding 0 (what a single DistConv shard computes) equals padding 1."""
     _, ours, x, _ = _two_arms(device, torch.bfloat16)
