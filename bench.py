@@ -346,6 +346,59 @@ def bench_unet_step(args, device, eager_only=False):
     return out
 
 
+#: every 3x3x3 convolution of the config-5 step (base width 32, 5 levels) on the 64 x 128 x 128 depth shard, as
+#: (Cin, Cout, interior extents); each runs on the (D + 2) x H x W slab at padding (0, 1, 1)
+CFG5_CONVS = [
+    (32, 32, (64, 128, 128)), (64, 32, (64, 128, 128)),
+    (32, 64, (32, 64, 64)), (64, 64, (32, 64, 64)), (128, 64, (32, 64, 64)),
+    (64, 128, (16, 32, 32)), (128, 128, (16, 32, 32)), (256, 128, (16, 32, 32)),
+    (128, 256, (8, 16, 16)), (256, 256, (8, 16, 16)), (512, 256, (8, 16, 16)),
+    (256, 512, (4, 8, 8)), (512, 512, (4, 8, 8)),
+]
+#: config 3 / config 4 shapes on full cubes at padding 1
+CUBE_CONVS = [(32, 32, (128, 128, 128)), (32, 64, (64, 64, 64)), (64, 64, (64, 64, 64)), (128, 64, (64, 64, 64))]
+
+
+def conv_table(device, iters=20):
+    """Per-shape table of the MFMA convolution launches: every direction of every shape in a loop of its own
+    (weights packed beforehand, outputs and workspaces allocated once), time per launch from HIP events, algorithmic
+    FLOPs 2 * voxels * Cin * Cout * 27 and the fraction of the dense bf16 MFMA peak."""
+    import scaffold_amd as sa
+
+    rows = []
+    for form, shapes in (("slab pad (0,1,1)", CFG5_CONVS), ("cube pad 1", CUBE_CONVS)):
+        for cin, cout, sp in shapes:
+            slab = form.startswith("slab")
+            in_sp = (sp[0] + 2, sp[1], sp[2]) if slab else sp
+            pad = (0, 1, 1) if slab else (1, 1, 1)
+            g = torch.Generator().manual_seed(3000 + cin + cout)
+            x = torch.randn((1, cin, *in_sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            w = ((torch.rand((cout, cin, 3, 3, 3), generator=g) * 2 - 1) / math.sqrt(cin * 27)).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            gy = torch.randn((1, cout, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            flops = 2 * math.prod(sp) * cin * cout * 27
+            pf, pd = sa.pack_weights(w, x.shape, 1, pad, 1)
+            y, gx = torch.empty_like(gy), torch.empty_like(x)
+            gw = torch.empty((cout, cin, 3, 3, 3), dtype=torch.float32, device=device).contiguous(memory_format=CL)
+            fns = {
+                "fwd": lambda: sa.conv3d_forward(x, w, None, 1, pad, 1, out=y, packed_weight=pf),
+                "dgrad": lambda: sa.conv3d_backward_data(gy, w, x.shape, 1, pad, 1, out=gx, packed_weight=pd),
+                "wgrad": lambda: sa.conv3d_backward_weight(x, w.shape, gy, 1, pad, 1, out=gw, grad_dtype=torch.float32),
+            }
+            for direction, fn in fns.items():
+                fn()
+                torch.cuda.synchronize()
+                chunk = 10
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(chunk):
+                        fn()
+                ms = event_time_ms(graph.replay, max(2, iters // chunk), warmup=1) / chunk
+                rows.append({"form": form, "cin": cin, "cout": cout, "spatial": list(sp), "direction": direction, "us": ms * 1e3,
+                             "gflop": flops / 1e9, "tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS})
+            del x, w, gy, y, gx, gw, pf, pd
+    return rows
+
+
 def cpu_baseline():
     """The reference's CPU path (torch conv3d + autograd, channels_last_3d bf16) on the bench workload itself,
     repeated for about 12 s of host time."""
@@ -392,6 +445,8 @@ def main():
                          "when a per-kernel breakdown of the step is wanted")
     ap.add_argument("--ingest-profile", action="store_true",
                     help="run only the shard ingest kernel (200 launches) and print its time: the command to trace for it")
+    ap.add_argument("--conv-table", action="store_true",
+                    help="run only the per-shape table of the MFMA convolution launches (config 3 / 4 / 5 shapes, all directions)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB (reference point for HBM counter runs)")
     args = ap.parse_args()
@@ -405,6 +460,13 @@ def main():
     device = torch.device("cuda:0")
     if args.ingest_profile:
         print(json.dumps({"shard_ingest": bench_ingest(args, device, iters=200)}))
+        return
+    if args.conv_table:
+        rows = conv_table(device)
+        for r in rows:
+            print(f"{r['form']:17s} {r['cin']:4d}->{r['cout']:<4d} {'x'.join(str(v) for v in r['spatial']):>11s} {r['direction']:6s} "
+                  f"{r['us']:8.1f} us {r['gflop']:8.2f} GFLOP {r['tflops']:7.1f} TFLOP/s {r['frac']:.3f}", file=sys.stderr)
+        print(json.dumps({"conv_table": rows}))
         return
     if args.unet_profile:
         print(json.dumps({"unet_step_cfg5": bench_unet_step(args, device, eager_only=True)}))
