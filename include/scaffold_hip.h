@@ -185,6 +185,18 @@ int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype
                            int64_t halo_rows, float* mean, float* rstd, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/* The forward for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc. It has no counterpart in the reference. Same kernels and results as sfh_groupnorm_fwd, but the
+ * scratch for the partial statistics is a device array inside the library (sfh_groupnorm_fwd_noalloc_max_bytes() =
+ * 256 KiB, held by every GPU the library runs on until the process ends) instead of a workspace argument; neither this
+ * call nor anything it calls allocates or frees memory. The tensors' device must be current. A problem whose scratch
+ * exceeds the built-in buffer returns SFH_ERR_WORKSPACE (compare sfh_groupnorm_fwd_workspace_bytes with the maximum).
+ * All calls on one GPU share the buffer: calls that overlap in time on one GPU (two streams) race. */
+size_t sfh_groupnorm_fwd_noalloc_max_bytes(void);
+int sfh_groupnorm_fwd_noalloc(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
+                              const void* x, const void* gamma, const void* beta, void* y, float* mean,
+                              float* rstd, void* stream);
+
 /* ---- GroupNorm backward --------------------------------------------------------------
  * Stands in for torch.ops.scaffold_gn.group_norm_backward (triton_group_norm.py:1394) and
  * its kernels _bwd_partial_kernel (:813) and _dx_kernel (:908).

@@ -126,6 +126,9 @@ _SIGNATURES = {
     "sfh_groupnorm_fwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
     "sfh_groupnorm_fwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_groupnorm_fwd_noalloc_max_bytes": (c_size_t, []),
+    "sfh_groupnorm_fwd_noalloc": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                          c_void_p, c_void_p, c_void_p]),
     "sfh_shard_ingest": (c_int, [POINTER(IngestDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_skip_concat_fwd": (c_int, [POINTER(ConcatDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_skip_concat_bwd": (c_int, [POINTER(ConcatDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),

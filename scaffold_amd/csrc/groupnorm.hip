@@ -22,6 +22,8 @@
 // Two code paths, chosen by shape only: the vector path (16-byte loads, a thread owns a fixed
 // set of channels) when C is a multiple of the vector width and the channels of a thread fall
 // into whole groups; the scalar path (one workgroup per (sample, group)) otherwise.
+#include <mutex>
+
 #include "common.hpp"
 #include "vec_io.hpp"
 
@@ -964,6 +966,54 @@ extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, 
                                       void* workspace, size_t workspace_bytes, void* stream) {
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, workspace,
                            workspace_bytes, stream);
+}
+
+// ---- the forward for callers that may not allocate ------------------------------------------------------------------
+// Same kernels, same launch plan, same results as sfh_groupnorm_fwd; the partial-statistics scratch is this file-scope
+// device array instead of a caller's workspace. Every GPU the library runs on holds its own copy of the array (256 KiB,
+// until the process ends) at its own address, looked up once per device with that device current. Calls on one GPU
+// share the array: two that overlap in time (different streams) race. Nothing has to be cleared between calls: the
+// statistics kernel writes every slot the later kernels read.
+constexpr size_t kNoAllocScratchFloats = 64 * 1024;
+static __device__ __align__(256) float g_gn_noalloc_scratch[kNoAllocScratchFloats];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_noalloc_mutex;
+float* g_noalloc_ptr[kMaxDevices];  // device address of the array on each device (null: not looked up yet)
+
+// Device address of the scratch array on the CURRENT device. The array's name is a host-side handle, not an address a
+// kernel could use: the address comes from hipGetSymbolAddress, per device.
+int noalloc_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(SFH_ERR_LAUNCH, "groupnorm: no current device");
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  if (g_noalloc_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_gn_noalloc_scratch));
+    if (err != hipSuccess || ptr == nullptr)
+      return fail(SFH_ERR_LAUNCH, "groupnorm: hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(err));
+    g_noalloc_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_noalloc_ptr[dev];
+  return SFH_OK;
+}
+}  // namespace
+
+extern "C" size_t sfh_groupnorm_fwd_noalloc_max_bytes(void) { return kNoAllocScratchFloats * sizeof(float); }
+
+extern "C" int sfh_groupnorm_fwd_noalloc(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
+                                         const void* gamma, const void* beta, void* y, float* mean, float* rstd, void* stream) {
+  if (int rc = check_desc(p, x_dtype)) return rc;
+  const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(y));
+  const size_t need = pl.vector ? fwd_ws_floats(*p, pl) * sizeof(float) : 0;
+  if (need > kNoAllocScratchFloats * sizeof(float))
+    return fail(SFH_ERR_WORKSPACE, "groupnorm fwd (no-alloc): this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "
+                "use sfh_groupnorm_fwd with a workspace", need, kNoAllocScratchFloats * sizeof(float));
+  float* scratch = nullptr;
+  if (int rc = noalloc_scratch(&scratch)) return rc;
+  return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y, 0, mean, rstd, scratch,
+                           kNoAllocScratchFloats * sizeof(float), stream);
 }
 
 extern "C" size_t sfh_groupnorm_bwd_workspace_bytes(const sfh_groupnorm_desc* p, int x_dtype) {
