@@ -36,9 +36,9 @@ if ROOT not in sys.path:
 
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the forward kernel on the bench workload, from rocprofv3 FETCH_SIZE and WRITE_SIZE
-# counter runs of this script scaled by the same counters on the 256 MiB copy kernel (profiles/ holds the runs).
-CONV_FWD_HBM_TRAFFIC_BYTES = int((115560.0 * 2.000 + 131163.9) * 1024)
+# The counter summary that holds the HBM bytes per launch of the dominant kernel (rocprofv3 FETCH_SIZE and WRITE_SIZE
+# runs of this script, scaled by the same counters on the 256 MiB copy kernel).
+HBM_COUNTER_SUMMARY = os.path.join("profiles", "conv3d_32x32_128cube_hbm_counters.txt")
 CL = torch.channels_last_3d
 
 
@@ -54,6 +54,68 @@ def event_time_ms(fn, iters: int, warmup: int = 2) -> float:
     e1.record()
     e1.synchronize()
     return e0.elapsed_time(e1) / iters
+
+
+#: larger than the 256 MiB memory-side cache: writing it evicts every operand of the kernel under test
+FLUSH_BYTES = 512 << 20
+_flush_buffer = None
+
+
+def flush_caches():
+    """Overwrites a 512 MiB buffer, so that the next launch finds none of its operands in L2 or the memory-side cache
+    (the cold-sample rule of the reference's harness, triton_conv3d/bench/harness.py:62-69)."""
+    global _flush_buffer
+    if _flush_buffer is None:
+        _flush_buffer = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
+    _flush_buffer.add_(1)
+
+
+def spread(samples_ms, target_rel=0.02):
+    """min / median / mean and the 95 % confidence half-width of the mean of a list of samples; ``converged`` says
+    whether that half-width is within ``target_rel`` of the mean (harness.py's Measurement: every number carries its
+    precision)."""
+    n = len(samples_ms)
+    srt = sorted(samples_ms)
+    mean = sum(srt) / n
+    var = sum((v - mean) ** 2 for v in srt) / max(n - 1, 1)
+    half = 1.96 * math.sqrt(var / n)
+    return {"n": n, "min_ms": srt[0], "median_ms": srt[n // 2], "mean_ms": mean, "ci95_ms": half,
+            "converged": bool(half <= target_rel * mean)}
+
+
+def cold_samples_ms(fn, samples: int = 12, group: int = 2):
+    """``samples`` timings of ``fn`` with the caches flushed before each: a sample is ``group`` back-to-back calls
+    between two events (the first call after the flush finds nothing cached; a group of 2 keeps the event pair's own
+    cost below 2 % of a 100 us kernel), divided by ``group``."""
+    fn()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(samples):
+        flush_caches()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(group):
+            fn()
+        e1.record()
+        e1.synchronize()
+        out.append(e0.elapsed_time(e1) / group)
+    return spread(out)
+
+
+def counter_traffic(kernel: str):
+    """HBM bytes per launch of ``kernel`` as the committed counter summary states them (its line
+    ``traffic_bytes_per_launch <kernel> <bytes>``), with the file it came from; (None, None) when there is none, so a
+    figure can never outlive the summary it was read from."""
+    path = os.path.join(ROOT, HBM_COUNTER_SUMMARY)
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
+                    return int(parts[2]), HBM_COUNTER_SUMMARY
+    except OSError:
+        pass
+    return None, None
 
 
 def conv_operands(cin, cout, spatial, device, seed=3000):
@@ -121,17 +183,23 @@ def bench_conv(args, device):
     torch.cuda.synchronize()
     in_step = {name: sum(m[i].elapsed_time(m[i + 1]) for m in marks) / len(marks)
                for i, name in enumerate(("fwd", "dgrad", "wgrad"))}
+    in_step_spread = {name: spread([m[i].elapsed_time(m[i + 1]) for m in marks])
+                      for i, name in enumerate(("fwd", "dgrad", "wgrad"))}
     # each direction in a loop of its own (default entry points: forward and data gradient pack per call), and the
     # forward kernel alone in such a loop (weight packed beforehand): with 128 MB of operands per launch these loops
     # run out of the 256 MB memory-side cache and are faster than the same kernels inside the step
     per_dir = {name: event_time_ms(fn, max(args.steps, 5)) for name, fn in (("fwd", fwd), ("dgrad", dgrad), ("wgrad", wgrad))}
     pf, _ = sa.pack_weights(w, x.shape, 1, 1, 1, backward_data=False)
     fwd_kernel_ms = event_time_ms(lambda: sa.conv3d_forward(x, w, None, 1, 1, 1, out=y, packed_weight=pf), max(args.steps, 5))
+    # cold samples: 512 MiB written between samples, so every operand comes from HBM
+    cold = {name: cold_samples_ms(fn) for name, fn in (("fwd", fwd), ("dgrad", dgrad), ("wgrad", wgrad))}
     return {
         "flops_per_direction": flops,
         "ms_per_step": ms_per_step,
         "wall_ms_per_step": wall_ms,
         "in_step_ms": in_step,
+        "in_step_spread": in_step_spread,
+        "cold_flushed": cold,
         "per_direction_ms": per_dir,
         "fwd_kernel_alone_ms": fwd_kernel_ms,
         "per_direction_tflops": {k: flops / (v * 1e-3) / 1e12 for k, v in per_dir.items()},
@@ -261,6 +329,43 @@ def copy_calibration(device, mib=256, reps=4):
     return {"bytes_read": src.numel(), "bytes_written": src.numel(), "launches": reps}
 
 
+def ifs_shard(grid=128, depth=64, n_fractals=3, n_maps=4, orbits=256, steps=2048, burn_in=64, seed=5000):
+    """Synthetic config-5 sample (BASELINE.json config 5: IFS fractal occupancy in, 10 fractal classes + background as
+    labels): ``n_fractals`` random 3-D iterated function systems (``n_maps`` affine maps each: a random rotation scaled
+    by a contraction factor U(0.3, 0.7), offset U(-1, 1)^3), each attractor sampled by ``orbits`` chaos-game orbits run
+    side by side, voxelised on a ``grid`` cube with one isotropic voxel size and the bounding box centred
+    (ScaFFold/datagen/generate_fractal_points.py:62-104, volumegen.py:103-160,259-292: mask value = class id + 1, later
+    fractals overwrite earlier ones).  Returns the first ``depth`` planes: occupancy float32 (1, 1, depth, grid, grid)
+    and labels int64 (1, depth, grid, grid)."""
+    import numpy as np
+
+    rng = np.random.default_rng(seed)
+    labels = np.zeros((grid, grid, grid), dtype=np.int64)
+    for _ in range(n_fractals):
+        cls = int(rng.integers(0, 10))
+        mats = np.stack([np.linalg.qr(rng.standard_normal((3, 3)))[0] * rng.uniform(0.3, 0.7) for _ in range(n_maps)])
+        offs = rng.uniform(-1.0, 1.0, size=(n_maps, 3))
+        p = np.zeros((orbits, 3))
+        pts = []
+        for i in range(steps):
+            t = rng.integers(0, n_maps, size=orbits)
+            p = np.einsum("nij,nj->ni", mats[t], p) + offs[t]
+            if i >= burn_in:
+                pts.append(p)
+        pts = np.concatenate(pts)
+        mins = pts.min(axis=0)
+        voxel = (float((pts.max(axis=0) - mins).max()) + 1e-6) / grid
+        scaled = (pts - mins) / voxel
+        idx = np.clip(np.floor(scaled + (grid - scaled.max(axis=0)) / 2.0).astype(np.int64), 0, grid - 1)
+        labels[idx[:, 0], idx[:, 1], idx[:, 2]] = cls + 1
+    lab = torch.from_numpy(labels[:depth].copy())[None]
+    occ = (lab > 0).to(torch.float32)[:, None]
+    return occ, lab
+
+
+UNET_SEED = 5001
+
+
 def bench_unet_step(args, device, eager_only=False):
     """Config 5: one Adam step of the base-32, 5-level U-Net on a 64x128x128 depth shard (zero halo),
     bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0 fused with the Adam update.
@@ -269,12 +374,12 @@ def bench_unet_step(args, device, eager_only=False):
     of the whole step: the eager step is bound by ~600 Python-side launches, not by the GPU."""
     import scaffold_amd as sa
 
-    g = torch.Generator().manual_seed(5000)
-    occ = (torch.rand((1, 1, 64, 128, 128), generator=g) < 0.05).float().contiguous(memory_format=CL).to(device)
-    lab = torch.randint(0, 11, (1, 64, 128, 128), generator=g).to(device)
+    occ, lab = ifs_shard()
+    occupancy = float(occ.mean())
+    occ, lab = occ.contiguous(memory_format=CL).to(device), lab.to(device)
 
     def make(shard_halo=True):
-        torch.manual_seed(5001)
+        torch.manual_seed(UNET_SEED)
         model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(shard_halo)
         # clip_grad_norm_(1.0) + Adam (trainer.py:678-694); the update kernel also keeps the bf16 copies of the weights
         # the convolutions read under autocast, and they return fp32 weight gradients: no per-step casts either way
@@ -295,7 +400,8 @@ def bench_unet_step(args, device, eager_only=False):
     model, opt = make()
     step = step_fn(model, opt)
     ms = event_time_ms(step, 10, warmup=3)
-    out = {"ms_per_step": ms, "input": "1x1x64x128x128 occupancy (5% ones), zero depth halo, padding (0,1,1)"}
+    out = {"ms_per_step": ms, "input": f"1x1x64x128x128 IFS fractal occupancy ({occupancy:.3f} occupied), labels 0..10, "
+                                        "zero depth halo, padding (0,1,1)"}
     if eager_only:
         return out
     # The same arithmetic without the halo emulation's copies (depth padding 1 inside the kernels; bitwise the same
@@ -339,6 +445,7 @@ def bench_unet_step(args, device, eager_only=False):
         ok = all(abs(a - b) <= 1e-5 * max(1.0, abs(a)) for a, b in zip(eager_losses, graph_losses))
         out["graph_replay_matches_eager"] = ok
         out["graph_check_losses"] = {"eager": eager_losses, "graph": graph_losses}
+        out["first_loss"] = eager_losses[0]
         if ok:
             out["graph_ms_per_step"] = event_time_ms(graph.replay, 10, warmup=2)
     except Exception as exc:  # report, do not hide
@@ -399,9 +506,40 @@ def conv_table(device, iters=20):
     return rows
 
 
-def cpu_baseline():
-    """The reference's CPU path (torch conv3d + autograd, channels_last_3d bf16) on the bench workload itself,
-    repeated for about 12 s of host time."""
+def conv_counter_launches(device, reps=3):
+    """The launches a counter run (rocprofv3 --pmc) is taken over: plain eager calls, no graph, of the three MFMA
+    convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_persist_kernel,
+    wgrad_mfma_kernel), 128->64 @64^3 and 64->32 on the 64x128x128 slab (conv_mfma_kernel, wgrad_mfma_kernel)."""
+    import scaffold_amd as sa
+
+    done = []
+    for cin, cout, in_sp, pad in ((32, 32, (128, 128, 128), (1, 1, 1)), (128, 64, (64, 64, 64), (1, 1, 1)),
+                                  (64, 32, (66, 128, 128), (0, 1, 1))):
+        sp = tuple(in_sp[i] + 2 * pad[i] - 2 for i in range(3))
+        g = torch.Generator().manual_seed(3000 + cin + cout)
+        x = torch.randn((1, cin, *in_sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+        w = ((torch.rand((cout, cin, 3, 3, 3), generator=g) * 2 - 1) / math.sqrt(cin * 27)).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+        gy = torch.randn((1, cout, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+        pf, pd = sa.pack_weights(w, x.shape, 1, pad, 1)
+        y, gx = torch.empty_like(gy), torch.empty_like(x)
+        gw = torch.empty((cout, cin, 3, 3, 3), dtype=torch.float32, device=device).contiguous(memory_format=CL)
+        for _ in range(reps):
+            sa.conv3d_forward(x, w, None, 1, pad, 1, out=y, packed_weight=pf)
+            sa.conv3d_backward_data(gy, w, x.shape, 1, pad, 1, out=gx, packed_weight=pd)
+            sa.conv3d_backward_weight(x, w.shape, gy, 1, pad, 1, out=gw, grad_dtype=torch.float32)
+        torch.cuda.synchronize()
+        done.append({"cin": cin, "cout": cout, "output_spatial": list(sp), "launches_per_direction": reps,
+                     "flops_per_launch": 2 * math.prod(sp) * cin * cout * 27})
+    return done
+
+
+def cpu_baseline(with_unet=True):
+    """The reference's CPU path for the hot path's three parts, timed on this box's host cores (bounded samples):
+    the bench workload itself (torch conv3d + autograd, channels_last_3d bf16: what ScaFFold/unet/conv3d.py:1371-1378
+    falls to off-GPU) repeated for about 12 s; config 2's GroupNorm + ReLU forward and backward with the stock
+    functions (ScaFFold/unet/group_norm.py:715-721); and one config-5 train step of the stock-module U-Net under bf16
+    autocast (loss recipe, clipping and Adam of ScaFFold/utils/trainer.py:640-694) on the same seeded weights and the
+    same IFS shard the GPU step runs, whose loss the GPU step's first loss is checked against."""
     import torch.nn.functional as F
 
     cin = cout = 32
@@ -424,11 +562,77 @@ def cpu_baseline():
         once()
         times.append(time.perf_counter() - t0)
     t = sorted(times)[len(times) // 2]
-    return {
+    out = {
         "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
         "sample": f"torch CPU conv3d fwd+dgrad+wgrad, bf16 channels_last_3d, 32->32 3x3x3 on 128^3 (the whole workload), "
                   f"median of {len(times)} runs over {sum(times):.1f} s, {t * 1e3:.1f} ms each",
     }
+    del x, w, gy
+    try:
+        out["groupnorm_cfg2"] = cpu_groupnorm()
+    except Exception as exc:  # report, do not hide
+        out["groupnorm_cfg2"] = {"error": repr(exc)}
+    if with_unet:
+        try:
+            out["unet_step_cfg5"] = cpu_unet_step()
+        except Exception as exc:  # report, do not hide
+            out["unet_step_cfg5"] = {"error": repr(exc)}
+    return out
+
+
+def cpu_groupnorm(budget_s=4.0):
+    """Config 2 on the host: ``F.relu(F.group_norm(x, 8, gamma, beta))`` forward and its backward, bf16 channels_last_3d,
+    N=2, C=64, 64^3; algorithmic bytes 3B / 5B as on the GPU."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(2000)
+    shape = (2, 64, 64, 64, 64)
+    x = (torch.randn(shape, generator=g) * 3 + 0.5).to(torch.bfloat16).contiguous(memory_format=CL).requires_grad_(True)
+    gamma = (1 + 0.1 * torch.randn(64, generator=g)).requires_grad_(True)
+    beta = (0.1 * torch.randn(64, generator=g)).requires_grad_(True)
+    dy = torch.randn(shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL)
+    B = x.numel() * x.element_size()
+    fwd_t, bwd_t = [], []
+    end = time.perf_counter() + budget_s
+    while len(fwd_t) < 2 or (time.perf_counter() < end and len(fwd_t) < 50):
+        t0 = time.perf_counter()
+        y = F.relu(F.group_norm(x, 8, gamma.to(x.dtype), beta.to(x.dtype), 1e-5))
+        t1 = time.perf_counter()
+        torch.autograd.grad(y, (x, gamma, beta), dy)
+        t2 = time.perf_counter()
+        fwd_t.append(t1 - t0)
+        bwd_t.append(t2 - t1)
+    f, b = sorted(fwd_t)[len(fwd_t) // 2], sorted(bwd_t)[len(bwd_t) // 2]
+    return {"fwd_ms": f * 1e3, "bwd_ms": b * 1e3, "fwd_gbs": 3 * B / f / 1e9, "bwd_gbs": 5 * B / b / 1e9,
+            "cores": torch.get_num_threads(), "sample": f"median of {len(fwd_t)} runs of the whole config-2 tensor"}
+
+
+def cpu_unet_step():
+    """One config-5 train step of the stock-module arm on the host: same seeded initial weights and the same IFS shard
+    as the GPU step, bf16 autocast over fp32 master weights, CE + mean-foreground-Dice loss, clip 1.0, Adam."""
+    import scaffold_amd as sa
+    from oracle import oracle as orc
+
+    occ, lab = ifs_shard()
+    torch.manual_seed(UNET_SEED)
+    init = sa.UNet(1, 11, layers=4, base_width=32)
+    stock = sa.UNet(1, 11, layers=4, base_width=32, stock=True)
+    stock.load_state_dict(init.state_dict())
+    del init
+    stock = stock.to(memory_format=CL)
+    opt = torch.optim.Adam(stock.parameters(), lr=1e-3)
+    x = occ.contiguous(memory_format=CL)
+    t0 = time.perf_counter()
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        logits = stock(x)
+    loss = orc.train_step_loss(logits, lab, 11)
+    loss.backward()
+    norm = torch.nn.utils.clip_grad_norm_(stock.parameters(), 1.0)
+    opt.step()
+    opt.zero_grad(set_to_none=True)
+    t = time.perf_counter() - t0
+    return {"ms_per_step": t * 1e3, "loss": float(loss.detach()), "grad_norm": float(norm), "cores": torch.get_num_threads(),
+            "sample": "1 step (the first, no warm-up) of the stock-module U-Net, 64x128x128 IFS shard, bf16 autocast on the host"}
 
 
 def main():
@@ -447,6 +651,8 @@ def main():
                     help="run only the shard ingest kernel (200 launches) and print its time: the command to trace for it")
     ap.add_argument("--conv-table", action="store_true",
                     help="run only the per-shape table of the MFMA convolution launches (config 3 / 4 / 5 shapes, all directions)")
+    ap.add_argument("--conv-counters", action="store_true",
+                    help="run only a few plain launches of the three MFMA convolution kernels: the command for counter runs")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB (reference point for HBM counter runs)")
     args = ap.parse_args()
@@ -467,6 +673,9 @@ def main():
             print(f"{r['form']:17s} {r['cin']:4d}->{r['cout']:<4d} {'x'.join(str(v) for v in r['spatial']):>11s} {r['direction']:6s} "
                   f"{r['us']:8.1f} us {r['gflop']:8.2f} GFLOP {r['tflops']:7.1f} TFLOP/s {r['frac']:.3f}", file=sys.stderr)
         print(json.dumps({"conv_table": rows}))
+        return
+    if args.conv_counters:
+        print(json.dumps({"conv_counter_launches": conv_counter_launches(device)}))
         return
     if args.unet_profile:
         print(json.dumps({"unet_step_cfg5": bench_unet_step(args, device, eager_only=True)}))
@@ -495,6 +704,16 @@ def main():
     flops = conv["flops_per_direction"]
     fwd_ms = conv["in_step_ms"]["fwd"]
     achieved = flops / (fwd_ms * 1e-3) / 1e12
+    traffic, traffic_source = counter_traffic("conv_persist_kernel")
+    cpu = None if args.skip_cpu else cpu_baseline(with_unet=not args.skip_unet)
+    # the one full-size parity point of the train step: the stock-module arm's loss on the host against the first loss
+    # of the GPU step, from the same weights and the same shard (bf16 on both sides: 2e-2 relative)
+    parity_ok = True
+    if cpu is not None and "loss" in cpu.get("unet_step_cfg5", {}) and "first_loss" in details.get("unet_step_cfg5", {}):
+        a, b = details["unet_step_cfg5"]["first_loss"], cpu["unet_step_cfg5"]["loss"]
+        parity_ok = abs(a - b) <= 2e-2 * abs(b)
+        details["unet_step_cfg5"]["first_loss_vs_cpu_stock_arm"] = {"gpu": a, "cpu": b, "rel": abs(a - b) / abs(b),
+                                                                     "tolerance": 2e-2, "ok": parity_ok}
     line = {
         "metric": "conv3d fwd+dgrad+wgrad TFLOP/s @128^3 bf16 (U-Net level-0 conv 32->32, 1 GPU)",
         "value": 3 * flops / (conv["ms_per_step"] * 1e-3) / 1e12,
@@ -512,13 +731,19 @@ def main():
                                "(BASELINE.json config 3, first encoder level)"},
         "roofline": {
             "bound": "mfma", "kernel": "conv_persist_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": CONV_FWD_HBM_TRAFFIC_BYTES,
+            "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
             "flops_per_launch": flops, "avg_launch_ms": fwd_ms,
+            # the other two launches of the step, same FLOPs per launch (wgrad = wgrad_mfma_kernel + its slice sum)
+            "frac_by_direction": {k: flops / (v * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS for k, v in conv["in_step_ms"].items()},
         },
-        "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
+        "cpu_baseline": cpu,
         "details": details,
     }
     print(json.dumps(line))
+    if not parity_ok:
+        print("bench.py: the GPU step's first loss and the host stock arm's loss differ by more than 2e-2 relative",
+              file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":
