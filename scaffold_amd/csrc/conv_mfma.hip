@@ -435,6 +435,7 @@ int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStrea
 }
 
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
+  if (mfma_conv_wide_applies(a)) return 0;
   const GatherPlan p = gather_plan(a);
   if (a.cred == kChunk || p.ksplit == 1) return 0;
   return align_up((size_t)p.ksplit * a.n * a.od * a.oh * a.ow * a.cout * sizeof(float), 256);
@@ -442,6 +443,7 @@ size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
 
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                      void* partial, hipStream_t st) {
+  if (mfma_conv_wide_applies(a)) return mfma_conv_wide(a, dtype, x, packed, bias, y, st);
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st);
   return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st);
 }

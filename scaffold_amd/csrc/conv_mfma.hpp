@@ -35,6 +35,10 @@ int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStrea
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a);
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                      void* partial, hipStream_t st);
+// Same contract, wide-tile kernel (64 or more reduction channels, rows of more than 16 voxels): `applies` is a pure
+// function of the shape; mfma_conv_gather routes to it (it needs no partial workspace).
+bool mfma_conv_wide_applies(const MfmaConvArgs& a);
+int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st);
 // Same contract, persistent one-workgroup-per-CU kernel with register-resident weights.
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st);

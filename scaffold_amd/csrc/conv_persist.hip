@@ -275,44 +275,46 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
     for (int ms = 0; ms < C::MS; ++ms) aq[d][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(d));
 #pragma unroll
   for (int it = 0; it < C::NIT; ++it) {
-    if (it + ADEPTH < C::NIT) {
-#pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms)
-        aq[(it + ADEPTH) % (ADEPTH + 1)][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(it + ADEPTH));
-    }
-    if (it % 2 == 0 && it / 2 < NLOAD) {
-      const int k = (it / 2) / 4, p = (it / 2) % 4;
-      // only the last group of a wavefront can have lanes past the end of the brick
-      const bool full = (3 + 4 * k) * 64 + 63 < C::BV;
-      if (full || voff[k] != -1)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(nxt + (wave + 4 * k) * 1024 + p * C::PLANE),
-                                                 16, voff[k] + p * 16, 0, 0, 0);
-    }
-    if (it % 2 == 1 && it / 2 < NSTORE) {
-      const int ms = (it / 2) / 2, h = (it / 2) % 2;
-      __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
-    }
-    if (it % 2 == 1 && it >= PLAN0 && (it - PLAN0) / 2 < C::GPW) {
-      const int k = (it - PLAN0) / 2;
-      voff[k] = brick_group_offset<C>(a, plan_tc, plan_live, lg.gcoord[k], lg.grel[k]);  // group k's loads are all issued
-    }
-    if (it % 2 == 1 && it >= OFF0 && (it - OFF0) / 2 < C::MS) {
-      const int ms = (it - OFF0) / 2;
-      done_off[ms] = store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]);  // the previous brick's pieces are all stored
-    }
     __builtin_amdgcn_sched_barrier(0);
-    if (it == 0) {
+    // The activation fragments of iteration it + ADEPTH are requested BETWEEN this iteration's MFMAs, one behind each: a
+    // ds_read issued while the matrix pipe is busy costs nothing, a block of them in front of the MFMAs leaves the pipe
+    // idle for as long as they take to issue.
+    f32x16_t zero;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+#pragma unroll
+    for (int ms = 0; ms < C::MS; ++ms) {
       // a brick starts from zero: the first MFMA takes a zero addend instead of a clearing pass
-      f32x16_t zero;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-#pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
-    } else {
-#pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms) {
-        if (it < C::NVEC) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
-        else MmaAcc<T>::run(wa[it - C::NVEC], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      if (it == 0) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
+      else if (it < C::NVEC) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      else MmaAcc<T>::run(wa[it - C::NVEC], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      __builtin_amdgcn_sched_barrier(0);
+      if (it + ADEPTH < C::NIT)
+        aq[(it + ADEPTH) % (ADEPTH + 1)][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(it + ADEPTH));
+      __builtin_amdgcn_sched_barrier(0);
+      // one piece of side work per iteration, behind the first MFMA
+      if (ms == 0) {
+        if (it % 2 == 0 && it / 2 < NLOAD) {
+          const int k = (it / 2) / 4, p = (it / 2) % 4;
+          // only the last group of a wavefront can have lanes past the end of the brick
+          const bool full = (3 + 4 * k) * 64 + 63 < C::BV;
+          if (full || voff[k] != -1)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(nxt + (wave + 4 * k) * 1024 + p * C::PLANE),
+                                                     16, voff[k] + p * 16, 0, 0, 0);
+        }
+        if (it % 2 == 1 && it / 2 < NSTORE) {
+          const int ms = (it / 2) / 2, h = (it / 2) % 2;
+          __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
+        }
+        if (it % 2 == 1 && it >= PLAN0 && (it - PLAN0) / 2 < C::GPW) {
+          const int k = (it - PLAN0) / 2;
+          voff[k] = brick_group_offset<C>(a, plan_tc, plan_live, lg.gcoord[k], lg.grel[k]);  // group k's loads are all issued
+        }
+        if (it % 2 == 1 && it >= OFF0 && (it - OFF0) / 2 < C::MS) {
+          const int ms = (it - OFF0) / 2;
+          done_off[ms] = store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]);  // the previous brick's pieces are all stored
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);

@@ -425,6 +425,97 @@ def test_full_size_128cube_properties(device):
     assert torch.equal(y[:, :, :9, :9, :39].cpu().double(), ref[:, :, :9, :9, :39])
 
 
+# --- wide-tile kernel (a 64-channel output from 128 or more reduction channels, rows of more than 16 voxels) ---------
+# (cin, cout, spatial, padding, direction): the forward reduces over cin and produces cout, the data gradient the
+# reverse. Both accumulator grids of the kernel (8 sub-tiles x 2 channel blocks when such workgroups fill the chip, else
+# 4 x 2), ragged edges in all three extents, a reduction of 12 chunks, and the depth-slab padding form.
+WIDE_SHAPES = [
+    (128, 64, (63, 61, 65), (1, 1, 1), "fwd"),
+    (64, 128, (63, 61, 65), (1, 1, 1), "bwd-data"),
+    (128, 64, (32, 64, 64), (0, 1, 1), "fwd"),
+    (64, 128, (30, 62, 34), (1, 1, 1), "bwd-data"),
+    (192, 64, (30, 62, 34), (1, 1, 1), "fwd"),
+]
+
+
+@pytest.mark.parametrize("cin,cout,spatial,padding,direction", WIDE_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_wide_tile_exact(device, dtype, cin, cout, spatial, padding, direction):
+    """Exact standard at sizes the fp64 oracle does not finish in seconds: operands in {-1, 0, 1}, thinned so every
+    partial sum is a small integer. The tiled kernel must agree bit for bit with the untiled direct kernel (an
+    independent index path, itself held to the oracle at small sizes), with the oracle on the corner block of the
+    volume, and the two directions must be exactly adjoint."""
+    cl = torch.channels_last_3d
+    g = torch.Generator().manual_seed(cin * 1000 + cout)
+    out_sp = tuple(spatial[i] + 2 * padding[i] - 2 for i in range(3))
+
+    def draw(shp, density):
+        keep = torch.rand(shp, generator=g) < density
+        sign = torch.randint(0, 2, shp, generator=g) * 2 - 1
+        return (keep * sign).to(dtype)
+
+    x = draw((1, cin, *spatial), 0.05).contiguous(memory_format=cl).to(device)
+    gy = draw((1, cout, *out_sp), 0.05).contiguous(memory_format=cl).to(device)
+    w = draw((cout, cin, 3, 3, 3), 0.5).contiguous(memory_format=cl).to(device)
+    assert c3.uses_mfma(x.shape, w.shape, 1, padding, 1, dtype, direction)
+    if direction == "fwd":
+        got = sa.conv3d_forward(x, w, None, 1, padding, 1)
+        ref_direct = sa.conv3d_forward(x, w, None, 1, padding, 1, force_generic=True)
+    else:
+        got = sa.conv3d_backward_data(gy, w, x.shape, 1, padding, 1)
+        ref_direct = sa.conv3d_backward_data(gy, w, x.shape, 1, padding, 1, force_generic=True)
+    assert got.abs().max() > 0 and got.abs().max() < 256
+    assert torch.equal(got, ref_direct)
+    # corner block against the oracle: outputs that depend on the first 10 x 10 x 40 input voxels only
+    if direction == "fwd":
+        corner = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=(10, 10, 40), padding=padding, dtype=dtype)
+        xc = x[:, :, :10, :10, :40].cpu().contiguous(memory_format=cl)
+        ref = orc.conv_reference(corner, {"input": xc, "weight": w.cpu(), "bias": None, "grad_output": None}, "fwd")
+        d, h, wd = (ref.shape[2] - 1, ref.shape[3] - 1, ref.shape[4] - 1)
+        assert torch.equal(got[:, :, :d, :h, :wd].cpu().double(), ref[:, :, :d, :h, :wd])
+        # adjointness with the data gradient: <fwd(x), g> = <x, dgrad(g)>, exactly (small integers)
+        gx = sa.conv3d_backward_data(gy, w, x.shape, 1, padding, 1)
+        assert (got.double() * gy.double()).sum().item() == (x.double() * gx.double()).sum().item()
+    else:
+        # gradient of the corner outputs alone, against the oracle on that corner's receptive field
+        gy_c = torch.zeros_like(gy)
+        gy_c[:, :, :6, :6, :30] = gy[:, :, :6, :6, :30]
+        got_c = sa.conv3d_backward_data(gy_c, w, x.shape, 1, padding, 1)
+        in_c = tuple(6 + 2 - 2 * padding[i] if i < 2 else 30 + 2 - 2 * padding[i] for i in range(3))
+        corner = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=in_c, padding=padding, dtype=dtype)
+        ops = {"input": torch.zeros((1, cin, *in_c), dtype=dtype).contiguous(memory_format=cl), "weight": w.cpu(), "bias": None,
+               "grad_output": gy[:, :, :6, :6, :30].cpu().contiguous(memory_format=cl)}
+        ref = orc.conv_reference(corner, ops, "bwd-data")
+        # away from the cut faces of the corner problem its data gradient is the full problem's
+        d, h, wd = in_c[0] - 2, in_c[1] - 2, in_c[2] - 2
+        assert torch.equal(got_c[:, :, :d, :h, :wd].cpu().double(), ref[:, :, :d, :h, :wd])
+        assert got_c[:, :, in_c[0] + 1:].abs().max() == 0
+
+
+@pytest.mark.parametrize("direction", ["fwd", "bwd-data"])
+def test_wide_tile_bias_and_gaussian_tolerance(device, direction):
+    """Gaussian operands (and a bias in the forward) through the wide-tile kernel at a size that selects it; held to
+    the bf16 tolerance of the fp64 oracle on the corner block of the volume (the oracle on the whole volume takes minutes)."""
+    cl = torch.channels_last_3d
+    cin, cout = (128, 64) if direction == "fwd" else (64, 128)
+    full = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=(32, 64, 64), padding=(1, 1, 1), dtype=torch.bfloat16, bias=direction == "fwd")
+    ops = orc.make_inputs(full, seed=11)
+    x, w, gy = (ops[k].to(device) for k in ("input", "weight", "grad_output"))
+    corner = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=(10, 10, 40), padding=(1, 1, 1), dtype=torch.bfloat16, bias=full.bias)
+    if direction == "fwd":
+        got = sa.conv3d_forward(x, w, ops["bias"].to(device), 1, 1, 1)
+        ref = orc.conv_reference(corner, {"input": ops["input"][:, :, :10, :10, :40].contiguous(memory_format=cl), "weight": ops["weight"],
+                                          "bias": ops["bias"], "grad_output": None}, "fwd")
+        orc.assert_baseline_tolerance(got[:, :, :9, :9, :39], ref[:, :, :9, :9, :39], torch.bfloat16, "wide fwd")
+    else:
+        gy_c = torch.zeros_like(gy)
+        gy_c[:, :, :10, :10, :40] = gy[:, :, :10, :10, :40]
+        got = sa.conv3d_backward_data(gy_c, w, x.shape, 1, 1, 1)
+        ref = orc.conv_reference(corner, {"input": ops["input"][:, :, :10, :10, :40].contiguous(memory_format=cl), "weight": ops["weight"], "bias": None,
+                                          "grad_output": ops["grad_output"][:, :, :10, :10, :40].contiguous(memory_format=cl)}, "bwd-data")
+        orc.assert_baseline_tolerance(got[:, :, :10, :10, :40], ref, torch.bfloat16, "wide bwd-data")
+
+
 # --- bias gradient --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("shape", [(1, 11, 7, 9, 13), (2, 32, 4, 5, 6), (1, 300, 2, 3, 3), (1, 1, 5, 5, 5), (1, 64, 33, 32, 31)])
