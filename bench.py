@@ -207,6 +207,41 @@ def bench_conv(args, device):
     }
 
 
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 MFMA
+
+
+def bench_conv_fp32_cfg1(device, iters=20):
+    """Config 1 of BASELINE.json: the 32 -> 32 convolution at 32^3 in fp32 (the reference's CPU-runnable case), all three
+    directions on the fp32 matrix pipe (v_mfma_f32_32x32x2_f32: true fp32 operands and products); each direction in a
+    captured graph of 10 launches, against the dense fp32 MFMA peak."""
+    import scaffold_amd as sa
+    from scaffold_amd import conv3d as c3
+
+    g = torch.Generator().manual_seed(1000)
+    sp = (32, 32, 32)
+    x = torch.randn((1, 32, *sp), generator=g).contiguous(memory_format=CL).to(device)
+    w = ((torch.rand((32, 32, 3, 3, 3), generator=g) * 2 - 1) / math.sqrt(32 * 27)).contiguous(memory_format=CL).to(device)
+    gy = torch.randn((1, 32, *sp), generator=g).contiguous(memory_format=CL).to(device)
+    y, gx = torch.empty_like(gy), torch.empty_like(x)
+    gw = sa.grad_weight_empty(32, 32, (3, 3, 3), dtype=torch.float32, device=device)
+    flops = 2 * math.prod(sp) * 32 * 32 * 27
+    out = {"flops_per_direction": flops, "uses_matrix_pipe": {d: bool(c3.uses_mfma(x.shape, w.shape, 1, 1, 1, torch.float32, d))
+                                                             for d in ("fwd", "bwd-data", "bwd-weight")}}
+    fns = {"fwd": lambda: sa.conv3d_forward(x, w, None, 1, 1, 1, out=y),
+           "dgrad": lambda: sa.conv3d_backward_data(gy, w, x.shape, 1, 1, 1, out=gx),
+           "wgrad": lambda: sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, 1, out=gw)}
+    for name, fn in fns.items():
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(10):
+                fn()
+        ms = event_time_ms(graph.replay, max(2, iters // 10), warmup=1) / 10
+        out[name] = {"us": ms * 1e3, "tflops": flops / (ms * 1e-3) / 1e12, "frac_of_fp32_mfma_peak": flops / (ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS}
+    return out
+
+
 def bench_groupnorm(args, device):
     """Config 2: N=2, C=64, 64^3, 8 groups, bf16, fused ReLU; algorithmic bytes 3B forward / 5B backward.
 
@@ -688,6 +723,10 @@ def main():
         details["vendor_gemm_reference"] = {"error": repr(exc)}
     if args.copy_calibration:
         details["copy_calibration"] = copy_calibration(device)
+    try:
+        details["conv_fp32_cfg1"] = bench_conv_fp32_cfg1(device)
+    except Exception as exc:  # report, do not hide
+        details["conv_fp32_cfg1"] = {"error": repr(exc)}
     try:
         details["groupnorm_cfg2"] = bench_groupnorm(args, device)
     except Exception as exc:  # report, do not hide

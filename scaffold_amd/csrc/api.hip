@@ -7,6 +7,7 @@
 #include "ingest.hpp"
 #include "conv_direct.hpp"
 #include "conv_mfma.hpp"
+#include "conv_f32.hpp"
 #include "conv_patch.hpp"
 #include "conv_thin.hpp"
 #include "halo.hpp"
@@ -88,6 +89,10 @@ MfmaConvArgs dgrad_mfma_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
 bool fwd_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return is_unit(p) && mfma_conv_supported(fwd_mfma_args(p, out), dtype);
 }
+// fp32 problems of the tiled shape run on the fp32 matrix pipe (the weight is packed per call into the workspace)
+bool fwd_uses_f32_tiles(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return dtype == SFH_FP32 && is_unit(p) && f32_conv_supported(fwd_mfma_args(p, out));
+}
 
 int check_dgrad(const sfh_conv3d_desc& p) {
   if (p.sd != 1 || p.sh != 1 || p.sw != 1)
@@ -101,6 +106,9 @@ int check_dgrad(const sfh_conv3d_desc& p) {
 bool dgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return is_unit(p) && mfma_conv_supported(dgrad_mfma_args(p, out), dtype);
 }
+bool dgrad_uses_f32_tiles(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return dtype == SFH_FP32 && is_unit(p) && f32_conv_supported(dgrad_mfma_args(p, out));
+}
 
 WgradArgs wgrad_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
   WgradArgs a{};
@@ -112,6 +120,10 @@ WgradArgs wgrad_args(const sfh_conv3d_desc& p, const int32_t out[3]) {
 
 bool wgrad_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return is_unit(p) && p.kd == 3 && p.kh == 3 && p.kw == 3 && p.n >= 1 && mfma_wgrad_supported(wgrad_args(p, out), dtype);
+}
+
+bool wgrad_uses_f32_tiles(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
+  return dtype == SFH_FP32 && is_unit(p) && p.kd == 3 && p.kh == 3 && p.kw == 3 && p.n >= 1 && f32_wgrad_supported(wgrad_args(p, out));
 }
 
 // ---- 2x2x2, stride-2, unpadded problems (the up-convolution family) ------------------------------
@@ -292,9 +304,10 @@ extern "C" int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]
 extern "C" int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (direction == 0) return (fwd_uses_mfma(*p, dtype, out) || fwd_uses_patch(*p, dtype, out)) ? 1 : 0;
-  if (direction == 1) return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out)) ? 1 : 0;
-  return (wgrad_uses_mfma(*p, dtype, out) || wgrad_uses_patch(*p, dtype, out)) ? 1 : 0;
+  if (direction == 0) return (fwd_uses_mfma(*p, dtype, out) || fwd_uses_patch(*p, dtype, out) || fwd_uses_f32_tiles(*p, dtype, out)) ? 1 : 0;
+  if (direction == 1)
+    return (check_dgrad(*p) == SFH_OK && (dgrad_uses_mfma(*p, dtype, out) || dgrad_uses_f32_tiles(*p, dtype, out))) ? 1 : 0;
+  return (wgrad_uses_mfma(*p, dtype, out) || wgrad_uses_patch(*p, dtype, out) || wgrad_uses_f32_tiles(*p, dtype, out)) ? 1 : 0;
 }
 
 // ---- forward ---------------------------------------------------------------------------
@@ -302,6 +315,7 @@ extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int d
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (fwd_uses_patch(*p, dtype, out)) return mfma_conv_packed_weight_bytes(patch_pack_args(p->cout, p->cin));
+  if (fwd_uses_f32_tiles(*p, dtype, out)) return f32_conv_packed_weight_bytes(fwd_mfma_args(*p, out));
   if (!fwd_uses_mfma(*p, dtype, out)) return 0;
   return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out)) + mfma_conv_partial_bytes(fwd_mfma_args(*p, out));
 }
@@ -329,6 +343,14 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
       return rc;
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st);
+  }
+  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && fwd_uses_f32_tiles(*p, dtype, out)) {
+    const MfmaConvArgs a = fwd_mfma_args(*p, out);
+    const size_t need = f32_conv_packed_weight_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    if (int rc = f32_pack_weight(a, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st)) return rc;
+    return f32_conv(a, x, workspace, bias, y, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && (flags & SFH_FLAG_WEIGHT_PACKED) && fwd_uses_patch(*p, dtype, out))
     return patch_gather(patch_args(*p, out), dtype, x, w, bias, y, st);
@@ -435,7 +457,9 @@ extern "C" int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t
 extern "C" size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
-  if (check_dgrad(*p) != SFH_OK || !dgrad_uses_mfma(*p, dtype, out)) return 0;
+  if (check_dgrad(*p) != SFH_OK) return 0;
+  if (dgrad_uses_f32_tiles(*p, dtype, out)) return f32_conv_packed_weight_bytes(dgrad_mfma_args(*p, out));
+  if (!dgrad_uses_mfma(*p, dtype, out)) return 0;
   return mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out)) + mfma_conv_partial_bytes(dgrad_mfma_args(*p, out));
 }
 
@@ -463,6 +487,15 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
       return rc;
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st);
+  }
+  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && dgrad_uses_f32_tiles(*p, dtype, out)) {
+    const MfmaConvArgs a = dgrad_mfma_args(*p, out);
+    const size_t need = f32_conv_packed_weight_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    // produced channel = Cin (stride w_stride[1]), reduction channel = Cout (w_stride[0]), taps flipped
+    if (int rc = f32_pack_weight(a, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, workspace, st)) return rc;
+    return f32_conv(a, gy, workspace, nullptr, gx, st);
   }
   if (flags & SFH_FLAG_WEIGHT_PACKED) return fail(SFH_ERR_INVALID, "conv3d dgrad: this problem does not read a packed weight");
   if (!(flags & SFH_FLAG_FORCE_GENERIC)) {
@@ -493,6 +526,7 @@ extern "C" int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_splits(wgrad_args(*p, out));
+  if (wgrad_uses_f32_tiles(*p, dtype, out)) return f32_wgrad_splits(wgrad_args(*p, out));
   if (wgrad_uses_patch(*p, dtype, out)) return patch_reduce_splits(patch_args(*p, out));
   ThinArgs t;
   bool thin_is_x;
@@ -504,6 +538,7 @@ extern "C" size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK) return 0;
   if (wgrad_uses_mfma(*p, dtype, out)) return mfma_wgrad_workspace_bytes(wgrad_args(*p, out));
+  if (wgrad_uses_f32_tiles(*p, dtype, out)) return f32_wgrad_workspace_bytes(wgrad_args(*p, out));
   if (wgrad_uses_patch(*p, dtype, out)) return patch_reduce_workspace_bytes(patch_args(*p, out));
   ThinArgs t;
   bool thin_is_x;
@@ -524,6 +559,13 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
     return mfma_wgrad(a, dtype, x, gy, gw, gw_dtype, workspace, st);
+  }
+  if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_f32_tiles(*p, dtype, out)) {
+    const WgradArgs a = wgrad_args(*p, out);
+    const size_t need = f32_wgrad_workspace_bytes(a);
+    if (workspace == nullptr || workspace_bytes < need)
+      return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+    return f32_wgrad(a, x, gy, gw, workspace, st);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_patch(*p, dtype, out)) {
     const PatchArgs a = patch_args(*p, out);

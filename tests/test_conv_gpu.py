@@ -207,6 +207,52 @@ def test_fp32_is_true_fp32(device, direction):
     orc.assert_baseline_tolerance(got, ref, torch.float32, direction)
 
 
+# fp32 problems of the tiled shape run on the fp32 matrix pipe (forward and data gradient); the reference runs them through
+# its tiled kernel at input_precision="ieee" (`triton_conv3d/gather_gemm.py:1334`).
+F32_TILE_SHAPES = [
+    # (n, cin, cout, spatial, padding, direction): both brick shapes (4 x 4 x 32 when such workgroups fill the chip, else
+    # 2 x 2 x 32), ragged extents, reductions of 1 / 2 / 3 / 4 chunks of 16 channels (the forward reduces over cin, the data
+    # gradient over cout), the three padding forms of a depth shard
+    (1, 32, 32, (8, 8, 32), (1, 1, 1), "fwd"),
+    (1, 32, 32, (8, 8, 32), (1, 1, 1), "bwd-data"),
+    (2, 16, 32, (5, 7, 33), (1, 1, 1), "fwd"),
+    (2, 32, 16, (5, 7, 33), (1, 1, 1), "bwd-data"),
+    (1, 48, 64, (6, 9, 40), (0, 1, 1), "fwd"),
+    (1, 64, 48, (6, 9, 40), (0, 1, 1), "bwd-data"),
+    (1, 32, 96, (4, 6, 20), (2, 2, 2), "fwd"),
+    (1, 96, 32, (4, 6, 20), (2, 2, 2), "bwd-data"),
+    (1, 64, 32, (3, 3, 5), (0, 0, 0), "fwd"),
+    (1, 32, 64, (33, 34, 70), (1, 1, 1), "fwd"),
+    (1, 32, 64, (33, 34, 70), (1, 1, 1), "bwd-data"),
+    # weight gradient (both channel counts multiples of 32): split over output rows, odd row lengths, batch > 1
+    (1, 32, 32, (8, 8, 32), (1, 1, 1), "bwd-weight"),
+    (2, 32, 64, (5, 7, 33), (1, 1, 1), "bwd-weight"),
+    (1, 64, 32, (6, 9, 40), (0, 1, 1), "bwd-weight"),
+    (1, 32, 96, (4, 6, 21), (2, 2, 2), "bwd-weight"),
+    (3, 64, 64, (3, 3, 5), (0, 0, 0), "bwd-weight"),
+    (1, 32, 32, (1, 1, 1), (1, 1, 1), "bwd-weight"),
+]
+
+
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,direction", F32_TILE_SHAPES)
+def test_fp32_tiles_exact(device, n, cin, cout, spatial, padding, direction):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=torch.float32, bias=direction == "fwd")
+    assert c3.uses_mfma(prob.input_shape, prob.weight_shape, 1, padding, 1, torch.float32, direction)
+    check_exact(prob, direction, device)
+    check_exact(prob, direction, device, force_generic=True)
+
+
+@pytest.mark.parametrize("direction", DIRS)
+def test_fp32_tiles_gaussian_is_true_fp32(device, direction):
+    """Gaussian operands through the fp32 matrix pipe: 1e-5 relative to the fp64 oracle, i.e. no 16-bit or tf32-like rounding
+    of operands or products anywhere (a bf16 product alone would be off by 4e-3)."""
+    prob = orc.ConvProblem(n=1, cin=64, cout=64, spatial=(9, 13, 35), padding=(1, 1, 1), dtype=torch.float32, bias=direction == "fwd")
+    ops = orc.make_inputs(prob, seed=21)
+    ref = orc.conv_reference(prob, ops, direction)
+    got = run(prob, ops, direction, device)
+    orc.assert_baseline_tolerance(got, ref, torch.float32, f"fp32 tiles {direction}")
+
+
 # --- transposed convolution ---------------------------------------------------------------------
 CONVT_SHAPES = [
     (1, 128, 64, (4, 4, 4), (2, 2, 2), True),
