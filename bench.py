@@ -451,7 +451,7 @@ def bench_unet_step(args, device, eager_only=False):
     try:
         model_e, opt_e = make()
         eager = step_fn(model_e, opt_e)
-        eager_losses = [float(eager()) for _ in range(4)]
+        eager_losses = [float(eager().detach()) for _ in range(4)]
         model_g, opt_g = make()
         gstep = step_fn(model_g, opt_g)
         side = torch.cuda.Stream()

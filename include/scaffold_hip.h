@@ -80,7 +80,10 @@ int sfh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t
 /* Output spatial extents of a conv3d problem; SFH_ERR_INVALID if the output would be empty. */
 int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]);
 /* 1 if the MFMA implicit-GEMM kernels (rather than the direct kernels) serve this problem
- * in the given direction: 0 = forward, 1 = data-gradient, 2 = weight-gradient. */
+ * in the given direction: 0 = forward, 1 = data-gradient, 2 = weight-gradient. SFH_BF16 / SFH_FP16
+ * problems run on the 16-bit matrix pipe with fp32 accumulation; SFH_FP32 problems of the tiled shape
+ * (3x3x3, stride 1, channel counts multiples of 16 / 32) on the fp32 matrix pipe with fp32 operands and
+ * products, the precision the reference asks of its fp32 path (gather_gemm.py:1334, "ieee"). */
 int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
 
 /* ---- conv3d forward ------------------------------------------------------------------
@@ -88,7 +91,7 @@ int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
  * kernel _conv3d_fwd_kernel (gather_gemm.py:112).
  * y[n,co,od,oh,ow] = bias[co] + sum_{ci,kd,kh,kw} x[n,ci,od*sd+kd*dd-pd,...] * w[co,ci,kd,kh,kw]
  * bias may be NULL; when given it has Cout elements of the activation dtype.
- * The workspace holds the weight repacked into MFMA fragment order. */
+ * The workspace holds the weight repacked into MFMA fragment order (16-bit and fp32 tiled problems). */
 size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
 int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w,
                    const int64_t w_stride[5], const void* bias, void* y, void* workspace,

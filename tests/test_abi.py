@@ -60,17 +60,20 @@ def test_kernel_selection_is_a_pure_function_of_the_problem():
     bf16, fp32 = 0, 2
     d = conv_desc(sp=(128, 128, 128))
     assert [L.sfh_conv3d_uses_mfma(ctypes.byref(d), bf16, i) for i in range(3)] == [1, 1, 1]
-    assert [L.sfh_conv3d_uses_mfma(ctypes.byref(d), fp32, i) for i in range(3)] == [0, 0, 0]          # fp32 is true fp32
+    assert [L.sfh_conv3d_uses_mfma(ctypes.byref(d), fp32, i) for i in range(3)] == [1, 1, 1]          # fp32: the fp32 matrix pipe
+    assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(cin=8)), fp32, 0) == 0                         # not a multiple of 16
     assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(cin=3)), bf16, 0) == 0                         # odd channels
     assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(s=(2, 2, 2))), bf16, 0) == 0                   # strided
     assert L.sfh_conv3d_uses_mfma(ctypes.byref(conv_desc(p=(0, 1, 1))), bf16, 1) == 1                   # shard form dgrad
     # workspace sizes: packed weight for fwd/dgrad, splits * Cout * 27 * Cin fp32 for wgrad
     assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(d), bf16) == 32 * 32 * 27 * 2
-    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(d), fp32) == 0
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(d), fp32) == 32 * 32 * 27 * 4              # fp32 packed weight
     splits = L.sfh_conv3d_wgrad_splits(ctypes.byref(d), bf16)
     assert splits >= 1 and splits == L.sfh_conv3d_wgrad_splits(ctypes.byref(d), bf16)
     assert L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(d), bf16) == splits * 32 * 27 * 32 * 4
-    assert L.sfh_conv3d_wgrad_splits(ctypes.byref(d), fp32) == 1
+    splits32 = L.sfh_conv3d_wgrad_splits(ctypes.byref(d), fp32)
+    assert splits32 >= 1 and L.sfh_conv3d_wgrad_workspace_bytes(ctypes.byref(d), fp32) == splits32 * 32 * 27 * 32 * 4
+    assert L.sfh_conv3d_wgrad_splits(ctypes.byref(conv_desc(cin=8)), fp32) == 1                         # untiled: one pass, no slices
 
 
 def test_wgrad_split_plan_partitions_the_bricks():
