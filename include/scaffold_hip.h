@@ -77,6 +77,13 @@ int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
 int sfh_device_info(char* name, size_t name_len, int32_t* compute_units, int32_t* lds_bytes);
+/* The compute-unit count the launch geometry (persistent grids, split counts) is written for: 256, MI355X. Split
+ * counts -- and with them the summation order of split results -- are functions of the problem shape and of this
+ * constant alone, never of the device the call runs on, so results are the same bits on every device; on a device
+ * with another count the geometry is merely not the best one (compare with sfh_device_info). No counterpart in
+ * the reference (its split counts are functions of shape and a compiled-in target as well,
+ * triton_conv3d/reduce_gemm.py:71-96). */
+int sfh_tuned_compute_units(void);
 /* Output spatial extents of a conv3d problem; SFH_ERR_INVALID if the output would be empty. */
 int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]);
 /* 1 if the MFMA implicit-GEMM kernels (rather than the direct kernels) serve this problem

@@ -105,6 +105,7 @@ _SIGNATURES = {
     "sfh_version": (c_int, []),
     "sfh_last_error": (c_char_p, []),
     "sfh_device_info": (c_int, [c_char_p, c_size_t, POINTER(c_int32), POINTER(c_int32)]),
+    "sfh_tuned_compute_units": (c_int, []),
     "sfh_conv3d_out_shape": (c_int, [POINTER(ConvDesc), POINTER(c_int32)]),
     "sfh_conv3d_uses_mfma": (c_int, [POINTER(ConvDesc), c_int, c_int]),
     "sfh_conv3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
@@ -219,7 +220,30 @@ def strides5(t: torch.Tensor):
     return _I64x5(*[int(s) for s in t.stride()])
 
 
+_devices_seen: set = set()
+
+
+def _note_device(device: torch.device) -> None:
+    """Once per device: compares its compute-unit count with the one the library's launch geometry is written for.
+    Split counts are functions of the problem shape and that compiled-in count, so results do not depend on the device;
+    on a device of another size the geometry is only not the best one, which is worth a warning, not an error."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index in _devices_seen:
+        return
+    _devices_seen.add(index)
+    units, lds = c_int32(0), c_int32(0)
+    with torch.cuda.device(index):
+        rc = lib().sfh_device_info(None, 0, ctypes.byref(units), ctypes.byref(lds))
+    tuned = int(lib().sfh_tuned_compute_units())
+    if rc == SFH_OK and units.value != tuned:
+        import warnings
+
+        warnings.warn(f"libscaffold_hip's launch geometry is written for {tuned} compute units; device {index} has "
+                      f"{units.value}: results are unaffected, launch shapes are not the best ones for it", RuntimeWarning, stacklevel=3)
+
+
 def stream_ptr(device: torch.device) -> int:
+    _note_device(device)
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 

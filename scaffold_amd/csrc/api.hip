@@ -296,6 +296,8 @@ extern "C" int sfh_device_info(char* name, size_t name_len, int32_t* compute_uni
   return SFH_OK;
 }
 
+extern "C" int sfh_tuned_compute_units(void) { return kComputeUnits; }
+
 extern "C" int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]) {
   if (out_dhw == nullptr) return fail(SFH_ERR_INVALID, "conv3d: null output");
   return check_conv(p, SFH_FP32, out_dhw);

@@ -23,28 +23,13 @@
 // The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
 // padding k-1-p (triton_conv3d/bwd_data.py:344-363).
 #include "conv_mfma.hpp"
+#include "mma.hpp"
 #include "reduce.hpp"
 
 namespace sfh {
 namespace {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
-};
-template <> struct Mma<fp16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_fp16x2(lo, hi); }
-};
 
 constexpr int kChunk = 32;  // reduction channels staged per pass (4 planes of 8)
 
@@ -195,7 +180,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 #pragma unroll
       for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
-        for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma<T>::run(wq[it][ns], aq[it & 1][ms], acc[ms][ns]);
+        for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma32<T>::run(wq[it][ns], aq[it & 1][ms], acc[ms][ns]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -235,8 +220,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
           const T* bp = bias + nb * C::NSUB * 32 + co;
           b0 = to_float(bp[0]); b1 = to_float(bp[1]); b2 = to_float(bp[2]); b3 = to_float(bp[3]);
         }
-        run[g][0] = Mma<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
-        run[g][1] = Mma<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
+        run[g][0] = Mma32<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
+        run[g][1] = Mma32<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
       }
       uint4 piece[2];
       trade_channel_runs(run, piece);  // all lanes take part, also those of voxels past the edge

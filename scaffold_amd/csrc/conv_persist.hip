@@ -22,44 +22,14 @@
 #include <stdlib.h>
 
 #include "conv_mfma.hpp"
+#include "mma.hpp"
 
 namespace sfh {
 namespace {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t sfh_u32x2_t __attribute__((ext_vector_type(2)));
 
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
-};
-// The same MFMA with the row operand held in an accumulation register (inline asm: the compiler would otherwise
-// copy such a fragment into a vector register before every use).
-typedef int sfh_i32x4_t __attribute__((ext_vector_type(4)));
-template <typename T> struct MmaAcc;
-template <> struct MmaAcc<bf16_t> {
-  static __device__ __forceinline__ void run(const sfh_i32x4_t& a, const uint4& b, f32x16_t& c) {
-    const sfh_i32x4_t bv = __builtin_bit_cast(sfh_i32x4_t, b);
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
-  }
-};
-template <> struct MmaAcc<fp16_t> {
-  static __device__ __forceinline__ void run(const sfh_i32x4_t& a, const uint4& b, f32x16_t& c) {
-    const sfh_i32x4_t bv = __builtin_bit_cast(sfh_i32x4_t, b);
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
-  }
-};
-template <> struct Mma<fp16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_fp16x2(lo, hi); }
-};
+typedef mma_frag_t sfh_i32x4_t;
 
 constexpr int plane_bytes(int voxels) {  // smallest size >= voxels*16 that is 64 modulo 256
   return ((voxels * 16 - 64 + 255) / 256) * 256 + 64;
@@ -232,8 +202,8 @@ __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const 
       float v[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) v[t] = BIAS ? acc[ms][4 * g + t] + bias[4 * g + t] : acc[ms][4 * g + t];
-      run[g][0] = Mma<T>::pack2(v[0], v[1]);
-      run[g][1] = Mma<T>::pack2(v[2], v[3]);
+      run[g][0] = Mma32<T>::pack2(v[0], v[1]);
+      run[g][1] = Mma32<T>::pack2(v[2], v[3]);
     }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
@@ -285,9 +255,9 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
 #pragma unroll
     for (int ms = 0; ms < C::MS; ++ms) {
       // a brick starts from zero: the first MFMA takes a zero addend instead of a clearing pass
-      if (it == 0) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
-      else if (it < C::NVEC) acc[ms] = Mma<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
-      else MmaAcc<T>::run(wa[it - C::NVEC], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      if (it == 0) acc[ms] = Mma32<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], zero);
+      else if (it < C::NVEC) acc[ms] = Mma32<T>::run(wq[it], aq[it % (ADEPTH + 1)][ms], acc[ms]);
+      else Mma32Pinned<T>::run_row_in_acc(wa[it - C::NVEC], aq[it % (ADEPTH + 1)][ms], acc[ms]);
       __builtin_amdgcn_sched_barrier(0);
       if (it + ADEPTH < C::NIT)
         aq[(it + ADEPTH) % (ADEPTH + 1)][ms] = *reinterpret_cast<const uint4*>(cur + lg.lbase[ms] + lds_off<C>(it + ADEPTH));

@@ -49,7 +49,7 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
-typedef int frag_t __attribute__((ext_vector_type(4)));  // one MFMA operand fragment of a lane (8 x 16 bit)
+typedef mma_frag_t frag_t;  // one MFMA operand fragment of a lane (8 x 16 bit)
 
 // LDS operand reads are issued as inline asm and waited for by hand (lgkmcnt): the compiler cannot tell which
 // direct-to-LDS loads in flight a ds_read depends on and would otherwise wait for all of them (vmcnt(0)) before the
@@ -61,21 +61,10 @@ __device__ __forceinline__ frag_t lds_read_frag(int addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET) : "memory");
   return v;
 }
-// The MFMA as inline asm with the accumulator pinned to accumulation registers: left to the compiler, the 256
+// The MFMAs are the inline-asm form with the accumulator pinned to accumulation registers: left to the compiler, the 256
 // accumulator values of a lane wander between the two register files around the loop and push the addresses the loop
 // needs out to scratch memory. An accumulator block is reused only every MS x NSUB MFMAs, so no wait states are needed
 // between them; the epilogue waits out the last ones by hand.
-template <typename T> struct MmaPinned;
-template <> struct MmaPinned<bf16_t> {
-  static __device__ __forceinline__ void run(const frag_t& w, const frag_t& x, f32x16_t& c) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(w), "v"(x));
-  }
-};
-template <> struct MmaPinned<fp16_t> {
-  static __device__ __forceinline__ void run(const frag_t& w, const frag_t& x, f32x16_t& c) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(w), "v"(x));
-  }
-};
 __device__ __forceinline__ void zero_pinned(f32x16_t& c) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -303,7 +292,7 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
         static_for<C::NM>([&](auto i_c) {
           constexpr int i = decltype(i_c)::value;
           constexpr int ms = i / C::NSUB, ns = i % C::NSUB;
-          MmaPinned<T>::run(b_cur[ns], a_cur[ms], acc[ms][ns]);
+          Mma32Pinned<T>::run(b_cur[ns], a_cur[ms], acc[ms][ns]);
           // reads [i * NREAD / NM, (i + 1) * NREAD / NM) of the next tap: the weight fragments first, then the activations
           static_for<(i + 1) * C::NREAD / C::NM - i * C::NREAD / C::NM>([&](auto q_c) {
             constexpr int r = i * C::NREAD / C::NM + decltype(q_c)::value;

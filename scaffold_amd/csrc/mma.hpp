@@ -26,6 +26,31 @@ template <> struct Mma32<fp16_t> {
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_fp16x2(lo, hi); }
 };
 
+// The same MFMA as inline asm: the accumulator pinned to accumulation registers and, in the first form, the row
+// operand read from accumulation registers too (the compiler would otherwise copy such a fragment into a vector
+// register before every use). The compiler does not know the result latency of an asm MFMA: an accumulator block
+// must not be read (by anything but another MFMA, a few instructions later) without a wait.
+typedef int mma_frag_t __attribute__((ext_vector_type(4)));  // one operand fragment of a lane (8 x 16 bit)
+template <typename T> struct Mma32Pinned;
+template <> struct Mma32Pinned<bf16_t> {
+  static __device__ __forceinline__ void run_row_in_acc(const mma_frag_t& a, const uint4& b, f32x16_t& c) {
+    const mma_frag_t bv = __builtin_bit_cast(mma_frag_t, b);
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
+  }
+  static __device__ __forceinline__ void run(const mma_frag_t& a, const mma_frag_t& b, f32x16_t& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+template <> struct Mma32Pinned<fp16_t> {
+  static __device__ __forceinline__ void run_row_in_acc(const mma_frag_t& a, const uint4& b, f32x16_t& c) {
+    const mma_frag_t bv = __builtin_bit_cast(mma_frag_t, b);
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(bv));
+  }
+  static __device__ __forceinline__ void run(const mma_frag_t& a, const mma_frag_t& b, f32x16_t& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+
 template <typename T>
 __device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<const uint4*>(p); }
 

@@ -22,26 +22,13 @@
 // walks the tiles of its K range; the next tile's operands are fetched into registers before the
 // current tile's MFMAs start, so global-memory latency is hidden behind the compute.
 #include "wgrad_mfma.hpp"
+#include "mma.hpp"
 #include "reduce.hpp"
 
 namespace sfh {
 namespace {
 
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  }
-};
-template <> struct Mma<fp16_t> {
-  static __device__ __forceinline__ f32x16_t run(const uint4& a, const uint4& b, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-  }
-};
 
 constexpr int kTargetWorkgroups = kComputeUnits;
 
@@ -153,22 +140,22 @@ __device__ __forceinline__ void wave_compute(const char* lds, int lane, int wave
     // first MFMA of this k-step, then the LDS reads of the next one, then the other six MFMAs: the wait for
     // this k-step's fragments comes before any younger read is in flight
     __builtin_amdgcn_sched_barrier(0);
-    acc[0] = Mma<T>::run(cur.af, cur.lo0, acc[0]);
+    acc[0] = Mma32<T>::run(cur.af, cur.lo0, acc[0]);
     __builtin_amdgcn_sched_barrier(0);
     KFrags nxt = cur;
     if (ks + 1 < C::NKS) nxt = load_frags<C>(gsrc, row0, row1, rowx, ks + 1);
     __builtin_amdgcn_sched_barrier(0);
-    acc[1] = Mma<T>::run(cur.af, shift_one(cur.lo0, cur.nx0), acc[1]);
-    acc[2] = Mma<T>::run(cur.af, make_uint4(cur.lo0.y, cur.lo0.z, cur.lo0.w, cur.nx0), acc[2]);
-    acc[3] = Mma<T>::run(cur.af, cur.lo1, acc[3]);
-    acc[4] = Mma<T>::run(cur.af, shift_one(cur.lo1, cur.nx1), acc[4]);
-    acc[5] = Mma<T>::run(cur.af, make_uint4(cur.lo1.y, cur.lo1.z, cur.lo1.w, cur.nx1), acc[5]);
+    acc[1] = Mma32<T>::run(cur.af, shift_one(cur.lo0, cur.nx0), acc[1]);
+    acc[2] = Mma32<T>::run(cur.af, make_uint4(cur.lo0.y, cur.lo0.z, cur.lo0.w, cur.nx0), acc[2]);
+    acc[3] = Mma32<T>::run(cur.af, cur.lo1, acc[3]);
+    acc[4] = Mma32<T>::run(cur.af, shift_one(cur.lo1, cur.nx1), acc[4]);
+    acc[5] = Mma32<T>::run(cur.af, make_uint4(cur.lo1.y, cur.lo1.z, cur.lo1.w, cur.nx1), acc[5]);
     uint4 fx;
     fx.x = next_dword ? cur.lox.y : __builtin_amdgcn_alignbit(cur.lox.y, cur.lox.x, shx);
     fx.y = next_dword ? cur.lox.z : __builtin_amdgcn_alignbit(cur.lox.z, cur.lox.y, shx);
     fx.z = next_dword ? cur.lox.w : __builtin_amdgcn_alignbit(cur.lox.w, cur.lox.z, shx);
     fx.w = next_dword ? cur.nxx : __builtin_amdgcn_alignbit(cur.nxx, cur.lox.w, shx);
-    acc[6] = Mma<T>::run(cur.af, fx, acc[6]);
+    acc[6] = Mma32<T>::run(cur.af, fx, acc[6]);
     __builtin_amdgcn_sched_barrier(0);
     cur = nxt;
   }

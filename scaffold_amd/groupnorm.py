@@ -238,28 +238,32 @@ def _(grad_out, input, weight, bias, mean, rstd, num_groups, activation):
     return d_input, d_weight, d_bias
 
 
-def _setup_context(ctx, inputs, output):
-    input, num_groups, weight, bias, eps, activation, out_dtype = inputs
-    _out, mean, rstd = output
-    ctx.mark_non_differentiable(mean, rstd)
-    ctx.save_for_backward(input, weight, bias, mean, rstd)
-    ctx.num_groups = num_groups
-    ctx.activation = activation
-    ctx.needs = (ctx.needs_input_grad[0], ctx.needs_input_grad[2], ctx.needs_input_grad[3])
+# Positions of the operator's arguments that can carry a gradient (the schema order of scaffold_gn::group_norm).
+_ARG_INPUT, _ARG_WEIGHT, _ARG_BIAS, _N_ARGS = 0, 2, 3, 7
 
 
-def _autograd_backward(ctx, grad_out, grad_mean, grad_rstd):
-    input, weight, bias, mean, rstd = ctx.saved_tensors
-    need_x, need_w, need_b = ctx.needs
-    if not (need_x or need_w or need_b):
-        return None, None, None, None, None, None, None
-    d_input, d_weight, d_bias = torch.ops.scaffold_gn.group_norm_backward(
-        grad_out, input, weight, bias, mean, rstd, ctx.num_groups, ctx.activation
-    )
-    return (d_input if need_x else None, None, d_weight if need_w else None, d_bias if need_b else None, None, None, None)
+def _remember_for_backward(ctx, inputs, output):
+    """What the backward launch reads: x, the affine parameters and the statistics the forward produced (they carry no
+    gradient of their own); which of the three gradients autograd asked for is kept per argument position."""
+    ctx.mark_non_differentiable(output[1], output[2])
+    ctx.save_for_backward(inputs[_ARG_INPUT], inputs[_ARG_WEIGHT], inputs[_ARG_BIAS], output[1], output[2])
+    ctx.gn_groups, ctx.gn_activation = inputs[1], inputs[5]
+    ctx.gn_wanted = tuple(pos for pos in (_ARG_INPUT, _ARG_WEIGHT, _ARG_BIAS) if ctx.needs_input_grad[pos])
 
 
-torch.library.register_autograd("scaffold_gn::group_norm", _autograd_backward, setup_context=_setup_context)
+def _gradients_through_the_op(ctx, grad_out, _grad_mean, _grad_rstd):
+    """One backward launch produces all three gradients; they are handed out at the positions that were asked for."""
+    grads = [None] * _N_ARGS
+    if ctx.gn_wanted:
+        x, gamma, beta, mean, rstd = ctx.saved_tensors
+        produced = torch.ops.scaffold_gn.group_norm_backward(grad_out, x, gamma, beta, mean, rstd, ctx.gn_groups, ctx.gn_activation)
+        for pos, grad in zip((_ARG_INPUT, _ARG_WEIGHT, _ARG_BIAS), produced):
+            if pos in ctx.gn_wanted:
+                grads[pos] = grad
+    return tuple(grads)
+
+
+torch.library.register_autograd("scaffold_gn::group_norm", _gradients_through_the_op, setup_context=_remember_for_backward)
 
 
 class _EagerGroupNormFn(torch.autograd.Function):
