@@ -568,6 +568,56 @@ def conv_counter_launches(device, reps=3):
     return done
 
 
+def operand_probe(device, iters=20):
+    """The same launches on operands of different bit activity: Gaussian (the bench's operands), Gaussian through a
+    ReLU (what a convolution after GroupNorm + ReLU reads), all ones, all zeros. The matrix pipe's sustained rate on this
+    chip follows the power its operands draw, so the distance between the Gaussian and the all-zero figure of one kernel
+    is the part of its distance to the peak that no instruction schedule can recover; the vendor GEMM is timed the same
+    way beside it."""
+    import scaffold_amd as sa
+
+    def make(kind, shape, scale, gen):
+        if kind == "zeros":
+            return torch.zeros(shape)
+        if kind == "ones":
+            return torch.ones(shape)
+        t = torch.randn(shape, generator=gen) * scale
+        return t.clamp_min(0) if kind == "relu(gaussian)" else t
+
+    rows = []
+    for kind in ("gaussian", "relu(gaussian)", "ones", "zeros"):
+        for cin, cout, sp in ((32, 32, (128, 128, 128)), (128, 64, (64, 64, 64))):
+            g = torch.Generator().manual_seed(3000)
+            x = make(kind, (1, cin, *sp), 1.0, g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            w = make(kind, (cout, cin, 3, 3, 3), 1.0 / math.sqrt(cin * 27), g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            gy = make(kind, (1, cout, *sp), 1.0, g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+            pf, pd = sa.pack_weights(w, x.shape, 1, 1, 1)
+            y, gx = torch.empty_like(gy), torch.empty_like(x)
+            gw = torch.empty((cout, cin, 3, 3, 3), dtype=torch.float32, device=device).contiguous(memory_format=CL)
+            flops = 2 * math.prod(sp) * cin * cout * 27
+            fns = {"fwd": lambda: sa.conv3d_forward(x, w, None, 1, 1, 1, out=y, packed_weight=pf),
+                   "dgrad": lambda: sa.conv3d_backward_data(gy, w, x.shape, 1, 1, 1, out=gx, packed_weight=pd),
+                   "wgrad": lambda: sa.conv3d_backward_weight(x, w.shape, gy, 1, 1, 1, out=gw, grad_dtype=torch.float32)}
+            for direction, fn in fns.items():
+                fn()
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(10):
+                        fn()
+                ms = event_time_ms(graph.replay, max(2, iters // 10), warmup=2) / 10
+                rows.append({"operands": kind, "launch": f"conv3d {cin}->{cout} @{'x'.join(map(str, sp))} {direction}", "us": ms * 1e3,
+                             "tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS})
+        n = 8192
+        g = torch.Generator().manual_seed(4000)
+        a = make(kind, (n, n), 1.0, g).to(torch.bfloat16).to(device)
+        b = make(kind, (n, n), 1.0, g).to(torch.bfloat16).to(device)
+        ms = event_time_ms(lambda: torch.matmul(a, b), iters, warmup=5)
+        rows.append({"operands": kind, "launch": "torch.matmul 8192^3 bf16 (vendor GEMM)", "us": ms * 1e3,
+                     "tflops": 2 * n ** 3 / (ms * 1e-3) / 1e12, "frac": 2 * n ** 3 / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS})
+    return rows
+
+
 def cpu_baseline(with_unet=True):
     """The reference's CPU path for the hot path's three parts, timed on this box's host cores (bounded samples):
     the bench workload itself (torch conv3d + autograd, channels_last_3d bf16: what ScaFFold/unet/conv3d.py:1371-1378
@@ -686,6 +736,8 @@ def main():
                     help="run only the shard ingest kernel (200 launches) and print its time: the command to trace for it")
     ap.add_argument("--conv-table", action="store_true",
                     help="run only the per-shape table of the MFMA convolution launches (config 3 / 4 / 5 shapes, all directions)")
+    ap.add_argument("--operand-probe", action="store_true",
+                    help="run only the convolution launches and the vendor GEMM on Gaussian / rectified / constant operands")
     ap.add_argument("--conv-counters", action="store_true",
                     help="run only a few plain launches of the three MFMA convolution kernels: the command for counter runs")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -711,6 +763,12 @@ def main():
         return
     if args.conv_counters:
         print(json.dumps({"conv_counter_launches": conv_counter_launches(device)}))
+        return
+    if args.operand_probe:
+        rows = operand_probe(device)
+        for r in rows:
+            print(f"{r['operands']:15s} {r['launch']:42s} {r['us']:8.1f} us {r['tflops']:7.1f} TFLOP/s {r['frac']:.3f}", file=sys.stderr)
+        print(json.dumps({"operand_probe": rows}))
         return
     if args.unet_profile:
         print(json.dumps({"unet_step_cfg5": bench_unet_step(args, device, eager_only=True)}))

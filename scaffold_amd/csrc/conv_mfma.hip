@@ -166,22 +166,29 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     for (int ms = 0; ms < C::MS; ++ms) aq[0][ms] = *reinterpret_cast<const uint4*>(lds + lbase[ms] + lds_off<C>(0));
 #pragma unroll
     for (int it = 0; it < NIT; ++it) {
-      if (it + WDEPTH < NIT) {
-#pragma unroll
-        for (int ns = 0; ns < C::NSUB; ++ns)
-          wq[it + WDEPTH][ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + (it + WDEPTH) * FRAG);
-      }
-      if (it + 1 < NIT) {
-#pragma unroll
-        for (int ms = 0; ms < C::MS; ++ms)
-          aq[(it + 1) & 1][ms] = *reinterpret_cast<const uint4*>(lds + lbase[ms] + lds_off<C>(it + 1));
-      }
+      // The requests of later iterations -- the weight fragments of iteration it + WDEPTH, the activation fragments of
+      // iteration it + 1 -- are issued BETWEEN this iteration's MFMAs, one behind each: a load issued while the matrix
+      // pipe is busy costs nothing, a block of them in front of the MFMAs leaves the pipe idle while they issue.
+      constexpr int NM = C::MS * C::NSUB;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ms = 0; ms < C::MS; ++ms)
+      for (int m = 0; m < NM; ++m) {
+        const int ms = m / C::NSUB, ns = m % C::NSUB;
+        acc[ms][ns] = Mma32<T>::run(wq[it][ns], aq[it & 1][ms], acc[ms][ns]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (m < C::NSUB) {
+          if (it + WDEPTH < NIT) wq[it + WDEPTH][m] = *reinterpret_cast<const uint4*>(wcc + m * wns + (it + WDEPTH) * FRAG);
+        } else if (m - C::NSUB < C::MS) {
+          if (it + 1 < NIT) aq[(it + 1) & 1][m - C::NSUB] = *reinterpret_cast<const uint4*>(lds + lbase[m - C::NSUB] + lds_off<C>(it + 1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (C::MS + C::NSUB > NM) {  // more requests than MFMAs (one channel block per workgroup): the rest behind the last
 #pragma unroll
-        for (int ns = 0; ns < C::NSUB; ++ns) acc[ms][ns] = Mma32<T>::run(wq[it][ns], aq[it & 1][ms], acc[ms][ns]);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int k = NM - C::NSUB; k < C::MS; ++k)
+          if (it + 1 < NIT) aq[(it + 1) & 1][k] = *reinterpret_cast<const uint4*>(lds + lbase[k] + lds_off<C>(it + 1));
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 
