@@ -92,6 +92,20 @@ int sfh_conv3d_out_shape(const sfh_conv3d_desc* p, int32_t out_dhw[3]);
  * (3x3x3, stride 1, channel counts multiples of 16 / 32) on the fp32 matrix pipe with fp32 operands and
  * products, the precision the reference asks of its fp32 path (gather_gemm.py:1334, "ieee"). */
 int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
+/* Which kernel serves a problem in a direction (0 forward, 1 data-gradient, 2 weight-gradient) and with what launch
+ * geometry: geometry[0] = SFH_KERNEL_*, [1] = output voxels per workgroup step, [2] = 32-channel output blocks a
+ * workgroup produces from one staged brick, [3] = slices of the reduction (channels for forward / data-gradient,
+ * voxels for the weight gradient) whose fp32 partials are summed in fixed order. A pure function of the problem and
+ * the compute-unit count the library is written for -- the property the reference's plan machinery exists to
+ * guarantee (triton_conv3d/_rungs.py, reduce_gemm.py:71-96: the split count must not depend on the device or the
+ * run). [1] and [2] are 0 for SFH_KERNEL_DIRECT and SFH_KERNEL_OTHER_MATRIX (thin-channel, 2x2x2, fp32 tiles). */
+#define SFH_KERNEL_DIRECT 0
+#define SFH_KERNEL_PERSIST 1
+#define SFH_KERNEL_BRICK 2
+#define SFH_KERNEL_WIDE 3
+#define SFH_KERNEL_WGRAD 4
+#define SFH_KERNEL_OTHER_MATRIX 5
+int sfh_conv3d_launch_geometry(const sfh_conv3d_desc* p, int dtype, int direction, int32_t geometry[4]);
 
 /* ---- conv3d forward ------------------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_forward (triton_conv3d/gather_gemm.py:1187) and its

@@ -108,6 +108,7 @@ _SIGNATURES = {
     "sfh_tuned_compute_units": (c_int, []),
     "sfh_conv3d_out_shape": (c_int, [POINTER(ConvDesc), POINTER(c_int32)]),
     "sfh_conv3d_uses_mfma": (c_int, [POINTER(ConvDesc), c_int, c_int]),
+    "sfh_conv3d_launch_geometry": (c_int, [POINTER(ConvDesc), c_int, c_int, POINTER(c_int32)]),
     "sfh_conv3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_fwd": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                c_void_p, c_size_t, c_uint32, c_void_p]),
@@ -242,8 +243,19 @@ def _note_device(device: torch.device) -> None:
                       f"{units.value}: results are unaffected, launch shapes are not the best ones for it", RuntimeWarning, stacklevel=3)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device: torch.device) -> int:
-    _note_device(device)
+    """The HIP stream handle torch is issuing work to on ``device`` (one C call where torch offers the raw query;
+    a ``torch.cuda.Stream`` object per launch costs several microseconds, which a step of a few hundred launches feels)."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _devices_seen:
+        _note_device(device)
+    if _raw_stream is not None:
+        return int(_raw_stream(index))
     return int(torch.cuda.current_stream(device).cuda_stream)
 
 

@@ -327,6 +327,23 @@ def uses_mfma(in_shape, weight_shape, stride, padding, dilation, dtype, directio
     return bool(_lib.lib().sfh_conv3d_uses_mfma(ctypes.byref(desc), _lib.dtype_code(dtype), code))
 
 
+KERNEL_NAMES = ("direct", "persist", "brick", "wide", "wgrad", "other-matrix")
+
+
+def launch_geometry(in_shape, weight_shape, stride, padding, dilation, dtype, direction: str = "fwd") -> dict:
+    """Which kernel serves a problem and with what launch geometry: ``{"kernel", "voxels", "blocks", "slices"}`` (the
+    kernel by name; output voxels per workgroup step; 32-channel output blocks per workgroup; slices of the reduction whose
+    fp32 partials are summed in fixed order). A pure function of the problem, never of the device or the run."""
+    s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
+    n, cin, *in_sp = (int(v) for v in in_shape)
+    cout, _, *k = (int(v) for v in weight_shape)
+    desc = _desc(n, cin, in_sp, cout, k, s, p, d)
+    code = {"fwd": 0, "bwd-data": 1, "bwd-weight": 2}[direction]
+    geom = (ctypes.c_int32 * 4)()
+    _lib.check(_lib.lib().sfh_conv3d_launch_geometry(ctypes.byref(desc), _lib.dtype_code(dtype), code, geom), "launch_geometry")
+    return {"kernel": KERNEL_NAMES[geom[0]], "voxels": int(geom[1]), "blocks": int(geom[2]), "slices": int(geom[3])}
+
+
 def split_count(in_shape, weight_shape, stride, padding, dilation, dtype) -> int:
     """Number of fp32 partial slices the weight gradient reduces (1 = no workspace)."""
     s, p, d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")

@@ -312,6 +312,26 @@ extern "C" int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int dir
   return (wgrad_uses_mfma(*p, dtype, out) || wgrad_uses_patch(*p, dtype, out) || wgrad_uses_f32_tiles(*p, dtype, out)) ? 1 : 0;
 }
 
+extern "C" int sfh_conv3d_launch_geometry(const sfh_conv3d_desc* p, int dtype, int direction, int32_t geometry[4]) {
+  if (geometry == nullptr) return fail(SFH_ERR_INVALID, "conv3d geometry: null output");
+  geometry[0] = SFH_KERNEL_DIRECT; geometry[1] = geometry[2] = 0; geometry[3] = 1;
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (direction < 0 || direction > 2) return fail(SFH_ERR_INVALID, "conv3d geometry: direction %d", direction);
+  if (!sfh_conv3d_uses_mfma(p, dtype, direction)) return SFH_OK;
+  geometry[0] = SFH_KERNEL_OTHER_MATRIX;
+  if (direction == 2) {
+    if (!wgrad_uses_mfma(*p, dtype, out)) return SFH_OK;
+    geometry[0] = SFH_KERNEL_WGRAD; geometry[1] = 256; geometry[2] = 1;
+    geometry[3] = mfma_wgrad_splits(wgrad_args(*p, out));
+    return SFH_OK;
+  }
+  if (direction == 0 ? !fwd_uses_mfma(*p, dtype, out) : !dgrad_uses_mfma(*p, dtype, out)) return SFH_OK;
+  const MfmaConvGeometry g = mfma_conv_geometry(direction == 0 ? fwd_mfma_args(*p, out) : dgrad_mfma_args(*p, out));
+  geometry[0] = g.kernel; geometry[1] = g.voxels; geometry[2] = g.blocks; geometry[3] = g.slices;
+  return SFH_OK;
+}
+
 // ---- forward ---------------------------------------------------------------------------
 extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];

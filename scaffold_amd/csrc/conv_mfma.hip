@@ -23,6 +23,10 @@
 // The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
 // padding k-1-p (triton_conv3d/bwd_data.py:344-363).
 #include "conv_mfma.hpp"
+#ifdef SFH_GATHER_TUNE
+#include <cstdio>
+#include <cstdlib>
+#endif
 #include "mma.hpp"
 #include "reduce.hpp"
 
@@ -109,6 +113,23 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 
   const int cc_begin = (int)((int64_t)ksp * ncc / ksplit), cc_end = (int)((int64_t)(ksp + 1) * ncc / ksplit);
   for (int cc = cc_begin; cc < cc_end; ++cc) {
+    // The first weight fragments of this chunk are requested before its brick is staged (one output block per
+    // workgroup; with two the staging needs the registers): they depend on nothing in LDS, and a chunk whose weights
+    // come from HBM (every chunk, each time a training step reaches the layer) would otherwise start its MFMAs one
+    // memory round trip late.
+    const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
+    const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
+    constexpr int NIT = C::TAPS * 2;
+    // Weight fragments in flight per wavefront. A fragment feeds MS x NSUB MFMAs (32 cycles each): the fewer those are,
+    // the more fragments must be under way to cover a trip to L2 or HBM.
+    constexpr int WWANT = C::NSUB > 1 ? 4 : (C::MS >= 4 ? 6 : 12);
+    constexpr int WDEPTH = NIT < WWANT ? NIT : WWANT;
+    uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
+    constexpr bool EARLY_WEIGHTS = C::NSUB == 1;  // with two output blocks the staging needs the registers
+    if constexpr (EARLY_WEIGHTS) {
+#pragma unroll
+      for (int it = 0; it < WDEPTH; ++it) wq[it][0] = *reinterpret_cast<const uint4*>(wcc + it * FRAG);
+    }
     __syncthreads();  // every wave is done reading the previous chunk
     {
       const T* xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cred + cc * kChunk;
@@ -152,16 +173,13 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     // Software pipeline over the TAPS*2 (tap, k-step) iterations of this chunk: the weight fragment
     // of iteration it+WDEPTH and the activation fragments of iteration it+1 are requested before the
     // MFMAs of iteration it are issued, so L2 and LDS latency overlap the matrix pipe.
-    const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
-    const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
-    constexpr int NIT = C::TAPS * 2;
-    constexpr int WDEPTH = NIT < 6 ? NIT : (C::NSUB > 1 ? 4 : 6);
-    uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
     uint4 aq[2][C::MS];
+    if constexpr (!EARLY_WEIGHTS) {
 #pragma unroll
-    for (int it = 0; it < WDEPTH; ++it)
+      for (int it = 0; it < WDEPTH; ++it)
 #pragma unroll
-      for (int ns = 0; ns < C::NSUB; ++ns) wq[it][ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + it * FRAG);
+        for (int ns = 0; ns < C::NSUB; ++ns) wq[it][ns] = *reinterpret_cast<const uint4*>(wcc + ns * wns + it * FRAG);
+    }
 #pragma unroll
     for (int ms = 0; ms < C::MS; ++ms) aq[0][ms] = *reinterpret_cast<const uint4*>(lds + lbase[ms] + lds_off<C>(0));
 #pragma unroll
@@ -307,24 +325,61 @@ __global__ void __launch_bounds__(256) pack_weight_batch_kernel(PackBatch b) {
 
 struct GatherPlan { int shape; int nsub; int ksplit; int64_t tiles; };
 
-// Launch geometry, a pure function of the problem: brick shape by row length; two output blocks per workgroup
-// when that still fills the chip, else one; and when even that leaves CUs idle (the deep, small-volume levels)
-// the reduction channels are cut into slices that are summed afterwards (one workgroup per CU: more slices cost more
-// in fp32 partials than the second resident workgroup gains).
+// Brick shapes: the row-length class (32-, 16- or 8-voxel rows) times the tile size (512, 256 or 128 output voxels).
+constexpr int kTileDims[3][3][3] = {
+    {{4, 4, 32}, {2, 4, 32}, {1, 4, 32}},
+    {{4, 8, 16}, {2, 8, 16}, {1, 8, 16}},
+    {{8, 8, 8}, {4, 8, 8}, {2, 8, 8}},
+};
+
+int64_t tiles_of(const MfmaConvArgs& a, int cls, int size) {
+  const int* t = kTileDims[cls][size];
+  return (int64_t)a.n * cdiv(a.od, t[0]) * cdiv(a.oh, t[1]) * cdiv(a.ow, t[2]);
+}
+
+// Launch geometry, a pure function of the problem. The row length picks the brick's row class; then, among 512- and
+// 256-voxel tiles with one or two 32-channel output blocks per workgroup, the choice that loads the busiest CU least:
+// workgroups are dealt round-robin, so that CU gets ceil(workgroups / CUs) of them, each worth tile voxels x blocks.
+// A 256-voxel tile re-stages more halo per output voxel (weight 1.15), two blocks share one staged brick (0.97); both
+// weights are fitted to timings of every convolution shape of a five-level U-Net on whole cubes and on depth shards.
+// On the depth slab of a shard (D + 2 planes of data gradient) this is what keeps 288 half-empty second rounds of
+// 512-voxel tiles from costing a whole round. When even the small tiles leave CUs idle (the deep, small-volume levels)
+// the reduction channels are cut into at most 8 slices that are summed afterwards: a power of two, no more than would
+// give every CU a workgroup (more slices cost more in fp32 partials than they gain).
 GatherPlan gather_plan(const MfmaConvArgs& a) {
   GatherPlan p{};
-  int td, th, tw;
-  if (a.ow > 16) { p.shape = 0; td = 4; th = 4; tw = 32; }
-  else if (a.ow > 8) { p.shape = 1; td = 4; th = 8; tw = 16; }
-  else { p.shape = 2; td = 8; th = 8; tw = 8; }
-  p.tiles = (int64_t)a.n * cdiv(a.od, td) * cdiv(a.oh, th) * cdiv(a.ow, tw);
-  p.nsub = (a.cout % 64 == 0 && p.tiles * (a.cout / 64) >= kComputeUnits) ? 2 : 1;
-  p.ksplit = 1;
-  const int64_t wgs = p.tiles * (a.cout / (32 * p.nsub));
+  const int cls = a.ow > 16 ? 0 : (a.ow > 8 ? 1 : 2);
   const int ncc = a.cred / kChunk;
-  if (wgs < kComputeUnits && ncc > 1) {
-    int64_t k = cdiv(kComputeUnits, wgs);
-    p.ksplit = (int)(k < ncc ? k : ncc);
+#ifdef SFH_GATHER_TUNE
+  if (const char* e = getenv("SFH_GATHER_FORCE")) {
+    int size = 0, nsub = 1, ksplit = 1;
+    if (sscanf(e, "%d,%d,%d", &size, &nsub, &ksplit) == 3 && size >= 0 && size < 3 && (nsub == 1 || (nsub == 2 && a.cout % 64 == 0)) &&
+        ksplit >= 1 && ksplit <= ncc) {
+      p.shape = cls * 3 + size;
+      p.tiles = tiles_of(a, cls, size);
+      p.nsub = nsub;
+      p.ksplit = ksplit;
+      return p;
+    }
+  }
+#endif
+  int64_t best = -1, best_wgs = 0;
+  for (int size = 0; size < 2; ++size) {
+    const int* t = kTileDims[cls][size];
+    const int64_t tiles = tiles_of(a, cls, size), voxels = (int64_t)t[0] * t[1] * t[2];
+    for (int nsub = 1; nsub <= (a.cout % 64 == 0 ? 2 : 1); ++nsub) {
+      const int64_t wgs = tiles * (a.cout / (32 * nsub));
+      const int64_t cost = cdiv(wgs, kComputeUnits) * voxels * nsub * (size == 1 ? 115 : 100) * (nsub == 2 ? 97 : 100);
+      if (best < 0 || cost < best) {
+        best = cost; best_wgs = wgs;
+        p.shape = cls * 3 + size; p.tiles = tiles; p.nsub = nsub;
+      }
+    }
+  }
+  p.ksplit = 1;
+  if (best_wgs > 0 && best_wgs < kComputeUnits) {
+    const int64_t room = kComputeUnits / best_wgs;
+    while (p.ksplit * 2 <= room && p.ksplit * 2 <= ncc && p.ksplit < 8) p.ksplit *= 2;
   }
   return p;
 }
@@ -346,9 +401,20 @@ template <typename T, int NSUB>
 int launch_k333(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
                 float* partial, hipStream_t st) {
   // Brick shape follows the row length: 32-voxel sub-tiles are one, two or four W rows.
-  if (p.shape == 0) return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-  if (p.shape == 1) return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-  return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+  switch (p.shape) {
+    case 0: return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 3: return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 6: return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+#ifdef SFH_GATHER_TUNE  // 128-voxel tiles: built only to be measured
+    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+#endif
+    default: return fail(SFH_ERR_UNSUPPORTED, "conv mfma: no kernel for brick shape %d", p.shape);
+  }
 }
 
 template <typename T>
@@ -431,6 +497,13 @@ size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
   const GatherPlan p = gather_plan(a);
   if (a.cred == kChunk || p.ksplit == 1) return 0;
   return align_up((size_t)p.ksplit * a.n * a.od * a.oh * a.ow * a.cout * sizeof(float), 256);
+}
+
+MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a) {
+  if (mfma_conv_wide_applies(a)) return mfma_conv_wide_geometry(a);
+  const GatherPlan p = gather_plan(a);
+  const int* t = kTileDims[p.shape / 3][p.shape % 3];
+  return MfmaConvGeometry{kKernelBrick, t[0] * t[1] * t[2], p.nsub, p.ksplit};
 }
 
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,

@@ -43,4 +43,14 @@ int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* 
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st);
 
+// Which of the three kernels mfma_conv_persist ends up launching for a problem, and with what geometry: a pure function of
+// the shape. `voxels` is the output tile of a workgroup step, `blocks` the 32-channel output blocks a workgroup produces
+// from one staged brick, `slices` the cuts of the reduction channels (1: none, no partial workspace).
+enum MfmaConvKernel { kKernelPersist = 1, kKernelBrick = 2, kKernelWide = 3 };
+struct MfmaConvGeometry { int kernel, voxels, blocks, slices; };
+MfmaConvGeometry mfma_conv_geometry(const MfmaConvArgs& a);
+bool mfma_conv_persist_applies(const MfmaConvArgs& a);
+MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a);
+MfmaConvGeometry mfma_conv_wide_geometry(const MfmaConvArgs& a);
+
 }  // namespace sfh

@@ -426,15 +426,23 @@ int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const
 
 }  // namespace
 
+// The persistent kernel pays off when the weight slab stays in registers for the whole launch, i.e. with a
+// single 32-channel reduction chunk; wider reductions run the brick-per-workgroup kernel. A brick (at most
+// 10 x 10 input rows deep and high) must also span less than kRange bytes of the input, a tile (at most 8 x 8 output
+// rows) less than kRange bytes of the output.
+bool mfma_conv_persist_applies(const MfmaConvArgs& a) {
+  return a.cred == 32 && ((int64_t)10 * a.ih + 10) * a.iw * a.cred * 2 + 64 < kRange &&
+         ((int64_t)8 * a.oh + 8) * a.ow * a.cout * 2 + 64 < kRange;
+}
+
+MfmaConvGeometry mfma_conv_geometry(const MfmaConvArgs& a) {
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather_geometry(a);
+  return MfmaConvGeometry{kKernelPersist, 512, 1, 1};
+}
+
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st) {
-  // The persistent kernel pays off when the weight slab stays in registers for the whole launch, i.e. with a
-  // single 32-channel reduction chunk; wider reductions run the brick-per-workgroup kernel. A brick (at most
-  // 10 x 10 input rows deep and high) must also span less than kRange bytes of the input, a tile (at most 8 x 8 output
-  // rows) less than kRange bytes of the output.
-  if (a.cred != 32 || ((int64_t)10 * a.ih + 10) * a.iw * a.cred * 2 + 64 >= kRange ||
-      ((int64_t)8 * a.oh + 8) * a.ow * a.cout * 2 + 64 >= kRange)
-    return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st);
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st);
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st);
   return launch_typed<fp16_t>(a, x, packed, bias, y, st);
 }

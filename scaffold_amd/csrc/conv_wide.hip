@@ -422,6 +422,12 @@ int launch_typed(const MfmaConvArgs& a, const WidePlan& p, const void* x, const 
 
 bool mfma_conv_wide_applies(const MfmaConvArgs& a) { return wide_plan(a).use; }
 
+MfmaConvGeometry mfma_conv_wide_geometry(const MfmaConvArgs& a) {
+  static const int td[5] = {4, 8, 8, 4, 4}, nsub[5] = {4, 2, 1, 2, 1};
+  const WidePlan p = wide_plan(a);
+  return MfmaConvGeometry{kKernelWide, td[p.shape] * 4 * 32, nsub[p.shape], 1};
+}
+
 int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
   const WidePlan p = wide_plan(a);
   if (!p.use) return fail(SFH_ERR_UNSUPPORTED, "conv wide: not applicable to this problem");

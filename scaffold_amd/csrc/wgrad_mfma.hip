@@ -22,6 +22,9 @@
 // walks the tiles of its K range; the next tile's operands are fetched into registers before the
 // current tile's MFMAs start, so global-memory latency is hidden behind the compute.
 #include "wgrad_mfma.hpp"
+#ifdef SFH_WGRAD_TUNE
+#include <cstdlib>
+#endif
 #include "mma.hpp"
 #include "reduce.hpp"
 
@@ -397,11 +400,28 @@ Plan make_plan(const WgradArgs& a) {
   p.ntiles = a.n * p.tiles_d * p.tiles_h * p.tiles_w;
   p.nblk_ci = a.cin / 32;
   p.nblk = p.nblk_ci * (a.cout / 32);
-  int want = kTargetWorkgroups / p.nblk;
+  // Slices along the voxel range: at most one workgroup per CU; from there the count is halved while a cost estimate
+  // says that pays. A workgroup's time is its tiles (2.4 us each at this kernel's rate); every slice of every 32 x 32
+  // block is 108 KiB of fp32 that is written and, when there is more than one slice, read again by the ordered sum
+  // (a launch of its own). Units of 0.01 us, constants fitted to timings of the U-Net's levels: the small-volume
+  // levels (8 tiles for 64-128 blocks) are cheaper with 1-4 slices than with one per CU.
+  int target = kTargetWorkgroups;
+#ifdef SFH_WGRAD_TUNE
+  if (const char* e = getenv("SFH_WGRAD_WANT")) target = atoi(e) > 0 ? atoi(e) : target;
+#endif
+  int want = target / p.nblk;
   if (want < 1) want = 1;
   if (want > p.ntiles) want = p.ntiles;
-  p.tiles_per_split = (int)cdiv(p.ntiles, want);
-  p.splits = (int)cdiv(p.ntiles, p.tiles_per_split);
+  int64_t best = -1;
+  for (int s = want; s >= 1; s /= 2) {
+    const int tps = (int)cdiv(p.ntiles, s), eff = (int)cdiv(p.ntiles, tps);
+    const int64_t cost = eff > 1 ? 240LL * tps + 1000 + 64LL * eff * p.nblk / 10 : 240LL * tps + 600 + 32LL * p.nblk / 10;
+    if (best < 0 || cost < best) {
+      best = cost;
+      p.tiles_per_split = tps;
+      p.splits = eff;
+    }
+  }
   return p;
 }
 

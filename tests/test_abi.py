@@ -76,6 +76,43 @@ def test_kernel_selection_is_a_pure_function_of_the_problem():
     assert L.sfh_conv3d_wgrad_splits(ctypes.byref(conv_desc(cin=8)), fp32) == 1                         # untiled: one pass, no slices
 
 
+def test_launch_geometry_is_stated_and_agrees_with_the_workspace():
+    """The geometry query names the kernel and its tile / block / slice counts; the workspace sizes follow from it."""
+    L = _lib.lib()
+    bf16, fp32 = 0, 2
+
+    def geometry(desc, dtype, direction):
+        out = (ctypes.c_int32 * 4)()
+        assert L.sfh_conv3d_launch_geometry(ctypes.byref(desc), dtype, direction, out) == 0
+        assert list(out) == list(geometry_again(desc, dtype, direction))
+        return list(out)
+
+    def geometry_again(desc, dtype, direction):
+        out = (ctypes.c_int32 * 4)()
+        L.sfh_conv3d_launch_geometry(ctypes.byref(desc), dtype, direction, out)
+        return out
+
+    DIRECT, PERSIST, BRICK, WIDE, WGRAD, OTHER = range(6)
+    cube = conv_desc(sp=(128, 128, 128))
+    assert geometry(cube, bf16, 0) == [PERSIST, 512, 1, 1] and geometry(cube, bf16, 1) == [PERSIST, 512, 1, 1]
+    assert geometry(cube, bf16, 2) == [WGRAD, 256, 1, L.sfh_conv3d_wgrad_splits(ctypes.byref(cube), bf16)]
+    assert geometry(cube, fp32, 0)[0] == OTHER and geometry(conv_desc(cin=3), bf16, 0)[0] == DIRECT
+    assert geometry(conv_desc(cin=128, cout=64, sp=(64, 64, 64)), bf16, 0) == [WIDE, 1024, 2, 1]
+    # the data gradient of a depth shard's slab (D + 2 planes): 256-voxel tiles, or a ninth of the workgroups would run a
+    # round of their own
+    assert geometry(conv_desc(cin=64, cout=64, sp=(34, 64, 64), p=(0, 1, 1)), bf16, 1) == [BRICK, 256, 1, 1]
+    assert geometry(conv_desc(cin=64, cout=64, sp=(64, 64, 64)), bf16, 0) == [BRICK, 512, 2, 1]
+    # a deep, small-volume level: the reduction channels are cut into slices, and the workspace holds their fp32 partials
+    deep = conv_desc(cin=256, cout=256, sp=(10, 16, 16), p=(0, 1, 1))
+    kernel, voxels, blocks, slices = geometry(deep, bf16, 0)
+    assert (kernel, voxels, blocks) == (BRICK, 256, 1) and 1 < slices <= 8 and slices & (slices - 1) == 0
+    packed = 256 * 256 * 27 * 2
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(deep), bf16) == packed + slices * 8 * 16 * 16 * 256 * 4
+    out = (ctypes.c_int32 * 4)()
+    assert L.sfh_conv3d_launch_geometry(ctypes.byref(cube), bf16, 3, out) == _lib.SFH_ERR_INVALID
+    assert L.sfh_conv3d_launch_geometry(ctypes.byref(cube), bf16, 0, None) == _lib.SFH_ERR_INVALID
+
+
 def test_wgrad_split_plan_partitions_the_bricks():
     """Every brick belongs to exactly one split: splits * ceil(bricks / splits) covers, (splits-1) * that does not."""
     L = _lib.lib()

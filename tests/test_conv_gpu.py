@@ -94,6 +94,35 @@ def test_mfma_exact(device, dtype, cin, cout, spatial, padding, direction):
         assert got.is_contiguous(memory_format=torch.channels_last_3d) or got.shape[2:] == (1, 1, 1)
 
 
+# The brick-per-workgroup kernel's launch geometry is picked by a cost rule (512- or 256-voxel tiles of the row class,
+# one or two 32-channel output blocks per workgroup, slices of the reduction channels on small volumes). One case per
+# tile shape and block count, with the geometry the rule must give for it, so that no instantiation goes untested and a
+# change of the rule shows up here.
+GEOMETRY_CASES = [
+    # (n, cin, cout, spatial, direction, voxels, blocks)
+    (1, 64, 128, (32, 32, 32), "fwd", 512, 1),        # rows of 32: 4 x 4 x 32
+    (1, 64, 128, (32, 64, 32), "fwd", 512, 2),
+    (1, 64, 128, (32, 32, 32), "bwd-data", 256, 1),   # 2 x 4 x 32
+    (1, 64, 128, (2, 128, 128), "fwd", 256, 2),
+    (1, 64, 512, (16, 32, 16), "fwd", 512, 1),        # rows of 16: 4 x 8 x 16
+    (1, 64, 256, (32, 64, 16), "fwd", 512, 2),
+    (1, 64, 64, (4, 8, 16), "fwd", 256, 1),           # 2 x 8 x 16
+    (4, 64, 256, (2, 128, 16), "fwd", 256, 2),
+    (1, 64, 512, (32, 32, 8), "fwd", 512, 1),         # rows of 8: 8 x 8 x 8
+    (1, 64, 256, (64, 64, 8), "fwd", 512, 2),
+    (1, 128, 64, (4, 8, 8), "fwd", 256, 1),           # 4 x 8 x 8
+    (4, 64, 256, (4, 128, 8), "fwd", 256, 2),
+]
+
+
+@pytest.mark.parametrize("n,cin,cout,spatial,direction,voxels,blocks", GEOMETRY_CASES)
+def test_brick_geometries_exact(device, n, cin, cout, spatial, direction, voxels, blocks):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=(1, 1, 1), dtype=torch.bfloat16)
+    geom = c3.launch_geometry(prob.input_shape, prob.weight_shape, 1, (1, 1, 1), 1, torch.bfloat16, direction)
+    assert (geom["kernel"], geom["voxels"], geom["blocks"]) == ("brick", voxels, blocks), geom
+    check_exact(prob, direction, device)
+
+
 # Shapes only the direct kernels serve: odd channel counts, strides, dilation, other kernel sizes,
 # fp32 (``triton_conv3d/shapes.py:611-684`` edge list).
 DIRECT_SHAPES = [
