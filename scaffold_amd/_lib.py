@@ -112,6 +112,9 @@ _SIGNATURES = {
     "sfh_conv3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_fwd": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_fwd_gn_records": (c_int32, [POINTER(ConvDesc), c_int, c_int]),
+    "sfh_conv3d_fwd_gn": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
+                                  c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_size_t, c_void_p]),
     "sfh_conv3d_dgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_dgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                  c_size_t, c_uint32, c_void_p]),
@@ -136,6 +139,8 @@ _SIGNATURES = {
     "sfh_skip_concat_bwd": (c_int, [POINTER(ConcatDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_groupnorm_fwd_slab": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "sfh_groupnorm_fwd_from_partials": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                                c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
     "sfh_groupnorm_bwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
     "sfh_groupnorm_bwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -284,12 +289,16 @@ def device_guard(device: torch.device):
 
 
 def _meta(v):
-    """Everything a gate may look at, as a hashable value: tensors by their metadata, sequences as tuples."""
+    """Everything a gate may look at, as a hashable value: tensors by their metadata, sequences as tuples. The common
+    argument kinds are told apart by exact type first: a gate runs in front of every launch."""
+    t = type(v)
+    if t is int or v is None:
+        return v
+    if t is tuple or t is list:
+        return tuple([e if type(e) is int else _meta(e) for e in v])
     if isinstance(v, torch.Tensor):
         return (torch.Tensor, v.shape, v.dtype, v.device, v.stride(), v.layout)
-    if isinstance(v, (list, tuple)):
-        return tuple(_meta(e) for e in v)
-    return (type(v), v)
+    return (t, v)
 
 
 def memoized_gate(fn):
@@ -299,7 +308,7 @@ def memoized_gate(fn):
 
     def wrapper(*args, **kwargs):
         try:
-            key = (tuple(_meta(a) for a in args), tuple((k, _meta(v)) for k, v in kwargs.items()),
+            key = (tuple([_meta(a) for a in args]), tuple([(k, _meta(v)) for k, v in kwargs.items()]) if kwargs else (),
                    torch.is_autocast_enabled("cuda"))
             hit = cache.get(key)
         except Exception:

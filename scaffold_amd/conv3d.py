@@ -96,7 +96,7 @@ class _Problem:
     """Everything about one convolution problem that does not depend on the tensors: parsed geometry, the descriptor
     the library takes, and (filled on first use) the workspace bytes of each direction."""
 
-    __slots__ = ("s", "p", "d", "k", "n", "cin", "in_sp", "cout", "y_shape", "desc", "code", "need", "packed")
+    __slots__ = ("s", "p", "d", "k", "n", "cin", "in_sp", "cout", "y_shape", "desc", "code", "need", "packed", "gn")
 
     def __init__(self, in_shape, w_shape, stride, padding, dilation, dtype):
         self.s, self.p, self.d = _triple(stride, "stride"), _triple(padding, "padding"), _triple(dilation, "dilation")
@@ -109,6 +109,14 @@ class _Problem:
         self.code = _lib.dtype_code(dtype)
         self.need = {}
         self.packed = None
+        self.gn = {}
+
+    def gn_records(self, groups: int) -> int:
+        """Records of GroupNorm partial sums per sample the forward launch leaves for ``groups`` groups (0: not offered)."""
+        rec = self.gn.get(groups)
+        if rec is None:
+            rec = self.gn[groups] = int(_lib.lib().sfh_conv3d_fwd_gn_records(ctypes.byref(self.desc), self.code, int(groups)))
+        return rec
 
     def packed_bytes(self, backward_data: bool) -> int:
         """Bytes of the packed weight this direction of the problem reads (0: it reads the weight where it lies)."""
@@ -559,6 +567,7 @@ def conv3d_forward(
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
     packed_weight: Optional[torch.Tensor] = None,
+    gn_groups: int = 0,
     _checked: bool = False,
 ) -> torch.Tensor:
     """Forward 3-D convolution; input and output are ``channels_last_3d``.
@@ -567,6 +576,11 @@ def conv3d_forward(
     ``channels_last_3d`` parameter, PyTorch's default layout and an RSCK copy all work without
     a host-side transform and give bitwise identical results.  ``weight_flip`` consumes the
     taps mirrored in all three axes (the data gradient's view of the weight).
+
+    ``gn_groups > 0`` announces a GroupNorm of that many groups on the result: where the kernel that serves the problem
+    offers it, the launch also leaves the per-group sums of its (rounded) output, which ride along as
+    ``result._sfh_gn_partials`` and spare :func:`scaffold_amd.group_norm` its statistics pass. The result itself is the
+    same bits either way.
     """
     if not _checked and not is_supported(x, w, bias, stride, padding, dilation, groups):
         raise NotImplementedError(
@@ -603,9 +617,19 @@ def conv3d_forward(
             flags |= _lib.SFH_FLAG_WEIGHT_PACKED
             w_eff = packed_weight
         ws = _lib.workspace(need, x.device)
-        rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
-                              None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
-                              _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(x.device))
+        records = prob.gn_records(gn_groups) if gn_groups > 0 and not force_generic else 0
+        if records > 0:
+            partials = torch.empty(prob.n * records * 2 * gn_groups, dtype=torch.float32, device=x.device)
+            rc = L.sfh_conv3d_fwd_gn(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
+                                     None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                                     _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
+                                     _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+            # valid for these bits of y only: the version lets the consumer see an in-place change
+            y._sfh_gn_partials = (partials, records, int(gn_groups), y._version)
+        else:
+            rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
+                                  None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                                  _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(x.device))
     _lib.check(rc, "conv3d_forward")
     return y
 

@@ -342,8 +342,9 @@ extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int d
   return mfma_conv_packed_weight_bytes(fwd_mfma_args(*p, out)) + mfma_conv_partial_bytes(fwd_mfma_args(*p, out));
 }
 
-extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
-                              const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                          const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream,
+                          const GnPartialOut* gn) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (x == nullptr || w == nullptr || y == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
@@ -356,7 +357,7 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
     if (flags & SFH_FLAG_WEIGHT_PACKED) {  // w is the packed weight; the workspace only holds the partial slices
       if (partial_bytes && (workspace == nullptr || workspace_bytes < partial_bytes))
         return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", partial_bytes, workspace_bytes);
-      return mfma_conv_persist(a, dtype, x, w, bias, y, partial_bytes ? workspace : nullptr, st);
+      return mfma_conv_persist(a, dtype, x, w, bias, y, partial_bytes ? workspace : nullptr, st, gn);
     }
     const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
@@ -364,8 +365,9 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
-    return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st);
+    return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st, gn);
   }
+  if (gn != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
   if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && fwd_uses_f32_tiles(*p, dtype, out)) {
     const MfmaConvArgs a = fwd_mfma_args(*p, out);
     const size_t need = f32_conv_packed_weight_bytes(a);
@@ -407,6 +409,31 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
   a.flip = 0;
   a.ws_co = w_stride[0]; a.ws_ci = w_stride[1]; a.ws_kd = w_stride[2]; a.ws_kh = w_stride[3]; a.ws_kw = w_stride[4];
   return direct_conv_gather(a, dtype, x, w, bias, y, st);
+}
+
+extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                              const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  return conv3d_fwd_any(p, dtype, x, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, nullptr);
+}
+
+extern "C" int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype, int groups) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK || groups < 1 || p->n == 0) return 0;
+  if (!fwd_uses_mfma(*p, dtype, out)) return 0;
+  return mfma_conv_gn_records(fwd_mfma_args(*p, out), groups);
+}
+
+extern "C" int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                                 const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, int groups,
+                                 float* gn_partials, size_t gn_partials_bytes, void* stream) {
+  if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d fwd: the direct kernels leave no GroupNorm partials");
+  const int32_t records = sfh_conv3d_fwd_gn_records(p, dtype, groups);
+  if (records == 0) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
+  const size_t need = (size_t)p->n * records * 2 * groups * sizeof(float);
+  if (gn_partials == nullptr || gn_partials_bytes < need || (reinterpret_cast<uintptr_t>(gn_partials) & 15u) != 0)
+    return fail(SFH_ERR_WORKSPACE, "conv3d fwd: GroupNorm partials need %zu bytes at a 16-byte boundary, got %zu", need, gn_partials_bytes);
+  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records};
+  return conv3d_fwd_any(p, dtype, x, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, &gn);
 }
 
 // ---- packing a weight once for both directions ------------------------------------------------

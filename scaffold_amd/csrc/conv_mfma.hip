@@ -28,6 +28,7 @@
 #include <cstdlib>
 #endif
 #include "mma.hpp"
+#include "gn_stats.hpp"
 #include "reduce.hpp"
 
 namespace sfh {
@@ -71,7 +72,7 @@ template <typename T, typename C>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
                  T* __restrict__ y, float* __restrict__ partial, int tiles_d, int tiles_h, int tiles_w, int nblocks, int ksplit,
-                 uint32_t total) {
+                 uint32_t total, GnPartialOut gn) {
   __shared__ __attribute__((aligned(16))) char lds[C::LDS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -210,6 +211,11 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     }
   }
 
+  // GroupNorm statistics of the rounded output, when the caller wants them (the reduction is not sliced then).
+  RunSums gn_sums[C::NSUB];
+#pragma unroll
+  for (int ns = 0; ns < C::NSUB; ++ns) gn_sums[ns].clear();
+
   // Epilogue. Accumulator register r of a lane is output channel 8*(r/4) + 4*kg + r%4 of the
   // sub-tile's voxel j: four runs of four consecutive channels per 32-channel block. For the 16-bit output the two
   // lanes of a voxel trade runs so that each stores two 16-byte pieces (32 contiguous bytes of a voxel per store
@@ -248,6 +254,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
         run[g][0] = Mma32<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
         run[g][1] = Mma32<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
       }
+      if (gn.part != nullptr) gn_sums[ns].template add<T>(run, inside);
       uint4 piece[2];
       trade_channel_runs(run, piece);  // all lanes take part, also those of voxels past the edge
       if (inside) {
@@ -255,6 +262,13 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
         *reinterpret_cast<uint4*>(yp + ns * 32 + 16 + 8 * kg) = piece[1];
       }
     }
+  }
+  if (gn.part != nullptr && ksplit == 1) {
+    __syncthreads();  // every wave is done reading the brick: the LDS is free
+    constexpr int SPAN = 32 * C::NSUB;
+    const int per_tile = gn.cg > SPAN ? gn.cg / SPAN : 1;  // workgroups that share a group of this tile
+    const int tile = (td_i * tiles_h + th_i) * tiles_w + tw_i;
+    write_group_partials<4, C::NSUB>(gn_sums, reinterpret_cast<float*>(lds), gn, n, tile * per_tile + nb % per_tile, nb * SPAN, tid);
   }
 }
 
@@ -386,46 +400,68 @@ GatherPlan gather_plan(const MfmaConvArgs& a) {
 
 template <typename T, typename C>
 int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
-               float* partial, hipStream_t st) {
+               float* partial, hipStream_t st, const GnPartialOut& gn) {
   const int tiles_d = (int)cdiv(a.od, C::TD), tiles_h = (int)cdiv(a.oh, C::TH), tiles_w = (int)cdiv(a.ow, C::TW);
   const int nblocks = a.cout / (32 * C::NSUB);
   const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks * p.ksplit;
   if (total == 0) return SFH_OK;
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: %lld workgroups exceed the grid limit", (long long)total);
   hipLaunchKernelGGL((conv_mfma_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
-                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total);
+                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total, gn);
   return check_launch("conv_mfma_kernel");
 }
 
 template <typename T, int NSUB>
 int launch_k333(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
-                float* partial, hipStream_t st) {
+                float* partial, hipStream_t st, const GnPartialOut& gn) {
   // Brick shape follows the row length: 32-voxel sub-tiles are one, two or four W rows.
   switch (p.shape) {
-    case 0: return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 3: return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 6: return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 0: return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 3: return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 6: return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
 #ifdef SFH_GATHER_TUNE  // 128-voxel tiles: built only to be measured
-    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
-    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st);
+    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
 #endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv mfma: no kernel for brick shape %d", p.shape);
   }
 }
 
+// Records of GroupNorm partials per sample the launch of plan p leaves for `groups` groups (0: not offered).
+int gather_gn_records(const MfmaConvArgs& a, const GatherPlan& p, int groups) {
+  if (p.ksplit > 1) return sum_slices_bias_stats_records((int64_t)a.od * a.oh * a.ow * a.cout, a.cout, groups);
+  const int span = 32 * p.nsub;
+  if (!gn_partials_fit(a.cout, groups, span)) return 0;
+  const int cg = a.cout / groups;
+  const int64_t records = p.tiles / a.n * (cg > span ? cg / span : 1);
+  return records <= 0x7fffffff ? (int)records : 0;
+}
+
 template <typename T>
 int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, void* partial,
-                 hipStream_t st) {
+                 hipStream_t st, const GnPartialOut* gn) {
   const GatherPlan p = gather_plan(a);
   if (p.ksplit > 1 && partial == nullptr) return fail(SFH_ERR_WORKSPACE, "conv mfma: the reduction split needs its workspace");
-  const int rc = p.nsub == 2 ? launch_k333<T, 2>(a, p, x, packed, bias, y, (float*)partial, st)
-                             : launch_k333<T, 1>(a, p, x, packed, bias, y, (float*)partial, st);
+  GnPartialOut out{nullptr, 0, 0, 0};
+  if (gn != nullptr && gn->part != nullptr) {
+    if (gn->records != gather_gn_records(a, p, gn->groups) || gn->records == 0)
+      return fail(SFH_ERR_INVALID, "conv mfma: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
+                  gather_gn_records(a, p, gn->groups));
+    out = *gn;
+    out.cg = a.cout / gn->groups;
+  }
+  const GnPartialOut none{nullptr, 0, 0, 0};
+  const GnPartialOut& in_kernel = p.ksplit == 1 ? out : none;
+  const int rc = p.nsub == 2 ? launch_k333<T, 2>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel)
+                             : launch_k333<T, 1>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel);
   if (rc != SFH_OK || p.ksplit == 1) return rc;
-  return sum_slices_bias(dtype, (const float*)partial, bias, y, (int64_t)a.n * a.od * a.oh * a.ow * a.cout, a.cout, p.ksplit, st);
+  const int64_t sample = (int64_t)a.od * a.oh * a.ow * a.cout;
+  if (out.part != nullptr) return sum_slices_bias_stats(dtype, (const float*)partial, bias, y, a.n, sample, a.cout, p.ksplit, out, st);
+  return sum_slices_bias(dtype, (const float*)partial, bias, y, a.n * sample, a.cout, p.ksplit, st);
 }
 
 }  // namespace
@@ -506,11 +542,16 @@ MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a) {
   return MfmaConvGeometry{kKernelBrick, t[0] * t[1] * t[2], p.nsub, p.ksplit};
 }
 
+int mfma_conv_gather_gn_records(const MfmaConvArgs& a, int groups) {
+  if (mfma_conv_wide_applies(a)) return mfma_conv_wide_gn_records(a, groups);
+  return gather_gn_records(a, gather_plan(a), groups);
+}
+
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                     void* partial, hipStream_t st) {
-  if (mfma_conv_wide_applies(a)) return mfma_conv_wide(a, dtype, x, packed, bias, y, st);
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st);
-  return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st);
+                     void* partial, hipStream_t st, const GnPartialOut* gn) {
+  if (mfma_conv_wide_applies(a)) return mfma_conv_wide(a, dtype, x, packed, bias, y, st, gn);
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st, gn);
+  return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st, gn);
 }
 
 }  // namespace sfh

@@ -1,6 +1,7 @@
 // Host-side interface of the MFMA implicit-GEMM convolution kernels (bf16 / fp16 only).
 #pragma once
 #include "common.hpp"
+#include "gn_stats.hpp"
 
 namespace sfh {
 
@@ -33,15 +34,23 @@ struct MfmaPackItem {
 int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStream_t st);
 // Bytes of fp32 slices the kernel needs when it cuts the reduction channels to fill the chip (0 when it does not).
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a);
+// `gn` (optional): also leave GroupNorm partials of the rounded output (gn_stats.hpp), gn->records per sample as
+// mfma_conv_gn_records says for gn->groups groups.
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                     void* partial, hipStream_t st);
+                     void* partial, hipStream_t st, const GnPartialOut* gn = nullptr);
 // Same contract, wide-tile kernel (64 or more reduction channels, rows of more than 16 voxels): `applies` is a pure
 // function of the shape; mfma_conv_gather routes to it (it needs no partial workspace).
 bool mfma_conv_wide_applies(const MfmaConvArgs& a);
-int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st);
+int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                   const GnPartialOut* gn = nullptr);
 // Same contract, persistent one-workgroup-per-CU kernel with register-resident weights.
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                      void* partial, hipStream_t st);
+                      void* partial, hipStream_t st, const GnPartialOut* gn = nullptr);
+// Records of GroupNorm partials per sample that mfma_conv_persist leaves for `groups` groups: a pure function of the
+// shape; 0 when the kernel that serves the problem does not offer them (the caller then runs the statistics pass).
+int mfma_conv_gn_records(const MfmaConvArgs& a, int groups);
+int mfma_conv_gather_gn_records(const MfmaConvArgs& a, int groups);
+int mfma_conv_wide_gn_records(const MfmaConvArgs& a, int groups);
 
 // Which of the three kernels mfma_conv_persist ends up launching for a problem, and with what geometry: a pure function of
 // the shape. `voxels` is the output tile of a workgroup step, `blocks` the 32-channel output blocks a workgroup produces

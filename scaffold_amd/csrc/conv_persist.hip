@@ -192,8 +192,10 @@ struct PendingStore {
   sfh_u32x4_t data[C::MS][2];
 };
 
-template <typename T, typename C, bool BIAS>
-__device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const float (&bias)[16], PendingStore<C>& ps) {
+// With GN, the rounded values of the voxels inside the output are also added to the lane's GroupNorm sums.
+template <typename T, typename C, bool BIAS, bool GN>
+__device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const float (&bias)[16], PendingStore<C>& ps,
+                                            const MfmaConvArgs& a, const TileCoord& tc, const LaneGeom<C>& lg, RunSums& sums) {
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     uint32_t run[4][2];
@@ -205,6 +207,7 @@ __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const 
       run[g][0] = Mma32<T>::pack2(v[0], v[1]);
       run[g][1] = Mma32<T>::pack2(v[2], v[3]);
     }
+    if constexpr (GN) sums.template add<T>(run, store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]) != kRange);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       // lanes 32-63 of run 2h <-> lanes 0-31 of run 2h+1
@@ -291,10 +294,10 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
   }
 }
 
-template <typename T, typename C, bool BIAS>
+template <typename T, typename C, bool BIAS, bool GN>
 __global__ void __launch_bounds__(256, 1)
 conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias_ptr,
-                    T* __restrict__ y, PersistGeom gm) {
+                    T* __restrict__ y, PersistGeom gm, GnPartialOut gn) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space builtins the host pass cannot type-check
   __shared__ __attribute__((aligned(16))) char buf0[C::BRICK];
   __shared__ __attribute__((aligned(16))) char buf1[C::BRICK];
@@ -366,6 +369,8 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) done_off[ms] = kRange;  // nothing to store during the first step
   T* done_origin = y;
+  RunSums gn_sums;  // GroupNorm statistics of this workgroup's rounded outputs (GN)
+  gn_sums.clear();
 
   for (int step = 0; step < nsteps; ++step) {
     const TileCoord tc2 = next_tile(tc1, gm);
@@ -375,7 +380,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     if (step & 1) persist_step<T, C>(a, buf1, buf0, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
     else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
     asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMAs are inline asm: the compiler does not know their result latency
-    round_brick<T, C, BIAS>(acc, bias, ps);  // its stores ride along with the next step's MFMAs
+    round_brick<T, C, BIAS, GN>(acc, bias, ps, a, tc, lg, gn_sums);  // its stores ride along with the next step's MFMAs
     done_origin = tile_origin<T, C>(a, y, tc, nb);
     tc = tc1;
     tc1 = tc2;
@@ -388,40 +393,66 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   for (int ms = 0; ms < C::MS; ++ms)
 #pragma unroll
     for (int h = 0; h < 2; ++h) __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
+  if constexpr (GN) {
+    // one record per workgroup (one sample): the loop's last barrier has freed the LDS
+    const int per_wg = gn.cg > 32 ? gn.cg / 32 : 1;  // output blocks that share a group
+    RunSums one[1] = {gn_sums};
+    write_group_partials<4, 1>(one, reinterpret_cast<float*>(buf0), gn, 0, (wg - nb * gm.wgs_per_block) * per_wg + nb % per_wg, nb * 32, tid);
+  }
 #endif
 }
 
-template <typename T, typename C>
-int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+PersistGeom persist_geom(const MfmaConvArgs& a, int td, int th, int tw) {
   PersistGeom gm{};
-  gm.tiles_d = (int)cdiv(a.od, C::TD);
-  gm.tiles_h = (int)cdiv(a.oh, C::TH);
-  gm.tiles_w = (int)cdiv(a.ow, C::TW);
+  gm.tiles_d = (int)cdiv(a.od, td);
+  gm.tiles_h = (int)cdiv(a.oh, th);
+  gm.tiles_w = (int)cdiv(a.ow, tw);
   const int64_t ntiles = (int64_t)a.n * gm.tiles_d * gm.tiles_h * gm.tiles_w;
-  if (ntiles > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: too many bricks");
-  gm.ntiles = (int)ntiles;
+  gm.ntiles = ntiles > 0x7fffffffLL ? -1 : (int)ntiles;
   gm.blocked = (gm.tiles_d % 4 == 0 && gm.tiles_h % 4 == 0) ? 1 : 0;
   gm.nblocks = a.cout / 32;
   int per_block = kComputeUnits / gm.nblocks;
   if (per_block < 1) per_block = 1;
   if (per_block > gm.ntiles) per_block = gm.ntiles;
-  gm.items_per_wg = (int)cdiv(gm.ntiles, per_block);
-  gm.wgs_per_block = (int)cdiv(gm.ntiles, gm.items_per_wg);
+  if (gm.ntiles > 0) {
+    gm.items_per_wg = (int)cdiv(gm.ntiles, per_block);
+    gm.wgs_per_block = (int)cdiv(gm.ntiles, gm.items_per_wg);
+  }
+  return gm;
+}
+PersistGeom persist_geom(const MfmaConvArgs& a) {
+  if (a.ow > 16) return persist_geom(a, 4, 4, 32);
+  if (a.ow > 8) return persist_geom(a, 4, 8, 16);
+  return persist_geom(a, 8, 8, 8);
+}
+
+template <typename T, typename C>
+int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                const GnPartialOut& gn) {
+  const PersistGeom gm = persist_geom(a, C::TD, C::TH, C::TW);
+  if (gm.ntiles < 0) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: too many bricks");
+  if (gm.ntiles == 0) return SFH_OK;
   const unsigned grid = (unsigned)(gm.wgs_per_block * gm.nblocks);
-  if (bias != nullptr)
-    hipLaunchKernelGGL((conv_persist_kernel<T, C, true>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
-                       (const T*)bias, (T*)y, gm);
-  else
-    hipLaunchKernelGGL((conv_persist_kernel<T, C, false>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
-                       (const T*)bias, (T*)y, gm);
+#define SFH_PERSIST(BIAS, GN)                                                                                                    \
+  hipLaunchKernelGGL((conv_persist_kernel<T, C, BIAS, GN>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed, \
+                     (const T*)bias, (T*)y, gm, gn)
+  if (bias != nullptr) {
+    if (gn.part != nullptr) SFH_PERSIST(true, true);
+    else SFH_PERSIST(true, false);
+  } else {
+    if (gn.part != nullptr) SFH_PERSIST(false, true);
+    else SFH_PERSIST(false, false);
+  }
+#undef SFH_PERSIST
   return check_launch("conv_persist_kernel");
 }
 
 template <typename T>
-int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
-  if (a.ow > 16) return launch_tile<T, PTile<4, 4, 32>>(a, x, packed, bias, y, st);
-  if (a.ow > 8) return launch_tile<T, PTile<4, 8, 16>>(a, x, packed, bias, y, st);
-  return launch_tile<T, PTile<8, 8, 8>>(a, x, packed, bias, y, st);
+int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                 const GnPartialOut& gn) {
+  if (a.ow > 16) return launch_tile<T, PTile<4, 4, 32>>(a, x, packed, bias, y, st, gn);
+  if (a.ow > 8) return launch_tile<T, PTile<4, 8, 16>>(a, x, packed, bias, y, st, gn);
+  return launch_tile<T, PTile<8, 8, 8>>(a, x, packed, bias, y, st, gn);
 }
 
 }  // namespace
@@ -440,11 +471,29 @@ MfmaConvGeometry mfma_conv_geometry(const MfmaConvArgs& a) {
   return MfmaConvGeometry{kKernelPersist, 512, 1, 1};
 }
 
+// One record per workgroup, so one sample only (a workgroup's run of bricks may cross samples).
+int mfma_conv_gn_records(const MfmaConvArgs& a, int groups) {
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather_gn_records(a, groups);
+  if (a.n != 1 || !gn_partials_fit(a.cout, groups, 32)) return 0;
+  const PersistGeom gm = persist_geom(a);
+  if (gm.ntiles <= 0) return 0;
+  const int cg = a.cout / groups;
+  return gm.wgs_per_block * (cg > 32 ? cg / 32 : 1);
+}
+
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                      void* partial, hipStream_t st) {
-  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st);
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st);
-  return launch_typed<fp16_t>(a, x, packed, bias, y, st);
+                      void* partial, hipStream_t st, const GnPartialOut* gn) {
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st, gn);
+  GnPartialOut out{nullptr, 0, 0, 0};
+  if (gn != nullptr && gn->part != nullptr) {
+    if (gn->records == 0 || gn->records != mfma_conv_gn_records(a, gn->groups))
+      return fail(SFH_ERR_INVALID, "conv persist: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
+                  mfma_conv_gn_records(a, gn->groups));
+    out = *gn;
+    out.cg = a.cout / gn->groups;
+  }
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st, out);
+  return launch_typed<fp16_t>(a, x, packed, bias, y, st, out);
 }
 
 }  // namespace sfh

@@ -183,7 +183,7 @@ __device__ __forceinline__ void weight_loads(const WideCtx<T, C>& k, int chunk, 
 template <typename T, typename C>
 __global__ void __launch_bounds__(256, 1)
 conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias, T* __restrict__ y,
-                 WideGeom gm) {
+                 WideGeom gm, GnPartialOut gn) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space builtins the host pass cannot type-check
   __shared__ __attribute__((aligned(16))) char brick0_[C::BRICK];
   __shared__ __attribute__((aligned(16))) char brick1_[C::BRICK];
@@ -331,6 +331,9 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   int tid_out = tid;
   asm volatile("" : "+v"(tid_out));
   const int wave_out = tid_out >> 6, j_out = tid_out & 31, kg_out = (tid_out >> 5) & 1;
+  RunSums gn_sums[C::NSUB];  // GroupNorm statistics of the rounded output, when the caller wants them
+#pragma unroll
+  for (int ns = 0; ns < C::NSUB; ++ns) gn_sums[ns].clear();
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     const int v = (wave_out * C::MS + ms) * 32 + j_out;
@@ -340,7 +343,16 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     const int64_t vox = (((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow;
     T* yp = y + vox * a.cout + nb * C::NSUB * 32;
 #pragma unroll
-    for (int ns = 0; ns < C::NSUB; ++ns) store_block<T>(acc[ms][ns], yp + ns * 32, bias, (nb * C::NSUB + ns) * 32, kg_out, inside);
+    for (int ns = 0; ns < C::NSUB; ++ns)
+      store_block<T>(acc[ms][ns], yp + ns * 32, bias, (nb * C::NSUB + ns) * 32, kg_out, inside, gn_sums[ns], gn.part != nullptr);
+  }
+  if (gn.part != nullptr) {
+    __syncthreads();  // every wave is done with the bricks: the LDS is free
+    constexpr int SPAN = 32 * C::NSUB;
+    const int per_tile = gn.cg > SPAN ? gn.cg / SPAN : 1;  // workgroups that share a group of this tile
+    const int tile = (td_i * gm.tiles_h + th_i) * gm.tiles_w + tw_i;
+    write_group_partials<4, C::NSUB>(gn_sums, reinterpret_cast<float*>(brick0_), gn, n, tile * per_tile + nb % per_tile, nb * SPAN,
+                                     tid_out);
   }
 #endif
 }
@@ -389,7 +401,8 @@ WidePlan wide_plan(const MfmaConvArgs& a) {
 }
 
 template <typename T, typename C>
-int launch_wide(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+int launch_wide(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                const GnPartialOut& gn) {
   WideGeom gm{};
   gm.tiles_d = (int)cdiv(a.od, C::TD);
   gm.tiles_h = (int)cdiv(a.oh, C::TH);
@@ -400,19 +413,20 @@ int launch_wide(const MfmaConvArgs& a, const void* x, const void* packed, const 
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv wide: %lld workgroups exceed the grid limit", (long long)total);
   gm.total = (uint32_t)total;
   hipLaunchKernelGGL((conv_wide_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed, (const T*)bias,
-                     (T*)y, gm);
+                     (T*)y, gm, gn);
   return check_launch("conv_wide_kernel");
 }
 
 template <typename T>
-int launch_typed(const MfmaConvArgs& a, const WidePlan& p, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+int launch_typed(const MfmaConvArgs& a, const WidePlan& p, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                 const GnPartialOut& gn) {
   switch (p.shape) {
-    case 1: return launch_wide<T, WTile<8, 4, 32, 2>>(a, x, packed, bias, y, st);
-    case 3: return launch_wide<T, WTile<4, 4, 32, 2>>(a, x, packed, bias, y, st);
+    case 1: return launch_wide<T, WTile<8, 4, 32, 2>>(a, x, packed, bias, y, st, gn);
+    case 3: return launch_wide<T, WTile<4, 4, 32, 2>>(a, x, packed, bias, y, st, gn);
 #ifdef SFH_WIDE_TUNE  // the other accumulator grids: built only to be measured
-    case 0: return launch_wide<T, WTile<4, 4, 32, 4>>(a, x, packed, bias, y, st);
-    case 2: return launch_wide<T, WTile<8, 4, 32, 1>>(a, x, packed, bias, y, st);
-    case 4: return launch_wide<T, WTile<4, 4, 32, 1>>(a, x, packed, bias, y, st);
+    case 0: return launch_wide<T, WTile<4, 4, 32, 4>>(a, x, packed, bias, y, st, gn);
+    case 2: return launch_wide<T, WTile<8, 4, 32, 1>>(a, x, packed, bias, y, st, gn);
+    case 4: return launch_wide<T, WTile<4, 4, 32, 1>>(a, x, packed, bias, y, st, gn);
 #endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv wide: no kernel for accumulator grid %d", p.shape);
   }
@@ -428,11 +442,32 @@ MfmaConvGeometry mfma_conv_wide_geometry(const MfmaConvArgs& a) {
   return MfmaConvGeometry{kKernelWide, td[p.shape] * 4 * 32, nsub[p.shape], 1};
 }
 
-int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st) {
+int mfma_conv_wide_gn_records(const MfmaConvArgs& a, int groups) {
+  const WidePlan p = wide_plan(a);
+  if (!p.use) return 0;
+  const MfmaConvGeometry g = mfma_conv_wide_geometry(a);
+  const int span = 32 * g.blocks;
+  if (!gn_partials_fit(a.cout, groups, span)) return 0;
+  const int cg = a.cout / groups;
+  const int64_t tiles = (int64_t)cdiv(a.od, g.voxels / 128) * cdiv(a.oh, 4) * cdiv(a.ow, 32);
+  const int64_t records = tiles * (cg > span ? cg / span : 1);
+  return records <= 0x7fffffff ? (int)records : 0;
+}
+
+int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                   const GnPartialOut* gn) {
   const WidePlan p = wide_plan(a);
   if (!p.use) return fail(SFH_ERR_UNSUPPORTED, "conv wide: not applicable to this problem");
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, p, x, packed, bias, y, st);
-  return launch_typed<fp16_t>(a, p, x, packed, bias, y, st);
+  GnPartialOut out{nullptr, 0, 0, 0};
+  if (gn != nullptr && gn->part != nullptr) {
+    if (gn->records == 0 || gn->records != mfma_conv_wide_gn_records(a, gn->groups))
+      return fail(SFH_ERR_INVALID, "conv wide: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
+                  mfma_conv_wide_gn_records(a, gn->groups));
+    out = *gn;
+    out.cg = a.cout / gn->groups;
+  }
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, p, x, packed, bias, y, st, out);
+  return launch_typed<fp16_t>(a, p, x, packed, bias, y, st, out);
 }
 
 }  // namespace sfh

@@ -223,7 +223,8 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
 }
 
 // One 64-lane workgroup per (group, sample): fixed-order sum of the split partials, then
-// mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps).
+// mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps). A null `shift` stands for K = 0 (partials that
+// the producer of x summed unshifted).
 __global__ void __launch_bounds__(64) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
                                                         float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
                                                         float m, float eps) {
@@ -240,7 +241,7 @@ __global__ void __launch_bounds__(64) gn_stats_finalize(const float* __restrict_
     const float d = s1 / m;
     float var = s2 / m - d * d;
     var = var < 0.f ? 0.f : var;
-    mean[n * G + g] = shift[n * G + g] + d;
+    mean[n * G + g] = (shift != nullptr ? shift[n * G + g] : 0.f) + d;
     rstd[n * G + g] = 1.f / sqrtf(var + eps);
   }
 }
@@ -299,7 +300,7 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
                                                        float* __restrict__ rstd, const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
                                                        int tpr, int rpp, int nsplit, int64_t rows_per_split, float m, float eps,
-                                                       int relu, int64_t y_halo) {
+                                                       int relu, int64_t y_halo, int npart) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float gstat[];  // sums[2 G] | mean[G] | rstd[G] | fold scratch (4 * kBlock)
   const int tid = threadIdx.x;
@@ -308,14 +309,16 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   const int r = tid / tpr, cv = tid - r * tpr;
   float* g_mean = gstat + 2 * G;
   float* g_rstd = gstat + 3 * G;
-  if (fold_in_consumer(G, nsplit)) {
-    fold_split_partials(part + (int64_t)n * nsplit * 2 * G, G, nsplit, gstat + 4 * G, [&](int c, float t) { gstat[c] = t; });
+  // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid), or the ones the
+  // producer of x left (then without a shift)
+  if (fold_in_consumer(G, npart)) {
+    fold_split_partials(part + (int64_t)n * npart * 2 * G, G, npart, gstat + 4 * G, [&](int c, float t) { gstat[c] = t; });
     __syncthreads();
     if (tid < G) {
       const float d = gstat[tid] / m;
       float var = gstat[G + tid] / m - d * d;
       var = var < 0.f ? 0.f : var;
-      const float mu_g = shift[n * G + tid] + d, rs_g = 1.f / sqrtf(var + eps);
+      const float mu_g = (shift != nullptr ? shift[n * G + tid] : 0.f) + d, rs_g = 1.f / sqrtf(var + eps);
       g_mean[tid] = mu_g;
       g_rstd[tid] = rs_g;
       if (blockIdx.x == 0) {  // for the backward pass
@@ -835,12 +838,14 @@ size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
 
 template <typename T, typename TO>
 int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
-              void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st) {
+              void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st, const float* given_part = nullptr,
+              int given_npart = 0) {
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
   if (y_halo > 0 && (!pl.vector || sizeof(T) != sizeof(TO) || (y_halo * C * sizeof(TO)) % 16 != 0))
     return fail(SFH_ERR_UNSUPPORTED, "groupnorm: the slab output needs the vector path and an output of the input's width");
   if (!pl.vector) {
+    if (given_part != nullptr) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: statistics from given partials need the vector path");
     hipLaunchKernelGGL(gn_scalar_stats<T>, dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, mean, rstd, S, C, G, p.eps);
     if (int rc = check_launch("gn_scalar_stats")) return rc;
     const int64_t total = (int64_t)p.n * S * C;
@@ -849,28 +854,35 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
                        (TO*)y, mean, rstd, gamma, beta, param_dtype, S, C, G, total, p.relu);
     return check_launch("gn_scalar_normalize");
   }
-  float* shift = ws;
-  float* part = ws + align_up((size_t)p.n * G, 4);
-  const size_t lds = (size_t)(2 * pl.slots * kBlock + 2 * G) * sizeof(float);
   const dim3 grid(pl.nsplit, p.n);
-#define SFH_GN_STATS(SL)                                                                                                   \
-  hipLaunchKernelGGL((gn_stats_partial<T, SL>), grid, dim3(kBlock), lds, st, (const T*)x, shift, part, S, C, G, pl.tpr, \
+  const float* shift = nullptr;
+  const float* part = given_part;
+  int npart = given_npart;
+  if (given_part == nullptr) {
+    float* my_shift = ws;
+    float* my_part = ws + align_up((size_t)p.n * G, 4);
+    const size_t lds = (size_t)(2 * pl.slots * kBlock + 2 * G) * sizeof(float);
+#define SFH_GN_STATS(SL)                                                                                                      \
+  hipLaunchKernelGGL((gn_stats_partial<T, SL>), grid, dim3(kBlock), lds, st, (const T*)x, my_shift, my_part, S, C, G, pl.tpr, \
                      pl.rpp, pl.nsplit, pl.rows_per_split)
-  switch (pl.slots) {
-    case 1: SFH_GN_STATS(1); break;
-    case 2: SFH_GN_STATS(2); break;
-    case 4: SFH_GN_STATS(4); break;
-    default: SFH_GN_STATS(8); break;
-  }
+    switch (pl.slots) {
+      case 1: SFH_GN_STATS(1); break;
+      case 2: SFH_GN_STATS(2); break;
+      case 4: SFH_GN_STATS(4); break;
+      default: SFH_GN_STATS(8); break;
+    }
 #undef SFH_GN_STATS
-  if (int rc = check_launch("gn_stats_partial")) return rc;
+    if (int rc = check_launch("gn_stats_partial")) return rc;
+    shift = my_shift; part = my_part; npart = pl.nsplit;
+  }
   const float m = (float)S * (float)(C / G);
-  if (!fold_in_consumer_host(G, pl.nsplit)) {
-    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, pl.nsplit, m, p.eps);
+  if (!fold_in_consumer_host(G, npart)) {
+    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, npart, m, p.eps);
     if (int rc = check_launch("gn_stats_finalize")) return rc;
   }
   hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
-                     mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu, y_halo);
+                     mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu, y_halo,
+                     npart);
   return check_launch("gn_normalize");
 }
 
@@ -929,20 +941,21 @@ extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p,
 
 static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x, const void* gamma,
                              const void* beta, void* y, int64_t y_halo, float* mean, float* rstd, void* workspace,
-                             size_t workspace_bytes, void* stream) {
+                             size_t workspace_bytes, void* stream, const float* given_part = nullptr, int given_npart = 0) {
   if (int rc = check_desc(p, x_dtype)) return rc;
   if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
   if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
   if (y_halo < 0) return fail(SFH_ERR_INVALID, "groupnorm: negative halo");
   const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(y));
-  if (pl.vector) {
+  if (pl.vector && given_part == nullptr) {
     const size_t need = fwd_ws_floats(*p, pl) * sizeof(float);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "groupnorm fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
   }
   hipStream_t st = (hipStream_t)stream;
   float* ws = (float*)workspace;
-#define SFH_GN_FWD(TX, TY) return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st)
+#define SFH_GN_FWD(TX, TY) \
+  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart)
   if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
@@ -966,6 +979,15 @@ extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, 
                                       void* workspace, size_t workspace_bytes, void* stream) {
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, workspace,
                            workspace_bytes, stream);
+}
+
+extern "C" int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
+                                               const void* gamma, const void* beta, void* y_slab, int64_t halo_rows, float* mean,
+                                               float* rstd, const float* partials, int32_t records, void* stream) {
+  if (partials == nullptr || records < 1) return fail(SFH_ERR_INVALID, "groupnorm from partials: no partial sums given");
+  if (!aligned16(partials)) return fail(SFH_ERR_INVALID, "groupnorm from partials: the partial sums must be 16-byte aligned");
+  return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, nullptr, 0, stream, partials,
+                           records);
 }
 
 // ---- the forward for callers that may not allocate ------------------------------------------------------------------

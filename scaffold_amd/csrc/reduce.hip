@@ -2,6 +2,7 @@
 // channels-last tensor (the bias gradient, ScaFFold/unet/conv3d.py:1231,1786). No atomics: every
 // partial has a fixed slot and every sum a fixed order, so a call gives the same bits every time.
 #include "reduce.hpp"
+#include "gn_stats.hpp"
 #include "vec_io.hpp"
 
 namespace sfh {
@@ -127,6 +128,50 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __
   out[e + 1] = elem<T>::from_float(s.y);
   out[e + 2] = elem<T>::from_float(s.z);
   out[e + 3] = elem<T>::from_float(s.w);
+}
+
+// sum_slices_bias that also leaves GroupNorm partials of the rounded result (16-bit outputs): a workgroup owns `chunks`
+// consecutive pieces of 1024 elements of one sample; 1024 is a multiple of the channel count, so a thread's four
+// consecutive channels are the same in every piece and belong to one group. One record per workgroup.
+constexpr int kStatsPiece = 4 * kBlock;
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const float* __restrict__ part, const T* __restrict__ bias,
+                                                                       T* __restrict__ out, int64_t sample_elems, int64_t nelem,
+                                                                       int channels, int splits, int chunks, GnPartialOut gn) {
+  __shared__ float sums[kBlock][2];
+  const int tid = threadIdx.x, n = blockIdx.y;
+  const int c = (tid * 4) % channels;
+  float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
+  if (bias != nullptr) { b0 = to_float(bias[c]); b1 = to_float(bias[c + 1]); b2 = to_float(bias[c + 2]); b3 = to_float(bias[c + 3]); }
+  float s1 = 0.f, s2 = 0.f;
+  for (int k = 0; k < chunks; ++k) {
+    const int64_t local = ((int64_t)blockIdx.x * chunks + k) * kStatsPiece + tid * 4;
+    if (local >= sample_elems) break;
+    const int64_t e = (int64_t)n * sample_elems + local;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int sp = 0; sp < splits; ++sp) {
+      const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const T o0 = elem<T>::from_float(s.x + b0), o1 = elem<T>::from_float(s.y + b1), o2 = elem<T>::from_float(s.z + b2),
+            o3 = elem<T>::from_float(s.w + b3);
+    out[e] = o0; out[e + 1] = o1; out[e + 2] = o2; out[e + 3] = o3;
+    const float r0 = to_float(o0), r1 = to_float(o1), r2 = to_float(o2), r3 = to_float(o3);
+    s1 += (r0 + r1) + (r2 + r3);
+    s2 += fmaf(r0, r0, r1 * r1) + fmaf(r2, r2, r3 * r3);
+  }
+  sums[tid][0] = s1;
+  sums[tid][1] = s2;
+  __syncthreads();
+  const int rows = kStatsPiece / channels, per_row = channels / 4, per_group = gn.cg / 4;
+  for (int t = tid; t < 2 * gn.groups; t += kBlock) {
+    const int q = t & 1, g = t >> 1;
+    float acc = 0.f;
+    for (int v = 0; v < rows; ++v)
+      for (int r = 0; r < per_group; ++r) acc += sums[v * per_row + g * per_group + r][q];
+    gn.part[(((int64_t)n * gn.records + blockIdx.x) * 2 + q) * gn.groups + g] = acc;
+  }
 }
 
 // Per-channel partial sums: thread = (row slot, channel); a workgroup walks its row range with rpp rows per
@@ -264,6 +309,32 @@ int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, i
     hipLaunchKernelGGL(sum_slices_bias_kernel<float>, grid, dim3(kBlock), 0, st, part, (const float*)bias, (float*)out, nelem,
                        channels, splits);
   return check_launch("sum_slices_bias_kernel");
+}
+
+int sum_slices_bias_stats_records(int64_t sample_elems, int channels, int groups) {
+  if (channels < 4 || kStatsPiece % channels != 0 || sample_elems % 4 != 0 || groups < 1 || channels % groups != 0 ||
+      (channels / groups) % 4 != 0)
+    return 0;
+  const int64_t pieces = cdiv(sample_elems, kStatsPiece);
+  const int64_t chunks = cdiv(pieces, 512);
+  return (int)cdiv(pieces, chunks);
+}
+
+int sum_slices_bias_stats(int dtype, const float* part, const void* bias, void* out, int n, int64_t sample_elems, int channels,
+                          int splits, const GnPartialOut& gn, hipStream_t st) {
+  if (n <= 0 || sample_elems <= 0) return SFH_OK;
+  const int records = sum_slices_bias_stats_records(sample_elems, channels, gn.groups);
+  if (records == 0 || records != gn.records || (dtype != SFH_BF16 && dtype != SFH_FP16))
+    return fail(SFH_ERR_UNSUPPORTED, "sum of slices with GroupNorm partials: not offered for this shape");
+  const int chunks = (int)cdiv(cdiv(sample_elems, kStatsPiece), records);
+  const dim3 grid((unsigned)records, (unsigned)n);
+  if (dtype == SFH_BF16)
+    hipLaunchKernelGGL(sum_slices_bias_stats_kernel<bf16_t>, grid, dim3(kBlock), 0, st, part, (const bf16_t*)bias, (bf16_t*)out,
+                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn);
+  else
+    hipLaunchKernelGGL(sum_slices_bias_stats_kernel<fp16_t>, grid, dim3(kBlock), 0, st, part, (const fp16_t*)bias, (fp16_t*)out,
+                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn);
+  return check_launch("sum_slices_bias_stats_kernel");
 }
 
 size_t bias_grad_workspace_bytes(int64_t rows, int channels) {

@@ -11,6 +11,13 @@ int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int split
 int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, int64_t nelem, int channels, int splits,
                     hipStream_t st);
 
+// The same with GroupNorm partials of the rounded result (gn_stats.hpp) for n samples of sample_elems elements each:
+// `records` per sample as sum_slices_bias_stats_records says (0: not offered for this shape; 16-bit outputs only).
+struct GnPartialOut;
+int sum_slices_bias_stats_records(int64_t sample_elems, int channels, int groups);
+int sum_slices_bias_stats(int dtype, const float* part, const void* bias, void* out, int n, int64_t sample_elems, int channels,
+                          int splits, const GnPartialOut& gn, hipStream_t st);
+
 // gb[c] = sum over rows of g[row * channels + c] for a dense (rows, channels) tensor of `dtype`; fp32
 // accumulation through partial slices in `ws`, result rounded once to `out_dtype`.
 size_t bias_grad_workspace_bytes(int64_t rows, int channels);

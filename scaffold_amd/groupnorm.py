@@ -103,6 +103,29 @@ def _plan(input, num_groups: int, eps: float, activation, backward: bool):
     return plan
 
 
+def _launch_forward(L, desc, xcode, odt, need, input, weight, bias, out, slab, out_halo, mean, rstd):
+    """The statistics pass + normalisation; returns the status, or ``(status, output)`` when the slab form was refused and
+    a plain output took its place."""
+    ws = _lib.workspace(need, input.device)
+    if slab is None:
+        return L.sfh_groupnorm_fwd(
+            ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+            _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
+            _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+    rc = L.sfh_groupnorm_fwd_slab(
+        ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+        _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(slab), out_halo * int(input.shape[3]) * int(input.shape[4]),
+        _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+    if rc == _lib.SFH_ERR_UNSUPPORTED:  # channel counts off the vector path: the plain form
+        out = torch.empty_like(input, dtype=odt)
+        rc = L.sfh_groupnorm_fwd(
+            ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
+            _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
+            _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+        return rc, out
+    return rc
+
+
 def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, out_halo: int = 0):
     """The forward launch: ``(output, mean, rstd)``; shared by the registered operator and the eager autograd node.
 
@@ -131,23 +154,19 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, o
     L = _lib.lib()
     desc, xcode, need = _plan(input, num_groups, eps, activation, False)
     with _lib.device_guard(input.device):
-        ws = _lib.workspace(need, input.device)
-        if slab is None:
-            rc = L.sfh_groupnorm_fwd(
+        rc = _lib.SFH_ERR_UNSUPPORTED
+        given = getattr(input, "_sfh_gn_partials", None)
+        if given is not None and given[2] == num_groups and given[3] == input._version and given[0].device == input.device:
+            # the producer of `input` left its per-group sums: no statistics pass
+            rc = L.sfh_groupnorm_fwd_from_partials(
                 ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
-                _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
-                _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
-        else:
-            rc = L.sfh_groupnorm_fwd_slab(
-                ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
-                _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(slab), out_halo * int(input.shape[3]) * int(input.shape[4]),
-                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
-            if rc == _lib.SFH_ERR_UNSUPPORTED:  # channel counts off the vector path: the plain form
-                out = torch.empty_like(input, dtype=odt)
-                rc = L.sfh_groupnorm_fwd(
-                    ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
-                    _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out), _lib.ptr(mean), _lib.ptr(rstd),
-                    _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.stream_ptr(input.device))
+                _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out if slab is None else slab),
+                0 if slab is None else out_halo * int(input.shape[3]) * int(input.shape[4]),
+                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(given[0]), given[1], _lib.stream_ptr(input.device))
+        if rc == _lib.SFH_ERR_UNSUPPORTED:
+            rc = _launch_forward(L, desc, xcode, odt, need, input, weight, bias, out, slab, out_halo, mean, rstd)
+            if isinstance(rc, tuple):
+                rc, out = rc
     _lib.check(rc, "group_norm")
     return out, mean, rstd
 

@@ -118,7 +118,8 @@ class _Conv3dFn(torch.autograd.Function):
     autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
 
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None):
+    def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None,
+                gn_groups=0):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
@@ -138,7 +139,8 @@ class _Conv3dFn(torch.autograd.Function):
             # That saves a launch per convolution on the GPU and costs a little more host time, so it is done where
             # host time is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
             pf, pd = _c3.pack_weights(wc, x.shape, stride, padding, dilation)
-        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, _checked=True)
+        # gn_groups: a GroupNorm of that many groups follows; the launch leaves its statistics on y where it can
+        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, _checked=True)
         ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
@@ -163,7 +165,7 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
@@ -207,6 +209,9 @@ class FastConv3d(nn.Conv3d):
 
     #: emulate one depth shard: zero halo on both depth faces + depth padding 0
     shard_halo = False
+    #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
+    #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
+    gn_groups = 0
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.padding_mode != "zeros" or isinstance(self.padding, str):
@@ -245,11 +250,11 @@ class FastConv3d(nn.Conv3d):
             inner = x
         if master:
             return _Conv3dFn.apply(inner, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab)
+                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
         if w is self.weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
-                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab)
-        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab)
+                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
+        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups)
 
 
 class FastConvTranspose3d(nn.ConvTranspose3d):

@@ -1,0 +1,150 @@
+"""GroupNorm statistics left by the producing convolution (``conv3d_forward(gn_groups=)``), through the C ABI.
+
+What is held to what:
+* the convolution's output is the same bits with and without the statistics;
+* the partial sums, added up, equal the per-group sum and sum of squares of that output -- bit for bit on integer-valued
+  draws (every voxel counted exactly once, none past a ragged edge), to fp32 round-off on Gaussian ones;
+* ``group_norm`` fed by them agrees with the stand-alone statistics pass to the last bit or so of the 16-bit output, and
+  with the fp64 ``F.group_norm`` oracle within the tolerance of the GroupNorm parity tests;
+* a tensor changed in place after the convolution is not normalised with stale statistics.
+"""
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import scaffold_amd as sa
+from oracle import oracle as orc
+from scaffold_amd import conv3d as c3
+from scaffold_amd.unet import DoubleConv
+
+pytestmark = pytest.mark.gpu
+CL = torch.channels_last_3d
+
+# (n, cin, cout, spatial, padding, groups, kernel that serves the forward)
+CASES = [
+    (1, 32, 32, (8, 8, 32), (1, 1, 1), 8, "persist"),          # 4 channels per group: two groups per lane run pair
+    (1, 32, 32, (5, 7, 33), (1, 1, 1), 4, "persist"),          # ragged tiles on every axis
+    (1, 32, 64, (6, 9, 40), (0, 1, 1), 8, "persist"),          # shard form, two output blocks
+    (1, 32, 128, (4, 8, 16), (1, 1, 1), 2, "persist"),         # a group wider than a workgroup's 32 channels
+    (1, 32, 32, (10, 8, 8), (1, 1, 1), 8, "persist"),          # rows of 8
+    (2, 64, 64, (16, 32, 64), (1, 1, 1), 8, "brick"),          # two samples, no slices
+    (1, 64, 128, (32, 64, 32), (1, 1, 1), 8, "brick"),         # two output blocks per workgroup
+    (1, 64, 128, (16, 32, 33), (1, 1, 1), 2, "brick"),         # a group wider than the workgroup's span, ragged rows
+    (2, 64, 64, (9, 10, 16), (1, 1, 1), 16, "brick"),          # small volume: the reduction is sliced, the slice sum counts
+    (1, 256, 512, (4, 8, 8), (1, 1, 1), 8, "brick"),           # deep level, sliced
+    (1, 128, 64, (32, 64, 64), (0, 1, 1), 8, "wide"),          # 4 x 4 x 32 tiles
+    (1, 128, 64, (63, 61, 65), (1, 1, 1), 16, "wide"),         # 8 x 4 x 32 tiles, ragged on every axis
+    (1, 192, 64, (30, 62, 34), (1, 1, 1), 1, "wide"),          # one group of all 64 channels
+]
+
+
+def group_sums(y, groups):
+    n, c = y.shape[:2]
+    v = y.double().reshape(n, groups, -1)
+    return v.sum(-1), (v * v).sum(-1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", CASES)
+def test_partials_are_the_sums_of_the_output(device, dtype, n, cin, cout, spatial, padding, groups, kernel):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=dtype)
+    geom = c3.launch_geometry(prob.input_shape, prob.weight_shape, 1, padding, 1, dtype, "fwd")
+    assert geom["kernel"] == kernel, geom
+    for exact in (True, False):
+        ops = orc.make_inputs(prob, seed=3, exact=True, density=0.02) if exact else orc.make_inputs(prob, seed=3)
+        x, w = ops["input"].to(device), ops["weight"].to(device)
+        b = (torch.arange(cout) % 5 - 2).to(dtype).to(device)  # small integers: the outputs stay integer-valued
+        plain = sa.conv3d_forward(x, w, b, 1, padding, 1)
+        y = sa.conv3d_forward(x, w, b, 1, padding, 1, gn_groups=groups)
+        assert torch.equal(plain, y), "the statistics must not change the convolution's result"
+        partials, records, g, version = y._sfh_gn_partials
+        assert g == groups and version == y._version and not hasattr(plain, "_sfh_gn_partials")
+        assert partials.numel() == n * records * 2 * groups
+        got = partials.view(n, records, 2, groups).double().sum(1)  # fp64 sum of the fp32 records
+        s1, s2 = group_sums(y, groups)
+        if exact:
+            # integer-valued outputs: every partial sum is exact in fp32, so the totals must be, too
+            assert partials.max() < 2 ** 24 and s2.min() > 0, "the draw must keep every record inside the fp32 mantissa"
+            assert torch.equal(got[:, 0], s1) and torch.equal(got[:, 1], s2), (got[:, 0] - s1, got[:, 1] - s2)
+        else:
+            scale = s2.sqrt() * (y[0].numel() / groups) ** 0.5  # |sum| <= sqrt(m * sum of squares)
+            assert ((got[:, 0] - s1).abs() <= 1e-6 * scale + 1e-3).all()
+            assert ((got[:, 1] - s2).abs() <= 1e-5 * s2 + 1e-3).all()
+
+
+@pytest.mark.parametrize("relu", [False, True])
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", CASES)
+def test_group_norm_from_partials_matches_the_statistics_pass(device, n, cin, cout, spatial, padding, groups, kernel, relu):
+    dtype = torch.bfloat16
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=dtype)
+    ops = orc.make_inputs(prob, seed=11)
+    x, w = ops["input"].to(device), ops["weight"].to(device)
+    gamma = torch.linspace(0.5, 1.5, cout, device=device)
+    beta = torch.linspace(-0.3, 0.3, cout, device=device)
+    act = "relu" if relu else None
+    y = sa.conv3d_forward(x, w, None, 1, padding, 1, gn_groups=groups)
+    assert hasattr(y, "_sfh_gn_partials")
+    fused = sa.group_norm(y, groups, gamma.to(dtype), beta.to(dtype), 1e-5, act, out_dtype=None)
+    plain_y = y.clone(memory_format=torch.preserve_format)  # same bits, no statistics attached
+    assert not hasattr(plain_y, "_sfh_gn_partials")
+    separate = sa.group_norm(plain_y, groups, gamma.to(dtype), beta.to(dtype), 1e-5, act, out_dtype=None)
+    # two routes to mean and rstd in fp32 (shifted and unshifted sums): the 16-bit outputs may differ in the last bit
+    diff = (fused.float() - separate.float()).abs()
+    assert (diff <= 2.0 ** -7 * separate.float().abs() + 1e-6).all(), diff.max()
+    assert (diff > 0).float().mean() < 0.02, "more than a rounding's worth of elements differ"
+    ref = F.group_norm(y.double(), groups, gamma.double(), beta.double(), 1e-5)
+    ref = F.relu(ref) if relu else ref
+    assert orc.gn_rel_error(fused, ref) < 2e-2
+
+
+def test_statistics_follow_the_tensor_not_the_name(device):
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(8, 8, 32), padding=(1, 1, 1), dtype=torch.bfloat16)
+    ops = orc.make_inputs(prob, seed=5)
+    x, w = ops["input"].to(device), ops["weight"].to(device)
+    y = sa.conv3d_forward(x, w, None, 1, 1, 1, gn_groups=8)
+    y.add_(3.0)  # in place: the statistics on the tensor are stale now and must not be used
+    got = sa.group_norm(y, 8, None, None, 1e-5, None, out_dtype=None)
+    want = sa.group_norm(y.clone(memory_format=torch.preserve_format), 8, None, None, 1e-5, None, out_dtype=None)
+    assert torch.equal(got, want)
+    # another group count than announced: the ordinary pass as well
+    y2 = sa.conv3d_forward(x, w, None, 1, 1, 1, gn_groups=8)
+    assert torch.equal(sa.group_norm(y2, 4, None, None, 1e-5, None, out_dtype=None),
+                       sa.group_norm(y2.clone(memory_format=torch.preserve_format), 4, None, None, 1e-5, None, out_dtype=None))
+
+
+def test_where_the_statistics_are_not_offered(device):
+    bf = torch.bfloat16
+    # two samples on the persistent kernel, groups of two channels, fp32 tiles, direct kernels: plain forward, no attribute
+    for n, cin, cout, groups, dtype in [(2, 32, 32, 8, bf), (1, 32, 32, 16, bf), (1, 32, 32, 8, torch.float32), (1, 3, 6, 2, bf)]:
+        x = torch.randn(n, cin, 8, 8, 32, device=device).to(dtype).contiguous(memory_format=CL)
+        w = torch.randn(cout, cin, 3, 3, 3, device=device).to(dtype)
+        y = sa.conv3d_forward(x, w, None, 1, 1, 1, gn_groups=groups)
+        assert not hasattr(y, "_sfh_gn_partials")
+        assert torch.equal(y, sa.conv3d_forward(x, w, None, 1, 1, 1))
+
+
+def test_double_conv_with_and_without_the_handoff(device):
+    """The U-Net block: convolutions that announce their GroupNorm against the same block with the announcement off."""
+    torch.manual_seed(0)
+    block = DoubleConv(32, 64, 8).to(device).to(memory_format=CL)
+    x = torch.randn(1, 32, 8, 16, 32, device=device).contiguous(memory_format=CL)
+    assert block.double_conv[0].gn_groups == 8 and block.double_conv[3].gn_groups == 8
+
+    def run():
+        for p in block.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            out = block(xi)
+        out.float().square().mean().backward()
+        return out.detach(), xi.grad, [p.grad.clone() for p in block.parameters()]
+
+    fused = run()
+    for conv in (block.double_conv[0], block.double_conv[3]):
+        conv.gn_groups = 0
+    separate = run()
+    assert orc.gn_rel_error(fused[0], separate[0].double()) < 1e-2
+    assert orc.gn_rel_error(fused[1], separate[1].double()) < 2e-2
+    for a, b in zip(fused[2], separate[2]):
+        assert orc.gn_rel_error(a, b.double()) < 2e-2
