@@ -17,14 +17,18 @@ struct GnPartialOut {
   int groups, cg, records;
 };
 
-__device__ __forceinline__ void unpack2(bf16_t, uint32_t u, float& lo, float& hi) {
-  lo = bf16_lo(u);
-  hi = bf16_hi(u);
+// acc + lo(a) * lo(b) + hi(a) * hi(b) of two packed 16-bit pairs, products and sum in fp32 (v_dot2_f32_bf16 /
+// v_dot2_f32_f16: one instruction where unpacking and two multiply-adds take four), and the pair (1, 1).
+typedef __bf16 gn_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 gn_f16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_acc(bf16_t, uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(gn_bf16x2_t, a), __builtin_bit_cast(gn_bf16x2_t, b), acc, false);
 }
-__device__ __forceinline__ void unpack2(fp16_t, uint32_t u, float& lo, float& hi) {
-  lo = fp16_lo(u);
-  hi = fp16_hi(u);
+__device__ __forceinline__ float dot2_acc(fp16_t, uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(gn_f16x2_t, a), __builtin_bit_cast(gn_f16x2_t, b), acc, false);
 }
+__device__ __forceinline__ constexpr uint32_t ones2(bf16_t) { return 0x3f803f80u; }
+__device__ __forceinline__ constexpr uint32_t ones2(fp16_t) { return 0x3c003c00u; }
 
 // Sums of the four channel runs a lane holds of a 32-channel result block (run g = channels 8g + 4kg .. + 3, packed
 // as two rounded pairs), over the voxels the lane has added so far.
@@ -38,13 +42,12 @@ struct RunSums {
   __device__ __forceinline__ void add(const uint32_t (&run)[4][2], bool inside) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      float a, b, c, d;
-      unpack2(T{}, run[g][0], a, b);
-      unpack2(T{}, run[g][1], c, d);
-      const float t1 = (a + b) + (c + d);
-      const float t2 = fmaf(a, a, b * b) + fmaf(c, c, d * d);
-      s1[g] += inside ? t1 : 0.f;
-      s2[g] += inside ? t2 : 0.f;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint32_t v = inside ? run[g][h] : 0u;  // a voxel past the ragged edge counts as zeros
+        s1[g] = dot2_acc(T{}, v, ones2(T{}), s1[g]);
+        s2[g] = dot2_acc(T{}, v, v, s2[g]);
+      }
     }
   }
 };

@@ -222,22 +222,42 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
   for (int i = tid; i < 2 * G; i += kBlock) dst[i] = out[i];
 }
 
-// One 64-lane workgroup per (group, sample): fixed-order sum of the split partials, then
+// One workgroup per (group, sample): fixed-order sum of the split partials, then
 // mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps). A null `shift` stands for K = 0 (partials that
 // the producer of x summed unshifted).
-__global__ void __launch_bounds__(64) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
-                                                        float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
-                                                        float m, float eps) {
-  const int g = blockIdx.x, n = blockIdx.y;
+__global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
+                                                            float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
+                                                            float m, float eps) {
+  __shared__ float wsum[kBlock / 64][2];
+  const int g = blockIdx.x, n = blockIdx.y, tid = threadIdx.x;
+  const float* base = part + (int64_t)n * nsplit * 2 * G + g;
   float s1 = 0.f, s2 = 0.f;
-  for (int i = threadIdx.x; i < nsplit; i += 64) {
-    const float* p = part + ((int64_t)n * nsplit + i) * 2 * G;
-    s1 += p[g];
-    s2 += p[G + g];
+  // thread t owns records t, t + 256, ...: eight at a time, their loads all in flight before the first add
+  int i = tid;
+  for (; i + 7 * kBlock < nsplit; i += 8 * kBlock) {
+    float a[8], b[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float* p = base + (int64_t)(i + u * kBlock) * 2 * G;
+      a[u] = p[0];
+      b[u] = p[G];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { s1 += a[u]; s2 += b[u]; }
+  }
+  for (; i < nsplit; i += kBlock) {
+    const float* p = base + (int64_t)i * 2 * G;
+    s1 += p[0];
+    s2 += p[G];
   }
   s1 = wave_sum(s1);
   s2 = wave_sum(s2);
-  if (threadIdx.x == 0) {
+  if ((tid & 63) == 0) { wsum[tid >> 6][0] = s1; wsum[tid >> 6][1] = s2; }
+  __syncthreads();
+  if (tid == 0) {
+    s1 = s2 = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) { s1 += wsum[w][0]; s2 += wsum[w][1]; }
     const float d = s1 / m;
     float var = s2 / m - d * d;
     var = var < 0.f ? 0.f : var;
@@ -877,7 +897,7 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
   }
   const float m = (float)S * (float)(C / G);
   if (!fold_in_consumer_host(G, npart)) {
-    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(64), 0, st, shift, part, mean, rstd, G, npart, m, p.eps);
+    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(kBlock), 0, st, shift, part, mean, rstd, G, npart, m, p.eps);
     if (int rc = check_launch("gn_stats_finalize")) return rc;
   }
   hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
