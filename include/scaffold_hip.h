@@ -98,7 +98,8 @@ int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
  * voxels for the weight gradient) whose fp32 partials are summed in fixed order. A pure function of the problem and
  * the compute-unit count the library is written for -- the property the reference's plan machinery exists to
  * guarantee (triton_conv3d/_rungs.py, reduce_gemm.py:71-96: the split count must not depend on the device or the
- * run). [1] and [2] are 0 for SFH_KERNEL_DIRECT and SFH_KERNEL_OTHER_MATRIX (thin-channel, 2x2x2, fp32 tiles). */
+ * run). [1] and [2] are 0 for SFH_KERNEL_DIRECT (the direct and the thin-channel kernels: whatever
+ * sfh_conv3d_uses_mfma answers 0 for) and SFH_KERNEL_OTHER_MATRIX (2x2x2 family, fp32 tiles). */
 #define SFH_KERNEL_DIRECT 0
 #define SFH_KERNEL_PERSIST 1
 #define SFH_KERNEL_BRICK 2
@@ -124,8 +125,9 @@ int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const voi
  * their squares, per group, in fp32, into gn_partials[N][records][2][groups] -- every slot written by exactly one
  * workgroup, no atomics, the same bits on every run; sfh_groupnorm_fwd_from_partials folds the records in a fixed
  * order. sfh_conv3d_fwd_gn_records gives `records` for a problem and group count, a pure function of both; 0 means
- * the kernel that serves the problem does not offer it (direct / thin / fp32 kernels, several samples on the
- * persistent kernel, groups of fewer than 4 or a non-multiple-of-4 channels) and the caller uses sfh_conv3d_fwd and
+ * the kernel that serves the problem does not offer it (direct / fp32 / 2x2x2 kernels, thin-channel ones other than
+ * the one-channel 3x3x3 stem, several samples on the persistent kernel, groups of fewer than 4 or a non-multiple-of-4
+ * channels) and the caller uses sfh_conv3d_fwd and
  * the ordinary GroupNorm. 16-bit dtypes only. gn_partials must be 16-byte aligned. */
 int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype, int groups);
 int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w,

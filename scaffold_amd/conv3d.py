@@ -624,9 +624,12 @@ def conv3d_forward(
                                      None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                      _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
                                      _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
-            # valid for these bits of y only: the version lets the consumer see an in-place change
-            y._sfh_gn_partials = (partials, records, int(gn_groups), y._version)
-        else:
+            if rc == _lib.SFH_ERR_UNSUPPORTED:  # e.g. an out= view off the 16-byte grid: the plain launch
+                records = 0
+            else:
+                # valid for these bits of y only: the version lets the consumer see an in-place change
+                y._sfh_gn_partials = (partials, records, int(gn_groups), y._version)
+        if records == 0:
             rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
                                   None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                   _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(x.device))

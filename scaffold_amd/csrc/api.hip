@@ -367,7 +367,14 @@ static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, co
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
     return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st, gn);
   }
-  if (gn != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
+  if (gn != nullptr) {  // the one-channel stem is the only other kernel that leaves them
+    ThinArgs t;
+    if ((flags & SFH_FLAG_WEIGHT_PACKED) || thin_fwd_plan(*p, dtype, out, t) != kThinWideOut || thin_wide_out_gn_records(t, dtype, gn->groups) == 0)
+      return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
+    t.ws_kd = w_stride[2]; t.ws_kh = w_stride[3]; t.ws_kw = w_stride[4];
+    t.ws_wide = w_stride[0]; t.ws_thin = w_stride[1];
+    return thin_wide_out(t, dtype, x, w, bias, y, st, gn);
+  }
   if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && fwd_uses_f32_tiles(*p, dtype, out)) {
     const MfmaConvArgs a = fwd_mfma_args(*p, out);
     const size_t need = f32_conv_packed_weight_bytes(a);
@@ -419,8 +426,11 @@ extern "C" int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x
 extern "C" int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype, int groups) {
   int32_t out[3];
   if (check_conv(p, dtype, out) != SFH_OK || groups < 1 || p->n == 0) return 0;
-  if (!fwd_uses_mfma(*p, dtype, out)) return 0;
-  return mfma_conv_gn_records(fwd_mfma_args(*p, out), groups);
+  if (fwd_uses_mfma(*p, dtype, out)) return mfma_conv_gn_records(fwd_mfma_args(*p, out), groups);
+  if (fwd_uses_f32_tiles(*p, dtype, out) || fwd_uses_patch(*p, dtype, out)) return 0;
+  ThinArgs t;
+  if (thin_fwd_plan(*p, dtype, out, t) == kThinWideOut) return thin_wide_out_gn_records(t, dtype, groups);
+  return 0;
 }
 
 extern "C" int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],

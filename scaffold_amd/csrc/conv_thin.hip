@@ -598,8 +598,8 @@ __device__ __forceinline__ int stem_tap_offset(int j) { return ((j / 9) * kSBH +
 template <typename T, int NC>
 __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const T* __restrict__ x, const T* __restrict__ wt,
                                                                const T* __restrict__ bias, T* __restrict__ out, int tiles_d,
-                                                               int tiles_h, int tiles_w) {
-  __shared__ uint16_t brick[kSBV];
+                                                               int tiles_h, int tiles_w, GnPartialOut gn) {
+  __shared__ __attribute__((aligned(16))) uint16_t brick[kSBV];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 31, kg = lane >> 5;
   // result tile: rows = output channels (weights), columns = voxels (taps of the voxel)
@@ -632,6 +632,9 @@ __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const
   const StemTile t = stem_tile(a, blockIdx.x, tiles_h, tiles_w, tiles_d);
   stem_stage_bits<T>(a, x, t, brick);
   __syncthreads();
+  RunSums gn_sums[NC];  // GroupNorm statistics of the rounded output, when the caller wants them
+#pragma unroll
+  for (int cc = 0; cc < NC; ++cc) gn_sums[cc].clear();
 #pragma unroll 1
   for (int i = 0; i < 4; ++i) {
     const int run = wave * 4 + i, row = run >> 1;
@@ -659,8 +662,14 @@ __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[ks], acc);
-      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid);
+      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid, gn_sums[cc], gn.part != nullptr);
     }
+  }
+  if (gn.part != nullptr) {
+    __syncthreads();  // every wave is done reading the brick: the LDS is free
+    static_assert(sizeof(brick) >= (kBlock / 64) * NC * 16 * sizeof(float), "room for the wavefronts' sums");
+    write_group_partials<kBlock / 64, NC>(gn_sums, reinterpret_cast<float*>(brick), gn, t.n,
+                                          (int)(blockIdx.x % (unsigned)(tiles_d * tiles_h * tiles_w)), 0, tid);
   }
 }
 
@@ -761,6 +770,11 @@ int64_t stem_tiles(const ThinArgs& a) {
   return (int64_t)a.n * cdiv(a.od, kSTD) * cdiv(a.oh, kSTH) * cdiv(a.ow, kSTW);
 }
 
+// the one-channel 3x3x3 stem on the matrix cores (16-bit types): 32 or 64 output channels
+bool stem_matrix_ok(const ThinArgs& a) {
+  return stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL && (a.cw == 32 || a.cw == 64);
+}
+
 int wide_channels_ok(const ThinArgs& a, int dtype) {
   const int v = dtype == SFH_FP32 ? 4 : 8;
   return a.cw % v == 0 && a.cw / v <= kBlock && a.cw >= v;
@@ -817,16 +831,18 @@ int launch_head_wide_out(const ThinArgs& a, const void* thin, const void* wt, co
 
 // J is padded to the next instantiated size; K in {0 (channels), 2, 3}.
 template <typename T>
-int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
+int dispatch_wide_out(const ThinArgs& a, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st,
+                      const GnPartialOut& gn) {
   if constexpr (sizeof(T) == 2) {
-    if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL && (a.cw == 32 || a.cw == 64) && (uintptr_t)out % 16 == 0) {
+    if (stem_matrix_ok(a) && (uintptr_t)out % 16 == 0) {
       const dim3 grid((unsigned)stem_tiles(a));
       const int td = (int)cdiv(a.od, kSTD), th = (int)cdiv(a.oh, kSTH), tw = (int)cdiv(a.ow, kSTW);
-      if (a.cw == 32) hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw);
-      else hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw);
+      if (a.cw == 32) hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw, gn);
+      else hipLaunchKernelGGL((stem_fwd_mfma_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt, (const T*)bias, (T*)out, td, th, tw, gn);
       return check_launch("stem_fwd_mfma_kernel");
     }
   }
+  if (gn.part != nullptr) return fail(SFH_ERR_UNSUPPORTED, "thin-channel conv: GroupNorm partials need the matrix-core stem kernel and a 16-byte aligned output");
   if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL) {
     hipLaunchKernelGGL(stem_fwd_kernel<T>, dim3((unsigned)stem_tiles(a)), dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wt,
                        (const T*)bias, (T*)out, (int)cdiv(a.od, kSTD), (int)cdiv(a.oh, kSTH), (int)cdiv(a.ow, kSTW));
@@ -927,8 +943,22 @@ size_t thin_reduce_workspace_bytes(const ThinArgs& a) {
     default: return fn<float>(__VA_ARGS__);                \
   }
 
-int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st) {
-  SFH_THIN_BY_DTYPE(dispatch_wide_out, a, thin, wt, bias, out, st)
+int thin_wide_out_gn_records(const ThinArgs& a, int dtype, int groups) {
+  if ((dtype != SFH_BF16 && dtype != SFH_FP16) || !stem_matrix_ok(a) || !gn_partials_fit(a.cw, groups, a.cw)) return 0;
+  return (int)(stem_tiles(a) / a.n);
+}
+
+int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st,
+                  const GnPartialOut* gn) {
+  GnPartialOut o{nullptr, 0, 0, 0};
+  if (gn != nullptr && gn->part != nullptr) {
+    if (gn->records == 0 || gn->records != thin_wide_out_gn_records(a, dtype, gn->groups))
+      return fail(SFH_ERR_INVALID, "thin-channel conv: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
+                  thin_wide_out_gn_records(a, dtype, gn->groups));
+    o = *gn;
+    o.cg = a.cw / gn->groups;
+  }
+  SFH_THIN_BY_DTYPE(dispatch_wide_out, a, thin, wt, bias, out, st, o)
 }
 int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st) {
   SFH_THIN_BY_DTYPE(dispatch_thin_out, a, wide, wt, bias, out, st)

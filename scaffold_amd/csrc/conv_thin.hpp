@@ -1,6 +1,7 @@
 // Host-side interface of the thin-channel convolution kernels (one channel count below MFMA tile size).
 #pragma once
 #include "common.hpp"
+#include "gn_stats.hpp"
 
 namespace sfh {
 
@@ -23,7 +24,11 @@ struct ThinArgs {
 
 bool thin_supported(const ThinArgs& a, int dtype);
 // out[v][c] = bias[c] + sum_j s_j(v) * W[j][c]
-int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st);
+// `gn` (optional): also leave GroupNorm partials of the rounded output (gn_stats.hpp), gn->records per sample as
+// thin_wide_out_gn_records says (0: this problem's kernel does not offer them).
+int thin_wide_out_gn_records(const ThinArgs& a, int dtype, int groups);
+int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st,
+                  const GnPartialOut* gn = nullptr);
 // out[v][j] = bias[j] + sum_c wide[v][c] * W[j][c]
 int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st);
 // G[j][c] = sum_v s_j(v) * wide[v][c], through fp32 partial slices in `ws`

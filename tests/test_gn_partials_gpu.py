@@ -23,6 +23,8 @@ CL = torch.channels_last_3d
 
 # (n, cin, cout, spatial, padding, groups, kernel that serves the forward)
 CASES = [
+    (1, 1, 32, (8, 16, 64), (1, 1, 1), 8, "direct"),           # the one-channel stem (thin-channel kernel on the matrix cores)
+    (2, 1, 64, (5, 6, 70), (0, 1, 1), 4, "direct"),            # two samples, ragged, 64 channels
     (1, 32, 32, (8, 8, 32), (1, 1, 1), 8, "persist"),          # 4 channels per group: two groups per lane run pair
     (1, 32, 32, (5, 7, 33), (1, 1, 1), 4, "persist"),          # ragged tiles on every axis
     (1, 32, 64, (6, 9, 40), (0, 1, 1), 8, "persist"),          # shard form, two output blocks
