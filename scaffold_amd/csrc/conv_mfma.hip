@@ -68,11 +68,12 @@ __device__ __forceinline__ constexpr int lds_off(int it) {
   return ((kd * C::BH + kh) * C::BW + kw) * 16 + ks * 2 * C::PLANE;
 }
 
-template <typename T, typename C>
+// WQ: weight fragments in flight per wavefront (see the chunk loop).
+template <typename T, typename C, int WQ>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
                  T* __restrict__ y, float* __restrict__ partial, int tiles_d, int tiles_h, int tiles_w, int nblocks, int ksplit,
-                 uint32_t total, GnPartialOut gn) {
+                 uint32_t total, GnPartialOut gn, int early_weights) {
   __shared__ __attribute__((aligned(16))) char lds[C::LDS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -121,13 +122,21 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     const T* wcc = wp + ((int64_t)(nb * C::NSUB) * ncc + cc) * (C::TAPS * 2 * FRAG) + lane * 8;
     const int64_t wns = (int64_t)ncc * (C::TAPS * 2 * FRAG);  // next 32-channel output block
     constexpr int NIT = C::TAPS * 2;
-    // Weight fragments in flight per wavefront. A fragment feeds MS x NSUB MFMAs (32 cycles each): the fewer those are,
-    // the more fragments must be under way to cover a trip to L2 or HBM.
-    constexpr int WWANT = C::NSUB > 1 ? 4 : (C::MS >= 4 ? 6 : 12);
+    // Weight fragments in flight per wavefront: WQ. A fragment feeds MS x NSUB MFMAs (32 cycles each): the fewer those
+    // are, the more fragments must be under way to cover a trip to L2 or HBM -- 4 with two output blocks (registers), 6
+    // for 512-voxel tiles, 12 for 256-voxel tiles when the launch is one round of workgroups (each then waits out its
+    // own cold misses), 6 when it is several rounds (two resident workgroups cover for each other; the deeper queue
+    // only costs registers and cache there).
+    constexpr int WWANT = WQ;
     constexpr int WDEPTH = NIT < WWANT ? NIT : WWANT;
     uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
-    constexpr bool EARLY_WEIGHTS = C::NSUB == 1;  // with two output blocks the staging needs the registers
-    if constexpr (EARLY_WEIGHTS) {
+    constexpr bool CAN_EARLY = C::NSUB == 1;  // with two output blocks the staging needs the registers
+#ifdef SFH_GATHER_TUNE  // a tuning build can switch it off per launch to measure it
+    const bool early = CAN_EARLY && early_weights != 0;
+#else
+    constexpr bool early = CAN_EARLY;
+#endif
+    if (early) {
 #pragma unroll
       for (int it = 0; it < WDEPTH; ++it) wq[it][0] = *reinterpret_cast<const uint4*>(wcc + it * FRAG);
     }
@@ -175,7 +184,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     // of iteration it+WDEPTH and the activation fragments of iteration it+1 are requested before the
     // MFMAs of iteration it are issued, so L2 and LDS latency overlap the matrix pipe.
     uint4 aq[2][C::MS];
-    if constexpr (!EARLY_WEIGHTS) {
+    if (!early) {
 #pragma unroll
       for (int it = 0; it < WDEPTH; ++it)
 #pragma unroll
@@ -398,6 +407,15 @@ GatherPlan gather_plan(const MfmaConvArgs& a) {
   return p;
 }
 
+// A chunk's first weight requests ahead of its brick staging: always, except that a tuning build reads an override.
+int early_weights(int64_t workgroups) {
+#ifdef SFH_GATHER_TUNE
+  if (const char* e = getenv("SFH_EARLY_WEIGHTS")) return atoi(e) == 2 ? (workgroups <= 2 * kComputeUnits) : atoi(e);
+#endif
+  (void)workgroups;
+  return 1;
+}
+
 template <typename T, typename C>
 int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
                float* partial, hipStream_t st, const GnPartialOut& gn) {
@@ -406,8 +424,15 @@ int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const 
   const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks * p.ksplit;
   if (total == 0) return SFH_OK;
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: %lld workgroups exceed the grid limit", (long long)total);
-  hipLaunchKernelGGL((conv_mfma_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
-                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total, gn);
+#define SFH_BRICK(WQ)                                                                                                      \
+  hipLaunchKernelGGL((conv_mfma_kernel<T, C, WQ>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed, \
+                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total, gn,     \
+                     early_weights(total))
+  if constexpr (C::NSUB > 1) SFH_BRICK(4);
+  else if constexpr (C::MS >= 4) SFH_BRICK(6);
+  else if (total <= 2 * kComputeUnits) SFH_BRICK(12);
+  else SFH_BRICK(6);
+#undef SFH_BRICK
   return check_launch("conv_mfma_kernel");
 }
 
