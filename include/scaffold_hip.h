@@ -124,7 +124,11 @@ int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const voi
  * written once) becomes one read and one write. The convolution's workgroups add up the ROUNDED values they store and
  * their squares, per group, in fp32, into gn_partials[N][records][2][groups] -- every slot written by exactly one
  * workgroup, no atomics, the same bits on every run; sfh_groupnorm_fwd_from_partials folds the records in a fixed
- * order. sfh_conv3d_fwd_gn_records gives `records` for a problem and group count, a pure function of both; 0 means
+ * order. The values are summed minus a shift gn_shift[N][groups] (device memory; NULL = zeros) that the same pointer
+ * hands to the GroupNorm call: any number near the group's mean -- the mean the layer had at its previous call is one --
+ * keeps the variance from cancelling however large the mean is against the spread, which is what the reference's
+ * Welford merge (triton_group_norm.py:148-165) is for; without one the variance carries a relative error of about
+ * 3e-7 (mean/std)^2. sfh_conv3d_fwd_gn_records gives `records` for a problem and group count, a pure function of both; 0 means
  * the kernel that serves the problem does not offer it (direct / fp32 / 2x2x2 kernels, thin-channel ones other than
  * the one-channel 3x3x3 stem, several samples on the persistent kernel, groups of fewer than 4 or a non-multiple-of-4
  * channels) and the caller uses sfh_conv3d_fwd and
@@ -132,8 +136,8 @@ int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const voi
 int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype, int groups);
 int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w,
                       const int64_t w_stride[5], const void* bias, void* y, void* workspace,
-                      size_t workspace_bytes, uint32_t flags, int groups, float* gn_partials,
-                      size_t gn_partials_bytes, void* stream);
+                      size_t workspace_bytes, uint32_t flags, int groups, const float* gn_shift,
+                      float* gn_partials, size_t gn_partials_bytes, void* stream);
 
 /* ---- conv3d data gradient ------------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_backward_data (triton_conv3d/bwd_data.py:275).
@@ -226,13 +230,14 @@ int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype
                            int64_t halo_rows, float* mean, float* rstd, void* workspace,
                            size_t workspace_bytes, void* stream);
 /* The same again with the statistics taken from partial sums the producer of x left
- * (sfh_conv3d_fwd_gn): partials[N][records][2][groups], unshifted sums and sums of squares of x per group.
+ * (sfh_conv3d_fwd_gn): partials[N][records][2][groups], sums of x - shift and of its square per group, and the
+ * shift[N][groups] they were taken about (NULL = zeros; must not be the `mean` output of this call).
  * No statistics pass and no workspace; halo_rows may be 0 (y_slab is then a plain output). Needs the vector path
  * (16-byte aligned tensors, channel counts the 16-byte vectors divide): SFH_ERR_UNSUPPORTED otherwise. */
 int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
                                     const void* x, const void* gamma, const void* beta, void* y_slab,
                                     int64_t halo_rows, float* mean, float* rstd, const float* partials,
-                                    int32_t records, void* stream);
+                                    int32_t records, const float* shift, void* stream);
 
 /* The forward for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc. It has no counterpart in the reference. Same kernels and results as sfh_groupnorm_fwd, but the

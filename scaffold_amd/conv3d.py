@@ -568,6 +568,7 @@ def conv3d_forward(
     force_generic: bool = False,
     packed_weight: Optional[torch.Tensor] = None,
     gn_groups: int = 0,
+    gn_shift: Optional[torch.Tensor] = None,
     _checked: bool = False,
 ) -> torch.Tensor:
     """Forward 3-D convolution; input and output are ``channels_last_3d``.
@@ -580,7 +581,9 @@ def conv3d_forward(
     ``gn_groups > 0`` announces a GroupNorm of that many groups on the result: where the kernel that serves the problem
     offers it, the launch also leaves the per-group sums of its (rounded) output, which ride along as
     ``result._sfh_gn_partials`` and spare :func:`scaffold_amd.group_norm` its statistics pass. The result itself is the
-    same bits either way.
+    same bits either way. ``gn_shift`` (fp32, ``(N, gn_groups)``, on the device) is what the values are summed about: any
+    number near each group's mean -- the means of the layer's previous call do -- keeps the variance exact at means far
+    larger than the spread; without it the sums are plain (fine up to a mean of some tens of standard deviations).
     """
     if not _checked and not is_supported(x, w, bias, stride, padding, dilation, groups):
         raise NotImplementedError(
@@ -619,16 +622,19 @@ def conv3d_forward(
         ws = _lib.workspace(need, x.device)
         records = prob.gn_records(gn_groups) if gn_groups > 0 and not force_generic else 0
         if records > 0:
+            if gn_shift is not None and (gn_shift.dtype is not torch.float32 or gn_shift.shape != (prob.n, gn_groups)
+                                         or gn_shift.device != x.device or not gn_shift.is_contiguous()):
+                gn_shift = None  # not the shape of this call (another batch size, say): plain sums
             partials = torch.empty(prob.n * records * 2 * gn_groups, dtype=torch.float32, device=x.device)
             rc = L.sfh_conv3d_fwd_gn(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
                                      None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                      _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
-                                     _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+                                     _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
             if rc == _lib.SFH_ERR_UNSUPPORTED:  # e.g. an out= view off the 16-byte grid: the plain launch
                 records = 0
             else:
                 # valid for these bits of y only: the version lets the consumer see an in-place change
-                y._sfh_gn_partials = (partials, records, int(gn_groups), y._version)
+                y._sfh_gn_partials = (partials, records, int(gn_groups), y._version, gn_shift)
         if records == 0:
             rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
                                   None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),

@@ -435,14 +435,14 @@ extern "C" int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype
 
 extern "C" int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
                                  const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, int groups,
-                                 float* gn_partials, size_t gn_partials_bytes, void* stream) {
+                                 const float* gn_shift, float* gn_partials, size_t gn_partials_bytes, void* stream) {
   if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d fwd: the direct kernels leave no GroupNorm partials");
   const int32_t records = sfh_conv3d_fwd_gn_records(p, dtype, groups);
   if (records == 0) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
   const size_t need = (size_t)p->n * records * 2 * groups * sizeof(float);
   if (gn_partials == nullptr || gn_partials_bytes < need || (reinterpret_cast<uintptr_t>(gn_partials) & 15u) != 0)
     return fail(SFH_ERR_WORKSPACE, "conv3d fwd: GroupNorm partials need %zu bytes at a 16-byte boundary, got %zu", need, gn_partials_bytes);
-  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records};
+  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records, gn_shift};
   return conv3d_fwd_any(p, dtype, x, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, &gn);
 }
 

@@ -223,7 +223,10 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   // GroupNorm statistics of the rounded output, when the caller wants them (the reduction is not sliced then).
   RunSums gn_sums[C::NSUB];
 #pragma unroll
-  for (int ns = 0; ns < C::NSUB; ++ns) gn_sums[ns].clear();
+  for (int ns = 0; ns < C::NSUB; ++ns) {
+    gn_sums[ns].clear();
+    if (gn.part != nullptr) gn_sums[ns].load_shift(gn.shift, n, gn.groups, gn.cg, (nb * C::NSUB + ns) * 32, kg);
+  }
 
   // Epilogue. Accumulator register r of a lane is output channel 8*(r/4) + 4*kg + r%4 of the
   // sub-tile's voxel j: four runs of four consecutive channels per 32-channel block. For the 16-bit output the two
@@ -471,7 +474,7 @@ int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* pa
                  hipStream_t st, const GnPartialOut* gn) {
   const GatherPlan p = gather_plan(a);
   if (p.ksplit > 1 && partial == nullptr) return fail(SFH_ERR_WORKSPACE, "conv mfma: the reduction split needs its workspace");
-  GnPartialOut out{nullptr, 0, 0, 0};
+  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records != gather_gn_records(a, p, gn->groups) || gn->records == 0)
       return fail(SFH_ERR_INVALID, "conv mfma: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
@@ -479,7 +482,7 @@ int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* pa
     out = *gn;
     out.cg = a.cout / gn->groups;
   }
-  const GnPartialOut none{nullptr, 0, 0, 0};
+  const GnPartialOut none{nullptr, 0, 0, 0, nullptr};
   const GnPartialOut& in_kernel = p.ksplit == 1 ? out : none;
   const int rc = p.nsub == 2 ? launch_k333<T, 2>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel)
                              : launch_k333<T, 1>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel);

@@ -10,6 +10,9 @@
 // [voxel][channel] layout and read with ds_read_b64_tr_b16, which hands each lane four consecutive
 // voxels of one channel.
 #include "conv_patch.hpp"
+#ifdef SFH_PATCH_TUNE
+#include <cstdlib>
+#endif
 #include <type_traits>
 #include "mma.hpp"
 #include "reduce.hpp"
@@ -318,11 +321,18 @@ int launch_scatter(const PatchArgs& a, const void* small, const void* packed, co
   const int64_t total = small_voxels(a);
   dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
   const int64_t wgs = (int64_t)grid.x * grid.y;
-  if (wgs < kComputeUnits) {  // under one workgroup per CU: one tap per workgroup
+  int force = 0;
+#ifdef SFH_PATCH_TUNE
+  if (const char* e = getenv("SFH_SCATTER_TS")) force = atoi(e);
+#endif
+  if (force == 8) {
+    hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
+                       (const T*)bias, (T*)big, total);
+  } else if (force == 1 || (force == 0 && wgs < kComputeUnits)) {  // under one workgroup per CU: one tap per workgroup
     grid.z = kTaps;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total);
-  } else if (wgs <= 4 * kComputeUnits) {  // up to four per CU: two taps (the big voxels next to each other along W)
+  } else if (force == 2 || (force == 0 && wgs <= 4 * kComputeUnits)) {  // up to four per CU: two taps (the big voxels next to each other along W)
     grid.z = kTaps / 2;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total);

@@ -371,6 +371,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   T* done_origin = y;
   RunSums gn_sums;  // GroupNorm statistics of this workgroup's rounded outputs (GN)
   gn_sums.clear();
+  if constexpr (GN) gn_sums.load_shift(gn.shift, 0, gn.groups, gn.cg, nb * 32, kg);
 
   for (int step = 0; step < nsteps; ++step) {
     const TileCoord tc2 = next_tile(tc1, gm);
@@ -484,7 +485,7 @@ int mfma_conv_gn_records(const MfmaConvArgs& a, int groups) {
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st, const GnPartialOut* gn) {
   if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st, gn);
-  GnPartialOut out{nullptr, 0, 0, 0};
+  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_gn_records(a, gn->groups))
       return fail(SFH_ERR_INVALID, "conv persist: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

@@ -634,7 +634,10 @@ __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const
   __syncthreads();
   RunSums gn_sums[NC];  // GroupNorm statistics of the rounded output, when the caller wants them
 #pragma unroll
-  for (int cc = 0; cc < NC; ++cc) gn_sums[cc].clear();
+  for (int cc = 0; cc < NC; ++cc) {
+    gn_sums[cc].clear();
+    if (gn.part != nullptr) gn_sums[cc].load_shift(gn.shift, t.n, gn.groups, gn.cg, cc * 32, kg);
+  }
 #pragma unroll 1
   for (int i = 0; i < 4; ++i) {
     const int run = wave * 4 + i, row = run >> 1;
@@ -950,7 +953,7 @@ int thin_wide_out_gn_records(const ThinArgs& a, int dtype, int groups) {
 
 int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st,
                   const GnPartialOut* gn) {
-  GnPartialOut o{nullptr, 0, 0, 0};
+  GnPartialOut o{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != thin_wide_out_gn_records(a, dtype, gn->groups))
       return fail(SFH_ERR_INVALID, "thin-channel conv: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

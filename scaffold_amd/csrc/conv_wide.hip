@@ -333,7 +333,10 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   const int wave_out = tid_out >> 6, j_out = tid_out & 31, kg_out = (tid_out >> 5) & 1;
   RunSums gn_sums[C::NSUB];  // GroupNorm statistics of the rounded output, when the caller wants them
 #pragma unroll
-  for (int ns = 0; ns < C::NSUB; ++ns) gn_sums[ns].clear();
+  for (int ns = 0; ns < C::NSUB; ++ns) {
+    gn_sums[ns].clear();
+    if (gn.part != nullptr) gn_sums[ns].load_shift(gn.shift, n, gn.groups, gn.cg, (nb * C::NSUB + ns) * 32, kg_out);
+  }
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     const int v = (wave_out * C::MS + ms) * 32 + j_out;
@@ -458,7 +461,7 @@ int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* 
                    const GnPartialOut* gn) {
   const WidePlan p = wide_plan(a);
   if (!p.use) return fail(SFH_ERR_UNSUPPORTED, "conv wide: not applicable to this problem");
-  GnPartialOut out{nullptr, 0, 0, 0};
+  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_wide_gn_records(a, gn->groups))
       return fail(SFH_ERR_INVALID, "conv wide: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

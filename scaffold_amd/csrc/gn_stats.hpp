@@ -1,53 +1,62 @@
-// GroupNorm statistics emitted by the kernel that produces the tensor: unshifted sums of the ROUNDED outputs (the bits
-// the normalisation will read back) and of their squares, per group, one record per producer workgroup:
+// GroupNorm statistics emitted by the kernel that produces the tensor: sums of the ROUNDED outputs (the bits the
+// normalisation will read back) minus a shift K, and of the squares of those differences, per group, one record per
+// producer workgroup:
 //   part[sample][record][2][G]      (the layout the GroupNorm kernels fold: quantity 0 = sum, 1 = sum of squares)
+// K[sample][group] comes from the caller -- any value near the group's mean, e.g. the mean the same layer had at its
+// previous call; a null pointer stands for zeros. With K within a few standard deviations of the mean the variance
+// S2/m - (S1/m)^2 does not cancel, however large the mean is against the spread (the job of the Welford merge in the
+// reference, triton_group_norm.py:148-165); with K = 0 the fp32 sums still carry a relative variance error of about
+// 3e-7 (mean/std)^2, below a bf16 output's own rounding up to |mean| = 100 std.
 // No atomics: every (record, group) slot is written by exactly one workgroup, the sums inside a workgroup are added in
 // a fixed order, and the GroupNorm kernels add the records in a fixed order, so the statistics are reproducible.
-// Offered for 16-bit outputs only: fp32 sums of 16-bit values keep more than the 8 (bf16) / 11 (fp16) bits of the data
-// for any mean a tensor of such values can have relative to its spread, so the shift the stand-alone statistics pass
-// uses (for fp32 tensors at mean >> std) is not needed here.
 #pragma once
 #include "common.hpp"
 
 namespace sfh {
 
-// Where a producer writes, or nothing (part == nullptr). `records` per sample; `cg` channels per group.
+// Where a producer writes, or nothing (part == nullptr). `records` per sample; `cg` channels per group; `shift` is
+// K[sample][group] or null.
 struct GnPartialOut {
   float* part;
   int groups, cg, records;
+  const float* shift;
 };
 
-// acc + lo(a) * lo(b) + hi(a) * hi(b) of two packed 16-bit pairs, products and sum in fp32 (v_dot2_f32_bf16 /
-// v_dot2_f32_f16: one instruction where unpacking and two multiply-adds take four), and the pair (1, 1).
-typedef __bf16 gn_bf16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 gn_f16x2_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ float dot2_acc(bf16_t, uint32_t a, uint32_t b, float acc) {
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(gn_bf16x2_t, a), __builtin_bit_cast(gn_bf16x2_t, b), acc, false);
+__device__ __forceinline__ void unpack2(bf16_t, uint32_t u, float& lo, float& hi) {
+  lo = bf16_lo(u);
+  hi = bf16_hi(u);
 }
-__device__ __forceinline__ float dot2_acc(fp16_t, uint32_t a, uint32_t b, float acc) {
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(gn_f16x2_t, a), __builtin_bit_cast(gn_f16x2_t, b), acc, false);
+__device__ __forceinline__ void unpack2(fp16_t, uint32_t u, float& lo, float& hi) {
+  lo = fp16_lo(u);
+  hi = fp16_hi(u);
 }
-__device__ __forceinline__ constexpr uint32_t ones2(bf16_t) { return 0x3f803f80u; }
-__device__ __forceinline__ constexpr uint32_t ones2(fp16_t) { return 0x3c003c00u; }
 
 // Sums of the four channel runs a lane holds of a 32-channel result block (run g = channels 8g + 4kg .. + 3, packed
-// as two rounded pairs), over the voxels the lane has added so far.
+// as two rounded pairs), over the voxels the lane has added so far; k[g] is the shift of run g's group.
 struct RunSums {
-  float s1[4], s2[4];
+  float s1[4], s2[4], k[4];
   __device__ __forceinline__ void clear() {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) s1[g] = s2[g] = 0.f;
+    for (int g = 0; g < 4; ++g) s1[g] = s2[g] = k[g] = 0.f;
+  }
+  // The shifts of the block whose first channel is c0 (a multiple of 32), for the lane's k-half kg and sample n.
+  __device__ __forceinline__ void load_shift(const float* shift, int n, int groups, int cg, int c0, int kg) {
+    if (shift == nullptr) return;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) k[g] = shift[n * groups + (c0 + 8 * g + 4 * kg) / cg];
   }
   template <typename T>
   __device__ __forceinline__ void add(const uint32_t (&run)[4][2], bool inside) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const uint32_t v = inside ? run[g][h] : 0u;  // a voxel past the ragged edge counts as zeros
-        s1[g] = dot2_acc(T{}, v, ones2(T{}), s1[g]);
-        s2[g] = dot2_acc(T{}, v, v, s2[g]);
-      }
+      float a, b, c, d;
+      unpack2(T{}, run[g][0], a, b);
+      unpack2(T{}, run[g][1], c, d);
+      a -= k[g]; b -= k[g]; c -= k[g]; d -= k[g];
+      const float t1 = (a + b) + (c + d);
+      const float t2 = fmaf(a, a, b * b) + fmaf(c, c, d * d);
+      s1[g] += inside ? t1 : 0.f;  // a voxel past the ragged edge counts as nothing
+      s2[g] += inside ? t2 : 0.f;
     }
   }
 };

@@ -859,7 +859,7 @@ size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
 template <typename T, typename TO>
 int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
               void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st, const float* given_part = nullptr,
-              int given_npart = 0) {
+              int given_npart = 0, const float* given_shift = nullptr) {
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
   if (y_halo > 0 && (!pl.vector || sizeof(T) != sizeof(TO) || (y_halo * C * sizeof(TO)) % 16 != 0))
@@ -875,7 +875,7 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
     return check_launch("gn_scalar_normalize");
   }
   const dim3 grid(pl.nsplit, p.n);
-  const float* shift = nullptr;
+  const float* shift = given_shift;  // of the given partials (null: zeros)
   const float* part = given_part;
   int npart = given_npart;
   if (given_part == nullptr) {
@@ -961,7 +961,8 @@ extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p,
 
 static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x, const void* gamma,
                              const void* beta, void* y, int64_t y_halo, float* mean, float* rstd, void* workspace,
-                             size_t workspace_bytes, void* stream, const float* given_part = nullptr, int given_npart = 0) {
+                             size_t workspace_bytes, void* stream, const float* given_part = nullptr, int given_npart = 0,
+                             const float* given_shift = nullptr) {
   if (int rc = check_desc(p, x_dtype)) return rc;
   if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
   if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
@@ -975,7 +976,7 @@ static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dty
   hipStream_t st = (hipStream_t)stream;
   float* ws = (float*)workspace;
 #define SFH_GN_FWD(TX, TY) \
-  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart)
+  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart, given_shift)
   if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
@@ -1003,11 +1004,12 @@ extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, 
 
 extern "C" int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
                                                const void* gamma, const void* beta, void* y_slab, int64_t halo_rows, float* mean,
-                                               float* rstd, const float* partials, int32_t records, void* stream) {
+                                               float* rstd, const float* partials, int32_t records, const float* shift,
+                                               void* stream) {
   if (partials == nullptr || records < 1) return fail(SFH_ERR_INVALID, "groupnorm from partials: no partial sums given");
   if (!aligned16(partials)) return fail(SFH_ERR_INVALID, "groupnorm from partials: the partial sums must be 16-byte aligned");
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, nullptr, 0, stream, partials,
-                           records);
+                           records, shift);
 }
 
 // ---- the forward for callers that may not allocate ------------------------------------------------------------------

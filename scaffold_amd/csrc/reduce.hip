@@ -144,6 +144,7 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const flo
   const int c = (tid * 4) % channels;
   float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
   if (bias != nullptr) { b0 = to_float(bias[c]); b1 = to_float(bias[c + 1]); b2 = to_float(bias[c + 2]); b3 = to_float(bias[c + 3]); }
+  const float shift = gn.shift != nullptr ? gn.shift[n * gn.groups + c / gn.cg] : 0.f;  // the thread's four channels share a group
   float s1 = 0.f, s2 = 0.f;
   for (int k = 0; k < chunks; ++k) {
     const int64_t local = ((int64_t)blockIdx.x * chunks + k) * kStatsPiece + tid * 4;
@@ -157,7 +158,7 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const flo
     const T o0 = elem<T>::from_float(s.x + b0), o1 = elem<T>::from_float(s.y + b1), o2 = elem<T>::from_float(s.z + b2),
             o3 = elem<T>::from_float(s.w + b3);
     out[e] = o0; out[e + 1] = o1; out[e + 2] = o2; out[e + 3] = o3;
-    const float r0 = to_float(o0), r1 = to_float(o1), r2 = to_float(o2), r3 = to_float(o3);
+    const float r0 = to_float(o0) - shift, r1 = to_float(o1) - shift, r2 = to_float(o2) - shift, r3 = to_float(o3) - shift;
     s1 += (r0 + r1) + (r2 + r3);
     s2 += fmaf(r0, r0, r1 * r1) + fmaf(r2, r2, r3 * r3);
   }

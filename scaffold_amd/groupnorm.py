@@ -162,12 +162,13 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, o
                 ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
                 _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out if slab is None else slab),
                 0 if slab is None else out_halo * int(input.shape[3]) * int(input.shape[4]),
-                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(given[0]), given[1], _lib.stream_ptr(input.device))
+                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(given[0]), given[1], _lib.ptr(given[4]), _lib.stream_ptr(input.device))
         if rc == _lib.SFH_ERR_UNSUPPORTED:
             rc = _launch_forward(L, desc, xcode, odt, need, input, weight, bias, out, slab, out_halo, mean, rstd)
             if isinstance(rc, tuple):
                 rc, out = rc
     _lib.check(rc, "group_norm")
+    out._sfh_gn_mean = mean  # for a producer that wants a shift for its next call's sums
     return out, mean, rstd
 
 

@@ -119,7 +119,7 @@ class _Conv3dFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None,
-                gn_groups=0):
+                gn_groups=0, gn_shift=None):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
@@ -140,7 +140,8 @@ class _Conv3dFn(torch.autograd.Function):
             # host time is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
             pf, pd = _c3.pack_weights(wc, x.shape, stride, padding, dilation)
         # gn_groups: a GroupNorm of that many groups follows; the launch leaves its statistics on y where it can
-        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, _checked=True)
+        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, gn_shift=gn_shift,
+                               _checked=True)
         ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
@@ -165,7 +166,7 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
@@ -212,6 +213,18 @@ class FastConv3d(nn.Conv3d):
     #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
+    #: that GroupNorm module, in a tuple (so that it is not registered as a child): the group means of its last call are
+    #: what this call's sums are taken about
+    gn_follower = ()
+
+    def _gn_shift(self):
+        if not self.gn_follower or self.gn_groups <= 0:
+            return None
+        mean = getattr(self.gn_follower[0], "_last_mean", None)
+        # A captured graph would keep reading this tensor's address after the module has let go of it: plain sums there.
+        if mean is None or torch.cuda.is_current_stream_capturing():
+            return None
+        return mean
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.padding_mode != "zeros" or isinstance(self.padding, str):
@@ -250,11 +263,12 @@ class FastConv3d(nn.Conv3d):
             inner = x
         if master:
             return _Conv3dFn.apply(inner, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
+                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
+                                   self._gn_shift())
         if w is self.weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
-                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
-        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups)
+                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups, self._gn_shift())
+        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups, self._gn_shift())
 
 
 class FastConvTranspose3d(nn.ConvTranspose3d):
@@ -312,5 +326,8 @@ class FastGroupNorm(nn.GroupNorm):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dim() == 5 and not x.is_contiguous(memory_format=_CL3D):
             x = x.contiguous(memory_format=_CL3D)
-        return _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
-                              out_halo=self.out_halo)
+        out = _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
+                             out_halo=self.out_halo)
+        # the group means of this call: the convolution in front takes its next call's sums about them
+        self._last_mean = getattr(out, "_sfh_gn_mean", None)
+        return out

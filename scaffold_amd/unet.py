@@ -100,6 +100,7 @@ class DoubleConv(nn.Module):
             # each convolution announces the GroupNorm that reads its output: its launch leaves the statistics
             for conv, norm in ((self.double_conv[0], self.double_conv[1]), (self.double_conv[3], self.double_conv[4])):
                 conv.gn_groups = norm.num_groups
+                conv.gn_follower = (norm,)
 
     def forward(self, x):
         return self.double_conv(x)

@@ -60,7 +60,7 @@ def test_partials_are_the_sums_of_the_output(device, dtype, n, cin, cout, spatia
         plain = sa.conv3d_forward(x, w, b, 1, padding, 1)
         y = sa.conv3d_forward(x, w, b, 1, padding, 1, gn_groups=groups)
         assert torch.equal(plain, y), "the statistics must not change the convolution's result"
-        partials, records, g, version = y._sfh_gn_partials
+        partials, records, g, version, _shift = y._sfh_gn_partials
         assert g == groups and version == y._version and not hasattr(plain, "_sfh_gn_partials")
         assert partials.numel() == n * records * 2 * groups
         got = partials.view(n, records, 2, groups).double().sum(1)  # fp64 sum of the fp32 records
@@ -100,6 +100,45 @@ def test_group_norm_from_partials_matches_the_statistics_pass(device, n, cin, co
     assert orc.gn_rel_error(fused, ref) < 2e-2
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", [CASES[0], CASES[2], CASES[7], CASES[10], CASES[12], CASES[13]])
+def test_sums_about_a_shift(device, dtype, n, cin, cout, spatial, padding, groups, kernel):
+    """With a shift K per (sample, group) the records hold sums of (y - K) and (y - K)^2: exact on integer draws, and the
+    normalisation then survives a mean a thousand times the spread, where plain fp32 sums have lost the variance."""
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=dtype)
+    ops = orc.make_inputs(prob, seed=4, exact=True, density=0.02)
+    x, w = ops["input"].to(device), ops["weight"].to(device)
+    b = (torch.arange(cout) % 5 - 2).to(dtype).to(device)
+    shift = (torch.arange(n * groups, dtype=torch.float32, device=device).reshape(n, groups) % 7) - 3.0  # integers
+    y = sa.conv3d_forward(x, w, b, 1, padding, 1, gn_groups=groups, gn_shift=shift)
+    assert torch.equal(y, sa.conv3d_forward(x, w, b, 1, padding, 1))
+    partials, records, g, version, kept = y._sfh_gn_partials
+    assert kept is shift
+    got = partials.view(n, records, 2, groups).double().sum(1)
+    v = y.double().reshape(n, groups, -1) - shift.double()[:, :, None]
+    assert torch.equal(got[:, 0], v.sum(-1)) and torch.equal(got[:, 1], (v * v).sum(-1))
+    # group_norm takes the shift from the tensor: same result as the statistics pass
+    fused = sa.group_norm(y, groups, None, None, 1e-5, None, out_dtype=None)
+    plain = sa.group_norm(y.clone(memory_format=torch.preserve_format), groups, None, None, 1e-5, None, out_dtype=None)
+    diff = (fused.float() - plain.float()).abs()
+    assert (diff <= 2.0 ** -7 * plain.float().abs() + 1e-6).all()
+
+    if dtype is torch.float16 and kernel != "direct":
+        # mean = 1000 x spread (fp16 resolves it; bf16 does not): a bias of 1000 on outputs of spread ~1
+        big = torch.full((cout,), 1000.0, dtype=dtype, device=device)
+        ops = orc.make_inputs(prob, seed=6)
+        x, w = ops["input"].to(device), (ops["weight"] * (1.0 / (cin * 27) ** 0.5)).to(dtype).to(device)
+        y0 = sa.conv3d_forward(x, w, big, 1, padding, 1)
+        ref = F.group_norm(y0.double(), groups, None, None, 1e-5)
+        near = y0.double().reshape(n, groups, -1).mean(-1).float() + 0.5   # "last call's means": close, not equal
+        y1 = sa.conv3d_forward(x, w, big, 1, padding, 1, gn_groups=groups, gn_shift=near)
+        good = sa.group_norm(y1, groups, None, None, 1e-5, None, out_dtype=torch.float32)
+        assert orc.gn_rel_error(good, ref) < 2e-3
+        y2 = sa.conv3d_forward(x, w, big, 1, padding, 1, gn_groups=groups)  # no shift: plain sums, the variance is noise
+        poor = sa.group_norm(y2, groups, None, None, 1e-5, None, out_dtype=torch.float32)
+        assert orc.gn_rel_error(poor, ref) > 10 * orc.gn_rel_error(good, ref)
+
+
 def test_statistics_follow_the_tensor_not_the_name(device):
     prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(8, 8, 32), padding=(1, 1, 1), dtype=torch.bfloat16)
     ops = orc.make_inputs(prob, seed=5)
@@ -132,6 +171,8 @@ def test_double_conv_with_and_without_the_handoff(device):
     block = DoubleConv(32, 64, 8).to(device).to(memory_format=CL)
     x = torch.randn(1, 32, 8, 16, 32, device=device).contiguous(memory_format=CL)
     assert block.double_conv[0].gn_groups == 8 and block.double_conv[3].gn_groups == 8
+    assert block.double_conv[0].gn_follower == (block.double_conv[1],) and "gn_follower" not in dict(block.named_modules())
+    assert set(block.state_dict()) == {f"double_conv.{i}.weight" for i in (0, 1, 3, 4)} | {f"double_conv.{i}.bias" for i in (1, 4)}
 
     def run():
         for p in block.parameters():
@@ -142,7 +183,10 @@ def test_double_conv_with_and_without_the_handoff(device):
         out.float().square().mean().backward()
         return out.detach(), xi.grad, [p.grad.clone() for p in block.parameters()]
 
-    fused = run()
+    fused = run()       # first call: plain sums
+    assert block.double_conv[1]._last_mean is not None and block.double_conv[1]._last_mean.shape == (1, 8)
+    shifted = run()     # second call: sums about the first call's means
+    assert orc.gn_rel_error(shifted[0], fused[0].double()) < 1e-2
     for conv in (block.double_conv[0], block.double_conv[3]):
         conv.gn_groups = 0
     separate = run()
