@@ -231,13 +231,16 @@ int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype
                            size_t workspace_bytes, void* stream);
 /* The same again with the statistics taken from partial sums the producer of x left
  * (sfh_conv3d_fwd_gn): partials[N][records][2][groups], sums of x - shift and of its square per group, and the
- * shift[N][groups] they were taken about (NULL = zeros; must not be the `mean` output of this call).
+ * shift[N][groups] they were taken about (NULL = zeros; must not be an output of this call). next_shift[N][groups]
+ * (optional output) is what the producer should take its next call's sums about: a group's mean where it exceeds 16
+ * standard deviations -- where plain sums would start to lose the variance -- and zero elsewhere, so that ordinary
+ * tensors give the same bits call after call whatever was normalised before.
  * No statistics pass and no workspace; halo_rows may be 0 (y_slab is then a plain output). Needs the vector path
  * (16-byte aligned tensors, channel counts the 16-byte vectors divide): SFH_ERR_UNSUPPORTED otherwise. */
 int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
                                     const void* x, const void* gamma, const void* beta, void* y_slab,
                                     int64_t halo_rows, float* mean, float* rstd, const float* partials,
-                                    int32_t records, const float* shift, void* stream);
+                                    int32_t records, const float* shift, float* next_shift, void* stream);
 
 /* The forward for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc. It has no counterpart in the reference. Same kernels and results as sfh_groupnorm_fwd, but the

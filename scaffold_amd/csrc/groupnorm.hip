@@ -225,9 +225,15 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
 // One workgroup per (group, sample): fixed-order sum of the split partials, then
 // mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps). A null `shift` stands for K = 0 (partials that
 // the producer of x summed unshifted).
+// The shift a producer of x should take its NEXT call's sums about, given this call's statistics: the mean where it
+// is large against the spread (there plain sums would cancel), else zero -- so that ordinary tensors give the same bits
+// call after call, whatever the history.
+constexpr float kShiftFromRatio = 16.f;
+__device__ __forceinline__ float next_shift_of(float mu, float rs) { return fabsf(mu) * rs > kShiftFromRatio ? mu : 0.f; }
+
 __global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
                                                             float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
-                                                            float m, float eps) {
+                                                            float m, float eps, float* __restrict__ next_shift) {
   __shared__ float wsum[kBlock / 64][2];
   const int g = blockIdx.x, n = blockIdx.y, tid = threadIdx.x;
   const float* base = part + (int64_t)n * nsplit * 2 * G + g;
@@ -261,8 +267,10 @@ __global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restr
     const float d = s1 / m;
     float var = s2 / m - d * d;
     var = var < 0.f ? 0.f : var;
-    mean[n * G + g] = (shift != nullptr ? shift[n * G + g] : 0.f) + d;
-    rstd[n * G + g] = 1.f / sqrtf(var + eps);
+    const float mu = (shift != nullptr ? shift[n * G + g] : 0.f) + d, rs = 1.f / sqrtf(var + eps);
+    mean[n * G + g] = mu;
+    rstd[n * G + g] = rs;
+    if (next_shift != nullptr) next_shift[n * G + g] = next_shift_of(mu, rs);
   }
 }
 
@@ -320,7 +328,7 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
                                                        float* __restrict__ rstd, const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
                                                        int tpr, int rpp, int nsplit, int64_t rows_per_split, float m, float eps,
-                                                       int relu, int64_t y_halo, int npart) {
+                                                       int relu, int64_t y_halo, int npart, float* __restrict__ next_shift) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float gstat[];  // sums[2 G] | mean[G] | rstd[G] | fold scratch (4 * kBlock)
   const int tid = threadIdx.x;
@@ -344,6 +352,7 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
       if (blockIdx.x == 0) {  // for the backward pass
         mean[n * G + tid] = mu_g;
         rstd[n * G + tid] = rs_g;
+        if (next_shift != nullptr) next_shift[n * G + tid] = next_shift_of(mu_g, rs_g);
       }
     }
   } else {
@@ -859,7 +868,7 @@ size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
 template <typename T, typename TO>
 int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
               void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st, const float* given_part = nullptr,
-              int given_npart = 0, const float* given_shift = nullptr) {
+              int given_npart = 0, const float* given_shift = nullptr, float* next_shift = nullptr) {
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
   if (y_halo > 0 && (!pl.vector || sizeof(T) != sizeof(TO) || (y_halo * C * sizeof(TO)) % 16 != 0))
@@ -897,12 +906,12 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
   }
   const float m = (float)S * (float)(C / G);
   if (!fold_in_consumer_host(G, npart)) {
-    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(kBlock), 0, st, shift, part, mean, rstd, G, npart, m, p.eps);
+    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(kBlock), 0, st, shift, part, mean, rstd, G, npart, m, p.eps, next_shift);
     if (int rc = check_launch("gn_stats_finalize")) return rc;
   }
   hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
                      mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu, y_halo,
-                     npart);
+                     npart, next_shift);
   return check_launch("gn_normalize");
 }
 
@@ -962,7 +971,7 @@ extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p,
 static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x, const void* gamma,
                              const void* beta, void* y, int64_t y_halo, float* mean, float* rstd, void* workspace,
                              size_t workspace_bytes, void* stream, const float* given_part = nullptr, int given_npart = 0,
-                             const float* given_shift = nullptr) {
+                             const float* given_shift = nullptr, float* next_shift = nullptr) {
   if (int rc = check_desc(p, x_dtype)) return rc;
   if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
   if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
@@ -976,7 +985,8 @@ static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dty
   hipStream_t st = (hipStream_t)stream;
   float* ws = (float*)workspace;
 #define SFH_GN_FWD(TX, TY) \
-  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart, given_shift)
+  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart, given_shift, \
+                           next_shift)
   if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
@@ -1005,11 +1015,11 @@ extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, 
 extern "C" int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
                                                const void* gamma, const void* beta, void* y_slab, int64_t halo_rows, float* mean,
                                                float* rstd, const float* partials, int32_t records, const float* shift,
-                                               void* stream) {
+                                               float* next_shift, void* stream) {
   if (partials == nullptr || records < 1) return fail(SFH_ERR_INVALID, "groupnorm from partials: no partial sums given");
   if (!aligned16(partials)) return fail(SFH_ERR_INVALID, "groupnorm from partials: the partial sums must be 16-byte aligned");
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, nullptr, 0, stream, partials,
-                           records, shift);
+                           records, shift, next_shift);
 }
 
 // ---- the forward for callers that may not allocate ------------------------------------------------------------------

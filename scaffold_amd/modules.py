@@ -213,18 +213,18 @@ class FastConv3d(nn.Conv3d):
     #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
-    #: that GroupNorm module, in a tuple (so that it is not registered as a child): the group means of its last call are
-    #: what this call's sums are taken about
+    #: that GroupNorm module, in a tuple (so that it is not registered as a child): its last call says what this call's
+    #: sums are taken about (zeros, unless a group's mean was far above its spread)
     gn_follower = ()
 
     def _gn_shift(self):
         if not self.gn_follower or self.gn_groups <= 0:
             return None
-        mean = getattr(self.gn_follower[0], "_last_mean", None)
+        shift = getattr(self.gn_follower[0], "_next_shift", None)
         # A captured graph would keep reading this tensor's address after the module has let go of it: plain sums there.
-        if mean is None or torch.cuda.is_current_stream_capturing():
+        if shift is None or torch.cuda.is_current_stream_capturing():
             return None
-        return mean
+        return shift
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.padding_mode != "zeros" or isinstance(self.padding, str):
@@ -328,6 +328,6 @@ class FastGroupNorm(nn.GroupNorm):
             x = x.contiguous(memory_format=_CL3D)
         out = _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
                              out_halo=self.out_halo)
-        # the group means of this call: the convolution in front takes its next call's sums about them
-        self._last_mean = getattr(out, "_sfh_gn_mean", None)
+        # what the convolution in front should take its next call's sums about
+        self._next_shift = getattr(out, "_sfh_gn_shift", None)
         return out

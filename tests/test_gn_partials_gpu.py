@@ -137,6 +137,11 @@ def test_sums_about_a_shift(device, dtype, n, cin, cout, spatial, padding, group
         y2 = sa.conv3d_forward(x, w, big, 1, padding, 1, gn_groups=groups)  # no shift: plain sums, the variance is noise
         poor = sa.group_norm(y2, groups, None, None, 1e-5, None, out_dtype=torch.float32)
         assert orc.gn_rel_error(poor, ref) > 10 * orc.gn_rel_error(good, ref)
+        # ... but that call reports the means as the shift for the next one (they exceed 16 spreads), and the next is right
+        nxt = poor._sfh_gn_shift
+        assert nxt is not None and (nxt - 1000.0).abs().max() < 5.0
+        y3 = sa.conv3d_forward(x, w, big, 1, padding, 1, gn_groups=groups, gn_shift=nxt)
+        assert orc.gn_rel_error(sa.group_norm(y3, groups, None, None, 1e-5, None, out_dtype=torch.float32), ref) < 2e-3
 
 
 def test_statistics_follow_the_tensor_not_the_name(device):
@@ -184,9 +189,10 @@ def test_double_conv_with_and_without_the_handoff(device):
         return out.detach(), xi.grad, [p.grad.clone() for p in block.parameters()]
 
     fused = run()       # first call: plain sums
-    assert block.double_conv[1]._last_mean is not None and block.double_conv[1]._last_mean.shape == (1, 8)
-    shifted = run()     # second call: sums about the first call's means
-    assert orc.gn_rel_error(shifted[0], fused[0].double()) < 1e-2
+    nxt = block.double_conv[1]._next_shift
+    assert nxt is not None and nxt.shape == (1, 8) and not nxt.any(), "ordinary activations: no shift, so call after call gives the same bits"
+    again = run()
+    assert torch.equal(again[0], fused[0]) and torch.equal(again[1], fused[1])
     for conv in (block.double_conv[0], block.double_conv[3]):
         conv.gn_groups = 0
     separate = run()
