@@ -284,7 +284,28 @@ def bench_groupnorm(args, device):
 
     fwd_ms = event_time_ms(abi_fwd, 20)
     bwd_ms = event_time_ms(abi_bwd, 20)
+
+    # The same normalisation fed by the convolution in front of it (what every GroupNorm of the U-Net step runs): a
+    # 64 -> 64 convolution of this shape leaves the per-group sums of its output, the forward is then one read and one
+    # write of the tensor (2 B) instead of two reads and a write (3 B).
+    import scaffold_amd as sa
+    xin = torch.randn(shape, generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    wconv = (torch.randn((64, 64, 3, 3, 3), generator=g) / math.sqrt(64 * 27)).to(torch.bfloat16).to(device)
+    yconv = sa.conv3d_forward(xin, wconv, None, 1, 1, 1, gn_groups=8)
+    handoff = getattr(yconv, "_sfh_gn_partials", None)
+    from_producer = {}
+    if handoff is not None:
+        partials, records = handoff[0], handoff[1]
+
+        def abi_fwd_from_partials():
+            _lib.check(L.sfh_groupnorm_fwd_from_partials(dref, BF16, BF16, FP32, P(yconv), P(gamma), P(beta), P(y), 0, P(mean), P(rstd),
+                                                         P(partials), records, None, None, stream), "sfh_groupnorm_fwd_from_partials")
+
+        ms = event_time_ms(abi_fwd_from_partials, 20)
+        from_producer = {"fwd_with_producer_statistics_ms": ms, "fwd_with_producer_statistics_bytes": 2 * B,
+                         "fwd_with_producer_statistics_gbs": 2 * B / (ms * 1e-3) / 1e9, "producer_records_per_sample": records}
     return {
+        **from_producer,
         "tensor_bytes": B,
         "fwd_ms": fwd_ms, "fwd_gbs": 3 * B / (fwd_ms * 1e-3) / 1e9, "fwd_frac_of_hbm_peak": 3 * B / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bwd_ms": bwd_ms, "bwd_gbs": 5 * B / (bwd_ms * 1e-3) / 1e9, "bwd_frac_of_hbm_peak": 5 * B / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
