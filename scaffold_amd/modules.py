@@ -213,16 +213,14 @@ class FastConv3d(nn.Conv3d):
     #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
-    #: that GroupNorm module, in a tuple (so that it is not registered as a child): its last call says what this call's
-    #: sums are taken about (zeros, unless a group's mean was far above its spread)
-    gn_follower = ()
+    #: what this call's sums are taken about: the ``_next_shift`` the GroupNorm behind this module reported at its last
+    #: call (zeros unless a group's mean was far above its spread), set by whoever owns the pair before each call
+    gn_shift = None
 
     def _gn_shift(self):
-        if not self.gn_follower or self.gn_groups <= 0:
-            return None
-        shift = getattr(self.gn_follower[0], "_next_shift", None)
-        # A captured graph would keep reading this tensor's address after the module has let go of it: plain sums there.
-        if shift is None or torch.cuda.is_current_stream_capturing():
+        shift = self.gn_shift
+        # A captured graph would keep reading this tensor's address after its owner has let go of it: plain sums there.
+        if shift is None or self.gn_groups <= 0 or torch.cuda.is_current_stream_capturing():
             return None
         return shift
 

@@ -96,14 +96,19 @@ class DoubleConv(nn.Module):
             nn.Identity(),
         )
 
-        if not stock:
-            # each convolution announces the GroupNorm that reads its output: its launch leaves the statistics
-            for conv, norm in ((self.double_conv[0], self.double_conv[1]), (self.double_conv[3], self.double_conv[4])):
-                conv.gn_groups = norm.num_groups
-                conv.gn_follower = (norm,)
+        self._pairs = () if stock else ((0, 1), (3, 4))
+        # each convolution announces the GroupNorm that reads its output: its launch leaves the statistics
+        for c, g in self._pairs:
+            self.double_conv[c].gn_groups = self.double_conv[g].num_groups
 
     def forward(self, x):
-        return self.double_conv(x)
+        if not self._pairs:
+            return self.double_conv(x)
+        for c, g in self._pairs:  # the Identity modules between the pairs only keep the reference's state-dict indices
+            conv, norm = self.double_conv[c], self.double_conv[g]
+            conv.gn_shift = getattr(norm, "_next_shift", None)  # what the norm's last call said to sum about
+            x = norm(conv(x))
+        return x
 
 
 class Down(nn.Module):

@@ -176,7 +176,6 @@ def test_double_conv_with_and_without_the_handoff(device):
     block = DoubleConv(32, 64, 8).to(device).to(memory_format=CL)
     x = torch.randn(1, 32, 8, 16, 32, device=device).contiguous(memory_format=CL)
     assert block.double_conv[0].gn_groups == 8 and block.double_conv[3].gn_groups == 8
-    assert block.double_conv[0].gn_follower == (block.double_conv[1],) and "gn_follower" not in dict(block.named_modules())
     assert set(block.state_dict()) == {f"double_conv.{i}.weight" for i in (0, 1, 3, 4)} | {f"double_conv.{i}.bias" for i in (1, 4)}
 
     def run():
