@@ -73,6 +73,8 @@ typedef struct sfh_groupnorm_desc {
 } sfh_groupnorm_desc;
 
 /* ---- library ------------------------------------------------------------------------ */
+/* 100: the first published set of entry points. 101: sfh_conv3d_launch_geometry, sfh_conv3d_fwd_gn_records,
+ * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
