@@ -123,6 +123,32 @@ def test_brick_geometries_exact(device, n, cin, cout, spatial, direction, voxels
     check_exact(prob, direction, device)
 
 
+def _random_tiled_problems(count, seed):
+    """Seeded random 3x3x3 stride-1 problems with channel counts in multiples of 32: extents around the tile sizes, the
+    three padding forms, one to three samples -- whatever geometry the launch rules pick for them."""
+    import random
+    rng = random.Random(seed)
+    out = []
+    while len(out) < count:
+        cin, cout = rng.choice([32, 64, 96, 128, 256]), rng.choice([32, 64, 96, 128, 256])
+        w = rng.choice([rng.randint(3, 8), rng.randint(9, 16), rng.randint(17, 48)])
+        d, h = rng.randint(2, 14), rng.randint(3, 24)
+        n = rng.choice([1, 1, 2, 3])
+        pad = rng.choice([(1, 1, 1), (0, 1, 1), (2, 2, 2), (1, 0, 2)])
+        if min(d + 2 * pad[0], h + 2 * pad[1], w + 2 * pad[2]) < 3 or n * max(cin, cout) * d * h * w > 3_000_000:
+            continue
+        out.append((n, cin, cout, (d, h, w), pad))
+    return out
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("n,cin,cout,spatial,padding", _random_tiled_problems(24, seed=77))
+def test_random_tiled_problems_exact(device, n, cin, cout, spatial, padding, direction):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=torch.bfloat16)
+    assert c3.uses_mfma(prob.input_shape, prob.weight_shape, 1, padding, 1, torch.bfloat16, direction)
+    check_exact(prob, direction, device)
+
+
 # Shapes only the direct kernels serve: odd channel counts, strides, dilation, other kernel sizes,
 # fp32 (``triton_conv3d/shapes.py:611-684`` edge list).
 DIRECT_SHAPES = [
