@@ -74,7 +74,8 @@ typedef struct sfh_groupnorm_desc {
 
 /* ---- library ------------------------------------------------------------------------ */
 /* 100: the first published set of entry points. 101: sfh_conv3d_launch_geometry, sfh_conv3d_fwd_gn_records,
- * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed. */
+ * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed.
+ * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair added. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -191,6 +192,38 @@ int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype);
 size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
 int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw,
                      void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* ---- conv3d over a skip connection that is never concatenated -----------------------------
+ * The decoder's first convolution reads torch.cat([skip, upsampled], dim=1) (unet_parts.py:107-120 writes that tensor,
+ * unet_parts.py:123-160 convolves it). Here the convolution takes the two tensors themselves: x_first holds the first
+ * cin_first input channels of every voxel, x_second the other p->cin - cin_first, both dense channels-last over the
+ * same (N, in_d, in_h, in_w) voxels; `p`, the weight and every other argument are those of the convolution over the
+ * concatenation. The forward stages each 32-channel chunk of its reduction from the tensor that holds it; the data
+ * gradient stores each 32-channel block of its result into gx_first or gx_second (what the concatenation's backward
+ * would have split); the weight gradient reads each 32-channel input block from its tensor. Every result is, bit for
+ * bit, that of the ordinary entry point on the concatenated tensor -- the same kernels, launch geometry and summation
+ * order -- while the concatenated activation and its gradient are neither written nor read (4 bytes x voxels x Cin of
+ * HBM traffic per direction pair, and the memory of both tensors).
+ * sfh_conv3d_pair_supported: 1 when `direction` (0 forward, 1 data gradient, 2 weight gradient) of the problem takes
+ * the cut, a pure function of problem, dtype and cut: 16-bit MFMA problems with cin_first a multiple of 32; the forward
+ * of a 64-channel output over 128 or more input channels at rows of more than 16 voxels (SFH_KERNEL_WIDE) only when
+ * the two tensors have the same channel count (a data gradient whose reduction is sliced, geometry[3] > 1, writes the
+ * two tensors from the sum of its slices). A caller asks for all three before it drops its concatenation, and
+ * concatenates otherwise.
+ * sfh_conv3d_fwd_pair with groups > 0 also leaves the GroupNorm partials of sfh_conv3d_fwd_gn (same records, same
+ * arguments); groups = 0 and NULL for the three gn arguments is the plain forward. Workspaces are those of the
+ * ordinary entry points. SFH_FLAG_FORCE_GENERIC is refused. */
+int sfh_conv3d_pair_supported(const sfh_conv3d_desc* p, int dtype, int32_t cin_first, int direction);
+int sfh_conv3d_fwd_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second,
+                        int32_t cin_first, const void* w, const int64_t w_stride[5], const void* bias, void* y,
+                        void* workspace, size_t workspace_bytes, uint32_t flags, int groups,
+                        const float* gn_shift, float* gn_partials, size_t gn_partials_bytes, void* stream);
+int sfh_conv3d_dgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w,
+                          const int64_t w_stride[5], void* gx_first, void* gx_second, int32_t cin_first,
+                          void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second,
+                          int32_t cin_first, const void* gy, void* gw, void* workspace, size_t workspace_bytes,
+                          uint32_t flags, void* stream);
 
 /* ---- bias gradient --------------------------------------------------------------------
  * Stands in for `grad_output.sum((0, 2, 3, 4))` in the reference's autograd functions

@@ -54,6 +54,10 @@ __all__ = [
     "split_count",
     "uses_mfma",
     "output_shape",
+    "is_supported_pair",
+    "conv3d_forward_pair",
+    "conv3d_backward_data_pair",
+    "conv3d_backward_weight_pair",
 ]
 
 _CL3D = torch.channels_last_3d
@@ -570,6 +574,7 @@ def conv3d_forward(
     gn_groups: int = 0,
     gn_shift: Optional[torch.Tensor] = None,
     _checked: bool = False,
+    _second: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Forward 3-D convolution; input and output are ``channels_last_3d``.
 
@@ -592,7 +597,11 @@ def conv3d_forward(
         )
     _no_config(config)
     x = x.contiguous(memory_format=_CL3D)
-    prob = _problem(x.shape, w.shape, stride, padding, dilation, x.dtype)
+    if _second is None:
+        prob = _problem(x.shape, w.shape, stride, padding, dilation, x.dtype)
+    else:  # conv3d_forward_pair: x holds the first channels of the input, _second the rest
+        _second = _second.contiguous(memory_format=_CL3D)
+        prob = _problem(_pair_shape(x, _second), w.shape, stride, padding, dilation, x.dtype)
     if out is None:
         y = torch.empty(prob.y_shape, device=x.device, dtype=x.dtype, memory_format=_CL3D)
     else:
@@ -626,16 +635,27 @@ def conv3d_forward(
                                          or gn_shift.device != x.device or not gn_shift.is_contiguous()):
                 gn_shift = None  # not the shape of this call (another batch size, say): plain sums
             partials = torch.empty(prob.n * records * 2 * gn_groups, dtype=torch.float32, device=x.device)
-            rc = L.sfh_conv3d_fwd_gn(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
-                                     None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
-                                     _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
-                                     _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+            if _second is None:
+                rc = L.sfh_conv3d_fwd_gn(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
+                                         None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                                         _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
+                                         _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+            else:
+                rc = L.sfh_conv3d_fwd_pair(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(_second), int(x.shape[1]), _lib.ptr(w_eff),
+                                           None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                                           _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
+                                           _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
             if rc == _lib.SFH_ERR_UNSUPPORTED:  # e.g. an out= view off the 16-byte grid: the plain launch
                 records = 0
             else:
                 # valid for these bits of y only: the version lets the consumer see an in-place change
                 y._sfh_gn_partials = (partials, records, int(gn_groups), y._version, gn_shift)
-        if records == 0:
+        if records == 0 and _second is not None:
+            rc = L.sfh_conv3d_fwd_pair(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(_second), int(x.shape[1]), _lib.ptr(w_eff),
+                                       None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
+                                       _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, 0, None, None, 0,
+                                       _lib.stream_ptr(x.device))
+        elif records == 0:
             rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
                                   None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                   _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(x.device))
@@ -661,7 +681,8 @@ def conv3d_backward_data(
     force_generic: bool = False,
     packed_weight: Optional[torch.Tensor] = None,
     _checked: bool = False,
-) -> torch.Tensor:
+    _cin_first: int = 0,
+):
     """Gradient of a conv3d with respect to its input (stride 1 only).
 
     Computed as a gather over ``grad_output`` with the channel roles of the weight swapped, the
@@ -679,7 +700,11 @@ def conv3d_backward_data(
     prob = _problem(input_shape if isinstance(input_shape, torch.Size) else tuple(input_shape), weight.shape, stride, padding,
                     dilation, gy.dtype)
     gx_shape = (prob.n, prob.cin, *prob.in_sp)
-    if out is None:
+    gx_second = None
+    if _cin_first:  # conv3d_backward_data_pair: the gradient as two tensors, cut at that channel
+        gx = torch.empty((prob.n, _cin_first, *prob.in_sp), device=gy.device, dtype=gy.dtype, memory_format=_CL3D)
+        gx_second = torch.empty((prob.n, prob.cin - _cin_first, *prob.in_sp), device=gy.device, dtype=gy.dtype, memory_format=_CL3D)
+    elif out is None:
         gx = torch.empty(gx_shape, device=gy.device, dtype=gy.dtype, memory_format=_CL3D)
     else:
         gx = out
@@ -701,11 +726,17 @@ def conv3d_backward_data(
             flags |= _lib.SFH_FLAG_WEIGHT_PACKED
             w_eff = packed_weight
         ws = _lib.workspace(need, gy.device)
-        rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff),
-                                None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(gx),
-                                _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(gy.device))
+        if gx_second is None:
+            rc = L.sfh_conv3d_dgrad(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff),
+                                    None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(gx),
+                                    _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, _lib.stream_ptr(gy.device))
+        else:
+            rc = L.sfh_conv3d_dgrad_pair(ctypes.byref(desc), code, _lib.ptr(gy), _lib.ptr(w_eff),
+                                         None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(gx), _lib.ptr(gx_second),
+                                         int(_cin_first), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags,
+                                         _lib.stream_ptr(gy.device))
     _lib.check(rc, "conv3d_backward_data")
-    return gx
+    return gx if gx_second is None else (gx, gx_second)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -744,6 +775,7 @@ def conv3d_backward_weight(
     force_generic: bool = False,
     grad_dtype: Optional[torch.dtype] = None,
     _checked: bool = False,
+    _second: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Gradient of a conv3d with respect to its weight, returned ``channels_last_3d``.
 
@@ -764,8 +796,10 @@ def conv3d_backward_weight(
         raise NotImplementedError("deterministic=False: this library has no atomic weight-gradient path")
     x = input.contiguous(memory_format=_CL3D)
     gy = grad_output.contiguous(memory_format=_CL3D)
-    prob = _problem(x.shape, weight_shape if isinstance(weight_shape, torch.Size) else tuple(weight_shape), stride, padding,
-                    dilation, x.dtype)
+    if _second is not None:  # conv3d_backward_weight_pair: x holds the first channels of the input, _second the rest
+        _second = _second.contiguous(memory_format=_CL3D)
+    prob = _problem(x.shape if _second is None else _pair_shape(x, _second),
+                    weight_shape if isinstance(weight_shape, torch.Size) else tuple(weight_shape), stride, padding, dilation, x.dtype)
     cout, cin, k, n = prob.cout, prob.cin, prob.k, prob.n
     gdt = x.dtype if grad_dtype is None else grad_dtype
     if gdt is not x.dtype and gdt is not torch.float32:
@@ -798,7 +832,107 @@ def conv3d_backward_weight(
                 )
             ws, ws_bytes = workspace, have
         flags = _flags(force_generic) | (_lib.SFH_FLAG_GRAD_FP32 if gdt is not x.dtype else 0)
-        rc = L.sfh_conv3d_wgrad(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(ws), ws_bytes,
-                                flags, _lib.stream_ptr(x.device))
+        if _second is None:
+            rc = L.sfh_conv3d_wgrad(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(ws), ws_bytes,
+                                    flags, _lib.stream_ptr(x.device))
+        else:
+            rc = L.sfh_conv3d_wgrad_pair(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(_second), int(x.shape[1]), _lib.ptr(gy),
+                                         _lib.ptr(gw), _lib.ptr(ws), ws_bytes, flags, _lib.stream_ptr(x.device))
     _lib.check(rc, "conv3d_backward_weight")
     return gw
+
+
+# ---------------------------------------------------------------------------------------------
+# a convolution over two tensors whose channels follow each other
+# ---------------------------------------------------------------------------------------------
+def _pair_shape(first: torch.Tensor, second: torch.Tensor) -> torch.Size:
+    return torch.Size((first.shape[0], first.shape[1] + second.shape[1], *first.shape[2:]))
+
+
+_PAIR_GATE: dict = {}
+
+
+def is_supported_pair(x_first, x_second, w, bias=None, stride=1, padding=0, dilation=1) -> bool:
+    """Whether all three directions of ``conv3d(torch.cat([x_first, x_second], 1), w)`` are served from the two tensors
+    themselves (:func:`conv3d_forward_pair` and its two gradients).  Total: never raises."""
+    try:
+        if not isinstance(x_first, torch.Tensor) or not isinstance(x_second, torch.Tensor) or x_first.dim() != 5 or x_second.dim() != 5:
+            return False
+        if x_first.dtype is not x_second.dtype or x_first.device != x_second.device:
+            return False
+        if x_first.shape[0] != x_second.shape[0] or x_first.shape[2:] != x_second.shape[2:] or x_first.shape[0] < 1:
+            return False
+        shape = _pair_shape(x_first, x_second)
+        stand_in = x_first.new_empty((1, 1, 1, 1, 1)).expand(shape)  # metadata only
+        if not is_supported_all(stand_in, w, bias, stride, padding, dilation, 1):
+            return False
+        key = (shape, int(x_first.shape[1]), w.shape, stride, padding, dilation, x_first.dtype)
+        hit = _PAIR_GATE.get(key)
+        if hit is None:
+            prob = _problem(shape, w.shape, stride, padding, dilation, x_first.dtype)
+            L = _lib.lib()
+            hit = all(L.sfh_conv3d_pair_supported(ctypes.byref(prob.desc), prob.code, int(x_first.shape[1]), d) == 1 for d in (0, 1, 2))
+            if len(_PAIR_GATE) > 4096:
+                _PAIR_GATE.clear()
+            _PAIR_GATE[key] = hit
+        return hit
+    except (TypeError, ValueError, AttributeError, RuntimeError, NotImplementedError):
+        return False
+
+
+def _refuse_pair(x_first, x_second, w):
+    raise NotImplementedError(
+        f"unsupported pair: x_first={tuple(getattr(x_first, 'shape', ()))}/{getattr(x_first, 'dtype', None)} "
+        f"x_second={tuple(getattr(x_second, 'shape', ()))} w={tuple(getattr(w, 'shape', ()))}: concatenate and use conv3d_forward")
+
+
+def conv3d_forward_pair(x_first, x_second, w, bias=None, stride=1, padding=0, dilation=1, *, packed_weight=None, gn_groups: int = 0,
+                        gn_shift=None, _checked: bool = False) -> torch.Tensor:
+    """``conv3d_forward(torch.cat([x_first, x_second], 1), w, ...)`` without the concatenation
+    (``ScaFFold/unet/unet_parts.py:107-120`` writes that tensor for the decoder's first convolution): the kernel stages each
+    32-channel chunk of its reduction from the tensor that holds it.  Same bits as the call on the concatenated tensor;
+    ``packed_weight`` / ``gn_groups`` / ``gn_shift`` as there.  ``NotImplementedError`` where :func:`is_supported_pair` says no."""
+    if not _checked and not is_supported_pair(x_first, x_second, w, bias, stride, padding, dilation):
+        _refuse_pair(x_first, x_second, w)
+    return conv3d_forward(x_first, w, bias, stride, padding, dilation, 1, packed_weight=packed_weight, gn_groups=gn_groups,
+                          gn_shift=gn_shift, _checked=True, _second=x_second)
+
+
+def conv3d_backward_data_pair(grad_output, weight, input_shape, cin_first: int, stride=1, padding=0, dilation=1, *,
+                              packed_weight=None, _checked: bool = False):
+    """The data gradient of that convolution as the two tensors the concatenation's backward would have split it into:
+    ``(grad_first, grad_second)`` with ``cin_first`` and ``Cin - cin_first`` channels; ``input_shape`` is the
+    concatenation's.  Same bits as ``conv3d_backward_data(...)`` split along the channels."""
+    cin_first = int(cin_first)
+    if not _checked:
+        shape = tuple(int(v) for v in input_shape)
+        ok = isinstance(grad_output, torch.Tensor) and len(shape) == 5 and 0 < cin_first < shape[1] and \
+            is_supported_bwd_data(grad_output, weight, shape, stride, padding, dilation, 1)
+        if ok:
+            prob = _problem(torch.Size(shape), weight.shape, stride, padding, dilation, grad_output.dtype)
+            ok = _lib.lib().sfh_conv3d_pair_supported(ctypes.byref(prob.desc), prob.code, cin_first, 1) == 1
+        if not ok:
+            raise NotImplementedError(f"unsupported pair: grad_output={tuple(getattr(grad_output, 'shape', ()))} "
+                                      f"input_shape={tuple(input_shape)} cut at channel {cin_first}")
+    return conv3d_backward_data(grad_output, weight, input_shape, stride, padding, dilation, 1, packed_weight=packed_weight,
+                                _checked=True, _cin_first=cin_first)
+
+
+def conv3d_backward_weight_pair(x_first, x_second, weight_shape, grad_output, stride=1, padding=0, dilation=1, *,
+                                grad_dtype=None, _checked: bool = False) -> torch.Tensor:
+    """``conv3d_backward_weight(torch.cat([x_first, x_second], 1), ...)`` without the concatenation; same bits."""
+    if not _checked:
+        ok = isinstance(x_first, torch.Tensor) and isinstance(x_second, torch.Tensor) and x_first.dim() == 5 and x_second.dim() == 5 \
+            and x_first.dtype is x_second.dtype and x_first.device == x_second.device and x_first.shape[0] == x_second.shape[0] \
+            and x_first.shape[2:] == x_second.shape[2:]
+        if ok:
+            shape = _pair_shape(x_first, x_second)
+            stand_in = x_first.new_empty((1, 1, 1, 1, 1)).expand(shape)
+            ok = is_supported_bwd_weight(stand_in, tuple(weight_shape), grad_output, stride, padding, dilation, 1)
+        if ok:
+            prob = _problem(shape, torch.Size(tuple(weight_shape)), stride, padding, dilation, x_first.dtype)
+            ok = _lib.lib().sfh_conv3d_pair_supported(ctypes.byref(prob.desc), prob.code, int(x_first.shape[1]), 2) == 1
+        if not ok:
+            _refuse_pair(x_first, x_second, None)
+    return conv3d_backward_weight(x_first, weight_shape, grad_output, stride, padding, dilation, 1, grad_dtype=grad_dtype,
+                                  _checked=True, _second=x_second)

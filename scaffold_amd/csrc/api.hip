@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restric
 
 using namespace sfh;
 
-extern "C" int sfh_version(void) { return 101; }
+extern "C" int sfh_version(void) { return 102; }
 
 extern "C" const char* sfh_last_error(void) { return g_error; }
 
@@ -344,7 +344,7 @@ extern "C" size_t sfh_conv3d_fwd_workspace_bytes(const sfh_conv3d_desc* p, int d
 
 static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
                           const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream,
-                          const GnPartialOut* gn) {
+                          const GnPartialOut* gn, const ChannelPair* in2 = nullptr) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (x == nullptr || w == nullptr || y == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
@@ -357,7 +357,7 @@ static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, co
     if (flags & SFH_FLAG_WEIGHT_PACKED) {  // w is the packed weight; the workspace only holds the partial slices
       if (partial_bytes && (workspace == nullptr || workspace_bytes < partial_bytes))
         return fail(SFH_ERR_WORKSPACE, "conv3d fwd: workspace of %zu bytes needed, got %zu", partial_bytes, workspace_bytes);
-      return mfma_conv_persist(a, dtype, x, w, bias, y, partial_bytes ? workspace : nullptr, st, gn);
+      return mfma_conv_persist(a, dtype, x, w, bias, y, partial_bytes ? workspace : nullptr, st, gn, in2);
     }
     const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
@@ -365,8 +365,9 @@ static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, co
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[0], w_stride[1], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
-    return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st, gn);
+    return mfma_conv_persist(a, dtype, x, workspace, bias, y, partial, st, gn, in2);
   }
+  if (in2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: this problem does not take its input as two tensors");
   if (gn != nullptr) {  // the one-channel stem is the only other kernel that leaves them
     ThinArgs t;
     if ((flags & SFH_FLAG_WEIGHT_PACKED) || thin_fwd_plan(*p, dtype, out, t) != kThinWideOut || thin_wide_out_gn_records(t, dtype, gn->groups) == 0)
@@ -522,8 +523,8 @@ extern "C" size_t sfh_conv3d_dgrad_workspace_bytes(const sfh_conv3d_desc* p, int
   return mfma_conv_packed_weight_bytes(dgrad_mfma_args(*p, out)) + mfma_conv_partial_bytes(dgrad_mfma_args(*p, out));
 }
 
-extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
-                                void* gx, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+static int conv3d_dgrad_any(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
+                            void* gx, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream, const ChannelPair* out2) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (int rc = check_dgrad(*p)) return rc;
@@ -536,7 +537,7 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
     if (flags & SFH_FLAG_WEIGHT_PACKED) {
       if (partial_bytes && (workspace == nullptr || workspace_bytes < partial_bytes))
         return fail(SFH_ERR_WORKSPACE, "conv3d dgrad: workspace of %zu bytes needed, got %zu", partial_bytes, workspace_bytes);
-      return mfma_conv_persist(a, dtype, gy, w, nullptr, gx, partial_bytes ? workspace : nullptr, st);
+      return mfma_conv_persist(a, dtype, gy, w, nullptr, gx, partial_bytes ? workspace : nullptr, st, nullptr, nullptr, out2);
     }
     const size_t need = packed_bytes + partial_bytes;
     if (workspace == nullptr || workspace_bytes < need)
@@ -545,8 +546,9 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
     if (int rc = mfma_pack_weight(a, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 1, workspace, st))
       return rc;
     void* partial = partial_bytes ? (char*)workspace + packed_bytes : nullptr;
-    return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st);
+    return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st, nullptr, nullptr, out2);
   }
+  if (out2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad: this problem does not write its result as two tensors");
   if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && dgrad_uses_f32_tiles(*p, dtype, out)) {
     const MfmaConvArgs a = dgrad_mfma_args(*p, out);
     const size_t need = f32_conv_packed_weight_bytes(a);
@@ -580,6 +582,11 @@ extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void*
   return direct_conv_gather(a, dtype, gy, w, nullptr, gx, st);
 }
 
+extern "C" int sfh_conv3d_dgrad(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
+                                void* gx, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  return conv3d_dgrad_any(p, dtype, gy, w, w_stride, gx, workspace, workspace_bytes, flags, stream, nullptr);
+}
+
 // ---- weight gradient -------------------------------------------------------------------
 extern "C" int sfh_conv3d_wgrad_splits(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
@@ -605,8 +612,8 @@ extern "C" size_t sfh_conv3d_wgrad_workspace_bytes(const sfh_conv3d_desc* p, int
   return 0;
 }
 
-extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* workspace,
-                                size_t workspace_bytes, uint32_t flags, void* stream) {
+static int conv3d_wgrad_any(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* workspace,
+                            size_t workspace_bytes, uint32_t flags, void* stream, const ChannelPair* x2) {
   int32_t out[3];
   if (int rc = check_conv(p, dtype, out)) return rc;
   if (x == nullptr || gy == nullptr || gw == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad: null tensor");
@@ -617,8 +624,9 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
     const size_t need = mfma_wgrad_workspace_bytes(a);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
-    return mfma_wgrad(a, dtype, x, gy, gw, gw_dtype, workspace, st);
+    return mfma_wgrad(a, dtype, x, gy, gw, gw_dtype, workspace, st, x2);
   }
+  if (x2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad: this problem does not take its input as two tensors");
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && wgrad_uses_f32_tiles(*p, dtype, out)) {
     const WgradArgs a = wgrad_args(*p, out);
     const size_t need = f32_wgrad_workspace_bytes(a);
@@ -652,6 +660,63 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
   a.kd = p->kd; a.kh = p->kh; a.kw = p->kw; a.sd = p->sd; a.sh = p->sh; a.sw = p->sw;
   a.pd = p->pd; a.ph = p->ph; a.pw = p->pw; a.dd = p->dd; a.dh = p->dh; a.dw = p->dw;
   return direct_conv_wgrad(a, dtype, x, gy, gw, st);
+}
+
+extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* workspace,
+                                size_t workspace_bytes, uint32_t flags, void* stream) {
+  return conv3d_wgrad_any(p, dtype, x, gy, gw, workspace, workspace_bytes, flags, stream, nullptr);
+}
+
+// ---- a convolution over two tensors whose channels follow each other (the skip connection, never concatenated) ------
+extern "C" int sfh_conv3d_pair_supported(const sfh_conv3d_desc* p, int dtype, int32_t cin_first, int direction) {
+  int32_t out[3];
+  if (check_conv(p, dtype, out) != SFH_OK || p->n == 0) return 0;
+  if (direction == 0) return (fwd_uses_mfma(*p, dtype, out) && mfma_conv_pair_ok(fwd_mfma_args(*p, out), cin_first, false)) ? 1 : 0;
+  if (direction == 1)
+    return (check_dgrad(*p) == SFH_OK && dgrad_uses_mfma(*p, dtype, out) && mfma_conv_pair_ok(dgrad_mfma_args(*p, out), cin_first, true)) ? 1 : 0;
+  if (direction == 2) return (wgrad_uses_mfma(*p, dtype, out) && mfma_wgrad_pair_ok(wgrad_args(*p, out), cin_first)) ? 1 : 0;
+  return 0;
+}
+
+extern "C" int sfh_conv3d_fwd_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second, int32_t cin_first,
+                                   const void* w, const int64_t w_stride[5], const void* bias, void* y, void* workspace,
+                                   size_t workspace_bytes, uint32_t flags, int groups, const float* gn_shift, float* gn_partials,
+                                   size_t gn_partials_bytes, void* stream) {
+  if (x_second == nullptr) return fail(SFH_ERR_INVALID, "conv3d fwd pair: null tensor");
+  if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d fwd pair: the direct kernels read one tensor");
+  if (!sfh_conv3d_pair_supported(p, dtype, cin_first, 0))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd pair: not offered for this problem cut at channel %d", (int)cin_first);
+  const ChannelPair in2{const_cast<void*>(x_second), cin_first};
+  if (groups <= 0) return conv3d_fwd_any(p, dtype, x_first, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, nullptr, &in2);
+  const int32_t records = sfh_conv3d_fwd_gn_records(p, dtype, groups);
+  if (records == 0) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd pair: GroupNorm partials are not offered for this problem");
+  const size_t need = (size_t)p->n * records * 2 * groups * sizeof(float);
+  if (gn_partials == nullptr || gn_partials_bytes < need || (reinterpret_cast<uintptr_t>(gn_partials) & 15u) != 0)
+    return fail(SFH_ERR_WORKSPACE, "conv3d fwd pair: GroupNorm partials need %zu bytes at a 16-byte boundary, got %zu", need,
+                gn_partials_bytes);
+  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records, gn_shift};
+  return conv3d_fwd_any(p, dtype, x_first, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, &gn, &in2);
+}
+
+extern "C" int sfh_conv3d_dgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w, const int64_t w_stride[5],
+                                     void* gx_first, void* gx_second, int32_t cin_first, void* workspace, size_t workspace_bytes,
+                                     uint32_t flags, void* stream) {
+  if (gx_second == nullptr) return fail(SFH_ERR_INVALID, "conv3d dgrad pair: null tensor");
+  if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d dgrad pair: the direct kernels write one tensor");
+  if (!sfh_conv3d_pair_supported(p, dtype, cin_first, 1))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad pair: not offered for this problem cut at channel %d", (int)cin_first);
+  const ChannelPair out2{gx_second, cin_first};
+  return conv3d_dgrad_any(p, dtype, gy, w, w_stride, gx_first, workspace, workspace_bytes, flags, stream, &out2);
+}
+
+extern "C" int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second, int32_t cin_first,
+                                     const void* gy, void* gw, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  if (x_second == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad pair: null tensor");
+  if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d wgrad pair: the direct kernels read one tensor");
+  if (!sfh_conv3d_pair_supported(p, dtype, cin_first, 2))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad pair: not offered for this problem cut at channel %d", (int)cin_first);
+  const ChannelPair x2{const_cast<void*>(x_second), cin_first};
+  return conv3d_wgrad_any(p, dtype, x_first, gy, gw, workspace, workspace_bytes, flags, stream, &x2);
 }
 
 // ---- bias gradient ---------------------------------------------------------------------

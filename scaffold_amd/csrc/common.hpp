@@ -92,4 +92,13 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t pid, uint32_t total) {
   return start + slot;
 }
 
+// A channels-last tensor handed over as two tensors over the same voxels whose channels follow each other: the first
+// `first` channels (a multiple of 32) lie in the tensor passed in the usual place, the rest in `second`. It stands for
+// the concatenation along the channels without anyone writing it: the reduction channels of a forward (its input), the
+// produced channels of a data gradient (its output), the input channels of a weight gradient.
+struct ChannelPair {
+  void* second;
+  int first;
+};
+
 }  // namespace sfh

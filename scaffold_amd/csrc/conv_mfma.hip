@@ -69,11 +69,13 @@ __device__ __forceinline__ constexpr int lds_off(int it) {
 }
 
 // WQ: weight fragments in flight per wavefront (see the chunk loop).
-template <typename T, typename C, int WQ>
+// PAIR: the input is two tensors whose channels follow each other (the first `c_first` in x, the rest in x1): every
+// 32-channel chunk is staged from the one that holds it. Independently, a non-null y1 splits the OUTPUT the same way.
+template <typename T, typename C, int WQ, bool PAIR>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
                  T* __restrict__ y, float* __restrict__ partial, int tiles_d, int tiles_h, int tiles_w, int nblocks, int ksplit,
-                 uint32_t total, GnPartialOut gn, int early_weights) {
+                 uint32_t total, GnPartialOut gn, int early_weights, const T* __restrict__ x1, T* __restrict__ y1, int c_first) {
   __shared__ __attribute__((aligned(16))) char lds[C::LDS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -142,7 +144,16 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     }
     __syncthreads();  // every wave is done reading the previous chunk
     {
-      const T* xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cred + cc * kChunk;
+      // channels per voxel of the tensor this chunk lies in, and the chunk's first channel in the sample
+      int row = a.cred;
+      const T* xn;
+      if constexpr (PAIR) {
+        const bool second = cc * kChunk >= c_first;
+        row = second ? a.cred - c_first : c_first;
+        xn = (second ? x1 : x) + (int64_t)n * a.id * a.ih * a.iw * row + (second ? cc * kChunk - c_first : cc * kChunk);
+      } else {
+        xn = x + (int64_t)n * a.id * a.ih * a.iw * a.cred + cc * kChunk;
+      }
 #pragma unroll
       for (int it0 = 0; it0 < ITERS; it0 += BATCH) {
         uint4 v[BATCH];
@@ -160,12 +171,12 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
             const int id = id0 + bd, ih = ih0 + bh, iw = iw0 + bw;
             const bool in = p < PIECES && (unsigned)id < (unsigned)a.id && (unsigned)ih < (unsigned)a.ih && (unsigned)iw < (unsigned)a.iw;
             if constexpr (C::NSUB > 1) {
-              const int64_t at = in ? (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8 : 0;
+              const int64_t at = in ? (((int64_t)id * a.ih + ih) * a.iw + iw) * row + piece * 8 : 0;
               const uint4 got = *reinterpret_cast<const uint4*>(xn + at);
               v[u] = in ? got : make_uint4(0, 0, 0, 0);
             } else {  // registers to spare: the compiler keeps the addresses across chunks and batches every load
               v[u] = make_uint4(0, 0, 0, 0);
-              if (in) v[u] = *reinterpret_cast<const uint4*>(xn + (((int64_t)id * a.ih + ih) * a.iw + iw) * a.cred + piece * 8);
+              if (in) v[u] = *reinterpret_cast<const uint4*>(xn + (((int64_t)id * a.ih + ih) * a.iw + iw) * row + piece * 8);
             }
           }
         }
@@ -251,9 +262,12 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
               make_float4(acc[ms][ns][4 * g], acc[ms][ns][4 * g + 1], acc[ms][ns][4 * g + 2], acc[ms][ns][4 * g + 3]);
       continue;
     }
-    T* yp = y + vox * a.cout + nb * C::NSUB * 32;
 #pragma unroll
     for (int ns = 0; ns < C::NSUB; ++ns) {
+      // the 32-channel block's place in the output: in y, or (an output given as two tensors) in the one that holds it
+      const int ch = (nb * C::NSUB + ns) * 32;
+      T* yp = y + vox * a.cout + ch;
+      if (y1 != nullptr) yp = ch >= c_first ? y1 + vox * (a.cout - c_first) + (ch - c_first) : y + vox * c_first + ch;
       uint32_t run[4][2];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -270,8 +284,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
       uint4 piece[2];
       trade_channel_runs(run, piece);  // all lanes take part, also those of voxels past the edge
       if (inside) {
-        *reinterpret_cast<uint4*>(yp + ns * 32 + 8 * kg) = piece[0];
-        *reinterpret_cast<uint4*>(yp + ns * 32 + 16 + 8 * kg) = piece[1];
+        *reinterpret_cast<uint4*>(yp + 8 * kg) = piece[0];
+        *reinterpret_cast<uint4*>(yp + 16 + 8 * kg) = piece[1];
       }
     }
   }
@@ -419,18 +433,20 @@ int early_weights(int64_t workgroups) {
   return 1;
 }
 
-template <typename T, typename C>
+struct PairPtrs { const void* x1; void* y1; int first; };
+
+template <typename T, typename C, bool PAIR>
 int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
-               float* partial, hipStream_t st, const GnPartialOut& gn) {
+               float* partial, hipStream_t st, const GnPartialOut& gn, const PairPtrs& pr) {
   const int tiles_d = (int)cdiv(a.od, C::TD), tiles_h = (int)cdiv(a.oh, C::TH), tiles_w = (int)cdiv(a.ow, C::TW);
   const int nblocks = a.cout / (32 * C::NSUB);
   const int64_t total = (int64_t)a.n * tiles_d * tiles_h * tiles_w * nblocks * p.ksplit;
   if (total == 0) return SFH_OK;
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: %lld workgroups exceed the grid limit", (long long)total);
 #define SFH_BRICK(WQ)                                                                                                      \
-  hipLaunchKernelGGL((conv_mfma_kernel<T, C, WQ>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed, \
-                     (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit, (uint32_t)total, gn,     \
-                     early_weights(total))
+  hipLaunchKernelGGL((conv_mfma_kernel<T, C, WQ, PAIR>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x,       \
+                     (const T*)packed, (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit,       \
+                     (uint32_t)total, gn, early_weights(total), (const T*)pr.x1, (T*)pr.y1, pr.first)
   if constexpr (C::NSUB > 1) SFH_BRICK(4);
   else if constexpr (C::MS >= 4) SFH_BRICK(6);
   else if (total <= 2 * kComputeUnits) SFH_BRICK(12);
@@ -439,21 +455,21 @@ int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const 
   return check_launch("conv_mfma_kernel");
 }
 
-template <typename T, int NSUB>
+template <typename T, int NSUB, bool PAIR>
 int launch_k333(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const void* packed, const void* bias, void* y,
-                float* partial, hipStream_t st, const GnPartialOut& gn) {
+                float* partial, hipStream_t st, const GnPartialOut& gn, const PairPtrs& pr) {
   // Brick shape follows the row length: 32-voxel sub-tiles are one, two or four W rows.
   switch (p.shape) {
-    case 0: return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 3: return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 6: return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 0: return launch_cfg<T, Tile<4, 4, 32, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 3: return launch_cfg<T, Tile<4, 8, 16, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 6: return launch_cfg<T, Tile<8, 8, 8, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
 #ifdef SFH_GATHER_TUNE  // 128-voxel tiles: built only to be measured
-    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
-    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>>(a, p, x, packed, bias, y, partial, st, gn);
+    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
+    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
 #endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv mfma: no kernel for brick shape %d", p.shape);
   }
@@ -469,11 +485,27 @@ int gather_gn_records(const MfmaConvArgs& a, const GatherPlan& p, int groups) {
   return records <= 0x7fffffff ? (int)records : 0;
 }
 
+// The brick kernel takes any cut of its input, or of its output, at a multiple of the 32-channel chunk (when the
+// reduction is sliced it is the sum of the slices that writes the two tensors).
+bool gather_pair_ok(const MfmaConvArgs& a, int first, bool as_output) {
+  const int channels = as_output ? a.cout : a.cred;
+  return first > 0 && first < channels && first % 32 == 0;
+}
+
 template <typename T>
 int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, void* partial,
-                 hipStream_t st, const GnPartialOut* gn) {
+                 hipStream_t st, const GnPartialOut* gn, const ChannelPair* in2, const ChannelPair* out2) {
   const GatherPlan p = gather_plan(a);
   if (p.ksplit > 1 && partial == nullptr) return fail(SFH_ERR_WORKSPACE, "conv mfma: the reduction split needs its workspace");
+  if (in2 != nullptr && out2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: input and output cannot both be pairs");
+  if (out2 != nullptr && gn != nullptr && gn->part != nullptr)
+    return fail(SFH_ERR_UNSUPPORTED, "conv mfma: no GroupNorm partials of an output written as two tensors");
+  if (in2 != nullptr && (in2->second == nullptr || !gather_pair_ok(a, in2->first, false)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv mfma: the input cannot be cut at channel %d of %d", in2->first, a.cred);
+  if (out2 != nullptr && (out2->second == nullptr || !gather_pair_ok(a, out2->first, true)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv mfma: the output cannot be cut at channel %d of %d", out2->first, a.cout);
+  const PairPtrs pr{in2 != nullptr ? in2->second : nullptr, (out2 != nullptr && p.ksplit == 1) ? out2->second : nullptr,
+                    in2 != nullptr ? in2->first : (out2 != nullptr ? out2->first : 0)};
   GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records != gather_gn_records(a, p, gn->groups) || gn->records == 0)
@@ -484,12 +516,17 @@ int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* pa
   }
   const GnPartialOut none{nullptr, 0, 0, 0, nullptr};
   const GnPartialOut& in_kernel = p.ksplit == 1 ? out : none;
-  const int rc = p.nsub == 2 ? launch_k333<T, 2>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel)
-                             : launch_k333<T, 1>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel);
+  int rc;
+  if (in2 != nullptr)
+    rc = p.nsub == 2 ? launch_k333<T, 2, true>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel, pr)
+                     : launch_k333<T, 1, true>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel, pr);
+  else
+    rc = p.nsub == 2 ? launch_k333<T, 2, false>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel, pr)
+                     : launch_k333<T, 1, false>(a, p, x, packed, bias, y, (float*)partial, st, in_kernel, pr);
   if (rc != SFH_OK || p.ksplit == 1) return rc;
   const int64_t sample = (int64_t)a.od * a.oh * a.ow * a.cout;
   if (out.part != nullptr) return sum_slices_bias_stats(dtype, (const float*)partial, bias, y, a.n, sample, a.cout, p.ksplit, out, st);
-  return sum_slices_bias(dtype, (const float*)partial, bias, y, a.n * sample, a.cout, p.ksplit, st);
+  return sum_slices_bias(dtype, (const float*)partial, bias, y, a.n * sample, a.cout, p.ksplit, st, out2);
 }
 
 }  // namespace
@@ -576,10 +613,18 @@ int mfma_conv_gather_gn_records(const MfmaConvArgs& a, int groups) {
 }
 
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                     void* partial, hipStream_t st, const GnPartialOut* gn) {
-  if (mfma_conv_wide_applies(a)) return mfma_conv_wide(a, dtype, x, packed, bias, y, st, gn);
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st, gn);
-  return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st, gn);
+                     void* partial, hipStream_t st, const GnPartialOut* gn, const ChannelPair* in2, const ChannelPair* out2) {
+  if (mfma_conv_wide_applies(a)) {
+    if (out2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv wide: the output cannot be a pair of tensors");
+    return mfma_conv_wide(a, dtype, x, packed, bias, y, st, gn, in2);
+  }
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st, gn, in2, out2);
+  return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st, gn, in2, out2);
+}
+
+bool mfma_conv_gather_pair_ok(const MfmaConvArgs& a, int first, bool as_output) {
+  if (mfma_conv_wide_applies(a)) return !as_output && mfma_conv_wide_pair_ok(a, first);
+  return gather_pair_ok(a, first, as_output);
 }
 
 }  // namespace sfh

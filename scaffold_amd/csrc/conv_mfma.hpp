@@ -16,6 +16,9 @@ struct MfmaConvArgs {
 };
 
 bool mfma_conv_supported(const MfmaConvArgs& a, int dtype);
+// Whether the kernel that serves problem `a` reads its input as a ChannelPair cut at `first` (as_output: writes its
+// output as one): a pure function of the shape. The results are the bits of the same launch on the concatenation.
+bool mfma_conv_pair_ok(const MfmaConvArgs& a, int first, bool as_output);
 size_t mfma_conv_packed_weight_bytes(const MfmaConvArgs& a);
 // Repacks the weight into per-wavefront MFMA fragment order:
 //   packed[cout/32][cred/32][tap][kstep(2)][lane(64)][8]
@@ -36,20 +39,25 @@ int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStrea
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a);
 // `gn` (optional): also leave GroupNorm partials of the rounded output (gn_stats.hpp), gn->records per sample as
 // mfma_conv_gn_records says for gn->groups groups.
+// `in2` / `out2` (optional, where mfma_conv_pair_ok says so): x / y given as a ChannelPair.
 int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                     void* partial, hipStream_t st, const GnPartialOut* gn = nullptr);
+                     void* partial, hipStream_t st, const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr,
+                     const ChannelPair* out2 = nullptr);
 // Same contract, wide-tile kernel (64 or more reduction channels, rows of more than 16 voxels): `applies` is a pure
 // function of the shape; mfma_conv_gather routes to it (it needs no partial workspace).
 bool mfma_conv_wide_applies(const MfmaConvArgs& a);
 int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                   const GnPartialOut* gn = nullptr);
+                   const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr);
 // Same contract, persistent one-workgroup-per-CU kernel with register-resident weights.
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                      void* partial, hipStream_t st, const GnPartialOut* gn = nullptr);
+                      void* partial, hipStream_t st, const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr,
+                      const ChannelPair* out2 = nullptr);
 // Records of GroupNorm partials per sample that mfma_conv_persist leaves for `groups` groups: a pure function of the
 // shape; 0 when the kernel that serves the problem does not offer them (the caller then runs the statistics pass).
 int mfma_conv_gn_records(const MfmaConvArgs& a, int groups);
 int mfma_conv_gather_gn_records(const MfmaConvArgs& a, int groups);
+bool mfma_conv_gather_pair_ok(const MfmaConvArgs& a, int first, bool as_output);
+bool mfma_conv_wide_pair_ok(const MfmaConvArgs& a, int first);  // input pairs only, cut in the middle
 int mfma_conv_wide_gn_records(const MfmaConvArgs& a, int groups);
 
 // Which of the three kernels mfma_conv_persist ends up launching for a problem, and with what geometry: a pure function of

@@ -176,9 +176,10 @@ __device__ __forceinline__ int store_offset(const MfmaConvArgs& a, const TileCoo
   const int ok = (tc.d * C::TD + td < a.od) & (tc.h * C::TH + th < a.oh) & (tc.w * C::TW + tw < a.ow);
   return ok ? vrel : kRange;
 }
+// `row`: channels per voxel of the tensor written, `c0`: the workgroup's first channel in it.
 template <typename T, typename C>
-__device__ __forceinline__ T* tile_origin(const MfmaConvArgs& a, T* y, const TileCoord& tc, int nb) {
-  return y + ((((int64_t)tc.n * a.od + tc.d * C::TD) * a.oh + tc.h * C::TH) * a.ow + tc.w * C::TW) * a.cout + nb * 32;
+__device__ __forceinline__ T* tile_origin(const MfmaConvArgs& a, T* y, const TileCoord& tc, int row, int c0) {
+  return y + ((((int64_t)tc.n * a.od + tc.d * C::TD) * a.oh + tc.h * C::TH) * a.ow + tc.w * C::TW) * row + c0;
 }
 
 // Output of a finished brick, rounded, waiting to be stored during the next step. Accumulator register 4g+t of a
@@ -297,7 +298,7 @@ __device__ __forceinline__ void persist_step(const MfmaConvArgs& a, const char* 
 template <typename T, typename C, bool BIAS, bool GN>
 __global__ void __launch_bounds__(256, 1)
 conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias_ptr,
-                    T* __restrict__ y, PersistGeom gm, GnPartialOut gn) {
+                    T* __restrict__ y, PersistGeom gm, GnPartialOut gn, T* __restrict__ y1, int c_first) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space builtins the host pass cannot type-check
   __shared__ __attribute__((aligned(16))) char buf0[C::BRICK];
   __shared__ __attribute__((aligned(16))) char buf1[C::BRICK];
@@ -314,6 +315,17 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   if (nb >= gm.nblocks || tile_begin >= tile_end) return;
   const int nsteps = tile_end - tile_begin;
 
+  // Where this workgroup's 32 output channels go: into y, or -- an output handed over as two tensors whose channels
+  // follow each other, the first c_first in y and the rest in y1 -- into the one that holds them. Fixed for the launch.
+  T* yout = y;
+  int yrow = a.cout, yc0 = nb * 32;
+  if (y1 != nullptr) {
+    const bool second = nb * 32 >= c_first;
+    yout = second ? y1 : y;
+    yrow = second ? a.cout - c_first : c_first;
+    yc0 = second ? nb * 32 - c_first : nb * 32;
+  }
+
   LaneGeom<C> lg;
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
@@ -321,7 +333,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     const int tw = v % C::TW, th = (v / C::TW) % C::TH, td = v / (C::TW * C::TH);
     lg.lbase[ms] = kg * C::PLANE + ((td * C::BH + th) * C::BW + tw) * 16;
     lg.vcoord[ms] = td | (th << 8) | (tw << 16);
-    lg.vrel[ms] = (((td * a.oh + th) * a.ow + tw) * a.cout + 8 * kg) * 2;
+    lg.vrel[ms] = (((td * a.oh + th) * a.ow + tw) * yrow + 8 * kg) * 2;
   }
   // Staging role of this lane, fixed for the whole launch: wave w fills the 64-voxel groups w, w+4, ... of every
   // plane; the lane's voxel inside the brick and its byte offset from the brick origin in the input tensor.
@@ -368,7 +380,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   int done_off[C::MS];
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) done_off[ms] = kRange;  // nothing to store during the first step
-  T* done_origin = y;
+  T* done_origin = yout;
   RunSums gn_sums;  // GroupNorm statistics of this workgroup's rounded outputs (GN)
   gn_sums.clear();
   if constexpr (GN) gn_sums.load_shift(gn.shift, 0, gn.groups, gn.cg, nb * 32, kg);
@@ -382,7 +394,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
     asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMAs are inline asm: the compiler does not know their result latency
     round_brick<T, C, BIAS, GN>(acc, bias, ps, a, tc, lg, gn_sums);  // its stores ride along with the next step's MFMAs
-    done_origin = tile_origin<T, C>(a, y, tc, nb);
+    done_origin = tile_origin<T, C>(a, yout, tc, yrow, yc0);
     tc = tc1;
     tc1 = tc2;
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // this wave's part of the next brick has landed
@@ -429,14 +441,14 @@ PersistGeom persist_geom(const MfmaConvArgs& a) {
 
 template <typename T, typename C>
 int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                const GnPartialOut& gn) {
+                const GnPartialOut& gn, const ChannelPair& out2) {
   const PersistGeom gm = persist_geom(a, C::TD, C::TH, C::TW);
   if (gm.ntiles < 0) return fail(SFH_ERR_UNSUPPORTED, "conv mfma: too many bricks");
   if (gm.ntiles == 0) return SFH_OK;
   const unsigned grid = (unsigned)(gm.wgs_per_block * gm.nblocks);
 #define SFH_PERSIST(BIAS, GN)                                                                                                    \
   hipLaunchKernelGGL((conv_persist_kernel<T, C, BIAS, GN>), dim3(grid), dim3(256), 0, st, a, (const T*)x, (const T*)packed, \
-                     (const T*)bias, (T*)y, gm, gn)
+                     (const T*)bias, (T*)y, gm, gn, (T*)out2.second, out2.first)
   if (bias != nullptr) {
     if (gn.part != nullptr) SFH_PERSIST(true, true);
     else SFH_PERSIST(true, false);
@@ -450,10 +462,10 @@ int launch_tile(const MfmaConvArgs& a, const void* x, const void* packed, const 
 
 template <typename T>
 int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                 const GnPartialOut& gn) {
-  if (a.ow > 16) return launch_tile<T, PTile<4, 4, 32>>(a, x, packed, bias, y, st, gn);
-  if (a.ow > 8) return launch_tile<T, PTile<4, 8, 16>>(a, x, packed, bias, y, st, gn);
-  return launch_tile<T, PTile<8, 8, 8>>(a, x, packed, bias, y, st, gn);
+                 const GnPartialOut& gn, const ChannelPair& out2) {
+  if (a.ow > 16) return launch_tile<T, PTile<4, 4, 32>>(a, x, packed, bias, y, st, gn, out2);
+  if (a.ow > 8) return launch_tile<T, PTile<4, 8, 16>>(a, x, packed, bias, y, st, gn, out2);
+  return launch_tile<T, PTile<8, 8, 8>>(a, x, packed, bias, y, st, gn, out2);
 }
 
 }  // namespace
@@ -482,9 +494,21 @@ int mfma_conv_gn_records(const MfmaConvArgs& a, int groups) {
   return gm.wgs_per_block * (cg > 32 ? cg / 32 : 1);
 }
 
+// A persistent workgroup owns one 32-channel output block for the whole launch: any cut of the OUTPUT at a multiple of
+// 32 channels falls between workgroups (a tile of either tensor spans less than the kernel's addressing range a
+// fortiori). Its 32 reduction channels cannot be cut.
+bool mfma_conv_pair_ok(const MfmaConvArgs& a, int first, bool as_output) {
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather_pair_ok(a, first, as_output);
+  return as_output && first > 0 && first < a.cout && first % 32 == 0;
+}
+
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
-                      void* partial, hipStream_t st, const GnPartialOut* gn) {
-  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st, gn);
+                      void* partial, hipStream_t st, const GnPartialOut* gn, const ChannelPair* in2, const ChannelPair* out2) {
+  if (!mfma_conv_persist_applies(a)) return mfma_conv_gather(a, dtype, x, packed, bias, y, partial, st, gn, in2, out2);
+  if (in2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv persist: 32 reduction channels cannot be a pair of tensors");
+  if (out2 != nullptr && (out2->second == nullptr || !mfma_conv_pair_ok(a, out2->first, true)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv persist: the output cannot be cut at channel %d of %d", out2->first, a.cout);
+  const ChannelPair pair = out2 != nullptr ? *out2 : ChannelPair{nullptr, 0};
   GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_gn_records(a, gn->groups))
@@ -493,8 +517,8 @@ int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const voi
     out = *gn;
     out.cg = a.cout / gn->groups;
   }
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st, out);
-  return launch_typed<fp16_t>(a, x, packed, bias, y, st, out);
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st, out, pair);
+  return launch_typed<fp16_t>(a, x, packed, bias, y, st, out, pair);
 }
 
 }  // namespace sfh

@@ -145,6 +145,9 @@ struct WideCtx {
   int lbase[C::MS];  // LDS byte offset of the lane's activation fragment voxel at tap (0,0,0), per sub-tile
   int voff[C::GPW];  // staging: byte offset of the lane's voxel from the brick origin; kRange outside the input, -1 past the brick
   __amdgpu_buffer_rsrc_t xrsrc, wrsrc;
+  // an input given as two tensors of equal channel counts: the second one's descriptor and its first 16-channel chunk
+  __amdgpu_buffer_rsrc_t xrsrc1;
+  int chunk1;
 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -158,14 +161,19 @@ __device__ __forceinline__ int frag_offset(const WideCtx<T, C>& k, int ns, int c
 }
 // I-th brick load of this wavefront for chunk `chunk` into the brick buffer `dst`: wavefront w fills the 64-voxel
 // groups w, w + 4, ... of both planes
-template <typename T, typename C, int I>
+template <typename T, typename C, int I, bool PAIR>
 __device__ __forceinline__ void brick_load(const WideCtx<T, C>& k, int chunk, lds_bytes dst) {
   constexpr int g = I >> 1, p = I & 1;
   constexpr bool full = (3 + 4 * g) * 64 + 63 < C::BV;  // only a wavefront's last group can have lanes past the brick
   // (the instruction's immediate offset would move the LDS destination as well: the plane's 16 bytes go into the scalar offset)
-  if (full || k.voff[g] != -1)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(k.xrsrc, (lds_ptr)(dst + p * C::PLANE + (k.wave + 4 * g) * 1024), 16, k.voff[g],
-                                             chunk * 32 + p * 16, 0, 0);
+  if (full || k.voff[g] != -1) {
+    if (PAIR && chunk >= k.chunk1)  // the chunk lies in the second tensor (same voxel offsets: equal channel counts)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k.xrsrc1, (lds_ptr)(dst + p * C::PLANE + (k.wave + 4 * g) * 1024), 16, k.voff[g],
+                                               (chunk - k.chunk1) * 32 + p * 16, 0, 0);
+    else
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(k.xrsrc, (lds_ptr)(dst + p * C::PLANE + (k.wave + 4 * g) * 1024), 16, k.voff[g],
+                                               chunk * 32 + p * 16, 0, 0);
+  }
 }
 // this wavefront's three fragments of step `u` of chunk `chunk` into the ring slot `dst`
 template <typename T, typename C>
@@ -180,10 +188,11 @@ __device__ __forceinline__ void weight_loads(const WideCtx<T, C>& k, int chunk, 
   }
 }
 
-template <typename T, typename C>
+// PAIR: the input is two tensors of a.cred / 2 channels each whose channels follow each other (x, then x1).
+template <typename T, typename C, bool PAIR>
 __global__ void __launch_bounds__(256, 1)
 conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias, T* __restrict__ y,
-                 WideGeom gm, GnPartialOut gn) {
+                 WideGeom gm, GnPartialOut gn, const T* __restrict__ x1) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses LDS address-space builtins the host pass cannot type-check
   __shared__ __attribute__((aligned(16))) char brick0_[C::BRICK];
   __shared__ __attribute__((aligned(16))) char brick1_[C::BRICK];
@@ -217,21 +226,28 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   }
   // Staging role of the lane: byte offset of its voxel of group wave + 4g from the (possibly virtual) brick origin,
   // kRange when the voxel lies outside the input (such loads return zeros), -1 past the brick.
+  const int row = PAIR ? a.cred / 2 : a.cred;  // channels per voxel of the tensor(s) read
 #pragma unroll
   for (int g = 0; g < C::GPW; ++g) {
     const int vox = (k.wave + 4 * g) * 64 + k.lane;
     const int bw = vox % C::BW, bh = (vox / C::BW) % C::BH, bd = vox / (C::BW * C::BH);
     const bool inside = (unsigned)(id0 + bd) < (unsigned)a.id && (unsigned)(ih0 + bh) < (unsigned)a.ih && (unsigned)(iw0 + bw) < (unsigned)a.iw;
-    k.voff[g] = vox >= C::BV ? -1 : (inside ? (((bd * a.ih + bh) * a.iw + bw) * a.cred) * 2 : kRange);
+    k.voff[g] = vox >= C::BV ? -1 : (inside ? (((bd * a.ih + bh) * a.iw + bw) * row) * 2 : kRange);
   }
-  const T* origin = x + ((((int64_t)n * a.id + id0) * a.ih + ih0) * a.iw + iw0) * a.cred;
-  k.xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(origin), 0, kRange, 0x00020000);
+  const int64_t origin = ((((int64_t)n * a.id + id0) * a.ih + ih0) * a.iw + iw0) * row;
+  k.xrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x + origin), 0, kRange, 0x00020000);
+  k.xrsrc1 = k.xrsrc;
+  k.chunk1 = 0;
+  if constexpr (PAIR) {
+    k.xrsrc1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x1 + origin), 0, kRange, 0x00020000);
+    k.chunk1 = row / 16;
+  }
   k.wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(wp), 0, 0x7fffffff, 0x00020000);
 
   f32x16_t acc[C::MS][C::NSUB];
   {
     // ---- prologue: the first chunk's brick, the first step's weights -------------------------------------------
-    static_for<C::NLOAD>([&](auto i_c) { brick_load<T, C, decltype(i_c)::value>(k, c_begin, brick0); });
+    static_for<C::NLOAD>([&](auto i_c) { brick_load<T, C, decltype(i_c)::value, PAIR>(k, c_begin, brick0); });
     weight_loads<T, C>(k, c_begin, 0, wslot0);
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
@@ -285,7 +301,7 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
         for (int ns = 0; ns < C::NSUB; ++ns) landed(b_cur[ns]);
         // brick loads of the next chunk: window u starts at the first tap of step u, one load per tap
         if constexpr ((tap - u * C::TPS) < C::window_loads(u)) {
-          if (more) brick_load<T, C, C::window_first(u) + tap - u * C::TPS>(k, c + 1, nxt);
+          if (more) brick_load<T, C, C::window_first(u) + tap - u * C::TPS, PAIR>(k, c + 1, nxt);
         }
         // This tap's MFMAs with the operand reads of the next tap spread between them.
         frag_t a_nxt[C::MS], b_nxt[C::NSUB];
@@ -405,7 +421,7 @@ WidePlan wide_plan(const MfmaConvArgs& a) {
 
 template <typename T, typename C>
 int launch_wide(const MfmaConvArgs& a, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                const GnPartialOut& gn) {
+                const GnPartialOut& gn, const void* x1) {
   WideGeom gm{};
   gm.tiles_d = (int)cdiv(a.od, C::TD);
   gm.tiles_h = (int)cdiv(a.oh, C::TH);
@@ -415,21 +431,25 @@ int launch_wide(const MfmaConvArgs& a, const void* x, const void* packed, const 
   if (total == 0) return SFH_OK;
   if (total > 0x7fffffffLL) return fail(SFH_ERR_UNSUPPORTED, "conv wide: %lld workgroups exceed the grid limit", (long long)total);
   gm.total = (uint32_t)total;
-  hipLaunchKernelGGL((conv_wide_kernel<T, C>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed, (const T*)bias,
-                     (T*)y, gm, gn);
+  if (x1 != nullptr)
+    hipLaunchKernelGGL((conv_wide_kernel<T, C, true>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
+                       (const T*)bias, (T*)y, gm, gn, (const T*)x1);
+  else
+    hipLaunchKernelGGL((conv_wide_kernel<T, C, false>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)packed,
+                       (const T*)bias, (T*)y, gm, gn, (const T*)nullptr);
   return check_launch("conv_wide_kernel");
 }
 
 template <typename T>
 int launch_typed(const MfmaConvArgs& a, const WidePlan& p, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                 const GnPartialOut& gn) {
+                 const GnPartialOut& gn, const void* x1) {
   switch (p.shape) {
-    case 1: return launch_wide<T, WTile<8, 4, 32, 2>>(a, x, packed, bias, y, st, gn);
-    case 3: return launch_wide<T, WTile<4, 4, 32, 2>>(a, x, packed, bias, y, st, gn);
+    case 1: return launch_wide<T, WTile<8, 4, 32, 2>>(a, x, packed, bias, y, st, gn, x1);
+    case 3: return launch_wide<T, WTile<4, 4, 32, 2>>(a, x, packed, bias, y, st, gn, x1);
 #ifdef SFH_WIDE_TUNE  // the other accumulator grids: built only to be measured
-    case 0: return launch_wide<T, WTile<4, 4, 32, 4>>(a, x, packed, bias, y, st, gn);
-    case 2: return launch_wide<T, WTile<8, 4, 32, 1>>(a, x, packed, bias, y, st, gn);
-    case 4: return launch_wide<T, WTile<4, 4, 32, 1>>(a, x, packed, bias, y, st, gn);
+    case 0: return launch_wide<T, WTile<4, 4, 32, 4>>(a, x, packed, bias, y, st, gn, x1);
+    case 2: return launch_wide<T, WTile<8, 4, 32, 1>>(a, x, packed, bias, y, st, gn, x1);
+    case 4: return launch_wide<T, WTile<4, 4, 32, 1>>(a, x, packed, bias, y, st, gn, x1);
 #endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv wide: no kernel for accumulator grid %d", p.shape);
   }
@@ -457,10 +477,16 @@ int mfma_conv_wide_gn_records(const MfmaConvArgs& a, int groups) {
   return records <= 0x7fffffff ? (int)records : 0;
 }
 
+// The staging offsets of a lane are those of one tensor: a pair must be two tensors of the same channel count.
+bool mfma_conv_wide_pair_ok(const MfmaConvArgs& a, int first) { return wide_plan(a).use && first * 2 == a.cred && first % 16 == 0; }
+
 int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
-                   const GnPartialOut* gn) {
+                   const GnPartialOut* gn, const ChannelPair* in2) {
   const WidePlan p = wide_plan(a);
   if (!p.use) return fail(SFH_ERR_UNSUPPORTED, "conv wide: not applicable to this problem");
+  if (in2 != nullptr && (in2->second == nullptr || !mfma_conv_wide_pair_ok(a, in2->first)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv wide: the input cannot be cut at channel %d of %d", in2->first, a.cred);
+  const void* x1 = in2 != nullptr ? in2->second : nullptr;
   GnPartialOut out{nullptr, 0, 0, 0, nullptr};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_wide_gn_records(a, gn->groups))
@@ -469,8 +495,8 @@ int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* 
     out = *gn;
     out.cg = a.cout / gn->groups;
   }
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, p, x, packed, bias, y, st, out);
-  return launch_typed<fp16_t>(a, p, x, packed, bias, y, st, out);
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, p, x, packed, bias, y, st, out, x1);
+  return launch_typed<fp16_t>(a, p, x, packed, bias, y, st, out, x1);
 }
 
 }  // namespace sfh

@@ -110,9 +110,12 @@ int launch_sum(const float* part, void* out, int64_t nelem, int splits, hipStrea
 }
 
 // Four consecutive elements per thread (16-byte loads of every slice), bias added before the one rounding.
+// A non-null out1 splits the result along the channels: the first c_first of every row of `channels` go to `out`, the
+// rest to out1 (both dense; c_first a multiple of 4, so a thread's four channels stay together).
 template <typename T>
 __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __restrict__ part, const T* __restrict__ bias,
-                                                                 T* __restrict__ out, int64_t nelem, int channels, int splits) {
+                                                                 T* __restrict__ out, int64_t nelem, int channels, int splits,
+                                                                 T* __restrict__ out1, int c_first) {
   const int64_t e = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4;
   if (e >= nelem) return;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -124,10 +127,16 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __
     const int c = (int)(e % channels);
     s.x += to_float(bias[c]); s.y += to_float(bias[c + 1]); s.z += to_float(bias[c + 2]); s.w += to_float(bias[c + 3]);
   }
-  out[e] = elem<T>::from_float(s.x);
-  out[e + 1] = elem<T>::from_float(s.y);
-  out[e + 2] = elem<T>::from_float(s.z);
-  out[e + 3] = elem<T>::from_float(s.w);
+  T* o = out + e;
+  if (out1 != nullptr) {
+    const int64_t row = e / channels;
+    const int c = (int)(e - row * channels);
+    o = c >= c_first ? out1 + row * (channels - c_first) + (c - c_first) : out + row * c_first + c;
+  }
+  o[0] = elem<T>::from_float(s.x);
+  o[1] = elem<T>::from_float(s.y);
+  o[2] = elem<T>::from_float(s.z);
+  o[3] = elem<T>::from_float(s.w);
 }
 
 // sum_slices_bias that also leaves GroupNorm partials of the rounded result (16-bit outputs): a workgroup owns `chunks`
@@ -297,18 +306,20 @@ int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int split
 }
 
 int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, int64_t nelem, int channels, int splits,
-                    hipStream_t st) {
+                    hipStream_t st, const ChannelPair* out2) {
+  void* out1 = out2 != nullptr ? out2->second : nullptr;
+  const int c_first = out2 != nullptr ? out2->first : 0;
   if (nelem <= 0) return SFH_OK;
   const dim3 grid((unsigned)cdiv(nelem / 4, kBlock));
   if (dtype == SFH_BF16)
     hipLaunchKernelGGL(sum_slices_bias_kernel<bf16_t>, grid, dim3(kBlock), 0, st, part, (const bf16_t*)bias, (bf16_t*)out, nelem,
-                       channels, splits);
+                       channels, splits, (bf16_t*)out1, c_first);
   else if (dtype == SFH_FP16)
     hipLaunchKernelGGL(sum_slices_bias_kernel<fp16_t>, grid, dim3(kBlock), 0, st, part, (const fp16_t*)bias, (fp16_t*)out, nelem,
-                       channels, splits);
+                       channels, splits, (fp16_t*)out1, c_first);
   else
     hipLaunchKernelGGL(sum_slices_bias_kernel<float>, grid, dim3(kBlock), 0, st, part, (const float*)bias, (float*)out, nelem,
-                       channels, splits);
+                       channels, splits, (float*)out1, c_first);
   return check_launch("sum_slices_bias_kernel");
 }
 

@@ -8,8 +8,9 @@ namespace sfh {
 int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st);
 
 // out[e] = bias[e % channels] + sum over s < splits, in index order, of part[s * nelem + e]; nelem a multiple of 4.
+// `out2` (optional): the result as two tensors cut at channel out2->first of every row of `channels`.
 int sum_slices_bias(int dtype, const float* part, const void* bias, void* out, int64_t nelem, int channels, int splits,
-                    hipStream_t st);
+                    hipStream_t st, const ChannelPair* out2 = nullptr);
 
 // The same with GroupNorm partials of the rounded result (gn_stats.hpp) for n samples of sample_elems elements each:
 // `records` per sample as sum_slices_bias_stats_records says (0: not offered for this shape; 16-bit outputs only).

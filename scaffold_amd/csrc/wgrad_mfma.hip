@@ -320,7 +320,8 @@ struct SlotLoop {
 template <typename T, typename C>
 __global__ void __launch_bounds__(512)
 wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws, int tiles_d,
-                  int tiles_h, int tiles_w, int ntiles, int tiles_per_split, int nblk_ci, int nblk, uint32_t total) {
+                  int tiles_h, int tiles_w, int ntiles, int tiles_per_split, int nblk_ci, int nblk, uint32_t total,
+                  const T* __restrict__ x1, int c_first) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) char buf0[C::LDS];
   __shared__ __attribute__((aligned(16))) char buf1[C::LDS];
@@ -339,14 +340,26 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   if (wave >= 4) {
     // ---- staging wavefronts ----
     if (t_begin >= t_end) return;
+    // An input handed over as two tensors whose channels follow each other (the first c_first in x, the rest in x1):
+    // the workgroup's 32 input channels lie in one of them, and from here on that tensor IS the input -- its channel
+    // count in `as`, the block's index inside it in `cis`. Only the gradient's own indexing keeps a.cin and cib.
+    WgradArgs as = a;
+    const T* xs = x;
+    int cis = cib;
+    if (x1 != nullptr) {
+      const bool second = cib * 32 >= c_first;
+      xs = second ? x1 : x;
+      as.cin = second ? a.cin - c_first : c_first;
+      cis = second ? cib - c_first / 32 : cib;
+    }
     Slots<C> sl;
-    init_slots<C>(a, tid - 256, sl);
+    init_slots<C>(as, tid - 256, sl);
     auto origin = [&](int tile) {
       return decode_tile(tile < t_end ? tile : t_end - 1, tiles_d, tiles_h, tiles_w, C::TD, C::TH, C::TW);
     };
-    SlotLoop<T, C, 0>::fetch_all(a, x, gy, origin(t_begin), cib, cob, sl);
+    SlotLoop<T, C, 0>::fetch_all(as, xs, gy, origin(t_begin), cis, cob, sl);
     SlotLoop<T, C, 0>::stage_all(buf0, sl);
-    SlotLoop<T, C, 0>::fetch_all(a, x, gy, origin(t_begin + 1), cib, cob, sl);
+    SlotLoop<T, C, 0>::fetch_all(as, xs, gy, origin(t_begin + 1), cis, cob, sl);
     __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
     __builtin_amdgcn_s_barrier();
     for (int tile = t_begin; tile < t_end; ++tile) {
@@ -354,7 +367,7 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
       // On the last tiles the staged / fetched data is never used; doing the work anyway keeps the loop free of
       // branches (the fetch is clamped to the split's last tile).
       const TileOrigin o2 = origin(tile + 2);
-      SlotLoop<T, C, 0>::stage_and_refill(idle, a, x, gy, o2, cib, cob, sl);
+      SlotLoop<T, C, 0>::stage_and_refill(idle, as, xs, gy, o2, cis, cob, sl);
       __builtin_amdgcn_s_waitcnt(kWaitLgkm0);  // the LDS writes of the next tile have landed
       __builtin_amdgcn_s_barrier();            // ... and the compute wavefronts are done reading the current one
     }
@@ -426,24 +439,26 @@ Plan make_plan(const WgradArgs& a) {
 }
 
 template <typename T, typename C>
-int launch_tile(const WgradArgs& a, const Plan& p, const void* x, const void* gy, float* ws, hipStream_t st) {
+int launch_tile(const WgradArgs& a, const Plan& p, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2) {
   const int64_t total = (int64_t)p.splits * p.nblk;
   hipLaunchKernelGGL((wgrad_mfma_kernel<T, C>), dim3((unsigned)total), dim3(512), 0, st, a, (const T*)x, (const T*)gy, ws,
-                     p.tiles_d, p.tiles_h, p.tiles_w, p.ntiles, p.tiles_per_split, p.nblk_ci, p.nblk, (uint32_t)total);
+                     p.tiles_d, p.tiles_h, p.tiles_w, p.ntiles, p.tiles_per_split, p.nblk_ci, p.nblk, (uint32_t)total,
+                     (const T*)x2.second, x2.first);
   return check_launch("wgrad_mfma_kernel");
 }
 
 template <typename T>
-int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace, hipStream_t st) {
+int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace, hipStream_t st,
+                 const ChannelPair& x2) {
   const Plan p = make_plan(a);
   // One slice and an fp32 gradient (the deepest levels under fp32 master weights): the kernel's slice IS the
   // gradient, so it is written in place and no sum pass follows.
   const bool direct = p.splits == 1 && gw_dtype == SFH_FP32;
   float* ws = direct ? (float*)gw : (float*)workspace;
   int rc;
-  if (p.tw == 32) rc = launch_tile<T, WTile<2, 4, 32>>(a, p, x, gy, ws, st);
-  else if (p.tw == 16) rc = launch_tile<T, WTile<2, 8, 16>>(a, p, x, gy, ws, st);
-  else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st);
+  if (p.tw == 32) rc = launch_tile<T, WTile<2, 4, 32>>(a, p, x, gy, ws, st, x2);
+  else if (p.tw == 16) rc = launch_tile<T, WTile<2, 8, 16>>(a, p, x, gy, ws, st, x2);
+  else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st, x2);
   if (rc != SFH_OK || direct) return rc;
   const int64_t nelem = (int64_t)a.cout * 27 * a.cin;
   return sum_slices(gw_dtype, ws, gw, nelem, p.splits, st);
@@ -471,10 +486,15 @@ size_t mfma_wgrad_workspace_bytes(const WgradArgs& a) {
   return align_up((size_t)p.splits * a.cout * 27 * a.cin * sizeof(float), 256);
 }
 
+bool mfma_wgrad_pair_ok(const WgradArgs& a, int first) { return first > 0 && first < a.cin && first % 32 == 0; }
+
 int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace,
-               hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, gy, gw, gw_dtype, workspace, st);
-  return launch_typed<fp16_t>(a, x, gy, gw, gw_dtype, workspace, st);
+               hipStream_t st, const ChannelPair* x2) {
+  if (x2 != nullptr && (x2->second == nullptr || !mfma_wgrad_pair_ok(a, x2->first)))
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad: the input cannot be cut at channel %d of %d", x2->first, a.cin);
+  const ChannelPair pair = x2 != nullptr ? *x2 : ChannelPair{nullptr, 0};
+  if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, gy, gw, gw_dtype, workspace, st, pair);
+  return launch_typed<fp16_t>(a, x, gy, gw, gw_dtype, workspace, st, pair);
 }
 
 }  // namespace sfh

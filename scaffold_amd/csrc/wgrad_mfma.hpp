@@ -15,7 +15,10 @@ bool mfma_wgrad_supported(const WgradArgs& a, int dtype);
 int mfma_wgrad_splits(const WgradArgs& a);
 size_t mfma_wgrad_workspace_bytes(const WgradArgs& a);
 // gw is written in gw_dtype (the operands' dtype, or SFH_FP32 for a full-precision gradient).
+// `x2` (optional, where mfma_wgrad_pair_ok says so): x given as two tensors whose channels follow each other (the
+// first x2->first in x, the rest in x2->second); the gradient is the one of their concatenation, bit for bit.
+bool mfma_wgrad_pair_ok(const WgradArgs& a, int first);
 int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace,
-               hipStream_t st);
+               hipStream_t st, const ChannelPair* x2 = nullptr);
 
 }  // namespace sfh
