@@ -119,7 +119,7 @@ class _Conv3dFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None,
-                gn_groups=0, gn_shift=None):
+                gn_groups=0, gn_shift=None, second=None, slab2=None):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
@@ -130,6 +130,12 @@ class _Conv3dFn(torch.autograd.Function):
         if slab is not None:
             ctx.halo, ctx.depth = slab[1], x.shape[2]
             x = slab[0]
+        # `second`: the input is the pair (x, second) whose channels follow each other -- a skip connection and the
+        # upsampled tensor, never concatenated; `slab2` is to `second` what `slab` is to x
+        ctx.pair = second is not None
+        if slab2 is not None:
+            second = slab2[0]
+        in_shape = x.shape if second is None else torch.Size((x.shape[0], x.shape[1] + second.shape[1], *x.shape[2:]))
         pf = pd = None
         if packs is not None:
             # packed forms that are current (kept by the module, refreshed by whoever writes the weight)
@@ -138,11 +144,16 @@ class _Conv3dFn(torch.autograd.Function):
             # When the data gradient will be wanted too, the weight can be packed for both directions in one launch.
             # That saves a launch per convolution on the GPU and costs a little more host time, so it is done where
             # host time is free (under graph capture) or when asked for (PACK_WEIGHTS_ONCE).
-            pf, pd = _c3.pack_weights(wc, x.shape, stride, padding, dilation)
+            pf, pd = _c3.pack_weights(wc, in_shape, stride, padding, dilation)
         # gn_groups: a GroupNorm of that many groups follows; the launch leaves its statistics on y where it can
-        y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, gn_shift=gn_shift,
-                               _checked=True)
-        ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
+        if second is None:
+            y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, gn_shift=gn_shift,
+                                   _checked=True)
+            ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
+        else:
+            y = _c3.conv3d_forward_pair(x, second, wc, bc, stride, padding, dilation, packed_weight=pf, gn_groups=gn_groups,
+                                        gn_shift=gn_shift, _checked=True)
+            ctx.save_for_backward(x, wc, second) if pd is None else ctx.save_for_backward(x, wc, second, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
         return y
@@ -150,6 +161,8 @@ class _Conv3dFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_output):
+        if ctx.pair:
+            return _Conv3dFn._backward_pair(ctx, grad_output)
         x, weight, *packed = ctx.saved_tensors
         stride, padding, dilation, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
@@ -166,17 +179,59 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
+
+    @staticmethod
+    def _backward_pair(ctx, grad_output):
+        """The three gradients of the convolution over (x, second): the data gradient comes back as the two tensors the
+        concatenation's backward would have cut it into."""
+        x, weight, second, *packed = ctx.saved_tensors
+        stride, padding, dilation, has_bias, bias_dtype, master = ctx.conv_args
+        needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
+        needs_second = ctx.needs_input_grad[12]
+        grad_output = grad_output.contiguous(memory_format=_CL3D)
+        grad_x = grad_second = None
+        if needs_x or needs_second:
+            in_shape = torch.Size((x.shape[0], x.shape[1] + second.shape[1], *x.shape[2:]))
+            grad_x, grad_second = _c3.conv3d_backward_data_pair(grad_output, weight, in_shape, int(x.shape[1]), stride, padding,
+                                                                dilation, packed_weight=packed[0] if packed else None, _checked=True)
+            if ctx.halo:  # both tensors are slabs of the same depth: the interiors are the inputs' gradients
+                grad_x = grad_x[:, :, ctx.halo:ctx.halo + ctx.depth]
+                grad_second = grad_second[:, :, ctx.halo:ctx.halo + ctx.depth]
+        grad_w = None
+        if needs_w:
+            if master:
+                grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight_pair, x, second, weight.shape, grad_output, stride, padding,
+                                           dilation, _checked=True)
+            else:
+                grad_w = _c3.conv3d_backward_weight_pair(x, second, weight.shape, grad_output, stride, padding, dilation, _checked=True)
+        grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
+        return (grad_x if needs_x else None, grad_w, grad_b, None, None, None, None, None, None, None, None, None,
+                grad_second if needs_second else None, None)
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, weight, bias, stride, weight_compute=None, bias_compute=None, packs=None):
+    def forward(ctx, x, weight, bias, stride, weight_compute=None, bias_compute=None, packs=None, out_halo=0):
         wc = weight if weight_compute is None else weight_compute
         bc = bias if bias_compute is None else bias_compute
+        # `out_halo` (one sample): the result is written into the interior of a depth slab with that many zero planes on
+        # each face, which rides along as y._sfh_slab for a following FastConv3d.shard_halo
+        out = slab = None
+        if out_halo > 0 and x.shape[0] == 1 and x.numel() > 0:
+            d, h, w_ = (int(x.shape[2 + i]) * int(stride[i]) for i in range(3))
+            slab = torch.empty((1, wc.shape[1], d + 2 * out_halo, h, w_), dtype=x.dtype, device=x.device, memory_format=_CL3D)
+            if out_halo == 1:
+                slab[:, :, ::d + 1].zero_()  # both face planes in one fill
+            else:
+                slab[:, :, :out_halo].zero_()
+                slab[:, :, out_halo + d:].zero_()
+            out = slab[:, :, out_halo:out_halo + d]
         # `packs`: kept packed forms of the kernel == stride convolution this op transposes; its data-gradient form is
         # what this forward reads, its forward form what the data gradient below reads
-        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad)
+        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad, out=out)
+        if slab is not None:
+            y._sfh_slab = (slab, out_halo)
         pf = None if packs is None else packs.fwd
         ctx.save_for_backward(x, wc) if pf is None else ctx.save_for_backward(x, wc, pf)
         ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype, weight.dtype is not wc.dtype)
@@ -198,7 +253,7 @@ class _ConvTranspose3dFn(torch.autograd.Function):
             else:
                 grad_w = _ct.conv_transpose3d_backward_weight(x, weight.shape, grad_output, stride, 0, 0, 1, 1)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None
 
 
 def _wants_grad(*tensors) -> bool:
@@ -224,7 +279,94 @@ class FastConv3d(nn.Conv3d):
             return None
         return shift
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def _pair_operands(self, x, second):
+        """The tensors the kernels would read for ``forward(x, second)`` and the padding they would run with, or ``None``
+        when the pair is not served as it stands: ``(x_read, second_read, padding, slab, slab2)``.  In the depth-shard
+        form both tensors must already lie in slabs with zero faces (their producers wrote them there)."""
+        if self.padding_mode != "zeros" or isinstance(self.padding, str) or self.groups != 1:
+            return None
+        if not isinstance(x, torch.Tensor) or not isinstance(second, torch.Tensor) or x.dtype is not second.dtype:
+            return None
+        dt = autocast_dtype(x)
+        if dt is not None and x.dtype is torch.float32:
+            return None  # the casts would make new tensors (outside the slabs); the caller concatenates instead
+        padding = tuple(self.padding)
+        slab = slab2 = None
+        if self.shard_halo and padding[0] > 0:
+            slab, slab2 = getattr(x, "_sfh_slab", None), getattr(second, "_sfh_slab", None)
+            if slab is None or slab2 is None or slab[1] != padding[0] or slab2[1] != padding[0]:
+                return None
+            if slab[0].dtype is not x.dtype or slab2[0].dtype is not x.dtype:
+                return None
+            x_read, second_read = slab[0], slab2[0]
+            padding = (0, padding[1], padding[2])
+        else:
+            x_read, second_read = x, second
+        if not (x_read.is_contiguous(memory_format=_CL3D) and second_read.is_contiguous(memory_format=_CL3D)):
+            return None
+        return x_read, second_read, padding, slab, slab2
+
+    def takes_pair(self, x, second) -> bool:
+        """Whether ``forward(x, second)`` is served: the convolution of ``torch.cat([x, second], 1)`` read from the two
+        tensors themselves, all three directions.  Total: never raises."""
+        try:
+            ops = self._pair_operands(x, second)
+            return ops is not None and self._pair_gate(ops[0], ops[1], ops[2])
+        except (TypeError, ValueError, AttributeError, RuntimeError):
+            return False
+
+    def _pair_gate(self, x_read, second_read, padding) -> bool:
+        """The library's answer for the tensors the kernels would read, remembered per shape (the parameters' shapes and
+        the module's geometry do not change; their dtypes under autocast are the activations')."""
+        key = (x_read.shape, second_read.shape, x_read.dtype, x_read.device, padding, self.bias is None)
+        table = self.__dict__.get("_pair_ok")
+        if table is None:
+            table = self.__dict__["_pair_ok"] = {}
+        ok = table.get(key)
+        if ok is None:
+            # stand-ins with the dtype the kernel's operands will have (metadata only)
+            w = self.weight if self.weight.dtype is x_read.dtype else self.weight.new_empty((1, 1, 1, 1, 1), dtype=x_read.dtype).expand(
+                self.weight.shape)
+            b = None
+            if self.bias is not None:
+                b = self.bias if self.bias.dtype is x_read.dtype else torch.empty(self.bias.shape, dtype=x_read.dtype, device=x_read.device)
+            ok = _c3.is_supported_pair(x_read, second_read, w, b, tuple(self.stride), padding, tuple(self.dilation))
+            if len(table) > 64:
+                table.clear()
+            table[key] = ok
+        return ok
+
+    def _forward_pair(self, x, second):
+        ops = self._pair_operands(x, second)
+        if ops is None:
+            raise NotImplementedError(f"FastConv3d: the pair x={tuple(x.shape)}/{x.dtype}, second={tuple(second.shape)}/{second.dtype} "
+                                      "is not served as it stands (see takes_pair); concatenate instead")
+        x_read, second_read, padding, slab, slab2 = ops
+        dt = autocast_dtype(x)
+        wc = compute_copy(self.weight, dt)
+        bc = compute_copy(self.bias, dt) if wc is not None else None
+        master = wc is not None and (self.bias is None or bc is not None)
+        w = wc if master else cast_operand(self.weight, dt)
+        b = bc if master else cast_operand(self.bias, dt)
+        stride, dilation = tuple(self.stride), tuple(self.dilation)
+        if w.dtype is not x_read.dtype or not self._pair_gate(x_read, second_read, padding):
+            raise NotImplementedError(
+                f"FastConv3d: pair not served: x={tuple(x_read.shape)}/{x_read.dtype} second={tuple(second_read.shape)} on {x.device}, "
+                f"weight={tuple(w.shape)}/{w.dtype}, stride={stride} padding={padding} dilation={dilation}")
+        in_shape = torch.Size((x_read.shape[0], x_read.shape[1] + second_read.shape[1], *x_read.shape[2:]))
+        if master:
+            return _Conv3dFn.apply(x, self.weight, self.bias, stride, padding, dilation, w, b,
+                                   _current_packs(self.weight, w, in_shape, stride, padding, dilation), slab, self.gn_groups,
+                                   self._gn_shift(), second, slab2)
+        packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is self.weight else None
+        return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, self._gn_shift(), second,
+                               slab2)
+
+    def forward(self, x: torch.Tensor, second: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``second``: the input is ``torch.cat([x, second], 1)``, read from the two tensors themselves (the decoder's skip
+        connection and upsampled tensor, ``ScaFFold/unet/unet_parts.py:107-120``); ask :meth:`takes_pair` first."""
+        if second is not None:
+            return self._forward_pair(x, second)
         if self.padding_mode != "zeros" or isinstance(self.padding, str):
             raise NotImplementedError(f"FastConv3d: padding_mode={self.padding_mode!r} padding={self.padding!r}")
         dt = autocast_dtype(x)
@@ -272,6 +414,9 @@ class FastConv3d(nn.Conv3d):
 class FastConvTranspose3d(nn.ConvTranspose3d):
     """``nn.ConvTranspose3d`` at ``kernel == stride`` served by the HIP kernels."""
 
+    #: depth planes of zero halo to leave around the output for a following ``FastConv3d.shard_halo`` (0: none)
+    out_halo = 0
+
     def forward(self, x: torch.Tensor, output_size=None) -> torch.Tensor:
         if output_size is not None:
             raise NotImplementedError("FastConvTranspose3d: output_size is not supported")
@@ -299,9 +444,9 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
             if packs is not None and (packs.fwd is None or packs.dgrad is None):
                 packs = None
             if master:
-                return _ConvTranspose3dFn.apply(x, self.weight, self.bias, stride, w, b, packs)
-            return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, packs)
-        return _ConvTranspose3dFn.apply(x, w, b, stride)
+                return _ConvTranspose3dFn.apply(x, self.weight, self.bias, stride, w, b, packs, self.out_halo)
+            return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, packs, self.out_halo)
+        return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, None, self.out_halo)
 
 
 class FastGroupNorm(nn.GroupNorm):

@@ -101,7 +101,11 @@ def max_pool3d_2x_with_skip(x: torch.Tensor):
         raise NotImplementedError(f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)}")
     if not x.is_contiguous(memory_format=_CL3D):
         return _MaxPool2Fn.apply(x), x
-    return _MaxPool2SkipFn.apply(x)
+    pooled, skip = _MaxPool2SkipFn.apply(x)
+    slab = getattr(x, "_sfh_slab", None)
+    if slab is not None:  # the alias is the same memory: still the interior of the slab its producer wrote it into
+        skip._sfh_slab = slab
+    return pooled, skip
 
 
 def max_pool3d_2x(x: torch.Tensor) -> torch.Tensor:

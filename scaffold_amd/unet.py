@@ -101,13 +101,16 @@ class DoubleConv(nn.Module):
         for c, g in self._pairs:
             self.double_conv[c].gn_groups = self.double_conv[g].num_groups
 
-    def forward(self, x):
+    def forward(self, x, second=None):
+        """``second``: the input is ``torch.cat([x, second], 1)``, handed over as the two tensors (the first convolution
+        must have said ``takes_pair``)."""
         if not self._pairs:
-            return self.double_conv(x)
+            return self.double_conv(x if second is None else torch.cat([x, second], dim=1))
         for c, g in self._pairs:  # the Identity modules between the pairs only keep the reference's state-dict indices
             conv, norm = self.double_conv[c], self.double_conv[g]
             conv.gn_shift = getattr(norm, "_next_shift", None)  # what the norm's last call said to sum about
-            x = norm(conv(x))
+            x = norm(conv(x) if second is None else conv(x, second))
+            second = None
         return x
 
 
@@ -121,6 +124,9 @@ class Down(nn.Module):
 
 
 class Up(nn.Module):
+    #: let the first convolution read [skip, upsampled] as two tensors where it serves them (False: always concatenate)
+    read_skip_in_place = True
+
     def __init__(self, in_channels, out_channels, group_norm_groups, stock=False):
         super().__init__()
         self.up = _conv_transpose3d(stock, in_channels, in_channels // 2, kernel_size=2, stride=2)
@@ -132,6 +138,12 @@ class Up(nn.Module):
         if dx or dy or dz:
             x1 = F.pad(x1, [dx // 2, dx - dx // 2, dy // 2, dy - dy // 2, dz // 2, dz - dz // 2])
         first = self.conv.double_conv[0]
+        if self.read_skip_in_place and isinstance(first, FastConv3d):
+            # the convolution reads the skip connection and the upsampled tensor where they lie: nothing is concatenated
+            dtype = _consumer_dtype(x2, x1)
+            skip, up = (x2 if x2.dtype is dtype else x2.to(dtype)), (x1 if x1.dtype is dtype else x1.to(dtype))
+            if first.takes_pair(skip, up):
+                return self.conv(skip, up)
         halo = int(first.padding[0]) if getattr(first, "shard_halo", False) else 0
         return self.conv(skip_concat(x2, x1, halo))
 
@@ -180,6 +192,19 @@ class UNet(nn.Module):
                 norm, conv = m.double_conv[1], m.double_conv[3]
                 if isinstance(norm, FastGroupNorm) and isinstance(conv, FastConv3d):
                     norm.out_halo = int(conv.padding[0]) if enabled else 0
+        # The decoder's first convolutions read the skip connection and the upsampled tensor as they lie: their
+        # producers (the encoder blocks' last GroupNorm, the up-convolutions) write them into slabs as well.
+        for i, up in enumerate(self.up_list[:-1]):
+            first = up.conv.double_conv[0]
+            if not isinstance(first, FastConv3d):
+                continue
+            halo = int(first.padding[0]) if enabled else 0
+            if isinstance(up.up, FastConvTranspose3d):
+                up.up.out_halo = halo
+            enc = self.down_list[self.layers - 1 - i]
+            block = enc if isinstance(enc, DoubleConv) else enc.maxpool_conv[1]
+            if isinstance(block.double_conv[4], FastGroupNorm):
+                block.double_conv[4].out_halo = halo
         return self
 
     def _run(self, block, *inputs):

@@ -447,6 +447,44 @@ def test_shard_form_gradients_equal_the_padded_form(device, batch, size, checkpo
     assert all(torch.equal(p, q) for p, q in zip(a, b))
 
 
+@pytest.mark.parametrize("layers,base,size,shard,batch", [
+    (3, 32, (16, 32, 64), False, 1),   # brick forward at every level, persist / brick data gradients, the deepest level sliced
+    (3, 32, (16, 32, 64), True, 1),    # the same on a depth shard: every source lies in a slab its producer wrote
+    (2, 32, (8, 12, 24), False, 2),    # a batch
+    (2, 32, (8, 12, 24), True, 2),     # a batch on a shard: no slabs, so the decoder concatenates into one
+    (1, 64, (32, 64, 64), True, 1),    # 128 -> 64 at 32 x 64 x 64: the wide-tile forward reads the pair
+])
+def test_decoder_reading_the_skip_in_place_changes_no_bits(device, monkeypatch, layers, base, size, shard, batch):
+    """The decoder's first convolution reads [skip, upsampled] as two tensors instead of their concatenation
+    (``unet_parts.py:107-120``): loss and every parameter gradient are the bits of the concatenating form."""
+    from scaffold_amd import conv3d as c3
+    from scaffold_amd.unet import Up
+
+    torch.manual_seed(21)
+    model = UNet(1, 5, layers=layers, base_width=base).to(device).to(memory_format=CL).set_shard_halo(shard)
+    g0 = torch.Generator().manual_seed(22)
+    x = (torch.rand((batch, 1, *size), generator=g0) < 0.1).float().contiguous(memory_format=CL).to(device)
+    lab = torch.randint(0, 5, (batch, *size), generator=g0).to(device)
+    calls = []
+    real = c3.conv3d_forward_pair
+    monkeypatch.setattr(c3, "conv3d_forward_pair", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+
+    def grads(in_place):
+        monkeypatch.setattr(Up, "read_skip_in_place", in_place)
+        model.zero_grad(set_to_none=True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(x)
+        loss = sa.ce_dice_loss(logits, lab)
+        loss.backward()
+        return [loss.detach().clone(), logits.detach().clone()] + [p.grad.clone() for p in model.parameters()]
+
+    want = grads(False)
+    assert not calls
+    got = grads(True)
+    assert len(calls) == (0 if (shard and batch > 1) else layers)
+    assert all(torch.equal(p, q) for p, q in zip(want, got))
+
+
 def test_from_shard_files_to_updated_weights(device, tmp_path):
     """The whole path on one rank's share: a volume / mask pair as the generator writes it (float32 (3, d, h, w) + uint16),
     read and ingested into the stem's slab, the 3-channel U-Net in shard form under bf16 autocast, the fused loss head and
