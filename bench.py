@@ -547,6 +547,13 @@ def conv_table(device, iters=20):
                 "dgrad": lambda: sa.conv3d_backward_data(gy, w, x.shape, 1, pad, 1, out=gx, packed_weight=pd),
                 "wgrad": lambda: sa.conv3d_backward_weight(x, w.shape, gy, 1, pad, 1, out=gw, grad_dtype=torch.float32),
             }
+            from scaffold_amd import conv3d as c3
+            first, second = x[:, :cin // 2].contiguous(memory_format=CL), x[:, cin // 2:].contiguous(memory_format=CL)
+            if cin == 2 * cout and c3.is_supported_pair(first, second, w, None, 1, pad, 1):
+                # a decoder shape: the same launches reading [skip, upsampled] as the two tensors they are ("2t" rows)
+                fns["fwd2t"] = lambda: c3.conv3d_forward_pair(first, second, w, None, 1, pad, 1, packed_weight=pf)
+                fns["dgr2t"] = lambda: c3.conv3d_backward_data_pair(gy, w, x.shape, cin // 2, 1, pad, 1, packed_weight=pd)
+                fns["wgr2t"] = lambda: c3.conv3d_backward_weight_pair(first, second, w.shape, gy, 1, pad, 1, grad_dtype=torch.float32)
             for direction, fn in fns.items():
                 fn()
                 torch.cuda.synchronize()
@@ -558,14 +565,15 @@ def conv_table(device, iters=20):
                 ms = event_time_ms(graph.replay, max(2, iters // chunk), warmup=1) / chunk
                 rows.append({"form": form, "cin": cin, "cout": cout, "spatial": list(sp), "direction": direction, "us": ms * 1e3,
                              "gflop": flops / 1e9, "tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS})
-            del x, w, gy, y, gx, gw, pf, pd
+            del x, w, gy, y, gx, gw, pf, pd, first, second
     return rows
 
 
 def conv_counter_launches(device, reps=3):
     """The launches a counter run (rocprofv3 --pmc) is taken over: plain eager calls, no graph, of the three MFMA
     convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_persist_kernel,
-    wgrad_mfma_kernel), 128->64 @64^3 and 64->32 on the 64x128x128 slab (conv_mfma_kernel, wgrad_mfma_kernel)."""
+    wgrad_mfma_kernel), 128->64 @64^3 and 64->32 on the 64x128x128 slab (conv_mfma_kernel, wgrad_mfma_kernel), the last
+    also with its input as two 32-channel tensors (what the U-Net's decoder hands it)."""
     import scaffold_amd as sa
 
     done = []
@@ -586,6 +594,17 @@ def conv_counter_launches(device, reps=3):
         torch.cuda.synchronize()
         done.append({"cin": cin, "cout": cout, "output_spatial": list(sp), "launches_per_direction": reps,
                      "flops_per_launch": 2 * math.prod(sp) * cin * cout * 27})
+        if pad[0] == 0 and cin == 2 * cout:
+            # the decoder's first convolution as the step runs it: the input as the two tensors it would be concatenated from
+            from scaffold_amd import conv3d as c3
+            first, second = x[:, :cin // 2].contiguous(memory_format=CL), x[:, cin // 2:].contiguous(memory_format=CL)
+            for _ in range(reps):
+                c3.conv3d_forward_pair(first, second, w, None, 1, pad, 1, packed_weight=pf)
+                c3.conv3d_backward_data_pair(gy, w, x.shape, cin // 2, 1, pad, 1, packed_weight=pd)
+                c3.conv3d_backward_weight_pair(first, second, w.shape, gy, 1, pad, 1, grad_dtype=torch.float32)
+            torch.cuda.synchronize()
+            done.append({"cin": cin, "cout": cout, "output_spatial": list(sp), "launches_per_direction": reps, "input": "two tensors",
+                         "flops_per_launch": 2 * math.prod(sp) * cin * cout * 27})
     return done
 
 
