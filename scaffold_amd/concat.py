@@ -55,7 +55,7 @@ class _SkipConcatFn(torch.autograd.Function):
         ctx.cat_args = (n, ca, cb, d, h, w)
         if halo == 0:
             return slab
-        out = slab[:, :, halo:halo + d]
+        out = slab.narrow(2, halo, d)
         out._sfh_slab = (slab, halo)
         return out
 

@@ -143,7 +143,7 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, o
     if out_halo > 0 and n == 1 and odt.itemsize == input.dtype.itemsize and input.numel() > 0:
         c, d, h, w = (int(v) for v in input.shape[1:])
         slab = torch.empty((1, c, d + 2 * out_halo, h, w), dtype=odt, device=input.device, memory_format=_CL3D)
-        out = slab[:, :, out_halo:out_halo + d]
+        out = slab.narrow(2, out_halo, d)
         out._sfh_slab = (slab, out_halo)
     else:
         out = torch.empty_like(input, dtype=odt)  # keeps the channels_last_3d strides

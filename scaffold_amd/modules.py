@@ -170,7 +170,7 @@ class _Conv3dFn(torch.autograd.Function):
         grad_x = _c3.conv3d_backward_data(grad_output, weight, x.shape, stride, padding, dilation, 1,
                                           packed_weight=packed[0] if packed else None, _checked=True) if needs_x else None
         if ctx.halo and grad_x is not None:
-            grad_x = grad_x[:, :, ctx.halo:ctx.halo + ctx.depth]
+            grad_x = grad_x.narrow(2, ctx.halo, ctx.depth)
         grad_w = None
         if needs_w:
             if master:
@@ -196,8 +196,8 @@ class _Conv3dFn(torch.autograd.Function):
             grad_x, grad_second = _c3.conv3d_backward_data_pair(grad_output, weight, in_shape, int(x.shape[1]), stride, padding,
                                                                 dilation, packed_weight=packed[0] if packed else None, _checked=True)
             if ctx.halo:  # both tensors are slabs of the same depth: the interiors are the inputs' gradients
-                grad_x = grad_x[:, :, ctx.halo:ctx.halo + ctx.depth]
-                grad_second = grad_second[:, :, ctx.halo:ctx.halo + ctx.depth]
+                grad_x = grad_x.narrow(2, ctx.halo, ctx.depth)
+                grad_second = grad_second.narrow(2, ctx.halo, ctx.depth)
         grad_w = None
         if needs_w:
             if master:
@@ -226,7 +226,7 @@ class _ConvTranspose3dFn(torch.autograd.Function):
             else:
                 slab[:, :, :out_halo].zero_()
                 slab[:, :, out_halo + d:].zero_()
-            out = slab[:, :, out_halo:out_halo + d]
+            out = slab.narrow(2, out_halo, d)
         # `packs`: kept packed forms of the kernel == stride convolution this op transposes; its data-gradient form is
         # what this forward reads, its forward form what the data gradient below reads
         y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad, out=out)
@@ -290,6 +290,8 @@ class FastConv3d(nn.Conv3d):
         dt = autocast_dtype(x)
         if dt is not None and x.dtype is torch.float32:
             return None  # the casts would make new tensors (outside the slabs); the caller concatenates instead
+        if (dt if (dt is not None and self.weight.dtype is torch.float32) else self.weight.dtype) is not x.dtype:
+            return None  # the weight the kernel would read (autocast narrows an fp32 parameter) is of another dtype
         padding = tuple(self.padding)
         slab = slab2 = None
         if self.shard_halo and padding[0] > 0:

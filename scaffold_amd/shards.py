@@ -180,7 +180,7 @@ def ingest(volume: torch.Tensor, mask: Optional[torch.Tensor] = None, *, dtype: 
     _lib.check(rc, "shard ingest")
     if halo == 0:
         return slab, labels
-    x = slab[:, :, halo:halo + d]
+    x = slab.narrow(2, halo, d)
     x._sfh_slab = (slab, halo)
     return x, labels
 

@@ -485,6 +485,59 @@ def test_decoder_reading_the_skip_in_place_changes_no_bits(device, monkeypatch, 
     assert all(torch.equal(p, q) for p, q in zip(want, got))
 
 
+def test_up_convolution_into_a_depth_slab_is_bitwise_the_plain_output(device):
+    """``FastConvTranspose3d.out_halo``: the result lies in the interior of a slab with zero faces and is otherwise the
+    plain result, values and gradients."""
+    torch.manual_seed(31)
+    x0 = torch.randn(1, 64, 3, 5, 9, device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    gy = torch.randn(1, 32, 6, 10, 18, device=device).to(torch.bfloat16).contiguous(memory_format=CL)
+    results = []
+    for halo in (0, 1, 2):
+        torch.manual_seed(32)
+        up = FastConvTranspose3d(64, 32, kernel_size=2, stride=2).to(device).to(torch.bfloat16)
+        up.out_halo = halo
+        x = x0.clone().requires_grad_(True)
+        y = up(x)
+        assert hasattr(y, "_sfh_slab") == bool(halo) and y.is_contiguous(memory_format=CL)
+        if halo:
+            slab, h = y._sfh_slab
+            assert h == halo and slab.shape == (1, 32, 6 + 2 * halo, 10, 18) and slab.data_ptr() < y.data_ptr()
+            assert torch.equal(slab[:, :, halo:halo + 6], y)
+            assert not slab[:, :, :halo].any() and not slab[:, :, halo + 6:].any()
+        y.backward(gy)
+        results.append((y.detach().clone(), x.grad, up.weight.grad, up.bias.grad))
+    for other in results[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(results[0], other))
+
+
+def test_where_the_decoder_still_concatenates(device):
+    """``FastConv3d.takes_pair`` says no -- and ``Up`` concatenates, with the concatenating form's result -- for fp32
+    operands, a cut off the 32-channel grid, tensors outside their slabs on a depth shard, and other voxels."""
+    from scaffold_amd.unet import Up
+
+    torch.manual_seed(41)
+    conv = FastConv3d(64, 32, 3, padding=1, bias=False).to(device).to(memory_format=CL)
+    mk = lambda c, dtype=torch.bfloat16, sp=(4, 8, 32): torch.randn(1, c, *sp, device=device).to(dtype).contiguous(memory_format=CL)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert conv.takes_pair(mk(32), mk(32))
+        assert not conv.takes_pair(mk(32, torch.float32), mk(32, torch.float32))  # autocast would cast: new tensors
+        assert not conv.takes_pair(mk(32), mk(32, torch.float32))
+        assert not conv.takes_pair(mk(16), mk(48))
+        assert not conv.takes_pair(mk(32), mk(32, sp=(4, 8, 16)))
+        assert not conv.takes_pair(mk(32), None)
+        conv.shard_halo = True
+        assert not conv.takes_pair(mk(32), mk(32))  # no producer wrote them into slabs
+        with pytest.raises(NotImplementedError):
+            conv(mk(32), mk(32))
+        conv.shard_halo = False
+    assert not conv.takes_pair(mk(32), mk(32))  # outside autocast the fp32 weight does not match bf16 tensors
+    # Up with fp32 tensors: the concatenating form, same result as torch.cat by hand
+    up = Up(64, 32, 8).to(device).to(memory_format=CL)
+    x1 = torch.randn(1, 64, 4, 4, 8, device=device).contiguous(memory_format=CL)
+    x2 = torch.randn(1, 32, 8, 8, 16, device=device).contiguous(memory_format=CL)
+    assert torch.equal(up(x1, x2), up.conv(torch.cat([x2, up.up(x1)], dim=1)))
+
+
 def test_from_shard_files_to_updated_weights(device, tmp_path):
     """The whole path on one rank's share: a volume / mask pair as the generator writes it (float32 (3, d, h, w) + uint16),
     read and ingested into the stem's slab, the 3-channel U-Net in shard form under bf16 autocast, the fused loss head and
