@@ -75,7 +75,8 @@ typedef struct sfh_groupnorm_desc {
 /* ---- library ------------------------------------------------------------------------ */
 /* 100: the first published set of entry points. 101: sfh_conv3d_launch_geometry, sfh_conv3d_fwd_gn_records,
  * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed.
- * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair added. */
+ * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair,
+ * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab added. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -244,6 +245,14 @@ size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int dtype);
 int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w,
                     const int64_t w_stride[5], const void* bias, void* y, void* workspace,
                     size_t workspace_bytes, uint32_t flags, void* stream);
+/* The same with y written into the interior of a depth slab: y_slab holds halo_elems elements of face, the result, and
+ * halo_elems elements of face again; the launch zeroes both faces. One sample, the 2x2x2 matrix-core kernel only
+ * (16-bit dtypes, channel counts multiples of 32), faces and tensor multiples of 16 bytes: SFH_ERR_UNSUPPORTED otherwise.
+ * With halo_elems = 0 it is sfh_convT3d_fwd. The decoder's up-convolution feeds a convolution whose halo exchange
+ * (ScaFFold/unet/conv3d.py:769-776) assembles exactly this buffer; here its producer writes it in place. */
+int sfh_convT3d_fwd_slab(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w,
+                         const int64_t w_stride[5], const void* bias, void* y_slab, int64_t halo_elems,
+                         void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
 /* ---- GroupNorm forward ---------------------------------------------------------------
  * Stands in for torch.ops.scaffold_gn.group_norm (ScaFFold/unet/triton_group_norm.py:1339)
@@ -337,6 +346,12 @@ typedef struct sfh_pool_desc {
 } sfh_pool_desc;
 int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x, void* y, uint8_t* idx,
                      void* stream);
+/* The same with y written into the interior of a depth slab: y_slab holds halo_elems elements of face, the pooled
+ * tensor, and halo_elems elements of face again; the launch zeroes both faces (one sample; faces and tensor multiples of
+ * 16 bytes, else SFH_ERR_UNSUPPORTED). It is the [recv_minus | x | recv_plus] buffer of the halo exchange
+ * (ScaFFold/unet/conv3d.py:769-776) for the convolution that follows the pooling, produced without a copy. */
+int sfh_maxpool2_fwd_slab(const sfh_pool_desc* p, int dtype, const void* x, void* y_slab, int64_t halo_elems,
+                          uint8_t* idx, void* stream);
 int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx,
                      void* grad_x, void* stream);
 /* grad_x = (the pooling gradient) + add, summed in fp32 and rounded once; `add` has the input's

@@ -135,6 +135,8 @@ _SIGNATURES = {
     "sfh_convT3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvTDesc), c_int]),
     "sfh_convT3d_fwd": (c_int, [POINTER(ConvTDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                 c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_convT3d_fwd_slab": (c_int, [POINTER(ConvTDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_int64,
+                                     c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_groupnorm_fwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
     "sfh_groupnorm_fwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -158,6 +160,7 @@ _SIGNATURES = {
                                 c_void_p]),
     "sfh_ce_dice_bwd": (c_int, [POINTER(LossDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_fwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "sfh_maxpool2_fwd_slab": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "sfh_maxpool2_bwd": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_maxpool2_bwd_add": (c_int, [POINTER(PoolDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sfh_halo_assemble": (c_int, [POINTER(HaloDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),

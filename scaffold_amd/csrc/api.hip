@@ -752,6 +752,16 @@ extern "C" int sfh_maxpool2_fwd(const sfh_pool_desc* p, int dtype, const void* x
   return maxpool2_fwd(*p, dtype, x, y, idx, (hipStream_t)stream);
 }
 
+extern "C" int sfh_maxpool2_fwd_slab(const sfh_pool_desc* p, int dtype, const void* x, void* y_slab, int64_t halo_elems, uint8_t* idx,
+                                     void* stream) {
+  if (int rc = check_pool(p, dtype, "maxpool fwd")) return rc;
+  if (halo_elems < 0) return fail(SFH_ERR_INVALID, "maxpool fwd: negative halo");
+  if (p->n == 0 || p->in_d < 2 || p->in_h < 2 || p->in_w < 2) return fail(SFH_ERR_UNSUPPORTED, "maxpool fwd: no slab around an empty output");
+  if (x == nullptr || y_slab == nullptr || idx == nullptr) return fail(SFH_ERR_INVALID, "maxpool fwd: null tensor");
+  const size_t elem = dtype == SFH_FP32 ? 4 : 2;
+  return maxpool2_fwd(*p, dtype, x, static_cast<char*>(y_slab) + (size_t)halo_elems * elem, idx, (hipStream_t)stream, halo_elems);
+}
+
 extern "C" int sfh_maxpool2_bwd(const sfh_pool_desc* p, int dtype, const void* grad_y, const uint8_t* idx, void* grad_x,
                                 void* stream) {
   if (int rc = check_pool(p, dtype, "maxpool bwd")) return rc;
@@ -787,8 +797,9 @@ extern "C" size_t sfh_convT3d_fwd_workspace_bytes(const sfh_convT3d_desc* p, int
   return 0;
 }
 
-extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
-                               const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+static int convT3d_fwd_any(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                           const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream,
+                           int64_t halo_elems) {
   if (int rc = check_convT(p, dtype)) return rc;
   if (x == nullptr || w == nullptr || y == nullptr || (w_stride == nullptr && !(flags & SFH_FLAG_WEIGHT_PACKED)))
     return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
@@ -797,7 +808,7 @@ extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void*
     // w is the packed form: the data-gradient packing of the kernel == stride convolution this one transposes
     if ((flags & SFH_FLAG_FORCE_GENERIC) || !convT_uses_patch(*p, dtype))
       return fail(SFH_ERR_INVALID, "convT3d fwd: this problem does not read a packed weight");
-    return patch_scatter(convT_patch_args(*p), dtype, x, w, bias, y, (hipStream_t)stream);
+    return patch_scatter(convT_patch_args(*p), dtype, x, w, bias, y, (hipStream_t)stream, halo_elems);
   }
   if (!(flags & SFH_FLAG_FORCE_GENERIC) && convT_uses_patch(*p, dtype)) {
     // produced channel = Cout (w_stride[1]), reduced channel = Cin (w_stride[0])
@@ -808,9 +819,26 @@ extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void*
     hipStream_t st = (hipStream_t)stream;
     if (int rc = mfma_pack_weight(pk, dtype, w, w_stride[1], w_stride[0], w_stride[2], w_stride[3], w_stride[4], 0, workspace, st))
       return rc;
-    return patch_scatter(convT_patch_args(*p), dtype, x, workspace, bias, y, st);
+    return patch_scatter(convT_patch_args(*p), dtype, x, workspace, bias, y, st, halo_elems);
   }
+  if (halo_elems > 0) return fail(SFH_ERR_UNSUPPORTED, "convT3d fwd: only the 2x2x2 matrix-core kernel writes into a slab");
   return direct_convT(*p, dtype, w_stride, x, w, bias, y, (hipStream_t)stream);
+}
+
+extern "C" int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                               const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  return convT3d_fwd_any(p, dtype, x, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, 0);
+}
+
+extern "C" int sfh_convT3d_fwd_slab(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
+                                    const void* bias, void* y_slab, int64_t halo_elems, void* workspace, size_t workspace_bytes,
+                                    uint32_t flags, void* stream) {
+  if (halo_elems < 0) return fail(SFH_ERR_INVALID, "convT3d fwd: negative halo");
+  if (y_slab == nullptr) return fail(SFH_ERR_INVALID, "convT3d fwd: null tensor");
+  if (p != nullptr && p->n == 0) return fail(SFH_ERR_UNSUPPORTED, "convT3d fwd: no slab around an empty output");
+  const size_t elem = dtype == SFH_FP32 ? 4 : 2;
+  return convT3d_fwd_any(p, dtype, x, w, w_stride, bias, static_cast<char*>(y_slab) + (size_t)halo_elems * elem, workspace, workspace_bytes,
+                         flags, stream, halo_elems);
 }
 
 // ---- loss head -------------------------------------------------------------------------

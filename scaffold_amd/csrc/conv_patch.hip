@@ -149,9 +149,22 @@ __global__ void __launch_bounds__(256) patch_gather_deep_kernel(PatchArgs a, con
 // grid = (voxel tiles of 128, cbig / 32, 8 / TS). TS = 8 reads the small tensor once; TS = 1 and 2 are for launches that
 // would otherwise leave most of the chip idle or give a CU a single long chain of dependent loads (the deeper levels):
 // more workgroups, each with a shorter chain, and the loads of several k-steps in flight per lane.
+// `face_pieces` > 0: `big` is the interior of a depth slab whose two faces of that many 16-byte pieces (in front of it and
+// behind its `big_elems` elements) the launch zeroes as well, spread over all its threads.
 template <typename T, int TS>
 __global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T* __restrict__ small, const T* __restrict__ packed,
-                                                            const T* __restrict__ bias, T* __restrict__ big, int64_t total) {
+                                                            const T* __restrict__ bias, T* __restrict__ big, int64_t total,
+                                                            int64_t face_pieces, int64_t big_elems) {
+  if (face_pieces > 0) {
+    const int64_t nthreads = (int64_t)gridDim.x * gridDim.y * gridDim.z * 256;
+    const int64_t me = (((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 256 + threadIdx.x;
+    uint4* lo = reinterpret_cast<uint4*>(big) - face_pieces;
+    uint4* hi = reinterpret_cast<uint4*>(big + big_elems);
+    for (int64_t p = me; p < face_pieces; p += nthreads) {
+      lo[p] = make_uint4(0, 0, 0, 0);
+      hi[p] = make_uint4(0, 0, 0, 0);
+    }
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kg = lane >> 5;
   const int64_t v = (int64_t)blockIdx.x * 128 + wave * 32 + (lane & 31);
@@ -317,8 +330,14 @@ int launch_gather(const PatchArgs& a, const void* big, const void* packed, const
 }
 
 template <typename T>
-int launch_scatter(const PatchArgs& a, const void* small, const void* packed, const void* bias, void* big, hipStream_t st) {
+int launch_scatter(const PatchArgs& a, const void* small, const void* packed, const void* bias, void* big, hipStream_t st,
+                   int64_t halo_elems) {
   const int64_t total = small_voxels(a);
+  const int64_t big_elems = (int64_t)a.n * a.bd * a.bh * a.bw * a.cbig;
+  if (halo_elems > 0 && (a.n != 1 || (reinterpret_cast<uintptr_t>(big) & 15) != 0 || (big_elems * (int64_t)sizeof(T)) % 16 != 0 ||
+                         (halo_elems * (int64_t)sizeof(T)) % 16 != 0))
+    return fail(SFH_ERR_UNSUPPORTED, "convT3d fwd: a slab output needs one sample and 16-byte aligned faces");
+  const int64_t face_pieces = halo_elems > 0 ? halo_elems * (int64_t)sizeof(T) / 16 : 0;
   dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
   const int64_t wgs = (int64_t)grid.x * grid.y;
   int force = 0;
@@ -327,18 +346,18 @@ int launch_scatter(const PatchArgs& a, const void* small, const void* packed, co
 #endif
   if (force == 8) {
     hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
-                       (const T*)bias, (T*)big, total);
+                       (const T*)bias, (T*)big, total, face_pieces, big_elems);
   } else if (force == 1 || (force == 0 && wgs < kComputeUnits)) {  // under one workgroup per CU: one tap per workgroup
     grid.z = kTaps;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
-                       (T*)big, total);
+                       (T*)big, total, face_pieces, big_elems);
   } else if (force == 2 || (force == 0 && wgs <= 4 * kComputeUnits)) {  // up to four per CU: two taps (the big voxels next to each other along W)
     grid.z = kTaps / 2;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
-                       (T*)big, total);
+                       (T*)big, total, face_pieces, big_elems);
   } else {
     hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
-                       (const T*)bias, (T*)big, total);
+                       (const T*)bias, (T*)big, total, face_pieces, big_elems);
   }
   return check_launch("patch_scatter_kernel");
 }
@@ -394,9 +413,10 @@ int patch_gather(const PatchArgs& a, int dtype, const void* big, const void* pac
   return launch_gather<fp16_t>(a, big, packed, bias, small, st);
 }
 
-int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_scatter<bf16_t>(a, small, packed, bias, big, st);
-  return launch_scatter<fp16_t>(a, small, packed, bias, big, st);
+int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st,
+                  int64_t halo_elems) {
+  if (dtype == SFH_BF16) return launch_scatter<bf16_t>(a, small, packed, bias, big, st, halo_elems);
+  return launch_scatter<fp16_t>(a, small, packed, bias, big, st, halo_elems);
 }
 
 int patch_reduce_splits(const PatchArgs& a) { return reduce_plan(a).splits; }

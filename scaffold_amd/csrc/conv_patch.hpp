@@ -21,7 +21,10 @@ bool patch_reduce_supported(const PatchArgs& a, int dtype);
 // `packed` holds the weight in MFMA fragment order [produced/32][reduced/32][tap][kstep][lane][8]
 // (mfma_pack_weight): produced = csmall for gather, cbig for scatter.
 int patch_gather(const PatchArgs& a, int dtype, const void* big, const void* packed, const void* bias, void* small, hipStream_t st);
-int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st);
+// `halo_elems` > 0 (one sample): big is the interior of a depth slab with that many elements of face on either side,
+// which the launch zeroes too.
+int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st,
+                  int64_t halo_elems = 0);
 int patch_reduce_splits(const PatchArgs& a);
 size_t patch_reduce_workspace_bytes(const PatchArgs& a);
 // g: dense [csmall][8][cbig] in the element type, from fp32 partial slices in ws summed in split order

@@ -30,10 +30,20 @@ template <typename T, int V> struct StN {
   }
 };
 
+// `face_pieces` > 0: y is the interior of a depth slab whose two faces of that many 16-byte pieces (in front of y and
+// behind its last element) the launch zeroes as well, spread over all its threads.
 template <typename T, int V>
 __global__ void __launch_bounds__(kBlock) maxpool2_fwd_kernel(PoolGeom g, int64_t total, const T* __restrict__ x, T* __restrict__ y,
-                                                              uint8_t* __restrict__ idx) {
+                                                              uint8_t* __restrict__ idx, int64_t face_pieces) {
   const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (face_pieces > 0) {
+    uint4* lo = reinterpret_cast<uint4*>(y) - face_pieces;
+    uint4* hi = reinterpret_cast<uint4*>(y + total * V);
+    for (int64_t p = i; p < face_pieces; p += (int64_t)gridDim.x * kBlock) {
+      lo[p] = make_uint4(0, 0, 0, 0);
+      hi[p] = make_uint4(0, 0, 0, 0);
+    }
+  }
   if (i >= total) return;
   const int64_t cv = i % g.cvec;
   int64_t v = i / g.cvec;
@@ -154,20 +164,24 @@ PoolGeom geom(const sfh_pool_desc& p, int vec) {
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 template <typename T>
-int fwd_typed(const sfh_pool_desc& p, const void* x, void* y, uint8_t* idx, hipStream_t st) {
+int fwd_typed(const sfh_pool_desc& p, const void* x, void* y, uint8_t* idx, int64_t halo_elems, hipStream_t st) {
   constexpr int V = VecOf<T>::N;
   const bool vec = p.c % V == 0 && aligned16(x) && aligned16(y) && (reinterpret_cast<uintptr_t>(idx) & 7) == 0;
   const PoolGeom g = geom(p, vec ? V : 1);
   const int64_t total = (int64_t)p.n * g.od * g.oh * g.ow * g.cvec;
+  const int64_t out_bytes = (int64_t)p.n * g.od * g.oh * g.ow * p.c * (int64_t)sizeof(T), halo_bytes = halo_elems * (int64_t)sizeof(T);
+  if (halo_elems > 0 && (p.n != 1 || total == 0 || !aligned16(y) || out_bytes % 16 != 0 || halo_bytes % 16 != 0))
+    return fail(SFH_ERR_UNSUPPORTED, "maxpool fwd: a slab output needs one sample and 16-byte aligned faces");
+  const int64_t face_pieces = halo_elems > 0 ? halo_bytes / 16 : 0;
   if (total == 0) return SFH_OK;
   const int64_t blocks = cdiv(total, kBlock);
   if (blocks > 0x7fffffff) return fail(SFH_ERR_UNSUPPORTED, "maxpool fwd: %lld workgroups exceed the grid limit", (long long)blocks);
   if (vec)
     hipLaunchKernelGGL((maxpool2_fwd_kernel<T, V>), dim3((unsigned)blocks), dim3(kBlock), 0, st, g, total, static_cast<const T*>(x),
-                       static_cast<T*>(y), idx);
+                       static_cast<T*>(y), idx, face_pieces);
   else
     hipLaunchKernelGGL((maxpool2_fwd_kernel<T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, st, g, total, static_cast<const T*>(x),
-                       static_cast<T*>(y), idx);
+                       static_cast<T*>(y), idx, face_pieces);
   return check_launch("maxpool2_fwd_kernel");
 }
 
@@ -192,10 +206,10 @@ int bwd_typed(const sfh_pool_desc& p, const void* gy, const uint8_t* idx, const 
 
 }  // namespace
 
-int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st) {
-  if (dtype == SFH_BF16) return fwd_typed<bf16_t>(p, x, y, idx, st);
-  if (dtype == SFH_FP16) return fwd_typed<fp16_t>(p, x, y, idx, st);
-  return fwd_typed<float>(p, x, y, idx, st);
+int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st, int64_t halo_elems) {
+  if (dtype == SFH_BF16) return fwd_typed<bf16_t>(p, x, y, idx, halo_elems, st);
+  if (dtype == SFH_FP16) return fwd_typed<fp16_t>(p, x, y, idx, halo_elems, st);
+  return fwd_typed<float>(p, x, y, idx, halo_elems, st);
 }
 
 int maxpool2_bwd(const sfh_pool_desc& p, int dtype, const void* gy, const uint8_t* idx, const void* add, void* gx, hipStream_t st) {

@@ -6,7 +6,9 @@ namespace sfh {
 
 // y[n][od][oh][ow][c] = max over the 2x2x2 cell; idx holds, per output element, which of the cell's eight voxels
 // (kd * 4 + kh * 2 + kw) supplied it. Odd trailing planes, rows and columns are dropped.
-int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st);
+// `halo_elems` > 0 (one sample): y is the interior of a depth slab with that many elements of face on either side,
+// which the launch zeroes too.
+int maxpool2_fwd(const sfh_pool_desc& p, int dtype, const void* x, void* y, uint8_t* idx, hipStream_t st, int64_t halo_elems = 0);
 
 // gx = gy routed to the voxel idx names, zero elsewhere (including dropped odd planes). Writes all of gx.
 // gx = the pooling gradient (+ `add`, a tensor of the input's shape, when given)

@@ -217,21 +217,10 @@ class _ConvTranspose3dFn(torch.autograd.Function):
         bc = bias if bias_compute is None else bias_compute
         # `out_halo` (one sample): the result is written into the interior of a depth slab with that many zero planes on
         # each face, which rides along as y._sfh_slab for a following FastConv3d.shard_halo
-        out = slab = None
-        if out_halo > 0 and x.shape[0] == 1 and x.numel() > 0:
-            d, h, w_ = (int(x.shape[2 + i]) * int(stride[i]) for i in range(3))
-            slab = torch.empty((1, wc.shape[1], d + 2 * out_halo, h, w_), dtype=x.dtype, device=x.device, memory_format=_CL3D)
-            if out_halo == 1:
-                slab[:, :, ::d + 1].zero_()  # both face planes in one fill
-            else:
-                slab[:, :, :out_halo].zero_()
-                slab[:, :, out_halo + d:].zero_()
-            out = slab.narrow(2, out_halo, d)
         # `packs`: kept packed forms of the kernel == stride convolution this op transposes; its data-gradient form is
         # what this forward reads, its forward form what the data gradient below reads
-        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad, out=out)
-        if slab is not None:
-            y._sfh_slab = (slab, out_halo)
+        y = _ct.conv_transpose3d_forward(x, wc, bc, stride, 0, 0, 1, 1, packed_weight=None if packs is None else packs.dgrad,
+                                         out_halo=out_halo)
         pf = None if packs is None else packs.fwd
         ctx.save_for_backward(x, wc) if pf is None else ctx.save_for_backward(x, wc, pf)
         ctx.conv_args = (stride, bias is not None, None if bias is None else bias.dtype, weight.dtype is not wc.dtype)

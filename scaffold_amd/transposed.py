@@ -171,10 +171,14 @@ def conv_transpose3d_forward(
     out: Optional[torch.Tensor] = None,
     force_generic: bool = False,
     packed_weight: Optional[torch.Tensor] = None,
+    out_halo: int = 0,
 ) -> torch.Tensor:
     """Transposed 3-D convolution at ``kernel == stride``; NDHWC in and out; the bias is per
     output channel (not per tap column).  ``packed_weight``: the data-gradient form from
-    ``pack_weights(w, output_shape, stride=kernel, padding=0)`` -- this op is the data gradient of that convolution."""
+    ``pack_weights(w, output_shape, stride=kernel, padding=0)`` -- this op is the data gradient of that convolution.
+    ``out_halo=h`` (one sample, the 2x2x2 matrix-core problems): the result is the interior view of a slab with ``h`` zero
+    depth planes on each face, carried as ``result._sfh_slab = (slab, h)`` for a following ``FastConv3d.shard_halo``; the
+    launch zeroes the faces itself.  Where the kernel does not offer it the result is the plain tensor."""
     if not is_supported_transposed(x, w, bias, stride, padding, output_padding, dilation, groups):
         raise NotImplementedError(
             f"unsupported: x={tuple(getattr(x, 'shape', ()))}/{getattr(x, 'dtype', None)} w={tuple(getattr(w, 'shape', ()))} "
@@ -186,6 +190,13 @@ def conv_transpose3d_forward(
     n, cin, *in_sp = (int(v) for v in x.shape)
     cout = int(w.shape[1])
     y_shape = (n, cout, in_sp[0] * k[0], in_sp[1] * k[1], in_sp[2] * k[2])
+    L = _lib.lib()
+    desc = ConvTDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2])
+    code = _lib.dtype_code(x.dtype)
+    if out_halo > 0 and out is None and n == 1 and not force_generic and min(in_sp) > 0:
+        done = _forward_into_slab(L, desc, code, x, w, bias, packed_weight, y_shape, k, int(out_halo))
+        if done is not None:
+            return done
     if out is None:
         y = torch.empty(y_shape, device=x.device, dtype=x.dtype, memory_format=_CL3D)
     else:
@@ -193,9 +204,6 @@ def conv_transpose3d_forward(
         _check_out(y, y_shape, x)
     if n == 0:
         return y
-    L = _lib.lib()
-    desc = ConvTDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2])
-    code = _lib.dtype_code(x.dtype)
     with _lib.device_guard(x.device):
         if packed_weight is not None:
             if force_generic:
@@ -210,6 +218,30 @@ def conv_transpose3d_forward(
                                    _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), _flags(force_generic),
                                    _lib.stream_ptr(x.device))
     _lib.check(rc, "conv_transpose3d_forward")
+    return y
+
+
+def _forward_into_slab(L, desc, code, x, w, bias, packed_weight, y_shape, k, halo):
+    """The forward launch with its result in the interior of a fresh depth slab, or ``None`` where the library does not
+    offer that for the problem (the caller then runs the plain launch)."""
+    _, cout, d, h, wd = y_shape
+    slab = torch.empty((1, cout, d + 2 * halo, h, wd), dtype=x.dtype, device=x.device, memory_format=_CL3D)
+    halo_elems = halo * h * wd * cout
+    with _lib.device_guard(x.device):
+        if packed_weight is not None:
+            _c3._problem(torch.Size(y_shape), torch.Size((int(x.shape[1]), cout, *k)), k, 0, 1, x.dtype).check_packed(packed_weight, True, x)
+            rc = L.sfh_convT3d_fwd_slab(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(packed_weight), None, _lib.ptr(bias),
+                                        _lib.ptr(slab), halo_elems, None, 0, _lib.SFH_FLAG_WEIGHT_PACKED, _lib.stream_ptr(x.device))
+        else:
+            ws = _lib.workspace(L.sfh_convT3d_fwd_workspace_bytes(ctypes.byref(desc), code), x.device)
+            rc = L.sfh_convT3d_fwd_slab(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w), _lib.strides5(w), _lib.ptr(bias),
+                                        _lib.ptr(slab), halo_elems, _lib.ptr(ws), 0 if ws is None else ws.numel(), 0,
+                                        _lib.stream_ptr(x.device))
+    if rc == _lib.SFH_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "conv_transpose3d_forward")
+    y = slab.narrow(2, halo, d)
+    y._sfh_slab = (slab, halo)
     return y
 
 

@@ -192,6 +192,11 @@ class UNet(nn.Module):
                 norm, conv = m.double_conv[1], m.double_conv[3]
                 if isinstance(norm, FastGroupNorm) and isinstance(conv, FastConv3d):
                     norm.out_halo = int(conv.padding[0]) if enabled else 0
+        # the pooling writes into the slab the first convolution of its level reads
+        for down in self.down_list[1:]:
+            pool, block = down.maxpool_conv
+            if isinstance(pool, FastMaxPool3d) and isinstance(block.double_conv[0], FastConv3d):
+                pool.out_halo = int(block.double_conv[0].padding[0]) if enabled else 0
         # The decoder's first convolutions read the skip connection and the upsampled tensor as they lie: their
         # producers (the encoder blocks' last GroupNorm, the up-convolutions) write them into slabs as well.
         for i, up in enumerate(self.up_list[:-1]):

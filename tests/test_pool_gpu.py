@@ -176,3 +176,40 @@ def test_pool_with_skip_sums_both_gradients_in_one_kernel(device, dtype, shape):
     _, s2 = max_pool3d_2x_with_skip(c2)
     s2.backward(gs)
     assert torch.equal(c2.grad, gs)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape,halo", [((1, 32, 8, 12, 20), 1), ((1, 64, 5, 9, 7), 1), ((1, 8, 4, 4, 6), 2), ((1, 3, 6, 6, 6), 1), ((2, 32, 4, 8, 8), 1)])
+def test_pooling_into_a_depth_slab_is_bitwise_the_plain_result(device, dtype, shape, halo):
+    """``max_pool3d_2x(x, out_halo=h)`` / ``with_skip``: the result lies in the interior of a slab whose faces the launch
+    zeroes, and is the plain result in values and gradients; where the library does not offer a slab (a batch, faces off the
+    16-byte grid) the plain tensor comes back."""
+    torch.manual_seed(7)
+    x0 = torch.randn(shape, device=device).to(dtype).contiguous(memory_format=CL)
+    n, c, d, h, w = shape
+    gy = torch.randn((n, c, d // 2, h // 2, w // 2), device=device).to(dtype).contiguous(memory_format=CL)
+    gs = torch.randn(shape, device=device).to(dtype).contiguous(memory_format=CL)
+    from scaffold_amd import pooling
+
+    def run(out_halo, with_skip):
+        x = x0.clone().requires_grad_(True)
+        if with_skip:
+            y, skip = pooling.max_pool3d_2x_with_skip(x, out_halo)
+            (y * gy).sum().backward(retain_graph=True)
+            skip.backward(gs)
+        else:
+            y = pooling.max_pool3d_2x(x, out_halo)
+            y.backward(gy)
+        return y, x.grad
+
+    for with_skip in (False, True):
+        y_plain, g_plain = run(0, with_skip)
+        y_slab, g_slab = run(halo, with_skip)
+        assert torch.equal(y_plain, y_slab) and torch.equal(g_plain, g_slab)
+        offered = n == 1 and (halo * (h // 2) * (w // 2) * c * x0.element_size()) % 16 == 0 and (y_plain.numel() * x0.element_size()) % 16 == 0
+        assert hasattr(y_slab, "_sfh_slab") == offered
+        if offered:
+            slab, hh = y_slab._sfh_slab
+            assert hh == halo and slab.shape == (1, c, d // 2 + 2 * halo, h // 2, w // 2)
+            assert y_slab.is_contiguous(memory_format=CL) and torch.equal(slab[:, :, halo:halo + d // 2], y_plain)
+            assert not slab[:, :, :halo].any() and not slab[:, :, halo + d // 2:].any()
