@@ -334,11 +334,12 @@ class FastConv3d(nn.Conv3d):
                                       "is not served as it stands (see takes_pair); concatenate instead")
         x_read, second_read, padding, slab, slab2 = ops
         dt = autocast_dtype(x)
-        wc = compute_copy(self.weight, dt)
-        bc = compute_copy(self.bias, dt) if wc is not None else None
-        master = wc is not None and (self.bias is None or bc is not None)
-        w = wc if master else cast_operand(self.weight, dt)
-        b = bc if master else cast_operand(self.bias, dt)
+        weight, bias = self.weight, self.bias  # (each lookup of a parameter is a call into Module.__getattr__)
+        wc = compute_copy(weight, dt)
+        bc = compute_copy(bias, dt) if wc is not None else None
+        master = wc is not None and (bias is None or bc is not None)
+        w = wc if master else cast_operand(weight, dt)
+        b = bc if master else cast_operand(bias, dt)
         stride, dilation = tuple(self.stride), tuple(self.dilation)
         if w.dtype is not x_read.dtype or not self._pair_gate(x_read, second_read, padding):
             raise NotImplementedError(
@@ -346,10 +347,10 @@ class FastConv3d(nn.Conv3d):
                 f"weight={tuple(w.shape)}/{w.dtype}, stride={stride} padding={padding} dilation={dilation}")
         in_shape = torch.Size((x_read.shape[0], x_read.shape[1] + second_read.shape[1], *x_read.shape[2:]))
         if master:
-            return _Conv3dFn.apply(x, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, in_shape, stride, padding, dilation), slab, self.gn_groups,
+            return _Conv3dFn.apply(x, weight, bias, stride, padding, dilation, w, b,
+                                   _current_packs(weight, w, in_shape, stride, padding, dilation), slab, self.gn_groups,
                                    self._gn_shift(), second, slab2)
-        packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is self.weight else None
+        packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is weight else None
         return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, self._gn_shift(), second,
                                slab2)
 
@@ -362,12 +363,13 @@ class FastConv3d(nn.Conv3d):
             raise NotImplementedError(f"FastConv3d: padding_mode={self.padding_mode!r} padding={self.padding!r}")
         dt = autocast_dtype(x)
         x = cast_operand(x, dt)
+        weight, bias = self.weight, self.bias  # (each lookup of a parameter is a call into Module.__getattr__)
         # under autocast, an up-to-date half-precision copy kept by the optimizer replaces the per-call cast
-        wc = compute_copy(self.weight, dt)
-        bc = compute_copy(self.bias, dt) if wc is not None else None
-        master = wc is not None and (self.bias is None or bc is not None)
-        w = wc if master else cast_operand(self.weight, dt)
-        b = bc if master else cast_operand(self.bias, dt)
+        wc = compute_copy(weight, dt)
+        bc = compute_copy(bias, dt) if wc is not None else None
+        master = wc is not None and (bias is None or bc is not None)
+        w = wc if master else cast_operand(weight, dt)
+        b = bc if master else cast_operand(bias, dt)
         padding = tuple(self.padding)
         inner, slab = x, None
         if self.shard_halo and padding[0] > 0:
@@ -393,10 +395,10 @@ class FastConv3d(nn.Conv3d):
         if slab is None:
             inner = x
         if master:
-            return _Conv3dFn.apply(inner, self.weight, self.bias, stride, padding, dilation, w, b,
-                                   _current_packs(self.weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
+            return _Conv3dFn.apply(inner, weight, bias, stride, padding, dilation, w, b,
+                                   _current_packs(weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
                                    self._gn_shift())
-        if w is self.weight:
+        if w is weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
                                    _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups, self._gn_shift())
         return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups, self._gn_shift())
@@ -413,11 +415,12 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
             raise NotImplementedError("FastConvTranspose3d: output_size is not supported")
         dt = autocast_dtype(x)
         x = cast_operand(x, dt)
-        wc = compute_copy(self.weight, dt)
-        bc = compute_copy(self.bias, dt) if wc is not None else None
-        master = wc is not None and (self.bias is None or bc is not None)
-        w = wc if master else cast_operand(self.weight, dt)
-        b = bc if master else cast_operand(self.bias, dt)
+        weight, bias = self.weight, self.bias
+        wc = compute_copy(weight, dt)
+        bc = compute_copy(bias, dt) if wc is not None else None
+        master = wc is not None and (bias is None or bc is not None)
+        w = wc if master else cast_operand(weight, dt)
+        b = bc if master else cast_operand(bias, dt)
         x = x.contiguous(memory_format=_CL3D)
         gate = _ct.is_supported_transposed_all if _wants_grad(x, w, b) else _ct.is_supported_transposed
         if not gate(x, w, b, self.stride, self.padding, self.output_padding, self.dilation, self.groups):
@@ -427,15 +430,15 @@ class FastConvTranspose3d(nn.ConvTranspose3d):
                 f"dilation={self.dilation} groups={self.groups}"
             )
         stride = tuple(self.stride)
-        if master or w is self.weight:
+        if master or w is weight:
             # the problem the packed forms belong to: the stride-k convolution over this op's output
             n, _, d, h, wd = x.shape
             big = torch.Size((n, w.shape[1], d * stride[0], h * stride[1], wd * stride[2]))
-            packs = _current_packs(self.weight, w, big, stride, (0, 0, 0), (1, 1, 1))
+            packs = _current_packs(weight, w, big, stride, (0, 0, 0), (1, 1, 1))
             if packs is not None and (packs.fwd is None or packs.dgrad is None):
                 packs = None
             if master:
-                return _ConvTranspose3dFn.apply(x, self.weight, self.bias, stride, w, b, packs, self.out_halo)
+                return _ConvTranspose3dFn.apply(x, weight, bias, stride, w, b, packs, self.out_halo)
             return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, packs, self.out_halo)
         return _ConvTranspose3dFn.apply(x, w, b, stride, None, None, None, self.out_halo)
 
@@ -462,6 +465,7 @@ class FastGroupNorm(nn.GroupNorm):
             x = x.contiguous(memory_format=_CL3D)
         out = _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
                              out_halo=self.out_halo)
-        # what the convolution in front should take its next call's sums about
-        self._next_shift = getattr(out, "_sfh_gn_shift", None)
+        # what the convolution in front should take its next call's sums about (a plain attribute: straight into the
+        # instance dictionary, past Module.__setattr__'s parameter / buffer / submodule checks)
+        self.__dict__["_next_shift"] = getattr(out, "_sfh_gn_shift", None)
         return out
