@@ -113,6 +113,41 @@ def test_launch_geometry_is_stated_and_agrees_with_the_workspace():
     assert L.sfh_conv3d_launch_geometry(ctypes.byref(cube), bf16, 0, None) == _lib.SFH_ERR_INVALID
 
 
+def test_which_problems_take_a_skip_connection_as_two_tensors():
+    """``sfh_conv3d_pair_supported`` is a pure function of problem, dtype, cut and direction; the entry points refuse what it
+    refuses before anything is launched."""
+    L = _lib.lib()
+    bf16, fp16, fp32 = 0, 1, 2
+
+    def offered(desc, dtype, first):
+        return [L.sfh_conv3d_pair_supported(ctypes.byref(desc), dtype, first, d) for d in (0, 1, 2)]
+
+    level0 = conv_desc(cin=64, cout=32, sp=(66, 128, 128), p=(0, 1, 1))   # the decoder's first convolution on a depth shard
+    assert offered(level0, bf16, 32) == [1, 1, 1] and offered(level0, fp16, 32) == [1, 1, 1]
+    assert offered(level0, fp32, 32) == [0, 0, 0]                        # the fp32 tiles read one tensor
+    assert offered(level0, bf16, 16) == [0, 0, 0] and offered(level0, bf16, 48) == [0, 0, 0]  # a cut off the 32-channel grid
+    assert offered(level0, bf16, 0) == [0, 0, 0] and offered(level0, bf16, 64) == [0, 0, 0]   # nothing on one side
+    assert L.sfh_conv3d_pair_supported(ctypes.byref(level0), bf16, 32, 3) == 0
+    wide = conv_desc(cin=128, cout=64, sp=(34, 64, 64), p=(0, 1, 1))      # forward on the wide-tile kernel: equal halves only
+    assert offered(wide, bf16, 64) == [1, 1, 1] and offered(wide, bf16, 32) == [0, 1, 1]
+    assert offered(conv_desc(cin=96, cout=32, sp=(8, 16, 16)), bf16, 64) == [1, 1, 1]        # an unequal cut elsewhere is fine
+    deep = conv_desc(cin=512, cout=256, sp=(8, 16, 16))                   # both directions sliced: the slice sum writes the pair
+    assert offered(deep, bf16, 256) == [1, 1, 1]
+    assert offered(conv_desc(cin=64, cout=32, k=(1, 1, 1), p=(0, 0, 0)), bf16, 32) == [0, 0, 0]      # not a 3x3x3 problem
+    assert offered(conv_desc(cin=64, cout=32, s=(2, 2, 2)), bf16, 32)[1] == 0                        # strided: no data gradient at all
+    assert offered(conv_desc(cin=64, cout=32, n=0), bf16, 32) == [0, 0, 0]
+    # refused calls launch nothing: null tensors are never touched
+    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, None, None, 16, None, None, None, None, None, 0, 0, 0, None, None, 0,
+                                 None) == _lib.SFH_ERR_INVALID
+    one = ctypes.c_void_p(16)  # a non-null stand-in that must not be dereferenced
+    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, one, one, 16, one, None, None, one, None, 0, 0, 0, None, None, 0,
+                                 None) == _lib.SFH_ERR_UNSUPPORTED
+    assert L.sfh_conv3d_dgrad_pair(ctypes.byref(level0), bf16, one, one, None, one, one, 48, None, 0, 0, None) == _lib.SFH_ERR_UNSUPPORTED
+    assert L.sfh_conv3d_wgrad_pair(ctypes.byref(level0), fp32, one, one, 32, one, one, None, 0, 0, None) == _lib.SFH_ERR_UNSUPPORTED
+    assert L.sfh_conv3d_wgrad_pair(ctypes.byref(level0), bf16, one, one, 32, one, one, None, 0, _lib.SFH_FLAG_FORCE_GENERIC,
+                                   None) == _lib.SFH_ERR_INVALID
+
+
 def test_wgrad_split_plan_partitions_the_bricks():
     """Every brick belongs to exactly one split: splits * ceil(bricks / splits) covers, (splits-1) * that does not."""
     L = _lib.lib()
