@@ -76,7 +76,7 @@ typedef struct sfh_groupnorm_desc {
 /* 100: the first published set of entry points. 101: sfh_conv3d_launch_geometry, sfh_conv3d_fwd_gn_records,
  * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed.
  * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair,
- * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab added. */
+ * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab, sfh_convT3d_wgrad_bias(_workspace_bytes) added. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -253,6 +253,16 @@ int sfh_convT3d_fwd(const sfh_convT3d_desc* p, int dtype, const void* x, const v
 int sfh_convT3d_fwd_slab(const sfh_convT3d_desc* p, int dtype, const void* x, const void* w,
                          const int64_t w_stride[5], const void* bias, void* y_slab, int64_t halo_elems,
                          void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
+
+/* Weight gradient AND bias gradient of the transposed convolution from one pass over its output gradient gy
+ * (the reference computes them apart: transposed.py:1113 and `grad_output.sum((0, 2, 3, 4))`, ScaFFold/unet/conv3d.py:1786).
+ * gw: [Cin][kd][kh][kw][Cout] dense, as sfh_conv3d_wgrad writes it for the swapped problem; gb: Cout elements; both in the
+ * operands' dtype, or fp32 with SFH_FLAG_GRAD_FP32; fp32 partial slices summed in a fixed order, no atomics. 2x2x2
+ * problems on the matrix cores only (16-bit dtypes, Cin a multiple of 64, Cout of 32): SFH_ERR_UNSUPPORTED otherwise, and
+ * the workspace query returns 0. */
+size_t sfh_convT3d_wgrad_bias_workspace_bytes(const sfh_convT3d_desc* p, int dtype);
+int sfh_convT3d_wgrad_bias(const sfh_convT3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* gb,
+                           void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
 /* ---- GroupNorm forward ---------------------------------------------------------------
  * Stands in for torch.ops.scaffold_gn.group_norm (ScaFFold/unet/triton_group_norm.py:1339)

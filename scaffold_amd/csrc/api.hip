@@ -841,6 +841,33 @@ extern "C" int sfh_convT3d_fwd_slab(const sfh_convT3d_desc* p, int dtype, const 
                          flags, stream, halo_elems);
 }
 
+// Weight and bias gradient of the transposed convolution in one pass over its output gradient (2x2x2 matrix-core
+// problems): the weight gradient is the stride-2 convolution's with the operands swapped, the bias gradient the column
+// sums of the same tiles.
+static bool convT_wgrad_bias_ok(const sfh_convT3d_desc& p, int dtype) {
+  return p.kd == 2 && p.kh == 2 && p.kw == 2 && p.n >= 1 && patch_reduce_supported(convT_patch_args(p), dtype);
+}
+
+extern "C" size_t sfh_convT3d_wgrad_bias_workspace_bytes(const sfh_convT3d_desc* p, int dtype) {
+  if (check_convT(p, dtype) != SFH_OK || !convT_wgrad_bias_ok(*p, dtype)) return 0;
+  return patch_reduce_workspace_bytes(convT_patch_args(*p), true);
+}
+
+extern "C" int sfh_convT3d_wgrad_bias(const sfh_convT3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* gb,
+                                      void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  if (int rc = check_convT(p, dtype)) return rc;
+  if (x == nullptr || gy == nullptr || gw == nullptr || gb == nullptr) return fail(SFH_ERR_INVALID, "convT3d wgrad: null tensor");
+  if ((flags & SFH_FLAG_FORCE_GENERIC) || !convT_wgrad_bias_ok(*p, dtype))
+    return fail(SFH_ERR_UNSUPPORTED, "convT3d wgrad with bias gradient: 2x2x2 matrix-core problems only");
+  const PatchArgs a = convT_patch_args(*p);
+  const size_t need = patch_reduce_workspace_bytes(a, true);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "convT3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  const int g_dtype = (flags & SFH_FLAG_GRAD_FP32) ? SFH_FP32 : dtype;
+  // small = the transposed convolution's input, big = its output gradient
+  return patch_reduce(a, dtype, x, gy, gw, g_dtype, workspace, (hipStream_t)stream, gb);
+}
+
 // ---- loss head -------------------------------------------------------------------------
 static int check_loss(const sfh_loss_desc* p, int dtype) {
   if (p == nullptr) return fail(SFH_ERR_INVALID, "ce_dice: null descriptor");

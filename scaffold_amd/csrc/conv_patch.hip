@@ -233,9 +233,13 @@ __device__ __forceinline__ uint4 tr_fragment(const T* tile, int row_stride, int 
 }
 
 // grid = (splits, csmall / 64, cbig / 32). Wavefront w accumulates taps 2w and 2w + 1 for both row blocks.
-template <typename T>
+// BIAS: the workgroups of the first small-channel tile also add up the big tensor itself over the voxels -- the bias
+// gradient of the transposed convolution whose weight gradient this is (every big voxel is a tap of exactly one small
+// voxel there) -- as one more MFMA row block of ones: bias_part[split][tap][cb], the same fixed order as the weights'.
+template <typename T, bool BIAS>
 __global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T* __restrict__ small, const T* __restrict__ big,
-                                                           float* __restrict__ part, int64_t total, int64_t per_split) {
+                                                           float* __restrict__ part, int64_t total, int64_t per_split,
+                                                           float* __restrict__ bias_part) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __shared__ __attribute__((aligned(16))) T s_tile[kVx * kSRow];
   __shared__ __attribute__((aligned(16))) T b_tile[kTaps * kVx * kBRow];
@@ -251,6 +255,14 @@ __global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T*
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  f32x16_t bacc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bacc[j][r] = 0.f;
+  const bool sums_big = BIAS && blockIdx.y == 0;
+  const uint32_t one2 = sizeof(T) == 2 && std::is_same<T, bf16_t>::value ? 0x3f803f80u : 0x3c003c00u;  // two ones of T
+  const uint4 ones = make_uint4(one2, one2, one2, one2);
   const int s_vox = tid >> 3, s_piece = tid & 7;          // small tile: 32 voxels x 8 pieces of 16 bytes
   const int b_vox = (tid >> 2) & 31, b_piece = tid & 3;   // big tiles: 4 taps (tid/128, +2, +4, +6) of one voxel
   const int b_tap0 = tid >> 7;
@@ -280,6 +292,12 @@ __global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T*
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j) acc[i][j] = Mma32<T>::run(af[i], bf[j], acc[i][j]);
+      if constexpr (BIAS) {
+        if (sums_big) {  // every row of the block is the column sum
+#pragma unroll
+          for (int j = 0; j < 2; ++j) bacc[j] = Mma32<T>::run(ones, bf[j], bacc[j]);
+        }
+      }
     }
   }
   // part[split][cs][tap][cb]: a lane holds column cb = lane % 32 and 16 rows of each block
@@ -294,6 +312,12 @@ __global__ void __launch_bounds__(256) patch_reduce_kernel(PatchArgs a, const T*
         const int cs = cs0 + i * 32 + 8 * (r >> 2) + 4 * kg + (r & 3);
         dst[((int64_t)cs * kTaps + 2 * wave + j) * a.cbig + cb0 + col] = acc[i][j][r];
       }
+  if constexpr (BIAS) {
+    if (sums_big && kg == 0) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bias_part[((int64_t)blockIdx.x * kTaps + 2 * wave + j) * a.cbig + cb0 + col] = bacc[j][0];
+    }
+  }
 #endif
 }
 
@@ -378,15 +402,22 @@ ReducePlan reduce_plan(const PatchArgs& a) {
 }
 
 template <typename T>
-int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st) {
+int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st, void* gb) {
   const ReducePlan p = reduce_plan(a);
   const int64_t total = small_voxels(a);
   const dim3 grid((unsigned)p.splits, (unsigned)(a.csmall / kSmallTile), (unsigned)(a.cbig / 32));
-  hipLaunchKernelGGL((patch_reduce_kernel<T>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)big, (float*)ws, total,
-                     p.per_split);
-  if (int rc = check_launch("patch_reduce_kernel")) return rc;
   const int64_t nelem = (int64_t)a.csmall * kTaps * a.cbig;
-  return sum_slices(g_dtype, (const float*)ws, g, nelem, p.splits, st);
+  float* bias_part = (float*)ws + (int64_t)p.splits * nelem;  // behind the weight slices
+  if (gb != nullptr)
+    hipLaunchKernelGGL((patch_reduce_kernel<T, true>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)big, (float*)ws, total,
+                       p.per_split, bias_part);
+  else
+    hipLaunchKernelGGL((patch_reduce_kernel<T, false>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)big, (float*)ws, total,
+                       p.per_split, (float*)nullptr);
+  if (int rc = check_launch("patch_reduce_kernel")) return rc;
+  if (int rc = sum_slices(g_dtype, (const float*)ws, g, nelem, p.splits, st)) return rc;
+  if (gb == nullptr) return SFH_OK;
+  return sum_slices(g_dtype, bias_part, gb, a.cbig, p.splits * kTaps, st);  // [split][tap][channel]: slices of cbig elements
 }
 
 bool geometry_ok(const PatchArgs& a, int dtype) {
@@ -421,13 +452,17 @@ int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* 
 
 int patch_reduce_splits(const PatchArgs& a) { return reduce_plan(a).splits; }
 
-size_t patch_reduce_workspace_bytes(const PatchArgs& a) {
-  return (size_t)reduce_plan(a).splits * a.csmall * kTaps * a.cbig * sizeof(float);
+size_t patch_reduce_workspace_bytes(const PatchArgs& a, bool with_bias) {
+  const size_t splits = (size_t)reduce_plan(a).splits;
+  return splits * a.csmall * kTaps * a.cbig * sizeof(float) + (with_bias ? splits * kTaps * a.cbig * sizeof(float) : 0);
 }
 
-int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st) {
-  if (dtype == SFH_BF16) return launch_reduce<bf16_t>(a, small, big, g, g_dtype, ws, st);
-  return launch_reduce<fp16_t>(a, small, big, g, g_dtype, ws, st);
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st,
+                 void* gb) {
+  if (gb != nullptr && (a.bd != 2 * a.sd || a.bh != 2 * a.sh || a.bw != 2 * a.sw))
+    return fail(SFH_ERR_UNSUPPORTED, "2x2x2 weight gradient: the bias gradient needs every big voxel under a tap");
+  if (dtype == SFH_BF16) return launch_reduce<bf16_t>(a, small, big, g, g_dtype, ws, st, gb);
+  return launch_reduce<fp16_t>(a, small, big, g, g_dtype, ws, st, gb);
 }
 
 }  // namespace sfh

@@ -26,8 +26,11 @@ int patch_gather(const PatchArgs& a, int dtype, const void* big, const void* pac
 int patch_scatter(const PatchArgs& a, int dtype, const void* small, const void* packed, const void* bias, void* big, hipStream_t st,
                   int64_t halo_elems = 0);
 int patch_reduce_splits(const PatchArgs& a);
-size_t patch_reduce_workspace_bytes(const PatchArgs& a);
-// g: dense [csmall][8][cbig] in the element type, from fp32 partial slices in ws summed in split order
-int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st);
+size_t patch_reduce_workspace_bytes(const PatchArgs& a, bool with_bias = false);
+// g: dense [csmall][8][cbig] in the element type, from fp32 partial slices in ws summed in split order.
+// gb (optional, big extents exactly twice the small ones): also the sum of `big` over all voxels per channel, cbig
+// elements of g's type -- the bias gradient of the transposed convolution -- from the same pass over `big`.
+int patch_reduce(const PatchArgs& a, int dtype, const void* small, const void* big, void* g, int g_dtype, void* ws, hipStream_t st,
+                 void* gb = nullptr);
 
 }  // namespace sfh

@@ -235,7 +235,16 @@ class _ConvTranspose3dFn(torch.autograd.Function):
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = _ct.conv_transpose3d_backward_data(grad_output, weight, x.shape, stride, 0, 0, 1, 1,
                                                     packed_weight=packed[0] if packed else None) if needs_x else None
-        grad_w = None
+        grad_w = grad_b = None
+        if needs_w and has_bias and needs_b:
+            # both from one pass over grad_output where the library offers it (the 2x2x2 matrix-core problems)
+            both = _ct.conv_transpose3d_backward_weight_bias(x, weight.shape, grad_output, stride, 0, 0, 1, 1,
+                                                             grad_dtype=torch.float32 if master else None)
+            if both is not None:
+                grad_w, grad_b = both
+                if grad_b.dtype is not bias_dtype:
+                    grad_b = grad_b.to(bias_dtype)
+                return grad_x, grad_w, grad_b, None, None, None, None, None
         if needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_ct.conv_transpose3d_backward_weight, x, weight.shape, grad_output, stride, 0, 0, 1, 1)

@@ -39,6 +39,7 @@ __all__ = [
     "conv_transpose3d_forward",
     "conv_transpose3d_backward_data",
     "conv_transpose3d_backward_weight",
+    "conv_transpose3d_backward_weight_bias",
     "is_supported_transposed",
     "is_supported_transposed_all",
     "is_supported_transposed_bwd_data",
@@ -219,6 +220,45 @@ def conv_transpose3d_forward(
                                    _lib.stream_ptr(x.device))
     _lib.check(rc, "conv_transpose3d_forward")
     return y
+
+
+def conv_transpose3d_backward_weight_bias(x: torch.Tensor, weight_shape: Sequence[int], grad_output: torch.Tensor, stride=1, padding=0,
+                                          output_padding=0, dilation=1, groups: int = 1, *, grad_dtype: Optional[torch.dtype] = None):
+    """``(grad_weight, grad_bias)`` of the transposed convolution from ONE pass over ``grad_output``: the weight gradient of
+    :func:`conv_transpose3d_backward_weight` (same bits) and ``grad_output.sum((0, 2, 3, 4))`` (fp32 accumulation in a fixed
+    order, one rounding; ``ScaFFold/unet/conv3d.py:1786``) from the tiles the weight gradient reads anyway.  Both come in
+    ``grad_dtype`` (default: the operands' dtype).  Returns ``None`` where the library does not offer the fused form (anything
+    but the 2x2x2 matrix-core problems): the caller then computes the two apart."""
+    if not is_supported_transposed_bwd_weight(x, weight_shape, grad_output, stride, padding, output_padding, dilation, groups):
+        raise NotImplementedError(
+            f"unsupported: x={tuple(getattr(x, 'shape', ()))} weight_shape={tuple(weight_shape)} "
+            f"grad_output={tuple(getattr(grad_output, 'shape', ()))} stride={stride}")
+    ws_shape = tuple(int(v) for v in weight_shape)
+    x = x.contiguous(memory_format=_CL3D)
+    gy = grad_output.contiguous(memory_format=_CL3D)
+    n, cin, *in_sp = (int(v) for v in x.shape)
+    cout, k = ws_shape[1], ws_shape[2:]
+    if n == 0:
+        return None
+    gdt = x.dtype if grad_dtype is None else grad_dtype
+    if gdt is not x.dtype and gdt is not torch.float32:
+        raise ValueError(f"grad_dtype must be the operands' dtype or torch.float32, got {grad_dtype}")
+    L = _lib.lib()
+    desc = ConvTDesc(n, cin, in_sp[0], in_sp[1], in_sp[2], cout, k[0], k[1], k[2])
+    code = _lib.dtype_code(x.dtype)
+    need = int(L.sfh_convT3d_wgrad_bias_workspace_bytes(ctypes.byref(desc), code))
+    if need == 0:
+        return None
+    gw = torch.empty(ws_shape, dtype=gdt, device=x.device, memory_format=_CL3D)
+    gb = torch.empty((cout,), dtype=gdt, device=x.device)
+    with _lib.device_guard(x.device):
+        ws = _lib.workspace(need, x.device)
+        rc = L.sfh_convT3d_wgrad_bias(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(gb), _lib.ptr(ws), need,
+                                      _lib.SFH_FLAG_GRAD_FP32 if gdt is not x.dtype else 0, _lib.stream_ptr(x.device))
+    if rc == _lib.SFH_ERR_UNSUPPORTED:
+        return None
+    _lib.check(rc, "conv_transpose3d_backward_weight_bias")
+    return gw, gb
 
 
 def _forward_into_slab(L, desc, code, x, w, bias, packed_weight, y_shape, k, halo):
