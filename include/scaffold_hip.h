@@ -76,7 +76,8 @@ typedef struct sfh_groupnorm_desc {
 /* 100: the first published set of entry points. 101: sfh_conv3d_launch_geometry, sfh_conv3d_fwd_gn_records,
  * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed.
  * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair,
- * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab, sfh_convT3d_wgrad_bias(_workspace_bytes) added. */
+ * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab, sfh_convT3d_wgrad_bias(_workspace_bytes),
+ * sfh_conv3d_wgrad_bias(_workspace_bytes) added. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -225,6 +226,15 @@ int sfh_conv3d_dgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* gy, c
 int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second,
                           int32_t cin_first, const void* gy, void* gw, void* workspace, size_t workspace_bytes,
                           uint32_t flags, void* stream);
+
+/* Weight gradient and bias gradient from one pass over gy, where the kernel that serves the problem reads gy tile by tile
+ * anyway: the 1x1x1 convolutions with at most 32 output channels over 32 / 64 / 128 input channels (the U-Net's head),
+ * 16-bit dtypes. gb: Cout elements in gw's dtype (the operands', or fp32 with SFH_FLAG_GRAD_FP32) =
+ * gy.sum over voxels (ScaFFold/unet/conv3d.py:1231), fp32 slices summed in a fixed order. The workspace query returns 0
+ * and the call SFH_ERR_UNSUPPORTED for every other problem: the caller then uses sfh_conv3d_wgrad and sfh_bias_grad. */
+size_t sfh_conv3d_wgrad_bias_workspace_bytes(const sfh_conv3d_desc* p, int dtype);
+int sfh_conv3d_wgrad_bias(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* gb,
+                          void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
 
 /* ---- bias gradient --------------------------------------------------------------------
  * Stands in for `grad_output.sum((0, 2, 3, 4))` in the reference's autograd functions

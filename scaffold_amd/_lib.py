@@ -135,6 +135,9 @@ _SIGNATURES = {
     "sfh_convT3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvTDesc), c_int]),
     "sfh_convT3d_fwd": (c_int, [POINTER(ConvTDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                 c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_wgrad_bias_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_wgrad_bias": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,
+                                      c_void_p]),
     "sfh_convT3d_wgrad_bias_workspace_bytes": (c_size_t, [POINTER(ConvTDesc), c_int]),
     "sfh_convT3d_wgrad_bias": (c_int, [POINTER(ConvTDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_uint32,
                                        c_void_p]),

@@ -58,6 +58,7 @@ __all__ = [
     "conv3d_forward_pair",
     "conv3d_backward_data_pair",
     "conv3d_backward_weight_pair",
+    "conv3d_backward_weight_bias",
 ]
 
 _CL3D = torch.channels_last_3d
@@ -840,6 +841,42 @@ def conv3d_backward_weight(
                                          _lib.ptr(gw), _lib.ptr(ws), ws_bytes, flags, _lib.stream_ptr(x.device))
     _lib.check(rc, "conv3d_backward_weight")
     return gw
+
+
+def conv3d_backward_weight_bias(input: torch.Tensor, weight_shape: Sequence[int], grad_output: torch.Tensor, stride=1, padding=0,
+                                dilation=1, groups: int = 1, *, grad_dtype: Optional[torch.dtype] = None, _checked: bool = False):
+    """``(grad_weight, grad_bias)`` from ONE pass over ``grad_output`` where the kernel that serves the problem reads it tile
+    by tile anyway (the 1x1x1 convolutions with few output channels: the U-Net's head): the weight gradient of
+    :func:`conv3d_backward_weight` (same bits) and ``grad_output.sum((0, 2, 3, 4))`` (``ScaFFold/unet/conv3d.py:1231``; fp32
+    slices summed in a fixed order, one rounding), both in ``grad_dtype`` (default: the operands' dtype).  ``None`` where the
+    library does not offer the fused form: the caller then computes the two apart."""
+    if not _checked and not is_supported_bwd_weight(input, weight_shape, grad_output, stride, padding, dilation, groups):
+        raise NotImplementedError(
+            f"unsupported: input={tuple(getattr(input, 'shape', ()))}/{getattr(input, 'dtype', None)} "
+            f"weight_shape={tuple(weight_shape)} grad_output={tuple(getattr(grad_output, 'shape', ()))}")
+    x = input.contiguous(memory_format=_CL3D)
+    gy = grad_output.contiguous(memory_format=_CL3D)
+    prob = _problem(x.shape, weight_shape if isinstance(weight_shape, torch.Size) else tuple(weight_shape), stride, padding,
+                    dilation, x.dtype)
+    if prob.n == 0:
+        return None
+    need = prob.workspace_bytes("wgrad_bias")
+    if need == 0:
+        return None
+    gdt = x.dtype if grad_dtype is None else grad_dtype
+    if gdt is not x.dtype and gdt is not torch.float32:
+        raise ValueError(f"grad_dtype must be the operands' dtype or torch.float32, got {grad_dtype}")
+    gw = torch.empty((prob.cout, prob.cin, *prob.k), dtype=gdt, device=x.device, memory_format=_CL3D)
+    gb = torch.empty((prob.cout,), dtype=gdt, device=x.device)
+    with _lib.device_guard(x.device):
+        ws = _lib.workspace(need, x.device)
+        rc = _lib.lib().sfh_conv3d_wgrad_bias(ctypes.byref(prob.desc), prob.code, _lib.ptr(x), _lib.ptr(gy), _lib.ptr(gw), _lib.ptr(gb),
+                                              _lib.ptr(ws), need, _lib.SFH_FLAG_GRAD_FP32 if gdt is not x.dtype else 0,
+                                              _lib.stream_ptr(x.device))
+    if rc == _lib.SFH_ERR_UNSUPPORTED:  # e.g. operands off the 16-byte grid
+        return None
+    _lib.check(rc, "conv3d_backward_weight_bias")
+    return gw, gb
 
 
 # ---------------------------------------------------------------------------------------------

@@ -667,6 +667,38 @@ extern "C" int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void*
   return conv3d_wgrad_any(p, dtype, x, gy, gw, workspace, workspace_bytes, flags, stream, nullptr);
 }
 
+// ---- weight gradient with the bias gradient from the same pass (the 1x1x1 head) ------------------------------------
+static bool wgrad_bias_plan(const sfh_conv3d_desc& p, int dtype, const int32_t out[3], ThinArgs& t) {
+  bool thin_is_x = false;
+  // the output gradient must be the thin operand: its sums over the voxels are the bias gradient
+  return thin_wgrad_plan(p, dtype, out, t, thin_is_x) == kThinReduce && !thin_is_x && thin_reduce_offers_thin_sums(t, dtype);
+}
+
+extern "C" size_t sfh_conv3d_wgrad_bias_workspace_bytes(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  ThinArgs t;
+  if (check_conv(p, dtype, out) != SFH_OK || wgrad_uses_mfma(*p, dtype, out) || wgrad_uses_f32_tiles(*p, dtype, out) ||
+      wgrad_uses_patch(*p, dtype, out) || !wgrad_bias_plan(*p, dtype, out, t))
+    return 0;
+  return thin_reduce_workspace_bytes(t, true);
+}
+
+extern "C" int sfh_conv3d_wgrad_bias(const sfh_conv3d_desc* p, int dtype, const void* x, const void* gy, void* gw, void* gb,
+                                     void* workspace, size_t workspace_bytes, uint32_t flags, void* stream) {
+  int32_t out[3];
+  if (int rc = check_conv(p, dtype, out)) return rc;
+  if (x == nullptr || gy == nullptr || gw == nullptr || gb == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad: null tensor");
+  const size_t need = sfh_conv3d_wgrad_bias_workspace_bytes(p, dtype);
+  if ((flags & SFH_FLAG_FORCE_GENERIC) || need == 0)
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad with bias gradient: the 1x1x1 thin-output problems on the matrix cores only");
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "conv3d wgrad: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  ThinArgs t;
+  wgrad_bias_plan(*p, dtype, out, t);
+  const int g_dtype = (flags & SFH_FLAG_GRAD_FP32) ? SFH_FP32 : dtype;
+  return thin_reduce(t, dtype, gy, x, gw, g_dtype, workspace, (hipStream_t)stream, gb);
+}
+
 // ---- a convolution over two tensors whose channels follow each other (the skip connection, never concatenated) ------
 extern "C" int sfh_conv3d_pair_supported(const sfh_conv3d_desc* p, int dtype, int32_t cin_first, int direction) {
   int32_t out[3];

@@ -13,6 +13,7 @@
 // The reference serves these shapes with the same implicit-GEMM kernels at small tile sizes
 // (triton_conv3d/gather_gemm.py:493-560, reduce_gemm.py:655-700).
 #include "conv_thin.hpp"
+#include <type_traits>
 #include "mma.hpp"
 #include "reduce.hpp"
 #include "vec_io.hpp"
@@ -290,7 +291,10 @@ __global__ void __launch_bounds__(kBlock) head_wide_out_kernel(ThinArgs a, const
 // never written out; voxels beyond the range are zero on both sides.
 template <typename T, int NC>
 __global__ void __launch_bounds__(kBlock) head_reduce_kernel(ThinArgs a, const T* __restrict__ thin, const T* __restrict__ wide,
-                                                             float* __restrict__ part, int64_t total, int64_t per_split) {
+                                                             float* __restrict__ part, int64_t total, int64_t per_split,
+                                                             float* __restrict__ bias_part) {
+  // bias_part (optional): also the sums of the thin tensor over the voxels, [split][J] -- the bias gradient when the
+  // thin tensor is the output gradient -- as one more MFMA against a column block of ones.
   constexpr int CW = NC * 32;
   __shared__ __align__(16) uint16_t trows[(kHeadVoxels + 1) * kHeadThinMax];
   constexpr int kFoldHalves = 4 * 32 * 33 * 2;  // the fold at the end reuses the wide rows
@@ -303,6 +307,11 @@ __global__ void __launch_bounds__(kBlock) head_reduce_kernel(ThinArgs a, const T
   for (int cc = 0; cc < NC; ++cc)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[cc][r] = 0.f;
+  f32x16_t bacc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) bacc[r] = 0.f;
+  const uint32_t one2 = std::is_same<T, bf16_t>::value ? 0x3f803f80u : 0x3c003c00u;  // two ones of T
+  const uint4 ones = make_uint4(one2, one2, one2, one2);
   const int64_t begin = (int64_t)blockIdx.x * per_split;
   int64_t end = begin + per_split;
   if (end > total) end = total;
@@ -328,6 +337,7 @@ __global__ void __launch_bounds__(kBlock) head_reduce_kernel(ThinArgs a, const T
 #pragma unroll
       for (int e = 0; e < 8; ++e) h[e] = trows[(v0 + e) * J + col];
       const uint4 tf = make_uint4(h[0] | h[1] << 16, h[2] | h[3] << 16, h[4] | h[5] << 16, h[6] | h[7] << 16);
+      if (bias_part != nullptr) bacc = Mma32<T>::run(tf, ones, bacc);  // every column is the row sum
 #pragma unroll
       for (int cc = 0; cc < NC; ++cc) {
 #pragma unroll
@@ -357,6 +367,16 @@ __global__ void __launch_bounds__(kBlock) head_reduce_kernel(ThinArgs a, const T
       dst[(int64_t)(cc * 32 + c) * a.so_wide + (int64_t)j * a.so_thin] = sum;
     }
     __syncthreads();
+  }
+  if (bias_part != nullptr) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int j = 8 * (r / 4) + 4 * kg + r % 4;
+      fold[(wave * 32 + j) * 33 + col] = bacc[r];
+    }
+    __syncthreads();
+    if (tid < J)
+      bias_part[(int64_t)blockIdx.x * J + tid] = (fold[tid * 33] + fold[(32 + tid) * 33]) + (fold[(64 + tid) * 33] + fold[(96 + tid) * 33]);
   }
 }
 
@@ -876,8 +896,15 @@ int dispatch_thin_out(const ThinArgs& a, const void* wide, const void* wt, const
   if (a.J <= 16) return launch_thin_out<T, 16>(a, wide, wt, bias, out, st);
   return launch_thin_out<T, 32>(a, wide, wt, bias, out, st);
 }
+// The kernel that leaves the thin tensor's sums beside the weight gradient: the 1x1x1 head with 32 / 64 / 128 wide channels.
+bool head_reduce_applies(const ThinArgs& a) {
+  return !stem_brick_ok(a) && a.K == 0 && (a.cw == 32 || a.cw == 64 || a.cw == 128);
+}
+
 template <typename T>
-int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
+int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st, void* gb) {
+  if (gb != nullptr && !(sizeof(T) == 2 && head_reduce_applies(a) && ((uintptr_t)thin | (uintptr_t)wide) % 16 == 0))
+    return fail(SFH_ERR_UNSUPPORTED, "thin-channel weight gradient: the sums of the thin tensor are not offered for this problem");
   if constexpr (sizeof(T) == 2) {
     if (stem_brick_ok(a) && stem_tiles(a) <= 0x7fffffffLL && (a.cw == 32 || a.cw == 64) && (uintptr_t)wide % 16 == 0) {
       const int nsplit = thin_reduce_splits(a);
@@ -905,11 +932,13 @@ int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void*
       const int nsplit = thin_reduce_splits(a);
       const int64_t per = cdiv(cdiv(total, nsplit), kHeadVoxels) * kHeadVoxels;  // keeps every range 16-byte aligned
       const dim3 grid(nsplit);
-      if (a.cw == 32) hipLaunchKernelGGL((head_reduce_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
-      else if (a.cw == 64) hipLaunchKernelGGL((head_reduce_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
-      else hipLaunchKernelGGL((head_reduce_kernel<T, 4>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per);
+      float* bias_part = gb != nullptr ? (float*)ws + (int64_t)nsplit * a.J * a.cw : nullptr;  // behind the weight slices
+      if (a.cw == 32) hipLaunchKernelGGL((head_reduce_kernel<T, 1>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per, bias_part);
+      else if (a.cw == 64) hipLaunchKernelGGL((head_reduce_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per, bias_part);
+      else hipLaunchKernelGGL((head_reduce_kernel<T, 4>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per, bias_part);
       if (int rc = check_launch("head_reduce_kernel")) return rc;
-      return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+      if (int rc = sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st)) return rc;
+      return gb != nullptr ? sum_slices(gw_dtype, bias_part, gb, a.J, nsplit, st) : SFH_OK;
     }
   }
   if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, gw_dtype, ws, st);
@@ -935,8 +964,12 @@ int thin_reduce_splits(const ThinArgs& a) {
   return (int)(n < 1 ? 1 : n);
 }
 
-size_t thin_reduce_workspace_bytes(const ThinArgs& a) {
-  return (size_t)thin_reduce_splits(a) * a.J * a.cw * sizeof(float);
+size_t thin_reduce_workspace_bytes(const ThinArgs& a, bool with_thin_sums) {
+  return (size_t)thin_reduce_splits(a) * a.J * (a.cw + (with_thin_sums ? 1 : 0)) * sizeof(float);
+}
+
+bool thin_reduce_offers_thin_sums(const ThinArgs& a, int dtype) {
+  return (dtype == SFH_BF16 || dtype == SFH_FP16) && head_reduce_applies(a);
 }
 
 #define SFH_THIN_BY_DTYPE(fn, ...)                         \
@@ -966,8 +999,9 @@ int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt
 int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st) {
   SFH_THIN_BY_DTYPE(dispatch_thin_out, a, wide, wt, bias, out, st)
 }
-int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st) {
-  SFH_THIN_BY_DTYPE(dispatch_reduce, a, thin, wide, gw, gw_dtype, ws, st)
+int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st,
+                void* thin_sums) {
+  SFH_THIN_BY_DTYPE(dispatch_reduce, a, thin, wide, gw, gw_dtype, ws, st, thin_sums)
 }
 
 }  // namespace sfh

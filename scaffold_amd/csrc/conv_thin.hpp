@@ -33,7 +33,11 @@ int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt
 int thin_out(const ThinArgs& a, int dtype, const void* wide, const void* wt, const void* bias, void* out, hipStream_t st);
 // G[j][c] = sum_v s_j(v) * wide[v][c], through fp32 partial slices in `ws`
 int thin_reduce_splits(const ThinArgs& a);
-size_t thin_reduce_workspace_bytes(const ThinArgs& a);
-int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st);
+size_t thin_reduce_workspace_bytes(const ThinArgs& a, bool with_thin_sums = false);
+// `thin_sums` (optional, where thin_reduce_offers_thin_sums says so): also the J sums of the thin tensor over all voxels,
+// in gw's dtype, from the same pass (the bias gradient, when the thin tensor is the output gradient of a 1x1x1 convolution).
+bool thin_reduce_offers_thin_sums(const ThinArgs& a, int dtype);
+int thin_reduce(const ThinArgs& a, int dtype, const void* thin, const void* wide, void* gw, int gw_dtype, void* ws, hipStream_t st,
+                void* thin_sums = nullptr);
 
 }  // namespace sfh

@@ -172,6 +172,15 @@ class _Conv3dFn(torch.autograd.Function):
         if ctx.halo and grad_x is not None:
             grad_x = grad_x.narrow(2, ctx.halo, ctx.depth)
         grad_w = None
+        if needs_w and has_bias and needs_b:
+            # both parameter gradients from one pass over grad_output where the library offers it (the 1x1x1 head)
+            both = _c3.conv3d_backward_weight_bias(x, weight.shape, grad_output, stride, padding, dilation, 1,
+                                                   grad_dtype=torch.float32 if master else None, _checked=True)
+            if both is not None:
+                grad_w, grad_b = both
+                if grad_b.dtype is not bias_dtype:
+                    grad_b = grad_b.to(bias_dtype)
+                return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
         if needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight, x, weight.shape, grad_output, stride, padding, dilation, 1,

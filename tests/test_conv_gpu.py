@@ -790,3 +790,39 @@ def test_transposed_weight_and_bias_gradient_in_one_pass(device, dtype, n, cin, 
     x3 = torch.randn(1, 8, 4, 4, 4, device=device).to(dtype).contiguous(memory_format=torch.channels_last_3d)
     gy3 = torch.randn(1, 8, 8, 8, 8, device=device).to(dtype).contiguous(memory_format=torch.channels_last_3d)
     assert ct.conv_transpose3d_backward_weight_bias(x3, (8, 8, 2, 2, 2), gy3, 2, 0, 0, 1, 1) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,cin,cout,spatial", [(1, 32, 11, (8, 16, 32)), (2, 64, 5, (3, 5, 7)), (1, 128, 32, (4, 8, 9)), (1, 32, 1, (5, 6, 7))])
+def test_pointwise_weight_and_bias_gradient_in_one_pass(device, dtype, n, cin, cout, spatial):
+    """``conv3d_backward_weight_bias`` on the head's kind of problem (1x1x1, few output channels): the weight gradient is the
+    bits of ``conv3d_backward_weight``; the bias gradient is ``grad_output.sum((0, 2, 3, 4))``, exact on integer-valued
+    gradients and within an fp32 sum's round-off (plus one rounding to the output type) on Gaussian ones."""
+    from scaffold_amd import conv3d as c3
+
+    g = torch.Generator().manual_seed(78)
+    x = torch.randn((n, cin, *spatial), generator=g).to(dtype).contiguous(memory_format=torch.channels_last_3d).to(device)
+    wshape = (cout, cin, 1, 1, 1)
+    for exact in (True, False):
+        gy = (torch.randint(-2, 3, (n, cout, *spatial), generator=g) if exact else torch.randn((n, cout, *spatial), generator=g)).to(dtype)
+        gy = gy.contiguous(memory_format=torch.channels_last_3d).to(device)
+        for grad_dtype in (None, torch.float32):
+            both = c3.conv3d_backward_weight_bias(x, wshape, gy, 1, 0, 1, grad_dtype=grad_dtype)
+            assert both is not None
+            gw, gb = both
+            want_w = sa.conv3d_backward_weight(x, wshape, gy, 1, 0, 1, grad_dtype=grad_dtype)
+            assert gw.dtype is want_w.dtype and torch.equal(gw, want_w) and gw.stride() == want_w.stride()
+            ref = gy.double().sum((0, 2, 3, 4))
+            assert gb.dtype is gw.dtype and gb.shape == (cout,)
+            if exact:
+                if grad_dtype is torch.float32 or ref.abs().max() < 256:
+                    assert torch.equal(gb.double(), ref if grad_dtype is torch.float32 else ref.to(dtype).double())
+            else:
+                scale = (gy.double() ** 2).sum((0, 2, 3, 4)).sqrt()
+                tol = 2e-6 * scale + 1e-3 + (0 if grad_dtype is torch.float32 else 2.0 ** -8 * ref.abs())
+                assert ((gb.double() - ref).abs() <= tol).all()
+    # not offered: a 3x3x3 convolution, fp32 operands
+    x3 = torch.randn(1, 32, 4, 4, 8, device=device).to(dtype).contiguous(memory_format=torch.channels_last_3d)
+    gy3 = torch.randn(1, 32, 4, 4, 8, device=device).to(dtype).contiguous(memory_format=torch.channels_last_3d)
+    assert c3.conv3d_backward_weight_bias(x3, (32, 32, 3, 3, 3), gy3, 1, 1, 1) is None
+    assert c3.conv3d_backward_weight_bias(x3.float(), (11, 32, 1, 1, 1), gy3[:, :11].float().contiguous(memory_format=torch.channels_last_3d), 1, 0, 1) is None
