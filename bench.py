@@ -299,7 +299,7 @@ def bench_groupnorm(args, device):
 
         def abi_fwd_from_partials():
             _lib.check(L.sfh_groupnorm_fwd_from_partials(dref, BF16, BF16, FP32, P(yconv), P(gamma), P(beta), P(y), 0, P(mean), P(rstd),
-                                                         P(partials), records, None, None, stream), "sfh_groupnorm_fwd_from_partials")
+                                                         P(partials), partials.numel() * 4, records, stream), "sfh_groupnorm_fwd_from_partials")
 
         ms = event_time_ms(abi_fwd_from_partials, 20)
         from_producer = {"fwd_with_producer_statistics_ms": ms, "fwd_with_producer_statistics_bytes": 2 * B,

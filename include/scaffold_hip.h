@@ -77,7 +77,13 @@ typedef struct sfh_groupnorm_desc {
  * sfh_conv3d_fwd_gn, sfh_groupnorm_fwd_from_partials, sfh_tuned_compute_units added; nothing removed or changed.
  * 102: sfh_conv3d_pair_supported, sfh_conv3d_fwd_pair, sfh_conv3d_dgrad_pair, sfh_conv3d_wgrad_pair,
  * sfh_maxpool2_fwd_slab, sfh_convT3d_fwd_slab, sfh_convT3d_wgrad_bias(_workspace_bytes),
- * sfh_conv3d_wgrad_bias(_workspace_bytes) added. */
+ * sfh_conv3d_wgrad_bias(_workspace_bytes) added.
+ * 103: the GroupNorm statistics a convolution leaves are self-contained Welford records: sfh_conv3d_fwd_gn,
+ * sfh_conv3d_fwd_pair and sfh_groupnorm_fwd_from_partials lost their shift arguments (CHANGED signatures, and the record
+ * is 4 floats per group instead of 2), sfh_groupnorm_fwd_from_partials takes the byte size of the records;
+ * sfh_groupnorm_fwd_noalloc_prepare, sfh_mfma_ceiling_probe added. fp32 problems of the tiled shape have needed a
+ * workspace since 102 (sfh_conv3d_{fwd,dgrad,wgrad}_workspace_bytes are non-zero for them; callers that sized their
+ * workspace with those functions are unaffected). */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -126,14 +132,14 @@ int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const voi
 /* The forward that also leaves the GroupNorm statistics of its output, so that the normalisation after it
  * (unet_parts.py:123-160: every convolution of a DoubleConv is followed by GroupNorm + ReLU) does not read the tensor
  * a first time to find them: the reference's traffic model of GroupNorm (triton_group_norm.py:116, x read twice, y
- * written once) becomes one read and one write. The convolution's workgroups add up the ROUNDED values they store and
- * their squares, per group, in fp32, into gn_partials[N][records][2][groups] -- every slot written by exactly one
- * workgroup, no atomics, the same bits on every run; sfh_groupnorm_fwd_from_partials folds the records in a fixed
- * order. The values are summed minus a shift gn_shift[N][groups] (device memory; NULL = zeros) that the same pointer
- * hands to the GroupNorm call: any number near the group's mean -- the mean the layer had at its previous call is one --
- * keeps the variance from cancelling however large the mean is against the spread, which is what the reference's
- * Welford merge (triton_group_norm.py:148-165) is for; without one the variance carries a relative error of about
- * 3e-7 (mean/std)^2. sfh_conv3d_fwd_gn_records gives `records` for a problem and group count, a pure function of both; 0 means
+ * written once) becomes one read and one write. Every workgroup of the convolution leaves, per group, the Welford
+ * record { count, mean, M2, 0 } of the ROUNDED values it stored, gn_partials[N][records][groups][4] in fp32 -- every slot
+ * written by exactly one workgroup, no atomics, the same bits on every run -- and sfh_groupnorm_fwd_from_partials
+ * merges the records in a fixed order with the pairwise rule of the reference's tile statistics
+ * (triton_group_norm.py:148-165,594-607). A record is a function of the values it covers alone: inside a workgroup the
+ * sums are taken about one of its own outputs, so the variance does not cancel however large the mean is against the
+ * spread, nothing is carried from call to call and nothing comes from the caller.
+ * sfh_conv3d_fwd_gn_records gives `records` for a problem and group count, a pure function of both; 0 means
  * the kernel that serves the problem does not offer it (direct / fp32 / 2x2x2 kernels, thin-channel ones other than
  * the one-channel 3x3x3 stem, several samples on the persistent kernel, groups of fewer than 4 or a non-multiple-of-4
  * channels) and the caller uses sfh_conv3d_fwd and
@@ -141,8 +147,8 @@ int sfh_conv3d_fwd(const sfh_conv3d_desc* p, int dtype, const void* x, const voi
 int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype, int groups);
 int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w,
                       const int64_t w_stride[5], const void* bias, void* y, void* workspace,
-                      size_t workspace_bytes, uint32_t flags, int groups, const float* gn_shift,
-                      float* gn_partials, size_t gn_partials_bytes, void* stream);
+                      size_t workspace_bytes, uint32_t flags, int groups, float* gn_partials,
+                      size_t gn_partials_bytes, void* stream);
 
 /* ---- conv3d data gradient ------------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_backward_data (triton_conv3d/bwd_data.py:275).
@@ -213,13 +219,13 @@ int sfh_conv3d_wgrad(const sfh_conv3d_desc* p, int dtype, const void* x, const v
  * two tensors from the sum of its slices). A caller asks for all three before it drops its concatenation, and
  * concatenates otherwise.
  * sfh_conv3d_fwd_pair with groups > 0 also leaves the GroupNorm partials of sfh_conv3d_fwd_gn (same records, same
- * arguments); groups = 0 and NULL for the three gn arguments is the plain forward. Workspaces are those of the
+ * arguments); groups = 0 and NULL / 0 for the two gn arguments is the plain forward. Workspaces are those of the
  * ordinary entry points. SFH_FLAG_FORCE_GENERIC is refused. */
 int sfh_conv3d_pair_supported(const sfh_conv3d_desc* p, int dtype, int32_t cin_first, int direction);
 int sfh_conv3d_fwd_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second,
                         int32_t cin_first, const void* w, const int64_t w_stride[5], const void* bias, void* y,
                         void* workspace, size_t workspace_bytes, uint32_t flags, int groups,
-                        const float* gn_shift, float* gn_partials, size_t gn_partials_bytes, void* stream);
+                        float* gn_partials, size_t gn_partials_bytes, void* stream);
 int sfh_conv3d_dgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* gy, const void* w,
                           const int64_t w_stride[5], void* gx_first, void* gx_second, int32_t cin_first,
                           void* workspace, size_t workspace_bytes, uint32_t flags, void* stream);
@@ -293,27 +299,35 @@ int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype
                            const void* x, const void* gamma, const void* beta, void* y_slab,
                            int64_t halo_rows, float* mean, float* rstd, void* workspace,
                            size_t workspace_bytes, void* stream);
-/* The same again with the statistics taken from partial sums the producer of x left
- * (sfh_conv3d_fwd_gn): partials[N][records][2][groups], sums of x - shift and of its square per group, and the
- * shift[N][groups] they were taken about (NULL = zeros; must not be an output of this call). next_shift[N][groups]
- * (optional output) is what the producer should take its next call's sums about: a group's mean where it exceeds 16
- * standard deviations -- where plain sums would start to lose the variance -- and zero elsewhere, so that ordinary
- * tensors give the same bits call after call whatever was normalised before.
+/* The same again with the statistics merged from the Welford records the producer of x left (sfh_conv3d_fwd_gn):
+ * partials[N][records][groups][4] = { count, mean, M2, - } in fp32, 16-byte aligned, partials_bytes of them
+ * (SFH_ERR_WORKSPACE when that is less than N * records * groups * 16). The merge is the reference's
+ * (triton_group_norm.py:594-607) in fixed order; the result depends on the records alone.
  * No statistics pass and no workspace; halo_rows may be 0 (y_slab is then a plain output). Needs the vector path
  * (16-byte aligned tensors, channel counts the 16-byte vectors divide): SFH_ERR_UNSUPPORTED otherwise. */
 int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
                                     const void* x, const void* gamma, const void* beta, void* y_slab,
                                     int64_t halo_rows, float* mean, float* rstd, const float* partials,
-                                    int32_t records, const float* shift, float* next_shift, void* stream);
+                                    size_t partials_bytes, int32_t records, void* stream);
 
 /* The forward for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc. It has no counterpart in the reference. Same kernels and results as sfh_groupnorm_fwd, but the
  * scratch for the partial statistics is a device array inside the library (sfh_groupnorm_fwd_noalloc_max_bytes() =
  * 256 KiB, held by every GPU the library runs on until the process ends) instead of a workspace argument; neither this
- * call nor anything it calls allocates or frees memory. The tensors' device must be current. A problem whose scratch
- * exceeds the built-in buffer returns SFH_ERR_WORKSPACE (compare sfh_groupnorm_fwd_workspace_bytes with the maximum).
- * All calls on one GPU share the buffer: calls that overlap in time on one GPU (two streams) race. */
+ * call nor anything it calls allocates or frees memory. A problem whose scratch exceeds the built-in buffer returns
+ * SFH_ERR_WORKSPACE (compare sfh_groupnorm_fwd_workspace_bytes with the maximum).
+ * Device: the scratch used is the CURRENT device's copy of the array, not the copy of the device the pointers live
+ * on -- the call does not look at its pointers' device. The caller must therefore have made the tensors' device current
+ * (hipSetDevice / a device guard) before the call, exactly as for a kernel launch of its own; a call with another
+ * device current would hand the kernels a scratch address of the wrong GPU.
+ * Capture: the first call on a device looks the array's address up (once per device); that lookup must not run on a
+ * capturing stream, so a first call that finds `stream` capturing is refused with SFH_ERR_INVALID. Call
+ * sfh_groupnorm_fwd_noalloc_prepare() once per device, with that device current and before any capture, to do the lookup
+ * ahead of time (idempotent, allocates nothing). At most 64 devices (SFH_ERR_UNSUPPORTED beyond).
+ * All calls on one GPU share the buffer: calls that overlap in time on one GPU (two streams, or two captured graphs
+ * replayed on different streams) race. */
 size_t sfh_groupnorm_fwd_noalloc_max_bytes(void);
+int sfh_groupnorm_fwd_noalloc_prepare(void);
 int sfh_groupnorm_fwd_noalloc(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype,
                               const void* x, const void* gamma, const void* beta, void* y, float* mean,
                               float* rstd, void* stream);

@@ -114,7 +114,7 @@ _SIGNATURES = {
                                c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_fwd_gn_records": (c_int32, [POINTER(ConvDesc), c_int, c_int]),
     "sfh_conv3d_fwd_gn": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
-                                  c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                  c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_size_t, c_void_p]),
     "sfh_conv3d_dgrad_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_dgrad": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                  c_size_t, c_uint32, c_void_p]),
@@ -127,7 +127,7 @@ _SIGNATURES = {
                                  c_void_p]),
     "sfh_conv3d_pair_supported": (c_int, [POINTER(ConvDesc), c_int, c_int32, c_int]),
     "sfh_conv3d_fwd_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_int32, c_void_p, POINTER(c_int64), c_void_p,
-                                    c_void_p, c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                    c_void_p, c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_size_t, c_void_p]),
     "sfh_conv3d_dgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_int32,
                                       c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_wgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,
@@ -147,6 +147,7 @@ _SIGNATURES = {
     "sfh_groupnorm_fwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "sfh_groupnorm_fwd_noalloc_max_bytes": (c_size_t, []),
+    "sfh_groupnorm_fwd_noalloc_prepare": (c_int, []),
     "sfh_groupnorm_fwd_noalloc": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_void_p, c_void_p]),
     "sfh_shard_ingest": (c_int, [POINTER(IngestDesc), c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -155,7 +156,7 @@ _SIGNATURES = {
     "sfh_groupnorm_fwd_slab": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                        c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "sfh_groupnorm_fwd_from_partials": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
-                                                c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
+                                                c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_int32, c_void_p]),
     "sfh_groupnorm_bwd_workspace_bytes": (c_size_t, [POINTER(GroupNormDesc), c_int]),
     "sfh_groupnorm_bwd": (c_int, [POINTER(GroupNormDesc), c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

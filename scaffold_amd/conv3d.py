@@ -573,7 +573,6 @@ def conv3d_forward(
     force_generic: bool = False,
     packed_weight: Optional[torch.Tensor] = None,
     gn_groups: int = 0,
-    gn_shift: Optional[torch.Tensor] = None,
     _checked: bool = False,
     _second: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
@@ -585,11 +584,9 @@ def conv3d_forward(
     taps mirrored in all three axes (the data gradient's view of the weight).
 
     ``gn_groups > 0`` announces a GroupNorm of that many groups on the result: where the kernel that serves the problem
-    offers it, the launch also leaves the per-group sums of its (rounded) output, which ride along as
-    ``result._sfh_gn_partials`` and spare :func:`scaffold_amd.group_norm` its statistics pass. The result itself is the
-    same bits either way. ``gn_shift`` (fp32, ``(N, gn_groups)``, on the device) is what the values are summed about: any
-    number near each group's mean -- the means of the layer's previous call do -- keeps the variance exact at means far
-    larger than the spread; without it the sums are plain (fine up to a mean of some tens of standard deviations).
+    offers it, the launch also leaves per-group Welford records (count, mean, M2) of its rounded output, which ride along
+    as ``result._sfh_gn_partials`` and spare :func:`scaffold_amd.group_norm` its statistics pass. The result itself is the
+    same bits either way, and the records are a function of the result alone (no state from earlier calls).
     """
     if not _checked and not is_supported(x, w, bias, stride, padding, dilation, groups):
         raise NotImplementedError(
@@ -632,29 +629,26 @@ def conv3d_forward(
         ws = _lib.workspace(need, x.device)
         records = prob.gn_records(gn_groups) if gn_groups > 0 and not force_generic else 0
         if records > 0:
-            if gn_shift is not None and (gn_shift.dtype is not torch.float32 or gn_shift.shape != (prob.n, gn_groups)
-                                         or gn_shift.device != x.device or not gn_shift.is_contiguous()):
-                gn_shift = None  # not the shape of this call (another batch size, say): plain sums
-            partials = torch.empty(prob.n * records * 2 * gn_groups, dtype=torch.float32, device=x.device)
+            partials = torch.empty(prob.n * records * gn_groups * 4, dtype=torch.float32, device=x.device)
             if _second is None:
                 rc = L.sfh_conv3d_fwd_gn(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
                                          None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                          _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
-                                         _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+                                         _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
             else:
                 rc = L.sfh_conv3d_fwd_pair(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(_second), int(x.shape[1]), _lib.ptr(w_eff),
                                            None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
                                            _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, int(gn_groups),
-                                           _lib.ptr(gn_shift), _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
+                                           _lib.ptr(partials), partials.numel() * 4, _lib.stream_ptr(x.device))
             if rc == _lib.SFH_ERR_UNSUPPORTED:  # e.g. an out= view off the 16-byte grid: the plain launch
                 records = 0
             else:
                 # valid for these bits of y only: the version lets the consumer see an in-place change
-                y._sfh_gn_partials = (partials, records, int(gn_groups), y._version, gn_shift)
+                y._sfh_gn_partials = (partials, records, int(gn_groups), y._version)
         if records == 0 and _second is not None:
             rc = L.sfh_conv3d_fwd_pair(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(_second), int(x.shape[1]), _lib.ptr(w_eff),
                                        None if packed_weight is not None else _lib.strides5(w_eff), _lib.ptr(bias),
-                                       _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, 0, None, None, 0,
+                                       _lib.ptr(y), _lib.ptr(ws), 0 if ws is None else ws.numel(), flags, 0, None, 0,
                                        _lib.stream_ptr(x.device))
         elif records == 0:
             rc = L.sfh_conv3d_fwd(ctypes.byref(desc), code, _lib.ptr(x), _lib.ptr(w_eff),
@@ -924,15 +918,15 @@ def _refuse_pair(x_first, x_second, w):
 
 
 def conv3d_forward_pair(x_first, x_second, w, bias=None, stride=1, padding=0, dilation=1, *, packed_weight=None, gn_groups: int = 0,
-                        gn_shift=None, _checked: bool = False) -> torch.Tensor:
+                        _checked: bool = False) -> torch.Tensor:
     """``conv3d_forward(torch.cat([x_first, x_second], 1), w, ...)`` without the concatenation
     (``ScaFFold/unet/unet_parts.py:107-120`` writes that tensor for the decoder's first convolution): the kernel stages each
     32-channel chunk of its reduction from the tensor that holds it.  Same bits as the call on the concatenated tensor;
-    ``packed_weight`` / ``gn_groups`` / ``gn_shift`` as there.  ``NotImplementedError`` where :func:`is_supported_pair` says no."""
+    ``packed_weight`` / ``gn_groups`` as there.  ``NotImplementedError`` where :func:`is_supported_pair` says no."""
     if not _checked and not is_supported_pair(x_first, x_second, w, bias, stride, padding, dilation):
         _refuse_pair(x_first, x_second, w)
     return conv3d_forward(x_first, w, bias, stride, padding, dilation, 1, packed_weight=packed_weight, gn_groups=gn_groups,
-                          gn_shift=gn_shift, _checked=True, _second=x_second)
+                          _checked=True, _second=x_second)
 
 
 def conv3d_backward_data_pair(grad_output, weight, input_shape, cin_first: int, stride=1, padding=0, dilation=1, *,

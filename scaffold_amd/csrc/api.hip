@@ -90,6 +90,8 @@ bool fwd_uses_mfma(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return is_unit(p) && mfma_conv_supported(fwd_mfma_args(p, out), dtype);
 }
 // fp32 problems of the tiled shape run on the fp32 matrix pipe (the weight is packed per call into the workspace)
+bool on_16_bytes(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }  // null counts as aligned
+
 bool fwd_uses_f32_tiles(const sfh_conv3d_desc& p, int dtype, const int32_t out[3]) {
   return dtype == SFH_FP32 && is_unit(p) && f32_conv_supported(fwd_mfma_args(p, out));
 }
@@ -278,7 +280,7 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restric
 
 using namespace sfh;
 
-extern "C" int sfh_version(void) { return 102; }
+extern "C" int sfh_version(void) { return 103; }
 
 extern "C" const char* sfh_last_error(void) { return g_error; }
 
@@ -376,7 +378,9 @@ static int conv3d_fwd_any(const sfh_conv3d_desc* p, int dtype, const void* x, co
     t.ws_wide = w_stride[0]; t.ws_thin = w_stride[1];
     return thin_wide_out(t, dtype, x, w, bias, y, st, gn);
   }
-  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && fwd_uses_f32_tiles(*p, dtype, out)) {
+  // the fp32 tiles move 16-byte pieces of x, bias and y: a view 4 bytes off that grid runs the direct kernel instead
+  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && fwd_uses_f32_tiles(*p, dtype, out) && on_16_bytes(x) &&
+      on_16_bytes(y) && on_16_bytes(bias)) {
     const MfmaConvArgs a = fwd_mfma_args(*p, out);
     const size_t need = f32_conv_packed_weight_bytes(a);
     if (workspace == nullptr || workspace_bytes < need)
@@ -436,14 +440,14 @@ extern "C" int32_t sfh_conv3d_fwd_gn_records(const sfh_conv3d_desc* p, int dtype
 
 extern "C" int sfh_conv3d_fwd_gn(const sfh_conv3d_desc* p, int dtype, const void* x, const void* w, const int64_t w_stride[5],
                                  const void* bias, void* y, void* workspace, size_t workspace_bytes, uint32_t flags, int groups,
-                                 const float* gn_shift, float* gn_partials, size_t gn_partials_bytes, void* stream) {
+                                 float* gn_partials, size_t gn_partials_bytes, void* stream) {
   if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d fwd: the direct kernels leave no GroupNorm partials");
   const int32_t records = sfh_conv3d_fwd_gn_records(p, dtype, groups);
   if (records == 0) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd: GroupNorm partials are not offered for this problem");
-  const size_t need = (size_t)p->n * records * 2 * groups * sizeof(float);
+  const size_t need = (size_t)p->n * records * groups * kGnRecordFloats * sizeof(float);
   if (gn_partials == nullptr || gn_partials_bytes < need || (reinterpret_cast<uintptr_t>(gn_partials) & 15u) != 0)
     return fail(SFH_ERR_WORKSPACE, "conv3d fwd: GroupNorm partials need %zu bytes at a 16-byte boundary, got %zu", need, gn_partials_bytes);
-  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records, gn_shift};
+  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records};
   return conv3d_fwd_any(p, dtype, x, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, &gn);
 }
 
@@ -549,7 +553,8 @@ static int conv3d_dgrad_any(const sfh_conv3d_desc* p, int dtype, const void* gy,
     return mfma_conv_persist(a, dtype, gy, workspace, nullptr, gx, partial, st, nullptr, nullptr, out2);
   }
   if (out2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv3d dgrad: this problem does not write its result as two tensors");
-  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && dgrad_uses_f32_tiles(*p, dtype, out)) {
+  if (!(flags & (SFH_FLAG_FORCE_GENERIC | SFH_FLAG_WEIGHT_PACKED)) && dgrad_uses_f32_tiles(*p, dtype, out) && on_16_bytes(gy) &&
+      on_16_bytes(gx)) {
     const MfmaConvArgs a = dgrad_mfma_args(*p, out);
     const size_t need = f32_conv_packed_weight_bytes(a);
     if (workspace == nullptr || workspace_bytes < need)
@@ -712,7 +717,7 @@ extern "C" int sfh_conv3d_pair_supported(const sfh_conv3d_desc* p, int dtype, in
 
 extern "C" int sfh_conv3d_fwd_pair(const sfh_conv3d_desc* p, int dtype, const void* x_first, const void* x_second, int32_t cin_first,
                                    const void* w, const int64_t w_stride[5], const void* bias, void* y, void* workspace,
-                                   size_t workspace_bytes, uint32_t flags, int groups, const float* gn_shift, float* gn_partials,
+                                   size_t workspace_bytes, uint32_t flags, int groups, float* gn_partials,
                                    size_t gn_partials_bytes, void* stream) {
   if (x_second == nullptr) return fail(SFH_ERR_INVALID, "conv3d fwd pair: null tensor");
   if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d fwd pair: the direct kernels read one tensor");
@@ -722,11 +727,11 @@ extern "C" int sfh_conv3d_fwd_pair(const sfh_conv3d_desc* p, int dtype, const vo
   if (groups <= 0) return conv3d_fwd_any(p, dtype, x_first, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, nullptr, &in2);
   const int32_t records = sfh_conv3d_fwd_gn_records(p, dtype, groups);
   if (records == 0) return fail(SFH_ERR_UNSUPPORTED, "conv3d fwd pair: GroupNorm partials are not offered for this problem");
-  const size_t need = (size_t)p->n * records * 2 * groups * sizeof(float);
+  const size_t need = (size_t)p->n * records * groups * kGnRecordFloats * sizeof(float);
   if (gn_partials == nullptr || gn_partials_bytes < need || (reinterpret_cast<uintptr_t>(gn_partials) & 15u) != 0)
     return fail(SFH_ERR_WORKSPACE, "conv3d fwd pair: GroupNorm partials need %zu bytes at a 16-byte boundary, got %zu", need,
                 gn_partials_bytes);
-  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records, gn_shift};
+  const GnPartialOut gn{gn_partials, groups, p->cout / groups, records};
   return conv3d_fwd_any(p, dtype, x_first, w, w_stride, bias, y, workspace, workspace_bytes, flags, stream, &gn, &in2);
 }
 

@@ -236,7 +236,6 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 #pragma unroll
   for (int ns = 0; ns < C::NSUB; ++ns) {
     gn_sums[ns].clear();
-    if (gn.part != nullptr) gn_sums[ns].load_shift(gn.shift, n, gn.groups, gn.cg, (nb * C::NSUB + ns) * 32, kg);
   }
 
   // Epilogue. Accumulator register r of a lane is output channel 8*(r/4) + 4*kg + r%4 of the
@@ -280,7 +279,7 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
         run[g][0] = Mma32<T>::pack2(acc[ms][ns][4 * g] + b0, acc[ms][ns][4 * g + 1] + b1);
         run[g][1] = Mma32<T>::pack2(acc[ms][ns][4 * g + 2] + b2, acc[ms][ns][4 * g + 3] + b3);
       }
-      if (gn.part != nullptr) gn_sums[ns].template add<T>(run, inside);
+      if (gn.part != nullptr) gn_sums[ns].template add<T>(run, inside, ms == 0);
       uint4 piece[2];
       trade_channel_runs(run, piece);  // all lanes take part, also those of voxels past the edge
       if (inside) {
@@ -506,7 +505,7 @@ int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* pa
     return fail(SFH_ERR_UNSUPPORTED, "conv mfma: the output cannot be cut at channel %d of %d", out2->first, a.cout);
   const PairPtrs pr{in2 != nullptr ? in2->second : nullptr, (out2 != nullptr && p.ksplit == 1) ? out2->second : nullptr,
                     in2 != nullptr ? in2->first : (out2 != nullptr ? out2->first : 0)};
-  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
+  GnPartialOut out{nullptr, 0, 0, 0};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records != gather_gn_records(a, p, gn->groups) || gn->records == 0)
       return fail(SFH_ERR_INVALID, "conv mfma: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,
@@ -514,7 +513,7 @@ int launch_typed(const MfmaConvArgs& a, int dtype, const void* x, const void* pa
     out = *gn;
     out.cg = a.cout / gn->groups;
   }
-  const GnPartialOut none{nullptr, 0, 0, 0, nullptr};
+  const GnPartialOut none{nullptr, 0, 0, 0};
   const GnPartialOut& in_kernel = p.ksplit == 1 ? out : none;
   int rc;
   if (in2 != nullptr)

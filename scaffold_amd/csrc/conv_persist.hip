@@ -193,10 +193,13 @@ struct PendingStore {
   sfh_u32x4_t data[C::MS][2];
 };
 
-// With GN, the rounded values of the voxels inside the output are also added to the lane's GroupNorm sums.
+// With GN, the rounded values of the voxels inside the output are also added to the lane's GroupNorm sums. Their shift
+// is picked at the first brick whose first voxel of this wavefront lies inside the output (`have_shift`, wave-uniform):
+// a workgroup's run of bricks may start on one that a ragged edge cuts off from this wavefront.
 template <typename T, typename C, bool BIAS, bool GN>
 __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const float (&bias)[16], PendingStore<C>& ps,
-                                            const MfmaConvArgs& a, const TileCoord& tc, const LaneGeom<C>& lg, RunSums& sums) {
+                                            const MfmaConvArgs& a, const TileCoord& tc, const LaneGeom<C>& lg, RunSums& sums,
+                                            int& have_shift) {
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
     uint32_t run[4][2];
@@ -208,7 +211,15 @@ __device__ __forceinline__ void round_brick(const f32x16_t (&acc)[C::MS], const 
       run[g][0] = Mma32<T>::pack2(v[0], v[1]);
       run[g][1] = Mma32<T>::pack2(v[2], v[3]);
     }
-    if constexpr (GN) sums.template add<T>(run, store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]) != kRange);
+    if constexpr (GN) {
+      const bool inside = store_offset<C>(a, tc, lg.vcoord[ms], lg.vrel[ms]) != kRange;
+      bool first = false;
+      if (ms == 0 && !have_shift) {
+        first = __builtin_amdgcn_readfirstlane((int)inside) != 0;  // lane 0 holds the wavefront's first voxel of the brick
+        have_shift = first ? 1 : 0;
+      }
+      sums.template add<T>(run, inside, first);
+    }
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       // lanes 32-63 of run 2h <-> lanes 0-31 of run 2h+1
@@ -383,7 +394,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
   T* done_origin = yout;
   RunSums gn_sums;  // GroupNorm statistics of this workgroup's rounded outputs (GN)
   gn_sums.clear();
-  if constexpr (GN) gn_sums.load_shift(gn.shift, 0, gn.groups, gn.cg, nb * 32, kg);
+  int gn_have_shift = 0;
 
   for (int step = 0; step < nsteps; ++step) {
     const TileCoord tc2 = next_tile(tc1, gm);
@@ -393,7 +404,7 @@ conv_persist_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict
     if (step & 1) persist_step<T, C>(a, buf1, buf0, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
     else persist_step<T, C>(a, buf0, buf1, wave, lg, wq, wa, acc, ps, fetch_origin, voff, done_rsrc, done_off, tc2, live2, tc);
     asm volatile("s_nop 15\n\ts_nop 15");  // the last MFMAs are inline asm: the compiler does not know their result latency
-    round_brick<T, C, BIAS, GN>(acc, bias, ps, a, tc, lg, gn_sums);  // its stores ride along with the next step's MFMAs
+    round_brick<T, C, BIAS, GN>(acc, bias, ps, a, tc, lg, gn_sums, gn_have_shift);  // its stores ride along with the next step's MFMAs
     done_origin = tile_origin<T, C>(a, yout, tc, yrow, yc0);
     tc = tc1;
     tc1 = tc2;
@@ -509,7 +520,7 @@ int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const voi
   if (out2 != nullptr && (out2->second == nullptr || !mfma_conv_pair_ok(a, out2->first, true)))
     return fail(SFH_ERR_UNSUPPORTED, "conv persist: the output cannot be cut at channel %d of %d", out2->first, a.cout);
   const ChannelPair pair = out2 != nullptr ? *out2 : ChannelPair{nullptr, 0};
-  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
+  GnPartialOut out{nullptr, 0, 0, 0};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_gn_records(a, gn->groups))
       return fail(SFH_ERR_INVALID, "conv persist: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

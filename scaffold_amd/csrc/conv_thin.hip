@@ -656,7 +656,6 @@ __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const
 #pragma unroll
   for (int cc = 0; cc < NC; ++cc) {
     gn_sums[cc].clear();
-    if (gn.part != nullptr) gn_sums[cc].load_shift(gn.shift, t.n, gn.groups, gn.cg, cc * 32, kg);
   }
 #pragma unroll 1
   for (int i = 0; i < 4; ++i) {
@@ -685,12 +684,12 @@ __global__ void __launch_bounds__(kBlock) stem_fwd_mfma_kernel(ThinArgs a, const
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) acc = Mma32<T>::run(wf[cc][ks], xf[ks], acc);
-      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid, gn_sums[cc], gn.part != nullptr);
+      store_block_plus<T>(acc, dst + cc * 32, bv[cc], kg, valid, gn_sums[cc], gn.part != nullptr, i == 0);
     }
   }
   if (gn.part != nullptr) {
     __syncthreads();  // every wave is done reading the brick: the LDS is free
-    static_assert(sizeof(brick) >= (kBlock / 64) * NC * 16 * sizeof(float), "room for the wavefronts' sums");
+    static_assert(sizeof(brick) >= gn_partials_lds_floats(kBlock / 64, NC) * sizeof(float), "room for the wavefronts' sums");
     write_group_partials<kBlock / 64, NC>(gn_sums, reinterpret_cast<float*>(brick), gn, t.n,
                                           (int)(blockIdx.x % (unsigned)(tiles_d * tiles_h * tiles_w)), 0, tid);
   }
@@ -986,7 +985,7 @@ int thin_wide_out_gn_records(const ThinArgs& a, int dtype, int groups) {
 
 int thin_wide_out(const ThinArgs& a, int dtype, const void* thin, const void* wt, const void* bias, void* out, hipStream_t st,
                   const GnPartialOut* gn) {
-  GnPartialOut o{nullptr, 0, 0, 0, nullptr};
+  GnPartialOut o{nullptr, 0, 0, 0};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != thin_wide_out_gn_records(a, dtype, gn->groups))
       return fail(SFH_ERR_INVALID, "thin-channel conv: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

@@ -351,7 +351,6 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 #pragma unroll
   for (int ns = 0; ns < C::NSUB; ++ns) {
     gn_sums[ns].clear();
-    if (gn.part != nullptr) gn_sums[ns].load_shift(gn.shift, n, gn.groups, gn.cg, (nb * C::NSUB + ns) * 32, kg_out);
   }
 #pragma unroll
   for (int ms = 0; ms < C::MS; ++ms) {
@@ -362,8 +361,12 @@ conv_wide_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     const int64_t vox = (((int64_t)n * a.od + od) * a.oh + oh) * a.ow + ow;
     T* yp = y + vox * a.cout + nb * C::NSUB * 32;
 #pragma unroll
-    for (int ns = 0; ns < C::NSUB; ++ns)
-      store_block<T>(acc[ms][ns], yp + ns * 32, bias, (nb * C::NSUB + ns) * 32, kg_out, inside, gn_sums[ns], gn.part != nullptr);
+    for (int ns = 0; ns < C::NSUB; ++ns) {
+      store_block<T>(acc[ms][ns], yp + ns * 32, bias, (nb * C::NSUB + ns) * 32, kg_out, inside, gn_sums[ns], gn.part != nullptr, ms == 0);
+      // one block at a time: left to itself the scheduler reads many accumulator blocks out ahead of their stores and
+      // runs out of vector registers (all 256 accumulation registers are taken by the 8 x 2 grid)
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   if (gn.part != nullptr) {
     __syncthreads();  // every wave is done with the bricks: the LDS is free
@@ -487,7 +490,7 @@ int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* 
   if (in2 != nullptr && (in2->second == nullptr || !mfma_conv_wide_pair_ok(a, in2->first)))
     return fail(SFH_ERR_UNSUPPORTED, "conv wide: the input cannot be cut at channel %d of %d", in2->first, a.cred);
   const void* x1 = in2 != nullptr ? in2->second : nullptr;
-  GnPartialOut out{nullptr, 0, 0, 0, nullptr};
+  GnPartialOut out{nullptr, 0, 0, 0};
   if (gn != nullptr && gn->part != nullptr) {
     if (gn->records == 0 || gn->records != mfma_conv_wide_gn_records(a, gn->groups))
       return fail(SFH_ERR_INVALID, "conv wide: GroupNorm partials asked for %d records, this launch leaves %d", gn->records,

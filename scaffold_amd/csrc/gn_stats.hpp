@@ -1,25 +1,55 @@
-// GroupNorm statistics emitted by the kernel that produces the tensor: sums of the ROUNDED outputs (the bits the
-// normalisation will read back) minus a shift K, and of the squares of those differences, per group, one record per
-// producer workgroup:
-//   part[sample][record][2][G]      (the layout the GroupNorm kernels fold: quantity 0 = sum, 1 = sum of squares)
-// K[sample][group] comes from the caller -- any value near the group's mean, e.g. the mean the same layer had at its
-// previous call; a null pointer stands for zeros. With K within a few standard deviations of the mean the variance
-// S2/m - (S1/m)^2 does not cancel, however large the mean is against the spread (the job of the Welford merge in the
-// reference, triton_group_norm.py:148-165); with K = 0 the fp32 sums still carry a relative variance error of about
-// 3e-7 (mean/std)^2, below a bf16 output's own rounding up to |mean| = 100 std.
-// No atomics: every (record, group) slot is written by exactly one workgroup, the sums inside a workgroup are added in
-// a fixed order, and the GroupNorm kernels add the records in a fixed order, so the statistics are reproducible.
+// GroupNorm statistics emitted by the kernel that produces the tensor, as Welford records: for every group a producer
+// workgroup leaves (count, mean, M2) of the ROUNDED outputs it stored (the bits the normalisation will read back),
+//   part[sample][record][group][4] = { count, mean, M2 = sum (v - mean)^2, 0 }
+// and the GroupNorm kernels merge the records with the pairwise rule of Chan et al. in its k-way form (the merge of
+// the reference's tile statistics, ScaFFold/unet/triton_group_norm.py:148-165,594-607). Nothing is carried from one
+// call to the next and nothing comes from the caller: a record is a function of the values it covers alone.
+//
+// How a record stays accurate when the mean is large against the spread: sums are taken about a value of their own
+// data. Every wavefront sums v - K and (v - K)^2 with K = the first output it stored inside the tensor (per 4-channel
+// run), which is within a few standard deviations of the mean, so S2 - S1^2/n does not cancel; the wavefronts' sums
+// become (n, mean, M2) and are merged about the first one's mean, where the correction terms n d^2 are small again.
+// No atomics: every (record, group) slot is written by exactly one workgroup and every sum has a fixed order, so the
+// statistics are the same bits on every run.
 #pragma once
 #include "common.hpp"
 
 namespace sfh {
 
-// Where a producer writes, or nothing (part == nullptr). `records` per sample; `cg` channels per group; `shift` is
-// K[sample][group] or null.
+constexpr int kGnRecordFloats = 4;  // floats per (record, group)
+
+// Where a producer writes, or nothing (part == nullptr). `records` per sample; `cg` channels per group.
 struct GnPartialOut {
   float* part;
   int groups, cg, records;
-  const float* shift;
+};
+
+// (count, mean, M2) being merged from pieces in a fixed order. The first non-empty piece's mean is the reference point
+// c; a piece (n, mean, M2) adds n, n d and M2 + n d^2 with d = mean - c (sums about c of the piece's data, exactly what
+// the pairwise merge accumulates), and the total is mean = c + A / N, M2 = Q - A^2 / N.
+struct WelfordMerge {
+  float n, c, a, q;
+  __device__ __forceinline__ void clear() { n = c = a = q = 0.f; }
+  __device__ __forceinline__ void add(float pn, float pmean, float pm2) {
+    if (pn <= 0.f) return;
+    if (n == 0.f) c = pmean;
+    const float d = pmean - c;
+    n += pn;
+    a = fmaf(pn, d, a);
+    q += fmaf(pn * d, d, pm2);
+  }
+  // a piece given as sums about K: s1 = sum (v - K), s2 = sum (v - K)^2 over pn values
+  __device__ __forceinline__ void add_sums(float pn, float s1, float s2, float k) {
+    if (pn <= 0.f) return;
+    const float dm = s1 / pn;
+    const float m2 = fmaf(-s1, dm, s2);
+    add(pn, k + dm, m2 < 0.f ? 0.f : m2);
+  }
+  __device__ __forceinline__ float mean() const { return n > 0.f ? c + a / n : 0.f; }
+  __device__ __forceinline__ float m2() const {
+    const float v = n > 0.f ? fmaf(-a, a / n, q) : 0.f;
+    return v < 0.f ? 0.f : v;
+  }
 };
 
 __device__ __forceinline__ void unpack2(bf16_t, uint32_t u, float& lo, float& hi) {
@@ -31,22 +61,41 @@ __device__ __forceinline__ void unpack2(fp16_t, uint32_t u, float& lo, float& hi
   hi = fp16_hi(u);
 }
 
+__device__ __forceinline__ int lane_index() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
 // Sums of the four channel runs a lane holds of a 32-channel result block (run g = channels 8g + 4kg .. + 3, packed
-// as two rounded pairs), over the voxels the lane has added so far; k[g] is the shift of run g's group.
+// as two rounded pairs), over the voxels the lane has added so far, about k[g]: the first channel of run g at the
+// wavefront's first voxel (the same value in all 32 lanes that hold the run). In every kernel that uses this, a
+// wavefront's first voxel -- lane 0 of its first 32-voxel piece -- has the smallest coordinates of all its voxels, so it
+// lies inside the tensor whenever any of them does: the shift is then one of the values summed. (A wavefront wholly past
+// a ragged edge counts nothing, whatever its shift.)
 struct RunSums {
   float s1[4], s2[4], k[4];
+  float cnt;  // voxels of this lane counted so far
   __device__ __forceinline__ void clear() {
 #pragma unroll
     for (int g = 0; g < 4; ++g) s1[g] = s2[g] = k[g] = 0.f;
+    cnt = 0.f;
   }
-  // The shifts of the block whose first channel is c0 (a multiple of 32), for the lane's k-half kg and sample n.
-  __device__ __forceinline__ void load_shift(const float* shift, int n, int groups, int cg, int c0, int kg) {
-    if (shift == nullptr) return;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) k[g] = shift[n * groups + (c0 + 8 * g + 4 * kg) / cg];
-  }
+  // Takes the shift from the wavefront's first voxel: `run` is the first piece the wavefront adds. All 64 lanes must
+  // call it.
   template <typename T>
-  __device__ __forceinline__ void add(const uint32_t (&run)[4][2], bool inside) {
+  __device__ __forceinline__ void pick_shift(const uint32_t (&run)[4][2]) {
+    const bool upper = (lane_index() & 32) != 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      // lane 0 holds the run for k-half 0, lane 32 for k-half 1
+      const uint32_t v0 = (uint32_t)__builtin_amdgcn_readlane((int)run[g][0], 0);
+      const uint32_t v1 = (uint32_t)__builtin_amdgcn_readlane((int)run[g][0], 32);
+      float lo, hi;
+      unpack2(T{}, upper ? v1 : v0, lo, hi);
+      k[g] = lo;
+    }
+  }
+  // `inside`: the lane's voxel lies inside the tensor; `first`: nothing has been added yet (then the shift is picked).
+  template <typename T>
+  __device__ __forceinline__ void add(const uint32_t (&run)[4][2], bool inside, bool first) {
+    if (first) pick_shift<T>(run);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       float a, b, c, d;
@@ -58,6 +107,7 @@ struct RunSums {
       s1[g] += inside ? t1 : 0.f;  // a voxel past the ragged edge counts as nothing
       s2[g] += inside ? t2 : 0.f;
     }
+    cnt += inside ? 1.f : 0.f;
   }
 };
 
@@ -69,37 +119,44 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return v;
 }
 
+// Floats of LDS write_group_partials needs.
+constexpr int gn_partials_lds_floats(int nw, int nsub) { return nw * nsub * 8 * 4; }
+
 // Workgroup of NW wavefronts, each lane with NSUB RunSums (result blocks ns = 0 .. NSUB-1 of the workgroup's channel
-// span, which starts at global channel c0): folds them per group and writes the workgroup's slots of record `rec` of
-// sample n. `lds` needs NW * NSUB * 16 floats and must be free for writing (the caller has synchronised). A group wider
-// than the span (cg > 32 * NSUB) is completed by the other workgroups of the same tile, each in a record of its own.
+// span, which starts at global channel c0): merges them per group and writes the workgroup's slots of record `rec` of
+// sample n. `lds` needs gn_partials_lds_floats(NW, NSUB) floats and must be free for writing (the caller has
+// synchronised). A group wider than the span (cg > 32 * NSUB) is completed by the other workgroups of the same tile,
+// each in a record of its own.
 template <int NW, int NSUB>
 __device__ __forceinline__ void write_group_partials(const RunSums (&rs)[NSUB], float* lds, const GnPartialOut& o, int n, int rec, int c0,
                                                      int tid) {
   const int lane = tid & 63, wave = tid >> 6, kg = lane >> 5;
-  // lds[wave][ns][run r = 2g + kg][q]
+  // lds[wave][ns][run r = 2g + kg] = { values, sum, sum of squares, shift }
 #pragma unroll
-  for (int ns = 0; ns < NSUB; ++ns)
+  for (int ns = 0; ns < NSUB; ++ns) {
+    const float voxels = half_wave_sum(rs[ns].cnt);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const float t1 = half_wave_sum(rs[ns].s1[g]), t2 = half_wave_sum(rs[ns].s2[g]);
-      if ((lane & 31) == 0) {
-        float* dst = lds + ((wave * NSUB + ns) * 8 + 2 * g + kg) * 2;
-        dst[0] = t1;
-        dst[1] = t2;
-      }
+      if ((lane & 31) == 0)
+        *reinterpret_cast<float4*>(lds + ((wave * NSUB + ns) * 8 + 2 * g + kg) * 4) = make_float4(4.f * voxels, t1, t2, rs[ns].k[g]);
     }
+  }
   __syncthreads();
   const int span = 32 * NSUB;
   const int runs_per_group = (o.cg < span ? o.cg : span) / 4;
   const int ngroups = span / (runs_per_group * 4);
-  if (tid < 2 * ngroups) {
-    const int q = tid & 1, gl = tid >> 1;
-    float t = 0.f;
+  if (tid < ngroups) {
+    WelfordMerge m;
+    m.clear();
     for (int w = 0; w < NW; ++w)
-      for (int r = 0; r < runs_per_group; ++r) t += lds[((w * (NSUB * 8)) + gl * runs_per_group + r) * 2 + q];
-    const int group = (c0 + gl * runs_per_group * 4) / o.cg;
-    o.part[(((int64_t)n * o.records + rec) * 2 + q) * o.groups + group] = t;
+      for (int r = 0; r < runs_per_group; ++r) {
+        const float4 e = *reinterpret_cast<const float4*>(lds + (w * (NSUB * 8) + tid * runs_per_group + r) * 4);
+        m.add_sums(e.x, e.y, e.z, e.w);
+      }
+    const int group = (c0 + tid * runs_per_group * 4) / o.cg;
+    *reinterpret_cast<float4*>(o.part + (((int64_t)n * o.records + rec) * o.groups + group) * kGnRecordFloats) =
+        make_float4(m.n, m.mean(), m.m2(), 0.f);
   }
 }
 

@@ -25,6 +25,7 @@
 #include <mutex>
 
 #include "common.hpp"
+#include "gn_stats.hpp"
 #include "vec_io.hpp"
 
 // No implicit mul+add contraction in this file: every FMA is written as fmaf(). The forward and the
@@ -223,17 +224,10 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
 }
 
 // One workgroup per (group, sample): fixed-order sum of the split partials, then
-// mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps). A null `shift` stands for K = 0 (partials that
-// the producer of x summed unshifted).
-// The shift a producer of x should take its NEXT call's sums about, given this call's statistics: the mean where it
-// is large against the spread (there plain sums would cancel), else zero -- so that ordinary tensors give the same bits
-// call after call, whatever the history.
-constexpr float kShiftFromRatio = 16.f;
-__device__ __forceinline__ float next_shift_of(float mu, float rs) { return fabsf(mu) * rs > kShiftFromRatio ? mu : 0.f; }
-
+// mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps).
 __global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restrict__ shift, const float* __restrict__ part,
                                                             float* __restrict__ mean, float* __restrict__ rstd, int G, int nsplit,
-                                                            float m, float eps, float* __restrict__ next_shift) {
+                                                            float m, float eps) {
   __shared__ float wsum[kBlock / 64][2];
   const int g = blockIdx.x, n = blockIdx.y, tid = threadIdx.x;
   const float* base = part + (int64_t)n * nsplit * 2 * G + g;
@@ -267,10 +261,54 @@ __global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restr
     const float d = s1 / m;
     float var = s2 / m - d * d;
     var = var < 0.f ? 0.f : var;
-    const float mu = (shift != nullptr ? shift[n * G + g] : 0.f) + d, rs = 1.f / sqrtf(var + eps);
+    const float mu = shift[n * G + g] + d, rs = 1.f / sqrtf(var + eps);
     mean[n * G + g] = mu;
     rstd[n * G + g] = rs;
-    if (next_shift != nullptr) next_shift[n * G + g] = next_shift_of(mu, rs);
+  }
+}
+
+// The same for Welford records a producer of x left, rec[sample][record][group] = { count, mean, M2, - } (gn_stats.hpp):
+// merged about the first record's mean c. A record adds n, n d and M2 + n d^2 with d = mean - c, which are the sums
+// about c of the values it covers; then mean = c + A/m, var = (Q - A^2/m)/m. Fixed order: thread t owns the records
+// t, t + 256, ..., the threads are added by wavefront, the wavefronts in order.
+__global__ void __launch_bounds__(kBlock) gn_welford_finalize(const float* __restrict__ rec, float* __restrict__ mean,
+                                                              float* __restrict__ rstd, int G, int nrec, float m, float eps) {
+  __shared__ float wsum[kBlock / 64][2];
+  const int g = blockIdx.x, n = blockIdx.y, tid = threadIdx.x;
+  const float4* base = reinterpret_cast<const float4*>(rec) + (int64_t)n * nrec * G + g;
+  const float c = base[0].y;
+  float a = 0.f, q = 0.f;
+  int i = tid;
+  for (; i + 7 * kBlock < nrec; i += 8 * kBlock) {
+    float4 e[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) e[u] = base[(int64_t)(i + u * kBlock) * G];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float d = e[u].y - c;
+      a = fmaf(e[u].x, d, a);
+      q += fmaf(e[u].x * d, d, e[u].z);
+    }
+  }
+  for (; i < nrec; i += kBlock) {
+    const float4 e = base[(int64_t)i * G];
+    const float d = e.y - c;
+    a = fmaf(e.x, d, a);
+    q += fmaf(e.x * d, d, e.z);
+  }
+  a = wave_sum(a);
+  q = wave_sum(q);
+  if ((tid & 63) == 0) { wsum[tid >> 6][0] = a; wsum[tid >> 6][1] = q; }
+  __syncthreads();
+  if (tid == 0) {
+    a = q = 0.f;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) { a += wsum[w][0]; q += wsum[w][1]; }
+    const float d = a / m;
+    float var = fmaf(-a, d, q) / m;
+    var = var < 0.f ? 0.f : var;
+    mean[n * G + g] = c + d;
+    rstd[n * G + g] = 1.f / sqrtf(var + eps);
   }
 }
 
@@ -282,14 +320,11 @@ __global__ void __launch_bounds__(kBlock) gn_stats_finalize(const float* __restr
 // total of column c (quantity c / G, group c % G) and passes it to emit(c, total).
 constexpr int kFoldFloats = 16384;
 
-__device__ __forceinline__ bool fold_in_consumer(int G, int nsplit) {
-  const int cols = 2 * G;
+__host__ __device__ __forceinline__ bool fold_in_consumer(int G, int nsplit, int per_group = 2) {
+  const int cols = per_group * G;
   return cols >= 4 && cols <= 64 && (cols & (cols - 1)) == 0 && (int64_t)nsplit * cols <= kFoldFloats;
 }
-inline bool fold_in_consumer_host(int G, int nsplit) {
-  const int cols = 2 * G;
-  return cols >= 4 && cols <= 64 && (cols & (cols - 1)) == 0 && (int64_t)nsplit * cols <= kFoldFloats;
-}
+inline bool fold_in_consumer_host(int G, int nsplit, int per_group = 2) { return fold_in_consumer(G, nsplit, per_group); }
 
 template <typename Emit>
 __device__ __forceinline__ void fold_split_partials(const float* __restrict__ rows, int G, int nsplit, float* lds /* 4 * kBlock */,
@@ -318,6 +353,40 @@ __device__ __forceinline__ void fold_split_partials(const float* __restrict__ ro
   }
 }
 
+// The same inside a consumer for a producer's Welford records rec[record][group] = { count, mean, M2, - } of one sample
+// (G a power of two, nrec * 4 G <= kFoldFloats): a thread's pieces t, t + 256, ... all belong to group t % G; it
+// merges them about the first record's mean c (see gn_welford_finalize), the threads of a group are added in thread
+// order. Thread g < G passes its group's (c, A, Q) to emit.
+template <typename Emit>
+__device__ __forceinline__ void fold_welford_records(const float* __restrict__ rec, int G, int nrec, float* lds /* 4 * kBlock */,
+                                                     Emit emit) {
+  const int tid = threadIdx.x;
+  const int total = nrec * G;
+  constexpr int NB = kFoldFloats / (4 * kBlock);
+  const float c = rec[(tid & (G - 1)) * kGnRecordFloats + 1];
+  float4 v[NB];
+#pragma unroll
+  for (int k = 0; k < NB; ++k) {
+    const int i = tid + k * kBlock;
+    v[k] = i < total ? *reinterpret_cast<const float4*>(rec + (int64_t)i * kGnRecordFloats) : make_float4(0.f, c, 0.f, 0.f);
+  }
+  float a = 0.f, q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NB; ++k) {
+    const float d = v[k].y - c;
+    a = fmaf(v[k].x, d, a);
+    q += fmaf(v[k].x * d, d, v[k].z);
+  }
+  lds[2 * tid] = a;
+  lds[2 * tid + 1] = q;
+  __syncthreads();
+  if (tid < G) {
+    float ta = 0.f, tq = 0.f;
+    for (int t = tid; t < kBlock; t += G) { ta += lds[2 * t]; tq += lds[2 * t + 1]; }
+    emit(tid, c, ta, tq);
+  }
+}
+
 // ---- forward: normalise + affine (+ReLU) (vector path) ------------------------------------
 // When the sample's split partials are few (fold_in_consumer), every workgroup derives mean and rstd from them itself
 // (mean = K + S1/m, var = S2/m - (S1/m)^2, rstd = 1/sqrt(var + eps)): 32 KiB from L2 cost less than a launch of their
@@ -328,7 +397,7 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
                                                        float* __restrict__ rstd, const void* __restrict__ gamma,
                                                        const void* __restrict__ beta, int param_dtype, int64_t S, int C, int G,
                                                        int tpr, int rpp, int nsplit, int64_t rows_per_split, float m, float eps,
-                                                       int relu, int64_t y_halo, int npart, float* __restrict__ next_shift) {
+                                                       int relu, int64_t y_halo, int npart, int welford) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float gstat[];  // sums[2 G] | mean[G] | rstd[G] | fold scratch (4 * kBlock)
   const int tid = threadIdx.x;
@@ -337,22 +406,34 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   const int r = tid / tpr, cv = tid - r * tpr;
   float* g_mean = gstat + 2 * G;
   float* g_rstd = gstat + 3 * G;
-  // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid), or the ones the
-  // producer of x left (then without a shift)
-  if (fold_in_consumer(G, npart)) {
+  // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid, sums about the
+  // common shift), or (`welford`) the records the producer of x left
+  if (welford && fold_in_consumer(G, npart, kGnRecordFloats)) {
+    fold_welford_records(part + (int64_t)n * npart * G * kGnRecordFloats, G, npart, gstat + 4 * G, [&](int g, float c, float a, float q) {
+      const float d = a / m;
+      float var = fmaf(-a, d, q) / m;
+      var = var < 0.f ? 0.f : var;
+      const float mu_g = c + d, rs_g = 1.f / sqrtf(var + eps);
+      g_mean[g] = mu_g;
+      g_rstd[g] = rs_g;
+      if (blockIdx.x == 0) {  // for the backward pass
+        mean[n * G + g] = mu_g;
+        rstd[n * G + g] = rs_g;
+      }
+    });
+  } else if (!welford && fold_in_consumer(G, npart)) {
     fold_split_partials(part + (int64_t)n * npart * 2 * G, G, npart, gstat + 4 * G, [&](int c, float t) { gstat[c] = t; });
     __syncthreads();
     if (tid < G) {
       const float d = gstat[tid] / m;
       float var = gstat[G + tid] / m - d * d;
       var = var < 0.f ? 0.f : var;
-      const float mu_g = (shift != nullptr ? shift[n * G + tid] : 0.f) + d, rs_g = 1.f / sqrtf(var + eps);
+      const float mu_g = shift[n * G + tid] + d, rs_g = 1.f / sqrtf(var + eps);
       g_mean[tid] = mu_g;
       g_rstd[tid] = rs_g;
       if (blockIdx.x == 0) {  // for the backward pass
         mean[n * G + tid] = mu_g;
         rstd[n * G + tid] = rs_g;
-        if (next_shift != nullptr) next_shift[n * G + tid] = next_shift_of(mu_g, rs_g);
       }
     }
   } else {
@@ -867,14 +948,14 @@ size_t bwd_ws_floats(const sfh_groupnorm_desc& p, const GnPlan& pl) {
 
 template <typename T, typename TO>
 int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, const void* x, const void* gamma, const void* beta,
-              void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st, const float* given_part = nullptr,
-              int given_npart = 0, const float* given_shift = nullptr, float* next_shift = nullptr) {
+              void* y, int64_t y_halo, float* mean, float* rstd, float* ws, hipStream_t st, const float* given_records = nullptr,
+              int given_nrec = 0) {
   const int G = p.groups, C = p.c;
   const int64_t S = p.spatial;
   if (y_halo > 0 && (!pl.vector || sizeof(T) != sizeof(TO) || (y_halo * C * sizeof(TO)) % 16 != 0))
     return fail(SFH_ERR_UNSUPPORTED, "groupnorm: the slab output needs the vector path and an output of the input's width");
   if (!pl.vector) {
-    if (given_part != nullptr) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: statistics from given partials need the vector path");
+    if (given_records != nullptr) return fail(SFH_ERR_UNSUPPORTED, "groupnorm: statistics from given records need the vector path");
     hipLaunchKernelGGL(gn_scalar_stats<T>, dim3(G, p.n), dim3(kBlock), 0, st, (const T*)x, mean, rstd, S, C, G, p.eps);
     if (int rc = check_launch("gn_scalar_stats")) return rc;
     const int64_t total = (int64_t)p.n * S * C;
@@ -884,10 +965,11 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
     return check_launch("gn_scalar_normalize");
   }
   const dim3 grid(pl.nsplit, p.n);
-  const float* shift = given_shift;  // of the given partials (null: zeros)
-  const float* part = given_part;
-  int npart = given_npart;
-  if (given_part == nullptr) {
+  const float* shift = nullptr;
+  const float* part = given_records;  // Welford records of x's producer, or this call's own shifted sums
+  int npart = given_nrec;
+  const int welford = given_records != nullptr ? 1 : 0;
+  if (given_records == nullptr) {
     float* my_shift = ws;
     float* my_part = ws + align_up((size_t)p.n * G, 4);
     const size_t lds = (size_t)(2 * pl.slots * kBlock + 2 * G) * sizeof(float);
@@ -905,13 +987,18 @@ int fwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
     shift = my_shift; part = my_part; npart = pl.nsplit;
   }
   const float m = (float)S * (float)(C / G);
-  if (!fold_in_consumer_host(G, npart)) {
-    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(kBlock), 0, st, shift, part, mean, rstd, G, npart, m, p.eps, next_shift);
+  if (welford) {
+    if (!fold_in_consumer_host(G, npart, kGnRecordFloats)) {
+      hipLaunchKernelGGL(gn_welford_finalize, dim3(G, p.n), dim3(kBlock), 0, st, part, mean, rstd, G, npart, m, p.eps);
+      if (int rc = check_launch("gn_welford_finalize")) return rc;
+    }
+  } else if (!fold_in_consumer_host(G, npart)) {
+    hipLaunchKernelGGL(gn_stats_finalize, dim3(G, p.n), dim3(kBlock), 0, st, shift, part, mean, rstd, G, npart, m, p.eps);
     if (int rc = check_launch("gn_stats_finalize")) return rc;
   }
   hipLaunchKernelGGL((gn_normalize<T, TO>), grid, dim3(kBlock), (size_t)(4 * G + 4 * kBlock) * sizeof(float), st, (const T*)x, (TO*)y, shift, part,
                      mean, rstd, gamma, beta, param_dtype, S, C, G, pl.tpr, pl.rpp, pl.nsplit, pl.rows_per_split, m, p.eps, p.relu, y_halo,
-                     npart, next_shift);
+                     npart, welford);
   return check_launch("gn_normalize");
 }
 
@@ -970,14 +1057,13 @@ extern "C" size_t sfh_groupnorm_fwd_workspace_bytes(const sfh_groupnorm_desc* p,
 
 static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x, const void* gamma,
                              const void* beta, void* y, int64_t y_halo, float* mean, float* rstd, void* workspace,
-                             size_t workspace_bytes, void* stream, const float* given_part = nullptr, int given_npart = 0,
-                             const float* given_shift = nullptr, float* next_shift = nullptr) {
+                             size_t workspace_bytes, void* stream, const float* given_records = nullptr, int given_nrec = 0) {
   if (int rc = check_desc(p, x_dtype)) return rc;
   if (!dtype_ok(y_dtype) || !dtype_ok(param_dtype)) return fail(SFH_ERR_INVALID, "groupnorm: bad output/param dtype");
   if (x == nullptr || y == nullptr || mean == nullptr || rstd == nullptr) return fail(SFH_ERR_INVALID, "groupnorm: null tensor");
   if (y_halo < 0) return fail(SFH_ERR_INVALID, "groupnorm: negative halo");
   const GnPlan pl = make_plan(*p, x_dtype, aligned16(x) && aligned16(y));
-  if (pl.vector && given_part == nullptr) {
+  if (pl.vector && given_records == nullptr) {
     const size_t need = fwd_ws_floats(*p, pl) * sizeof(float);
     if (workspace == nullptr || workspace_bytes < need)
       return fail(SFH_ERR_WORKSPACE, "groupnorm fwd: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
@@ -985,8 +1071,7 @@ static int groupnorm_fwd_any(const sfh_groupnorm_desc* p, int x_dtype, int y_dty
   hipStream_t st = (hipStream_t)stream;
   float* ws = (float*)workspace;
 #define SFH_GN_FWD(TX, TY) \
-  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_part, given_npart, given_shift, \
-                           next_shift)
+  return fwd_typed<TX, TY>(*p, pl, param_dtype, x, gamma, beta, y, y_halo, mean, rstd, ws, st, given_records, given_nrec)
   if (x_dtype == SFH_BF16 && y_dtype == SFH_BF16) SFH_GN_FWD(bf16_t, bf16_t);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP32) SFH_GN_FWD(bf16_t, float);
   if (x_dtype == SFH_BF16 && y_dtype == SFH_FP16) SFH_GN_FWD(bf16_t, fp16_t);
@@ -1014,12 +1099,16 @@ extern "C" int sfh_groupnorm_fwd_slab(const sfh_groupnorm_desc* p, int x_dtype, 
 
 extern "C" int sfh_groupnorm_fwd_from_partials(const sfh_groupnorm_desc* p, int x_dtype, int y_dtype, int param_dtype, const void* x,
                                                const void* gamma, const void* beta, void* y_slab, int64_t halo_rows, float* mean,
-                                               float* rstd, const float* partials, int32_t records, const float* shift,
-                                               float* next_shift, void* stream) {
-  if (partials == nullptr || records < 1) return fail(SFH_ERR_INVALID, "groupnorm from partials: no partial sums given");
-  if (!aligned16(partials)) return fail(SFH_ERR_INVALID, "groupnorm from partials: the partial sums must be 16-byte aligned");
+                                               float* rstd, const float* partials, size_t partials_bytes, int32_t records,
+                                               void* stream) {
+  if (int rc = check_desc(p, x_dtype)) return rc;
+  if (partials == nullptr || records < 1) return fail(SFH_ERR_INVALID, "groupnorm from partials: no records given");
+  if (!aligned16(partials)) return fail(SFH_ERR_INVALID, "groupnorm from partials: the records must be 16-byte aligned");
+  const size_t need = (size_t)p->n * records * p->groups * kGnRecordFloats * sizeof(float);
+  if (partials_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "groupnorm from partials: %d records per sample are %zu bytes, got %zu", records, need, partials_bytes);
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y_slab, halo_rows, mean, rstd, nullptr, 0, stream, partials,
-                           records, shift, next_shift);
+                           records);
 }
 
 // ---- the forward for callers that may not allocate ------------------------------------------------------------------
@@ -1037,12 +1126,19 @@ std::mutex g_noalloc_mutex;
 float* g_noalloc_ptr[kMaxDevices];  // device address of the array on each device (null: not looked up yet)
 
 // Device address of the scratch array on the CURRENT device. The array's name is a host-side handle, not an address a
-// kernel could use: the address comes from hipGetSymbolAddress, per device.
-int noalloc_scratch(float** out) {
+// kernel could use: the address comes from hipGetSymbolAddress, per device. The first lookup on a device may load the
+// code object, so it must not happen while `st` is capturing: such a call is refused (prepare first).
+int noalloc_scratch(float** out, hipStream_t st, bool may_look_up) {
   int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(SFH_ERR_LAUNCH, "groupnorm: no current device");
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return fail(SFH_ERR_LAUNCH, "groupnorm (no-alloc): no current device");
+  if (dev >= kMaxDevices)
+    return fail(SFH_ERR_UNSUPPORTED, "groupnorm (no-alloc): device %d is beyond the %d devices the scratch table holds", dev, kMaxDevices);
   std::lock_guard<std::mutex> lock(g_noalloc_mutex);
   if (g_noalloc_ptr[dev] == nullptr) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (!may_look_up || hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone)
+      return fail(SFH_ERR_INVALID, "groupnorm (no-alloc): the first call on device %d arrived on a capturing stream; call "
+                  "sfh_groupnorm_fwd_noalloc_prepare() on the device before the capture", dev);
     void* ptr = nullptr;
     const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_gn_noalloc_scratch));
     if (err != hipSuccess || ptr == nullptr)
@@ -1053,6 +1149,11 @@ int noalloc_scratch(float** out) {
   return SFH_OK;
 }
 }  // namespace
+
+extern "C" int sfh_groupnorm_fwd_noalloc_prepare(void) {
+  float* unused = nullptr;
+  return noalloc_scratch(&unused, nullptr, true);
+}
 
 extern "C" size_t sfh_groupnorm_fwd_noalloc_max_bytes(void) { return kNoAllocScratchFloats * sizeof(float); }
 
@@ -1065,7 +1166,7 @@ extern "C" int sfh_groupnorm_fwd_noalloc(const sfh_groupnorm_desc* p, int x_dtyp
     return fail(SFH_ERR_WORKSPACE, "groupnorm fwd (no-alloc): this problem needs %zu bytes of scratch, the built-in buffer holds %zu; "
                 "use sfh_groupnorm_fwd with a workspace", need, kNoAllocScratchFloats * sizeof(float));
   float* scratch = nullptr;
-  if (int rc = noalloc_scratch(&scratch)) return rc;
+  if (int rc = noalloc_scratch(&scratch, (hipStream_t)stream, true)) return rc;
   return groupnorm_fwd_any(p, x_dtype, y_dtype, param_dtype, x, gamma, beta, y, 0, mean, rstd, scratch,
                            kNoAllocScratchFloats * sizeof(float), stream);
 }

@@ -59,17 +59,18 @@ __device__ __forceinline__ uint4 load16(const T* p) { return *reinterpret_cast<c
 // this lane is channel 8 * (r / 4) + 4 * kg + r % 4): this lane's voxel row starts at `row` (element pointer at
 // channel 0 of the block). The two lanes of a voxel trade channel runs first, so each stores two 16-byte pieces.
 // All 64 lanes must call it; `valid` masks the stores.
-// With `want`, the block's rounded values are also added to the lane's GroupNorm sums (valid voxels only).
+// With `want`, the block's rounded values are also added to the lane's GroupNorm sums (valid voxels only); `first`: it
+// is the first block added to `sums`.
 template <typename T>
 __device__ __forceinline__ void store_block_plus(const f32x16_t& acc, T* row, const float (&add)[16], int kg, bool valid,
-                                                 RunSums& sums, bool want) {
+                                                 RunSums& sums, bool want, bool first) {
   uint32_t run[4][2];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
     run[g][0] = Mma32<T>::pack2(acc[4 * g] + add[4 * g], acc[4 * g + 1] + add[4 * g + 1]);
     run[g][1] = Mma32<T>::pack2(acc[4 * g + 2] + add[4 * g + 2], acc[4 * g + 3] + add[4 * g + 3]);
   }
-  if (want) sums.template add<T>(run, valid);
+  if (want) sums.template add<T>(run, valid, first);
   uint4 piece[2];
   trade_channel_runs(run, piece);
   if (valid) {
@@ -81,7 +82,7 @@ __device__ __forceinline__ void store_block_plus(const f32x16_t& acc, T* row, co
 template <typename T>
 __device__ __forceinline__ void store_block_plus(const f32x16_t& acc, T* row, const float (&add)[16], int kg, bool valid) {
   RunSums unused;
-  store_block_plus<T>(acc, row, add, kg, valid, unused, false);
+  store_block_plus<T>(acc, row, add, kg, valid, unused, false, false);
 }
 
 // This lane's 16 bias values of the channel block from c0 (zeros without a bias), in result-register order.
@@ -101,15 +102,15 @@ __device__ __forceinline__ void load_block_bias(const T* bias, int c0, int kg, f
 // As store_block_plus with bias[c0 + channel] (when given) as the addend.
 template <typename T>
 __device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid, RunSums& sums,
-                                            bool want) {
+                                            bool want, bool first) {
   float add[16];
   load_block_bias<T>(bias, c0, kg, add);
-  store_block_plus<T>(acc, row, add, kg, valid, sums, want);
+  store_block_plus<T>(acc, row, add, kg, valid, sums, want, first);
 }
 template <typename T>
 __device__ __forceinline__ void store_block(const f32x16_t& acc, T* row, const T* bias, int c0, int kg, bool valid) {
   RunSums unused;
-  store_block<T>(acc, row, bias, c0, kg, valid, unused, false);
+  store_block<T>(acc, row, bias, c0, kg, valid, unused, false, false);
 }
 
 }  // namespace sfh

@@ -139,22 +139,22 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __
   o[3] = elem<T>::from_float(s.w);
 }
 
-// sum_slices_bias that also leaves GroupNorm partials of the rounded result (16-bit outputs): a workgroup owns `chunks`
-// consecutive pieces of 1024 elements of one sample; 1024 is a multiple of the channel count, so a thread's four
-// consecutive channels are the same in every piece and belong to one group. One record per workgroup.
+// sum_slices_bias that also leaves GroupNorm records of the rounded result (16-bit outputs, layout and merge rule in
+// gn_stats.hpp): a workgroup owns `chunks` consecutive pieces of 1024 elements of one sample; 1024 is a multiple of the
+// channel count, so a thread's four consecutive channels are the same in every piece and belong to one group. A thread
+// sums about its own first rounded value; the threads of a group are merged in thread order. One record per workgroup.
 constexpr int kStatsPiece = 4 * kBlock;
 
 template <typename T>
 __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const float* __restrict__ part, const T* __restrict__ bias,
                                                                        T* __restrict__ out, int64_t sample_elems, int64_t nelem,
                                                                        int channels, int splits, int chunks, GnPartialOut gn) {
-  __shared__ float sums[kBlock][2];
+  __shared__ float4 sums[kBlock];  // { values, sum, sum of squares, shift } of every thread
   const int tid = threadIdx.x, n = blockIdx.y;
   const int c = (tid * 4) % channels;
   float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
   if (bias != nullptr) { b0 = to_float(bias[c]); b1 = to_float(bias[c + 1]); b2 = to_float(bias[c + 2]); b3 = to_float(bias[c + 3]); }
-  const float shift = gn.shift != nullptr ? gn.shift[n * gn.groups + c / gn.cg] : 0.f;  // the thread's four channels share a group
-  float s1 = 0.f, s2 = 0.f;
+  float shift = 0.f, s1 = 0.f, s2 = 0.f, cnt = 0.f;
   for (int k = 0; k < chunks; ++k) {
     const int64_t local = ((int64_t)blockIdx.x * chunks + k) * kStatsPiece + tid * 4;
     if (local >= sample_elems) break;
@@ -167,20 +167,25 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const flo
     const T o0 = elem<T>::from_float(s.x + b0), o1 = elem<T>::from_float(s.y + b1), o2 = elem<T>::from_float(s.z + b2),
             o3 = elem<T>::from_float(s.w + b3);
     out[e] = o0; out[e + 1] = o1; out[e + 2] = o2; out[e + 3] = o3;
+    if (k == 0) shift = to_float(o0);
     const float r0 = to_float(o0) - shift, r1 = to_float(o1) - shift, r2 = to_float(o2) - shift, r3 = to_float(o3) - shift;
     s1 += (r0 + r1) + (r2 + r3);
     s2 += fmaf(r0, r0, r1 * r1) + fmaf(r2, r2, r3 * r3);
+    cnt += 4.f;
   }
-  sums[tid][0] = s1;
-  sums[tid][1] = s2;
+  sums[tid] = make_float4(cnt, s1, s2, shift);
   __syncthreads();
   const int rows = kStatsPiece / channels, per_row = channels / 4, per_group = gn.cg / 4;
-  for (int t = tid; t < 2 * gn.groups; t += kBlock) {
-    const int q = t & 1, g = t >> 1;
-    float acc = 0.f;
+  for (int g = tid; g < gn.groups; g += kBlock) {
+    WelfordMerge m;
+    m.clear();
     for (int v = 0; v < rows; ++v)
-      for (int r = 0; r < per_group; ++r) acc += sums[v * per_row + g * per_group + r][q];
-    gn.part[(((int64_t)n * gn.records + blockIdx.x) * 2 + q) * gn.groups + g] = acc;
+      for (int r = 0; r < per_group; ++r) {
+        const float4 e = sums[v * per_row + g * per_group + r];
+        m.add_sums(e.x, e.y, e.z, e.w);
+      }
+    *reinterpret_cast<float4*>(gn.part + (((int64_t)n * gn.records + blockIdx.x) * gn.groups + g) * kGnRecordFloats) =
+        make_float4(m.n, m.mean(), m.m2(), 0.f);
   }
 }
 

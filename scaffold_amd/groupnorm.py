@@ -156,24 +156,19 @@ def _forward_impl(input, num_groups, weight, bias, eps, activation, out_dtype, o
     with _lib.device_guard(input.device):
         rc = _lib.SFH_ERR_UNSUPPORTED
         given = getattr(input, "_sfh_gn_partials", None)
-        next_shift = None
         if given is not None and given[2] == num_groups and given[3] == input._version and given[0].device == input.device:
-            # the producer of `input` left its per-group sums: no statistics pass; and it gets back what to take its next
-            # call's sums about (zeros unless a group's mean is far above its spread)
-            next_shift = torch.empty((n, num_groups), dtype=torch.float32, device=input.device)
+            # the producer of `input` left per-group Welford records of these very bits: no statistics pass
             rc = L.sfh_groupnorm_fwd_from_partials(
                 ctypes.byref(desc), xcode, _lib.dtype_code(odt), _lib.dtype_code(_param_dtype(weight, bias, input)),
                 _lib.ptr(input), _lib.ptr(weight), _lib.ptr(bias), _lib.ptr(out if slab is None else slab),
                 0 if slab is None else out_halo * int(input.shape[3]) * int(input.shape[4]),
-                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(given[0]), given[1], _lib.ptr(given[4]), _lib.ptr(next_shift),
+                _lib.ptr(mean), _lib.ptr(rstd), _lib.ptr(given[0]), given[0].numel() * 4, given[1],
                 _lib.stream_ptr(input.device))
         if rc == _lib.SFH_ERR_UNSUPPORTED:
-            next_shift = None
             rc = _launch_forward(L, desc, xcode, odt, need, input, weight, bias, out, slab, out_halo, mean, rstd)
             if isinstance(rc, tuple):
                 rc, out = rc
     _lib.check(rc, "group_norm")
-    out._sfh_gn_shift = next_shift  # for the producer's next call (None: no statistics came from a producer)
     return out, mean, rstd
 
 

@@ -113,13 +113,17 @@ def _fp32_weight_grad(fn, *args, **kwargs):
         return fn(*args, **kwargs).to(torch.float32)
 
 
+# positions in _Conv3dFn.forward's argument list (after ctx): the gradients come back in this order
+_ARG_SECOND, _N_ARGS = 11, 13
+
+
 class _Conv3dFn(torch.autograd.Function):
     """The caller (``FastConv3d.forward``) has passed the gate for all three directions with these very operands, and
     autograd hands ``backward`` a gradient of the output's shape and dtype: the per-call gates are not repeated."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None,
-                gn_groups=0, gn_shift=None, second=None, slab2=None):
+                gn_groups=0, second=None, slab2=None):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
@@ -147,12 +151,11 @@ class _Conv3dFn(torch.autograd.Function):
             pf, pd = _c3.pack_weights(wc, in_shape, stride, padding, dilation)
         # gn_groups: a GroupNorm of that many groups follows; the launch leaves its statistics on y where it can
         if second is None:
-            y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, gn_shift=gn_shift,
-                                   _checked=True)
+            y = _c3.conv3d_forward(x, wc, bc, stride, padding, dilation, 1, packed_weight=pf, gn_groups=gn_groups, _checked=True)
             ctx.save_for_backward(x, wc) if pd is None else ctx.save_for_backward(x, wc, pd)
         else:
             y = _c3.conv3d_forward_pair(x, second, wc, bc, stride, padding, dilation, packed_weight=pf, gn_groups=gn_groups,
-                                        gn_shift=gn_shift, _checked=True)
+                                        _checked=True)
             ctx.save_for_backward(x, wc, second) if pd is None else ctx.save_for_backward(x, wc, second, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
@@ -180,7 +183,7 @@ class _Conv3dFn(torch.autograd.Function):
                 grad_w, grad_b = both
                 if grad_b.dtype is not bias_dtype:
                     grad_b = grad_b.to(bias_dtype)
-                return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
+                return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None
         if needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight, x, weight.shape, grad_output, stride, padding, dilation, 1,
@@ -188,7 +191,7 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None
 
     @staticmethod
     def _backward_pair(ctx, grad_output):
@@ -197,7 +200,7 @@ class _Conv3dFn(torch.autograd.Function):
         x, weight, second, *packed = ctx.saved_tensors
         stride, padding, dilation, has_bias, bias_dtype, master = ctx.conv_args
         needs_x, needs_w, needs_b = ctx.needs_input_grad[:3]
-        needs_second = ctx.needs_input_grad[12]
+        needs_second = ctx.needs_input_grad[_ARG_SECOND]
         grad_output = grad_output.contiguous(memory_format=_CL3D)
         grad_x = grad_second = None
         if needs_x or needs_second:
@@ -215,8 +218,10 @@ class _Conv3dFn(torch.autograd.Function):
             else:
                 grad_w = _c3.conv3d_backward_weight_pair(x, second, weight.shape, grad_output, stride, padding, dilation, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return (grad_x if needs_x else None, grad_w, grad_b, None, None, None, None, None, None, None, None, None,
-                grad_second if needs_second else None, None)
+        grads = [None] * _N_ARGS
+        grads[0], grads[1], grads[2] = (grad_x if needs_x else None), grad_w, grad_b
+        grads[_ARG_SECOND] = grad_second if needs_second else None
+        return tuple(grads)
 
 
 class _ConvTranspose3dFn(torch.autograd.Function):
@@ -275,16 +280,6 @@ class FastConv3d(nn.Conv3d):
     #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
-    #: what this call's sums are taken about: the ``_next_shift`` the GroupNorm behind this module reported at its last
-    #: call (zeros unless a group's mean was far above its spread), set by whoever owns the pair before each call
-    gn_shift = None
-
-    def _gn_shift(self):
-        shift = self.gn_shift
-        # A captured graph would keep reading this tensor's address after its owner has let go of it: plain sums there.
-        if shift is None or self.gn_groups <= 0 or torch.cuda.is_current_stream_capturing():
-            return None
-        return shift
 
     def _pair_operands(self, x, second):
         """The tensors the kernels would read for ``forward(x, second)`` and the padding they would run with, or ``None``
@@ -367,9 +362,9 @@ class FastConv3d(nn.Conv3d):
         if master:
             return _Conv3dFn.apply(x, weight, bias, stride, padding, dilation, w, b,
                                    _current_packs(weight, w, in_shape, stride, padding, dilation), slab, self.gn_groups,
-                                   self._gn_shift(), second, slab2)
+                                   second, slab2)
         packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is weight else None
-        return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, self._gn_shift(), second,
+        return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, second,
                                slab2)
 
     def forward(self, x: torch.Tensor, second: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -414,12 +409,11 @@ class FastConv3d(nn.Conv3d):
             inner = x
         if master:
             return _Conv3dFn.apply(inner, weight, bias, stride, padding, dilation, w, b,
-                                   _current_packs(weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
-                                   self._gn_shift())
+                                   _current_packs(weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
         if w is weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
-                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups, self._gn_shift())
-        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups, self._gn_shift())
+                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
+        return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups)
 
 
 class FastConvTranspose3d(nn.ConvTranspose3d):
@@ -481,9 +475,5 @@ class FastGroupNorm(nn.GroupNorm):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.dim() == 5 and not x.is_contiguous(memory_format=_CL3D):
             x = x.contiguous(memory_format=_CL3D)
-        out = _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
-                             out_halo=self.out_halo)
-        # what the convolution in front should take its next call's sums about (a plain attribute: straight into the
-        # instance dictionary, past Module.__setattr__'s parameter / buffer / submodule checks)
-        self.__dict__["_next_shift"] = getattr(out, "_sfh_gn_shift", None)
-        return out
+        return _gn.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, out_dtype=None,
+                              out_halo=self.out_halo)

@@ -108,8 +108,6 @@ class DoubleConv(nn.Module):
             return self.double_conv(x if second is None else torch.cat([x, second], dim=1))
         for c, g in self._pairs:  # the Identity modules between the pairs only keep the reference's state-dict indices
             conv, norm = self.double_conv[c], self.double_conv[g]
-            # what the norm's last call said to sum about (a plain attribute, set past Module.__setattr__'s checks)
-            conv.__dict__["gn_shift"] = norm.__dict__.get("_next_shift")
             x = norm(conv(x) if second is None else conv(x, second))
             second = None
         return x

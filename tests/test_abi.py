@@ -137,10 +137,10 @@ def test_which_problems_take_a_skip_connection_as_two_tensors():
     assert offered(conv_desc(cin=64, cout=32, s=(2, 2, 2)), bf16, 32)[1] == 0                        # strided: no data gradient at all
     assert offered(conv_desc(cin=64, cout=32, n=0), bf16, 32) == [0, 0, 0]
     # refused calls launch nothing: null tensors are never touched
-    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, None, None, 16, None, None, None, None, None, 0, 0, 0, None, None, 0,
+    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, None, None, 16, None, None, None, None, None, 0, 0, 0, None, 0,
                                  None) == _lib.SFH_ERR_INVALID
     one = ctypes.c_void_p(16)  # a non-null stand-in that must not be dereferenced
-    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, one, one, 16, one, None, None, one, None, 0, 0, 0, None, None, 0,
+    assert L.sfh_conv3d_fwd_pair(ctypes.byref(level0), bf16, one, one, 16, one, None, None, one, None, 0, 0, 0, None, 0,
                                  None) == _lib.SFH_ERR_UNSUPPORTED
     assert L.sfh_conv3d_dgrad_pair(ctypes.byref(level0), bf16, one, one, None, one, one, 48, None, 0, 0, None) == _lib.SFH_ERR_UNSUPPORTED
     assert L.sfh_conv3d_wgrad_pair(ctypes.byref(level0), fp32, one, one, 32, one, one, None, 0, 0, None) == _lib.SFH_ERR_UNSUPPORTED
@@ -170,6 +170,25 @@ def test_groupnorm_workspace_and_checks():
     assert L.sfh_groupnorm_fwd_workspace_bytes(ctypes.byref(GroupNormDesc(2, 64, 7, 0, 8, 1e-5)), 0) == 0   # C % G != 0
     rc = L.sfh_groupnorm_fwd(ctypes.byref(d), 0, 0, 2, None, None, None, None, None, None, None, 0, None)
     assert rc == _lib.SFH_ERR_INVALID and b"null" in L.sfh_last_error()
+
+
+def test_groupnorm_from_records_checks_their_size_before_launching():
+    """The records a producer left are bounded by their byte size: a count that does not fit is refused, nothing is read."""
+    L = _lib.lib()
+    d = GroupNormDesc(1, 32, 8, 1, 8 * 8 * 32, 1e-5)
+    one = ctypes.c_void_p(256)  # non-null, 16-byte aligned stand-ins that must not be dereferenced
+    need = 1 * 16 * 8 * 4 * 4   # N x records x groups x 4 floats
+    call = lambda nbytes, records, rec=one: L.sfh_groupnorm_fwd_from_partials(
+        ctypes.byref(d), 0, 0, 2, one, None, None, one, 0, one, one, rec, nbytes, records, None)
+    assert call(need - 1, 16) == _lib.SFH_ERR_WORKSPACE and b"records" in L.sfh_last_error()
+    assert call(need, 0) == _lib.SFH_ERR_INVALID and call(need, 16, None) == _lib.SFH_ERR_INVALID
+    assert call(need, 16, ctypes.c_void_p(260)) == _lib.SFH_ERR_INVALID   # off the 16-byte grid
+    # the producer side: too few bytes for the records of the problem
+    conv = conv_desc(cin=32, cout=32, sp=(8, 8, 32))
+    records = L.sfh_conv3d_fwd_gn_records(ctypes.byref(conv), 0, 8)
+    assert records > 0
+    rc = L.sfh_conv3d_fwd_gn(ctypes.byref(conv), 0, one, one, None, None, one, None, 0, 0, 8, one, records * 8 * 16 - 1, None)
+    assert rc == _lib.SFH_ERR_WORKSPACE
 
 
 def test_transposed_and_copy_entry_points_check_arguments():

@@ -308,6 +308,22 @@ def test_fp32_tiles_gaussian_is_true_fp32(device, direction):
     orc.assert_baseline_tolerance(got, ref, torch.float32, f"fp32 tiles {direction}")
 
 
+def test_fp32_tiles_step_aside_for_operands_off_the_16_byte_grid(device):
+    """The fp32 tiles move 16-byte pieces of x, bias and y. A bias that is a view 4 bytes into its storage must not go
+    down that path: the call is served (by the direct kernel) with the same result as the aligned call."""
+    prob = orc.ConvProblem(n=1, cin=32, cout=32, spatial=(6, 9, 33), padding=(1, 1, 1), dtype=torch.float32, bias=True)
+    ops = orc.make_inputs(prob, seed=23, exact=True, density=0.05)
+    x, w, b = (ops[k].to(device) for k in ("input", "weight", "bias"))
+    aligned = sa.conv3d_forward(x, w, b, 1, 1, 1)
+    store = torch.zeros(33, device=device)
+    store[1:] = b
+    off = store[1:]
+    assert off.data_ptr() % 16 == 4
+    assert torch.equal(sa.conv3d_forward(x, w, off, 1, 1, 1), aligned)
+    ref = orc.conv_reference(prob, ops, "fwd")
+    assert torch.equal(aligned.cpu().double(), ref.double())
+
+
 # --- transposed convolution ---------------------------------------------------------------------
 CONVT_SHAPES = [
     (1, 128, 64, (4, 4, 4), (2, 2, 2), True),

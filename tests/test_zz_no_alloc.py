@@ -70,3 +70,44 @@ def test_a_problem_beyond_the_built_in_scratch_is_refused_before_any_launch(devi
     assert rc == _lib.SFH_ERR_WORKSPACE and b"built-in buffer" in L.sfh_last_error()
     torch.cuda.synchronize()
     assert bool((y == 7.0).all())                   # nothing ran
+
+
+def test_captured_into_a_graph_after_prepare_replays_to_the_workspace_forms_bits(device):
+    """The caller this entry point is for: the call recorded into a HIP graph. The scratch address is looked up ahead of
+    the capture (``sfh_groupnorm_fwd_noalloc_prepare``); the graph is replayed three times with eager work and
+    synchronisations between, and every replay must give the workspace form's bits."""
+    torch.cuda.set_device(device)
+    L = _lib.lib()
+    assert L.sfh_groupnorm_fwd_noalloc_prepare() == 0 and L.sfh_groupnorm_fwd_noalloc_prepare() == 0  # idempotent
+    shape, groups = (2, 32, 6, 10, 12), 8
+    (want_y, want_mean, want_rstd), _ = _both_ways(device, shape, groups, True, torch.bfloat16, seed=9)
+    g = torch.Generator().manual_seed(9)
+    n, c, d, h, w = shape
+    x = (torch.randn(shape, generator=g) * 3 + 0.5).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+    gamma = (1 + 0.1 * torch.randn(c, generator=g)).to(device)
+    beta = (0.1 * torch.randn(c, generator=g)).to(device)
+    desc = GroupNormDesc(n, c, groups, 1, d * h * w, 1e-5)
+    y = torch.empty_like(x)
+    mean = torch.empty((n, groups), device=device)
+    rstd = torch.empty((n, groups), device=device)
+
+    def call():
+        _lib.check(L.sfh_groupnorm_fwd_noalloc(ctypes.byref(desc), 0, 0, 2, _lib.ptr(x), _lib.ptr(gamma), _lib.ptr(beta), _lib.ptr(y),
+                                               _lib.ptr(mean), _lib.ptr(rstd), _lib.stream_ptr(x.device)), "no-alloc forward")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for _ in range(3):
+        y.fill_(float("nan"))
+        mean.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want_y) and torch.equal(mean, want_mean) and torch.equal(rstd, want_rstd)
+        _both_ways(device, (1, 32, 5, 7, 9), 8, False, torch.bfloat16, seed=2)  # eager calls that overwrite the shared scratch
+        torch.cuda.synchronize()
