@@ -119,6 +119,21 @@ int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
 #define SFH_KERNEL_OTHER_MATRIX 5
 int sfh_conv3d_launch_geometry(const sfh_conv3d_desc* p, int dtype, int direction, int32_t geometry[4]);
 
+/* ---- measurement: what the matrix pipe sustains ----------------------------------------
+ * No counterpart in the reference's operator interface; its bench measures its ceiling with a vendor GEMM
+ * (triton_conv3d/bench/baseline.py). One launch of `workgroups` 4-wavefront workgroups (one per CU at 256), each
+ * wavefront running `tiles` x 216 v_mfma_f32_32x32x16_bf16 on four accumulators, under one of three instruction mixes:
+ *   0  nothing but the MFMAs;   1  plus one 16-byte LDS read per MFMA (the 3x3x3 convolution's operand rate);
+ *   2  plus, per tile and workgroup, 80 KiB of direct-to-LDS loads streaming through src and 32 KiB of stores
+ *      streaming through sink, and a barrier per tile (the persistent convolution's traffic per 512-voxel brick).
+ * operands: 64 KiB of bf16 bits the MFMAs multiply (the sustained clock depends on them: Gaussian values and zeros are
+ * the two cases worth timing); src / sink: 1 MiB .. 2 GiB each, multiples of 1 KiB, only read / written by mix 2 (may be
+ * NULL otherwise); out: workgroups * 256 floats. The caller times the launch; sfh_mfma_ceiling_probe_flops gives its
+ * FLOP count. */
+double sfh_mfma_ceiling_probe_flops(int32_t workgroups, int32_t tiles);
+int sfh_mfma_ceiling_probe(int32_t mix, int32_t workgroups, int32_t tiles, const void* operands, const void* src,
+                           size_t src_bytes, void* sink, size_t sink_bytes, float* out, void* stream);
+
 /* ---- conv3d forward ------------------------------------------------------------------
  * Stands in for triton_conv3d.conv3d_forward (triton_conv3d/gather_gemm.py:1187) and its
  * kernel _conv3d_fwd_kernel (gather_gemm.py:112).

@@ -15,7 +15,7 @@ from __future__ import annotations
 import ctypes
 import os
 import threading
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint32, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_uint32, c_void_p
 
 import torch
 
@@ -109,6 +109,8 @@ _SIGNATURES = {
     "sfh_conv3d_out_shape": (c_int, [POINTER(ConvDesc), POINTER(c_int32)]),
     "sfh_conv3d_uses_mfma": (c_int, [POINTER(ConvDesc), c_int, c_int]),
     "sfh_conv3d_launch_geometry": (c_int, [POINTER(ConvDesc), c_int, c_int, POINTER(c_int32)]),
+    "sfh_mfma_ceiling_probe_flops": (c_double, [c_int32, c_int32]),
+    "sfh_mfma_ceiling_probe": (c_int, [c_int32, c_int32, c_int32, c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_void_p]),
     "sfh_conv3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvDesc), c_int]),
     "sfh_conv3d_fwd": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p,
                                c_void_p, c_size_t, c_uint32, c_void_p]),

@@ -73,6 +73,34 @@ def test_fastconv3d_matches_stock_in_all_directions(device, dtype):
     assert y1.dtype is dtype and gx1.dtype is dtype and gp1["weight"].dtype is dtype and y1.is_contiguous(memory_format=CL)
 
 
+@pytest.mark.parametrize("cin,cout,spatial", [(32, 32, (16, 32, 32)), (64, 64, (8, 16, 32))])
+def test_no_worse_than_the_incumbent_in_all_directions(device, cin, cout, spatial):
+    """The reference's module-level standard (tests/test_conv3d.py:1170-1217, triton_conv3d/reference.py:241-261): the
+    error against fp64 may not exceed max(error_bound, 4 x the incumbent's error), the incumbent being the stock module
+    on the same GPU (MIOpen) with the same rounded parameters and inputs, in all three directions."""
+    torch.manual_seed(12)
+    dtype = torch.bfloat16
+    truth = nn.Conv3d(cin, cout, 3, padding=1, bias=True).double()
+    fast = FastConv3d(cin, cout, 3, padding=1, bias=True).to(device).to(dtype).to(memory_format=CL)
+    fast.load_state_dict({k: v.to(dtype) for k, v in truth.state_dict().items()})
+    truth.load_state_dict({k: v.double() for k, v in fast.state_dict().items()})
+    incumbent = nn.Conv3d(cin, cout, 3, padding=1, bias=True).to(device).to(dtype).to(memory_format=CL)
+    incumbent.load_state_dict(fast.state_dict())
+    x = torch.randn(1, cin, *spatial).to(dtype)
+    gy = torch.randn(1, cout, *spatial).to(dtype)
+    xd, gyd = x.to(device).contiguous(memory_format=CL), gy.to(device).contiguous(memory_format=CL)
+    y0, gx0, gp0 = _grads(truth, x.double(), gy.double())
+    y1, gx1, gp1 = _grads(fast, xd, gyd)
+    y2, gx2, gp2 = _grads(incumbent, xd, gyd)
+    prob = orc.ConvProblem(n=1, cin=cin, cout=cout, spatial=spatial, bias=True, dtype=dtype)
+    for direction, ours, theirs, ref in (("fwd", y1, y2, y0), ("bwd-data", gx1, gx2, gx0),
+                                         ("bwd-weight", gp1["weight"], gp2["weight"], gp0["weight"])):
+        stock_error = orc.compare(theirs, ref)
+        orc.assert_close(ours, ref, prob, direction, incumbent_error=stock_error)
+        # and without the incumbent's allowance: ours holds the bound on its own account
+        orc.assert_close(ours, ref, prob, direction)
+
+
 def test_autocast_casts_outside_the_node_and_returns_fp32_parameter_grads(device):
     fast = FastConv3d(32, 32, 3, padding=1, bias=False).to(device).to(memory_format=CL)
     up = FastConvTranspose3d(32, 32, 2, stride=2).to(device).to(memory_format=CL)
