@@ -52,6 +52,12 @@ int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* 
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st, const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr,
                       const ChannelPair* out2 = nullptr);
+// The persistent kernel's form for rows of more than 16 voxels: columns walked along depth with a ring of input planes in
+// LDS (conv_ring.hip). `applies` is a pure function of the shape; mfma_conv_persist routes to it. gn.cg must be set.
+bool mfma_conv_ring_applies(const MfmaConvArgs& a);
+int mfma_conv_ring_workgroups_per_block(const MfmaConvArgs& a);
+int mfma_conv_ring(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                   const GnPartialOut& gn, const ChannelPair& out2);
 // Records of GroupNorm partials per sample that mfma_conv_persist leaves for `groups` groups: a pure function of the
 // shape; 0 when the kernel that serves the problem does not offer them (the caller then runs the statistics pass).
 int mfma_conv_gn_records(const MfmaConvArgs& a, int groups);

@@ -481,6 +481,15 @@ int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const
 
 }  // namespace
 
+// Rows of more than 16 voxels take the column-walking form of the persistent kernel.
+static bool ring_serves(const MfmaConvArgs& a) {
+#ifdef SFH_NO_RING
+  return false;
+#else
+  return mfma_conv_ring_applies(a) && a.od > 0 && a.n > 0;
+#endif
+}
+
 // The persistent kernel pays off when the weight slab stays in registers for the whole launch, i.e. with a
 // single 32-channel reduction chunk; wider reductions run the brick-per-workgroup kernel. A brick (at most
 // 10 x 10 input rows deep and high) must also span less than kRange bytes of the input, a tile (at most 8 x 8 output
@@ -499,9 +508,10 @@ MfmaConvGeometry mfma_conv_geometry(const MfmaConvArgs& a) {
 int mfma_conv_gn_records(const MfmaConvArgs& a, int groups) {
   if (!mfma_conv_persist_applies(a)) return mfma_conv_gather_gn_records(a, groups);
   if (a.n != 1 || !gn_partials_fit(a.cout, groups, 32)) return 0;
+  const int cg = a.cout / groups;
+  if (ring_serves(a)) return mfma_conv_ring_workgroups_per_block(a) * (cg > 32 ? cg / 32 : 1);
   const PersistGeom gm = persist_geom(a);
   if (gm.ntiles <= 0) return 0;
-  const int cg = a.cout / groups;
   return gm.wgs_per_block * (cg > 32 ? cg / 32 : 1);
 }
 
@@ -528,6 +538,7 @@ int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const voi
     out = *gn;
     out.cg = a.cout / gn->groups;
   }
+  if (ring_serves(a)) return mfma_conv_ring(a, dtype, x, packed, bias, y, st, out, pair);
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, packed, bias, y, st, out, pair);
   return launch_typed<fp16_t>(a, x, packed, bias, y, st, out, pair);
 }
