@@ -13,8 +13,8 @@
 // Each wavefront owns a 2 x 2 block of the step's rows (two planes x two rows of 32 voxels). An activation fragment --
 // 32 voxels of one input row, shifted by kw, one k-step -- then serves up to four MFMAs (the taps (kd, kh) under which
 // the row is seen from the wavefront's four output rows) and is read from LDS once: 96 reads for 216 MFMAs. The order
-// of MFMAs and reads is a compile-time schedule (RingSchedule) that never issues two MFMAs on one accumulator closer
-// than three apart and requests every fragment several MFMAs ahead of its first use.
+// of MFMAs and reads is a compile-time schedule (RingSchedule): the same order of taps for every output voxel, the four
+// accumulators in turn, every fragment requested several MFMAs ahead of its first use.
 //
 // The three plane pairs are three separate LDS arrays and the ring position is a template parameter of the step: the
 // compiler then sees that the MFMA operands never alias the array being filled, and every LDS address is an immediate
@@ -46,41 +46,49 @@ static_assert(kGroups * 1024 - kPiece < 64 * 16 && kPiece >= kPairVoxels * 16, "
 
 // ---- the compile-time schedule of a step ---------------------------------------------------------------------------------------
 // Block b = 0..5 handles kw = b % 3 and k-step ks = b / 3 (the first three blocks use the weight fragments held in vector
-// registers, the last three those in accumulation registers). Inside a block the 16 input-row fragments F(D, H) --
-// plane D = 0..3 of the step, row H = 0..3 of the wavefront's two output rows with halo -- are visited in an order
-// that spreads the accumulators; fragment F(D, H) feeds accumulator (dd, hl) under tap (kd, kh) = (D - dd, H - hl).
+// registers, the last three those in accumulation registers). Inside a block the nine taps (kd, kh) come in row-major
+// order, and each is applied to the wavefront's four accumulators (dd, hl) in turn: accumulator (dd, hl) under tap
+// (kd, kh) reads input-row fragment F(D, H) = (kd + dd, kh + hl) -- plane D = 0..3 of the step, row H = 0..3 of the
+// wavefront's two output rows with halo. Every output voxel therefore accumulates its 54 products in the same order
+// whatever its place in the step (results do not depend on where a tensor's planes fall in the walk: a depth shard's
+// slab and the padded volume give the same bits), two MFMAs on one accumulator are always four apart, and a fragment is
+// read from LDS once and kept until the last tap that sees it.
 struct RingSchedule {
   static constexpr int kFragsPerBlock = 16, kMfmasPerBlock = 36, kBlocks = 6;
   static constexpr int kFrags = kFragsPerBlock * kBlocks, kMfmas = kMfmasPerBlock * kBlocks;
   static constexpr int kLead = 5;      // a fragment is requested at least this many MFMAs before its first use
-  static constexpr int kBuffers = 8;   // fragment registers in rotation
-  int frag_d[kFragsPerBlock], frag_h[kFragsPerBlock];
+  static constexpr int kBuffers = 8;   // fragment registers (the schedule's need is checked against it)
+  int frag_d[kFragsPerBlock], frag_h[kFragsPerBlock];  // in order of first use
   int mf_frag[kMfmasPerBlock], mf_acc[kMfmasPerBlock], mf_tap9[kMfmasPerBlock];
   int first_use[kFragsPerBlock], last_use[kFragsPerBlock];
   int issue_after[kFrags];  // global MFMA index after which fragment f is requested (negative: before the loop)
+  int buffer[kFrags];       // the register set fragment f is read into
   int request_at[kMfmas];   // the fragment requested behind MFMA m, or -1
+  int buffers_used;
 };
 
 constexpr RingSchedule make_ring_schedule() {
   RingSchedule s{};
-  const int order[16][2] = {{0, 0}, {0, 3}, {3, 0}, {3, 3}, {0, 1}, {3, 1}, {0, 2}, {3, 2},
-                            {1, 0}, {1, 3}, {2, 0}, {2, 3}, {1, 1}, {1, 2}, {2, 1}, {2, 2}};
-  int m = 0;
-  for (int f = 0; f < 16; ++f) {
-    s.frag_d[f] = order[f][0];
-    s.frag_h[f] = order[f][1];
-    s.first_use[f] = m;
-    for (int dd = 0; dd < 2; ++dd)
-      for (int hl = 0; hl < 2; ++hl) {
-        const int kd = order[f][0] - dd, kh = order[f][1] - hl;
-        if (kd < 0 || kd > 2 || kh < 0 || kh > 2) continue;
-        s.mf_frag[m] = f;
-        s.mf_acc[m] = dd * 2 + hl;
-        s.mf_tap9[m] = kd * 3 + kh;
-        s.last_use[f] = m;
-        ++m;
-      }
-  }
+  int slot_of[4][4] = {{-1, -1, -1, -1}, {-1, -1, -1, -1}, {-1, -1, -1, -1}, {-1, -1, -1, -1}};
+  int nf = 0, m = 0;
+  for (int kd = 0; kd < 3; ++kd)
+    for (int kh = 0; kh < 3; ++kh)
+      for (int dd = 0; dd < 2; ++dd)
+        for (int hl = 0; hl < 2; ++hl) {
+          const int d = kd + dd, h = kh + hl;
+          if (slot_of[d][h] < 0) {
+            slot_of[d][h] = nf;
+            s.frag_d[nf] = d;
+            s.frag_h[nf] = h;
+            s.first_use[nf] = m;
+            ++nf;
+          }
+          s.mf_frag[m] = slot_of[d][h];
+          s.mf_acc[m] = dd * 2 + hl;
+          s.mf_tap9[m] = kd * 3 + kh;
+          s.last_use[slot_of[d][h]] = m;
+          ++m;
+        }
   // request times, latest first: as late as the lead allows, never two after the same MFMA
   int next = RingSchedule::kMfmas;
   for (int f = RingSchedule::kFrags - 1; f >= 0; --f) {
@@ -93,38 +101,40 @@ constexpr RingSchedule make_ring_schedule() {
   for (int k = 0; k < RingSchedule::kMfmas; ++k) s.request_at[k] = -1;
   for (int f = 0; f < RingSchedule::kFrags; ++f)
     if (s.issue_after[f] >= 0) s.request_at[s.issue_after[f]] = f;
+  // register sets: a set is free again once the MFMA of its fragment's last use has been issued
+  int busy_until[RingSchedule::kFrags] = {};
+  int nb = 0;
+  for (int f = 0; f < RingSchedule::kFrags; ++f) {
+    const int last = (f / 16) * 36 + s.last_use[f % 16];
+    int pick = -1;
+    for (int b = 0; b < nb && pick < 0; ++b)
+      if (busy_until[b] <= s.issue_after[f]) pick = b;
+    if (pick < 0) pick = nb++;
+    busy_until[pick] = last;
+    s.buffer[f] = pick;
+  }
+  s.buffers_used = nb;
   return s;
 }
 
 constexpr RingSchedule kSched = make_ring_schedule();
 
 constexpr bool ring_schedule_ok() {
-  int count = 0;
-  for (int i = 0; i < 36; ++i) count += 1;
-  // every accumulator is touched in the first four MFMAs (they start from zero), and never twice within three MFMAs
-  for (int a = 0; a < 4; ++a) {
-    bool seen = false;
-    for (int i = 0; i < 4; ++i) seen = seen || kSched.mf_acc[i] == a;
-    if (!seen) return false;
-  }
+  // the first four MFMAs touch the four accumulators (they start from zero); afterwards the accumulators take turns
   for (int i = 0; i < 36; ++i)
-    for (int k = 1; k < 3; ++k)
-      if (kSched.mf_acc[i] == kSched.mf_acc[(i + k) % 36]) return false;
-  // a fragment's register is not requested again before its last use
-  for (int f = 0; f + RingSchedule::kBuffers < RingSchedule::kFrags; ++f) {
-    const int last = (f / 16) * 36 + kSched.last_use[f % 16];
-    if (kSched.issue_after[f + RingSchedule::kBuffers] < last) return false;
-  }
-  // the fragments requested before the loop fit the rotation
-  int before = 0;
-  for (int f = 0; f < RingSchedule::kFrags; ++f) before += kSched.issue_after[f] < 0 ? 1 : 0;
-  return before <= RingSchedule::kBuffers && kSched.mf_frag[35] == 15 && count == 36;
+    if (kSched.mf_acc[i] != i % 4) return false;
+  // every fragment is requested ahead of its first use
+  for (int f = 0; f < RingSchedule::kFrags; ++f)
+    if (kSched.issue_after[f] > (f / 16) * 36 + kSched.first_use[f % 16] - 2) return false;
+  return kSched.buffers_used <= RingSchedule::kBuffers;
 }
 static_assert(ring_schedule_ok(), "step schedule");
 
-// Side work of a step rides behind every eighth MFMA: first the loads of the next pair, then the stores of the previous
-// step's rounded result.
-constexpr int kSidePeriod = 8, kSidePhase = 3;
+// Side work of a step rides behind every tenth MFMA: first the loads of the next pair (they need the rest of the step to
+// arrive), then the stores of the previous step's rounded result. Measured against closer spacings and interleaved
+// orders: the kernel is insensitive to it within 2 %, spreading the memory instructions out is marginally the best.
+constexpr int kSidePeriod = 10, kSidePhase = 3;
+constexpr int side_kind(int slot) { return slot < kLoads + kStores ? slot : -1; }  // which load (0 ..) or store (kLoads ..) a slot carries
 static_assert((RingSchedule::kMfmas - kSidePhase + kSidePeriod - 1) / kSidePeriod >= kLoads + kStores, "a slot per load and store");
 
 // s_waitcnt immediate (gfx9 encoding) that waits for vmcnt <= n and nothing else.
@@ -228,7 +238,7 @@ struct RingStep {
     constexpr int b = F / 16, fi = F % 16;
     constexpr int d = kSched.frag_d[fi], h = kSched.frag_h[fi];
     constexpr int off = ring_frag_off(d % 2, h, b % 3, b / 3);
-    fr[F % S::kBuffers] = *reinterpret_cast<const uint4*>((d < 2 ? lane_lo : lane_hi) + off);
+    fr[kSched.buffer[F]] = *reinterpret_cast<const uint4*>((d < 2 ? lane_lo : lane_hi) + off);
   }
   template <int F>
   __device__ __forceinline__ void request_if_early() {
@@ -251,12 +261,12 @@ struct RingStep {
         f32x16_t zero;
 #pragma unroll
         for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-        acc[ac] = Mma32<T>::run(wq[tap], fr[f % S::kBuffers], zero);
+        acc[ac] = Mma32<T>::run(wq[tap], fr[kSched.buffer[f]], zero);
       } else {
-        acc[ac] = Mma32<T>::run(wq[tap], fr[f % S::kBuffers], acc[ac]);
+        acc[ac] = Mma32<T>::run(wq[tap], fr[kSched.buffer[f]], acc[ac]);
       }
     } else {
-      Mma32Pinned<T>::run_row_in_acc(wa[tap], fr[f % S::kBuffers], acc[ac]);
+      Mma32Pinned<T>::run_row_in_acc(wa[tap], fr[kSched.buffer[f]], acc[ac]);
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (kSched.request_at[M] >= 0) {  // at most one fragment request behind an MFMA
@@ -264,14 +274,14 @@ struct RingStep {
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (M % kSidePeriod == kSidePhase) {
-      constexpr int slot = M / kSidePeriod;
-      if constexpr (slot < kLoads) {
-        constexpr int k = slot / 4, p = slot % 4;
+      constexpr int kind = side_kind(M / kSidePeriod);
+      if constexpr (kind >= 0 && kind < kLoads) {
+        constexpr int k = kind / 4, p = kind % 4;
         if (voff[k] != -1)
           __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(fill + (wave + 4 * k) * 1024 + p * kPiece), 16,
                                                    voff[k] + p * 16, 0, 0, 0);
-      } else if constexpr (slot < kLoads + kStores) {
-        constexpr int ms = (slot - kLoads) / 2, h = (slot - kLoads) % 2;
+      } else if constexpr (kind >= kLoads) {
+        constexpr int ms = (kind - kLoads) / 2, h = (kind - kLoads) % 2;
         __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
