@@ -374,9 +374,10 @@ def gemm_reference(device):
 
 def mfma_ceiling(device, operand_kinds=("gaussian", "zeros"), reps=5, tiles=64):
     """What the matrix pipe sustains on this box in this run under the persistent convolution's instruction mix
-    (``sfh_mfma_ceiling_probe``): nothing but v_mfma_f32_32x32x16_bf16; plus one 16-byte LDS read per MFMA; plus the
-    convolution's HBM bytes per FLOP (80 KiB streamed in and 32 KiB out per 216 x 4 MFMAs of a workgroup) and its
-    barrier per tile.  One workgroup per CU, every launch ~3 ms (so the clocks have settled), timed with events."""
+    (``sfh_mfma_ceiling_probe``): nothing but v_mfma_f32_32x32x16_bf16; plus one 16-byte LDS read per two MFMAs (the
+    kernel's operand rate: its ceiling without any global traffic); plus the kernel's global loads and stores per step
+    streamed from and to HBM (48 KiB in, 32 KiB out per 216 x 4 MFMAs of a workgroup) and its barrier.  One workgroup per
+    CU, timed with events."""
     import ctypes
 
     from scaffold_amd import _lib
@@ -396,7 +397,7 @@ def mfma_ceiling(device, operand_kinds=("gaussian", "zeros"), reps=5, tiles=64):
             src = torch.randn(src_bytes // 2, generator=g, device=device, dtype=torch.bfloat16)
         else:
             src = torch.zeros(src_bytes // 2, device=device, dtype=torch.bfloat16)
-        for mix, name in ((0, "mfma only"), (1, "+ 1 LDS read / MFMA"), (2, "+ conv HBM bytes/FLOP + barrier")):
+        for mix, name in ((0, "mfma only"), (1, "+ 1 LDS read / 2 MFMAs"), (2, "+ conv loads/stores from HBM + barrier")):
             def launch():
                 _lib.check(L.sfh_mfma_ceiling_probe(mix, wgs, tiles, P(src), P(src), src_bytes, P(sink), sink.numel(), P(out), stream),
                            "sfh_mfma_ceiling_probe")
@@ -979,11 +980,11 @@ def main():
     fwd_ms = conv["in_step_ms"]["fwd"]
     achieved = flops / (fwd_ms * 1e-3) / 1e12
     traffic, traffic_source = counter_traffic("conv_persist_kernel")
-    # the measured ceiling of this run for the kernel's instruction mix on Gaussian operands (beside, never instead of,
-    # the nominal peak)
+    # the measured ceiling of this run for the kernel's MFMA + LDS-read mix on Gaussian operands, no global traffic
+    # (beside, never instead of, the nominal peak)
     ceiling = None
     if isinstance(details.get("mfma_ceiling"), list):
-        ceiling = next((r["tflops"] for r in details["mfma_ceiling"] if r["operands"] == "gaussian" and r["mix"] == 2), None)
+        ceiling = next((r["tflops"] for r in details["mfma_ceiling"] if r["operands"] == "gaussian" and r["mix"] == 1), None)
     cpu = None if args.skip_cpu else cpu_baseline(with_unet=not args.skip_unet)
     # the one full-size parity point of the train step: the stock-module arm's loss on the host against the first loss
     # of the GPU step, from the same weights and the same shard (bf16 on both sides: 2e-2 relative)

@@ -123,9 +123,11 @@ int sfh_conv3d_launch_geometry(const sfh_conv3d_desc* p, int dtype, int directio
  * No counterpart in the reference's operator interface; its bench measures its ceiling with a vendor GEMM
  * (triton_conv3d/bench/baseline.py). One launch of `workgroups` 4-wavefront workgroups (one per CU at 256), each
  * wavefront running `tiles` x 216 v_mfma_f32_32x32x16_bf16 on four accumulators, under one of three instruction mixes:
- *   0  nothing but the MFMAs;   1  plus one 16-byte LDS read per MFMA (the 3x3x3 convolution's operand rate);
- *   2  plus, per tile and workgroup, 80 KiB of direct-to-LDS loads streaming through src and 32 KiB of stores
- *      streaming through sink, and a barrier per tile (the persistent convolution's traffic per 512-voxel brick).
+ *   0  nothing but the MFMAs;   1  plus one 16-byte LDS read per two MFMAs (the persistent 3x3x3 convolution's
+ *      operand rate): the ceiling for that kernel's instruction mix without any global memory traffic;
+ *   2  plus, per tile and workgroup, 48 KiB of direct-to-LDS loads streaming through src and 32 KiB of stores
+ *      streaming through sink, and a barrier per tile (the convolution's traffic per 512-voxel step, all of it from
+ *      and to HBM: a reference point, not a bound -- the convolution finds its halo rows in L2).
  * operands: 64 KiB of bf16 bits the MFMAs multiply (the sustained clock depends on them: Gaussian values and zeros are
  * the two cases worth timing); src / sink: 1 MiB .. 2 GiB each, multiples of 1 KiB, only read / written by mix 2 (may be
  * NULL otherwise); out: workgroups * 256 floats. The caller times the launch; sfh_mfma_ceiling_probe_flops gives its

@@ -3,10 +3,12 @@
 // read against a measured ceiling as well as against the nominal peak. One 4-wavefront workgroup per CU, as the
 // persistent kernel runs; a "tile" is its unit of 54 x 4 MFMAs per wavefront on four accumulators.
 //   mix 0: nothing but the MFMAs (operands stay in registers);
-//   mix 1: one ds_read_b128 per MFMA feeding its column operand (the convolution's LDS read rate);
-//   mix 2: mix 1 plus, per tile and wavefront, 20 direct-to-LDS loads of 1 KiB that stream through `src` and 8 stores of
-//          1 KiB that stream through `sink` (the convolution's 78 KiB in / 32 KiB out per 512-voxel tile), and a
-//          workgroup barrier per tile.
+//   mix 1: one ds_read_b128 per two MFMAs feeding their column operand (the convolution reads 96 fragments for 216 MFMAs):
+//          the ceiling of a kernel with this operand traffic and no global memory traffic at all;
+//   mix 2: mix 1 plus, per tile and wavefront, 12 direct-to-LDS loads of 1 KiB that stream through `src` and 8 stores of
+//          1 KiB that stream through `sink` (the convolution's 44 KiB in / 32 KiB out per 512-voxel step), and a
+//          workgroup barrier per tile. Every byte of it comes from and goes to HBM, where the convolution finds its halo
+//          rows in L2: a reference point for the cost of the traffic, not a bound.
 // The operand values come from the caller's buffers (Gaussian or zero bits: the sustained clock depends on them).
 #include "common.hpp"
 #include "mma.hpp"
@@ -16,7 +18,8 @@ namespace {
 
 typedef uint32_t sfh_probe_u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int kProbeLdsBytes = 64 * 1024;
-constexpr int kProbeTileIn = 80 * 1024;   // bytes a workgroup fetches per tile in mix 2 (4 wavefronts x 20 x 1 KiB)
+constexpr int kProbeLoads = 12;           // direct-to-LDS loads per wavefront and tile in mix 2
+constexpr int kProbeTileIn = 4 * kProbeLoads * 1024;  // bytes a workgroup fetches per tile in mix 2
 constexpr int kProbeTileOut = 32 * 1024;  // bytes it stores (4 x 8 x 1 KiB)
 
 template <int MIX>
@@ -55,16 +58,16 @@ mfma_probe_kernel(const uint4* __restrict__ operands, const char* __restrict__ s
         __builtin_amdgcn_sched_barrier(0);
         acc[ms] = Mma32<bf16_t>::run(a[(it + ms) & 7], b[ms], acc[ms]);
         __builtin_amdgcn_sched_barrier(0);
-        if (MIX >= 1) b[ms] = *reinterpret_cast<const uint4*>(rd + ((it * 4 + ms) * 1024 + wave * 256) % (kProbeLdsBytes - 1024));
-        if (MIX >= 2 && ms == 0) {
-          if (it % 2 == 0 && it / 2 < 20) {
-            const uint32_t off = (in0 + (uint32_t)((wave * 20 + it / 2) * 1024 + lane * 16)) % src_bytes;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (__attribute__((address_space(3))) void*)(lds_fill + ((wave * 20 + it / 2) % 64) * 1024),
+        if (MIX >= 1 && ms % 2 == 0) b[ms] = *reinterpret_cast<const uint4*>(rd + ((it * 4 + ms) * 1024 + wave * 256) % (kProbeLdsBytes - 1024));
+        if (MIX >= 2 && ms == 0) {  // a load or a store behind every tenth MFMA or so, loads first (as the convolution issues them)
+          if (it % 2 == 0 && it / 2 < kProbeLoads) {
+            const uint32_t off = (in0 + (uint32_t)((wave * kProbeLoads + it / 2) * 1024 + lane * 16)) % src_bytes;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_in, (__attribute__((address_space(3))) void*)(lds_fill + ((wave * kProbeLoads + it / 2) % 64) * 1024),
                                                      16, off, 0, 0, 0);
           }
-          if (it % 2 == 1 && it / 2 < 8) {
-            const uint32_t off = (out0 + (uint32_t)((wave * 8 + it / 2) * 1024 + lane * 16)) % sink_bytes;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(sfh_probe_u32x4_t, b[it % 4]), rs_out, off, 0, 0);
+          if (it % 2 == 0 && it / 2 >= kProbeLoads && it / 2 < kProbeLoads + 8) {
+            const uint32_t off = (out0 + (uint32_t)((wave * 8 + it / 2 - kProbeLoads) * 1024 + lane * 16)) % sink_bytes;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(sfh_probe_u32x4_t, a[it % 8]), rs_out, off, 0, 0);
           }
         }
       }

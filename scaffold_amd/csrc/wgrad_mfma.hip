@@ -25,13 +25,13 @@
 #ifdef SFH_WGRAD_TUNE
 #include <cstdlib>
 #endif
+#include <type_traits>
+
 #include "mma.hpp"
 #include "reduce.hpp"
 
 namespace sfh {
 namespace {
-
-
 
 constexpr int kTargetWorkgroups = kComputeUnits;
 
@@ -401,8 +401,22 @@ struct Plan {
   int splits, tiles_per_split;
 };
 
+// Rows of more than 16 voxels take the column-walking kernel.
+bool ring_serves(const WgradArgs& a) {
+#ifdef SFH_NO_WRING
+  return false;
+#else
+  return mfma_wgrad_ring_applies(a);
+#endif
+}
+
 Plan make_plan(const WgradArgs& a) {
   Plan p{};
+  if (ring_serves(a)) {
+    p.tw = 32;
+    p.splits = mfma_wgrad_ring_splits(a);
+    return p;
+  }
   int td, th;
   if (a.ow > 16) { p.tw = 32; td = 2; th = 4; }
   else if (a.ow > 8) { p.tw = 16; td = 2; th = 8; }
@@ -456,7 +470,8 @@ int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, in
   const bool direct = p.splits == 1 && gw_dtype == SFH_FP32;
   float* ws = direct ? (float*)gw : (float*)workspace;
   int rc;
-  if (p.tw == 32) rc = launch_tile<T, WTile<2, 4, 32>>(a, p, x, gy, ws, st, x2);
+  if (ring_serves(a)) rc = mfma_wgrad_ring(a, std::is_same<T, bf16_t>::value ? SFH_BF16 : SFH_FP16, x, gy, ws, st, x2);
+  else if (p.tw == 32) rc = launch_tile<T, WTile<2, 4, 32>>(a, p, x, gy, ws, st, x2);
   else if (p.tw == 16) rc = launch_tile<T, WTile<2, 8, 16>>(a, p, x, gy, ws, st, x2);
   else rc = launch_tile<T, WTile<4, 8, 8>>(a, p, x, gy, ws, st, x2);
   if (rc != SFH_OK || direct) return rc;

@@ -21,4 +21,11 @@ bool mfma_wgrad_pair_ok(const WgradArgs& a, int first);
 int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, void* gw, int gw_dtype, void* workspace,
                hipStream_t st, const ChannelPair* x2 = nullptr);
 
+// The same gradient for rows of more than 16 voxels (wgrad_ring.hip): columns walked along depth, operands staged as
+// they lie in memory and transposed by the LDS reads. `applies` and the slice count are pure functions of the shape;
+// the kernel writes `splits` fp32 slices [Cout][27][Cin] into ws. mfma_wgrad routes to it.
+bool mfma_wgrad_ring_applies(const WgradArgs& a);
+int mfma_wgrad_ring_splits(const WgradArgs& a);
+int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2);
+
 }  // namespace sfh

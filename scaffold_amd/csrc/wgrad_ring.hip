@@ -1,0 +1,491 @@
+// MFMA weight gradient of a 3x3x3 stride-1 convolution for gfx950 (bf16 / fp16, rows of more than 16 voxels) that
+// stages both operands in LDS exactly as they lie in memory and lets the LDS do the transposition.
+//
+//   gw[co][kd][kh][kw][ci] = sum over output voxels v of gy[v][co] * x[v + tap - pad][ci]
+//
+// GEMM view (triton_conv3d/reduce_gemm.py:137-393): M = Cout, N = 27 x Cin, K = output voxels, split over workgroups
+// along K, fp32 partial slices at fixed workspace slots and an ordered reduction (reduce_gemm.py:396-435) -- no float
+// atomics, split count a pure function of shape.
+//
+// Both MFMA operands need the contraction index (voxels) along a lane's register while memory is channel-contiguous.
+// gfx950's ds_read_b64_tr_b16 does that transposition on the way out of LDS (within 16 lanes: lane m gives the address
+// of 4 channels of voxel m / 4 and receives channel m of the four voxels), so nothing is transposed by hand:
+//   * a workgroup (four wavefronts, one per SIMD) walks a column 4 rows high and 32 voxels wide along depth, two
+//     planes per step, as the persistent forward kernel does (conv_ring.hip): LDS holds a ring of three input plane
+//     PAIRS (2 x 6 x 34 voxels with the halo) and three gy tiles (2 x 4 x 32 voxels); while the MFMAs of a step read two
+//     pairs and one tile, the next step's new pair and tile stream in straight from memory (buffer_load ... lds);
+//   * every voxel is stored as four 16-byte channel pieces in four piece planes (the forward kernel's layout), which
+//     makes the transposing reads bank-conflict free at any voxel offset: a tap's shift along W is an address offset,
+//     not a funnel shift;
+//   * wavefront (s, g) owns the half-rows s (16 voxels = one MFMA k-step) and the tap group g (14 / 13 of the 27 taps):
+//     224 accumulation registers. Its gy fragments of the step (8) stay in registers; it walks the input rows of the
+//     step once, and an input-row fragment (plane D, row H, shift kw) feeds up to six MFMAs -- the taps (kd, kh) under
+//     which that row is seen from the step's output rows: 0.8 LDS reads per MFMA, no vector-ALU work between them;
+//   * at the end the two wavefronts that hold the same taps add their accumulators through LDS in a fixed order and
+//     the workgroup writes one fp32 slice.
+#include <utility>
+
+#include "mma.hpp"
+#include "reduce.hpp"
+#include "wgrad_mfma.hpp"
+
+namespace sfh {
+namespace {
+
+constexpr int kTD = 2, kTH = 4, kTW = 32;             // output voxels of a step
+constexpr int kBH = kTH + 2, kBW = kTW + 2;           // rows / voxels per row of an input plane with its halo
+constexpr int kXVoxels = 2 * kBH * kBW;               // voxels of an input plane pair (408)
+constexpr int kGVoxels = kTD * kTH * kTW;             // voxels of a gy tile (256)
+constexpr int wring_piece_bytes(int voxels) { return ((voxels * 16 - 64 + 255) / 256) * 256 + 64; }  // 64 modulo 256
+constexpr int kXPiece = wring_piece_bytes(kXVoxels), kXPair = 4 * kXPiece;
+constexpr int kGPiece = wring_piece_bytes(kGVoxels), kGTile = 4 * kGPiece;
+constexpr int kXGroups = (kXVoxels + 63) / 64;        // 64-voxel groups a pair is fetched in (7, the last one partial)
+constexpr int kXGroupsPerWave = (kXGroups + 3) / 4;   // 2
+constexpr int kLoads = (kXGroupsPerWave + 1) * 4;     // load instructions per wavefront and step (x groups + one gy group)
+constexpr int kRange = 0x40000000;                    // buffer range: offsets at or above it read as zero
+constexpr int kTaps0 = 14, kTaps1 = 13;               // taps of the two groups
+static_assert(3 * kXPair + 3 * kGTile <= 160 * 1024, "three plane pairs and three gy tiles in the LDS of a CU");
+static_assert(kGVoxels == 4 * 64, "one gy group per wavefront");
+constexpr int kHandTaps = kXPair / 4096, kHandRounds = (kTaps0 + kHandTaps - 1) / kHandTaps;  // accumulators (4 KiB per tap) handed over per round
+constexpr int kWaitLgkm0 = 0xC07F;  // s_waitcnt immediate (gfx9): lgkmcnt(0), vmcnt and expcnt untouched
+
+// Tap (kd, kh, kw) -> group and accumulator. Group 0: kw = 0, and kw = 1 for the first five (kd, kh); group 1: kw = 2, and
+// kw = 1 for the other four.
+constexpr int tap_group(int t9, int kw) { return kw == 0 ? 0 : (kw == 2 ? 1 : (t9 < 5 ? 0 : 1)); }
+constexpr int tap_slot(int t9, int kw) { return kw == 0 ? t9 : (kw == 2 ? t9 : (t9 < 5 ? 9 + t9 : 9 + t9 - 5)); }
+
+// ---- the compile-time schedule of a step, per tap group ---------------------------------------------------------------------
+// The input rows of the step are visited in the order (H = 0..5, D = 0..3, kw); fragment X(D, H, kw) is requested if the
+// group has a tap that sees it, and then feeds the MFMAs acc[(kd, kh, kw)] += gy(d, h) x X for all (d, kd = D - d),
+// (h, kh = H - h) of the group.
+struct WSchedule {
+  static constexpr int kMaxMfmas = 8 * kTaps0, kMaxFrags = 72, kLead = 4, kBuffers = 4;
+  int nm, nf;
+  int mf_frag[kMaxMfmas], mf_acc[kMaxMfmas], mf_gy[kMaxMfmas];
+  int fr_d[kMaxFrags], fr_h[kMaxFrags], fr_kw[kMaxFrags], fr_first[kMaxFrags], fr_last[kMaxFrags];
+  int issue_after[kMaxFrags], buffer[kMaxFrags], request_at[kMaxMfmas];
+  int buffers_used, min_acc_distance;
+};
+
+constexpr WSchedule make_wschedule(int g) {
+  WSchedule s{};
+  for (int h = 0; h < kBH; ++h)
+    for (int d = 0; d < 4; ++d)
+      for (int kw = 0; kw < 3; ++kw) {
+        int first = -1;
+        for (int dd = 0; dd < kTD; ++dd)
+          for (int hh = 0; hh < kTH; ++hh) {
+            const int kd = d - dd, kh = h - hh;
+            if (kd < 0 || kd > 2 || kh < 0 || kh > 2 || tap_group(kd * 3 + kh, kw) != g) continue;
+            if (first < 0) {
+              first = s.nm;
+              s.fr_d[s.nf] = d; s.fr_h[s.nf] = h; s.fr_kw[s.nf] = kw; s.fr_first[s.nf] = s.nm;
+            }
+            s.mf_frag[s.nm] = s.nf;
+            s.mf_acc[s.nm] = tap_slot(kd * 3 + kh, kw);
+            s.mf_gy[s.nm] = dd * kTH + hh;
+            s.fr_last[s.nf] = s.nm;
+            ++s.nm;
+          }
+        if (first >= 0) ++s.nf;
+      }
+  int next = s.nm;
+  for (int f = s.nf - 1; f >= 0; --f) {
+    int at = s.fr_first[f] - WSchedule::kLead;
+    if (at >= next) at = next - 1;
+    s.issue_after[f] = at;
+    next = at;
+  }
+  for (int k = 0; k < WSchedule::kMaxMfmas; ++k) s.request_at[k] = -1;
+  for (int f = 0; f < s.nf; ++f)
+    if (s.issue_after[f] >= 0) s.request_at[s.issue_after[f]] = f;
+  int busy_until[WSchedule::kMaxFrags] = {};
+  int nb = 0;
+  for (int f = 0; f < s.nf; ++f) {
+    int pick = -1;
+    for (int b = 0; b < nb && pick < 0; ++b)
+      if (busy_until[b] <= s.issue_after[f]) pick = b;
+    if (pick < 0) pick = nb++;
+    busy_until[pick] = s.fr_last[f];
+    s.buffer[f] = pick;
+  }
+  s.buffers_used = nb;
+  s.min_acc_distance = s.nm;
+  for (int i = 0; i < s.nm; ++i)
+    for (int k = i + 1; k < s.nm && k < i + 8; ++k)
+      if (s.mf_acc[i] == s.mf_acc[k] && k - i < s.min_acc_distance) s.min_acc_distance = k - i;
+  return s;
+}
+
+constexpr WSchedule kWSched0 = make_wschedule(0), kWSched1 = make_wschedule(1);
+static_assert(kWSched0.nm == 8 * kTaps0 && kWSched1.nm == 8 * kTaps1, "every (row, tap) of the group exactly once");
+static_assert(kWSched0.buffers_used <= WSchedule::kBuffers && kWSched1.buffers_used <= WSchedule::kBuffers, "fragment registers");
+static_assert(kWSched0.min_acc_distance >= 2 && kWSched1.min_acc_distance >= 2, "no two MFMAs in a row on one accumulator");
+
+constexpr int kSidePeriod = 8, kSidePhase = 3;
+static_assert((8 * kTaps1 - kSidePhase + kSidePeriod - 1) / kSidePeriod >= kLoads, "a slot per load");
+
+constexpr int wring_waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+
+struct WRingGeom {
+  int tiles_h, tiles_w, steps, segs, seg_steps;
+  int nblk_ci, nblk;                       // 32 x 32 blocks of (co, ci)
+  int items, splits, items_per_split;      // items = columns x segments; a workgroup (split) takes consecutive ones
+};
+
+struct WRingLane {
+  int xrel[kXGroupsPerWave], xcoord[kXGroupsPerWave];  // staging of x: byte offset from the pair's first voxel; dl | bh << 8 | bw << 16 or -1
+  int grel, gcoord;                                    // staging of gy: byte offset from the tile's first voxel; d | h << 8 | w << 16
+  int xread, gread;                                    // transposing reads: per-lane byte offset inside a pair / a tile
+};
+
+struct WRingColumn { int n, h0, w0; };
+
+__device__ __forceinline__ WRingColumn wring_column(int col, const WRingGeom& gm) {
+  WRingColumn c;
+  c.w0 = (col % gm.tiles_w) * kTW; col /= gm.tiles_w;
+  c.h0 = (col % gm.tiles_h) * kTH;
+  c.n = col / gm.tiles_h;
+  return c;
+}
+
+// Buffer offsets of the lane's voxels of the input pair whose first plane is `plane`, and of the gy tile whose first
+// plane is `d0`: out-of-range (zeros) for whatever lies outside the tensors; `live` false does that to all of it.
+__device__ __forceinline__ void wring_offsets(const WgradArgs& a, const WRingColumn& c, const WRingLane& ln, int plane, int d0, bool live,
+                                              int (&xoff)[kXGroupsPerWave], int& goff) {
+  const int ih0 = c.h0 - a.ph, iw0 = c.w0 - a.pw;
+#pragma unroll
+  for (int k = 0; k < kXGroupsPerWave; ++k) {
+    const int dl = ln.xcoord[k] & 0xff, bh = (ln.xcoord[k] >> 8) & 0xff, bw = (ln.xcoord[k] >> 16) & 0xff;
+    const int inside = (int)((unsigned)(plane + dl) < (unsigned)a.id) & (int)((unsigned)(ih0 + bh) < (unsigned)a.ih) &
+                       (int)((unsigned)(iw0 + bw) < (unsigned)a.iw) & (int)live;
+    xoff[k] = ln.xcoord[k] < 0 ? -1 : (inside ? ln.xrel[k] : kRange);
+  }
+  const int d = ln.gcoord & 0xff, h = (ln.gcoord >> 8) & 0xff, w = (ln.gcoord >> 16) & 0xff;
+  const int inside = (int)(d0 + d < a.od) & (int)(c.h0 + h < a.oh) & (int)(c.w0 + w < a.ow) & (int)live;
+  goff = inside ? ln.grel : kRange;
+}
+
+template <typename T>
+__device__ __forceinline__ void wring_fetch(char* xdst, char* gdst, int wave, const T* xorigin, const T* gorigin,
+                                            const int (&xoff)[kXGroupsPerWave], int goff) {
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xorigin), 0, kRange, 0x00020000);
+#pragma unroll
+  for (int k = 0; k < kXGroupsPerWave; ++k)
+    if (xoff[k] != -1) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (__attribute__((address_space(3))) void*)(xdst + (wave + 4 * k) * 1024 + p * kXPiece), 16,
+                                                 xoff[k] + p * 16, 0, 0, 0);
+    }
+  if (gdst != nullptr) {
+    const __amdgpu_buffer_rsrc_t gr = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin), 0, kRange, 0x00020000);
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(gr, (__attribute__((address_space(3))) void*)(gdst + wave * 1024 + p * kGPiece), 16, goff + p * 16,
+                                               0, 0, 0);
+  }
+}
+
+typedef short wring_v4s __attribute__((__vector_size__(4 * sizeof(short))));
+
+// A 32-channel x 16-voxel operand fragment from the piece planes at `p` (the lane's address of its first four voxels).
+__device__ __forceinline__ uint4 wring_fragment(const char* p) {
+  const wring_v4s r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) wring_v4s*)(p));
+  const wring_v4s r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) wring_v4s*)(p + 64));
+  uint4 out;
+  out.x = __builtin_bit_cast(uint2, r0).x; out.y = __builtin_bit_cast(uint2, r0).y;
+  out.z = __builtin_bit_cast(uint2, r1).x; out.w = __builtin_bit_cast(uint2, r1).y;
+  return out;
+}
+
+// One step of wavefront (s, G): the MFMAs of tap group G over the pairs `lo` (planes 0, 1) and `hi` (planes 2, 3) and the
+// gy tile `gt`, with the loads of the next step's pair and tile riding along.
+template <typename T, int G>
+struct WRingStep {
+  static constexpr const WSchedule& S = G == 0 ? kWSched0 : kWSched1;
+  static constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  const char* xlo;
+  const char* xhi;
+  const char* gt;
+  char* xfill;
+  char* gfill;
+  int wave;
+  f32x16_t (&acc)[NACC];
+  const int (&xoff)[kXGroupsPerWave];
+  int goff;
+  __amdgpu_buffer_rsrc_t xrsrc, grsrc;
+  uint4 gyf[kTD * kTH];
+  uint4 fr[WSchedule::kBuffers];
+
+  template <int F>
+  __device__ __forceinline__ void request() {
+    constexpr int d = S.fr_d[F], h = S.fr_h[F], kw = S.fr_kw[F];
+    constexpr int off = (((d % 2) * kBH + h) * kBW + kw) * 16;
+    fr[S.buffer[F]] = wring_fragment((d < 2 ? xlo : xhi) + off);
+  }
+  template <int F>
+  __device__ __forceinline__ void request_if_early() {
+    if constexpr (F < S.nf) {
+      if constexpr (S.issue_after[F] < 0) request<F>();
+    }
+  }
+  template <int... Fs>
+  __device__ __forceinline__ void prologue(std::integer_sequence<int, Fs...>) {
+#pragma unroll
+    for (int r = 0; r < kTD * kTH; ++r) gyf[r] = wring_fragment(gt + r * kTW * 16);
+    (request_if_early<Fs>(), ...);
+  }
+  template <int M>
+  __device__ __forceinline__ void mfma() {
+    if constexpr (M < S.nm) {
+      constexpr int f = S.mf_frag[M], ac = S.mf_acc[M], r = S.mf_gy[M];
+      __builtin_amdgcn_sched_barrier(0);
+      acc[ac] = Mma32<T>::run(gyf[r], fr[S.buffer[f]], acc[ac]);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (S.request_at[M] >= 0) {
+        request<S.request_at[M]>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (M % kSidePeriod == kSidePhase && M / kSidePeriod < kLoads) {
+        constexpr int slot = M / kSidePeriod;
+        if constexpr (slot < kXGroupsPerWave * 4) {
+          constexpr int k = slot / 4, p = slot % 4;
+          if (xoff[k] != -1)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, (__attribute__((address_space(3))) void*)(xfill + (wave + 4 * k) * 1024 + p * kXPiece),
+                                                     16, xoff[k] + p * 16, 0, 0, 0);
+        } else {
+          constexpr int p = slot - kXGroupsPerWave * 4;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(grsrc, (__attribute__((address_space(3))) void*)(gfill + wave * 1024 + p * kGPiece), 16,
+                                                   goff + p * 16, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  template <int... Ms>
+  __device__ __forceinline__ void run(std::integer_sequence<int, Ms...>) {
+    (mfma<Ms>(), ...);
+  }
+};
+
+template <typename T, int G>
+__device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws,
+                                          const WRingGeom& gm, int split, int cib, int cob, int x_cin, int tid, char* xp0, char* xp1,
+                                          char* xp2, char* gt0, char* gt1, char* gt2) {
+  constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int seg16 = wave & 1;  // which 16 voxels of every row this wavefront contracts over
+
+  WRingLane ln;
+#pragma unroll
+  for (int k = 0; k < kXGroupsPerWave; ++k) {
+    const int vox = (wave + 4 * k) * 64 + lane;
+    const int dl = vox / (kBH * kBW), r = vox % (kBH * kBW), bh = r / kBW, bw = r % kBW;
+    ln.xcoord[k] = vox < kXVoxels ? (dl | (bh << 8) | (bw << 16)) : -1;
+    ln.xrel[k] = ((dl * a.ih + bh) * a.iw + bw) * x_cin * 2;
+  }
+  {
+    const int vox = wave * 64 + lane;
+    const int d = vox / (kTH * kTW), h = (vox / kTW) % kTH, w = vox % kTW;
+    ln.gcoord = d | (h << 8) | (w << 16);
+    ln.grel = ((d * a.oh + h) * a.ow + w) * a.cout * 2;
+  }
+  {
+    // transposing read: 16-lane group q supplies channels 16 (q & 1) .. + 15 of voxels 8 (q >> 1) .. + 7; inside it lane m
+    // gives the address of channels 4 (m & 3) .. + 3 of voxel m >> 2
+    const int q = lane >> 4, m = lane & 15;
+    const int piece = 2 * (q & 1) + ((m & 3) >> 1);
+    const int vox = 8 * (q >> 1) + (m >> 2) + 16 * seg16;
+    ln.xread = piece * kXPiece + vox * 16 + (m & 1) * 8;
+    ln.gread = piece * kGPiece + vox * 16 + (m & 1) * 8;
+  }
+
+  f32x16_t acc[NACC];
+#pragma unroll
+  for (int t = 0; t < NACC; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+
+  const int item_begin = split * gm.items_per_split;
+  int item_end = item_begin + gm.items_per_split;
+  if (item_end > gm.items) item_end = gm.items;
+  const int ncols = gm.items / gm.segs;
+  int xoff[kXGroupsPerWave];
+  int goff;
+  for (int item = item_begin; item < item_end; ++item) {
+    const int seg = item / ncols;
+    const WRingColumn col = wring_column(item - seg * ncols, gm);
+    const int s_begin = seg * gm.seg_steps;
+    int s_end = s_begin + gm.seg_steps;
+    if (s_end > gm.steps) s_end = gm.steps;
+    const int nsteps = s_end - s_begin;
+    if (nsteps <= 0) continue;
+    const int plane0 = kTD * s_begin - a.pd;
+    auto xorigin = [&](int plane) {
+      return x + ((((int64_t)col.n * a.id + plane) * a.ih + (col.h0 - a.ph)) * a.iw + (col.w0 - a.pw)) * x_cin + cib * 32;
+    };
+    auto gorigin = [&](int d0) { return gy + ((((int64_t)col.n * a.od + d0) * a.oh + col.h0) * a.ow + col.w0) * a.cout + cob * 32; };
+
+    wring_offsets(a, col, ln, plane0, kTD * s_begin, true, xoff, goff);
+    wring_fetch<T>(xp0, gt0, wave, xorigin(plane0), gorigin(kTD * s_begin), xoff, goff);
+    wring_offsets(a, col, ln, plane0 + 2, 0, true, xoff, goff);
+    wring_fetch<T>(xp1, nullptr, wave, xorigin(plane0 + 2), gorigin(0), xoff, goff);
+    __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));
+    __builtin_amdgcn_s_barrier();
+
+    auto step = [&](int i, const char* lo, const char* hi, const char* gt, char* xfill, char* gfill) {
+      const int plane = plane0 + 2 * i + 4, d_next = kTD * (s_begin + i + 1);
+      wring_offsets(a, col, ln, plane, d_next, i + 1 < nsteps, xoff, goff);
+      WRingStep<T, G> st{lo + ln.xread, hi + ln.xread, gt + ln.gread, xfill, gfill, wave, acc, xoff, goff,
+                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xorigin(plane)), 0, kRange, 0x00020000),
+                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin(d_next)), 0, kRange, 0x00020000), {}, {}};
+      st.prologue(std::make_integer_sequence<int, WSchedule::kMaxFrags>{});
+      st.run(std::make_integer_sequence<int, WSchedule::kMaxMfmas>{});
+      __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));  // this wavefront's part of the next pair and tile has landed
+      __builtin_amdgcn_s_barrier();                     // ... and every wavefront is done reading this step's
+    };
+    for (int i = 0; i < nsteps; i += 3) {
+      step(i, xp0, xp1, gt0, xp2, gt1);
+      if (i + 1 < nsteps) step(i + 1, xp1, xp2, gt1, xp0, gt2);
+      if (i + 2 < nsteps) step(i + 2, xp2, xp0, gt2, xp1, gt0);
+    }
+  }
+
+  // The wavefronts (0, G) and (1, G) hold sums over different voxels for the same taps: the second hands its
+  // accumulators over through LDS (the last barrier has freed it), kHandTaps taps at a time through the group's own
+  // array, the first adds them -- a fixed order -- and writes the workgroup's slice.
+  char* handover = G == 0 ? xp0 : xp1;
+  float* dst = ws + ((int64_t)split * a.cout + cob * 32) * 27 * a.cin + cib * 32;
+  const int j = lane & 31, kg = lane >> 5;
+#pragma unroll
+  for (int round = 0; round < kHandRounds; ++round) {
+    if (seg16 == 1) {
+#pragma unroll
+      for (int t = round * kHandTaps; t < (round + 1) * kHandTaps; ++t) {
+        if (t >= NACC) continue;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+          *reinterpret_cast<float4*>(handover + ((t - round * kHandTaps) * 4 + r4) * 1024 + lane * 16) =
+              make_float4(acc[t][4 * r4], acc[t][4 * r4 + 1], acc[t][4 * r4 + 2], acc[t][4 * r4 + 3]);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __builtin_amdgcn_s_barrier();
+    if (seg16 == 0) {
+#pragma unroll
+      for (int t9 = 0; t9 < 9; ++t9)
+#pragma unroll
+        for (int kw = 0; kw < 3; ++kw) {
+          if (tap_group(t9, kw) != G) continue;
+          const int t = tap_slot(t9, kw), tap = t9 * 3 + kw;
+          if (t < round * kHandTaps || t >= (round + 1) * kHandTaps) continue;
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const float4 o = *reinterpret_cast<const float4*>(handover + ((t - round * kHandTaps) * 4 + r4) * 1024 + lane * 16);
+            const float v[4] = {acc[t][4 * r4] + o.x, acc[t][4 * r4 + 1] + o.y, acc[t][4 * r4 + 2] + o.z, acc[t][4 * r4 + 3] + o.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int co = 8 * r4 + 4 * kg + e;
+              dst[((int64_t)co * 27 + tap) * a.cin + j] = v[e];
+            }
+          }
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __builtin_amdgcn_s_barrier();  // the array is free for the next round
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256, 1)
+wgrad_ring_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws, WRingGeom gm, uint32_t total,
+                  const T* __restrict__ x1, int c_first) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char xp0[kXPair];
+  __shared__ __attribute__((aligned(16))) char xp1[kXPair];
+  __shared__ __attribute__((aligned(16))) char xp2[kXPair];
+  __shared__ __attribute__((aligned(16))) char gt0[kGTile];
+  __shared__ __attribute__((aligned(16))) char gt1[kGTile];
+  __shared__ __attribute__((aligned(16))) char gt2[kGTile];
+  const int tid = threadIdx.x;
+  const uint32_t wg = xcd_remap(blockIdx.x, total);
+  const int blk = wg % gm.nblk, split = wg / gm.nblk;
+  int cib = blk % gm.nblk_ci;
+  const int cob = blk / gm.nblk_ci;
+  // An input handed over as two tensors whose channels follow each other (the first c_first in x, the rest in x1): the
+  // workgroup's 32 input channels lie in one of them, and that tensor is the one staged; the gradient's own indexing
+  // keeps a.cin and the block's index in the whole.
+  const T* xs = x;
+  int x_cin = a.cin, cis = cib;
+  if (x1 != nullptr) {
+    const bool second = cib * 32 >= c_first;
+    xs = second ? x1 : x;
+    x_cin = second ? a.cin - c_first : c_first;
+    cis = second ? cib - c_first / 32 : cib;
+  }
+  // wavefronts 0, 1 hold tap group 0, wavefronts 2, 3 tap group 1 (wave-uniform branch)
+  WgradArgs as = a;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  float* wsb = ws;
+  if (wave < 2) {
+    // (the slice is indexed with the whole tensor's cin and block index)
+    wring_run<T, 0>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, xp0, xp1, xp2, gt0, gt1, gt2);
+  } else {
+    wring_run<T, 1>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, xp0, xp1, xp2, gt0, gt1, gt2);
+  }
+#endif
+}
+
+WRingGeom wring_geom(const WgradArgs& a) {
+  WRingGeom gm{};
+  gm.tiles_h = (int)cdiv(a.oh, kTH);
+  gm.tiles_w = (int)cdiv(a.ow, kTW);
+  gm.steps = (int)cdiv(a.od, kTD);
+  gm.nblk_ci = a.cin / 32;
+  gm.nblk = gm.nblk_ci * (a.cout / 32);
+  const int64_t ncols = (int64_t)a.n * gm.tiles_h * gm.tiles_w;
+  int want = kComputeUnits / gm.nblk;  // workgroups per block: at most one workgroup per CU over all blocks
+  if (want < 1) want = 1;
+  int64_t segs = ncols >= want ? 1 : cdiv(want, ncols);
+  if (segs > gm.steps) segs = gm.steps;
+  gm.seg_steps = (int)cdiv(gm.steps, segs);
+  gm.segs = (int)cdiv(gm.steps, gm.seg_steps);
+  const int64_t items = ncols * gm.segs;
+  gm.items = items > 0x7fffffffLL ? -1 : (int)items;
+  if (gm.items > 0) {
+    if (want > gm.items) want = gm.items;
+    gm.items_per_split = (int)cdiv(gm.items, want);
+    gm.splits = (int)cdiv(gm.items, gm.items_per_split);
+  }
+  return gm;
+}
+
+template <typename T>
+int launch_wring(const WgradArgs& a, const WRingGeom& gm, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2) {
+  const int64_t total = (int64_t)gm.splits * gm.nblk;
+  hipLaunchKernelGGL((wgrad_ring_kernel<T>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x, (const T*)gy, ws, gm, (uint32_t)total,
+                     (const T*)x2.second, x2.first);
+  return check_launch("wgrad_ring_kernel");
+}
+
+}  // namespace
+
+// Rows of more than 16 voxels; a plane pair with its halo and a gy tile must span less than the buffer range.
+bool mfma_wgrad_ring_applies(const WgradArgs& a) {
+  if (a.ow <= 16 || a.od < 1 || a.oh < 1 || a.n < 1) return false;
+  if (((int64_t)(a.ih + kBH) * a.iw + kBW) * a.cin * 2 + 64 >= kRange || ((int64_t)(a.oh + kTH) * a.ow + kTW) * a.cout * 2 + 64 >= kRange)
+    return false;
+  return wring_geom(a).items > 0;
+}
+
+int mfma_wgrad_ring_splits(const WgradArgs& a) { return wring_geom(a).splits; }
+
+int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2) {
+  const WRingGeom gm = wring_geom(a);
+  if (dtype == SFH_BF16) return launch_wring<bf16_t>(a, gm, x, gy, ws, st, x2);
+  return launch_wring<fp16_t>(a, gm, x, gy, ws, st, x2);
+}
+
+}  // namespace sfh
