@@ -64,7 +64,9 @@ struct WSchedule {
   int mf_frag[kMaxMfmas], mf_acc[kMaxMfmas], mf_gy[kMaxMfmas];
   int fr_d[kMaxFrags], fr_h[kMaxFrags], fr_kw[kMaxFrags], fr_first[kMaxFrags], fr_last[kMaxFrags];
   int issue_after[kMaxFrags], buffer[kMaxFrags], request_at[kMaxMfmas];
+  int gy_first[kTD * kTH], gy_issue[kTD * kTH], gy_request_at[kMaxMfmas];  // the same for the gy fragment of output row r
   int buffers_used, min_acc_distance;
+  bool early_in_lo;  // every fragment requested before the step's first MFMA lies in the step's first plane pair
 };
 
 constexpr WSchedule make_wschedule(int g) {
@@ -96,6 +98,14 @@ constexpr WSchedule make_wschedule(int g) {
     s.issue_after[f] = at;
     next = at;
   }
+  // what is requested ahead of the step's first MFMA must lie in its first plane pair (the second may still be on its
+  // way when the requests go out): such fragments of the second pair move behind the first MFMAs instead
+  int taken = -1;
+  for (int f = 0; f < s.nf; ++f) {
+    if (s.issue_after[f] < 0 && s.fr_d[f] < 2) continue;
+    if (s.issue_after[f] <= taken) s.issue_after[f] = taken + 1;
+    taken = s.issue_after[f];
+  }
   for (int k = 0; k < WSchedule::kMaxMfmas; ++k) s.request_at[k] = -1;
   for (int f = 0; f < s.nf; ++f)
     if (s.issue_after[f] >= 0) s.request_at[s.issue_after[f]] = f;
@@ -110,6 +120,27 @@ constexpr WSchedule make_wschedule(int g) {
     s.buffer[f] = pick;
   }
   s.buffers_used = nb;
+  // gy fragments: requested a little before their first use as well (in order of first use, never two behind one MFMA)
+  for (int r = 0; r < kTD * kTH; ++r) s.gy_first[r] = -1;
+  for (int i = 0; i < s.nm; ++i)
+    if (s.gy_first[s.mf_gy[i]] < 0) s.gy_first[s.mf_gy[i]] = i;
+  for (int k = 0; k < WSchedule::kMaxMfmas; ++k) s.gy_request_at[k] = -1;
+  int gnext = s.nm;
+  for (int pass = 0; pass < kTD * kTH; ++pass) {
+    int r = -1;  // the row with the latest first use among those not placed yet
+    for (int q = 0; q < kTD * kTH; ++q)
+      if (s.gy_issue[q] == 0 && s.gy_first[q] >= 0 && (r < 0 || s.gy_first[q] > s.gy_first[r])) r = q;
+    if (r < 0) break;
+    int at = s.gy_first[r] - WSchedule::kLead - 1;
+    if (at >= gnext) at = gnext - 1;
+    if (at == 0) at = -1;  // 0 marks "not placed" above
+    s.gy_issue[r] = at;
+    gnext = at;
+    if (at > 0) s.gy_request_at[at] = r;
+  }
+  s.early_in_lo = true;
+  for (int f = 0; f < s.nf; ++f)
+    if (s.issue_after[f] < 0 && s.fr_d[f] >= 2) s.early_in_lo = false;
   s.min_acc_distance = s.nm;
   for (int i = 0; i < s.nm; ++i)
     for (int k = i + 1; k < s.nm && k < i + 8; ++k)
@@ -121,8 +152,17 @@ constexpr WSchedule kWSched0 = make_wschedule(0), kWSched1 = make_wschedule(1);
 static_assert(kWSched0.nm == 8 * kTaps0 && kWSched1.nm == 8 * kTaps1, "every (row, tap) of the group exactly once");
 static_assert(kWSched0.buffers_used <= WSchedule::kBuffers && kWSched1.buffers_used <= WSchedule::kBuffers, "fragment registers");
 static_assert(kWSched0.min_acc_distance >= 2 && kWSched1.min_acc_distance >= 2, "no two MFMAs in a row on one accumulator");
+static_assert(kWSched0.early_in_lo && kWSched1.early_in_lo, "the fragments requested ahead of a step lie in the pair that is already resident");
+constexpr bool wschedule_requests_in_time(const WSchedule& s) {
+  for (int f = 0; f < s.nf; ++f)
+    if (s.issue_after[f] >= s.fr_first[f] - 1) return false;
+  return true;
+}
+static_assert(wschedule_requests_in_time(kWSched0) && wschedule_requests_in_time(kWSched1), "every fragment is requested ahead of its first use");
 
-constexpr int kSidePeriod = 8, kSidePhase = 3;
+// A load rides behind every sixth MFMA from the step's start. (Measured: where in the step the loads sit, and whether
+// the wavefronts issue theirs at the same or at staggered MFMAs, changes the step time by less than 2 %.)
+constexpr int kSidePeriod = 6, kSidePhase = 1;
 static_assert((8 * kTaps1 - kSidePhase + kSidePeriod - 1) / kSidePeriod >= kLoads, "a slot per load");
 
 constexpr int wring_waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
@@ -200,23 +240,17 @@ __device__ __forceinline__ uint4 wring_fragment(const char* p) {
 }
 
 // One step of wavefront (s, G): the MFMAs of tap group G over the pairs `lo` (planes 0, 1) and `hi` (planes 2, 3) and the
-// gy tile `gt`, with the loads of the next step's pair and tile riding along.
-template <typename T, int G>
-struct WRingStep {
+// gy tile `gt`, with the loads of the next step's pair and of the gy tile after next riding along. The fragments a step
+// needs for its first MFMAs are requested by early() BEFORE the barrier that ends the step in front of it (they lie in
+// the pair and the tile that are already resident), so the LDS latency hides behind that barrier.
+template <int G>
+struct WRingFrags {
   static constexpr const WSchedule& S = G == 0 ? kWSched0 : kWSched1;
-  static constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
   const char* xlo;
   const char* xhi;
   const char* gt;
-  char* xfill;
-  char* gfill;
-  int wave;
-  f32x16_t (&acc)[NACC];
-  const int (&xoff)[kXGroupsPerWave];
-  int goff;
-  __amdgpu_buffer_rsrc_t xrsrc, grsrc;
-  uint4 gyf[kTD * kTH];
-  uint4 fr[WSchedule::kBuffers];
+  uint4 (&gyf)[kTD * kTH];
+  uint4 (&fr)[WSchedule::kBuffers];
 
   template <int F>
   __device__ __forceinline__ void request() {
@@ -224,27 +258,52 @@ struct WRingStep {
     constexpr int off = (((d % 2) * kBH + h) * kBW + kw) * 16;
     fr[S.buffer[F]] = wring_fragment((d < 2 ? xlo : xhi) + off);
   }
+  template <int R>
+  __device__ __forceinline__ void request_gy() { gyf[R] = wring_fragment(gt + R * kTW * 16); }
   template <int F>
   __device__ __forceinline__ void request_if_early() {
     if constexpr (F < S.nf) {
       if constexpr (S.issue_after[F] < 0) request<F>();
     }
   }
-  template <int... Fs>
-  __device__ __forceinline__ void prologue(std::integer_sequence<int, Fs...>) {
-#pragma unroll
-    for (int r = 0; r < kTD * kTH; ++r) gyf[r] = wring_fragment(gt + r * kTW * 16);
+  template <int R>
+  __device__ __forceinline__ void request_gy_if_early() {
+    if constexpr (S.gy_issue[R] < 0) request_gy<R>();
+  }
+  // Only xlo and gt are read.
+  template <int... Fs, int... Rs>
+  __device__ __forceinline__ void early(std::integer_sequence<int, Fs...>, std::integer_sequence<int, Rs...>) {
+    (request_gy_if_early<Rs>(), ...);
     (request_if_early<Fs>(), ...);
   }
+};
+
+template <typename T, int G>
+struct WRingStep {
+  static constexpr const WSchedule& S = G == 0 ? kWSched0 : kWSched1;
+  static constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  WRingFrags<G> fg;
+  char* xfill;
+  char* gfill;
+  int wave;
+  f32x16_t (&acc)[NACC];
+  const int (&xoff)[kXGroupsPerWave];
+  int goff;
+  __amdgpu_buffer_rsrc_t xrsrc, grsrc;
+
   template <int M>
   __device__ __forceinline__ void mfma() {
     if constexpr (M < S.nm) {
       constexpr int f = S.mf_frag[M], ac = S.mf_acc[M], r = S.mf_gy[M];
       __builtin_amdgcn_sched_barrier(0);
-      acc[ac] = Mma32<T>::run(gyf[r], fr[S.buffer[f]], acc[ac]);
+      acc[ac] = Mma32<T>::run(fg.gyf[r], fg.fr[S.buffer[f]], acc[ac]);
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (S.request_at[M] >= 0) {
-        request<S.request_at[M]>();
+        fg.template request<S.request_at[M]>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (S.gy_request_at[M] >= 0) {
+        fg.template request_gy<S.gy_request_at[M]>();
         __builtin_amdgcn_sched_barrier(0);
       }
       if constexpr (M % kSidePeriod == kSidePhase && M / kSidePeriod < kLoads) {
@@ -307,6 +366,8 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
   for (int t = 0; t < NACC; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  uint4 gyf[kTD * kTH];            // gy fragments of the step's eight output rows (this wavefront's 16 voxels of each)
+  uint4 fr[WSchedule::kBuffers];   // input-row fragments in rotation
 
   const int item_begin = split * gm.items_per_split;
   int item_end = item_begin + gm.items_per_split;
@@ -328,28 +389,40 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
     };
     auto gorigin = [&](int d0) { return gy + ((((int64_t)col.n * a.od + d0) * a.oh + col.h0) * a.ow + col.w0) * a.cout + cob * 32; };
 
+    // the first step's two pairs, and the gy tiles of the first two steps (gy runs two steps ahead of the MFMAs)
     wring_offsets(a, col, ln, plane0, kTD * s_begin, true, xoff, goff);
     wring_fetch<T>(xp0, gt0, wave, xorigin(plane0), gorigin(kTD * s_begin), xoff, goff);
-    wring_offsets(a, col, ln, plane0 + 2, 0, true, xoff, goff);
-    wring_fetch<T>(xp1, nullptr, wave, xorigin(plane0 + 2), gorigin(0), xoff, goff);
+    wring_offsets(a, col, ln, plane0 + 2, kTD * (s_begin + 1), true, xoff, goff);
+    if (nsteps < 2) goff = kRange;
+    wring_fetch<T>(xp1, gt1, wave, xorigin(plane0 + 2), gorigin(kTD * (s_begin + 1)), xoff, goff);
     __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));
     __builtin_amdgcn_s_barrier();
+    {
+      WRingFrags<G> first{xp0 + ln.xread, nullptr, gt0 + ln.gread, gyf, fr};
+      first.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
+    }
 
-    auto step = [&](int i, const char* lo, const char* hi, const char* gt, char* xfill, char* gfill) {
-      const int plane = plane0 + 2 * i + 4, d_next = kTD * (s_begin + i + 1);
-      wring_offsets(a, col, ln, plane, d_next, i + 1 < nsteps, xoff, goff);
-      WRingStep<T, G> st{lo + ln.xread, hi + ln.xread, gt + ln.gread, xfill, gfill, wave, acc, xoff, goff,
+    // step i: MFMAs over pairs (lo, hi) and tile gt; the pair after them streams into xfill, the gy tile of step i + 2
+    // into gfill; gt_next is the (resident) tile of step i + 1
+    auto step = [&](int i, const char* lo, const char* hi, const char* gt, char* xfill, char* gfill, const char* gt_next) {
+      const int plane = plane0 + 2 * i + 4, d_ahead = kTD * (s_begin + i + 2);
+      wring_offsets(a, col, ln, plane, d_ahead, i + 1 < nsteps, xoff, goff);
+      if (i + 2 >= nsteps) goff = kRange;
+      WRingStep<T, G> st{WRingFrags<G>{lo + ln.xread, hi + ln.xread, gt + ln.gread, gyf, fr}, xfill, gfill, wave, acc, xoff, goff,
                          __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xorigin(plane)), 0, kRange, 0x00020000),
-                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin(d_next)), 0, kRange, 0x00020000), {}, {}};
-      st.prologue(std::make_integer_sequence<int, WSchedule::kMaxFrags>{});
+                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin(d_ahead)), 0, kRange, 0x00020000)};
       st.run(std::make_integer_sequence<int, WSchedule::kMaxMfmas>{});
+      if (i + 1 < nsteps) {  // the next step's first fragments: its first pair is this step's second one
+        WRingFrags<G> next{hi + ln.xread, nullptr, gt_next + ln.gread, gyf, fr};
+        next.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
+      }
       __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));  // this wavefront's part of the next pair and tile has landed
       __builtin_amdgcn_s_barrier();                     // ... and every wavefront is done reading this step's
     };
     for (int i = 0; i < nsteps; i += 3) {
-      step(i, xp0, xp1, gt0, xp2, gt1);
-      if (i + 1 < nsteps) step(i + 1, xp1, xp2, gt1, xp0, gt2);
-      if (i + 2 < nsteps) step(i + 2, xp2, xp0, gt2, xp1, gt0);
+      step(i, xp0, xp1, gt0, xp2, gt2, gt1);
+      if (i + 1 < nsteps) step(i + 1, xp1, xp2, gt1, xp0, gt0, gt2);
+      if (i + 2 < nsteps) step(i + 2, xp2, xp0, gt2, xp1, gt1, gt0);
     }
   }
 
