@@ -357,3 +357,19 @@ def test_train_step_loss_weighted_ce_closed_form():
     dice1 = (2 * i1 + 1e-6) / (p1 + 1.0 + 1e-6)
     got = orc.train_step_loss(logits, labels, 2, class_weight=w, dtype=torch.float64)
     assert abs(got.item() - (ce + 1 - dice1)) < 1e-12
+
+
+def test_committed_ifs_shard_is_the_pinned_generators_output():
+    """bench.py and the full-size checks read config 5's input from tests/golden/ifs_cfg5_shard.npz; it must be exactly
+    what ``ifs_volume`` (pinned above by its closed forms) produces for 128^3, 2e5 iterations, seed 5000, planes 0..63."""
+    import os
+
+    import numpy as np
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "ifs_cfg5_shard.npz")
+    with np.load(path) as f:
+        labels, grid, depth, iterations, seed = f["labels"], int(f["grid"]), int(f["depth"]), int(f["iterations"]), int(f["seed"])
+    assert (grid, depth, iterations, seed) == (128, 64, 200_000, 5000) and labels.dtype == np.uint8 and labels.shape == (64, 128, 128)
+    occ, lab = orc.ifs_volume(grid, iterations=iterations, seed=seed)
+    assert np.array_equal(lab[0, :depth].numpy(), labels.astype(np.int64))
+    assert 0.01 < float((labels > 0).mean()) < 0.2 and labels.max() <= 10
