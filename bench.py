@@ -672,9 +672,10 @@ def conv_table(device, iters=20):
 
 def conv_counter_launches(device, reps=3):
     """The launches a counter run (rocprofv3 --pmc) is taken over: plain eager calls, no graph, of the three MFMA
-    convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_persist_kernel,
-    wgrad_mfma_kernel), 128->64 @64^3 and 64->32 on the 64x128x128 slab (conv_mfma_kernel, wgrad_mfma_kernel), the last
-    also with its input as two 32-channel tensors (what the U-Net's decoder hands it)."""
+    convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_ring_kernel,
+    wgrad_ring_kernel), 128->64 @64^3 (conv_wide_kernel, conv_mfma_kernel, wgrad_ring_kernel) and 64->32 on the 64x128x128
+    slab (conv_mfma_kernel, conv_ring_kernel, wgrad_ring_kernel), the last also with its input as two 32-channel tensors
+    (what the U-Net's decoder hands it)."""
     import scaffold_amd as sa
 
     done = []
@@ -972,7 +973,7 @@ def main():
     flops = conv["flops_per_direction"]
     fwd_ms = conv["in_step_ms"]["fwd"]
     achieved = flops / (fwd_ms * 1e-3) / 1e12
-    traffic, traffic_source = counter_traffic("conv_persist_kernel")
+    traffic, traffic_source = counter_traffic("conv_ring_kernel")
     # the measured ceiling of this run for the kernel's MFMA + LDS-read mix on Gaussian operands, no global traffic
     # (beside, never instead of, the nominal peak)
     ceiling = None
@@ -1017,11 +1018,11 @@ def main():
         "config": {"workload": "conv3d 3x3x3 stride 1 pad 1, Cin=Cout=32, 128^3, N=1, NDHWC bf16: fwd + dgrad + wgrad "
                                "(BASELINE.json config 3, first encoder level)"},
         "roofline": {
-            "bound": "mfma", "kernel": "conv_persist_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
+            "bound": "mfma", "kernel": "conv_ring_kernel (forward)", "achieved": achieved, "peak": MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
             "flops_per_launch": flops, "avg_launch_ms": fwd_ms,
             "measured_ceiling_tflops": ceiling, "frac_of_measured_ceiling": None if not ceiling else achieved / ceiling,
-            # the other two launches of the step, same FLOPs per launch (wgrad = wgrad_mfma_kernel + its slice sum)
+            # the other two launches of the step, same FLOPs per launch (wgrad = wgrad_ring_kernel + its slice sum)
             "frac_by_direction": {k: flops / (v * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS for k, v in conv["in_step_ms"].items()},
         },
         "cpu_baseline": cpu,

@@ -23,10 +23,6 @@
 // The data gradient runs this same kernel with the weight packed transposed and tap-flipped and
 // padding k-1-p (triton_conv3d/bwd_data.py:344-363).
 #include "conv_mfma.hpp"
-#ifdef SFH_GATHER_TUNE
-#include <cstdio>
-#include <cstdlib>
-#endif
 #include "mma.hpp"
 #include "gn_stats.hpp"
 #include "reduce.hpp"
@@ -75,7 +71,7 @@ template <typename T, typename C, int WQ, bool PAIR>
 __global__ void __launch_bounds__(256, 2)
 conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ wp, const T* __restrict__ bias,
                  T* __restrict__ y, float* __restrict__ partial, int tiles_d, int tiles_h, int tiles_w, int nblocks, int ksplit,
-                 uint32_t total, GnPartialOut gn, int early_weights, const T* __restrict__ x1, T* __restrict__ y1, int c_first) {
+                 uint32_t total, GnPartialOut gn, const T* __restrict__ x1, T* __restrict__ y1, int c_first) {
   __shared__ __attribute__((aligned(16))) char lds[C::LDS];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -132,12 +128,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     constexpr int WWANT = WQ;
     constexpr int WDEPTH = NIT < WWANT ? NIT : WWANT;
     uint4 wq[NIT][C::NSUB];  // fully unrolled: every slot is its own register set, live for WDEPTH iterations
-    constexpr bool CAN_EARLY = C::NSUB == 1;  // with two output blocks the staging needs the registers
-#ifdef SFH_GATHER_TUNE  // a tuning build can switch it off per launch to measure it
-    const bool early = CAN_EARLY && early_weights != 0;
-#else
-    constexpr bool early = CAN_EARLY;
-#endif
+    // a chunk's first weight requests go out ahead of its brick staging; with two output blocks the staging needs the registers
+    constexpr bool early = C::NSUB == 1;
     if (early) {
 #pragma unroll
       for (int it = 0; it < WDEPTH; ++it) wq[it][0] = *reinterpret_cast<const uint4*>(wcc + it * FRAG);
@@ -389,19 +381,6 @@ GatherPlan gather_plan(const MfmaConvArgs& a) {
   GatherPlan p{};
   const int cls = a.ow > 16 ? 0 : (a.ow > 8 ? 1 : 2);
   const int ncc = a.cred / kChunk;
-#ifdef SFH_GATHER_TUNE
-  if (const char* e = getenv("SFH_GATHER_FORCE")) {
-    int size = 0, nsub = 1, ksplit = 1;
-    if (sscanf(e, "%d,%d,%d", &size, &nsub, &ksplit) == 3 && size >= 0 && size < 3 && (nsub == 1 || (nsub == 2 && a.cout % 64 == 0)) &&
-        ksplit >= 1 && ksplit <= ncc) {
-      p.shape = cls * 3 + size;
-      p.tiles = tiles_of(a, cls, size);
-      p.nsub = nsub;
-      p.ksplit = ksplit;
-      return p;
-    }
-  }
-#endif
   int64_t best = -1, best_wgs = 0;
   for (int size = 0; size < 2; ++size) {
     const int* t = kTileDims[cls][size];
@@ -423,15 +402,6 @@ GatherPlan gather_plan(const MfmaConvArgs& a) {
   return p;
 }
 
-// A chunk's first weight requests ahead of its brick staging: always, except that a tuning build reads an override.
-int early_weights(int64_t workgroups) {
-#ifdef SFH_GATHER_TUNE
-  if (const char* e = getenv("SFH_EARLY_WEIGHTS")) return atoi(e) == 2 ? (workgroups <= 2 * kComputeUnits) : atoi(e);
-#endif
-  (void)workgroups;
-  return 1;
-}
-
 struct PairPtrs { const void* x1; void* y1; int first; };
 
 template <typename T, typename C, bool PAIR>
@@ -445,7 +415,7 @@ int launch_cfg(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const 
 #define SFH_BRICK(WQ)                                                                                                      \
   hipLaunchKernelGGL((conv_mfma_kernel<T, C, WQ, PAIR>), dim3((unsigned)total), dim3(256), 0, st, a, (const T*)x,       \
                      (const T*)packed, (const T*)bias, (T*)y, partial, tiles_d, tiles_h, tiles_w, nblocks, p.ksplit,       \
-                     (uint32_t)total, gn, early_weights(total), (const T*)pr.x1, (T*)pr.y1, pr.first)
+                     (uint32_t)total, gn, (const T*)pr.x1, (T*)pr.y1, pr.first)
   if constexpr (C::NSUB > 1) SFH_BRICK(4);
   else if constexpr (C::MS >= 4) SFH_BRICK(6);
   else if (total <= 2 * kComputeUnits) SFH_BRICK(12);
@@ -465,11 +435,6 @@ int launch_k333(const MfmaConvArgs& a, const GatherPlan& p, const void* x, const
     case 1: return launch_cfg<T, Tile<2, 4, 32, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
     case 4: return launch_cfg<T, Tile<2, 8, 16, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
     case 7: return launch_cfg<T, Tile<4, 8, 8, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
-#ifdef SFH_GATHER_TUNE  // 128-voxel tiles: built only to be measured
-    case 2: return launch_cfg<T, Tile<1, 4, 32, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
-    case 5: return launch_cfg<T, Tile<1, 8, 16, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
-    case 8: return launch_cfg<T, Tile<2, 8, 8, 3, 3, 3, NSUB>, PAIR>(a, p, x, packed, bias, y, partial, st, gn, pr);
-#endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv mfma: no kernel for brick shape %d", p.shape);
   }
 }

@@ -10,9 +10,6 @@
 // [voxel][channel] layout and read with ds_read_b64_tr_b16, which hands each lane four consecutive
 // voxels of one channel.
 #include "conv_patch.hpp"
-#ifdef SFH_PATCH_TUNE
-#include <cstdlib>
-#endif
 #include <type_traits>
 #include "mma.hpp"
 #include "reduce.hpp"
@@ -364,18 +361,11 @@ int launch_scatter(const PatchArgs& a, const void* small, const void* packed, co
   const int64_t face_pieces = halo_elems > 0 ? halo_elems * (int64_t)sizeof(T) / 16 : 0;
   dim3 grid((unsigned)cdiv(total, 128), (unsigned)(a.cbig / 32));
   const int64_t wgs = (int64_t)grid.x * grid.y;
-  int force = 0;
-#ifdef SFH_PATCH_TUNE
-  if (const char* e = getenv("SFH_SCATTER_TS")) force = atoi(e);
-#endif
-  if (force == 8) {
-    hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
-                       (const T*)bias, (T*)big, total, face_pieces, big_elems);
-  } else if (force == 1 || (force == 0 && wgs < kComputeUnits)) {  // under one workgroup per CU: one tap per workgroup
+  if (wgs < kComputeUnits) {  // under one workgroup per CU: one tap per workgroup
     grid.z = kTaps;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total, face_pieces, big_elems);
-  } else if (force == 2 || (force == 0 && wgs <= 4 * kComputeUnits)) {  // up to four per CU: two taps (the big voxels next to each other along W)
+  } else if (wgs <= 4 * kComputeUnits) {  // up to four per CU: two taps (the big voxels next to each other along W)
     grid.z = kTaps / 2;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total, face_pieces, big_elems);

@@ -483,11 +483,7 @@ int launch_typed(const MfmaConvArgs& a, const void* x, const void* packed, const
 
 // Rows of more than 16 voxels take the column-walking form of the persistent kernel.
 static bool ring_serves(const MfmaConvArgs& a) {
-#ifdef SFH_NO_RING
-  return false;
-#else
   return mfma_conv_ring_applies(a) && a.od > 0 && a.n > 0;
-#endif
 }
 
 // The persistent kernel pays off when the weight slab stays in registers for the whole launch, i.e. with a

@@ -399,22 +399,13 @@ WidePlan wide_plan(const MfmaConvArgs& a) {
   // a brick (at most 10 input planes and 6 rows) must span less than kRange bytes of the input
   if (((int64_t)10 * a.ih + 6) * a.iw * a.cred * 2 + 64 >= kRange) return p;
   int shape = -1;
-#ifdef SFH_WIDE_TUNE
-  if (const char* e = getenv("SFH_WIDE_FORCE")) {
-    shape = atoi(e);
-    if (shape < 0 || shape > 4) return p;
-    if ((shape == 0 && a.cout % 128 != 0) || ((shape == 1 || shape == 3) && a.cout % 64 != 0)) return p;
-  } else
-#endif
-  {
-    // Measured against the brick-per-workgroup kernel on every shape of the U-Net and of the cube configurations, this
-    // kernel wins where a 64-channel output meets 128 or more reduction channels (one workgroup then produces all of a
-    // voxel's channels from one staged brick): 8 x 2 accumulator blocks per wavefront when such workgroups fill the
-    // chip, else 4 x 2. Everything else stays with the other kernels.
-    if (a.cout == 64 && a.cred >= 128) {
-      if (wide_workgroups(a, 1) >= kComputeUnits) shape = 1;
-      else if (wide_workgroups(a, 3) >= kComputeUnits) shape = 3;
-    }
+  // Measured against the brick-per-workgroup kernel on every shape of the U-Net and of the cube configurations, this
+  // kernel wins where a 64-channel output meets 128 or more reduction channels (one workgroup then produces all of a
+  // voxel's channels from one staged brick): 8 x 2 accumulator blocks per wavefront when such workgroups fill the
+  // chip, else 4 x 2. Everything else stays with the other kernels.
+  if (a.cout == 64 && a.cred >= 128) {
+    if (wide_workgroups(a, 1) >= kComputeUnits) shape = 1;
+    else if (wide_workgroups(a, 3) >= kComputeUnits) shape = 3;
   }
   if (shape < 0) return p;
   p.use = true;
@@ -449,11 +440,6 @@ int launch_typed(const MfmaConvArgs& a, const WidePlan& p, const void* x, const 
   switch (p.shape) {
     case 1: return launch_wide<T, WTile<8, 4, 32, 2>>(a, x, packed, bias, y, st, gn, x1);
     case 3: return launch_wide<T, WTile<4, 4, 32, 2>>(a, x, packed, bias, y, st, gn, x1);
-#ifdef SFH_WIDE_TUNE  // the other accumulator grids: built only to be measured
-    case 0: return launch_wide<T, WTile<4, 4, 32, 4>>(a, x, packed, bias, y, st, gn, x1);
-    case 2: return launch_wide<T, WTile<8, 4, 32, 1>>(a, x, packed, bias, y, st, gn, x1);
-    case 4: return launch_wide<T, WTile<4, 4, 32, 1>>(a, x, packed, bias, y, st, gn, x1);
-#endif
     default: return fail(SFH_ERR_UNSUPPORTED, "conv wide: no kernel for accumulator grid %d", p.shape);
   }
 }

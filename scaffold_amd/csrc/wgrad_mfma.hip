@@ -22,9 +22,6 @@
 // walks the tiles of its K range; the next tile's operands are fetched into registers before the
 // current tile's MFMAs start, so global-memory latency is hidden behind the compute.
 #include "wgrad_mfma.hpp"
-#ifdef SFH_WGRAD_TUNE
-#include <cstdlib>
-#endif
 #include <type_traits>
 
 #include "mma.hpp"
@@ -402,13 +399,7 @@ struct Plan {
 };
 
 // Rows of more than 16 voxels take the column-walking kernel.
-bool ring_serves(const WgradArgs& a) {
-#ifdef SFH_NO_WRING
-  return false;
-#else
-  return mfma_wgrad_ring_applies(a);
-#endif
-}
+bool ring_serves(const WgradArgs& a) { return mfma_wgrad_ring_applies(a); }
 
 Plan make_plan(const WgradArgs& a) {
   Plan p{};
@@ -433,9 +424,6 @@ Plan make_plan(const WgradArgs& a) {
   // (a launch of its own). Units of 0.01 us, constants fitted to timings of the U-Net's levels: the small-volume
   // levels (8 tiles for 64-128 blocks) are cheaper with 1-4 slices than with one per CU.
   int target = kTargetWorkgroups;
-#ifdef SFH_WGRAD_TUNE
-  if (const char* e = getenv("SFH_WGRAD_WANT")) target = atoi(e) > 0 ? atoi(e) : target;
-#endif
   int want = target / p.nblk;
   if (want < 1) want = 1;
   if (want > p.ntiles) want = p.ntiles;
