@@ -289,6 +289,15 @@ def bench_groupnorm(args, device):
     fwd_ms = event_time_ms(abi_fwd, 20)
     bwd_ms = event_time_ms(abi_bwd, 20)
 
+    # The stream floor these passes are held to, measured in this run: the library's plain copy kernel on this very tensor
+    # (B read + B written, 16-byte accesses, nothing computed). 3 B / 5 B at that rate is what a GroupNorm that did nothing
+    # but move its algorithmic bytes would take on this chip.
+    def abi_copy():
+        _lib.check(L.sfh_stream_copy(P(x), P(y), B, stream), "sfh_stream_copy")
+
+    copy_ms = event_time_ms(abi_copy, 20)
+    copy_gbs = 2 * B / (copy_ms * 1e-3) / 1e9
+
     # The same normalisation fed by the convolution in front of it (what every GroupNorm of the U-Net step runs): a
     # 64 -> 64 convolution of this shape leaves the per-group sums of its output, the forward is then one read and one
     # write of the tensor (2 B) instead of two reads and a write (3 B).
@@ -314,6 +323,12 @@ def bench_groupnorm(args, device):
         "fwd_ms": fwd_ms, "fwd_gbs": 3 * B / (fwd_ms * 1e-3) / 1e9, "fwd_frac_of_hbm_peak": 3 * B / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "bwd_ms": bwd_ms, "bwd_gbs": 5 * B / (bwd_ms * 1e-3) / 1e9, "bwd_frac_of_hbm_peak": 5 * B / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "torch_op_fwd_ms": op_fwd_ms, "torch_op_bwd_ms": op_bwd_ms,
+        "measured_stream_floor": {
+            "what": "sfh_stream_copy of the same tensor (B read + B written) in this run; floors = 3 B / 5 B at that rate",
+            "copy_ms": copy_ms, "copy_gbs": copy_gbs, "copy_frac_of_hbm_peak": copy_gbs / HBM_PEAK_GBS,
+            "fwd_floor_ms": 3 * B / (copy_gbs * 1e9) * 1e3, "bwd_floor_ms": 5 * B / (copy_gbs * 1e9) * 1e3,
+            "fwd_frac_of_floor": (3 * B / (copy_gbs * 1e9) * 1e3) / fwd_ms, "bwd_frac_of_floor": (5 * B / (copy_gbs * 1e9) * 1e3) / bwd_ms,
+        },
     }
 
 

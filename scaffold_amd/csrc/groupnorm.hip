@@ -153,6 +153,12 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
   const int r = tid / tpr, cv = tid - r * tpr;
   const bool active = r < rpp;
   const T* xs = x + (int64_t)n * S * C + cv * V;
+  const int64_t begin = (int64_t)split * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  constexpr int U = 4;  // rows per batch: the next batch's loads are in flight while the current one is summed
 
   // Shift K: mean of every group over the first voxels of the sample, bit-identical in every
   // workgroup of the sample because it is computed from the same rows in the same order.
@@ -161,13 +167,16 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
 #pragma unroll
   for (int s = 0; s < SLOTS; ++s) kv[s] = 0.f;
   if (active) {
-    for (int64_t row = r; row < krows; row += rpp) {
+    for (int64_t krow = r; krow < krows; krow += rpp) {
       float f[V];
-      Ld<T, V>::run(xs + row * C, f);
+      Ld<T, V>::run(xs + krow * C, f);
 #pragma unroll
       for (int e = 0; e < V; ++e) kv[e * SLOTS / V] += f[e];
     }
   }
+  // the workgroup's first rows are requested before the shift is known: the reductions below wait for nothing of theirs
+  Piece<T, V> cur[U];
+  fetch_rows<T, V, U>(cur, xs, row, step, end, begin, C, active);
   block_row_reduce<SLOTS>(kv, buf, tpr, rpp, active);
   fold_groups<SLOTS, 1>(buf, out, G, cg, V);
   const float kinv = 1.f / ((float)krows * (float)cg);
@@ -183,38 +192,47 @@ __global__ void __launch_bounds__(kBlock) gn_stats_partial(const T* __restrict__
   float acc[2 * SLOTS];
 #pragma unroll
   for (int s = 0; s < 2 * SLOTS; ++s) acc[s] = 0.f;
-  const int64_t begin = (int64_t)split * rows_per_split;
-  int64_t end = begin + rows_per_split;
-  if (end > S) end = S;
   if (active) {
-    int64_t row = begin + r;
-    const int64_t step = rpp;
-    for (; row + 3 * step < end; row += 4 * step) {  // four independent loads in flight
-      float f0[V], f1[V], f2[V], f3[V];
-      Ld<T, V>::run(xs + row * C, f0);
-      Ld<T, V>::run(xs + (row + step) * C, f1);
-      Ld<T, V>::run(xs + (row + 2 * step) * C, f2);
-      Ld<T, V>::run(xs + (row + 3 * step) * C, f3);
+    while (row < end) {
+      const int64_t next = row + U * step;
+      Piece<T, V> nxt[U];
+      if (next < end) fetch_rows<T, V, U>(nxt, xs, next, step, end, begin, C, true);
+      if (row + (U - 1) * step < end) {  // a whole batch
+        float f0[V], f1[V], f2[V], f3[V];
+        cur[0].unpack(f0);
+        cur[1].unpack(f1);
+        cur[2].unpack(f2);
+        cur[3].unpack(f3);
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const int s = e * SLOTS / V;
-        const float d0 = f0[e] - K[s], d1 = f1[e] - K[s], d2 = f2[e] - K[s], d3 = f3[e] - K[s];
-        acc[s] += (d0 + d1) + (d2 + d3);
-        float q = acc[SLOTS + s];
-        q = fmaf(d0, d0, q); q = fmaf(d1, d1, q); q = fmaf(d2, d2, q); q = fmaf(d3, d3, q);
-        acc[SLOTS + s] = q;
-      }
-    }
-    for (; row < end; row += step) {
-      float f0[V];
-      Ld<T, V>::run(xs + row * C, f0);
+        for (int e = 0; e < V; ++e) {
+          const int s = e * SLOTS / V;
+          const float d0 = f0[e] - K[s], d1 = f1[e] - K[s], d2 = f2[e] - K[s], d3 = f3[e] - K[s];
+          acc[s] += (d0 + d1) + (d2 + d3);
+          float q = acc[SLOTS + s];
+          q = fmaf(d0, d0, q); q = fmaf(d1, d1, q); q = fmaf(d2, d2, q); q = fmaf(d3, d3, q);
+          acc[SLOTS + s] = q;
+        }
+      } else {
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const int s = e * SLOTS / V;
-        const float d0 = f0[e] - K[s];
-        acc[s] += d0;
-        acc[SLOTS + s] = fmaf(d0, d0, acc[SLOTS + s]);
+        for (int u = 0; u < U; ++u) {
+          if (row + u * step < end) {
+            float f0[V];
+            cur[u].unpack(f0);
+#pragma unroll
+            for (int e = 0; e < V; ++e) {
+              const int s = e * SLOTS / V;
+              const float d0 = f0[e] - K[s];
+              acc[s] += d0;
+              acc[SLOTS + s] = fmaf(d0, d0, acc[SLOTS + s]);
+            }
+          }
+        }
       }
+      if (next < end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) cur[u] = nxt[u];
+      }
+      row = next;
     }
   }
   block_row_reduce<2 * SLOTS>(acc, buf, tpr, rpp, active);
@@ -406,6 +424,16 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   const int r = tid / tpr, cv = tid - r * tpr;
   float* g_mean = gstat + 2 * G;
   float* g_rstd = gstat + 3 * G;
+  // the workgroup's first rows are requested before anything else: the fold of the statistics below reads other memory
+  constexpr int U = 4;  // rows per batch: the next batch's loads are in flight while the current one is normalised
+  const T* xs = x + (int64_t)n * S * C + cv * V;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  Piece<T, V> cur[U];
+  fetch_rows<T, V, U>(cur, xs, row, step, end, begin, C, r < rpp);
   // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid, sums about the
   // common shift), or (`welford`) the records the producer of x left
   if (welford && fold_in_consumer(G, npart, kGnRecordFloats)) {
@@ -464,39 +492,30 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
     ga[e] = load_param(gamma, param_dtype, c, 1.f);
     be[e] = load_param(beta, param_dtype, c, 0.f);
   }
-  const T* xs = x + (int64_t)n * S * C + cv * V;
   TO* ys = y + y_sample + y_halo * C + cv * V;
-  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
-  int64_t end = begin + rows_per_split;
-  if (end > S) end = S;
-  const int64_t step = rpp;
-  int64_t row = begin + r;
-  for (; row + 3 * step < end; row += 4 * step) {
-    float f[4][V];
+  while (row < end) {
+    const int64_t next = row + U * step;
+    Piece<T, V> nxt[U];
+    if (next < end) fetch_rows<T, V, U>(nxt, xs, next, step, end, begin, C, true);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) Ld<T, V>::run(xs + (row + u * step) * C, f[u]);
+    for (int u = 0; u < U; ++u) {
+      if (row + u * step < end) {
+        float f[V], o[V];
+        cur[u].unpack(f);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float o[V];
-#pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const float xh = (f[u][e] - mu[e]) * rs[e];
-        const float v = fmaf(xh, ga[e], be[e]);
-        o[e] = relu ? relu_keep_nan(v) : v;
+        for (int e = 0; e < V; ++e) {
+          const float xh = (f[e] - mu[e]) * rs[e];
+          const float v = fmaf(xh, ga[e], be[e]);
+          o[e] = relu ? relu_keep_nan(v) : v;
+        }
+        St<TO, V>::run(ys + (row + u * step) * C, o);
       }
-      St<TO, V>::run(ys + (row + u * step) * C, o);
     }
-  }
-  for (; row < end; row += step) {
-    float f[V], o[V];
-    Ld<T, V>::run(xs + row * C, f);
+    if (next < end) {
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const float xh = (f[e] - mu[e]) * rs[e];
-      const float v = fmaf(xh, ga[e], be[e]);
-      o[e] = relu ? relu_keep_nan(v) : v;
+      for (int u = 0; u < U; ++u) cur[u] = nxt[u];
     }
-    St<TO, V>::run(ys + row * C, o);
+    row = next;
   }
 }
 
@@ -516,6 +535,20 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
   const int cg = C / G;
   const int r = tid / tpr, cv = tid - r * tpr;
   const bool active = r < rpp;
+  // the workgroup's first rows are requested before the statistics and parameters they will be combined with
+  constexpr int U = 2;  // rows per batch: the next batch's loads are in flight while the current one is summed
+  const int64_t base = (int64_t)n * S * C + cv * V;
+  const T* xs = x + base;
+  const TG* gs = dy + base;
+  const int64_t begin = (int64_t)split * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  Piece<T, V> cx[U];
+  Piece<TG, V> cg_[U];
+  fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, active);
+  fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, active);
   float mu[V], rs[V], ga[V], be[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
@@ -529,45 +562,53 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
 #pragma unroll
   for (int e = 0; e < 2 * V; ++e) acc[e] = 0.f;
   if (active) {
-    const int64_t base = (int64_t)n * S * C + cv * V;
-    const T* xs = x + base;
-    const TG* gs = dy + base;
-    const int64_t begin = (int64_t)split * rows_per_split;
-    int64_t end = begin + rows_per_split;
-    if (end > S) end = S;
-    const int64_t step = rpp;
-    int64_t row = begin + r;
-    for (; row + step < end; row += 2 * step) {
-      float f0[V], g0[V], f1[V], g1[V];
-      Ld<T, V>::run(xs + row * C, f0);
-      Ld<TG, V>::run(gs + row * C, g0);
-      Ld<T, V>::run(xs + (row + step) * C, f1);
-      Ld<TG, V>::run(gs + (row + step) * C, g1);
+    while (row < end) {
+      const int64_t next = row + U * step;
+      Piece<T, V> nx[U];
+      Piece<TG, V> ng[U];
+      if (next < end) {
+        fetch_rows<T, V, U>(nx, xs, next, step, end, begin, C, true);
+        fetch_rows<TG, V, U>(ng, gs, next, step, end, begin, C, true);
+      }
+      if (row + step < end) {  // a whole batch
+        float f0[V], g0[V], f1[V], g1[V];
+        cx[0].unpack(f0);
+        cg_[0].unpack(g0);
+        cx[1].unpack(f1);
+        cg_[1].unpack(g1);
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const float xh0 = (f0[e] - mu[e]) * rs[e], xh1 = (f1[e] - mu[e]) * rs[e];
-        float d0 = g0[e], d1 = g1[e];
-        if (relu) {
-          d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
-          d1 = fmaf(xh1, ga[e], be[e]) <= 0.f ? 0.f : d1;
+        for (int e = 0; e < V; ++e) {
+          const float xh0 = (f0[e] - mu[e]) * rs[e], xh1 = (f1[e] - mu[e]) * rs[e];
+          float d0 = g0[e], d1 = g1[e];
+          if (relu) {
+            d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
+            d1 = fmaf(xh1, ga[e], be[e]) <= 0.f ? 0.f : d1;
+          }
+          acc[e] = fmaf(d0, xh0, acc[e]);
+          acc[e] = fmaf(d1, xh1, acc[e]);
+          acc[V + e] += d0 + d1;
         }
-        acc[e] = fmaf(d0, xh0, acc[e]);
-        acc[e] = fmaf(d1, xh1, acc[e]);
-        acc[V + e] += d0 + d1;
-      }
-    }
-    for (; row < end; row += step) {
-      float f0[V], g0[V];
-      Ld<T, V>::run(xs + row * C, f0);
-      Ld<TG, V>::run(gs + row * C, g0);
+      } else {
+        float f0[V], g0[V];
+        cx[0].unpack(f0);
+        cg_[0].unpack(g0);
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const float xh0 = (f0[e] - mu[e]) * rs[e];
-        float d0 = g0[e];
-        if (relu) d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
-        acc[e] = fmaf(d0, xh0, acc[e]);
-        acc[V + e] += d0;
+        for (int e = 0; e < V; ++e) {
+          const float xh0 = (f0[e] - mu[e]) * rs[e];
+          float d0 = g0[e];
+          if (relu) d0 = fmaf(xh0, ga[e], be[e]) <= 0.f ? 0.f : d0;
+          acc[e] = fmaf(d0, xh0, acc[e]);
+          acc[V + e] += d0;
+        }
       }
+      if (next < end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          cx[u] = nx[u];
+          cg_[u] = ng[u];
+        }
+      }
+      row = next;
     }
   }
   block_row_reduce<2 * V>(acc, smem, tpr, rpp, active);
@@ -679,6 +720,20 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   const int n = blockIdx.y;
   const int cg = C / G;
   const int r = tid / tpr, cv = tid - r * tpr;
+  // the workgroup's first rows are requested before anything else: the fold of the partials below reads other memory
+  constexpr int U = 2;  // rows per batch: the next batch's loads are in flight while the current one is worked on
+  const int64_t base = (int64_t)n * S * C + cv * V;
+  const T* xs = x + base;
+  const TG* gs = dy + base;
+  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
+  int64_t end = begin + rows_per_split;
+  if (end > S) end = S;
+  const int64_t step = rpp;
+  int64_t row = begin + r;
+  Piece<T, V> cx[U];
+  Piece<TG, V> cg_[U];
+  fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, r < rpp);
+  fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, r < rpp);
   const bool fused = fold_in_consumer(G, nsplit);
   if (fused) {
     // gpart quantity 0 = sum dy'*gamma*xhat (-> B), quantity 1 = sum dy'*gamma (-> A)
@@ -703,47 +758,39 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
     ca[e] = gco[G + g];
     cb[e] = gco[g];
   }
-  const int64_t base = (int64_t)n * S * C + cv * V;
-  const T* xs = x + base;
-  const TG* gs = dy + base;
   T* ds = dx + base;
-  const int64_t begin = (int64_t)blockIdx.x * rows_per_split;
-  int64_t end = begin + rows_per_split;
-  if (end > S) end = S;
-  const int64_t step = rpp;
-  int64_t row = begin + r;
-  for (; row + step < end; row += 2 * step) {
-    float f[2][V], g[2][V];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      Ld<T, V>::run(xs + (row + u * step) * C, f[u]);
-      Ld<TG, V>::run(gs + (row + u * step) * C, g[u]);
+  while (row < end) {
+    const int64_t next = row + U * step;
+    Piece<T, V> nx[U];
+    Piece<TG, V> ng[U];
+    if (next < end) {
+      fetch_rows<T, V, U>(nx, xs, next, step, end, begin, C, true);
+      fetch_rows<TG, V, U>(ng, gs, next, step, end, begin, C, true);
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      float o[V];
+    for (int u = 0; u < U; ++u) {
+      if (row + u * step < end) {
+        float f[V], g[V], o[V];
+        cx[u].unpack(f);
+        cg_[u].unpack(g);
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const float xh = (f[u][e] - mu[e]) * rs[e];
-        float d = g[u][e];
-        if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
-        o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
+        for (int e = 0; e < V; ++e) {
+          const float xh = (f[e] - mu[e]) * rs[e];
+          float d = g[e];
+          if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
+          o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
+        }
+        St<T, V>::run(ds + (row + u * step) * C, o);
       }
-      St<T, V>::run(ds + (row + u * step) * C, o);
     }
-  }
-  for (; row < end; row += step) {
-    float f[V], g[V], o[V];
-    Ld<T, V>::run(xs + row * C, f);
-    Ld<TG, V>::run(gs + row * C, g);
+    if (next < end) {
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const float xh = (f[e] - mu[e]) * rs[e];
-      float d = g[e];
-      if (relu) d = fmaf(xh, ga[e], be[e]) <= 0.f ? 0.f : d;
-      o[e] = rs[e] * ((d * ga[e] - ca[e]) - xh * cb[e]);
+      for (int u = 0; u < U; ++u) {
+        cx[u] = nx[u];
+        cg_[u] = ng[u];
+      }
     }
-    St<T, V>::run(ds + row * C, o);
+    row = next;
   }
   }
   if (fused && n == 0 && (dgamma != nullptr || dbeta != nullptr)) {
