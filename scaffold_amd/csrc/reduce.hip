@@ -139,6 +139,15 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __
   o[3] = elem<T>::from_float(s.w);
 }
 
+// Four consecutive 16-bit elements (8-byte aligned) as one store.
+template <typename T>
+__device__ __forceinline__ void store4(T* p, T a, T b, T c, T d) {
+  static_assert(sizeof(T) == 2, "16-bit elements");
+  const uint32_t lo = (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+  const uint32_t hi = (uint32_t)__builtin_bit_cast(uint16_t, c) | ((uint32_t)__builtin_bit_cast(uint16_t, d) << 16);
+  *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+}
+
 // sum_slices_bias that also leaves GroupNorm records of the rounded result (16-bit outputs, layout and merge rule in
 // gn_stats.hpp): a workgroup owns `chunks` consecutive pieces of 1024 elements of one sample; 1024 is a multiple of the
 // channel count, so a thread's four consecutive channels are the same in every piece and belong to one group. A thread
@@ -148,7 +157,8 @@ constexpr int kStatsPiece = 4 * kBlock;
 template <typename T>
 __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const float* __restrict__ part, const T* __restrict__ bias,
                                                                        T* __restrict__ out, int64_t sample_elems, int64_t nelem,
-                                                                       int channels, int splits, int chunks, GnPartialOut gn) {
+                                                                       int channels, int splits, int chunks, GnPartialOut gn,
+                                                                       int whole_store) {
   __shared__ float4 sums[kBlock];  // { values, sum, sum of squares, shift } of every thread
   const int tid = threadIdx.x, n = blockIdx.y;
   const int c = (tid * 4) % channels;
@@ -159,33 +169,73 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_stats_kernel(const flo
     const int64_t local = ((int64_t)blockIdx.x * chunks + k) * kStatsPiece + tid * 4;
     if (local >= sample_elems) break;
     const int64_t e = (int64_t)n * sample_elems + local;
+    // the first eight slices' loads are in flight together (the reduction channels are cut into at most eight); the
+    // sum keeps the slice order
+    constexpr int kInFlight = 8;
+    float4 v[kInFlight];
+#pragma unroll
+    for (int sp = 0; sp < kInFlight; ++sp)
+      v[sp] = sp < splits ? *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e) : make_float4(0.f, 0.f, 0.f, 0.f);
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int sp = 0; sp < splits; ++sp) {
-      const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
-      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+#pragma unroll
+    for (int sp = 0; sp < kInFlight; ++sp) {
+      if (sp < splits) { s.x += v[sp].x; s.y += v[sp].y; s.z += v[sp].z; s.w += v[sp].w; }
+    }
+    for (int sp = kInFlight; sp < splits; ++sp) {
+      const float4 w = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
+      s.x += w.x; s.y += w.y; s.z += w.z; s.w += w.w;
     }
     const T o0 = elem<T>::from_float(s.x + b0), o1 = elem<T>::from_float(s.y + b1), o2 = elem<T>::from_float(s.z + b2),
             o3 = elem<T>::from_float(s.w + b3);
-    out[e] = o0; out[e + 1] = o1; out[e + 2] = o2; out[e + 3] = o3;
+    if (whole_store) store4(out + e, o0, o1, o2, o3);
+    else { out[e] = o0; out[e + 1] = o1; out[e + 2] = o2; out[e + 3] = o3; }
     if (k == 0) shift = to_float(o0);
     const float r0 = to_float(o0) - shift, r1 = to_float(o1) - shift, r2 = to_float(o2) - shift, r3 = to_float(o3) - shift;
     s1 += (r0 + r1) + (r2 + r3);
     s2 += fmaf(r0, r0, r1 * r1) + fmaf(r2, r2, r3 * r3);
     cnt += 4.f;
   }
-  sums[tid] = make_float4(cnt, s1, s2, shift);
+  // Every thread turns its sums into (count, mean, M2); then the 256 / groups threads' pieces of each group (kStatsPiece is
+  // a multiple of the channel count and a group a multiple of four channels, so that many there are) are merged about the
+  // mean of the group's first piece -- count, sum of n d and sum of M2 + n d^2 are plain sums, taken by a fixed tree over
+  // LDS. (One thread per group walking its 32 pieces in turn, a division each, took 4 of this kernel's 9 us.)
+  float pm = 0.f, pm2 = 0.f;
+  if (cnt > 0.f) {
+    const float dm = s1 / cnt;
+    pm = shift + dm;
+    pm2 = fmaf(-s1, dm, s2);
+    pm2 = pm2 < 0.f ? 0.f : pm2;
+  }
+  sums[tid] = make_float4(cnt, pm, pm2, 0.f);
   __syncthreads();
-  const int rows = kStatsPiece / channels, per_row = channels / 4, per_group = gn.cg / 4;
-  for (int g = tid; g < gn.groups; g += kBlock) {
-    WelfordMerge m;
-    m.clear();
-    for (int v = 0; v < rows; ++v)
-      for (int r = 0; r < per_group; ++r) {
-        const float4 e = sums[v * per_row + g * per_group + r];
-        m.add_sums(e.x, e.y, e.z, e.w);
-      }
+  const int per_row = channels / 4, per_group = gn.cg / 4;
+  const int epg = kBlock / gn.groups;  // pieces per group
+  const int g = tid / epg, l = tid - g * epg;
+  const int v = l / per_group, r = l - v * per_group;
+  const float4 e = sums[v * per_row + g * per_group + r];
+  // the group's first piece belongs to the lowest thread of the group: when it is empty (past the end of the sample) all are
+  const float about = sums[g * per_group].y;
+  const float d = e.y - about;
+  __syncthreads();
+  sums[tid] = make_float4(e.x, e.x * d, fmaf(e.x * d, d, e.z), 0.f);
+  __syncthreads();
+  for (int stride = epg >> 1; stride > 0; stride >>= 1) {
+    if (l < stride) {
+      const float4 a = sums[tid], b = sums[tid + stride];
+      sums[tid] = make_float4(a.x + b.x, a.y + b.y, a.z + b.z, 0.f);
+    }
+    __syncthreads();
+  }
+  if (l == 0) {
+    const float4 t = sums[tid];
+    float mean = 0.f, m2 = 0.f;
+    if (t.x > 0.f) {
+      mean = about + t.y / t.x;
+      m2 = fmaf(-t.y, t.y / t.x, t.z);
+      m2 = m2 < 0.f ? 0.f : m2;
+    }
     *reinterpret_cast<float4*>(gn.part + (((int64_t)n * gn.records + blockIdx.x) * gn.groups + g) * kGnRecordFloats) =
-        make_float4(m.n, m.mean(), m.m2(), 0.f);
+        make_float4(t.x, mean, m2, 0.f);
   }
 }
 
@@ -345,12 +395,13 @@ int sum_slices_bias_stats(int dtype, const float* part, const void* bias, void* 
     return fail(SFH_ERR_UNSUPPORTED, "sum of slices with GroupNorm partials: not offered for this shape");
   const int chunks = (int)cdiv(cdiv(sample_elems, kStatsPiece), records);
   const dim3 grid((unsigned)records, (unsigned)n);
+  const int whole_store = (reinterpret_cast<uintptr_t>(out) & 7u) == 0 ? 1 : 0;  // a thread's four outputs as one 8-byte store
   if (dtype == SFH_BF16)
     hipLaunchKernelGGL(sum_slices_bias_stats_kernel<bf16_t>, grid, dim3(kBlock), 0, st, part, (const bf16_t*)bias, (bf16_t*)out,
-                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn);
+                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn, whole_store);
   else
     hipLaunchKernelGGL(sum_slices_bias_stats_kernel<fp16_t>, grid, dim3(kBlock), 0, st, part, (const fp16_t*)bias, (fp16_t*)out,
-                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn);
+                       sample_elems, (int64_t)n * sample_elems, channels, splits, chunks, gn, whole_store);
   return check_launch("sum_slices_bias_stats_kernel");
 }
 
