@@ -769,7 +769,8 @@ def test_outputs_are_allocated_once_in_their_final_layout(device):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("n,cin,cout,spatial", [(1, 64, 32, (8, 16, 32)), (2, 128, 64, (3, 5, 7)), (1, 256, 128, (4, 8, 8)), (1, 64, 96, (5, 4, 6))])
+@pytest.mark.parametrize("n,cin,cout,spatial", [(1, 64, 32, (8, 16, 32)), (2, 128, 64, (3, 5, 7)), (1, 256, 128, (4, 8, 8)), (1, 64, 96, (5, 4, 6)),
+                                                 (1, 64, 32, (32, 64, 64))])  # the last: the U-Net's level 0, thousands of bias slices
 def test_transposed_weight_and_bias_gradient_in_one_pass(device, dtype, n, cin, cout, spatial):
     """``conv_transpose3d_backward_weight_bias``: the weight gradient is the bits of ``conv_transpose3d_backward_weight``; the
     bias gradient is ``grad_output.sum((0, 2, 3, 4))`` -- exactly on integer-valued gradients (fp32 sums of small integers in
