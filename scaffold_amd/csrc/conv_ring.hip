@@ -6,8 +6,8 @@
 // voxels reads the four input planes d-1 .. d+2 (10 x 34 voxels each with the halo); the next step needs d+1 .. d+4,
 // of which two are already in LDS. LDS therefore holds a ring of three plane PAIRS: two are read by the MFMAs of the
 // current step while the third receives the next step's two new planes straight from memory (buffer_load ... lds).
-// Per step a workgroup fetches 680 voxels for 512 outputs (1.33x) in 11 load instructions per wavefront, where a brick
-// with its own halo in all three directions needs 1224 voxels (2.39x) and 20: global-memory instructions are what this
+// Per step a workgroup fetches 680 voxels for 512 outputs (1.33x) in 44 load instructions (12, 12, 12 and 8 over its four
+// wavefronts), where a brick with its own halo in all three directions needs 1224 voxels (2.39x) and 80: global-memory instructions are what this
 // kernel's matrix pipe waits for most.
 //
 // Each wavefront owns a 2 x 2 block of the step's rows (two planes x two rows of 32 voxels). An activation fragment --
