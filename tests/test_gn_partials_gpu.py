@@ -38,6 +38,8 @@ CASES = [
     (1, 64, 128, (16, 32, 33), (1, 1, 1), 2, "brick"),         # a group wider than the workgroup's span, ragged rows
     (2, 64, 64, (9, 10, 16), (1, 1, 1), 16, "brick"),          # small volume: the reduction is sliced, the slice sum counts
     (1, 256, 512, (4, 8, 8), (1, 1, 1), 8, "brick"),           # deep level, sliced
+    (1, 128, 256, (4, 8, 8), (1, 1, 1), 1, "brick"),           # sliced, one group of all channels (256 pieces merged per record)
+    (1, 256, 256, (4, 8, 8), (1, 1, 1), 64, "brick"),          # sliced, 4 channels per group (a piece per row of the workgroup's 1024 elements)
     (1, 128, 64, (32, 64, 64), (0, 1, 1), 8, "wide"),          # 4 x 4 x 32 tiles
     (1, 128, 64, (63, 61, 65), (1, 1, 1), 16, "wide"),         # 8 x 4 x 32 tiles, ragged on every axis
     (1, 192, 64, (30, 62, 34), (1, 1, 1), 1, "wide"),          # one group of all 64 channels
@@ -161,7 +163,7 @@ def test_group_norm_from_partials_matches_the_statistics_pass(device, n, cin, co
     assert orc.gn_rel_error(fused, ref) < 2e-2
 
 
-@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", [CASES[2], CASES[7], CASES[10], CASES[12], CASES[13]])
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", [CASES[2], CASES[7], CASES[10], CASES[14], CASES[15]])
 def test_large_mean_small_std_on_the_first_call(device, n, cin, cout, spatial, padding, groups, kernel):
     """A mean a thousand times the spread (fp16 resolves it; bf16 does not), the case of the reference's
     ``test_large_mean_small_std`` (tests/test_triton_group_norm.py:502-547): plain fp32 sums of y and y^2 lose the variance
