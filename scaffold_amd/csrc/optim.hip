@@ -12,7 +12,7 @@ namespace sfh {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kMaxTensors = 48;
+constexpr int kMaxTensors = 64;  // per launch: the table travels in the kernel arguments (4 KiB at most); 64 hold a whole 5-level U-Net
 
 struct SumsqTable {
   const float* g[kMaxTensors];
@@ -31,6 +31,8 @@ struct AdamTable {
   int chunk_start[kMaxTensors + 1];
   int n;
 };
+
+static_assert(sizeof(AdamTable) + 128 <= 4096, "the table and the other arguments fit the kernel argument segment");
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -135,23 +137,40 @@ __global__ void __launch_bounds__(kBlock) clip_adam_kernel(AdamTable t, AdamCoef
   int64_t done = 0;
   if (aligned) {
     const int64_t nvec = len / 4;
-    for (int64_t i = threadIdx.x; i < nvec; i += kBlock) {
-      float4 pq = reinterpret_cast<float4*>(p)[i];
-      const float4 gq = reinterpret_cast<const float4*>(g)[i];
-      float4 mq = reinterpret_cast<float4*>(m)[i];
-      float4 vq = reinterpret_cast<float4*>(v)[i];
-      update(pq.x, gq.x, mq.x, vq.x);
-      update(pq.y, gq.y, mq.y, vq.y);
-      update(pq.z, gq.z, mq.z, vq.z);
-      update(pq.w, gq.w, mq.w, vq.w);
-      reinterpret_cast<float4*>(p)[i] = pq;
-      reinterpret_cast<float4*>(m)[i] = mq;
-      reinterpret_cast<float4*>(v)[i] = vq;
-      if (SHADOW != 0 && sh != nullptr) {
-        uint2 pk;
-        if (SHADOW == 1) { pk.x = pack_bf16x2(pq.x, pq.y); pk.y = pack_bf16x2(pq.z, pq.w); }
-        else { pk.x = pack_fp16x2(pq.x, pq.y); pk.y = pack_fp16x2(pq.z, pq.w); }
-        reinterpret_cast<uint2*>(static_cast<char*>(sh) + 2 * begin)[i] = pk;
+    // Four of a thread's pieces at a time, all sixteen loads in flight before the first update: a launch of a few dozen
+    // chunks (the tail of the parameter list) has nothing else on its CUs to cover a trip to memory, and one piece
+    // per trip made its chunk of 8192 elements a chain of eight (15.8 us for half a megabyte of parameters).
+    constexpr int U = 4;
+    for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += U * kBlock) {
+      float4 pq[U], gq[U], mq[U], vq[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = i0 + u * kBlock;
+        if (i < nvec) {
+          pq[u] = reinterpret_cast<float4*>(p)[i];
+          gq[u] = reinterpret_cast<const float4*>(g)[i];
+          mq[u] = reinterpret_cast<float4*>(m)[i];
+          vq[u] = reinterpret_cast<float4*>(v)[i];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t i = i0 + u * kBlock;
+        if (i < nvec) {
+          update(pq[u].x, gq[u].x, mq[u].x, vq[u].x);
+          update(pq[u].y, gq[u].y, mq[u].y, vq[u].y);
+          update(pq[u].z, gq[u].z, mq[u].z, vq[u].z);
+          update(pq[u].w, gq[u].w, mq[u].w, vq[u].w);
+          reinterpret_cast<float4*>(p)[i] = pq[u];
+          reinterpret_cast<float4*>(m)[i] = mq[u];
+          reinterpret_cast<float4*>(v)[i] = vq[u];
+          if (SHADOW != 0 && sh != nullptr) {
+            uint2 pk;
+            if (SHADOW == 1) { pk.x = pack_bf16x2(pq[u].x, pq[u].y); pk.y = pack_bf16x2(pq[u].z, pq[u].w); }
+            else { pk.x = pack_fp16x2(pq[u].x, pq[u].y); pk.y = pack_fp16x2(pq[u].z, pq[u].w); }
+            reinterpret_cast<uint2*>(static_cast<char*>(sh) + 2 * begin)[i] = pk;
+          }
+        }
       }
     }
     done = nvec * 4;

@@ -4,7 +4,7 @@ Stands where the reference's trainer calls ``torch.nn.utils.clip_grad_norm_(mode
 and then ``optimizer.step()`` on ``torch.optim.Adam(..., fused=True)`` (``ScaFFold/utils/trainer.py:678-694``,
 ``:268-274``).  Same arithmetic (torch's Adam formulas, bias corrections from a step counter that lives on the
 device, the clipping factor ``min(1, max_norm / (norm + 1e-6))``), but the gradients are scaled on the fly instead
-of being rewritten, the norm is a fixed-order sum (bitwise reproducible), and the whole step is two launches per 48
+of being rewritten, the norm is a fixed-order sum (bitwise reproducible), and the whole step is two launches per 64
 tensors with nothing that synchronises, so it can be captured in a graph.
 
 ``state_dict()`` has the layout of ``torch.optim.Adam`` (``step``, ``exp_avg``, ``exp_avg_sq`` per parameter), so
