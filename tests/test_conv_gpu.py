@@ -123,6 +123,28 @@ def test_brick_geometries_exact(device, n, cin, cout, spatial, direction, voxels
     check_exact(prob, direction, device)
 
 
+# The column-walking kernels (32 reduction channels / any weight gradient at rows of more than 16 voxels) on volumes that
+# make a workgroup take several columns one after the other (more columns than workgroups), long columns in several
+# segments, and columns cut by every edge.
+RING_WALKS = [
+    # (n, cin, cout, spatial, padding)
+    (2, 32, 32, (5, 130, 259), (1, 1, 1)),     # 2 x 17 x 9 = 306 columns of 8 rows for 256 workgroups
+    (1, 32, 64, (3, 200, 170), (0, 1, 1)),     # two output blocks of 128 workgroups each, 150 columns, shard form
+    (1, 32, 32, (45, 9, 33), (1, 1, 1)),       # 4 columns of 23 steps: cut into segments, ragged in every direction
+    (3, 32, 96, (7, 17, 40), (2, 2, 2)),       # three blocks, padding 2
+]
+
+
+@pytest.mark.parametrize("direction", DIRS)
+@pytest.mark.parametrize("n,cin,cout,spatial,padding", RING_WALKS)
+def test_column_walks_exact(device, n, cin, cout, spatial, padding, direction):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=torch.bfloat16)
+    check_exact(prob, direction, device)
+    # the data gradient of the mirrored problem runs the same kernel with the roles of the channel counts swapped
+    if direction == "bwd-data" and cout != cin:
+        check_exact(orc.ConvProblem(n=n, cin=cout, cout=cin, spatial=spatial, padding=padding, dtype=torch.bfloat16), direction, device)
+
+
 def _random_tiled_problems(count, seed):
     """Seeded random 3x3x3 stride-1 problems with channel counts in multiples of 32: extents around the tile sizes, the
     three padding forms, one to three samples -- whatever geometry the launch rules pick for them."""
