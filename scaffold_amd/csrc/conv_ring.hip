@@ -41,7 +41,10 @@ constexpr int kGroupsPerWave = (kGroups + 3) / 4;      // 3
 constexpr int kLoads = kGroupsPerWave * 4;             // load instructions per wavefront and step
 constexpr int kStores = 8;                             // store instructions per wavefront and step (4 sub-tiles x 2)
 constexpr int kRange = 0x40000000;                     // buffer range: offsets at or above it read as zero / are not stored
-static_assert(3 * kPair <= 160 * 1024, "three plane pairs in the LDS of a CU");
+constexpr int kWeightFrags = 54;                       // (tap, k-step) fragments of a 32-channel output block, 1 KiB each
+constexpr int kWeightInPair = kPair / 1024;            // ... of which the third pair's array holds this many while the kernel starts
+constexpr int kWeightSpare = (kWeightFrags - kWeightInPair) * 1024;  // and a small array of its own the rest
+static_assert(3 * kPair + kWeightSpare <= 160 * 1024, "three plane pairs and the rest of the weights in the LDS of a CU");
 static_assert(kGroups * 1024 - kPiece < 64 * 16 && kPiece >= kPairVoxels * 16, "only the last group runs past a piece, by masked lanes");
 
 // ---- the compile-time schedule of a step ---------------------------------------------------------------------------------------
@@ -349,6 +352,7 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   __shared__ __attribute__((aligned(16))) char pair0[kPair];
   __shared__ __attribute__((aligned(16))) char pair1[kPair];
   __shared__ __attribute__((aligned(16))) char pair2[kPair];
+  __shared__ __attribute__((aligned(16))) char wrest[kWeightSpare];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -388,15 +392,24 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   }
 
   constexpr int FRAG = 512;
-  const T* wblock = wp + (int64_t)nb * 54 * FRAG + lane * 8;
-  // k-step 0 of every tap in vector registers, k-step 1 in accumulation registers (the MFMA reads its row operand from
-  // either file; there are not 216 vector registers to spare beside the activation fragments)
   uint4 wq[27];
   ring_i32x4_t wa[27];
+  // The block's 54 fragments come into LDS once per workgroup (direct-to-LDS loads, a quarter per wavefront: the packed
+  // weight is in fragment order, a fragment is 1 KiB as it lies) and every wavefront takes its copy from there: four
+  // copies straight from memory cost the CU's address path 216 KiB beside the first plane pairs' 86. They land in the
+  // third pair's array, which nothing reads before the first step fills it, and in `wrest`.
+  {
+    const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(wp + (int64_t)nb * kWeightFrags * FRAG), 0,
+                                                                            kWeightFrags * 1024, 0x00020000);
 #pragma unroll
-  for (int tap = 0; tap < 27; ++tap) wq[tap] = *reinterpret_cast<const uint4*>(wblock + (2 * tap) * FRAG);
-#pragma unroll
-  for (int tap = 0; tap < 27; ++tap) wa[tap] = *reinterpret_cast<const ring_i32x4_t*>(wblock + (2 * tap + 1) * FRAG);
+    for (int k = 0; k < (kWeightFrags + 3) / 4; ++k) {
+      const int f = wave + 4 * k;  // wave-uniform
+      if (f < kWeightFrags) {
+        char* dst = f < kWeightInPair ? pair2 + f * 1024 : wrest + (f - kWeightInPair) * 1024;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, (__attribute__((address_space(3))) void*)dst, 16, f * 1024 + lane * 16, 0, 0, 0);
+      }
+    }
+  }
   float bias[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) bias[r] = BIAS ? to_float(bias_ptr[nb * 32 + 8 * (r / 4) + 4 * kg + (r % 4)]) : 0.f;
@@ -409,7 +422,7 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
   int done_off[4];
   int voff[kGroupsPerWave];
 
-  for (int item = item_begin; item < item_end; ++item) {
+  auto run_item = [&](int item, auto with_weights) {
     // item = segment * columns + column: the workgroups of an XCD work on neighbouring columns over the same depth range
     const int ncols = gm.items / gm.segs;
     const int seg = item / ncols;
@@ -418,8 +431,7 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     int s_end = s_begin + gm.seg_steps;
     if (s_end > gm.steps) s_end = gm.steps;
     const int nsteps = s_end - s_begin;
-    if (nsteps <= 0) continue;
-    const int plane0 = 2 * s_begin - a.pd;  // first input plane of the segment's first step
+    const int plane0 = 2 * s_begin - a.pd;  // first input plane of the segment's first step (every segment has at least one)
 
     // the first step's four planes
     ring_pair_offsets(a, col, ln, plane0, true, voff);
@@ -435,6 +447,19 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     T* done_origin = yout;
     __builtin_amdgcn_s_waitcnt(ring_waitcnt_vm(0));
     __syncthreads();
+    if constexpr (decltype(with_weights)::value) {
+      // the weights have landed with the first pairs: k-step 0 of every tap into vector registers, k-step 1 into
+      // accumulation registers (the MFMA reads its row operand from either file; there are not 216 vector registers to
+      // spare beside the activation fragments)
+#pragma unroll
+      for (int tap = 0; tap < 27; ++tap) {
+        const int f0 = 2 * tap, f1 = 2 * tap + 1;
+        wq[tap] = *reinterpret_cast<const uint4*>((f0 < kWeightInPair ? pair2 + f0 * 1024 : wrest + (f0 - kWeightInPair) * 1024) + lane * 16);
+        wa[tap] = *reinterpret_cast<const ring_i32x4_t*>((f1 < kWeightInPair ? pair2 + f1 * 1024 : wrest + (f1 - kWeightInPair) * 1024) + lane * 16);
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the copies are in registers ...
+      __syncthreads();                     // ... in every wavefront, before the first step's loads may overwrite them
+    }
 
     auto step = [&](int i, const char* lo, const char* hi, char* fill) {
       // the pair after this step's: planes plane0 + 2 i + 4, + 5
@@ -460,7 +485,11 @@ conv_ring_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
     for (int ms = 0; ms < 4; ++ms)
 #pragma unroll
       for (int h = 0; h < 2; ++h) __builtin_amdgcn_raw_buffer_store_b128(ps.data[ms][h], done_rsrc, done_off[ms] + 32 * h, 0, 0);
-  }
+  };
+  // the workgroup's first item also takes the weights out of LDS (a copy of the item's code of its own: the register
+  // arrays they go to are then defined on every path into the steps)
+  run_item(item_begin, std::true_type{});
+  for (int item = item_begin + 1; item < item_end; ++item) run_item(item, std::false_type{});
   if constexpr (GN) {
     // one record per workgroup (one sample): the last barrier has freed the LDS
     const int per_wg = gn.cg > 32 ? gn.cg / 32 : 1;  // output blocks that share a group
