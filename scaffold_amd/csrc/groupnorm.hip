@@ -40,7 +40,7 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kShiftRows = 32;   // voxels that define the shift K
 constexpr int kMaxSplit = 2048;  // workgroups per sample
-constexpr int kFillWorkgroups = 512;   // workgroups a launch aims for when the sample is small
+constexpr int kFillWorkgroups = 256;   // workgroups a launch aims for when the sample is small: one per compute unit
 
 struct GnPlan {
   bool vector;
@@ -65,10 +65,15 @@ GnPlan make_plan(const sfh_groupnorm_desc& p, int x_dtype, bool aligned) {
   pl.tpr = p.c / pl.vec;
   pl.rpp = kBlock / pl.tpr;
   pl.slots = cg >= pl.vec ? 1 : pl.vec / cg;
-  // 16 passes of 4 KiB per workgroup on large samples; fewer on small ones, so that a launch still has about
-  // kFillWorkgroups workgroups and no workgroup walks a long serial chain of dependent loads.
-  const int64_t want = cdiv((int64_t)kFillWorkgroups, std::max(1, p.n));
+  // 16 passes of 4 KiB per workgroup on large samples. On small ones a launch aims at one workgroup per compute unit
+  // (every workgroup pays for folding the sample's partial records, and all of them run at once), at two when that
+  // would take more than 8 passes: a 16 MiB sample is quickest as 512 x 8 passes, a 4 MiB one as 256 x 4.
+  int64_t want = cdiv((int64_t)kFillWorkgroups, std::max(1, p.n));
   int64_t passes = p.spatial / ((int64_t)pl.rpp * want);
+  if (passes > 8) {
+    want = cdiv((int64_t)2 * kFillWorkgroups, std::max(1, p.n));
+    passes = p.spatial / ((int64_t)pl.rpp * want);
+  }
   passes = std::min<int64_t>(16, std::max<int64_t>(1, passes));
   int64_t rows = (int64_t)pl.rpp * passes;
   if (cdiv(p.spatial, rows) > kMaxSplit) rows = cdiv(cdiv(p.spatial, kMaxSplit), pl.rpp) * pl.rpp;
@@ -334,8 +339,9 @@ __global__ void __launch_bounds__(kBlock) gn_welford_finalize(const float* __res
 // all of them get the same bits). `rows` points at the sample's slots [split][quantity][group], 2 * G floats per
 // split, nsplit * 2 * G <= kFoldFloats in total and 2 * G a power of two <= 64. Thread t reads the 16-byte pieces
 // t, t + 256, ... (all loads in flight at once) and keeps one running sum per float of its piece's column; the
-// threads that share a column are then added in thread order through LDS. Thread c < 2 * G ends up holding the
-// total of column c (quantity c / G, group c % G) and passes it to emit(c, total).
+// threads that share a column are then added by a fixed butterfly inside each wavefront and the four wavefronts in
+// order through LDS. Thread c < 2 * G ends up holding the total of column c (quantity c / G, group c % G) and passes
+// it to emit(c, total).
 constexpr int kFoldFloats = 16384;
 
 __host__ __device__ __forceinline__ bool fold_in_consumer(int G, int nsplit, int per_group = 2) {
@@ -360,21 +366,25 @@ __device__ __forceinline__ void fold_split_partials(const float* __restrict__ ro
   float4 s = v[0];
 #pragma unroll
   for (int k = 1; k < NB; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
-  *reinterpret_cast<float4*>(lds + tid * 4) = s;
-  __syncthreads();
-  if (tid < cols) {
-    // column tid appears in the pieces of threads tid / 4 + j * (cols / 4), at float tid % 4
-    const int per = cols / 4, nthr = kBlock / per;
-    float t = 0.f;
-    for (int j = 0; j < nthr; ++j) t += lds[(tid / 4 + j * per) * 4 + (tid & 3)];
-    emit(tid, t);
+  // threads tid % (cols / 4) alike hold the same four columns: a butterfly over them inside the wavefront, then the four
+  // wavefronts in order through LDS
+  const int per = cols / 4;
+  for (int off = 32; off >= per; off >>= 1) {
+    s.x += __shfl_xor(s.x, off, 64);
+    s.y += __shfl_xor(s.y, off, 64);
+    s.z += __shfl_xor(s.z, off, 64);
+    s.w += __shfl_xor(s.w, off, 64);
   }
+  const int lane = tid & 63, wave = tid >> 6;
+  if (lane < per) *reinterpret_cast<float4*>(lds + wave * cols + lane * 4) = s;
+  __syncthreads();
+  if (tid < cols) emit(tid, (lds[tid] + lds[cols + tid]) + (lds[2 * cols + tid] + lds[3 * cols + tid]));
 }
 
 // The same inside a consumer for a producer's Welford records rec[record][group] = { count, mean, M2, - } of one sample
 // (G a power of two, nrec * 4 G <= kFoldFloats): a thread's pieces t, t + 256, ... all belong to group t % G; it
-// merges them about the first record's mean c (see gn_welford_finalize), the threads of a group are added in thread
-// order. Thread g < G passes its group's (c, A, Q) to emit.
+// merges them about the first record's mean c (see gn_welford_finalize), the threads of a group are added by a fixed
+// butterfly inside each wavefront and the four wavefronts in order. Thread g < G passes its group's (c, A, Q) to emit.
 template <typename Emit>
 __device__ __forceinline__ void fold_welford_records(const float* __restrict__ rec, int G, int nrec, float* lds /* 4 * kBlock */,
                                                      Emit emit) {
@@ -395,12 +405,21 @@ __device__ __forceinline__ void fold_welford_records(const float* __restrict__ r
     a = fmaf(v[k].x, d, a);
     q += fmaf(v[k].x * d, d, v[k].z);
   }
-  lds[2 * tid] = a;
-  lds[2 * tid + 1] = q;
+  // threads tid % G alike hold the same group: a butterfly over them inside the wavefront, then the four wavefronts in
+  // order through LDS
+  for (int off = 32; off >= G; off >>= 1) {
+    a += __shfl_xor(a, off, 64);
+    q += __shfl_xor(q, off, 64);
+  }
+  const int lane = tid & 63, wave = tid >> 6;
+  if (lane < G) {
+    lds[(wave * G + lane) * 2] = a;
+    lds[(wave * G + lane) * 2 + 1] = q;
+  }
   __syncthreads();
   if (tid < G) {
-    float ta = 0.f, tq = 0.f;
-    for (int t = tid; t < kBlock; t += G) { ta += lds[2 * t]; tq += lds[2 * t + 1]; }
+    const float ta = (lds[2 * tid] + lds[2 * (G + tid)]) + (lds[2 * (2 * G + tid)] + lds[2 * (3 * G + tid)]);
+    const float tq = (lds[2 * tid + 1] + lds[2 * (G + tid) + 1]) + (lds[2 * (2 * G + tid) + 1] + lds[2 * (3 * G + tid) + 1]);
     emit(tid, c, ta, tq);
   }
 }
@@ -434,6 +453,12 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   int64_t row = begin + r;
   Piece<T, V> cur[U];
   fetch_rows<T, V, U>(cur, xs, row, step, end, begin, C, r < rpp);
+  float ga[V], be[V];  // asked for with the rows, so that the fold below is the only wait for memory before the stores
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    ga[e] = load_param(gamma, param_dtype, cv * V + e, 1.f);
+    be[e] = load_param(beta, param_dtype, cv * V + e, 0.f);
+  }
   // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid, sums about the
   // common shift), or (`welford`) the records the producer of x left
   if (welford && fold_in_consumer(G, npart, kGnRecordFloats)) {
@@ -483,14 +508,12 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
     }
   }
   if (r >= rpp) return;
-  float mu[V], rs[V], ga[V], be[V];
+  float mu[V], rs[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = cv * V + e;
     mu[e] = g_mean[c / cg];
     rs[e] = g_rstd[c / cg];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
   }
   TO* ys = y + y_sample + y_halo * C + cv * V;
   while (row < end) {
@@ -734,6 +757,15 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   Piece<TG, V> cg_[U];
   fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, r < rpp);
   fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, r < rpp);
+  float mu[V], rs[V], ga[V], be[V];  // asked for with the rows: the fold below is the only other wait for memory
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const int c = cv * V + e;
+    mu[e] = mean[n * G + c / cg];
+    rs[e] = rstd[n * G + c / cg];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
+  }
   const bool fused = fold_in_consumer(G, nsplit);
   if (fused) {
     // gpart quantity 0 = sum dy'*gamma*xhat (-> B), quantity 1 = sum dy'*gamma (-> A)
@@ -746,15 +778,10 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   }
   __syncthreads();
   if (r < rpp) {
-  float mu[V], rs[V], ga[V], be[V], ca[V], cb[V];
+  float ca[V], cb[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
-    const int c = cv * V + e;
-    const int g = c / cg;
-    mu[e] = mean[n * G + g];
-    rs[e] = rstd[n * G + g];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
+    const int g = (cv * V + e) / cg;
     ca[e] = gco[G + g];
     cb[e] = gco[g];
   }
