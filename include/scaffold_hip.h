@@ -117,6 +117,7 @@ int sfh_conv3d_uses_mfma(const sfh_conv3d_desc* p, int dtype, int direction);
 #define SFH_KERNEL_WIDE 3
 #define SFH_KERNEL_WGRAD 4
 #define SFH_KERNEL_OTHER_MATRIX 5
+#define SFH_KERNEL_SPLIT 6 /* 64-voxel bricks, the reduction cut over the wavefronts of a workgroup: one slice in memory */
 int sfh_conv3d_launch_geometry(const sfh_conv3d_desc* p, int dtype, int direction, int32_t geometry[4]);
 
 /* ---- measurement: what the matrix pipe sustains ----------------------------------------

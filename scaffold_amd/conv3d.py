@@ -340,7 +340,7 @@ def uses_mfma(in_shape, weight_shape, stride, padding, dilation, dtype, directio
     return bool(_lib.lib().sfh_conv3d_uses_mfma(ctypes.byref(desc), _lib.dtype_code(dtype), code))
 
 
-KERNEL_NAMES = ("direct", "persist", "brick", "wide", "wgrad", "other-matrix")
+KERNEL_NAMES = ("direct", "persist", "brick", "wide", "wgrad", "other-matrix", "split")
 
 
 def launch_geometry(in_shape, weight_shape, stride, padding, dilation, dtype, direction: str = "fwd") -> dict:

@@ -558,7 +558,7 @@ int mfma_pack_weight_batch(const MfmaPackItem* items, int n, int dtype, hipStrea
 }
 
 size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
-  if (mfma_conv_wide_applies(a)) return 0;
+  if (mfma_conv_wide_applies(a) || mfma_conv_split_applies(a)) return 0;
   const GatherPlan p = gather_plan(a);
   if (a.cred == kChunk || p.ksplit == 1) return 0;
   return align_up((size_t)p.ksplit * a.n * a.od * a.oh * a.ow * a.cout * sizeof(float), 256);
@@ -566,6 +566,7 @@ size_t mfma_conv_partial_bytes(const MfmaConvArgs& a) {
 
 MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a) {
   if (mfma_conv_wide_applies(a)) return mfma_conv_wide_geometry(a);
+  if (mfma_conv_split_applies(a)) return mfma_conv_split_geometry(a);
   const GatherPlan p = gather_plan(a);
   const int* t = kTileDims[p.shape / 3][p.shape % 3];
   return MfmaConvGeometry{kKernelBrick, t[0] * t[1] * t[2], p.nsub, p.ksplit};
@@ -573,6 +574,7 @@ MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a) {
 
 int mfma_conv_gather_gn_records(const MfmaConvArgs& a, int groups) {
   if (mfma_conv_wide_applies(a)) return mfma_conv_wide_gn_records(a, groups);
+  if (mfma_conv_split_applies(a)) return mfma_conv_split_gn_records(a, groups);
   return gather_gn_records(a, gather_plan(a), groups);
 }
 
@@ -582,12 +584,14 @@ int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void
     if (out2 != nullptr) return fail(SFH_ERR_UNSUPPORTED, "conv wide: the output cannot be a pair of tensors");
     return mfma_conv_wide(a, dtype, x, packed, bias, y, st, gn, in2);
   }
+  if (mfma_conv_split_applies(a)) return mfma_conv_split(a, dtype, x, packed, bias, y, st, gn, in2, out2);
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, dtype, x, packed, bias, y, partial, st, gn, in2, out2);
   return launch_typed<fp16_t>(a, dtype, x, packed, bias, y, partial, st, gn, in2, out2);
 }
 
 bool mfma_conv_gather_pair_ok(const MfmaConvArgs& a, int first, bool as_output) {
   if (mfma_conv_wide_applies(a)) return !as_output && mfma_conv_wide_pair_ok(a, first);
+  if (mfma_conv_split_applies(a)) return mfma_conv_split_pair_ok(a, first, as_output);
   return gather_pair_ok(a, first, as_output);
 }
 

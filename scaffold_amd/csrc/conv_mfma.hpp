@@ -48,6 +48,14 @@ int mfma_conv_gather(const MfmaConvArgs& a, int dtype, const void* x, const void
 bool mfma_conv_wide_applies(const MfmaConvArgs& a);
 int mfma_conv_wide(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
                    const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr);
+// Same contract, the kernel for the small volumes of the deep levels: 64-voxel bricks, the reduction cut over the four
+// wavefronts of a workgroup and summed in LDS (conv_split.hip). `applies` is a pure function of the shape; mfma_conv_gather
+// routes to it (it needs no partial workspace). Input or output may be a ChannelPair cut at a multiple of 32.
+bool mfma_conv_split_applies(const MfmaConvArgs& a);
+int mfma_conv_split(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y, hipStream_t st,
+                    const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr, const ChannelPair* out2 = nullptr);
+int mfma_conv_split_gn_records(const MfmaConvArgs& a, int groups);
+bool mfma_conv_split_pair_ok(const MfmaConvArgs& a, int first, bool as_output);
 // Same contract, persistent one-workgroup-per-CU kernel with register-resident weights.
 int mfma_conv_persist(const MfmaConvArgs& a, int dtype, const void* x, const void* packed, const void* bias, void* y,
                       void* partial, hipStream_t st, const GnPartialOut* gn = nullptr, const ChannelPair* in2 = nullptr,
@@ -69,11 +77,12 @@ int mfma_conv_wide_gn_records(const MfmaConvArgs& a, int groups);
 // Which of the three kernels mfma_conv_persist ends up launching for a problem, and with what geometry: a pure function of
 // the shape. `voxels` is the output tile of a workgroup step, `blocks` the 32-channel output blocks a workgroup produces
 // from one staged brick, `slices` the cuts of the reduction channels (1: none, no partial workspace).
-enum MfmaConvKernel { kKernelPersist = 1, kKernelBrick = 2, kKernelWide = 3 };
+enum MfmaConvKernel { kKernelPersist = 1, kKernelBrick = 2, kKernelWide = 3, kKernelSplit = 6 };
 struct MfmaConvGeometry { int kernel, voxels, blocks, slices; };
 MfmaConvGeometry mfma_conv_geometry(const MfmaConvArgs& a);
 bool mfma_conv_persist_applies(const MfmaConvArgs& a);
 MfmaConvGeometry mfma_conv_gather_geometry(const MfmaConvArgs& a);
 MfmaConvGeometry mfma_conv_wide_geometry(const MfmaConvArgs& a);
+MfmaConvGeometry mfma_conv_split_geometry(const MfmaConvArgs& a);
 
 }  // namespace sfh

@@ -8,7 +8,8 @@
 // How a record stays accurate when the mean is large against the spread: sums are taken about a value of their own
 // data. Every wavefront sums v - K and (v - K)^2 with K = the first output it stored inside the tensor (per 4-channel
 // run), which is within a few standard deviations of the mean, so S2 - S1^2/n does not cancel; the wavefronts' sums
-// become (n, mean, M2) and are merged about the first one's mean, where the correction terms n d^2 are small again.
+// become (n, mean, M2) and are merged pairwise (mean and M2 of two pieces from their counts, means and M2s), where the
+// correction terms are small again.
 // No atomics: every (record, group) slot is written by exactly one workgroup and every sum has a fixed order, so the
 // statistics are the same bits on every run.
 #pragma once
@@ -144,19 +145,60 @@ __device__ __forceinline__ void write_group_partials(const RunSums (&rs)[NSUB], 
   }
   __syncthreads();
   const int span = 32 * NSUB;
-  const int runs_per_group = (o.cg < span ? o.cg : span) / 4;
-  const int ngroups = span / (runs_per_group * 4);
-  if (tid < ngroups) {
-    WelfordMerge m;
-    m.clear();
-    for (int w = 0; w < NW; ++w)
-      for (int r = 0; r < runs_per_group; ++r) {
-        const float4 e = *reinterpret_cast<const float4*>(lds + (w * (NSUB * 8) + tid * runs_per_group + r) * 4);
-        m.add_sums(e.x, e.y, e.z, e.w);
+  const int runs_per_group = (o.cg < span ? o.cg : span) / 4;  // a power of two (gn_partials_fit)
+  constexpr int RUNS = NSUB * 8, ENTRIES = NW * RUNS;
+  if constexpr (ENTRIES <= 64 && (NW & (NW - 1)) == 0) {
+    // One lane of the first wavefront per (wavefront, run) entry: each turns its sums into (n, mean, M2), then the
+    // entries of a group -- runs_per_group neighbouring runs of every wavefront -- are merged pairwise (Chan et al.) in a
+    // fixed butterfly: both partners of a step merge (lower lane, upper lane) in that order and get the same bits.
+    if (tid < 64) {
+      float pn = 0.f, mean = 0.f, m2 = 0.f;
+      if (tid < ENTRIES) {
+        const float4 e = *reinterpret_cast<const float4*>(lds + tid * 4);
+        if (e.x > 0.f) {
+          const float dm = e.y / e.x;
+          pn = e.x;
+          mean = e.w + dm;
+          m2 = fmaf(-e.y, dm, e.z);
+          m2 = m2 < 0.f ? 0.f : m2;
+        }
       }
-    const int group = (c0 + tid * runs_per_group * 4) / o.cg;
-    *reinterpret_cast<float4*>(o.part + (((int64_t)n * o.records + rec) * o.groups + group) * kGnRecordFloats) =
-        make_float4(m.n, m.mean(), m.m2(), 0.f);
+      auto merge_with = [&](int off) {
+        const float qn = __shfl_xor(pn, off, 64), qmean = __shfl_xor(mean, off, 64), qm2 = __shfl_xor(m2, off, 64);
+        const bool upper = (tid & off) != 0;
+        const float n1 = upper ? qn : pn, n2 = upper ? pn : qn;
+        const float mean1 = upper ? qmean : mean, mean2 = upper ? mean : qmean;
+        const float ma = upper ? qm2 : m2, mb = upper ? m2 : qm2;
+        const float nn = n1 + n2;
+        const float w2 = nn > 0.f ? n2 / nn : 0.f;
+        const float d = mean2 - mean1;
+        pn = nn;
+        mean = n1 > 0.f ? fmaf(d, w2, mean1) : mean2;
+        m2 = (ma + mb) + (n1 > 0.f && n2 > 0.f ? d * d * n1 * w2 : 0.f);
+      };
+      for (int off = 1; off < runs_per_group; off <<= 1) merge_with(off);
+#pragma unroll
+      for (int off = RUNS; off < ENTRIES; off <<= 1) merge_with(off);
+      if (tid < RUNS && (tid & (runs_per_group - 1)) == 0) {
+        const int group = (c0 + tid * 4) / o.cg;
+        *reinterpret_cast<float4*>(o.part + (((int64_t)n * o.records + rec) * o.groups + group) * kGnRecordFloats) =
+            make_float4(pn, mean, m2, 0.f);
+      }
+    }
+  } else {
+    const int ngroups = span / (runs_per_group * 4);
+    if (tid < ngroups) {
+      WelfordMerge m;
+      m.clear();
+      for (int w = 0; w < NW; ++w)
+        for (int r = 0; r < runs_per_group; ++r) {
+          const float4 e = *reinterpret_cast<const float4*>(lds + (w * RUNS + tid * runs_per_group + r) * 4);
+          m.add_sums(e.x, e.y, e.z, e.w);
+        }
+      const int group = (c0 + tid * runs_per_group * 4) / o.cg;
+      *reinterpret_cast<float4*>(o.part + (((int64_t)n * o.records + rec) * o.groups + group) * kGnRecordFloats) =
+          make_float4(m.n, m.mean(), m.m2(), 0.f);
+    }
   }
 }
 

@@ -92,7 +92,7 @@ def test_launch_geometry_is_stated_and_agrees_with_the_workspace():
         L.sfh_conv3d_launch_geometry(ctypes.byref(desc), dtype, direction, out)
         return out
 
-    DIRECT, PERSIST, BRICK, WIDE, WGRAD, OTHER = range(6)
+    DIRECT, PERSIST, BRICK, WIDE, WGRAD, OTHER, SPLIT = range(7)
     cube = conv_desc(sp=(128, 128, 128))
     assert geometry(cube, bf16, 0) == [PERSIST, 512, 1, 1] and geometry(cube, bf16, 1) == [PERSIST, 512, 1, 1]
     assert geometry(cube, bf16, 2) == [WGRAD, 256, 1, L.sfh_conv3d_wgrad_splits(ctypes.byref(cube), bf16)]
@@ -102,12 +102,17 @@ def test_launch_geometry_is_stated_and_agrees_with_the_workspace():
     # round of their own
     assert geometry(conv_desc(cin=64, cout=64, sp=(34, 64, 64), p=(0, 1, 1)), bf16, 1) == [BRICK, 256, 1, 1]
     assert geometry(conv_desc(cin=64, cout=64, sp=(64, 64, 64)), bf16, 0) == [BRICK, 512, 2, 1]
-    # a deep, small-volume level: the reduction channels are cut into slices, and the workspace holds their fp32 partials
-    deep = conv_desc(cin=256, cout=256, sp=(10, 16, 16), p=(0, 1, 1))
+    # a small-volume level: 64-voxel bricks, the reduction cut over the wavefronts of a workgroup -- no slices, no partials
+    small = conv_desc(cin=256, cout=256, sp=(10, 16, 16), p=(0, 1, 1))
+    assert geometry(small, bf16, 0) == [SPLIT, 64, 2, 1] and geometry(small, bf16, 1) == [SPLIT, 64, 2, 1]
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(small), bf16) == 256 * 256 * 27 * 2
+    # the deepest level: too few bricks for that, the reduction channels are cut into slices and the workspace holds their
+    # fp32 partials
+    deep = conv_desc(cin=256, cout=512, sp=(6, 8, 8), p=(0, 1, 1))
     kernel, voxels, blocks, slices = geometry(deep, bf16, 0)
     assert (kernel, voxels, blocks) == (BRICK, 256, 1) and 1 < slices <= 8 and slices & (slices - 1) == 0
-    packed = 256 * 256 * 27 * 2
-    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(deep), bf16) == packed + slices * 8 * 16 * 16 * 256 * 4
+    packed = 256 * 512 * 27 * 2
+    assert L.sfh_conv3d_fwd_workspace_bytes(ctypes.byref(deep), bf16) == packed + slices * 4 * 8 * 8 * 512 * 4
     out = (ctypes.c_int32 * 4)()
     assert L.sfh_conv3d_launch_geometry(ctypes.byref(cube), bf16, 3, out) == _lib.SFH_ERR_INVALID
     assert L.sfh_conv3d_launch_geometry(ctypes.byref(cube), bf16, 0, None) == _lib.SFH_ERR_INVALID

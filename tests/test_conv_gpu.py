@@ -99,20 +99,58 @@ def test_mfma_exact(device, dtype, cin, cout, spatial, padding, direction):
 # tile shape and block count, with the geometry the rule must give for it, so that no instantiation goes untested and a
 # change of the rule shows up here.
 GEOMETRY_CASES = [
-    # (n, cin, cout, spatial, direction, voxels, blocks)
-    (1, 64, 128, (32, 32, 32), "fwd", 512, 1),        # rows of 32: 4 x 4 x 32
+    # (n, cin, cout, spatial, direction, voxels, blocks); planes of more than 32 x 32 voxels, or 96 channels: small
+    # planes with blocks of 64 channels belong to the kernel that cuts the reduction inside the workgroup (SPLIT_CASES)
+    (1, 64, 128, (32, 33, 32), "bwd-data", 512, 1),   # rows of 32: 4 x 4 x 32
     (1, 64, 128, (32, 64, 32), "fwd", 512, 2),
-    (1, 64, 128, (32, 32, 32), "bwd-data", 256, 1),   # 2 x 4 x 32
+    (1, 64, 128, (32, 33, 32), "fwd", 256, 1),        # 2 x 4 x 32
     (1, 64, 128, (2, 128, 128), "fwd", 256, 2),
-    (1, 64, 512, (16, 32, 16), "fwd", 512, 1),        # rows of 16: 4 x 8 x 16
-    (1, 64, 256, (32, 64, 16), "fwd", 512, 2),
+    (1, 64, 96, (16, 128, 16), "fwd", 512, 1),        # rows of 16: 4 x 8 x 16
+    (1, 64, 64, (32, 256, 16), "fwd", 512, 2),
     (1, 64, 64, (4, 8, 16), "fwd", 256, 1),           # 2 x 8 x 16
-    (4, 64, 256, (2, 128, 16), "fwd", 256, 2),
-    (1, 64, 512, (32, 32, 8), "fwd", 512, 1),         # rows of 8: 8 x 8 x 8
-    (1, 64, 256, (64, 64, 8), "fwd", 512, 2),
+    (1, 64, 128, (9, 192, 16), "fwd", 256, 2),
+    (1, 64, 96, (24, 128, 8), "fwd", 512, 1),         # rows of 8: 8 x 8 x 8
+    (1, 64, 128, (32, 256, 8), "fwd", 512, 2),
     (1, 128, 64, (4, 8, 8), "fwd", 256, 1),           # 4 x 8 x 8
-    (4, 64, 256, (4, 128, 8), "fwd", 256, 2),
+    (1, 64, 128, (17, 192, 8), "fwd", 256, 2),
 ]
+
+
+# Small volumes with 64 or more reduction channels and output channels in blocks of 64 go to the kernel that cuts the
+# reduction over the wavefronts of a workgroup (64-voxel bricks, two output blocks): both round sizes (four chunks, two
+# chunks), several rounds, ragged bricks on every axis, several samples, the padding forms of a depth shard -- and the
+# edges of its launch rule (the plane bound, the workgroup bound, channel counts it does not take).
+SPLIT_CASES = [
+    # (n, cin, cout, spatial, padding, direction, kernel)
+    (1, 128, 128, (16, 32, 32), (1, 1, 1), "fwd", "split"),       # a 16 x 32 x 32 level: one round of four chunks
+    (1, 128, 128, (18, 32, 32), (0, 1, 1), "fwd", "split"),       # ... on a depth shard's slab
+    (1, 128, 128, (18, 32, 32), (0, 1, 1), "bwd-data", "split"),  # ... and the data gradient onto the slab (18 planes)
+    (1, 64, 128, (16, 32, 32), (1, 1, 1), "fwd", "split"),        # two chunks: the wavefront pairs share a chunk's k-steps
+    (1, 128, 64, (7, 13, 35), (1, 1, 1), "bwd-data", "split"),    # two chunks, ragged on every axis
+    (1, 256, 128, (9, 18, 27), (1, 1, 1), "fwd", "split"),        # two rounds of four chunks, ragged
+    (1, 192, 128, (8, 16, 40), (1, 1, 1), "fwd", "split"),        # six chunks: three rounds of two
+    (2, 512, 256, (4, 8, 16), (1, 1, 1), "fwd", "split"),         # four rounds, two samples
+    (3, 128, 192, (3, 9, 11), (2, 2, 2), "fwd", "split"),         # padding 2, three samples, three block pairs
+    (1, 256, 256, (8, 16, 16), (1, 1, 1), "bwd-data", "split"),   # an 8 x 16 x 16 level
+    (1, 128, 128, (40, 32, 32), (1, 1, 1), "fwd", "split"),       # whatever the depth: several rounds of workgroups
+    (1, 128, 128, (6, 32, 33), (1, 1, 1), "fwd", "brick"),        # a plane of more than 32 x 32 voxels
+    (1, 256, 192, (8, 16, 16), (1, 1, 1), "fwd", "split"),        # 24 workgroups per two planes: the fewest it takes
+    (1, 256, 128, (8, 16, 16), (1, 1, 1), "fwd", "brick"),        # 16
+    (1, 256, 512, (4, 8, 8), (1, 1, 1), "fwd", "brick"),          # 16 per two planes: too few, the brick kernel slices
+    (1, 128, 96, (16, 32, 32), (1, 1, 1), "fwd", "brick"),        # 96 output channels are not blocks of 64
+    (1, 96, 128, (16, 32, 32), (1, 1, 1), "fwd", "brick"),        # three chunks are not an even number
+]
+
+
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,direction,kernel", SPLIT_CASES)
+def test_small_volume_kernel_exact(device, n, cin, cout, spatial, padding, direction, kernel):
+    for dtype in (torch.bfloat16, torch.float16):
+        prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=dtype)
+        geom = c3.launch_geometry(prob.input_shape, prob.weight_shape, 1, padding, 1, dtype, direction)
+        assert geom["kernel"] == kernel, geom
+        if kernel == "split":
+            assert (geom["voxels"], geom["blocks"], geom["slices"]) == (64, 2, 1), geom
+        check_exact(prob, direction, device)
 
 
 @pytest.mark.parametrize("n,cin,cout,spatial,direction,voxels,blocks", GEOMETRY_CASES)

@@ -29,10 +29,13 @@ CASES = [
     (1, 64, 64, 64, (32, 64, 64), (0, 1, 1), "wide", "brick"),       # the level-1 decoder shape: wide forward
     (1, 64, 64, 64, (31, 61, 65), (1, 1, 1), "wide", "brick"),       # ragged on every axis
     (1, 32, 96, 64, (32, 64, 64), (1, 1, 1), None, "brick"),         # wide forward takes equal halves only: not offered
-    (1, 64, 64, 64, (16, 32, 16), (1, 1, 1), "brick", "brick"),      # rows of 16: the brick kernel, two blocks a workgroup
-    (2, 128, 128, 128, (10, 20, 32), (1, 1, 1), "brick", "brick"),   # the level-2 decoder shape
-    (1, 256, 256, 256, (10, 16, 16), (0, 1, 1), "brick", "brick"),   # level 3 on a shard: forward sliced
-    (1, 256, 256, 256, (8, 16, 16), (1, 1, 1), "brick", "brick"),    # ... and as a cube: both directions sliced
+    (1, 64, 64, 128, (9, 192, 16), (1, 1, 1), "brick", "brick"),     # rows of 16: the brick kernel, two blocks a workgroup
+    (1, 64, 64, 128, (16, 32, 16), (1, 1, 1), "split", "split"),     # a small volume: the reduction cut over the wavefronts
+    (2, 128, 128, 128, (10, 20, 32), (1, 1, 1), "split", "split"),   # the level-2 decoder shape, two rounds of four chunks
+    (1, 256, 256, 256, (10, 16, 16), (0, 1, 1), "split", "split"),   # level 3 on a shard
+    (1, 256, 256, 256, (8, 16, 16), (1, 1, 1), "split", "split"),    # ... and as a cube
+    (1, 96, 160, 128, (7, 13, 35), (1, 1, 1), "split", "split"),     # unequal cut inside a round, ragged
+    (1, 256, 256, 512, (4, 8, 8), (1, 1, 1), "brick", "brick"),      # level 4: both directions sliced
     (1, 128, 64, 96, (4, 8, 8), (1, 1, 1), "brick", "brick"),        # sliced, unequal cut, 96 output channels
     (3, 32, 32, 64, (4, 8, 24), (1, 1, 1), "brick", "brick"),        # three samples, two output blocks
 ]
@@ -88,7 +91,8 @@ def test_pair_is_bitwise_the_concatenation(device, dtype, case):
         assert got.dtype is want.dtype and torch.equal(got, want)
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[4], CASES[9], CASES[11]], ids=["brick-persist", "wide", "sliced-shard", "sliced-unequal"])
+@pytest.mark.parametrize("case", [CASES[0], CASES[4], CASES[10], CASES[12], CASES[13], CASES[14]],
+                         ids=["brick-persist", "wide", "split-shard", "split-unequal", "sliced", "sliced-unequal"])
 def test_pair_against_the_oracle(device, case):
     """Straight to the fp64 oracle on the concatenated operands, with the error bound of the convolution parity tests."""
     n, c0, c1, cout, spatial, padding, _, _ = case

@@ -35,7 +35,11 @@ CASES = [
     (1, 32, 32, (10, 8, 8), (1, 1, 1), 8, "persist"),          # rows of 8
     (2, 64, 64, (16, 32, 64), (1, 1, 1), 8, "brick"),          # two samples, no slices
     (1, 64, 128, (32, 64, 32), (1, 1, 1), 8, "brick"),         # two output blocks per workgroup
-    (1, 64, 128, (16, 32, 33), (1, 1, 1), 2, "brick"),         # a group wider than the workgroup's span, ragged rows
+    (1, 64, 96, (16, 32, 33), (1, 1, 1), 1, "brick"),          # a group wider than the workgroup's span, ragged rows
+    (1, 64, 128, (16, 32, 31), (1, 1, 1), 2, "split"),         # small volume, reduction cut over the wavefronts: a group = the workgroup's 64 channels
+    (1, 128, 256, (10, 16, 16), (0, 1, 1), 8, "split"),        # two groups per workgroup, shard form
+    (1, 128, 256, (8, 16, 16), (1, 1, 1), 1, "split"),         # one group of all channels: four workgroups of a brick leave a record each
+    (2, 256, 128, (5, 9, 21), (1, 1, 1), 32, "split"),         # 4 channels per group, two samples, ragged bricks
     (2, 64, 64, (9, 10, 16), (1, 1, 1), 16, "brick"),          # small volume: the reduction is sliced, the slice sum counts
     (1, 256, 512, (4, 8, 8), (1, 1, 1), 8, "brick"),           # deep level, sliced
     (1, 128, 256, (4, 8, 8), (1, 1, 1), 1, "brick"),           # sliced, one group of all channels (256 pieces merged per record)
@@ -163,7 +167,7 @@ def test_group_norm_from_partials_matches_the_statistics_pass(device, n, cin, co
     assert orc.gn_rel_error(fused, ref) < 2e-2
 
 
-@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", [CASES[2], CASES[7], CASES[10], CASES[14], CASES[15]])
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,groups,kernel", [CASES[2], CASES[7], CASES[11], CASES[14], CASES[18], CASES[19]])
 def test_large_mean_small_std_on_the_first_call(device, n, cin, cout, spatial, padding, groups, kernel):
     """A mean a thousand times the spread (fp16 resolves it; bf16 does not), the case of the reference's
     ``test_large_mean_small_std`` (tests/test_triton_group_norm.py:502-547): plain fp32 sums of y and y^2 lose the variance
