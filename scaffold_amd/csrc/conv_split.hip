@@ -284,16 +284,21 @@ int launch_split_typed(const MfmaConvArgs& a, const void* x, const void* packed,
 // brick kernel on every convolution of a five-level U-Net step: 10-25 % faster at 16 x 32 x 32 and 8 x 16 x 16, where the
 // brick kernel runs as one round of workgroups or needs slices; slower on 32 x 64 x 64 (several rounds of bricks overlap
 // staging and MFMAs by themselves, and 64-voxel bricks stage 3.75 voxels per output voxel) and at 4 x 8 x 8 (a handful
-// of workgroups cannot pull 7-14 MiB of weights fast enough: that level needs the slices over many CUs).
+// of workgroups cannot pull 7-14 MiB of weights fast enough: that level needs the slices over many CUs). For the same
+// reason it leaves reductions of 512 channels or more to the slices where its workgroups would number 32 or fewer per
+// two planes (8 x 16 x 16 with 256 produced channels: 128 workgroups of 1.7 MiB of weights each, 41 us against 30 with
+// the weights cold; eight wavefronts per workgroup instead of four changed nothing, which is how the bound was found).
 // The rule does not look at the depth: the data gradient of a depth shard's slab (D + 2 planes) and of the padded volume
 // (D planes) must come from the same kernel, or a shard and the whole volume would disagree in the last bit.
-constexpr int kSplitMaxPlane = 32 * 32, kSplitMinPerDepth = 24;
+constexpr int kSplitMaxPlane = 32 * 32, kSplitMinPerDepth = 24, kSplitFewPerDepth = 32, kSplitFewMaxChunks = 16;
 
 bool mfma_conv_split_applies(const MfmaConvArgs& a) {
   if (a.kd != 3 || a.kh != 3 || a.kw != 3) return false;
   if (a.cred < 2 * kChunk || a.cred % (2 * kChunk) != 0 || a.cout % (32 * NSUB) != 0) return false;
   if ((int64_t)a.oh * a.ow > kSplitMaxPlane) return false;
-  return (int64_t)a.n * cdiv(a.oh, TH) * cdiv(a.ow, TW) * (a.cout / (32 * NSUB)) >= kSplitMinPerDepth;
+  const int64_t per_depth = (int64_t)a.n * cdiv(a.oh, TH) * cdiv(a.ow, TW) * (a.cout / (32 * NSUB));
+  if (per_depth <= kSplitFewPerDepth && a.cred / kChunk >= kSplitFewMaxChunks) return false;
+  return per_depth >= kSplitMinPerDepth;
 }
 
 MfmaConvGeometry mfma_conv_split_geometry(const MfmaConvArgs&) { return MfmaConvGeometry{kKernelSplit, TD * TH * TW, NSUB, 1}; }

@@ -129,7 +129,8 @@ SPLIT_CASES = [
     (1, 128, 64, (7, 13, 35), (1, 1, 1), "bwd-data", "split"),    # two chunks, ragged on every axis
     (1, 256, 128, (9, 18, 27), (1, 1, 1), "fwd", "split"),        # two rounds of four chunks, ragged
     (1, 192, 128, (8, 16, 40), (1, 1, 1), "fwd", "split"),        # six chunks: three rounds of two
-    (2, 512, 256, (4, 8, 16), (1, 1, 1), "fwd", "split"),         # four rounds, two samples
+    (2, 512, 256, (4, 16, 16), (1, 1, 1), "fwd", "split"),        # four rounds, two samples
+    (1, 512, 256, (8, 16, 16), (1, 1, 1), "fwd", "brick"),        # 512 channels to reduce for 32 workgroups per two planes: slices
     (3, 128, 192, (3, 9, 11), (2, 2, 2), "fwd", "split"),         # padding 2, three samples, three block pairs
     (1, 256, 256, (8, 16, 16), (1, 1, 1), "bwd-data", "split"),   # an 8 x 16 x 16 level
     (1, 128, 128, (40, 32, 32), (1, 1, 1), "fwd", "split"),       # whatever the depth: several rounds of workgroups

@@ -32,8 +32,9 @@ CASES = [
     (1, 64, 64, 128, (9, 192, 16), (1, 1, 1), "brick", "brick"),     # rows of 16: the brick kernel, two blocks a workgroup
     (1, 64, 64, 128, (16, 32, 16), (1, 1, 1), "split", "split"),     # a small volume: the reduction cut over the wavefronts
     (2, 128, 128, 128, (10, 20, 32), (1, 1, 1), "split", "split"),   # the level-2 decoder shape, two rounds of four chunks
-    (1, 256, 256, 256, (10, 16, 16), (0, 1, 1), "split", "split"),   # level 3 on a shard
-    (1, 256, 256, 256, (8, 16, 16), (1, 1, 1), "split", "split"),    # ... and as a cube
+    (1, 256, 256, 256, (10, 16, 16), (0, 1, 1), "brick", "split"),   # level 3 on a shard: forward sliced
+    (1, 256, 256, 256, (8, 16, 16), (1, 1, 1), "brick", "split"),    # ... and as a cube
+    (1, 128, 128, 256, (8, 16, 16), (1, 1, 1), "split", "split"),    # two rounds of four chunks from the two tensors in turn
     (1, 96, 160, 128, (7, 13, 35), (1, 1, 1), "split", "split"),     # unequal cut inside a round, ragged
     (1, 256, 256, 512, (4, 8, 8), (1, 1, 1), "brick", "brick"),      # level 4: both directions sliced
     (1, 128, 64, 96, (4, 8, 8), (1, 1, 1), "brick", "brick"),        # sliced, unequal cut, 96 output channels
@@ -91,8 +92,8 @@ def test_pair_is_bitwise_the_concatenation(device, dtype, case):
         assert got.dtype is want.dtype and torch.equal(got, want)
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[4], CASES[10], CASES[12], CASES[13], CASES[14]],
-                         ids=["brick-persist", "wide", "split-shard", "split-unequal", "sliced", "sliced-unequal"])
+@pytest.mark.parametrize("case", [CASES[0], CASES[4], CASES[10], CASES[12], CASES[13], CASES[14], CASES[15]],
+                         ids=["brick-persist", "wide", "sliced-shard", "split", "split-unequal", "sliced", "sliced-unequal"])
 def test_pair_against_the_oracle(device, case):
     """Straight to the fp64 oracle on the concatenated operands, with the error bound of the convolution parity tests."""
     n, c0, c1, cout, spatial, padding, _, _ = case
