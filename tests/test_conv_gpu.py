@@ -154,6 +154,32 @@ def test_small_volume_kernel_exact(device, n, cin, cout, spatial, padding, direc
         check_exact(prob, direction, device)
 
 
+def _small_volume_cases(count, seed):
+    """Seeded random problems inside the small-volume kernel's launch rule: channel counts, one to three samples, extents
+    around the 2 x 4 x 8 brick (ragged on any axis), the padding forms of a depth shard, both directions."""
+    import random
+    rng = random.Random(seed)
+    cases = []
+    while len(cases) < count:
+        cin, cout = rng.choice([64, 128, 192, 256, 320]), rng.choice([64, 128, 192, 256])
+        n = rng.choice([1, 1, 2, 3])
+        d, h, w = rng.randint(1, 9), rng.randint(3, 32), rng.randint(3, 32)
+        pad = rng.choice([(1, 1, 1), (0, 1, 1), (2, 1, 1), (1, 0, 2)])
+        direction = rng.choice(["fwd", "bwd-data"])
+        if min(d + 2 * pad[0], h + 2 * pad[1], w + 2 * pad[2]) < 3 or n * max(cin, cout) * (d + 2) * h * w > 3_000_000:
+            continue
+        geom = c3.launch_geometry((n, cin, d, h, w), (cout, cin, 3, 3, 3), 1, pad, 1, torch.bfloat16, direction)
+        if geom["kernel"] == "split":
+            cases.append((n, cin, cout, (d, h, w), pad, direction))
+    return cases
+
+
+@pytest.mark.parametrize("n,cin,cout,spatial,padding,direction", _small_volume_cases(32, seed=20250311))
+def test_small_volume_kernel_random_problems_exact(device, n, cin, cout, spatial, padding, direction):
+    prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=padding, dtype=torch.bfloat16)
+    check_exact(prob, direction, device, seed=cin + cout + n)
+
+
 @pytest.mark.parametrize("n,cin,cout,spatial,direction,voxels,blocks", GEOMETRY_CASES)
 def test_brick_geometries_exact(device, n, cin, cout, spatial, direction, voxels, blocks):
     prob = orc.ConvProblem(n=n, cin=cin, cout=cout, spatial=spatial, padding=(1, 1, 1), dtype=torch.bfloat16)
