@@ -689,13 +689,15 @@ def conv_counter_launches(device, reps=3):
     """The launches a counter run (rocprofv3 --pmc) is taken over: plain eager calls, no graph, of the three MFMA
     convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_ring_kernel,
     wgrad_ring_kernel), 128->64 @64^3 (conv_wide_kernel, conv_mfma_kernel, wgrad_ring_kernel) and 64->32 on the 64x128x128
-    slab (conv_mfma_kernel, conv_ring_kernel, wgrad_ring_kernel), the last also with its input as two 32-channel tensors
-    (what the U-Net's decoder hands it)."""
+    slab (conv_mfma_kernel, conv_ring_kernel, wgrad_ring_kernel), also with its input as two 32-channel tensors
+    (what the U-Net's decoder hands it), and the two small-volume shapes 128->128 on the 16x32x32 slab and 256->256 on the
+    8x16x16 slab (conv_split_kernel; wgrad_ring_kernel / wgrad_mfma_kernel)."""
     import scaffold_amd as sa
 
     done = []
     for cin, cout, in_sp, pad in ((32, 32, (128, 128, 128), (1, 1, 1)), (128, 64, (64, 64, 64), (1, 1, 1)),
-                                  (64, 32, (66, 128, 128), (0, 1, 1))):
+                                  (64, 32, (66, 128, 128), (0, 1, 1)), (128, 128, (18, 32, 32), (0, 1, 1)),
+                                  (256, 256, (10, 16, 16), (0, 1, 1))):
         sp = tuple(in_sp[i] + 2 * pad[i] - 2 for i in range(3))
         g = torch.Generator().manual_seed(3000 + cin + cout)
         x = torch.randn((1, cin, *in_sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
