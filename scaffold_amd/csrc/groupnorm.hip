@@ -453,12 +453,6 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   int64_t row = begin + r;
   Piece<T, V> cur[U];
   fetch_rows<T, V, U>(cur, xs, row, step, end, begin, C, r < rpp);
-  float ga[V], be[V];  // asked for with the rows, so that the fold below is the only wait for memory before the stores
-#pragma unroll
-  for (int e = 0; e < V; ++e) {
-    ga[e] = load_param(gamma, param_dtype, cv * V + e, 1.f);
-    be[e] = load_param(beta, param_dtype, cv * V + e, 0.f);
-  }
   // `npart` partial records per sample: the statistics pass's own (one per workgroup of this grid, sums about the
   // common shift), or (`welford`) the records the producer of x left
   if (welford && fold_in_consumer(G, npart, kGnRecordFloats)) {
@@ -508,12 +502,14 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
     }
   }
   if (r >= rpp) return;
-  float mu[V], rs[V];
+  float mu[V], rs[V], ga[V], be[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = cv * V + e;
     mu[e] = g_mean[c / cg];
     rs[e] = g_rstd[c / cg];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
   }
   TO* ys = y + y_sample + y_halo * C + cv * V;
   while (row < end) {
@@ -757,15 +753,6 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   Piece<TG, V> cg_[U];
   fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, r < rpp);
   fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, r < rpp);
-  float mu[V], rs[V], ga[V], be[V];  // asked for with the rows: the fold below is the only other wait for memory
-#pragma unroll
-  for (int e = 0; e < V; ++e) {
-    const int c = cv * V + e;
-    mu[e] = mean[n * G + c / cg];
-    rs[e] = rstd[n * G + c / cg];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
-  }
   const bool fused = fold_in_consumer(G, nsplit);
   if (fused) {
     // gpart quantity 0 = sum dy'*gamma*xhat (-> B), quantity 1 = sum dy'*gamma (-> A)
@@ -778,10 +765,15 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   }
   __syncthreads();
   if (r < rpp) {
-  float ca[V], cb[V];
+  float mu[V], rs[V], ga[V], be[V], ca[V], cb[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) {
-    const int g = (cv * V + e) / cg;
+    const int c = cv * V + e;
+    const int g = c / cg;
+    mu[e] = mean[n * G + g];
+    rs[e] = rstd[n * G + g];
+    ga[e] = load_param(gamma, param_dtype, c, 1.f);
+    be[e] = load_param(beta, param_dtype, c, 0.f);
     ca[e] = gco[G + g];
     cb[e] = gco[g];
   }
