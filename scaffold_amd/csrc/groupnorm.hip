@@ -89,6 +89,42 @@ __device__ __forceinline__ float load_param(const void* p, int dtype, int i, flo
   return to_float(static_cast<const fp16_t*>(p)[i]);
 }
 
+// V consecutive parameters from element c0 (a multiple of V) as one or two vector loads behind ONE branch on the
+// dtype: a thread's eight gammas and eight betas fetched one scalar at a time, each behind its own dtype test, were
+// sixteen trips to memory one after the other (1.8 us of a 6 us launch on a small tensor).
+template <int V>
+__device__ __forceinline__ void load_params(const void* p, int dtype, int c0, float dflt, float (&out)[V]) {
+  static_assert(V == 4 || V == 8, "a thread's channel vector");
+  if (p == nullptr) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) out[e] = dflt;
+  } else if (dtype == SFH_FP32) {
+    const float* f = static_cast<const float*>(p) + c0;
+    if ((reinterpret_cast<uintptr_t>(f) & 15) == 0) {
+      Ld<float, V>::run(f, out);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = f[e];
+    }
+  } else if (dtype == SFH_BF16) {
+    const bf16_t* h = static_cast<const bf16_t*>(p) + c0;
+    if ((reinterpret_cast<uintptr_t>(h) & (2 * V - 1)) == 0) {
+      Ld<bf16_t, V>::run(h, out);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = to_float(h[e]);
+    }
+  } else {
+    const fp16_t* h = static_cast<const fp16_t*>(p) + c0;
+    if ((reinterpret_cast<uintptr_t>(h) & (2 * V - 1)) == 0) {
+      Ld<fp16_t, V>::run(h, out);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = to_float(h[e]);
+    }
+  }
+}
+
 __device__ __forceinline__ float relu_keep_nan(float y) { return y <= 0.f ? 0.f : y; }
 
 // Fixed-order sum over a 64-lane wavefront; lane 0 holds the result.
@@ -99,11 +135,48 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // Sums NVAL per-thread values over the voxel rows of the workgroup (threads sharing a channel
-// vector cv) with a fixed binary tree. Afterwards buf[v * kBlock + cv], cv < tpr, holds the
-// totals. buf needs NVAL * kBlock floats.
+// vector cv) in a fixed order. Afterwards buf[v * kBlock + cv], cv < tpr, holds the totals. buf needs
+// NVAL * kBlock floats.
+// Where tpr divides the wavefront (a power of two up to 64, every thread active): a butterfly over the lanes of a
+// wavefront that share cv, then the four wavefronts' totals through LDS in wavefront order -- three barriers whatever
+// the row count. (A binary tree over the rows through LDS, one barrier per level, took 1.9 us of a 4.8 us launch at 8
+// rows per workgroup and 3.1 us at 32.) Otherwise that tree.
 template <int NVAL>
 __device__ __forceinline__ void block_row_reduce(const float (&val)[NVAL], float* buf, int tpr, int rpp, bool active) {
   const int tid = threadIdx.x;
+  if (tpr <= 64 && (tpr & (tpr - 1)) == 0) {  // uniform over the workgroup
+    const int lane = tid & 63, wave = tid >> 6;
+    float part[NVAL];
+#pragma unroll
+    for (int v = 0; v < NVAL; ++v) part[v] = val[v];
+    for (int off = tpr; off < 64; off <<= 1) {
+#pragma unroll
+      for (int v = 0; v < NVAL; ++v) part[v] += __shfl_xor(part[v], off, 64);
+    }
+    __syncthreads();  // buf is free
+    if (lane < tpr) {
+#pragma unroll
+      for (int v = 0; v < NVAL; ++v) buf[(v * 4 + wave) * 64 + lane] = part[v];
+    }
+    __syncthreads();
+    // thread -> (value v, channel vector cv): the four wavefront totals in order
+    constexpr int PER = (NVAL * 64 + kBlock - 1) / kBlock;  // outputs per thread at most (tpr = 64)
+    float tot[PER];
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int idx = tid + k * kBlock, v = idx / tpr, cv = idx - v * tpr;
+      tot[k] = 0.f;
+      if (v < NVAL) tot[k] = (buf[(v * 4) * 64 + cv] + buf[(v * 4 + 1) * 64 + cv]) + (buf[(v * 4 + 2) * 64 + cv] + buf[(v * 4 + 3) * 64 + cv]);
+    }
+    __syncthreads();  // every total is in a register: the staging area becomes the result
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int idx = tid + k * kBlock, v = idx / tpr, cv = idx - v * tpr;
+      if (v < NVAL) buf[v * kBlock + cv] = tot[k];
+    }
+    __syncthreads();
+    return;
+  }
   const int r = tid / tpr;
   __syncthreads();
   if (active) {
@@ -503,13 +576,13 @@ __global__ void __launch_bounds__(kBlock) gn_normalize(const T* __restrict__ x, 
   }
   if (r >= rpp) return;
   float mu[V], rs[V], ga[V], be[V];
+  load_params<V>(gamma, param_dtype, cv * V, 1.f, ga);
+  load_params<V>(beta, param_dtype, cv * V, 0.f, be);
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = cv * V + e;
     mu[e] = g_mean[c / cg];
     rs[e] = g_rstd[c / cg];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
   }
   TO* ys = y + y_sample + y_halo * C + cv * V;
   while (row < end) {
@@ -569,13 +642,13 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
   fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, active);
   fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, active);
   float mu[V], rs[V], ga[V], be[V];
+  load_params<V>(gamma, param_dtype, active ? cv * V : 0, 1.f, ga);
+  load_params<V>(beta, param_dtype, active ? cv * V : 0, 0.f, be);
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = active ? cv * V + e : 0;
     mu[e] = mean[n * G + c / cg];
     rs[e] = rstd[n * G + c / cg];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
   }
   float acc[2 * V];
 #pragma unroll
@@ -766,14 +839,14 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   __syncthreads();
   if (r < rpp) {
   float mu[V], rs[V], ga[V], be[V], ca[V], cb[V];
+  load_params<V>(gamma, param_dtype, cv * V, 1.f, ga);
+  load_params<V>(beta, param_dtype, cv * V, 0.f, be);
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const int c = cv * V + e;
     const int g = c / cg;
     mu[e] = mean[n * G + g];
     rs[e] = rstd[n * G + g];
-    ga[e] = load_param(gamma, param_dtype, c, 1.f);
-    be[e] = load_param(beta, param_dtype, c, 0.f);
     ca[e] = gco[G + g];
     cb[e] = gco[g];
   }
