@@ -621,7 +621,8 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
                                                          int64_t S, int C, int G, int tpr, int rpp, int nsplit,
                                                          int64_t rows_per_split, int relu) {
   constexpr int V = VecOf<T>::N;
-  extern __shared__ float smem[];  // 2 * V * kBlock
+  extern __shared__ float smem[];  // 2 * V * kBlock | gamma[C]
+  float* gam = smem + 2 * V * kBlock;
   const int tid = threadIdx.x;
   const int n = blockIdx.y, split = blockIdx.x;
   const int cg = C / G;
@@ -703,6 +704,10 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
       row = next;
     }
   }
+  if (tid < tpr) {  // the first row's threads hold every channel's gamma: the per-group fold below reads it from LDS
+#pragma unroll
+    for (int e = 0; e < V; ++e) gam[cv * V + e] = ga[e];
+  }
   block_row_reduce<2 * V>(acc, smem, tpr, rpp, active);
   float* dst = part + ((int64_t)n * nsplit + split) * 2 * C;
   for (int i = tid; i < 2 * C; i += kBlock) {
@@ -717,7 +722,7 @@ __global__ void __launch_bounds__(kBlock) gn_bwd_partial(const T* __restrict__ x
     float t = 0.f;
     for (int cc = tid & 15; cc < cg; cc += 16) {
       const int c = g * cg + cc;
-      t = fmaf(load_param(gamma, param_dtype, c, 1.f), smem[(q * V + c % V) * kBlock + c / V], t);
+      t = fmaf(gam[c], smem[(q * V + c % V) * kBlock + c / V], t);
     }
 #pragma unroll
     for (int off = 8; off > 0; off >>= 1) t += __shfl_down(t, off, 16);
@@ -732,6 +737,20 @@ __device__ __forceinline__ float block_sum256(float v, float* red4) {
   if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = v;
   __syncthreads();
   return (red4[0] + red4[1]) + (red4[2] + red4[3]);
+}
+
+// Two sums at once (the same trees, one pair of barriers).
+__device__ __forceinline__ void block_sum256_pair(float& a, float& b, float* red8) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) {
+    red8[threadIdx.x >> 6] = a;
+    red8[4 + (threadIdx.x >> 6)] = b;
+  }
+  __syncthreads();
+  a = (red8[0] + red8[1]) + (red8[2] + red8[3]);
+  b = (red8[4] + red8[5]) + (red8[6] + red8[7]);
 }
 
 // Workgroups [0, N*G): coef[n][g] = (A, B) with A = mean(dy'*gamma), B = mean(dy'*gamma*xhat)
@@ -807,7 +826,7 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
                                                 int nsplit, int64_t rows_per_split, float m, int relu) {
   constexpr int V = VecOf<T>::N;
   extern __shared__ float gco[];  // sums[2 G] | fold scratch (4 * kBlock)
-  __shared__ float red4[4];
+  __shared__ float red8[8];
   const int tid = threadIdx.x;
   const int n = blockIdx.y;
   const int cg = C / G;
@@ -827,6 +846,22 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
   fetch_rows<T, V, U>(cx, xs, row, step, end, begin, C, r < rpp);
   fetch_rows<TG, V, U>(cg_, gs, row, step, end, begin, C, r < rpp);
   const bool fused = fold_in_consumer(G, nsplit);
+  // The workgroup's share of the parameter gradients (the tail of this kernel) reads the per-channel partials of the
+  // launch before: its first loads go out now, so that the tail does not start with a trip to memory of its own.
+  const bool param_sums = fused && n == 0 && (dgamma != nullptr || dbeta != nullptr);
+  const int total = N * nsplit;
+  const int grp = tid >> 5, li = tid & 31;
+  const bool one_channel = C <= (int)gridDim.x;  // at most one channel per workgroup: all 256 threads on it
+  float pre1 = 0.f, pre2 = 0.f;
+  if (param_sums) {
+    const int c = one_channel ? (int)blockIdx.x : (int)blockIdx.x + grp * (int)gridDim.x;
+    const int i = one_channel ? tid : li;
+    if (c < C && i < total) {
+      const float* p = part + (int64_t)i * 2 * C;
+      pre1 = p[c];
+      pre2 = p[C + c];
+    }
+  }
   if (fused) {
     // gpart quantity 0 = sum dy'*gamma*xhat (-> B), quantity 1 = sum dy'*gamma (-> A)
     fold_split_partials(gpart + (int64_t)n * nsplit * 2 * G, G, nsplit, gco + 2 * G, [&](int c, float t) { gco[c] = t / m; });
@@ -885,23 +920,22 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
     row = next;
   }
   }
-  if (fused && n == 0 && (dgamma != nullptr || dbeta != nullptr)) {
+  if (param_sums) {
     // More channels than workgroups (the deepest levels): eight at a time, one per group of 32 lanes (workgroup b takes
     // channels b, b + gridDim.x, ...): each lane
     // adds every 32nd split partial of its channel, the 32 lanes meet in a butterfly; no LDS and no barrier. (One channel
     // at a time over all 256 threads cost the deepest level, 512 channels over 64 workgroups, 6 us of serial rounds.)
-    const int total = N * nsplit;
-    const int grp = tid >> 5, li = tid & 31;
-    if (C <= (int)gridDim.x) {  // at most one channel per workgroup: all 256 threads on it
+    // The first partial of every thread's first channel is in pre1 / pre2 already.
+    if (one_channel) {
       for (int c = blockIdx.x; c < C; c += gridDim.x) {
-        float s1 = 0.f, s2 = 0.f;
-        for (int i = tid; i < total; i += kBlock) {
+        const bool first = c == (int)blockIdx.x;
+        float s1 = first ? pre1 : 0.f, s2 = first ? pre2 : 0.f;
+        for (int i = first ? tid + kBlock : tid; i < total; i += kBlock) {
           const float* p = part + (int64_t)i * 2 * C;
           s1 += p[c];
           s2 += p[C + c];
         }
-        s1 = block_sum256(s1, red4);
-        s2 = block_sum256(s2, red4);
+        block_sum256_pair(s1, s2, red8);
         if (tid == 0) {
           if (dgamma != nullptr) dgamma[c] = s1;
           if (dbeta != nullptr) dbeta[c] = s2;
@@ -910,9 +944,10 @@ __global__ void __launch_bounds__(kBlock) gn_dx(const T* __restrict__ x, const T
     } else
     for (int c0 = blockIdx.x; c0 < C; c0 += 8 * gridDim.x) {  // c0: the channel of group 0, uniform over the workgroup
       const int c = c0 + grp * gridDim.x;
-      float s1 = 0.f, s2 = 0.f;
+      const bool first = c0 == (int)blockIdx.x;
+      float s1 = first ? pre1 : 0.f, s2 = first ? pre2 : 0.f;
       if (c < C) {
-        for (int i = li; i < total; i += 32) {
+        for (int i = first ? li + 32 : li; i < total; i += 32) {
           const float* p = part + (int64_t)i * 2 * C;
           s1 += p[c];
           s2 += p[C + c];
@@ -1166,7 +1201,7 @@ int bwd_typed(const sfh_groupnorm_desc& p, const GnPlan& pl, int param_dtype, co
   }
   constexpr int V = VecOf<T>::N;
   const dim3 grid(pl.nsplit, p.n);
-  hipLaunchKernelGGL((gn_bwd_partial<T, TG>), grid, dim3(kBlock), (size_t)2 * V * kBlock * sizeof(float), st, (const T*)x,
+  hipLaunchKernelGGL((gn_bwd_partial<T, TG>), grid, dim3(kBlock), ((size_t)2 * V * kBlock + C) * sizeof(float), st, (const T*)x,
                      (const TG*)dy, mean, rstd, gamma, beta, param_dtype, part, gpart, S, C, G, pl.tpr, pl.rpp, pl.nsplit,
                      pl.rows_per_split, p.relu);
   if (int rc = check_launch("gn_bwd_partial")) return rc;
