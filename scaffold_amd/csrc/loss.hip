@@ -133,6 +133,22 @@ __global__ void __launch_bounds__(kBlock) ce_dice_partial(const T* __restrict__ 
   }
 }
 
+// Slots lane, lane + 64, ... of a quantity (stride `q` floats between slots), added in that order with sixteen loads in
+// flight at a time (one slot per trip to memory made a launch of 1024 slots sixteen trips long).
+__device__ __forceinline__ float lane_slots_sum(const float* __restrict__ src, int slots, int q, int lane) {
+  float s = 0.f;
+  int sp = lane;
+  for (; sp + 15 * 64 < slots; sp += 16 * 64) {
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) v[k] = src[(int64_t)(sp + 64 * k) * q];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) s += v[k];
+  }
+  for (; sp < slots; sp += 64) s += src[(int64_t)sp * q];
+  return s;
+}
+
 // One 64-lane workgroup per quantity: lane l adds slots l, l + 64, ... and the lane totals meet in a fixed tree.
 // stats: inter[N][C] | psum[N][C] | tsum[N][C] | ce_sum | normaliser
 __global__ void __launch_bounds__(64) ce_dice_sum(const float* __restrict__ part, float* __restrict__ stats, int N, int C, int nsplit,
@@ -143,12 +159,11 @@ __global__ void __launch_bounds__(64) ce_dice_sum(const float* __restrict__ part
   int dst;
   if (b < N * 3 * C) {
     const int n = b / (3 * C), q = b - n * 3 * C;
-    const float* src = part + (int64_t)n * nsplit * Q + q;
-    for (int sp = lane; sp < nsplit; sp += 64) s += src[(int64_t)sp * Q];
+    s = lane_slots_sum(part + (int64_t)n * nsplit * Q + q, nsplit, Q, lane);
     dst = (q / C) * N * C + n * C + q % C;
   } else {
     const int q = 3 * C + (b - N * 3 * C);  // ce_sum or normaliser, over all samples
-    for (int i = lane; i < N * nsplit; i += 64) s += part[(int64_t)i * Q + q];
+    s = lane_slots_sum(part + q, N * nsplit, Q, lane);
     dst = b;
   }
   s = wave_sum_all(s);
@@ -163,6 +178,8 @@ __global__ void __launch_bounds__(64) ce_dice_scalar(const float* __restrict__ s
   const float* inter = stats;
   const float* psum = stats + N * C;
   const float* tsum = stats + 2 * N * C;
+  // (asked for now: thread 0 needs them after the tree)
+  const float ce_sum = stats[N * 3 * C], normaliser = stats[N * 3 * C + 1];
   float dice = 0.f;
   for (int i = threadIdx.x; i < N * C; i += 64) {
     const int c = i % C;
@@ -176,7 +193,7 @@ __global__ void __launch_bounds__(64) ce_dice_scalar(const float* __restrict__ s
   dice = wave_sum_all(dice);
   if (threadIdx.x == 0) {
     dice /= (float)(N * (C - 1));
-    const float ce = stats[N * 3 * C] / fmaxf(stats[N * 3 * C + 1], 1.1920929e-07f);
+    const float ce = ce_sum / fmaxf(normaliser, 1.1920929e-07f);
     loss[0] = ce + (1.f - dice);
   }
 }
