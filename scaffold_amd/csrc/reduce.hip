@@ -151,7 +151,30 @@ __global__ void __launch_bounds__(kBlock) sum_slices_bias_kernel(const float* __
   const int64_t e = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4;
   if (e >= nelem) return;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int sp = 0; sp < splits; ++sp) {
+  // the slices in their order, eight, four or two loads in flight (one slice per trip to memory made the sum of eight
+  // slices eight trips long)
+  int sp = 0;
+  for (; sp + 7 < splits; sp += 8) {
+    float4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const float4*>(part + (int64_t)(sp + k) * nelem + e);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+  }
+  for (; sp + 3 < splits; sp += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const float4*>(part + (int64_t)(sp + k) * nelem + e);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+  }
+  for (; sp + 1 < splits; sp += 2) {
+    const float4 v0 = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
+    const float4 v1 = *reinterpret_cast<const float4*>(part + (int64_t)(sp + 1) * nelem + e);
+    s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
+    s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
+  }
+  for (; sp < splits; ++sp) {
     const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem + e);
     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
   }
