@@ -251,6 +251,35 @@ int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* x_fir
                           int32_t cin_first, const void* gy, void* gw, void* workspace, size_t workspace_bytes,
                           uint32_t flags, void* stream);
 
+/* ---- several conv3d weight gradients in one launch ------------------------------------------
+ * The weight gradients of a training step (triton_conv3d.conv3d_backward_weight once per convolution,
+ * triton_conv3d/reduce_gemm.py:1177; nothing reads them before the optimizer, ScaFFold/utils/trainer.py:678-694) as ONE
+ * launch of the weight-gradient kernel and ONE sum pass: what a launch of sfh_conv3d_wgrad costs whatever the problem --
+ * all workgroups fetching their first operands at once, all writing their partial slice at once, the sum pass reading the
+ * slices back, two launch gaps: 15-20 us on MI355X -- is paid once for up to SFH_WGRAD_BATCH_MAX problems. The work of
+ * all problems is laid on one line and cut evenly over the workgroups; a workgroup that covers parts of several
+ * 32 x 32 channel blocks writes a slice for each. Each item is one sfh_conv3d_wgrad (x_second NULL) or
+ * sfh_conv3d_wgrad_pair call; all share `dtype` and the gradient dtype (SFH_FLAG_GRAD_FP32). Results: every gradient is
+ * the sum of fp32 partials in a fixed order that is a pure function of the LIST of problems (their shapes, in order) --
+ * the same bits on every run, and within fp32 summation-order rounding of sfh_conv3d_wgrad's (whose cuts differ).
+ * Served: the problems sfh_conv3d_wgrad_batch_supported answers 1 for -- 3 x 3 x 3, unit stride and dilation, SFH_BF16 /
+ * SFH_FP16, channel counts multiples of 32, output rows of more than 16 voxels; anything else in the list fails the
+ * call with SFH_ERR_UNSUPPORTED before any launch (the caller runs those through sfh_conv3d_wgrad).
+ * The batching itself has no counterpart in the reference. */
+#define SFH_WGRAD_BATCH_MAX 16
+typedef struct sfh_conv3d_wgrad_item {
+  sfh_conv3d_desc desc;
+  const void* x;        /* the input, or its first cin_first channels when x_second is given */
+  const void* x_second; /* NULL: one tensor */
+  int32_t cin_first;
+  const void* gy;
+  void* gw;             /* [Cout][3][3][3][Cin] dense */
+} sfh_conv3d_wgrad_item;
+int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dtype);
+size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype); /* pointers unused; 0: refused */
+int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, void* workspace,
+                           size_t workspace_bytes, uint32_t flags, void* stream);
+
 /* Weight gradient and bias gradient from one pass over gy, where the kernel that serves the problem reads gy tile by tile
  * anyway: the 1x1x1 convolutions with at most 32 output channels over 32 / 64 / 128 input channels (the U-Net's head),
  * 16-bit dtypes. gb: Cout elements in gw's dtype (the operands', or fp32 with SFH_FLAG_GRAD_FP32) =

@@ -65,6 +65,11 @@ class PackItem(ctypes.Structure):
                 ("packed_dgrad", c_void_p)]
 
 
+class WgradItem(ctypes.Structure):
+    _fields_ = [("desc", ConvDesc), ("x", c_void_p), ("x_second", c_void_p), ("cin_first", c_int32), ("gy", c_void_p),
+                ("gw", c_void_p)]
+
+
 class ConvTDesc(ctypes.Structure):
     _fields_ = [(k, c_int32) for k in ("n", "cin", "in_d", "in_h", "in_w", "cout", "kd", "kh", "kw")]
 
@@ -132,6 +137,9 @@ _SIGNATURES = {
                                     c_void_p, c_void_p, c_size_t, c_uint32, c_int, c_void_p, c_size_t, c_void_p]),
     "sfh_conv3d_dgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_int32,
                                       c_void_p, c_size_t, c_uint32, c_void_p]),
+    "sfh_conv3d_wgrad_batch_supported": (c_int, [POINTER(ConvDesc), c_int]),
+    "sfh_conv3d_wgrad_batch_workspace_bytes": (c_size_t, [POINTER(WgradItem), c_int32, c_int]),
+    "sfh_conv3d_wgrad_batch": (c_int, [POINTER(WgradItem), c_int32, c_int, c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_wgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,
                                       c_uint32, c_void_p]),
     "sfh_convT3d_fwd_workspace_bytes": (c_size_t, [POINTER(ConvTDesc), c_int]),

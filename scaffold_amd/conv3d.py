@@ -837,6 +837,85 @@ def conv3d_backward_weight(
     return gw
 
 
+WGRAD_BATCH_MAX = 16  # SFH_WGRAD_BATCH_MAX
+
+
+def weight_grad_batchable(input_shape, weight_shape, stride, padding, dilation, dtype) -> bool:
+    """Whether :func:`conv3d_backward_weight_batch` takes this problem (3x3x3, unit stride and dilation, bf16 / fp16,
+    channel counts multiples of 32, output rows of more than 16 voxels): a pure function of the problem."""
+    if dtype not in (torch.bfloat16, torch.float16):
+        return False
+    try:
+        prob = _problem(torch.Size(input_shape), torch.Size(weight_shape), stride, padding, dilation, dtype)
+    except (ValueError, NotImplementedError):
+        return False
+    if prob.n == 0:
+        return False
+    return bool(_lib.lib().sfh_conv3d_wgrad_batch_supported(ctypes.byref(prob.desc), prob.code))
+
+
+def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] = None, outs=None):
+    """The weight gradients of several convolutions from one launch of the weight-gradient kernel and one sum pass.
+
+    ``problems``: a sequence of ``(input, weight_shape, grad_output, padding)`` or ``((first, second), weight_shape,
+    grad_output, padding)`` -- the arguments of :func:`conv3d_backward_weight` / :func:`conv3d_backward_weight_pair` at unit
+    stride and dilation -- every one of them a problem :func:`weight_grad_batchable` accepts, all of one dtype and device.
+    What a single launch costs whatever the problem (first fetch, slices written and read back, launch gaps: 15-20 us on
+    MI355X) is paid once for the list.  Returns the gradients (``channels_last_3d``, ``grad_dtype`` or the operands' dtype)
+    in order; ``outs`` supplies the tensors to write.  Each gradient is a fixed-order fp32 sum that depends on the LIST of
+    shapes only: the same bits on every run, within summation-order rounding of the one-problem call's."""
+    problems = list(problems)
+    if not problems:
+        return []
+    L = _lib.lib()
+    keep, gws = [], []
+    dev = dt = None
+    for i, (inp, wshape, gy, padding) in enumerate(problems):
+        first, second = inp if isinstance(inp, (tuple, list)) else (inp, None)
+        x = first.contiguous(memory_format=_CL3D)
+        x2 = None if second is None else second.contiguous(memory_format=_CL3D)
+        g = gy.contiguous(memory_format=_CL3D)
+        if dev is None:
+            dev, dt = x.device, x.dtype
+        if x.device != dev or x.dtype is not dt or g.dtype is not dt or g.device != dev or (x2 is not None and (x2.dtype is not dt or x2.device != dev)):
+            raise ValueError("conv3d_backward_weight_batch: all operands share one dtype and one device")
+        in_shape = x.shape if x2 is None else _pair_shape(x, x2)
+        wshape = wshape if isinstance(wshape, torch.Size) else torch.Size(wshape)
+        prob = _problem(in_shape, wshape, 1, padding, 1, dt)
+        if tuple(g.shape) != tuple(prob.y_shape):
+            raise ValueError(f"conv3d_backward_weight_batch: problem {i}: grad_output {tuple(g.shape)} does not match {tuple(prob.y_shape)}")
+        gdt = dt if grad_dtype is None else grad_dtype
+        if gdt is not dt and gdt is not torch.float32:
+            raise ValueError(f"grad_dtype must be the operands' dtype or torch.float32, got {grad_dtype}")
+        if outs is None:
+            gw = torch.empty((prob.cout, prob.cin, *prob.k), dtype=gdt, device=dev, memory_format=_CL3D)
+        else:
+            gw = outs[i]
+            why = _validate_gw_out(gw, prob.cout, prob.cin, tuple(prob.k), gdt, dev)
+            if why is not None:
+                raise ValueError(f"outs[{i}] is not usable for this problem: {why}")
+        keep.append((prob, x, x2, g))
+        gws.append(gw)
+    flags = _lib.SFH_FLAG_GRAD_FP32 if (grad_dtype is not None and grad_dtype is not dt) else 0
+    with _lib.device_guard(dev):
+        for lo in range(0, len(keep), WGRAD_BATCH_MAX):
+            part = keep[lo:lo + WGRAD_BATCH_MAX]
+            items = (_lib.WgradItem * len(part))()
+            for it, (prob, x, x2, g), gw in zip(items, part, gws[lo:]):
+                it.desc = prob.desc
+                it.x, it.x_second, it.cin_first = _lib.ptr(x), (None if x2 is None else _lib.ptr(x2)), (0 if x2 is None else int(x.shape[1]))
+                it.gy, it.gw = _lib.ptr(g), _lib.ptr(gw)
+            code = part[0][0].code
+            need = int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, len(part), code))
+            if need == 0:
+                raise NotImplementedError("conv3d_backward_weight_batch: a problem of the list is not served in a batch "
+                                          "(weight_grad_batchable says which)")
+            ws = _lib.workspace(need, dev)
+            _lib.check(L.sfh_conv3d_wgrad_batch(items, len(part), code, _lib.ptr(ws), need, flags, _lib.stream_ptr(dev)),
+                       "conv3d_backward_weight_batch")
+    return gws
+
+
 def conv3d_backward_weight_bias(input: torch.Tensor, weight_shape: Sequence[int], grad_output: torch.Tensor, stride=1, padding=0,
                                 dilation=1, groups: int = 1, *, grad_dtype: Optional[torch.dtype] = None, _checked: bool = False):
     """``(grad_weight, grad_bias)`` from ONE pass over ``grad_output`` where the kernel that serves the problem reads it tile

@@ -756,6 +756,49 @@ extern "C" int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const 
   return conv3d_wgrad_any(p, dtype, x_first, gy, gw, workspace, workspace_bytes, flags, stream, &x2);
 }
 
+// ---- several weight gradients in one launch ----------------------------------------------
+static_assert(kWgradBatchMax == SFH_WGRAD_BATCH_MAX, "the header's limit is the kernel table's");
+static int wgrad_batch_items(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, WgradBatchItem* out_items) {
+  if (items == nullptr || count < 1) return fail(SFH_ERR_INVALID, "conv3d wgrad batch: no problems");
+  if (count > SFH_WGRAD_BATCH_MAX) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: at most %d problems a call", SFH_WGRAD_BATCH_MAX);
+  for (int32_t i = 0; i < count; ++i) {
+    int32_t out[3];
+    if (int rc = check_conv(&items[i].desc, dtype, out)) return rc;
+    const sfh_conv3d_desc& d = items[i].desc;
+    if (!wgrad_uses_mfma(d, dtype, out) || !mfma_wgrad_batch_applies(wgrad_args(d, out), dtype))
+      return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: problem %d is not a 3x3x3 unit-stride 16-bit problem with rows of more than 16 voxels", (int)i);
+    WgradBatchItem& o = out_items[i];
+    o.a = wgrad_args(d, out);
+    o.x = items[i].x; o.x1 = items[i].x_second; o.c_first = items[i].cin_first; o.gy = items[i].gy; o.gw = items[i].gw;
+    if (o.x1 != nullptr && !mfma_wgrad_pair_ok(o.a, o.c_first))
+      return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: problem %d cannot be cut at channel %d", (int)i, (int)o.c_first);
+  }
+  return SFH_OK;
+}
+
+extern "C" int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dtype) {
+  int32_t out[3];
+  if (p == nullptr || sfh_conv3d_out_shape(p, out) != SFH_OK || !dtype_ok(dtype)) return 0;
+  return (wgrad_uses_mfma(*p, dtype, out) && mfma_wgrad_batch_applies(wgrad_args(*p, out), dtype)) ? 1 : 0;
+}
+
+extern "C" size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype) {
+  WgradBatchItem list[SFH_WGRAD_BATCH_MAX];
+  if (wgrad_batch_items(items, count, dtype, list) != SFH_OK) return 0;
+  return mfma_wgrad_batch_workspace_bytes(list, count);
+}
+
+extern "C" int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, void* workspace, size_t workspace_bytes,
+                                      uint32_t flags, void* stream) {
+  WgradBatchItem list[SFH_WGRAD_BATCH_MAX];
+  if (int rc = wgrad_batch_items(items, count, dtype, list)) return rc;
+  for (int32_t i = 0; i < count; ++i)
+    if (list[i].x == nullptr || list[i].gy == nullptr || list[i].gw == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad batch: null tensor");
+  if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d wgrad batch: the direct kernels take one problem a call");
+  const int gw_dtype = (flags & SFH_FLAG_GRAD_FP32) ? SFH_FP32 : dtype;
+  return mfma_wgrad_batch(list, count, dtype, gw_dtype, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
 // ---- bias gradient ---------------------------------------------------------------------
 extern "C" size_t sfh_bias_grad_workspace_bytes(int64_t rows, int32_t channels) {
   if (rows < 1 || channels < 1) return 0;

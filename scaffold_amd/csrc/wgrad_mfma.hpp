@@ -28,4 +28,22 @@ bool mfma_wgrad_ring_applies(const WgradArgs& a);
 int mfma_wgrad_ring_splits(const WgradArgs& a);
 int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2);
 
+// Several ring-served weight gradients in one launch and one sum pass (wgrad_ring.hip): the cost every launch pays
+// once -- the first fetch of all workgroups, the slices written and read back, two launch gaps -- is paid once for the
+// batch. All problems share dtype and the gradient's dtype; how the work is cut over the workgroups is a pure function
+// of the list of problems, every sum has a fixed order (not that of the one-problem launch: the cuts differ).
+constexpr int kWgradBatchMax = 16;
+struct WgradBatchItem {
+  WgradArgs a;
+  const void* x;
+  const void* x1;  // with c_first: the input as two tensors (mfma_wgrad_pair_ok), or null
+  int c_first;
+  const void* gy;
+  void* gw;
+};
+bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype);
+size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count);  // 0: the list cannot share a launch
+int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
+                     hipStream_t st);
+
 }  // namespace sfh

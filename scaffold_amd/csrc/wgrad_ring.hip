@@ -181,11 +181,11 @@ struct WRingLane {
 
 struct WRingColumn { int n, h0, w0; };
 
-__device__ __forceinline__ WRingColumn wring_column(int col, const WRingGeom& gm) {
+__device__ __forceinline__ WRingColumn wring_column(int col, int tiles_h, int tiles_w) {
   WRingColumn c;
-  c.w0 = (col % gm.tiles_w) * kTW; col /= gm.tiles_w;
-  c.h0 = (col % gm.tiles_h) * kTH;
-  c.n = col / gm.tiles_h;
+  c.w0 = (col % tiles_w) * kTW; col /= tiles_w;
+  c.h0 = (col % tiles_h) * kTH;
+  c.n = col / tiles_h;
   return c;
 }
 
@@ -328,15 +328,11 @@ struct WRingStep {
   }
 };
 
-template <typename T, int G>
-__device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws,
-                                          const WRingGeom& gm, int split, int cib, int cob, int x_cin, int tid, char* xp0, char* xp1,
-                                          char* xp2, char* gt0, char* gt1, char* gt2) {
-  constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+// The per-lane constants of a problem: where the lane's voxels of a staged pair / tile lie in memory and in LDS.
+__device__ __forceinline__ WRingLane wring_lane(const WgradArgs& a, int x_cin, int tid) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int seg16 = wave & 1;  // which 16 voxels of every row this wavefront contracts over
-
   WRingLane ln;
 #pragma unroll
   for (int k = 0; k < kXGroupsPerWave; ++k) {
@@ -360,78 +356,83 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
     ln.xread = piece * kXPiece + vox * 16 + (m & 1) * 8;
     ln.gread = piece * kGPiece + vox * 16 + (m & 1) * 8;
   }
+  return ln;
+}
 
-  f32x16_t acc[NACC];
-#pragma unroll
-  for (int t = 0; t < NACC; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
-  uint4 gyf[kTD * kTH];            // gy fragments of the step's eight output rows (this wavefront's 16 voxels of each)
-  uint4 fr[WSchedule::kBuffers];   // input-row fragments in rotation
+// The LDS of a workgroup: a ring of three input plane pairs and three gy tiles.
+struct WRingLds {
+  char *xp0, *xp1, *xp2, *gt0, *gt1, *gt2;
+};
 
-  const int item_begin = split * gm.items_per_split;
-  int item_end = item_begin + gm.items_per_split;
-  if (item_end > gm.items) item_end = gm.items;
-  const int ncols = gm.items / gm.segs;
+// Steps s_begin .. s_begin + nsteps - 1 of column `col` of the 32 x 32 block (cob, cib), added to acc. `x` is the tensor
+// that holds the block's input channels, moved so that the block's index in the whole input addresses them; x_cin its
+// channel count.
+template <typename T, int G>
+__device__ __forceinline__ void wring_segment(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ gy, const WRingColumn& col,
+                                              int s_begin, int nsteps, int cib, int cob, int x_cin, const WRingLane& ln, int wave,
+                                              f32x16_t (&acc)[G == 0 ? kTaps0 : kTaps1], uint4 (&gyf)[kTD * kTH],
+                                              uint4 (&fr)[WSchedule::kBuffers], const WRingLds& m) {
   int xoff[kXGroupsPerWave];
   int goff;
-  for (int item = item_begin; item < item_end; ++item) {
-    const int seg = item / ncols;
-    const WRingColumn col = wring_column(item - seg * ncols, gm);
-    const int s_begin = seg * gm.seg_steps;
-    int s_end = s_begin + gm.seg_steps;
-    if (s_end > gm.steps) s_end = gm.steps;
-    const int nsteps = s_end - s_begin;
-    if (nsteps <= 0) continue;
-    const int plane0 = kTD * s_begin - a.pd;
-    auto xorigin = [&](int plane) {
-      return x + ((((int64_t)col.n * a.id + plane) * a.ih + (col.h0 - a.ph)) * a.iw + (col.w0 - a.pw)) * x_cin + cib * 32;
-    };
-    auto gorigin = [&](int d0) { return gy + ((((int64_t)col.n * a.od + d0) * a.oh + col.h0) * a.ow + col.w0) * a.cout + cob * 32; };
+  const int plane0 = kTD * s_begin - a.pd;
+  auto xorigin = [&](int plane) {
+    return x + ((((int64_t)col.n * a.id + plane) * a.ih + (col.h0 - a.ph)) * a.iw + (col.w0 - a.pw)) * x_cin + cib * 32;
+  };
+  auto gorigin = [&](int d0) { return gy + ((((int64_t)col.n * a.od + d0) * a.oh + col.h0) * a.ow + col.w0) * a.cout + cob * 32; };
 
-    // the first step's two pairs, and the gy tiles of the first two steps (gy runs two steps ahead of the MFMAs)
-    wring_offsets(a, col, ln, plane0, kTD * s_begin, true, xoff, goff);
-    wring_fetch<T>(xp0, gt0, wave, xorigin(plane0), gorigin(kTD * s_begin), xoff, goff);
-    wring_offsets(a, col, ln, plane0 + 2, kTD * (s_begin + 1), true, xoff, goff);
-    if (nsteps < 2) goff = kRange;
-    wring_fetch<T>(xp1, gt1, wave, xorigin(plane0 + 2), gorigin(kTD * (s_begin + 1)), xoff, goff);
-    __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));
-    __builtin_amdgcn_s_barrier();
-    {
-      WRingFrags<G> first{xp0 + ln.xread, nullptr, gt0 + ln.gread, gyf, fr};
-      first.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
-    }
-
-    // step i: MFMAs over pairs (lo, hi) and tile gt; the pair after them streams into xfill, the gy tile of step i + 2
-    // into gfill; gt_next is the (resident) tile of step i + 1
-    auto step = [&](int i, const char* lo, const char* hi, const char* gt, char* xfill, char* gfill, const char* gt_next) {
-      const int plane = plane0 + 2 * i + 4, d_ahead = kTD * (s_begin + i + 2);
-      wring_offsets(a, col, ln, plane, d_ahead, i + 1 < nsteps, xoff, goff);
-      if (i + 2 >= nsteps) goff = kRange;
-      WRingStep<T, G> st{WRingFrags<G>{lo + ln.xread, hi + ln.xread, gt + ln.gread, gyf, fr}, xfill, gfill, wave, acc, xoff, goff,
-                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xorigin(plane)), 0, kRange, 0x00020000),
-                         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin(d_ahead)), 0, kRange, 0x00020000)};
-      st.run(std::make_integer_sequence<int, WSchedule::kMaxMfmas>{});
-      if (i + 1 < nsteps) {  // the next step's first fragments: its first pair is this step's second one
-        WRingFrags<G> next{hi + ln.xread, nullptr, gt_next + ln.gread, gyf, fr};
-        next.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
-      }
-      __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));  // this wavefront's part of the next pair and tile has landed
-      __builtin_amdgcn_s_barrier();                     // ... and every wavefront is done reading this step's
-    };
-    for (int i = 0; i < nsteps; i += 3) {
-      step(i, xp0, xp1, gt0, xp2, gt2, gt1);
-      if (i + 1 < nsteps) step(i + 1, xp1, xp2, gt1, xp0, gt0, gt2);
-      if (i + 2 < nsteps) step(i + 2, xp2, xp0, gt2, xp1, gt1, gt0);
-    }
+  // the first step's two pairs, and the gy tiles of the first two steps (gy runs two steps ahead of the MFMAs)
+  wring_offsets(a, col, ln, plane0, kTD * s_begin, true, xoff, goff);
+  wring_fetch<T>(m.xp0, m.gt0, wave, xorigin(plane0), gorigin(kTD * s_begin), xoff, goff);
+  wring_offsets(a, col, ln, plane0 + 2, kTD * (s_begin + 1), true, xoff, goff);
+  if (nsteps < 2) goff = kRange;
+  wring_fetch<T>(m.xp1, m.gt1, wave, xorigin(plane0 + 2), gorigin(kTD * (s_begin + 1)), xoff, goff);
+  __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));
+  __builtin_amdgcn_s_barrier();
+  {
+    WRingFrags<G> first{m.xp0 + ln.xread, nullptr, m.gt0 + ln.gread, gyf, fr};
+    first.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
   }
 
-  // The wavefronts (0, G) and (1, G) hold sums over different voxels for the same taps: the second hands its
-  // accumulators over through LDS (the last barrier has freed it), kHandTaps taps at a time through the group's own
-  // array, the first adds them -- a fixed order -- and writes the workgroup's slice.
-  char* handover = G == 0 ? xp0 : xp1;
-  float* dst = ws + ((int64_t)split * a.cout + cob * 32) * 27 * a.cin + cib * 32;
-  const int j = lane & 31, kg = lane >> 5;
+  // step i: MFMAs over pairs (lo, hi) and tile gt; the pair after them streams into xfill, the gy tile of step i + 2
+  // into gfill; gt_next is the (resident) tile of step i + 1
+  auto step = [&](int i, const char* lo, const char* hi, const char* gt, char* xfill, char* gfill, const char* gt_next) {
+    const int plane = plane0 + 2 * i + 4, d_ahead = kTD * (s_begin + i + 2);
+    wring_offsets(a, col, ln, plane, d_ahead, i + 1 < nsteps, xoff, goff);
+    if (i + 2 >= nsteps) goff = kRange;
+    WRingStep<T, G> st{WRingFrags<G>{lo + ln.xread, hi + ln.xread, gt + ln.gread, gyf, fr}, xfill, gfill, wave, acc, xoff, goff,
+                       __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(xorigin(plane)), 0, kRange, 0x00020000),
+                       __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(gorigin(d_ahead)), 0, kRange, 0x00020000)};
+    st.run(std::make_integer_sequence<int, WSchedule::kMaxMfmas>{});
+    if (i + 1 < nsteps) {  // the next step's first fragments: its first pair is this step's second one
+      WRingFrags<G> next{hi + ln.xread, nullptr, gt_next + ln.gread, gyf, fr};
+      next.early(std::make_integer_sequence<int, WSchedule::kMaxFrags>{}, std::make_integer_sequence<int, kTD * kTH>{});
+    }
+    __builtin_amdgcn_s_waitcnt(wring_waitcnt_vm(0));  // this wavefront's part of the next pair and tile has landed
+    __builtin_amdgcn_s_barrier();                     // ... and every wavefront is done reading this step's
+  };
+  for (int i = 0; i < nsteps; i += 3) {
+    step(i, m.xp0, m.xp1, m.gt0, m.xp2, m.gt2, m.gt1);
+    if (i + 1 < nsteps) step(i + 1, m.xp1, m.xp2, m.gt1, m.xp0, m.gt0, m.gt2);
+    if (i + 2 < nsteps) step(i + 2, m.xp2, m.xp0, m.gt2, m.xp1, m.gt1, m.gt0);
+  }
+}
+
+// The wavefronts (0, G) and (1, G) hold sums over different voxels for the same taps: the second hands its
+// accumulators over through LDS (the last barrier has freed it), kHandTaps taps at a time through the group's own
+// array, the first adds them -- a fixed order -- and writes the block's part of a slice: dst points at element
+// (co = first of the block, tap 0, ci = first of the block) of a [Cout][27][cin] slice.
+template <int G, bool IN_LOOP>
+__device__ __forceinline__ void wring_handover(const f32x16_t (&acc)[G == 0 ? kTaps0 : kTaps1], float* __restrict__ dst, int cin, int tid,
+                                               const WRingLds& m) {
+  constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  const int lane = tid & 63;
+  const int seg16 = __builtin_amdgcn_readfirstlane(tid >> 6) & 1;
+  char* handover = G == 0 ? m.xp0 : m.xp1;
+  const int j = lane & 31;
+  int kg = lane >> 5;
+  // (opaque to the optimiser where the call sits in a loop over blocks: it would otherwise compute all 224 store offsets
+  // ahead of the loop and keep them in scratch memory)
+  if constexpr (IN_LOOP) asm volatile("" : "+v"(kg));
 #pragma unroll
   for (int round = 0; round < kHandRounds; ++round) {
     if (seg16 == 1) {
@@ -461,7 +462,7 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int co = 8 * r4 + 4 * kg + e;
-              dst[((int64_t)co * 27 + tap) * a.cin + j] = v[e];
+              dst[((int64_t)co * 27 + tap) * cin + j] = v[e];
             }
           }
         }
@@ -469,6 +470,199 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
     __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
     __builtin_amdgcn_s_barrier();  // the array is free for the next round
   }
+}
+
+template <typename T, int G>
+__device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ gy, float* __restrict__ ws,
+                                          const WRingGeom& gm, int split, int cib, int cob, int x_cin, int tid, const WRingLds& m) {
+  constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const WRingLane ln = wring_lane(a, x_cin, tid);
+
+  f32x16_t acc[NACC];
+#pragma unroll
+  for (int t = 0; t < NACC; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  uint4 gyf[kTD * kTH];            // gy fragments of the step's eight output rows (this wavefront's 16 voxels of each)
+  uint4 fr[WSchedule::kBuffers];   // input-row fragments in rotation
+
+  const int item_begin = split * gm.items_per_split;
+  int item_end = item_begin + gm.items_per_split;
+  if (item_end > gm.items) item_end = gm.items;
+  const int ncols = gm.items / gm.segs;
+  for (int item = item_begin; item < item_end; ++item) {
+    const int seg = item / ncols;
+    const WRingColumn col = wring_column(item - seg * ncols, gm.tiles_h, gm.tiles_w);
+    const int s_begin = seg * gm.seg_steps;
+    int s_end = s_begin + gm.seg_steps;
+    if (s_end > gm.steps) s_end = gm.steps;
+    if (s_end <= s_begin) continue;
+    wring_segment<T, G>(a, x, gy, col, s_begin, s_end - s_begin, cib, cob, x_cin, ln, wave, acc, gyf, fr, m);
+  }
+  wring_handover<G, false>(acc, ws + ((int64_t)split * a.cout + cob * 32) * 27 * a.cin + cib * 32, a.cin, tid, m);
+}
+
+// ---- several weight gradients in one launch ------------------------------------------------------------------------------------
+// A launch of the kernel above costs the same whatever the problem: every workgroup fetches its first two steps at once
+// (all CUs asking together: 4.4 us), at the end every workgroup writes its 110 KB slice at once (6-7 us), a sum pass
+// reads the 256 slices back (6 us), and two launches start. A batch pays that once for all its problems. All blocks of
+// all problems lie on one line of cost -- problem after problem, inside a problem block after block, inside a block
+// column after column, a column being kFillCost positions for the ring's start and one per step -- and workgroup w of W
+// takes the positions [w total / W, (w + 1) total / W): whole columns, parts of columns, blocks of several problems. For
+// every block it touches it walks its steps of the block's columns, hands its accumulators over and writes a slice:
+// slice number w - (the first workgroup that touches the block). The sum pass knows from the same arithmetic how many
+// slices a block has. The cut is a pure function of the list of problems; nothing is added atomically.
+constexpr int kFillCost = 4;  // (the captured U-Net step: 2 -> 4 is 20 us faster, 4, 6 and 8 are alike)
+
+struct WRingBatchEntry {
+  WgradArgs a;
+  const void* x;
+  const void* x1;       // second tensor of the input (channels c_first ..), or null
+  const void* gy;
+  float* ws;            // this problem's slices: [slices][Cout][27][Cin]
+  void* gw;
+  int c_first;
+  int tiles_h, tiles_w, steps, nblk_ci, nblk;
+  int ncols;            // columns of a block
+  int pos_begin;        // the problem's first position on the line
+  int slices;           // the most slices any of its blocks gets
+  int quad_begin;       // the problem's first float4 in the sum pass (a multiple of 256)
+};
+
+struct WRingBatch {
+  int count, wgs, total, quads;
+  WRingBatchEntry e[kWgradBatchMax];
+};
+
+// (32-bit arithmetic: wring_batch_plan refuses a line of kBatchMaxTotal positions or more)
+constexpr int kBatchMaxTotal = 0x7fffff;
+__host__ __device__ __forceinline__ int batch_cut(int w, int total, int wgs) { return (int)((uint32_t)w * (uint32_t)total / (uint32_t)wgs); }
+// The workgroup whose range holds position q (total >= wgs: ranges are never empty).
+__host__ __device__ __forceinline__ int batch_owner(int q, int total, int wgs) {
+  int w = (int)((uint32_t)q * (uint32_t)wgs / (uint32_t)total);
+  if (batch_cut(w + 1, total, wgs) <= q) ++w;
+  return w;
+}
+
+template <typename T, int G>
+__device__ __forceinline__ void wring_batch_run(const WRingBatch& b, int w, int tid, const WRingLds& m) {
+  constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  f32x16_t acc[NACC];
+  uint4 gyf[kTD * kTH];
+  uint4 fr[WSchedule::kBuffers];
+  const int hi = batch_cut(w + 1, b.total, b.wgs);
+  int pos = batch_cut(w, b.total, b.wgs);
+  while (pos < hi) {
+    int p = 0;
+    for (int k = 1; k < b.count; ++k)
+      if (pos >= b.e[k].pos_begin) p = k;
+    const WgradArgs a = b.e[p].a;
+    const int steps = b.e[p].steps, nblk_ci = b.e[p].nblk_ci, tiles_h = b.e[p].tiles_h, tiles_w = b.e[p].tiles_w;
+    const int colcost = steps + kFillCost, blockcost = b.e[p].ncols * colcost;
+    const int blk = (pos - b.e[p].pos_begin) / blockcost;
+    const int b0 = b.e[p].pos_begin + blk * blockcost;
+    const int seg_hi = hi < b0 + blockcost ? hi : b0 + blockcost;
+    const int cib = blk % nblk_ci, cob = blk / nblk_ci;
+    const T* xs = (const T*)b.e[p].x;
+    int x_cin = a.cin, cis = cib;
+    if (b.e[p].x1 != nullptr) {
+      const int c_first = b.e[p].c_first;
+      const bool second = cib * 32 >= c_first;
+      xs = second ? (const T*)b.e[p].x1 : xs;
+      x_cin = second ? a.cin - c_first : c_first;
+      cis = second ? cib - c_first / 32 : cib;
+    }
+    const T* gy = (const T*)b.e[p].gy;
+    const WRingLane ln = wring_lane(a, x_cin, tid);
+#pragma unroll
+    for (int t = 0; t < NACC; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    for (int q = pos; q < seg_hi;) {
+      const int c = (q - b0) / colcost, first_step = b0 + c * colcost + kFillCost;  // the position of the column's step 0
+      int s_begin = q - first_step, s_end = seg_hi - first_step;
+      if (s_begin < 0) s_begin = 0;
+      if (s_end > steps) s_end = steps;
+      if (s_end > s_begin)
+        wring_segment<T, G>(a, xs + (cis - cib) * 32, gy, wring_column(c, tiles_h, tiles_w), s_begin, s_end - s_begin, cib, cob, x_cin, ln,
+                            wave, acc, gyf, fr, m);
+      q = first_step + steps;
+    }
+    const int slice = w - batch_owner(b0, b.total, b.wgs);
+    wring_handover<G, true>(acc, b.e[p].ws + ((int64_t)slice * a.cout + cob * 32) * 27 * a.cin + cib * 32, a.cin, tid, m);
+    pos = seg_hi;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256, 1) wgrad_ring_batch_kernel(WRingBatch b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char xp0[kXPair];
+  __shared__ __attribute__((aligned(16))) char xp1[kXPair];
+  __shared__ __attribute__((aligned(16))) char xp2[kXPair];
+  __shared__ __attribute__((aligned(16))) char gt0[kGTile];
+  __shared__ __attribute__((aligned(16))) char gt1[kGTile];
+  __shared__ __attribute__((aligned(16))) char gt2[kGTile];
+  const WRingLds m{xp0, xp1, xp2, gt0, gt1, gt2};
+  const int tid = threadIdx.x;
+  const int w = (int)xcd_remap(blockIdx.x, (uint32_t)b.wgs);
+  if (__builtin_amdgcn_readfirstlane(tid >> 6) < 2) wring_batch_run<T, 0>(b, w, tid, m);
+  else wring_batch_run<T, 1>(b, w, tid, m);
+#endif
+}
+
+// The sum over the slices of every block of every problem of a batch, in slice order (eight, four, two loads in
+// flight), one rounding to the gradient's dtype. A thread owns four consecutive input channels of one (co, tap).
+template <typename TOut>
+__global__ void __launch_bounds__(256) wgrad_ring_batch_sum(WRingBatch b) {
+  const int q0 = blockIdx.x * 256;  // a workgroup's 256 float4s lie in one problem (quad_begin is a multiple of 256)
+  int p = 0;
+  for (int k = 1; k < b.count; ++k)
+    if (q0 >= b.e[k].quad_begin) p = k;
+  const int q = q0 + threadIdx.x;
+  const int cin = b.e[p].a.cin, cout = b.e[p].a.cout;
+  const uint32_t nelem = (uint32_t)cout * 27u * (uint32_t)cin;  // below 2^31 (wring_batch_plan)
+  const uint32_t el = (uint32_t)(q - b.e[p].quad_begin) * 4u;
+  if (el >= nelem) return;
+  const int ci = (int)(el % (uint32_t)cin), co = (int)(el / (27u * (uint32_t)cin));
+  const int blk = (co / 32) * b.e[p].nblk_ci + ci / 32;
+  const int blockcost = b.e[p].ncols * (b.e[p].steps + kFillCost);
+  const int b0 = b.e[p].pos_begin + blk * blockcost;
+  const int n = batch_owner(b0 + blockcost - 1, b.total, b.wgs) - batch_owner(b0, b.total, b.wgs) + 1;
+  const float* part = b.e[p].ws + el;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  int sp = 0;
+  for (; sp + 7 < n; sp += 8) {
+    float4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const float4*>(part + (int64_t)(sp + k) * nelem);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+  }
+  for (; sp + 3 < n; sp += 4) {
+    float4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const float4*>(part + (int64_t)(sp + k) * nelem);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { s.x += v[k].x; s.y += v[k].y; s.z += v[k].z; s.w += v[k].w; }
+  }
+  for (; sp + 1 < n; sp += 2) {
+    const float4 v0 = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem);
+    const float4 v1 = *reinterpret_cast<const float4*>(part + (int64_t)(sp + 1) * nelem);
+    s.x += v0.x; s.y += v0.y; s.z += v0.z; s.w += v0.w;
+    s.x += v1.x; s.y += v1.y; s.z += v1.z; s.w += v1.w;
+  }
+  for (; sp < n; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  TOut* out = (TOut*)b.e[p].gw + el;
+  out[0] = elem<TOut>::from_float(s.x);
+  out[1] = elem<TOut>::from_float(s.y);
+  out[2] = elem<TOut>::from_float(s.z);
+  out[3] = elem<TOut>::from_float(s.w);
 }
 
 template <typename T>
@@ -482,6 +676,7 @@ wgrad_ring_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   __shared__ __attribute__((aligned(16))) char gt0[kGTile];
   __shared__ __attribute__((aligned(16))) char gt1[kGTile];
   __shared__ __attribute__((aligned(16))) char gt2[kGTile];
+  const WRingLds m{xp0, xp1, xp2, gt0, gt1, gt2};
   const int tid = threadIdx.x;
   const uint32_t wg = xcd_remap(blockIdx.x, total);
   const int blk = wg % gm.nblk, split = wg / gm.nblk;
@@ -504,9 +699,9 @@ wgrad_ring_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
   float* wsb = ws;
   if (wave < 2) {
     // (the slice is indexed with the whole tensor's cin and block index)
-    wring_run<T, 0>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, xp0, xp1, xp2, gt0, gt1, gt2);
+    wring_run<T, 0>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, m);
   } else {
-    wring_run<T, 1>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, xp0, xp1, xp2, gt0, gt1, gt2);
+    wring_run<T, 1>(as, xs + (cis - cib) * 32, gy, wsb, gm, split, cib, cob, x_cin, tid, m);
   }
 #endif
 }
@@ -543,6 +738,53 @@ int launch_wring(const WgradArgs& a, const WRingGeom& gm, const void* x, const v
   return check_launch("wgrad_ring_kernel");
 }
 
+// The line of cost and the slices of a batch; ws_bytes: the workspace all problems need together. False when the batch
+// cannot be laid out (too many problems, too much work for 32-bit positions).
+bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, size_t& ws_bytes) {
+  if (count < 1 || count > kWgradBatchMax) return false;
+  b = WRingBatch{};
+  b.count = count;
+  int64_t pos = 0, quads = 0;
+  for (int i = 0; i < count; ++i) {
+    const WgradArgs& a = items[i].a;
+    WRingBatchEntry& e = b.e[i];
+    e.a = a;
+    e.x = items[i].x; e.x1 = items[i].x1; e.c_first = items[i].c_first; e.gy = items[i].gy; e.gw = items[i].gw;
+    e.tiles_h = (int)cdiv(a.oh, kTH);
+    e.tiles_w = (int)cdiv(a.ow, kTW);
+    e.steps = (int)cdiv(a.od, kTD);
+    e.nblk_ci = a.cin / 32;
+    e.nblk = e.nblk_ci * (a.cout / 32);
+    const int64_t ncols = (int64_t)a.n * e.tiles_h * e.tiles_w;
+    const int64_t cost = (int64_t)e.nblk * ncols * (e.steps + kFillCost);
+    if (ncols > kBatchMaxTotal || cost > kBatchMaxTotal) return false;
+    e.ncols = (int)ncols;
+    e.pos_begin = (int)pos;
+    e.quad_begin = (int)quads;
+    pos += cost;
+    quads += (int64_t)a.cout * 27 * a.cin / 4;  // a multiple of 256 (Cout and Cin in blocks of 32)
+    if ((int64_t)a.cout * 27 * a.cin > 0x7fffffffLL) return false;
+    if (pos > kBatchMaxTotal || quads > 0x3fffffffLL) return false;
+  }
+  b.total = (int)pos;
+  b.quads = (int)quads;
+  b.wgs = b.total < kComputeUnits ? b.total : kComputeUnits;
+  ws_bytes = 0;
+  for (int i = 0; i < count; ++i) {
+    WRingBatchEntry& e = b.e[i];
+    const int blockcost = e.ncols * (e.steps + kFillCost);
+    int most = 1;
+    for (int blk = 0; blk < e.nblk; ++blk) {
+      const int b0 = e.pos_begin + blk * blockcost;
+      const int n = batch_owner(b0 + blockcost - 1, b.total, b.wgs) - batch_owner(b0, b.total, b.wgs) + 1;
+      if (n > most) most = n;
+    }
+    e.slices = most;
+    ws_bytes += align_up((size_t)most * e.a.cout * 27 * e.a.cin * sizeof(float), 256);
+  }
+  return true;
+}
+
 }  // namespace
 
 // Rows of more than 16 voxels; a plane pair with its halo and a gy tile must span less than the buffer range.
@@ -559,6 +801,37 @@ int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy
   const WRingGeom gm = wring_geom(a);
   if (dtype == SFH_BF16) return launch_wring<bf16_t>(a, gm, x, gy, ws, st, x2);
   return launch_wring<fp16_t>(a, gm, x, gy, ws, st, x2);
+}
+
+bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype) { return mfma_wgrad_supported(a, dtype) && mfma_wgrad_ring_applies(a); }
+
+size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count) {
+  WRingBatch b;
+  size_t bytes = 0;
+  return wring_batch_plan(items, count, b, bytes) ? bytes : 0;
+}
+
+int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
+                     hipStream_t st) {
+  WRingBatch b;
+  size_t need = 0;
+  if (!wring_batch_plan(items, count, b, need)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: %d problems cannot share a launch", count);
+  if (workspace == nullptr || workspace_bytes < need)
+    return fail(SFH_ERR_WORKSPACE, "conv3d wgrad batch: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
+  char* ws = (char*)workspace;
+  for (int i = 0; i < count; ++i) {
+    b.e[i].ws = (float*)ws;
+    ws += align_up((size_t)b.e[i].slices * b.e[i].a.cout * 27 * b.e[i].a.cin * sizeof(float), 256);
+  }
+  if (b.total == 0) return SFH_OK;
+  if (dtype == SFH_BF16) hipLaunchKernelGGL((wgrad_ring_batch_kernel<bf16_t>), dim3((unsigned)b.wgs), dim3(256), 0, st, b);
+  else hipLaunchKernelGGL((wgrad_ring_batch_kernel<fp16_t>), dim3((unsigned)b.wgs), dim3(256), 0, st, b);
+  if (int rc = check_launch("wgrad_ring_batch_kernel")) return rc;
+  const unsigned sum_grid = (unsigned)cdiv(b.quads, 256);
+  if (gw_dtype == SFH_FP32) hipLaunchKernelGGL((wgrad_ring_batch_sum<float>), dim3(sum_grid), dim3(256), 0, st, b);
+  else if (gw_dtype == SFH_BF16) hipLaunchKernelGGL((wgrad_ring_batch_sum<bf16_t>), dim3(sum_grid), dim3(256), 0, st, b);
+  else hipLaunchKernelGGL((wgrad_ring_batch_sum<fp16_t>), dim3(sum_grid), dim3(256), 0, st, b);
+  return check_launch("wgrad_ring_batch_sum");
 }
 
 }  // namespace sfh

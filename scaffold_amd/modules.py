@@ -39,7 +39,8 @@ from . import groupnorm as _gn
 from . import halo as _halo
 from . import transposed as _ct
 
-__all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand", "compute_copy"]
+__all__ = ["FastConv3d", "FastConvTranspose3d", "FastGroupNorm", "autocast_dtype", "cast_operand", "compute_copy",
+           "flush_weight_gradients"]
 
 _CL3D = torch.channels_last_3d
 
@@ -113,8 +114,73 @@ def _fp32_weight_grad(fn, *args, **kwargs):
         return fn(*args, **kwargs).to(torch.float32)
 
 
+# ---- weight gradients of a backward pass in one launch -----------------------------------------------------------------
+# Nothing reads a weight gradient before the optimizer (``ScaFFold/utils/trainer.py:678-694``), and a launch of the
+# weight-gradient kernel costs 15-20 us whatever the problem.  A convolution whose module has ``defer_weight_grad`` set
+# therefore does not compute its weight gradient in its own backward node: the node leaves (parameter, operands) in a
+# queue and returns no gradient for the weight, and a callback the autograd engine runs when the backward pass has
+# finished -- still inside ``backward()`` -- computes all queued gradients with :func:`conv3d_backward_weight_batch` and
+# adds them to the parameters' ``.grad``.  After ``backward()`` returns the gradients are where they always are.  What
+# differs: hooks on the parameter's gradient accumulation do not see these gradients, and the operands stay alive until
+# the end of the pass.
+class _QueuedWeightGrad:
+    __slots__ = ("param", "inp", "wshape", "gy", "padding", "grad_dtype")
+
+    def __init__(self, param, inp, wshape, gy, padding, grad_dtype):
+        self.param, self.inp, self.wshape, self.gy, self.padding, self.grad_dtype = param, inp, wshape, gy, padding, grad_dtype
+
+
+_WEIGHT_GRAD_QUEUE: list = []
+_BATCHABLE: dict = {}
+
+
+def _deferrable(param, in_shape, wshape, stride, padding, dilation, dtype) -> bool:
+    """Whether a weight gradient can wait for the end of the pass: the parameter is a leaf that takes a ``.grad`` and the
+    library batches the problem."""
+    if param is None or not param.is_leaf or not param.requires_grad:
+        return False
+    key = (in_shape, wshape, stride, padding, dilation, dtype)
+    ok = _BATCHABLE.get(key)
+    if ok is None:
+        ok = _c3.weight_grad_batchable(in_shape, wshape, stride, padding, dilation, dtype)
+        if len(_BATCHABLE) > 256:
+            _BATCHABLE.clear()
+        _BATCHABLE[key] = ok
+    return ok
+
+
+def _queue_weight_grad(item: _QueuedWeightGrad) -> None:
+    _WEIGHT_GRAD_QUEUE.append(item)
+    # one callback per queued gradient: the first to run takes the whole queue, the others find it empty (a pass that
+    # raised before its callbacks ran leaves its entries to the next pass's callbacks, or to flush_weight_gradients())
+    torch.autograd.Variable._execution_engine.queue_callback(flush_weight_gradients)
+
+
+def flush_weight_gradients() -> None:
+    """Compute the queued weight gradients and add them to their parameters' ``.grad`` (runs by itself at the end of a
+    backward pass; callable by hand after a pass that raised)."""
+    if not _WEIGHT_GRAD_QUEUE:
+        return
+    queue = list(_WEIGHT_GRAD_QUEUE)
+    _WEIGHT_GRAD_QUEUE.clear()
+    groups: dict = {}
+    for it in queue:
+        groups.setdefault((it.gy.device, it.gy.dtype, it.grad_dtype), []).append(it)
+    with torch.no_grad():
+        for (_, dt, gdt), items in groups.items():
+            grads = _c3.conv3d_backward_weight_batch([(it.inp, it.wshape, it.gy, it.padding) for it in items],
+                                                     grad_dtype=None if gdt is dt else gdt)
+            for it, gw in zip(items, grads):
+                p = it.param
+                if p.grad is None:
+                    # in the parameter's own layout, as the engine's accumulation would leave it
+                    p.grad = gw if gw.stride() == p.stride() else torch.empty_like(p).copy_(gw)
+                else:
+                    p.grad.add_(gw)
+
+
 # positions in _Conv3dFn.forward's argument list (after ctx): the gradients come back in this order
-_ARG_SECOND, _N_ARGS = 11, 13
+_ARG_SECOND, _N_ARGS = 11, 14
 
 
 class _Conv3dFn(torch.autograd.Function):
@@ -123,7 +189,7 @@ class _Conv3dFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, weight, bias, stride, padding, dilation, weight_compute=None, bias_compute=None, packs=None, slab=None,
-                gn_groups=0, second=None, slab2=None):
+                gn_groups=0, second=None, slab2=None, defer_weight_grad=False):
         # weight / bias are the tensors that receive gradients; when half-precision copies of fp32 masters are
         # given, the kernels read those and the gradients are produced in the masters' dtype directly
         wc = weight if weight_compute is None else weight_compute
@@ -159,6 +225,8 @@ class _Conv3dFn(torch.autograd.Function):
             ctx.save_for_backward(x, wc, second) if pd is None else ctx.save_for_backward(x, wc, second, pd)
         ctx.conv_args = (stride, padding, dilation, bias is not None, None if bias is None else bias.dtype,
                          weight.dtype is not wc.dtype)
+        # the parameter whose .grad a deferred weight gradient is added to (see flush_weight_gradients)
+        ctx.defer_param = weight if defer_weight_grad else None
         return y
 
     @staticmethod
@@ -183,15 +251,18 @@ class _Conv3dFn(torch.autograd.Function):
                 grad_w, grad_b = both
                 if grad_b.dtype is not bias_dtype:
                     grad_b = grad_b.to(bias_dtype)
-                return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None
-        if needs_w:
+                return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
+        if needs_w and _deferrable(ctx.defer_param, x.shape, weight.shape, stride, padding, dilation, x.dtype):
+            _queue_weight_grad(_QueuedWeightGrad(ctx.defer_param, x, weight.shape, grad_output, padding,
+                                                 torch.float32 if master else x.dtype))
+        elif needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight, x, weight.shape, grad_output, stride, padding, dilation, 1,
                                            _checked=True)
             else:
                 grad_w = _c3.conv3d_backward_weight(x, weight.shape, grad_output, stride, padding, dilation, 1, _checked=True)
         grad_b = _c3.bias_grad(grad_output, bias_dtype) if (has_bias and needs_b) else None
-        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None
+        return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
 
     @staticmethod
     def _backward_pair(ctx, grad_output):
@@ -211,7 +282,11 @@ class _Conv3dFn(torch.autograd.Function):
                 grad_x = grad_x.narrow(2, ctx.halo, ctx.depth)
                 grad_second = grad_second.narrow(2, ctx.halo, ctx.depth)
         grad_w = None
-        if needs_w:
+        if needs_w and _deferrable(ctx.defer_param, torch.Size((x.shape[0], x.shape[1] + second.shape[1], *x.shape[2:])), weight.shape,
+                                   stride, padding, dilation, x.dtype):
+            _queue_weight_grad(_QueuedWeightGrad(ctx.defer_param, (x, second), weight.shape, grad_output, padding,
+                                                 torch.float32 if master else x.dtype))
+        elif needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight_pair, x, second, weight.shape, grad_output, stride, padding,
                                            dilation, _checked=True)
@@ -280,6 +355,9 @@ class FastConv3d(nn.Conv3d):
     #: groups of a GroupNorm that reads this module's output next (0: none): the forward launch then also leaves that
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
+    #: leave this module's weight gradient to the end of the backward pass, where all such gradients come from one launch
+    #: (see flush_weight_gradients); taken up only where the weight is the parameter itself and the library batches the shape
+    defer_weight_grad = False
 
     def _pair_operands(self, x, second):
         """The tensors the kernels would read for ``forward(x, second)`` and the padding they would run with, or ``None``
@@ -362,10 +440,10 @@ class FastConv3d(nn.Conv3d):
         if master:
             return _Conv3dFn.apply(x, weight, bias, stride, padding, dilation, w, b,
                                    _current_packs(weight, w, in_shape, stride, padding, dilation), slab, self.gn_groups,
-                                   second, slab2)
+                                   second, slab2, self.defer_weight_grad)
         packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is weight else None
         return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, second,
-                               slab2)
+                               slab2, self.defer_weight_grad and w is weight)
 
     def forward(self, x: torch.Tensor, second: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``second``: the input is ``torch.cat([x, second], 1)``, read from the two tensors themselves (the decoder's skip
@@ -409,10 +487,12 @@ class FastConv3d(nn.Conv3d):
             inner = x
         if master:
             return _Conv3dFn.apply(inner, weight, bias, stride, padding, dilation, w, b,
-                                   _current_packs(weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
+                                   _current_packs(weight, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
+                                   None, None, self.defer_weight_grad)
         if w is weight:
             return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None,
-                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups)
+                                   _current_packs(w, w, x.shape, stride, padding, dilation), slab, self.gn_groups,
+                                   None, None, self.defer_weight_grad)
         return _Conv3dFn.apply(inner, w, b, stride, padding, dilation, None, None, None, slab, self.gn_groups)
 
 

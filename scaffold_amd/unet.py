@@ -211,6 +211,15 @@ class UNet(nn.Module):
                 block.double_conv[4].out_halo = halo
         return self
 
+    def defer_weight_gradients(self, enabled: bool = True):
+        """Leave the weight gradients of the 3x3x3 convolutions to the end of the backward pass, where one launch computes
+        all that the library batches (``modules.flush_weight_gradients``): ``.grad`` is complete when ``backward()``
+        returns, as always; hooks on the parameters' gradient accumulation do not see these gradients."""
+        for m in self.modules():
+            if isinstance(m, FastConv3d):
+                m.defer_weight_grad = bool(enabled)
+        return self
+
     def _run(self, block, *inputs):
         if self.checkpointing:
             return torch.utils.checkpoint.checkpoint(block, *inputs, use_reentrant=False)
