@@ -254,17 +254,22 @@ int sfh_conv3d_wgrad_pair(const sfh_conv3d_desc* p, int dtype, const void* x_fir
 /* ---- several conv3d weight gradients in one launch ------------------------------------------
  * The weight gradients of a training step (triton_conv3d.conv3d_backward_weight once per convolution,
  * triton_conv3d/reduce_gemm.py:1177; nothing reads them before the optimizer, ScaFFold/utils/trainer.py:678-694) as ONE
- * launch of the weight-gradient kernel and ONE sum pass: what a launch of sfh_conv3d_wgrad costs whatever the problem --
- * all workgroups fetching their first operands at once, all writing their partial slice at once, the sum pass reading the
- * slices back, two launch gaps: 15-20 us on MI355X -- is paid once for up to SFH_WGRAD_BATCH_MAX problems. The work of
- * all problems is laid on one line and cut evenly over the workgroups; a workgroup that covers parts of several
- * 32 x 32 channel blocks writes a slice for each. Each item is one sfh_conv3d_wgrad (x_second NULL) or
- * sfh_conv3d_wgrad_pair call; all share `dtype` and the gradient dtype (SFH_FLAG_GRAD_FP32). Results: every gradient is
- * the sum of fp32 partials in a fixed order that is a pure function of the LIST of problems (their shapes, in order) --
- * the same bits on every run, and within fp32 summation-order rounding of sfh_conv3d_wgrad's (whose cuts differ).
+ * few launches instead of one kernel launch and one sum pass per convolution: what a launch of sfh_conv3d_wgrad costs
+ * whatever the problem -- all workgroups fetching their first operands at once, all writing their partial slice at once,
+ * the sum pass reading the slices back, two launch gaps: 15-20 us on MI355X -- is paid once for up to
+ * SFH_WGRAD_BATCH_MAX problems. Problems with output rows of more than 16 voxels share one launch and one sum pass: the
+ * work of all of them is laid on one line and cut evenly over the workgroups; a workgroup that covers parts of several
+ * 32 x 32 channel blocks writes a slice for each. Small-volume problems (rows of 16 or 8 voxels, at most 32 tiles of
+ * 256 voxels) share a second launch in which every 32 x 32 block is walked from its first tile to its last by one
+ * workgroup and stored straight into the gradient: no slices, no sum pass. Each item is one sfh_conv3d_wgrad
+ * (x_second NULL) or sfh_conv3d_wgrad_pair call; all share `dtype` and the gradient dtype (SFH_FLAG_GRAD_FP32).
+ * Results: every gradient is the sum of fp32 partials in a fixed order that is a pure function of the LIST of problems
+ * (their shapes, in order) -- the same bits on every run, and within fp32 summation-order rounding of
+ * sfh_conv3d_wgrad's (whose cuts differ).
  * Served: the problems sfh_conv3d_wgrad_batch_supported answers 1 for -- 3 x 3 x 3, unit stride and dilation, SFH_BF16 /
- * SFH_FP16, channel counts multiples of 32, output rows of more than 16 voxels; anything else in the list fails the
- * call with SFH_ERR_UNSUPPORTED before any launch (the caller runs those through sfh_conv3d_wgrad).
+ * SFH_FP16, channel counts multiples of 32, and either rows of more than 16 voxels or a small volume as above; anything
+ * else in the list fails the call with SFH_ERR_UNSUPPORTED before any launch (the caller runs those through
+ * sfh_conv3d_wgrad). The workspace query answers 0 for a refused list and is never 0 for a served one.
  * The batching itself has no counterpart in the reference. */
 #define SFH_WGRAD_BATCH_MAX 16
 typedef struct sfh_conv3d_wgrad_item {

@@ -842,7 +842,8 @@ WGRAD_BATCH_MAX = 16  # SFH_WGRAD_BATCH_MAX
 
 def weight_grad_batchable(input_shape, weight_shape, stride, padding, dilation, dtype) -> bool:
     """Whether :func:`conv3d_backward_weight_batch` takes this problem (3x3x3, unit stride and dilation, bf16 / fp16,
-    channel counts multiples of 32, output rows of more than 16 voxels): a pure function of the problem."""
+    channel counts multiples of 32, and output rows of more than 16 voxels or a volume of at most 32 tiles of 256
+    voxels): a pure function of the problem."""
     if dtype not in (torch.bfloat16, torch.float16):
         return False
     try:

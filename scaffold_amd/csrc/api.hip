@@ -766,7 +766,7 @@ static int wgrad_batch_items(const sfh_conv3d_wgrad_item* items, int32_t count, 
     if (int rc = check_conv(&items[i].desc, dtype, out)) return rc;
     const sfh_conv3d_desc& d = items[i].desc;
     if (!wgrad_uses_mfma(d, dtype, out) || !mfma_wgrad_batch_applies(wgrad_args(d, out), dtype))
-      return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: problem %d is not a 3x3x3 unit-stride 16-bit problem with rows of more than 16 voxels", (int)i);
+      return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: problem %d is served only by a launch of its own (sfh_conv3d_wgrad_batch_supported)", (int)i);
     WgradBatchItem& o = out_items[i];
     o.a = wgrad_args(d, out);
     o.x = items[i].x; o.x1 = items[i].x_second; o.c_first = items[i].cin_first; o.gy = items[i].gy; o.gw = items[i].gw;

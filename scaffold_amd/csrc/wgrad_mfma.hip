@@ -391,6 +391,143 @@ wgrad_mfma_kernel(WgradArgs a, const T* __restrict__ x, const T* __restrict__ gy
 #endif
 }
 
+// ---- several small-volume weight gradients in one launch ----------------------------------------------------------------------
+// The deep levels of a U-Net have many 32 x 32 blocks and few tiles under each (8 tiles at 8 x 16 x 16, one at
+// 4 x 8 x 8): launched one problem at a time every workgroup walks a handful of tiles, writes a slice and a sum pass
+// follows -- 23-44 us for 4-29 GFLOP. In a batch the UNITS -- (problem, block) with all its tiles -- of all problems lie
+// on one line of cost (tiles + kUnitCost each), workgroup w of W takes the units that start in
+// [w total / W, (w + 1) total / W), walks each from its first tile to its last and stores the finished block straight
+// into the gradient: no slices, no sum pass, and the order of additions of a block is that of its tiles, whatever else
+// is in the list. The two tile shapes (rows of 16 and of 8 voxels) share a launch.
+constexpr int kUnitCost = 2;          // what starting and storing a unit costs, in tiles (1 .. 5 measure alike)
+constexpr int kBatchMaxTiles = 32;    // longer units would not balance: such problems are launched alone
+
+struct WTileBatchEntry {
+  WgradArgs a;
+  const void* x;
+  const void* x1;
+  const void* gy;
+  void* gw;
+  int c_first;
+  int tw;                              // 16 or 8
+  int tiles_d, tiles_h, tiles_w, ntiles;
+  int nblk_ci, nblk;
+  int pos_begin;
+};
+
+struct WTileBatch {
+  int count, wgs, total;
+  WTileBatchEntry e[kWgradBatchMax];
+};
+
+template <typename C, typename TOut>
+__device__ __forceinline__ void wave_store_block(const f32x16_t (&acc)[7], TOut* __restrict__ dst, int cin, int lane, int wave) {
+  const int j = lane & 31;
+  int kg = lane >> 5;
+  // (opaque to the optimiser: in the loop over units it would otherwise compute all 112 store offsets ahead of the loop
+  // and keep them in scratch memory)
+  asm volatile("" : "+v"(kg));
+#pragma unroll
+  for (int t = 0; t < 7; ++t) {
+    if (t == 6 && wave == 3) break;
+    const int tap = t < 3 ? 6 * wave + t : (t < 6 ? 6 * wave + t : 24 + wave);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int co = 8 * (r / 4) + 4 * kg + (r % 4);
+      dst[((int64_t)co * 27 + tap) * cin + j] = elem<TOut>::from_float(acc[t][r]);
+    }
+  }
+}
+
+// One unit: all tiles of block (cob, cib) of a problem, the finished block stored at gw. The staging wavefronts and
+// the compute wavefronts meet at 1 + ntiles barriers, as in the kernel above.
+template <typename T, typename C, typename TOut>
+__device__ __forceinline__ void wtile_unit(const WgradArgs& a, const T* __restrict__ x, const T* __restrict__ x1, int c_first,
+                                           const T* __restrict__ gy, TOut* __restrict__ gw, int tiles_d, int tiles_h, int tiles_w,
+                                           int ntiles, int cib, int cob, char* buf0, char* buf1, int tid) {
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (wave >= 4) {
+    WgradArgs as = a;
+    const T* xs = x;
+    int cis = cib;
+    if (x1 != nullptr) {
+      const bool second = cib * 32 >= c_first;
+      xs = second ? x1 : x;
+      as.cin = second ? a.cin - c_first : c_first;
+      cis = second ? cib - c_first / 32 : cib;
+    }
+    Slots<C> sl;
+    init_slots<C>(as, tid - 256, sl);
+    auto origin = [&](int tile) { return decode_tile(tile < ntiles ? tile : ntiles - 1, tiles_d, tiles_h, tiles_w, C::TD, C::TH, C::TW); };
+    SlotLoop<T, C, 0>::fetch_all(as, xs, gy, origin(0), cis, cob, sl);
+    SlotLoop<T, C, 0>::stage_all(buf0, sl);
+    SlotLoop<T, C, 0>::fetch_all(as, xs, gy, origin(1), cis, cob, sl);
+    __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+    __builtin_amdgcn_s_barrier();
+    for (int tile = 0; tile < ntiles; ++tile) {
+      char* idle = (tile & 1) ? buf0 : buf1;
+      SlotLoop<T, C, 0>::stage_and_refill(idle, as, xs, gy, origin(tile + 2), cis, cob, sl);
+      __builtin_amdgcn_s_waitcnt(kWaitLgkm0);
+      __builtin_amdgcn_s_barrier();
+    }
+  } else {
+    f32x16_t acc[7];
+#pragma unroll
+    for (int t = 0; t < 7; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    __builtin_amdgcn_s_barrier();  // the first tile is staged
+    for (int tile = 0; tile < ntiles; ++tile) {
+      const char* cur = (tile & 1) ? buf1 : buf0;
+      asm volatile("" ::: "memory");  // LDS changes behind this wavefront's back: reload every tile
+      wave_compute<T, C>(cur, lane, wave, acc);
+      __builtin_amdgcn_s_barrier();
+    }
+    wave_store_block<C, TOut>(acc, gw + ((int64_t)cob * 32 * 27) * a.cin + cib * 32, a.cin, lane, wave);
+  }
+}
+
+typedef WTile<2, 8, 16> WTile16;
+typedef WTile<4, 8, 8> WTile8;
+constexpr int kBatchLds = WTile16::LDS > WTile8::LDS ? WTile16::LDS : WTile8::LDS;
+
+__host__ __device__ __forceinline__ int tile_batch_cut(int w, int total, int wgs) { return (int)((uint32_t)w * (uint32_t)total / (uint32_t)wgs); }
+
+template <typename T, typename TOut>
+__global__ void __launch_bounds__(512) wgrad_mfma_batch_kernel(WTileBatch b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __shared__ __attribute__((aligned(16))) char buf0[kBatchLds];
+  __shared__ __attribute__((aligned(16))) char buf1[kBatchLds];
+  const int tid = threadIdx.x;
+  const int w = (int)xcd_remap(blockIdx.x, (uint32_t)b.wgs);
+  const int hi = tile_batch_cut(w + 1, b.total, b.wgs);
+  int pos = tile_batch_cut(w, b.total, b.wgs);
+  while (pos < hi) {
+    int p = 0;
+    for (int k = 1; k < b.count; ++k)
+      if (pos >= b.e[k].pos_begin) p = k;
+    const int ntiles = b.e[p].ntiles, cost = ntiles + kUnitCost;
+    const int unit = (pos - b.e[p].pos_begin + cost - 1) / cost;  // the first unit that starts at or behind pos
+    if (unit >= b.e[p].nblk) {  // none left in this problem: on to the next one's first unit
+      pos = p + 1 < b.count ? b.e[p + 1].pos_begin : hi;
+      continue;
+    }
+    const int start = b.e[p].pos_begin + unit * cost;
+    if (start >= hi) break;
+    const WgradArgs a = b.e[p].a;
+    const int nblk_ci = b.e[p].nblk_ci;
+    const int cib = unit % nblk_ci, cob = unit / nblk_ci;
+    if (b.e[p].tw == 16)
+      wtile_unit<T, WTile16, TOut>(a, (const T*)b.e[p].x, (const T*)b.e[p].x1, b.e[p].c_first, (const T*)b.e[p].gy, (TOut*)b.e[p].gw,
+                                   b.e[p].tiles_d, b.e[p].tiles_h, b.e[p].tiles_w, ntiles, cib, cob, buf0, buf1, tid);
+    else
+      wtile_unit<T, WTile8, TOut>(a, (const T*)b.e[p].x, (const T*)b.e[p].x1, b.e[p].c_first, (const T*)b.e[p].gy, (TOut*)b.e[p].gw,
+                                  b.e[p].tiles_d, b.e[p].tiles_h, b.e[p].tiles_w, ntiles, cib, cob, buf0, buf1, tid);
+    pos = start + cost;
+  }
+#endif
+}
+
 struct Plan {
   int tw;  // 32, 16 or 8
   int tiles_d, tiles_h, tiles_w, ntiles;
@@ -467,6 +604,39 @@ int launch_typed(const WgradArgs& a, const void* x, const void* gy, void* gw, in
   return sum_slices(gw_dtype, ws, gw, nelem, p.splits, st);
 }
 
+bool tile_batch_plan(const WgradBatchItem* items, int count, WTileBatch& b) {
+  if (count < 1 || count > kWgradBatchMax) return false;
+  b = WTileBatch{};
+  b.count = count;
+  int64_t pos = 0;
+  for (int i = 0; i < count; ++i) {
+    const WgradArgs& a = items[i].a;
+    if (ring_serves(a)) return false;
+    const Plan p = make_plan(a);
+    if (p.tw == 32 || p.ntiles > kBatchMaxTiles) return false;
+    WTileBatchEntry& e = b.e[i];
+    e.a = a;
+    e.x = items[i].x; e.x1 = items[i].x1; e.c_first = items[i].c_first; e.gy = items[i].gy; e.gw = items[i].gw;
+    e.tw = p.tw;
+    e.tiles_d = p.tiles_d; e.tiles_h = p.tiles_h; e.tiles_w = p.tiles_w; e.ntiles = p.ntiles;
+    e.nblk_ci = p.nblk_ci; e.nblk = p.nblk;
+    e.pos_begin = (int)pos;
+    pos += (int64_t)p.nblk * (p.ntiles + kUnitCost);
+    if (pos > 0x7fffff) return false;  // 32-bit cuts
+  }
+  b.total = (int)pos;
+  b.wgs = b.total < kTargetWorkgroups ? b.total : kTargetWorkgroups;
+  return true;
+}
+
+template <typename T>
+int launch_tile_batch(const WTileBatch& b, int gw_dtype, hipStream_t st) {
+  if (b.total == 0) return SFH_OK;
+  if (gw_dtype == SFH_FP32) hipLaunchKernelGGL((wgrad_mfma_batch_kernel<T, float>), dim3((unsigned)b.wgs), dim3(512), 0, st, b);
+  else hipLaunchKernelGGL((wgrad_mfma_batch_kernel<T, T>), dim3((unsigned)b.wgs), dim3(512), 0, st, b);
+  return check_launch("wgrad_mfma_batch_kernel");
+}
+
 }  // namespace
 
 bool mfma_wgrad_supported(const WgradArgs& a, int dtype) {
@@ -498,6 +668,56 @@ int mfma_wgrad(const WgradArgs& a, int dtype, const void* x, const void* gy, voi
   const ChannelPair pair = x2 != nullptr ? *x2 : ChannelPair{nullptr, 0};
   if (dtype == SFH_BF16) return launch_typed<bf16_t>(a, x, gy, gw, gw_dtype, workspace, st, pair);
   return launch_typed<fp16_t>(a, x, gy, gw, gw_dtype, workspace, st, pair);
+}
+
+// ---- a list of problems: the ring-served ones in one launch + sum pass, the small-volume ones in one launch -------------
+namespace {
+bool tile_batch_applies(const WgradArgs& a) {
+  if (ring_serves(a)) return false;
+  const Plan p = make_plan(a);
+  return p.tw != 32 && p.ntiles <= kBatchMaxTiles;
+}
+// Splits a list by family, keeping the order inside each.
+int split_list(const WgradBatchItem* items, int count, WgradBatchItem* ring, int& nring, WgradBatchItem* tile, int& ntile) {
+  nring = ntile = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ring_serves(items[i].a)) ring[nring++] = items[i];
+    else if (tile_batch_applies(items[i].a)) tile[ntile++] = items[i];
+    else return SFH_ERR_UNSUPPORTED;
+  }
+  return SFH_OK;
+}
+}  // namespace
+
+bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype) {
+  return mfma_wgrad_supported(a, dtype) && (ring_serves(a) || tile_batch_applies(a));
+}
+
+size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count) {
+  if (count < 1 || count > kWgradBatchMax) return 0;
+  WgradBatchItem ring[kWgradBatchMax], tile[kWgradBatchMax];
+  int nring, ntile;
+  if (split_list(items, count, ring, nring, tile, ntile) != SFH_OK) return 0;
+  WTileBatch tb;
+  if (ntile > 0 && !tile_batch_plan(tile, ntile, tb)) return 0;
+  if (nring == 0) return 256;  // (nothing is needed; a non-zero answer says the list is taken)
+  const size_t bytes = mfma_wgrad_ring_batch_workspace_bytes(ring, nring);
+  return bytes;
+}
+
+int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
+                     hipStream_t st) {
+  if (count < 1 || count > kWgradBatchMax) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: 1 .. %d problems a call", kWgradBatchMax);
+  WgradBatchItem ring[kWgradBatchMax], tile[kWgradBatchMax];
+  int nring, ntile;
+  if (split_list(items, count, ring, nring, tile, ntile) != SFH_OK)
+    return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: a problem of the list is served only by a launch of its own");
+  WTileBatch tb;
+  if (ntile > 0 && !tile_batch_plan(tile, ntile, tb)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: the small-volume problems cannot share a launch");
+  if (nring > 0)
+    if (int rc = mfma_wgrad_ring_batch(ring, nring, dtype, gw_dtype, workspace, workspace_bytes, st)) return rc;
+  if (ntile > 0) return dtype == SFH_BF16 ? launch_tile_batch<bf16_t>(tb, gw_dtype, st) : launch_tile_batch<fp16_t>(tb, gw_dtype, st);
+  return SFH_OK;
 }
 
 }  // namespace sfh

@@ -28,10 +28,12 @@ bool mfma_wgrad_ring_applies(const WgradArgs& a);
 int mfma_wgrad_ring_splits(const WgradArgs& a);
 int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy, float* ws, hipStream_t st, const ChannelPair& x2);
 
-// Several ring-served weight gradients in one launch and one sum pass (wgrad_ring.hip): the cost every launch pays
-// once -- the first fetch of all workgroups, the slices written and read back, two launch gaps -- is paid once for the
-// batch. All problems share dtype and the gradient's dtype; how the work is cut over the workgroups is a pure function
-// of the list of problems, every sum has a fixed order (not that of the one-problem launch: the cuts differ).
+// Several weight gradients from as few launches as possible: the ring-served problems of a list (rows of more than 16
+// voxels) in one launch and one sum pass (wgrad_ring.hip), its small-volume problems (rows of 16 or 8 voxels, at most 32
+// tiles under a block) in one launch that writes the gradients directly (wgrad_mfma.hip). The cost every launch pays
+// -- the first fetch of all workgroups, the slices written and read back, launch gaps -- is paid once per family. All
+// problems share dtype and the gradient's dtype; how the work is cut over the workgroups is a pure function of the
+// list of problems, every sum has a fixed order (not that of the one-problem launch: the cuts differ).
 constexpr int kWgradBatchMax = 16;
 struct WgradBatchItem {
   WgradArgs a;
@@ -45,5 +47,9 @@ bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype);
 size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count);  // 0: the list cannot share a launch
 int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
                      hipStream_t st);
+// the ring-served family alone (every item must be ring-served)
+size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count);
+int mfma_wgrad_ring_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t st);
 
 }  // namespace sfh

@@ -803,16 +803,14 @@ int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy
   return launch_wring<fp16_t>(a, gm, x, gy, ws, st, x2);
 }
 
-bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype) { return mfma_wgrad_supported(a, dtype) && mfma_wgrad_ring_applies(a); }
-
-size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count) {
+size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count) {
   WRingBatch b;
   size_t bytes = 0;
   return wring_batch_plan(items, count, b, bytes) ? bytes : 0;
 }
 
-int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
-                     hipStream_t st) {
+int mfma_wgrad_ring_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
+                          hipStream_t st) {
   WRingBatch b;
   size_t need = 0;
   if (!wring_batch_plan(items, count, b, need)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: %d problems cannot share a launch", count);

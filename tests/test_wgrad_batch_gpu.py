@@ -5,7 +5,8 @@ The reference computes each weight gradient with a launch of its own (``triton_c
 the same arithmetic -- fp32 partial sums over voxel ranges, added in a fixed order -- with the ranges cut differently, so
 what it is held to is: the fp64 oracle's error bound for every problem of a list (ragged extents, several samples, the
 depth-shard form, inputs handed over as two tensors, lists long enough that a workgroup covers parts of several problems
-and lists so short that a problem spans many workgroups), agreement with the one-problem entry point to fp32
+and lists so short that a problem spans many workgroups, small volumes whose blocks are walked whole, both kinds in one
+list), agreement with the one-problem entry point to fp32
 summation-order rounding, the same bits on every run and for every list with the same shapes, and refusal -- before any
 launch -- of a list with a problem the batch does not serve.
 """
@@ -33,6 +34,14 @@ LISTS = {
                (1, 128, 128, (4, 8, 32), (1, 1, 1), 0), (1, 256, 128, (4, 8, 32), (1, 1, 1), 128)],
     "many-blocks": [(1, 128, 256, (2, 4, 32), (1, 1, 1), 0), (1, 96, 160, (3, 5, 40), (1, 1, 1), 32),
                     (1, 32, 32, (2, 4, 17), (1, 1, 1), 0)],                          # more blocks than workgroups
+    # small volumes (rows of 16 and of 8 voxels): whole blocks per workgroup, no slices
+    "deep": [(1, 128, 256, (8, 16, 16), (0, 1, 1), 0), (1, 256, 256, (8, 16, 16), (0, 1, 1), 0),
+             (1, 512, 256, (8, 16, 16), (0, 1, 1), 256), (1, 256, 512, (4, 8, 8), (0, 1, 1), 0)],
+    "deep-ragged": [(2, 32, 64, (3, 5, 7), (1, 1, 1), 0), (1, 64, 32, (5, 9, 13), (1, 1, 1), 32), (3, 32, 32, (1, 1, 1), (1, 1, 1), 0),
+                    (1, 96, 64, (9, 16, 16), (0, 1, 1), 64)],
+    # both families in one list (two launches and a sum pass)
+    "mixed": [(1, 64, 64, (8, 16, 32), (0, 1, 1), 0), (1, 128, 256, (4, 8, 16), (1, 1, 1), 0), (1, 64, 128, (4, 8, 32), (1, 1, 1), 32),
+              (1, 256, 256, (4, 8, 8), (1, 1, 1), 128)],
 }
 
 
@@ -98,12 +107,13 @@ def test_more_problems_than_a_launch_takes(device):
 def test_what_is_refused(device):
     dtype = torch.bfloat16
     ok = (1, 32, 32, (4, 8, 32), (1, 1, 1), 0)
-    assert not c3.weight_grad_batchable((1, 32, 4, 8, 16), (32, 32, 3, 3, 3), 1, 1, 1, dtype)        # rows of 16 voxels
+    assert c3.weight_grad_batchable((1, 32, 4, 8, 16), (32, 32, 3, 3, 3), 1, 1, 1, dtype)            # rows of 16 voxels, two tiles
+    assert not c3.weight_grad_batchable((1, 32, 40, 64, 16), (32, 32, 3, 3, 3), 1, 1, 1, dtype)      # ... and 160 tiles
     assert not c3.weight_grad_batchable((1, 32, 4, 8, 32), (32, 32, 1, 1, 1), 1, 0, 1, dtype)        # not 3x3x3
     assert not c3.weight_grad_batchable((1, 32, 4, 8, 32), (32, 32, 3, 3, 3), 2, 1, 1, dtype)        # strided
     assert not c3.weight_grad_batchable((1, 48, 4, 8, 32), (32, 48, 3, 3, 3), 1, 1, 1, dtype)        # channels off the grid
     assert not c3.weight_grad_batchable((1, 32, 4, 8, 32), (32, 32, 3, 3, 3), 1, 1, 1, torch.float32)
-    problems, _ = _make([ok, (1, 32, 32, (4, 8, 16), (1, 1, 1), 0)], dtype, device)
+    problems, _ = _make([ok, (1, 32, 32, (40, 64, 16), (1, 1, 1), 0)], dtype, device)
     with pytest.raises(NotImplementedError):
         sa.conv3d_backward_weight_batch(problems)
     # through the C ABI: the list is refused as a whole, with the library's own code, and a short workspace is an error
@@ -185,15 +195,15 @@ def test_backward_pass_with_deferred_weight_gradients(device, master):
 
 
 def test_flush_by_hand_and_unbatchable_weights_are_computed_in_place(device):
-    """A convolution the batch does not serve (rows of 16 voxels) computes its gradient in its own node although the flag is
-    set; a queue left by a pass that raised is emptied by ``flush_weight_gradients()``."""
+    """A convolution the batch does not serve (rows of 16 voxels, 160 tiles) computes its gradient in its own node although
+    the flag is set; a queue left by a pass that raised is emptied by ``flush_weight_gradients()``."""
     torch.manual_seed(1)
     conv = sa.FastConv3d(32, 32, 3, padding=1, bias=False).to(device).to(torch.bfloat16).to(memory_format=CL)
     conv.defer_weight_grad = True
-    x = torch.randn(1, 32, 4, 8, 16, device=device, dtype=torch.bfloat16).contiguous(memory_format=CL).requires_grad_()
+    x = torch.randn(1, 32, 40, 64, 16, device=device, dtype=torch.bfloat16).contiguous(memory_format=CL).requires_grad_()
     conv(x).sum().backward()
     assert conv.weight.grad is not None and not modules._WEIGHT_GRAD_QUEUE
-    ref = sa.conv3d_backward_weight(x.detach(), conv.weight.shape, torch.ones(1, 32, 4, 8, 16, device=device, dtype=torch.bfloat16), 1, 1, 1)
+    ref = sa.conv3d_backward_weight(x.detach(), conv.weight.shape, torch.ones(1, 32, 40, 64, 16, device=device, dtype=torch.bfloat16), 1, 1, 1)
     assert torch.equal(conv.weight.grad, ref)
     # a queued entry that no callback took: flush by hand
     conv.weight.grad = None
