@@ -280,6 +280,8 @@ typedef struct sfh_conv3d_wgrad_item {
   const void* gy;
   void* gw;             /* [Cout][3][3][3][Cin] dense */
 } sfh_conv3d_wgrad_item;
+/* 0: not served in a batch; 1: served, in the launch of the problems with rows of more than 16 voxels; 2: served, in the
+ * launch of the small-volume problems (a caller with more than SFH_WGRAD_BATCH_MAX problems fills its calls by family). */
 int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dtype);
 size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype); /* pointers unused; 0: refused */
 int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, void* workspace,

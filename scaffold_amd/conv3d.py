@@ -898,11 +898,20 @@ def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] 
         keep.append((prob, x, x2, g))
         gws.append(gw)
     flags = _lib.SFH_FLAG_GRAD_FP32 if (grad_dtype is not None and grad_dtype is not dt) else 0
+    # calls of at most WGRAD_BATCH_MAX problems, filled family by family (the problems of a family share a launch)
+    family = [int(L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(k[0].desc), k[0].code)) for k in keep]
+    if 0 in family:
+        raise NotImplementedError(f"conv3d_backward_weight_batch: problem {family.index(0)} of the list is not served in a batch "
+                                  "(weight_grad_batchable says which)")
+    calls = []
+    for f in (1, 2):
+        members = [i for i in range(len(keep)) if family[i] == f]
+        calls += [members[lo:lo + WGRAD_BATCH_MAX] for lo in range(0, len(members), WGRAD_BATCH_MAX)]
     with _lib.device_guard(dev):
-        for lo in range(0, len(keep), WGRAD_BATCH_MAX):
-            part = keep[lo:lo + WGRAD_BATCH_MAX]
+        for idx in calls:
+            part = [keep[i] for i in idx]
             items = (_lib.WgradItem * len(part))()
-            for it, (prob, x, x2, g), gw in zip(items, part, gws[lo:]):
+            for it, (prob, x, x2, g), gw in zip(items, part, [gws[i] for i in idx]):
                 it.desc = prob.desc
                 it.x, it.x_second, it.cin_first = _lib.ptr(x), (None if x2 is None else _lib.ptr(x2)), (0 if x2 is None else int(x.shape[1]))
                 it.gy, it.gw = _lib.ptr(g), _lib.ptr(gw)

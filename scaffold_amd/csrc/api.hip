@@ -779,7 +779,8 @@ static int wgrad_batch_items(const sfh_conv3d_wgrad_item* items, int32_t count, 
 extern "C" int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dtype) {
   int32_t out[3];
   if (p == nullptr || sfh_conv3d_out_shape(p, out) != SFH_OK || !dtype_ok(dtype)) return 0;
-  return (wgrad_uses_mfma(*p, dtype, out) && mfma_wgrad_batch_applies(wgrad_args(*p, out), dtype)) ? 1 : 0;
+  if (!wgrad_uses_mfma(*p, dtype, out) || !mfma_wgrad_batch_applies(wgrad_args(*p, out), dtype)) return 0;
+  return mfma_wgrad_ring_applies(wgrad_args(*p, out)) ? 1 : 2;
 }
 
 extern "C" size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype) {
