@@ -83,7 +83,9 @@ typedef struct sfh_groupnorm_desc {
  * is 4 floats per group instead of 2), sfh_groupnorm_fwd_from_partials takes the byte size of the records;
  * sfh_groupnorm_fwd_noalloc_prepare, sfh_mfma_ceiling_probe added. fp32 problems of the tiled shape have needed a
  * workspace since 102 (sfh_conv3d_{fwd,dgrad,wgrad}_workspace_bytes are non-zero for them; callers that sized their
- * workspace with those functions are unaffected). */
+ * workspace with those functions are unaffected).
+ * 104: sfh_conv3d_wgrad_batch, sfh_conv3d_wgrad_batch_supported, sfh_conv3d_wgrad_batch_workspace_bytes added;
+ * SFH_KERNEL_SPLIT (6) is a value sfh_conv3d_launch_geometry may report. Nothing removed or changed. */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */

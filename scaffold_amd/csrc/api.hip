@@ -280,7 +280,7 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restric
 
 using namespace sfh;
 
-extern "C" int sfh_version(void) { return 103; }
+extern "C" int sfh_version(void) { return 104; }
 
 extern "C" const char* sfh_last_error(void) { return g_error; }
 
