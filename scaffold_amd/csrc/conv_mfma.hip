@@ -339,7 +339,7 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(PackJob first, PackJob
 }
 
 // Many packings in one launch: a workgroup finds its job from the table of first workgroups.
-constexpr int kPackBatch = 16;
+constexpr int kPackBatch = 40;  // (the table stays under 4 KB of kernel arguments)
 struct PackBatch {
   PackJob job[kPackBatch];
   int first_block[kPackBatch + 1];

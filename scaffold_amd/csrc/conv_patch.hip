@@ -405,9 +405,9 @@ int launch_reduce(const PatchArgs& a, const void* small, const void* big, void* 
     hipLaunchKernelGGL((patch_reduce_kernel<T, false>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)big, (float*)ws, total,
                        p.per_split, (float*)nullptr);
   if (int rc = check_launch("patch_reduce_kernel")) return rc;
-  if (int rc = sum_slices(g_dtype, (const float*)ws, g, nelem, p.splits, st)) return rc;
-  if (gb == nullptr) return SFH_OK;
-  return sum_slices(g_dtype, bias_part, gb, a.cbig, p.splits * kTaps, st);  // [split][tap][channel]: slices of cbig elements
+  if (gb == nullptr) return sum_slices(g_dtype, (const float*)ws, g, nelem, p.splits, st);
+  // both sums in one launch; the bias partials are [split][tap][channel]: slices of cbig elements
+  return sum_slices_two(g_dtype, (const float*)ws, g, nelem, p.splits, bias_part, gb, a.cbig, p.splits * kTaps, st);
 }
 
 bool geometry_ok(const PatchArgs& a, int dtype) {

@@ -936,8 +936,8 @@ int dispatch_reduce(const ThinArgs& a, const void* thin, const void* wide, void*
       else if (a.cw == 64) hipLaunchKernelGGL((head_reduce_kernel<T, 2>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per, bias_part);
       else hipLaunchKernelGGL((head_reduce_kernel<T, 4>), grid, dim3(kBlock), 0, st, a, (const T*)thin, (const T*)wide, (float*)ws, total, per, bias_part);
       if (int rc = check_launch("head_reduce_kernel")) return rc;
-      if (int rc = sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st)) return rc;
-      return gb != nullptr ? sum_slices(gw_dtype, bias_part, gb, a.J, nsplit, st) : SFH_OK;
+      if (gb == nullptr) return sum_slices(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, st);
+      return sum_slices_two(gw_dtype, (const float*)ws, gw, (int64_t)a.J * a.cw, nsplit, bias_part, gb, a.J, nsplit, st);
     }
   }
   if (a.K == 3) return launch_reduce<T, 3, 27>(a, thin, wide, gw, gw_dtype, ws, st);

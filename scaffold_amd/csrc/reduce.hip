@@ -11,9 +11,9 @@ namespace {
 constexpr int kBlock = 256;
 
 template <typename T>
-__global__ void __launch_bounds__(kBlock) sum_slices_flat(const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
+__device__ __forceinline__ void sum_slices_flat_body(unsigned block, const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
                                                           int splits) {
-  const int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int64_t e = (int64_t)block * kBlock + threadIdx.x;
   if (e >= nelem) return;
   float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
   int sp = 0;
@@ -30,11 +30,11 @@ __global__ void __launch_bounds__(kBlock) sum_slices_flat(const float* __restric
 // Many slices, few elements: 16 elements x 16 slice lanes per workgroup; lane l sums slices l, l+16, ...
 // and the 16 lane totals are added in lane order.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) sum_slices_grouped(const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
+__device__ __forceinline__ void sum_slices_grouped_body(unsigned block, const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
                                                              int splits) {
   __shared__ float buf[16][17];
   const int el = threadIdx.x & 15, sl = threadIdx.x >> 4;
-  const int64_t e = (int64_t)blockIdx.x * 16 + el;
+  const int64_t e = (int64_t)block * 16 + el;
   float s = 0.f;
   if (e < nelem) {
     // eight loads in flight per thread; the additions keep the slice order
@@ -61,11 +61,11 @@ __global__ void __launch_bounds__(kBlock) sum_slices_grouped(const float* __rest
 // The same with four consecutive elements per thread: a workgroup reads 256 contiguous bytes of each slice (whole
 // cache lines) with 16-byte loads. 64 elements x 16 slice lanes per workgroup.
 template <typename T>
-__global__ void __launch_bounds__(kBlock) sum_slices_grouped4(const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
+__device__ __forceinline__ void sum_slices_grouped4_body(unsigned block, const float* __restrict__ part, T* __restrict__ out, int64_t nelem,
                                                               int splits) {
   __shared__ float4 buf[16][17];
   const int el = threadIdx.x & 15, sl = threadIdx.x >> 4;
-  const int64_t e = ((int64_t)blockIdx.x * 16 + el) * 4;
+  const int64_t e = ((int64_t)block * 16 + el) * 4;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   if (e < nelem) {
     int sp = sl;
@@ -99,10 +99,10 @@ __global__ void __launch_bounds__(kBlock) sum_slices_grouped4(const float* __res
 // flight, then a fixed tree over the 256 thread totals. (With 16 slice lanes per element a lane walked 2048 slices:
 // 12.7 us for 4 MB.)
 template <typename T>
-__global__ void __launch_bounds__(kBlock) sum_slices_tall(const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
+__device__ __forceinline__ void sum_slices_tall_body(unsigned block, const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
   __shared__ float buf[kBlock];
   const int tid = threadIdx.x;
-  const int64_t e = blockIdx.x;
+  const int64_t e = block;
   float s = 0.f;
   int sp = tid;
   for (; sp + 7 * kBlock < splits; sp += 8 * kBlock) {
@@ -120,6 +120,61 @@ __global__ void __launch_bounds__(kBlock) sum_slices_tall(const float* __restric
     __syncthreads();
   }
   if (tid == 0) out[e] = elem<T>::from_float(buf[0]);
+}
+
+// What launch_sum picks for a job: the kernel body and its number of workgroups.
+enum SumKind { kSumNone = 0, kSumTall, kSumGrouped4, kSumGrouped, kSumFlat };
+struct SumJob {
+  const float* part;
+  void* out;
+  int64_t nelem;
+  int splits, kind;
+  unsigned blocks;
+};
+
+inline SumJob sum_job(const float* part, void* out, int64_t nelem, int splits) {
+  SumJob j{part, out, nelem, splits, kSumNone, 0u};
+  if (nelem <= 0) return j;
+  if (nelem <= 64 && splits >= 2048) { j.kind = kSumTall; j.blocks = (unsigned)nelem; }
+  else if (splits >= 32 && nelem <= (1 << 22) && nelem % 4 == 0 && nelem >= 64 * 128 && (reinterpret_cast<uintptr_t>(part) & 15) == 0) {
+    j.kind = kSumGrouped4; j.blocks = (unsigned)cdiv(nelem, 64);
+  } else if (splits >= 32 && nelem <= (1 << 22)) { j.kind = kSumGrouped; j.blocks = (unsigned)cdiv(nelem, 16); }
+  else { j.kind = kSumFlat; j.blocks = (unsigned)cdiv(nelem, kBlock); }
+  return j;
+}
+
+template <typename T>
+__device__ __forceinline__ void sum_job_body(const SumJob& j, unsigned block) {
+  switch (j.kind) {
+    case kSumTall: sum_slices_tall_body<T>(block, j.part, (T*)j.out, j.nelem, j.splits); break;
+    case kSumGrouped4: sum_slices_grouped4_body<T>(block, j.part, (T*)j.out, j.nelem, j.splits); break;
+    case kSumGrouped: sum_slices_grouped_body<T>(block, j.part, (T*)j.out, j.nelem, j.splits); break;
+    default: sum_slices_flat_body<T>(block, j.part, (T*)j.out, j.nelem, j.splits); break;
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_flat(const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
+  sum_slices_flat_body<T>(blockIdx.x, part, out, nelem, splits);
+}
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_grouped(const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
+  sum_slices_grouped_body<T>(blockIdx.x, part, out, nelem, splits);
+}
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_grouped4(const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
+  sum_slices_grouped4_body<T>(blockIdx.x, part, out, nelem, splits);
+}
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_tall(const float* __restrict__ part, T* __restrict__ out, int64_t nelem, int splits) {
+  sum_slices_tall_body<T>(blockIdx.x, part, out, nelem, splits);
+}
+// Two sums in one launch (a weight gradient's slices and its bias gradient's): the first a.blocks workgroups run job a,
+// the rest job b, each exactly as a launch of its own would.
+template <typename T>
+__global__ void __launch_bounds__(kBlock) sum_slices_two(SumJob a, SumJob b) {
+  if (blockIdx.x < a.blocks) sum_job_body<T>(a, blockIdx.x);
+  else sum_job_body<T>(b, blockIdx.x - a.blocks);
 }
 
 template <typename T>
@@ -406,6 +461,28 @@ int launch_bias(const void* g, int64_t rows, int C, float* ws, hipStream_t st) {
 }
 
 }  // namespace
+
+int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st);
+
+template <typename T>
+int launch_sum_two(const SumJob& a, const SumJob& b, hipStream_t st) {
+  hipLaunchKernelGGL(sum_slices_two<T>, dim3(a.blocks + b.blocks), dim3(kBlock), 0, st, a, b);
+  return check_launch("sum_slices_two");
+}
+
+int sum_slices_two(int dtype, const float* part_a, void* out_a, int64_t nelem_a, int splits_a, const float* part_b, void* out_b,
+                   int64_t nelem_b, int splits_b, hipStream_t st) {
+  const SumJob a = sum_job(part_a, out_a, nelem_a, splits_a), b = sum_job(part_b, out_b, nelem_b, splits_b);
+  if (a.kind == kSumNone || b.kind == kSumNone || (uint64_t)a.blocks + b.blocks > 0x7fffffffu) {
+    if (int rc = sum_slices(dtype, part_a, out_a, nelem_a, splits_a, st)) return rc;
+    return sum_slices(dtype, part_b, out_b, nelem_b, splits_b, st);
+  }
+  switch (dtype) {
+    case SFH_BF16: return launch_sum_two<bf16_t>(a, b, st);
+    case SFH_FP16: return launch_sum_two<fp16_t>(a, b, st);
+    default: return launch_sum_two<float>(a, b, st);
+  }
+}
 
 int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st) {
   switch (dtype) {

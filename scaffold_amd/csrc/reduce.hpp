@@ -6,6 +6,9 @@ namespace sfh {
 
 // out[e] = sum over s < splits, in index order within fixed groups, of part[s * nelem + e]; one rounding to `dtype`.
 int sum_slices(int dtype, const float* part, void* out, int64_t nelem, int splits, hipStream_t st);
+// Two such sums from one launch (same bits as two calls of sum_slices).
+int sum_slices_two(int dtype, const float* part_a, void* out_a, int64_t nelem_a, int splits_a, const float* part_b, void* out_b,
+                   int64_t nelem_b, int splits_b, hipStream_t st);
 
 // out[e] = bias[e % channels] + sum over s < splits, in index order, of part[s * nelem + e]; nelem a multiple of 4.
 // `out2` (optional): the result as two tensors cut at channel out2->first of every row of `channels`.
