@@ -536,12 +536,14 @@ def bench_unet_step(args, device, eager_only=False):
     bf16 autocast, fp32 master weights, fused CE + Dice loss head, gradient clipping at 1.0 fused with the Adam update.
 
     Timed eagerly (how the reference's trainer runs) and, when the replay check passes, as a captured HIP graph
-    of the whole step: the eager step is bound by ~600 Python-side launches, not by the GPU."""
+    of the whole step: on boxes with slow host cores the eager step is bound by its ~280 Python-side launches, not by the GPU."""
     import scaffold_amd as sa
 
     occ, lab = ifs_shard()
     occupancy = float(occ.mean())
     occ, lab = occ.contiguous(memory_format=CL).to(device), lab.to(device)
+    # what the data loader hands over on the device: the float32 volume and the int16 mask (ScaFFold/utils/trainer.py:575-583)
+    mask16 = lab.to(torch.int16)
 
     def make(shard_halo=True):
         torch.manual_seed(UNET_SEED)
@@ -554,11 +556,14 @@ def bench_unet_step(args, device, eager_only=False):
         opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
         return model, opt
 
-    def step_fn(model, opt):
+    def step_fn(model, opt, shard_halo=True):
         def step():
+            # the trainer's device-side conversions of a batch (float32 channels-last volume, int64 labels) and autocast's
+            # rounding of the stem's input in one launch, straight into the slab the stem reads
+            x, labels = sa.ingest(occ, mask16, dtype=torch.bfloat16, out_halo=1 if shard_halo else 0)
             with torch.autocast("cuda", dtype=torch.bfloat16):
-                logits = model(occ)
-            loss = sa.ce_dice_loss(logits, lab)
+                logits = model(x)
+            loss = sa.ce_dice_loss(logits, labels)
             loss.backward()
             opt.step()
             opt.zero_grad(set_to_none=True)  # ScaFFold/utils/trainer.py:694
@@ -576,7 +581,7 @@ def bench_unet_step(args, device, eager_only=False):
     # result): what remains is the cost of the step itself, the difference is the bench's stand-in for DistConv's
     # halo exchange.
     model_p, opt_p = make(shard_halo=False)
-    out["ms_per_step_padded_form"] = event_time_ms(step_fn(model_p, opt_p), 10, warmup=3)
+    out["ms_per_step_padded_form"] = event_time_ms(step_fn(model_p, opt_p, shard_halo=False), 10, warmup=3)
     del model_p, opt_p
 
     # The same step as one HIP graph. Checked before it is reported: from identical initial state, the losses of

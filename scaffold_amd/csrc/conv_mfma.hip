@@ -295,7 +295,8 @@ conv_mfma_kernel(MfmaConvArgs a, const T* __restrict__ x, const T* __restrict__ 
 struct PackJob {
   const void* w;
   void* packed;
-  int cout, cred, kd, kh, kw, flip;
+  int cout, cred;
+  int taps;  // kd | kh << 8 | kw << 16 | flip << 24 (one word: 48 jobs fit a 4 KB table of kernel arguments)
   int64_t s_out, s_red, s_kd, s_kh, s_kw;
   int64_t pieces;
 };
@@ -304,7 +305,8 @@ template <typename T>
 __device__ __forceinline__ void pack_piece(const PackJob& j, int64_t idx) {
   const T* w = static_cast<const T*>(j.w);
   T* packed = static_cast<T*>(j.packed);
-  const int taps = j.kd * j.kh * j.kw;
+  const int kh = (j.taps >> 8) & 0xff, kw = (j.taps >> 16) & 0xff, flip = j.taps >> 24;
+  const int taps = (j.taps & 0xff) * kh * kw;
   int64_t r = idx;
   const int lane = (int)(r % 64); r /= 64;
   const int ks = (int)(r % 2); r /= 2;
@@ -314,8 +316,8 @@ __device__ __forceinline__ void pack_piece(const PackJob& j, int64_t idx) {
   const int nblk = (int)(r / ncc);
   const int co = nblk * 32 + (lane & 31);
   const int ci = cc * kChunk + ks * 16 + (lane >> 5) * 8;
-  if (j.flip) tap = taps - 1 - tap;
-  const int tkw = tap % j.kw, tkh = (tap / j.kw) % j.kh, tkd = tap / (j.kw * j.kh);
+  if (flip) tap = taps - 1 - tap;
+  const int tkw = tap % kw, tkh = (tap / kw) % kh, tkd = tap / (kw * kh);
   const T* src = w + co * j.s_out + ci * j.s_red + tkd * j.s_kd + tkh * j.s_kh + tkw * j.s_kw;
   uint4 v;
   if (j.s_red == 1 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {
@@ -339,12 +341,13 @@ __global__ void __launch_bounds__(256) pack_weight_kernel(PackJob first, PackJob
 }
 
 // Many packings in one launch: a workgroup finds its job from the table of first workgroups.
-constexpr int kPackBatch = 40;  // (the table stays under 4 KB of kernel arguments)
+constexpr int kPackBatch = 48;  // (the table stays under 4 KB of kernel arguments)
 struct PackBatch {
   PackJob job[kPackBatch];
   int first_block[kPackBatch + 1];
   int njobs;
 };
+static_assert(sizeof(PackBatch) <= 4096, "kernel arguments");
 
 template <typename T>
 __global__ void __launch_bounds__(256) pack_weight_batch_kernel(PackBatch b) {
@@ -513,7 +516,7 @@ PackJob pack_job(const MfmaConvArgs& a, const void* w, int64_t s_out, int64_t s_
                  void* packed) {
   PackJob j{};
   j.w = w; j.packed = packed;
-  j.cout = a.cout; j.cred = a.cred; j.kd = a.kd; j.kh = a.kh; j.kw = a.kw; j.flip = flip;
+  j.cout = a.cout; j.cred = a.cred; j.taps = a.kd | (a.kh << 8) | (a.kw << 16) | ((flip ? 1 : 0) << 24);  // (kernel extents are at most 3)
   j.s_out = s_out; j.s_red = s_red; j.s_kd = s_kd; j.s_kh = s_kh; j.s_kw = s_kw;
   j.pieces = (int64_t)a.cout * a.cred * a.kd * a.kh * a.kw / 8;  // 16-byte pieces
   return j;
