@@ -173,58 +173,6 @@ __global__ void __launch_bounds__(64) ce_dice_sum(const float* __restrict__ part
   }
 }
 
-// The two kernels below in one launch for few quantities (one or two samples): sixteen wavefronts take the quantities in
-// turn -- each exactly as ce_dice_sum's workgroup would -- and leave them in stats and in LDS; the first wavefront then
-// does ce_dice_scalar's arithmetic from the LDS copy. Same bits as the pair of launches.
-constexpr int kFusedQuantities = 96;
-__global__ void __launch_bounds__(1024) ce_dice_sum_scalar(const float* __restrict__ part, float* __restrict__ stats, float* __restrict__ loss,
-                                                           int N, int C, int nsplit, int unweighted, float count, float eps) {
-  __shared__ float held[kFusedQuantities];
-  const int Q = 3 * C + 2, total = N * 3 * C + 2;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int b = wave; b < total; b += 16) {
-    float s;
-    int dst;
-    if (b < N * 3 * C) {
-      const int n = b / (3 * C), q = b - n * 3 * C;
-      s = lane_slots_sum(part + (int64_t)n * nsplit * Q + q, nsplit, Q, lane);
-      dst = (q / C) * N * C + n * C + q % C;
-    } else {
-      const int q = 3 * C + (b - N * 3 * C);
-      s = lane_slots_sum(part + q, N * nsplit, Q, lane);
-      dst = b;
-    }
-    s = wave_sum_all(s);
-    if (lane == 0) {
-      if (b == N * 3 * C + 1 && unweighted) s = count;
-      stats[dst] = s;
-      held[dst] = s;
-    }
-  }
-  __syncthreads();
-  if (wave != 0) return;
-  const float* inter = held;
-  const float* psum = held + N * C;
-  const float* tsum = held + 2 * N * C;
-  const float ce_sum = held[N * 3 * C], normaliser = held[N * 3 * C + 1];
-  float dice = 0.f;
-  for (int i = lane; i < N * C; i += 64) {
-    const int c = i % C;
-    if (c >= 1) {
-      const float two_i = 2.f * inter[i];
-      float sets = psum[i] + tsum[i];
-      if (sets == 0.f) sets = two_i;
-      dice += (two_i + eps) / (sets + eps);
-    }
-  }
-  dice = wave_sum_all(dice);
-  if (lane == 0) {
-    dice /= (float)(N * (C - 1));
-    const float ce = ce_sum / fmaxf(normaliser, 1.1920929e-07f);
-    loss[0] = ce + (1.f - dice);
-  }
-}
-
 __global__ void __launch_bounds__(64) ce_dice_scalar(const float* __restrict__ stats, float* __restrict__ loss, int N, int C, float eps) {
   // one lane per (sample, foreground class) pass; the Dice terms meet in the fixed wavefront tree
   const float* inter = stats;
@@ -360,11 +308,6 @@ int fwd_typed(const sfh_loss_desc& p, const void* logits, const int64_t* labels,
   hipLaunchKernelGGL((ce_dice_partial<T, CMAX>), dim3(pl.nsplit, p.n), dim3(kBlock), lds, st, (const T*)logits, labels, cw, ws,
                      p.spatial, p.classes, pl.nsplit, pl.per_split, tiles_on_16_bytes<T>(p, logits, nullptr));
   if (int rc = check_launch("ce_dice_partial")) return rc;
-  if (p.n * 3 * p.classes + 2 <= kFusedQuantities) {
-    hipLaunchKernelGGL(ce_dice_sum_scalar, dim3(1), dim3(1024), 0, st, ws, stats, loss, p.n, p.classes, pl.nsplit, cw == nullptr ? 1 : 0,
-                       (float)p.n * (float)p.spatial, p.eps);
-    return check_launch("ce_dice_sum_scalar");
-  }
   hipLaunchKernelGGL(ce_dice_sum, dim3(p.n * 3 * p.classes + 2), dim3(64), 0, st, ws, stats, p.n, p.classes, pl.nsplit,
                      cw == nullptr ? 1 : 0, (float)p.n * (float)p.spatial);
   if (int rc = check_launch("ce_dice_sum")) return rc;

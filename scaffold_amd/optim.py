@@ -91,11 +91,27 @@ class FusedClipAdam(torch.optim.Optimizer):
     def _state_of(self, p):
         st = self.state[p]
         if not st:
-            st["step"] = torch.zeros((), dtype=torch.float32, device=p.device)
+            # One counter tensor for all parameters whose state is created before the first step (torch keeps one per
+            # parameter, all equal; state_dict() shows the same values either way): the kernels advance it once, and
+            # no multi-tensor add is needed for the others.
+            fresh = self.__dict__.get("_fresh_step")
+            if fresh is None or fresh[0].device != p.device or fresh[1]:
+                fresh = self._fresh_step = [torch.zeros((), dtype=torch.float32, device=p.device), False]
+            st["step"] = fresh[0]
             st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
             st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
         self._check_state(p, st)
         return st
+
+    @staticmethod
+    def _other_steps(states):
+        """The step tensors that are not the first parameter's, each once."""
+        seen, out = {id(states[0]["step"])}, []
+        for st in states[1:]:
+            if id(st["step"]) not in seen:
+                seen.add(id(st["step"]))
+                out.append(st["step"])
+        return out
 
     def _plan(self, active, device):
         """Pointer tables of everything that does not move between steps (parameters, moments, shadow copies),
@@ -114,7 +130,7 @@ class FusedClipAdam(torch.optim.Optimizer):
         numel = (ctypes.c_int64 * len(params))(*[p.numel() for p in params])
         plan = {
             "params": params, "states": states, "numel": numel, "nslots": int(L.sfh_adam_slots(len(params), numel)),
-            "others": [st["step"] for st in states[1:]], "groups": [],
+            "others": self._other_steps(states), "groups": [],
         }
         for group in self.param_groups:
             idx = [i for i, (g, _) in enumerate(active) if g is group]
@@ -161,6 +177,9 @@ class FusedClipAdam(torch.optim.Optimizer):
             # per parameter, all equal, and a checkpoint must hold them as separate tensors: the others are advanced
             # by one multi-tensor add.
             step = states[0]["step"]
+            fresh = self.__dict__.get("_fresh_step")
+            if fresh is not None:
+                fresh[1] = True  # stepped: parameters that join later get a counter of their own
             if plan["others"]:
                 torch._foreach_add_(plan["others"], 1.0)
             nslots = plan["nslots"]
@@ -210,6 +229,14 @@ class FusedClipAdam(torch.optim.Optimizer):
                 e.version = p._version
                 e.maintained = True
 
+    def state_dict(self):
+        """As ``torch.optim.Optimizer.state_dict``; every parameter's ``step`` is a tensor of its own there (inside the
+        optimizer the parameters share one), so that a consumer which advances them one by one -- ``torch.optim.Adam``
+        after ``load_state_dict`` -- counts right."""
+        sd = super().state_dict()
+        sd["state"] = {k: (dict(v, step=v["step"].clone()) if torch.is_tensor(v.get("step")) else v) for k, v in sd["state"].items()}
+        return sd
+
     def load_state_dict(self, state_dict):
         """As ``torch.optim.Optimizer.load_state_dict``, then the state is brought into the form the kernels read.
 
@@ -238,6 +265,16 @@ class FusedClipAdam(torch.optim.Optimizer):
                     st[k] = self._like_param(p, st[k], k)
         if len(steps) > 1:
             raise NotImplementedError(f"FusedClipAdam: the kernels keep one step counter for all parameters, the loaded state has {sorted(steps)}")
+        # all equal: one tensor serves every parameter again
+        shared = None
+        for group in self.param_groups:
+            for p in group["params"]:
+                st = self.state.get(p)
+                if st:
+                    if shared is None or shared.device != st["step"].device:
+                        shared = st["step"]
+                    st["step"] = shared
+        self._fresh_step = None
 
     @staticmethod
     def _like_param(p, t, what):
