@@ -768,7 +768,11 @@ bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, siz
   }
   b.total = (int)pos;
   b.quads = (int)quads;
-  b.wgs = b.total < kComputeUnits ? b.total : kComputeUnits;
+  // one workgroup per CU, fewer when that would leave a workgroup less than two columns' start cost of positions (a range
+  // without a step still costs its block a slice of zeros)
+  b.wgs = b.total / (2 * kFillCost);
+  if (b.wgs > kComputeUnits) b.wgs = kComputeUnits;
+  if (b.wgs < 1) b.wgs = 1;
   ws_bytes = 0;
   for (int i = 0; i < count; ++i) {
     WRingBatchEntry& e = b.e[i];
