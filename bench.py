@@ -693,6 +693,64 @@ def conv_table(device, iters=20):
     return rows
 
 
+#: the 17 3x3x3 convolutions of the config-5 step that have a weight gradient on the matrix cores, in the order the
+#: backward pass meets them (decoder level 0 first): (Cin, Cout, interior extents, input given as two tensors)
+CFG5_WGRADS = (
+    [(32, 32, (64, 128, 128), False), (64, 32, (64, 128, 128), True)]
+    + [(64, 64, (32, 64, 64), False), (128, 64, (32, 64, 64), True)]
+    + [(128, 128, (16, 32, 32), False), (256, 128, (16, 32, 32), True)]
+    + [(256, 256, (8, 16, 16), False), (512, 256, (8, 16, 16), True)]
+    + [(512, 512, (4, 8, 8), False), (256, 512, (4, 8, 8), False)]
+    + [(256, 256, (8, 16, 16), False), (128, 256, (8, 16, 16), False)]
+    + [(128, 128, (16, 32, 32), False), (64, 128, (16, 32, 32), False)]
+    + [(64, 64, (32, 64, 64), False), (32, 64, (32, 64, 64), False)]
+    + [(32, 32, (64, 128, 128), False)]
+)
+
+
+def bench_wgrad_batch(device, iters=6):
+    """The weight gradients of one config-5 backward pass (CFG5_WGRADS, slab form, fp32 gradients): as 17 calls of
+    conv3d_backward_weight (one launch and one sum pass each) and as one conv3d_backward_weight_batch (two launches and
+    one sum pass); each form captured as a graph, HIP events. FLOPs 2 * voxels * Cin * Cout * 27 summed over the list."""
+    import scaffold_amd as sa
+    from scaffold_amd import conv3d as c3
+
+    problems, flops = [], 0
+    for i, (cin, cout, sp, pair) in enumerate(CFG5_WGRADS):
+        g = torch.Generator().manual_seed(7000 + i)
+        x = torch.randn((1, cin, sp[0] + 2, sp[1], sp[2]), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+        gy = torch.randn((1, cout, *sp), generator=g).to(torch.bfloat16).contiguous(memory_format=CL).to(device)
+        inp = (x[:, :cin // 2].contiguous(memory_format=CL), x[:, cin // 2:].contiguous(memory_format=CL)) if pair else x
+        problems.append((inp, (cout, cin, 3, 3, 3), gy, (0, 1, 1)))
+        flops += 2 * math.prod(sp) * cin * cout * 27
+
+    def separate():
+        out = []
+        for inp, ws, gy, pad in problems:
+            if isinstance(inp, tuple):
+                out.append(c3.conv3d_backward_weight_pair(inp[0], inp[1], ws, gy, 1, pad, 1, grad_dtype=torch.float32))
+            else:
+                out.append(sa.conv3d_backward_weight(inp, ws, gy, 1, pad, 1, grad_dtype=torch.float32))
+        return out
+
+    def batched():
+        return sa.conv3d_backward_weight_batch(problems, grad_dtype=torch.float32)
+
+    a, b = separate(), batched()
+    torch.cuda.synchronize()
+    worst = max(float((p.double() - q.double()).abs().max() / p.double().abs().max()) for p, q in zip(a, b))
+    del a, b
+    out = {"problems": len(problems), "gflop": flops / 1e9, "max_rel_difference_between_the_forms": worst}
+    for name, fn in (("separate", separate), ("batched", batched)):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        ms = event_time_ms(graph.replay, iters, warmup=2)
+        out[name + "_us"] = ms * 1e3
+        out[name + "_frac_of_mfma_peak"] = flops / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS
+    return out
+
+
 def conv_counter_launches(device, reps=3):
     """The launches a counter run (rocprofv3 --pmc) is taken over: plain eager calls, no graph, of the three MFMA
     convolution kernels on the shapes their roofline fractions are quoted for -- 32->32 @128^3 (conv_ring_kernel,
@@ -934,7 +992,11 @@ def main():
         for r in rows:
             print(f"{r['form']:17s} {r['cin']:4d}->{r['cout']:<4d} {'x'.join(str(v) for v in r['spatial']):>11s} {r['direction']:6s} "
                   f"{r['us']:8.1f} us {r['gflop']:8.2f} GFLOP {r['tflops']:7.1f} TFLOP/s {r['frac']:.3f}", file=sys.stderr)
-        print(json.dumps({"conv_table": rows}))
+        wb = bench_wgrad_batch(device)
+        print(f"weight gradients of one config-5 backward pass ({wb['problems']} problems, {wb['gflop']:.1f} GFLOP): one launch pair each "
+              f"{wb['separate_us']:.1f} us ({wb['separate_frac_of_mfma_peak']:.3f} of peak), batched {wb['batched_us']:.1f} us "
+              f"({wb['batched_frac_of_mfma_peak']:.3f})", file=sys.stderr)
+        print(json.dumps({"conv_table": rows, "wgrad_batch_cfg5": wb}))
         return
     if args.conv_counters:
         print(json.dumps({"conv_counter_launches": conv_counter_launches(device)}))
@@ -990,6 +1052,10 @@ def main():
         details["shard_ingest"] = bench_ingest(args, device)
     except Exception as exc:  # report, do not hide
         details["shard_ingest"] = {"error": repr(exc)}
+    try:
+        details["wgrad_batch_cfg5"] = bench_wgrad_batch(device)
+    except Exception as exc:  # report, do not hide
+        details["wgrad_batch_cfg5"] = {"error": repr(exc)}
     if not args.skip_unet:
         try:
             details["unet_step_cfg5"] = bench_unet_step(args, device)
