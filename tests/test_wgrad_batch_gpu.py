@@ -213,3 +213,61 @@ def test_flush_by_hand_and_unbatchable_weights_are_computed_in_place(device):
     modules.flush_weight_gradients()
     assert not modules._WEIGHT_GRAD_QUEUE
     assert torch.equal(conv.weight.grad, sa.conv3d_backward_weight_batch([(x2, conv.weight.shape, gy, (1, 1, 1))])[0])
+
+
+def test_deferred_step_as_a_hip_graph_and_under_checkpointing(device):
+    """The step with deferred weight gradients (fused clip + Adam keeping the bf16 copies) captured once and replayed gives
+    the eager step's losses from the same state, replay after replay; and with activation checkpointing the nested backward
+    passes flush their own queues: same gradients as without."""
+    x = torch.randn(1, 1, 8, 32, 64, device=device).contiguous(memory_format=CL)
+    target = torch.randint(0, 3, (1, 8, 32, 64), device=device)
+
+    def make():
+        net = _tiny_net(device, defer=True)
+        opt = sa.FusedClipAdam(net.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+
+        def step():
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                logits = net(x)
+            loss = sa.ce_dice_loss(logits, target)
+            loss.backward()
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+            return loss.detach()
+        return net, opt, step
+
+    _, _, eager = make()
+    want = [eager().item() for _ in range(4)]
+    net2, opt2, step2 = make()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        warm = step2().item()  # the first step eagerly (libraries initialise, the optimizer state appears), the second captured
+    torch.cuda.current_stream().wait_stream(side)
+    assert warm == want[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = step2()
+    got = []
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        got.append(static_loss.item())
+        torch.randn(1 << 16, device=device).sum().item()
+    assert got == want[1:]
+    assert not modules._WEIGHT_GRAD_QUEUE
+
+    grads = {}
+    for ckpt in (False, True):
+        net = _tiny_net(device, defer=True)
+        opt = sa.FusedClipAdam(net.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+        if ckpt:
+            net.use_checkpointing()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = net(x.clone().requires_grad_(True) if ckpt else x)
+        sa.ce_dice_loss(logits, target).backward()
+        assert not modules._WEIGHT_GRAD_QUEUE
+        grads[ckpt] = {n: p.grad.detach().clone() for n, p in net.named_parameters()}
+    for n, g in grads[False].items():
+        d = grads[True][n].float()
+        assert (g.float() - d).abs().max().item() <= 2e-2 * max(g.float().abs().max().item(), 1e-30), n
