@@ -507,12 +507,13 @@ __device__ __forceinline__ void wring_run(const WgradArgs& a, const T* __restric
 // A launch of the kernel above costs the same whatever the problem: every workgroup fetches its first two steps at once
 // (all CUs asking together: 4.4 us), at the end every workgroup writes its 110 KB slice at once (6-7 us), a sum pass
 // reads the 256 slices back (6 us), and two launches start. A batch pays that once for all its problems. All blocks of
-// all problems lie on one line of cost -- problem after problem, inside a problem block after block, inside a block
-// column after column, a column being kFillCost positions for the ring's start and one per step -- and workgroup w of W
-// takes the positions [w total / W, (w + 1) total / W): whole columns, parts of columns, blocks of several problems. For
-// every block it touches it walks its steps of the block's columns, hands its accumulators over and writes a slice:
-// slice number w - (the first workgroup that touches the block). The sum pass knows from the same arithmetic how many
-// slices a block has. The cut is a pure function of the list of problems; nothing is added atomically.
+// all problems lie on one line of cost -- problem after problem, inside a problem in UNITS (a chunk of columns of one
+// 32 x 32 block, see batch_unit), inside a unit column after column, a column being kFillCost positions for the ring's
+// start and one per step -- and workgroup w of W takes the positions [w total / W, (w + 1) total / W): whole columns,
+// parts of columns, units of several blocks and problems. For every unit it touches it walks its steps of the unit's
+// columns, hands its accumulators over and writes a slice of the unit's block: slice number (the block's slices from
+// earlier units) + w - (the first workgroup that touches the unit). The sum pass knows from the same arithmetic how
+// many slices a block has. The cut is a pure function of the list of problems; nothing is added atomically.
 constexpr int kFillCost = 4;  // (the captured U-Net step: 2 -> 4 is 20 us faster, 4, 6 and 8 are alike)
 
 struct WRingBatchEntry {
@@ -525,6 +526,7 @@ struct WRingBatchEntry {
   int c_first;
   int tiles_h, tiles_w, steps, nblk_ci, nblk;
   int ncols;            // columns of a block
+  int chunk;            // columns of a unit: the line runs [chunk of columns][block][column], see batch_unit
   int pos_begin;        // the problem's first position on the line
   int slices;           // the most slices any of its blocks gets
   int quad_begin;       // the problem's first float4 in the sum pass (a multiple of 256)
@@ -545,6 +547,39 @@ __host__ __device__ __forceinline__ int batch_owner(int q, int total, int wgs) {
   return w;
 }
 
+// Inside a problem the line runs chunk of columns after chunk, inside a chunk block after block, inside a block's
+// chunk -- a UNIT -- column after column. A chunk is about one workgroup's range, so the workgroups that walk the same
+// columns for the problem's different 32 x 32 blocks are neighbours (same XCD) and do it at the same time: what one
+// fetches of a 128-byte line of a 64-channel tensor, the other finds in L2. (Block after block over all columns, the
+// launch fetched 1.9 times the bytes of the one-problem launches, FETCH_SIZE, and ran its level-1 steps a third slower.)
+struct WUnit {
+  int blk, col0, cols, begin;  // block, first column, columns, first position
+};
+__host__ __device__ __forceinline__ WUnit batch_unit(int rel, int pos_begin, int nblk, int ncols, int chunk, int colcost) {
+  const int nfull = ncols / chunk, uc = chunk * colcost, span = nfull * nblk * uc;
+  WUnit u;
+  if (rel < span) {
+    const int i = rel / uc;
+    u.blk = i % nblk; u.col0 = (i / nblk) * chunk; u.cols = chunk; u.begin = pos_begin + i * uc;
+  } else {
+    const int rest = ncols - nfull * chunk, ur = rest * colcost, i = (rel - span) / ur;
+    u.blk = i; u.col0 = nfull * chunk; u.cols = rest; u.begin = pos_begin + span + i * ur;
+  }
+  return u;
+}
+// Slices of block `blk` that belong to its first `chunks` units: each unit has one slice per workgroup that touches it.
+__host__ __device__ __forceinline__ int batch_slices_before(int blk, int chunks, int pos_begin, int nblk, int ncols, int chunk, int colcost,
+                                                            int total, int wgs) {
+  const int nfull = ncols / chunk, uc = chunk * colcost;
+  int n = 0;
+  for (int k = 0; k < chunks; ++k) {
+    const int cols = k < nfull ? chunk : ncols - nfull * chunk;
+    const int begin = k < nfull ? pos_begin + (k * nblk + blk) * uc : pos_begin + nfull * nblk * uc + blk * cols * colcost;
+    n += batch_owner(begin + cols * colcost - 1, total, wgs) - batch_owner(begin, total, wgs) + 1;
+  }
+  return n;
+}
+
 template <typename T, int G>
 __device__ __forceinline__ void wring_batch_run(const WRingBatch& b, int w, int tid, const WRingLds& m) {
   constexpr int NACC = G == 0 ? kTaps0 : kTaps1;
@@ -560,10 +595,10 @@ __device__ __forceinline__ void wring_batch_run(const WRingBatch& b, int w, int 
       if (pos >= b.e[k].pos_begin) p = k;
     const WgradArgs a = b.e[p].a;
     const int steps = b.e[p].steps, nblk_ci = b.e[p].nblk_ci, tiles_h = b.e[p].tiles_h, tiles_w = b.e[p].tiles_w;
-    const int colcost = steps + kFillCost, blockcost = b.e[p].ncols * colcost;
-    const int blk = (pos - b.e[p].pos_begin) / blockcost;
-    const int b0 = b.e[p].pos_begin + blk * blockcost;
-    const int seg_hi = hi < b0 + blockcost ? hi : b0 + blockcost;
+    const int colcost = steps + kFillCost, chunk = b.e[p].chunk;
+    const WUnit u = batch_unit(pos - b.e[p].pos_begin, b.e[p].pos_begin, b.e[p].nblk, b.e[p].ncols, chunk, colcost);
+    const int blk = u.blk, b0 = u.begin, unit_end = u.begin + u.cols * colcost;
+    const int seg_hi = hi < unit_end ? hi : unit_end;
     const int cib = blk % nblk_ci, cob = blk / nblk_ci;
     const T* xs = (const T*)b.e[p].x;
     int x_cin = a.cin, cis = cib;
@@ -586,11 +621,12 @@ __device__ __forceinline__ void wring_batch_run(const WRingBatch& b, int w, int 
       if (s_begin < 0) s_begin = 0;
       if (s_end > steps) s_end = steps;
       if (s_end > s_begin)
-        wring_segment<T, G>(a, xs + (cis - cib) * 32, gy, wring_column(c, tiles_h, tiles_w), s_begin, s_end - s_begin, cib, cob, x_cin, ln,
-                            wave, acc, gyf, fr, m);
+        wring_segment<T, G>(a, xs + (cis - cib) * 32, gy, wring_column(u.col0 + c, tiles_h, tiles_w), s_begin, s_end - s_begin, cib, cob,
+                            x_cin, ln, wave, acc, gyf, fr, m);
       q = first_step + steps;
     }
-    const int slice = w - batch_owner(b0, b.total, b.wgs);
+    const int slice = batch_slices_before(blk, u.col0 / chunk, b.e[p].pos_begin, b.e[p].nblk, b.e[p].ncols, chunk, colcost, b.total, b.wgs) +
+                      (w - batch_owner(b0, b.total, b.wgs));
     wring_handover<G, true>(acc, b.e[p].ws + ((int64_t)slice * a.cout + cob * 32) * 27 * a.cin + cib * 32, a.cin, tid, m);
     pos = seg_hi;
   }
@@ -628,9 +664,9 @@ __global__ void __launch_bounds__(256) wgrad_ring_batch_sum(WRingBatch b) {
   if (el >= nelem) return;
   const int ci = (int)(el % (uint32_t)cin), co = (int)(el / (27u * (uint32_t)cin));
   const int blk = (co / 32) * b.e[p].nblk_ci + ci / 32;
-  const int blockcost = b.e[p].ncols * (b.e[p].steps + kFillCost);
-  const int b0 = b.e[p].pos_begin + blk * blockcost;
-  const int n = batch_owner(b0 + blockcost - 1, b.total, b.wgs) - batch_owner(b0, b.total, b.wgs) + 1;
+  const int chunk = b.e[p].chunk, ncols = b.e[p].ncols;
+  const int n = batch_slices_before(blk, (ncols + chunk - 1) / chunk, b.e[p].pos_begin, b.e[p].nblk, ncols, chunk, b.e[p].steps + kFillCost,
+                                    b.total, b.wgs);
   const float* part = b.e[p].ws + el;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   int sp = 0;
@@ -776,11 +812,16 @@ bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, siz
   ws_bytes = 0;
   for (int i = 0; i < count; ++i) {
     WRingBatchEntry& e = b.e[i];
-    const int blockcost = e.ncols * (e.steps + kFillCost);
+    // a chunk of columns costs about one workgroup's range (a problem of one block is a single run of columns either way;
+    // bending the column-start cost of a problem so that its units are exactly a range long was measured: no better)
+    const int colcost = e.steps + kFillCost, range = b.total / b.wgs;
+    int chunk = (range + colcost / 2) / colcost;
+    if (chunk < 1) chunk = 1;
+    if (chunk > e.ncols || e.nblk == 1) chunk = e.ncols;
+    e.chunk = chunk;
     int most = 1;
     for (int blk = 0; blk < e.nblk; ++blk) {
-      const int b0 = e.pos_begin + blk * blockcost;
-      const int n = batch_owner(b0 + blockcost - 1, b.total, b.wgs) - batch_owner(b0, b.total, b.wgs) + 1;
+      const int n = batch_slices_before(blk, (e.ncols + chunk - 1) / chunk, e.pos_begin, e.nblk, e.ncols, chunk, colcost, b.total, b.wgs);
       if (n > most) most = n;
     }
     e.slices = most;
