@@ -198,6 +198,8 @@ __global__ void __launch_bounds__(256) patch_scatter_kernel(PatchArgs a, const T
     for (; k + 8 <= 2 * nchunks; k += 8) step(k, std::integral_constant<int, 8>{});
   if constexpr (TS == 2)
     for (; k + 4 <= 2 * nchunks; k += 4) step(k, std::integral_constant<int, 4>{});
+  if constexpr (TS == 4)
+    for (; k + 2 <= 2 * nchunks; k += 2) step(k, std::integral_constant<int, 2>{});
   for (; k < 2 * nchunks; ++k) step(k, std::integral_constant<int, 1>{});
   const Voxel vx = decode_small(a, vc);
 #pragma unroll
@@ -365,13 +367,17 @@ int launch_scatter(const PatchArgs& a, const void* small, const void* packed, co
     grid.z = kTaps;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 1>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total, face_pieces, big_elems);
-  } else if (wgs <= 4 * kComputeUnits) {  // up to four per CU: two taps (the big voxels next to each other along W)
+  } else if (wgs < 4 * kComputeUnits) {  // under four per CU: two taps (the big voxels next to each other along W)
     grid.z = kTaps / 2;
     hipLaunchKernelGGL((patch_scatter_kernel<T, 2>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
                        (T*)big, total, face_pieces, big_elems);
   } else {
-    hipLaunchKernelGGL((patch_scatter_kernel<T, kTaps>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed,
-                       (const T*)bias, (T*)big, total, face_pieces, big_elems);
+    // four taps (one big depth plane of the 2 x 2 x 2 patch) per workgroup: eight taps need 295 registers a lane, i.e. one
+    // wavefront per SIMD walking four dependent trips to memory each (31 us at 64 -> 32 on 32 x 64 x 64); with half the
+    // accumulators three wavefronts share a SIMD, and the small tensor read twice costs less than that gains
+    grid.z = 2;
+    hipLaunchKernelGGL((patch_scatter_kernel<T, 4>), grid, dim3(256), 0, st, a, (const T*)small, (const T*)packed, (const T*)bias,
+                       (T*)big, total, face_pieces, big_elems);
   }
   return check_launch("patch_scatter_kernel");
 }
