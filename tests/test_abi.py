@@ -166,6 +166,55 @@ def test_wgrad_split_plan_partitions_the_bricks():
             assert 1 <= splits <= bricks and splits * per >= bricks and (splits - 1) * per < bricks
 
 
+def test_weight_gradient_batch_plan_and_refusals():
+    """The batched weight gradient without a GPU: which problems join which launch, the workspace of a list (a pure
+    function of its shapes, never 0 for a served list), and the refusals that come before any launch."""
+    L = _lib.lib()
+    bf16, fp32 = 0, 2
+    ring = conv_desc(cin=64, cout=32, sp=(18, 32, 64), p=(0, 1, 1))      # rows of more than 16 voxels
+    small = conv_desc(cin=256, cout=256, sp=(10, 16, 16), p=(0, 1, 1))   # a small volume: 8 tiles under a block
+    large16 = conv_desc(cin=32, cout=32, sp=(64, 64, 16))                  # rows of 16 voxels, hundreds of tiles
+    strided = conv_desc(cin=32, cout=32, sp=(8, 8, 32)); strided.sd = 2
+    assert L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(ring), bf16) == 1
+    assert L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(small), bf16) == 2
+    assert L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(large16), bf16) == 0
+    assert L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(strided), bf16) == 0
+    assert L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(ring), fp32) == 0
+    assert L.sfh_conv3d_wgrad_batch_supported(None, bf16) == 0
+
+    def items(*descs):
+        arr = (_lib.WgradItem * len(descs))()
+        for it, d in zip(arr, descs):
+            it.desc = d
+        return arr
+
+    one = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16)
+    two = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, ring), 2, bf16)
+    mixed = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, small), 2, bf16)
+    assert one > 0 and two > 0 and mixed > 0
+    # every workgroup writes one 32 x 32 x 27 fp32 slice per unit it touches: at least a slice a block, a few hundred at most
+    block = 32 * 32 * 27 * 4
+    assert 2 * block <= one <= 1024 * block
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16) == one        # a pure function of the list
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(small, small), 2, bf16) > 0   # nothing needed, still not 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, large16), 2, bf16) == 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 0, bf16) == 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(*([ring] * 17)), 17, bf16) == 0
+    addr = ctypes.c_void_p(256)  # never dereferenced: every call below is refused before a launch
+    bad = items(ring, large16)
+    for it in bad:
+        it.x, it.gy, it.gw = addr, addr, addr
+    assert L.sfh_conv3d_wgrad_batch(bad, 2, bf16, addr, 1 << 30, 0, None) == _lib.SFH_ERR_UNSUPPORTED
+    ok = items(ring)
+    assert L.sfh_conv3d_wgrad_batch(ok, 1, bf16, addr, 1 << 30, 0, None) == _lib.SFH_ERR_INVALID          # null tensors
+    ok[0].x, ok[0].gy, ok[0].gw = addr, addr, addr
+    assert L.sfh_conv3d_wgrad_batch(ok, 1, bf16, addr, one - 256, 0, None) == _lib.SFH_ERR_WORKSPACE
+    assert L.sfh_conv3d_wgrad_batch(ok, 1, bf16, None, 0, 0, None) == _lib.SFH_ERR_WORKSPACE
+    assert L.sfh_conv3d_wgrad_batch(ok, 1, bf16, addr, one, _lib.SFH_FLAG_FORCE_GENERIC, None) == _lib.SFH_ERR_INVALID
+    ok[0].x_second, ok[0].cin_first = addr, 16                                                             # a cut off the 32-channel grid
+    assert L.sfh_conv3d_wgrad_batch(ok, 1, bf16, addr, one, 0, None) == _lib.SFH_ERR_UNSUPPORTED
+
+
 def test_groupnorm_workspace_and_checks():
     L = _lib.lib()
     d = GroupNormDesc(2, 64, 8, 1, 64 ** 3, 1e-5)
