@@ -503,7 +503,7 @@ extern "C" int sfh_conv3d_pack_weights_batch(const sfh_pack_item* items, int32_t
         return rc;
     }
   }
-  constexpr int kGroup = 32;
+  constexpr int kGroup = 46;  // (an item adds up to two jobs; 48 jobs are one launch)
   MfmaPackItem jobs[kGroup + 2];
   int njobs = 0;
   for (int i = 0; i < nitems; ++i) {
