@@ -189,6 +189,17 @@ def bench_conv(args, device):
                for i, name in enumerate(("fwd", "dgrad", "wgrad"))}
     in_step_spread = {name: spread([m[i].elapsed_time(m[i + 1]) for m in marks])
                       for i, name in enumerate(("fwd", "dgrad", "wgrad"))}
+    # the same step as a captured HIP graph of ten steps (reported beside the eager figure, which stays the headline):
+    # what the five launches of a step cost when the host is out of the way
+    graph_ms = None
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(10):
+                step()
+        graph_ms = event_time_ms(graph.replay, max(2, args.steps // 10), warmup=1) / 10
+    except Exception as exc:  # report, do not hide
+        graph_ms = repr(exc)
     # each direction in a loop of its own (default entry points: forward and data gradient pack per call), and the
     # forward kernel alone in such a loop (weight packed beforehand): with 128 MB of operands per launch these loops
     # run out of the 256 MB memory-side cache and are faster than the same kernels inside the step
@@ -201,6 +212,7 @@ def bench_conv(args, device):
         "flops_per_direction": flops,
         "ms_per_step": ms_per_step,
         "wall_ms_per_step": wall_ms,
+        "graph_ms_per_step": graph_ms,
         "in_step_ms": in_step,
         "in_step_spread": in_step_spread,
         "cold_flushed": cold,
