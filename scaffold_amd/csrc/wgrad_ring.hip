@@ -420,7 +420,11 @@ __device__ __forceinline__ void wring_segment(const WgradArgs& a, const T* __res
 // The wavefronts (0, G) and (1, G) hold sums over different voxels for the same taps: the second hands its
 // accumulators over through LDS (the last barrier has freed it), kHandTaps taps at a time through the group's own
 // array, the first adds them -- a fixed order -- and writes the block's part of a slice: dst points at element
-// (co = first of the block, tap 0, ci = first of the block) of a [Cout][27][cin] slice.
+// (co = first of the block, tap 0, ci = first of the block) of a [Cout][27][cin] slice. IN_LOOP (the batch, where a
+// workgroup hands over in the middle of its range, while the others stream): dst is the block's own 27 x 1024 floats
+// of a slice, written as they lie in the registers -- [tap][r4][lane][4]: lane (kg, j) holds output channels
+// 8 r4 + 4 kg .. + 3 at input channel j -- in 16-byte stores, a quarter of the store instructions; the batch's sum
+// pass puts them in place.
 template <int G, bool IN_LOOP>
 __device__ __forceinline__ void wring_handover(const f32x16_t (&acc)[G == 0 ? kTaps0 : kTaps1], float* __restrict__ dst, int cin, int tid,
                                                const WRingLds& m) {
@@ -433,6 +437,8 @@ __device__ __forceinline__ void wring_handover(const f32x16_t (&acc)[G == 0 ? kT
   // (opaque to the optimiser where the call sits in a loop over blocks: it would otherwise compute all 224 store offsets
   // ahead of the loop and keep them in scratch memory)
   if constexpr (IN_LOOP) asm volatile("" : "+v"(kg));
+  float4* dst4 = reinterpret_cast<float4*>(dst) + lane;
+  if constexpr (IN_LOOP) asm volatile("" : "+v"(dst4));
 #pragma unroll
   for (int round = 0; round < kHandRounds; ++round) {
     if (seg16 == 1) {
@@ -459,10 +465,14 @@ __device__ __forceinline__ void wring_handover(const f32x16_t (&acc)[G == 0 ? kT
           for (int r4 = 0; r4 < 4; ++r4) {
             const float4 o = *reinterpret_cast<const float4*>(handover + ((t - round * kHandTaps) * 4 + r4) * 1024 + lane * 16);
             const float v[4] = {acc[t][4 * r4] + o.x, acc[t][4 * r4 + 1] + o.y, acc[t][4 * r4 + 2] + o.z, acc[t][4 * r4 + 3] + o.w};
+            if constexpr (IN_LOOP) {
+              dst4[(tap * 4 + r4) * 64] = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int co = 8 * r4 + 4 * kg + e;
-              dst[((int64_t)co * 27 + tap) * cin + j] = v[e];
+              for (int e = 0; e < 4; ++e) {
+                const int co = 8 * r4 + 4 * kg + e;
+                dst[((int64_t)co * 27 + tap) * cin + j] = v[e];
+              }
             }
           }
         }
@@ -521,7 +531,7 @@ struct WRingBatchEntry {
   const void* x;
   const void* x1;       // second tensor of the input (channels c_first ..), or null
   const void* gy;
-  float* ws;            // this problem's slices: [slices][Cout][27][Cin]
+  float* ws;            // this problem's slices: [slices][block][27 x 1024 floats in register order, see wring_handover]
   void* gw;
   int c_first;
   int tiles_h, tiles_w, steps, nblk_ci, nblk;
@@ -627,7 +637,7 @@ __device__ __forceinline__ void wring_batch_run(const WRingBatch& b, int w, int 
     }
     const int slice = batch_slices_before(blk, u.col0 / chunk, b.e[p].pos_begin, b.e[p].nblk, b.e[p].ncols, chunk, colcost, b.total, b.wgs) +
                       (w - batch_owner(b0, b.total, b.wgs));
-    wring_handover<G, true>(acc, b.e[p].ws + ((int64_t)slice * a.cout + cob * 32) * 27 * a.cin + cib * 32, a.cin, tid, m);
+    wring_handover<G, true>(acc, b.e[p].ws + ((int64_t)slice * b.e[p].nblk + blk) * (27 * 1024), a.cin, tid, m);
     pos = seg_hi;
   }
 }
@@ -650,7 +660,9 @@ __global__ void __launch_bounds__(256, 1) wgrad_ring_batch_kernel(WRingBatch b) 
 }
 
 // The sum over the slices of every block of every problem of a batch, in slice order (eight, four, two loads in
-// flight), one rounding to the gradient's dtype. A thread owns four consecutive input channels of one (co, tap).
+// flight), one rounding to the gradient's dtype. A slice holds its blocks one after the other, each as the kernel's
+// registers held it ([tap][r4][lane][4], see wring_handover); a thread owns one float4 of a block -- four consecutive
+// output channels at one input channel of one tap -- and the lanes of a wavefront write rows of 32 input channels.
 template <typename TOut>
 __global__ void __launch_bounds__(256) wgrad_ring_batch_sum(WRingBatch b) {
   const int q0 = blockIdx.x * 256;  // a workgroup's 256 float4s lie in one problem (quad_begin is a multiple of 256)
@@ -662,8 +674,9 @@ __global__ void __launch_bounds__(256) wgrad_ring_batch_sum(WRingBatch b) {
   const uint32_t nelem = (uint32_t)cout * 27u * (uint32_t)cin;  // below 2^31 (wring_batch_plan)
   const uint32_t el = (uint32_t)(q - b.e[p].quad_begin) * 4u;
   if (el >= nelem) return;
-  const int ci = (int)(el % (uint32_t)cin), co = (int)(el / (27u * (uint32_t)cin));
-  const int blk = (co / 32) * b.e[p].nblk_ci + ci / 32;
+  const uint32_t quad = el / 4u;
+  const int lane = (int)(quad % 64u), r4 = (int)(quad / 64u % 4u), tap = (int)(quad / 256u % 27u), blk = (int)(quad / (256u * 27u));
+  const int ci = (blk % b.e[p].nblk_ci) * 32 + (lane & 31), co = (blk / b.e[p].nblk_ci) * 32 + 8 * r4 + 4 * (lane >> 5);
   const int chunk = b.e[p].chunk, ncols = b.e[p].ncols;
   const int n = batch_slices_before(blk, (ncols + chunk - 1) / chunk, b.e[p].pos_begin, b.e[p].nblk, ncols, chunk, b.e[p].steps + kFillCost,
                                     b.total, b.wgs);
@@ -694,11 +707,12 @@ __global__ void __launch_bounds__(256) wgrad_ring_batch_sum(WRingBatch b) {
     const float4 v = *reinterpret_cast<const float4*>(part + (int64_t)sp * nelem);
     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
   }
-  TOut* out = (TOut*)b.e[p].gw + el;
+  TOut* out = (TOut*)b.e[p].gw + ((int64_t)co * 27 + tap) * cin + ci;
+  const int64_t row = (int64_t)27 * cin;
   out[0] = elem<TOut>::from_float(s.x);
-  out[1] = elem<TOut>::from_float(s.y);
-  out[2] = elem<TOut>::from_float(s.z);
-  out[3] = elem<TOut>::from_float(s.w);
+  out[row] = elem<TOut>::from_float(s.y);
+  out[2 * row] = elem<TOut>::from_float(s.z);
+  out[3 * row] = elem<TOut>::from_float(s.w);
 }
 
 template <typename T>
