@@ -562,7 +562,7 @@ def bench_unet_step(args, device, eager_only=False):
         model = sa.UNet(1, 11, layers=4, base_width=32).to(device).to(memory_format=CL).set_shard_halo(shard_halo)
         # the weight gradients of the 3x3x3 convolutions wait for the end of the backward pass, where those of levels 0-2
         # (rows of more than 16 voxels) come from one launch and one sum pass instead of eleven of each
-        model.defer_weight_gradients()
+        model.defer_weight_gradients(early=True)
         # clip_grad_norm_(1.0) + Adam (trainer.py:678-694); the update kernel also keeps the bf16 copies of the weights
         # the convolutions read under autocast, and they return fp32 weight gradients: no per-step casts either way
         opt = sa.FusedClipAdam(model.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)

@@ -48,6 +48,12 @@ extern "C" {
                                      autocast) instead of the operands' dtype: the fp32 sum of the slices is
                                      stored as it is, saving the rounding and the caller's up-cast. Served by
                                      the tiled kernels; SFH_ERR_UNSUPPORTED where only the untiled one applies. */
+#define SFH_FLAG_SHARE_DEVICE 8u  /* sfh_conv3d_wgrad_batch (and its workspace query: the workspace depends on it):
+                                     the launch of the problems with rows of more than 16 voxels takes half of the
+                                     compute units, for a batch issued on a stream of its own beside other work (a
+                                     workgroup of that kernel fills a CU's LDS; on the CUs it leaves alone the other
+                                     stream's kernels run undisturbed). Same bits on every run; within summation-order
+                                     rounding of the full-width call's. */
 
 /* A convolution problem as torch.nn.functional.conv3d names it (groups == 1). */
 typedef struct sfh_conv3d_desc {
@@ -85,7 +91,8 @@ typedef struct sfh_groupnorm_desc {
  * workspace since 102 (sfh_conv3d_{fwd,dgrad,wgrad}_workspace_bytes are non-zero for them; callers that sized their
  * workspace with those functions are unaffected).
  * 104: sfh_conv3d_wgrad_batch, sfh_conv3d_wgrad_batch_supported, sfh_conv3d_wgrad_batch_workspace_bytes added;
- * SFH_KERNEL_SPLIT (6) is a value sfh_conv3d_launch_geometry may report. Nothing removed or changed. */
+ * SFH_KERNEL_SPLIT (6) is a value sfh_conv3d_launch_geometry may report. Nothing removed or changed.
+ * 105: SFH_FLAG_SHARE_DEVICE; sfh_conv3d_wgrad_batch_workspace_bytes takes the call's flags (changed: one more argument). */
 int sfh_version(void);
 const char* sfh_last_error(void);
 /* Fills name (<= name_len bytes), compute-unit count, LDS bytes per workgroup. */
@@ -285,7 +292,8 @@ typedef struct sfh_conv3d_wgrad_item {
 /* 0: not served in a batch; 1: served, in the launch of the problems with rows of more than 16 voxels; 2: served, in the
  * launch of the small-volume problems (a caller with more than SFH_WGRAD_BATCH_MAX problems fills its calls by family). */
 int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dtype);
-size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype); /* pointers unused; 0: refused */
+size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype,
+                                              uint32_t flags); /* pointers unused; flags as in the call; 0: refused */
 int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, void* workspace,
                            size_t workspace_bytes, uint32_t flags, void* stream);
 

@@ -19,7 +19,7 @@ _EXPORTS = {
     "is_supported": "conv3d", "is_supported_all": "conv3d", "is_supported_bwd_data": "conv3d",
     "is_supported_bwd_weight": "conv3d", "bwd_data_padding": "conv3d", "grad_weight_empty": "conv3d",
     "workspace_elements": "conv3d", "split_count": "conv3d", "bias_grad": "conv3d",
-    "conv3d_backward_weight_batch": "conv3d", "weight_grad_batchable": "conv3d",
+    "conv3d_backward_weight_batch": "conv3d", "weight_grad_batchable": "conv3d", "weight_grad_batch_family": "conv3d",
     "pack_weights": "conv3d", "packed_weight_bytes": "conv3d", "pack_weights_batch": "conv3d", "PackedWeights": "conv3d",
     "conv_transpose3d_forward": "transposed", "conv_transpose3d_backward_data": "transposed",
     "conv_transpose3d_backward_weight": "transposed", "is_supported_transposed": "transposed",

@@ -41,6 +41,7 @@ SFH_OK, SFH_ERR_INVALID, SFH_ERR_UNSUPPORTED, SFH_ERR_WORKSPACE, SFH_ERR_LAUNCH 
 SFH_FLAG_FORCE_GENERIC = 1
 SFH_FLAG_GRAD_FP32 = 2
 SFH_FLAG_WEIGHT_PACKED = 4
+SFH_FLAG_SHARE_DEVICE = 8
 
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 SUPPORTED_DTYPES = tuple(_DTYPE_CODE)
@@ -138,7 +139,7 @@ _SIGNATURES = {
     "sfh_conv3d_dgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, POINTER(c_int64), c_void_p, c_void_p, c_int32,
                                       c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_wgrad_batch_supported": (c_int, [POINTER(ConvDesc), c_int]),
-    "sfh_conv3d_wgrad_batch_workspace_bytes": (c_size_t, [POINTER(WgradItem), c_int32, c_int]),
+    "sfh_conv3d_wgrad_batch_workspace_bytes": (c_size_t, [POINTER(WgradItem), c_int32, c_int, c_uint32]),
     "sfh_conv3d_wgrad_batch": (c_int, [POINTER(WgradItem), c_int32, c_int, c_void_p, c_size_t, c_uint32, c_void_p]),
     "sfh_conv3d_wgrad_pair": (c_int, [POINTER(ConvDesc), c_int, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,
                                       c_uint32, c_void_p]),

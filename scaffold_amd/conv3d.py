@@ -840,22 +840,28 @@ def conv3d_backward_weight(
 WGRAD_BATCH_MAX = 16  # SFH_WGRAD_BATCH_MAX
 
 
-def weight_grad_batchable(input_shape, weight_shape, stride, padding, dilation, dtype) -> bool:
-    """Whether :func:`conv3d_backward_weight_batch` takes this problem (3x3x3, unit stride and dilation, bf16 / fp16,
-    channel counts multiples of 32, and output rows of more than 16 voxels or a volume of at most 32 tiles of 256
-    voxels): a pure function of the problem."""
+def weight_grad_batch_family(input_shape, weight_shape, stride, padding, dilation, dtype) -> int:
+    """Which launch of :func:`conv3d_backward_weight_batch` takes this problem: 1, the one of the problems with output rows of
+    more than 16 voxels; 2, the one of the small volumes (at most 32 tiles of 256 voxels); 0, neither (it is not 3x3x3 at
+    unit stride and dilation in bf16 / fp16 with channel counts multiples of 32, or fits neither family).  A pure function
+    of the problem."""
     if dtype not in (torch.bfloat16, torch.float16):
-        return False
+        return 0
     try:
         prob = _problem(torch.Size(input_shape), torch.Size(weight_shape), stride, padding, dilation, dtype)
     except (ValueError, NotImplementedError):
-        return False
+        return 0
     if prob.n == 0:
-        return False
-    return bool(_lib.lib().sfh_conv3d_wgrad_batch_supported(ctypes.byref(prob.desc), prob.code))
+        return 0
+    return int(_lib.lib().sfh_conv3d_wgrad_batch_supported(ctypes.byref(prob.desc), prob.code))
 
 
-def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] = None, outs=None):
+def weight_grad_batchable(input_shape, weight_shape, stride, padding, dilation, dtype) -> bool:
+    """Whether :func:`conv3d_backward_weight_batch` takes this problem (see :func:`weight_grad_batch_family`)."""
+    return weight_grad_batch_family(input_shape, weight_shape, stride, padding, dilation, dtype) != 0
+
+
+def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] = None, outs=None, share_device: bool = False):
     """The weight gradients of several convolutions from one launch of the weight-gradient kernel and one sum pass.
 
     ``problems``: a sequence of ``(input, weight_shape, grad_output, padding)`` or ``((first, second), weight_shape,
@@ -864,7 +870,11 @@ def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] 
     What a single launch costs whatever the problem (first fetch, slices written and read back, launch gaps: 15-20 us on
     MI355X) is paid once for the list.  Returns the gradients (``channels_last_3d``, ``grad_dtype`` or the operands' dtype)
     in order; ``outs`` supplies the tensors to write.  Each gradient is a fixed-order fp32 sum that depends on the LIST of
-    shapes only: the same bits on every run, within summation-order rounding of the one-problem call's."""
+    shapes only: the same bits on every run, within summation-order rounding of the one-problem call's.
+
+    ``share_device``: the launch of the problems with rows of more than 16 voxels takes half of the compute units -- for a
+    batch issued on a stream of its own while the current stream has other work (the deferred weight gradients of a
+    backward pass, see ``modules.flush_weight_gradients``)."""
     problems = list(problems)
     if not problems:
         return []
@@ -898,6 +908,8 @@ def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] 
         keep.append((prob, x, x2, g))
         gws.append(gw)
     flags = _lib.SFH_FLAG_GRAD_FP32 if (grad_dtype is not None and grad_dtype is not dt) else 0
+    if share_device:
+        flags |= _lib.SFH_FLAG_SHARE_DEVICE
     # calls of at most WGRAD_BATCH_MAX problems, filled family by family (the problems of a family share a launch)
     family = [int(L.sfh_conv3d_wgrad_batch_supported(ctypes.byref(k[0].desc), k[0].code)) for k in keep]
     if 0 in family:
@@ -916,7 +928,7 @@ def conv3d_backward_weight_batch(problems, *, grad_dtype: Optional[torch.dtype] 
                 it.x, it.x_second, it.cin_first = _lib.ptr(x), (None if x2 is None else _lib.ptr(x2)), (0 if x2 is None else int(x.shape[1]))
                 it.gy, it.gw = _lib.ptr(g), _lib.ptr(gw)
             code = part[0][0].code
-            need = int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, len(part), code))
+            need = int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, len(part), code, flags))
             if need == 0:
                 raise NotImplementedError("conv3d_backward_weight_batch: a problem of the list is not served in a batch "
                                           "(weight_grad_batchable says which)")

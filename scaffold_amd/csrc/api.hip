@@ -280,7 +280,7 @@ __global__ void __launch_bounds__(256) stream_copy_kernel(const uint4* __restric
 
 using namespace sfh;
 
-extern "C" int sfh_version(void) { return 104; }
+extern "C" int sfh_version(void) { return 105; }
 
 extern "C" const char* sfh_last_error(void) { return g_error; }
 
@@ -783,10 +783,13 @@ extern "C" int sfh_conv3d_wgrad_batch_supported(const sfh_conv3d_desc* p, int dt
   return mfma_wgrad_ring_applies(wgrad_args(*p, out)) ? 1 : 2;
 }
 
-extern "C" size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype) {
+// SFH_FLAG_SHARE_DEVICE: the launch of the large-row family takes half of the compute units
+static int wgrad_batch_max_wgs(uint32_t flags) { return (flags & SFH_FLAG_SHARE_DEVICE) ? kComputeUnits / 2 : 0; }
+
+extern "C" size_t sfh_conv3d_wgrad_batch_workspace_bytes(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, uint32_t flags) {
   WgradBatchItem list[SFH_WGRAD_BATCH_MAX];
   if (wgrad_batch_items(items, count, dtype, list) != SFH_OK) return 0;
-  return mfma_wgrad_batch_workspace_bytes(list, count);
+  return mfma_wgrad_batch_workspace_bytes(list, count, wgrad_batch_max_wgs(flags));
 }
 
 extern "C" int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_t count, int dtype, void* workspace, size_t workspace_bytes,
@@ -797,7 +800,7 @@ extern "C" int sfh_conv3d_wgrad_batch(const sfh_conv3d_wgrad_item* items, int32_
     if (list[i].x == nullptr || list[i].gy == nullptr || list[i].gw == nullptr) return fail(SFH_ERR_INVALID, "conv3d wgrad batch: null tensor");
   if (flags & SFH_FLAG_FORCE_GENERIC) return fail(SFH_ERR_INVALID, "conv3d wgrad batch: the direct kernels take one problem a call");
   const int gw_dtype = (flags & SFH_FLAG_GRAD_FP32) ? SFH_FP32 : dtype;
-  return mfma_wgrad_batch(list, count, dtype, gw_dtype, workspace, workspace_bytes, (hipStream_t)stream);
+  return mfma_wgrad_batch(list, count, dtype, gw_dtype, workspace, workspace_bytes, (hipStream_t)stream, wgrad_batch_max_wgs(flags));
 }
 
 // ---- bias gradient ---------------------------------------------------------------------

@@ -693,7 +693,7 @@ bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype) {
   return mfma_wgrad_supported(a, dtype) && (ring_serves(a) || tile_batch_applies(a));
 }
 
-size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count) {
+size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count, int max_wgs) {
   if (count < 1 || count > kWgradBatchMax) return 0;
   WgradBatchItem ring[kWgradBatchMax], tile[kWgradBatchMax];
   int nring, ntile;
@@ -701,12 +701,12 @@ size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count) 
   WTileBatch tb;
   if (ntile > 0 && !tile_batch_plan(tile, ntile, tb)) return 0;
   if (nring == 0) return 256;  // (nothing is needed; a non-zero answer says the list is taken)
-  const size_t bytes = mfma_wgrad_ring_batch_workspace_bytes(ring, nring);
+  const size_t bytes = mfma_wgrad_ring_batch_workspace_bytes(ring, nring, max_wgs);
   return bytes;
 }
 
 int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
-                     hipStream_t st) {
+                     hipStream_t st, int max_wgs) {
   if (count < 1 || count > kWgradBatchMax) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: 1 .. %d problems a call", kWgradBatchMax);
   WgradBatchItem ring[kWgradBatchMax], tile[kWgradBatchMax];
   int nring, ntile;
@@ -715,7 +715,7 @@ int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_d
   WTileBatch tb;
   if (ntile > 0 && !tile_batch_plan(tile, ntile, tb)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: the small-volume problems cannot share a launch");
   if (nring > 0)
-    if (int rc = mfma_wgrad_ring_batch(ring, nring, dtype, gw_dtype, workspace, workspace_bytes, st)) return rc;
+    if (int rc = mfma_wgrad_ring_batch(ring, nring, dtype, gw_dtype, workspace, workspace_bytes, st, max_wgs)) return rc;
   if (ntile > 0) return dtype == SFH_BF16 ? launch_tile_batch<bf16_t>(tb, gw_dtype, st) : launch_tile_batch<fp16_t>(tb, gw_dtype, st);
   return SFH_OK;
 }

@@ -44,12 +44,13 @@ struct WgradBatchItem {
   void* gw;
 };
 bool mfma_wgrad_batch_applies(const WgradArgs& a, int dtype);
-size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count);  // 0: the list cannot share a launch
+// max_wgs > 0: the ring-served launch takes at most that many workgroups (it is meant to run beside other work)
+size_t mfma_wgrad_batch_workspace_bytes(const WgradBatchItem* items, int count, int max_wgs);  // 0: the list cannot share a launch
 int mfma_wgrad_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
-                     hipStream_t st);
+                     hipStream_t st, int max_wgs);
 // the ring-served family alone (every item must be ring-served)
-size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count);
+size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count, int max_wgs);
 int mfma_wgrad_ring_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
-                          hipStream_t st);
+                          hipStream_t st, int max_wgs);
 
 }  // namespace sfh

@@ -790,7 +790,7 @@ int launch_wring(const WgradArgs& a, const WRingGeom& gm, const void* x, const v
 
 // The line of cost and the slices of a batch; ws_bytes: the workspace all problems need together. False when the batch
 // cannot be laid out (too many problems, too much work for 32-bit positions).
-bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, size_t& ws_bytes) {
+bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, size_t& ws_bytes, int max_wgs) {
   if (count < 1 || count > kWgradBatchMax) return false;
   b = WRingBatch{};
   b.count = count;
@@ -822,6 +822,8 @@ bool wring_batch_plan(const WgradBatchItem* items, int count, WRingBatch& b, siz
   // without a step still costs its block a slice of zeros)
   b.wgs = b.total / (2 * kFillCost);
   if (b.wgs > kComputeUnits) b.wgs = kComputeUnits;
+  // (a launch meant to run beside other work takes fewer workgroups: one to a CU, the CUs it leaves alone are the others')
+  if (max_wgs > 0 && b.wgs > max_wgs) b.wgs = max_wgs;
   if (b.wgs < 1) b.wgs = 1;
   ws_bytes = 0;
   for (int i = 0; i < count; ++i) {
@@ -862,17 +864,17 @@ int mfma_wgrad_ring(const WgradArgs& a, int dtype, const void* x, const void* gy
   return launch_wring<fp16_t>(a, gm, x, gy, ws, st, x2);
 }
 
-size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count) {
+size_t mfma_wgrad_ring_batch_workspace_bytes(const WgradBatchItem* items, int count, int max_wgs) {
   WRingBatch b;
   size_t bytes = 0;
-  return wring_batch_plan(items, count, b, bytes) ? bytes : 0;
+  return wring_batch_plan(items, count, b, bytes, max_wgs) ? bytes : 0;
 }
 
 int mfma_wgrad_ring_batch(const WgradBatchItem* items, int count, int dtype, int gw_dtype, void* workspace, size_t workspace_bytes,
-                          hipStream_t st) {
+                          hipStream_t st, int max_wgs) {
   WRingBatch b;
   size_t need = 0;
-  if (!wring_batch_plan(items, count, b, need)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: %d problems cannot share a launch", count);
+  if (!wring_batch_plan(items, count, b, need, max_wgs)) return fail(SFH_ERR_UNSUPPORTED, "conv3d wgrad batch: %d problems cannot share a launch", count);
   if (workspace == nullptr || workspace_bytes < need)
     return fail(SFH_ERR_WORKSPACE, "conv3d wgrad batch: workspace of %zu bytes needed, got %zu", need, workspace_bytes);
   char* ws = (char*)workspace;

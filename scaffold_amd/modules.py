@@ -124,25 +124,26 @@ def _fp32_weight_grad(fn, *args, **kwargs):
 # differs: hooks on the parameter's gradient accumulation do not see these gradients, and the operands stay alive until
 # the end of the pass.
 class _QueuedWeightGrad:
-    __slots__ = ("param", "inp", "wshape", "gy", "padding", "grad_dtype")
+    __slots__ = ("param", "inp", "wshape", "gy", "padding", "grad_dtype", "family", "early")
 
-    def __init__(self, param, inp, wshape, gy, padding, grad_dtype):
+    def __init__(self, param, inp, wshape, gy, padding, grad_dtype, family=1, early=False):
         self.param, self.inp, self.wshape, self.gy, self.padding, self.grad_dtype = param, inp, wshape, gy, padding, grad_dtype
+        self.family, self.early = family, early  # the launch that takes it (1: large rows, 2: small volumes); early mode
 
 
 _WEIGHT_GRAD_QUEUE: list = []
 _BATCHABLE: dict = {}
 
 
-def _deferrable(param, in_shape, wshape, stride, padding, dilation, dtype) -> bool:
+def _deferrable(param, in_shape, wshape, stride, padding, dilation, dtype) -> int:
     """Whether a weight gradient can wait for the end of the pass: the parameter is a leaf that takes a ``.grad`` and the
-    library batches the problem."""
+    library batches the problem.  0, or the launch of the batch that takes it (``conv3d.weight_grad_batch_family``)."""
     if param is None or not param.is_leaf or not param.requires_grad:
-        return False
+        return 0
     key = (in_shape, wshape, stride, padding, dilation, dtype)
     ok = _BATCHABLE.get(key)
     if ok is None:
-        ok = _c3.weight_grad_batchable(in_shape, wshape, stride, padding, dilation, dtype)
+        ok = _c3.weight_grad_batch_family(in_shape, wshape, stride, padding, dilation, dtype)
         if len(_BATCHABLE) > 256:
             _BATCHABLE.clear()
         _BATCHABLE[key] = ok
@@ -154,11 +155,56 @@ def _queue_weight_grad(item: _QueuedWeightGrad) -> None:
     # one callback per queued gradient: the first to run takes the whole queue, the others find it empty (a pass that
     # raised before its callbacks ran leaves its entries to the next pass's callbacks, or to flush_weight_gradients())
     torch.autograd.Variable._execution_engine.queue_callback(flush_weight_gradients)
+    if item.early and item.family == 2:
+        # The pass has reached a small volume: the deep levels, whose kernels are bound by latency and leave most of the
+        # device idle. The large-row gradients queued so far (the decoder's upper levels) go out now, on a stream of their own
+        # and on half of the compute units, beside the rest of the pass; flush_weight_gradients() joins them.
+        waiting = [it for it in _WEIGHT_GRAD_QUEUE if it.family == 1 and it.early and it.gy.device == item.gy.device and
+                   it.gy.dtype is item.gy.dtype and it.grad_dtype is item.grad_dtype]
+        if len(waiting) >= 2:
+            for it in waiting:
+                _WEIGHT_GRAD_QUEUE.remove(it)
+            _send_early(waiting)
+
+
+_EARLY_STREAMS: dict = {}
+_EARLY_DONE: list = []
+
+
+def _send_early(items) -> None:
+    dev = items[0].gy.device
+    side = _EARLY_STREAMS.get(dev)
+    if side is None:
+        side = _EARLY_STREAMS[dev] = torch.cuda.Stream(device=dev)
+    # Every use of the side stream starts by waiting for the current one and ends (in flush_weight_gradients) with the
+    # current one waiting for it, and the operands stay referenced until then: memory the caching allocator hands to
+    # either stream is never in use on the other.
+    side.wait_stream(torch.cuda.current_stream(dev))
+    gdt, dt = items[0].grad_dtype, items[0].gy.dtype
+    with torch.no_grad(), torch.cuda.stream(side):
+        grads = _c3.conv3d_backward_weight_batch([(it.inp, it.wshape, it.gy, it.padding) for it in items],
+                                                 grad_dtype=None if gdt is dt else gdt, share_device=True)
+    _EARLY_DONE.append((items, grads, side))
+
+
+def _add_to_grads(items, grads) -> None:
+    for it, gw in zip(items, grads):
+        p = it.param
+        if p.grad is None:
+            # in the parameter's own layout, as the engine's accumulation would leave it
+            p.grad = gw if gw.stride() == p.stride() else torch.empty_like(p).copy_(gw)
+        else:
+            p.grad.add_(gw)
 
 
 def flush_weight_gradients() -> None:
     """Compute the queued weight gradients and add them to their parameters' ``.grad`` (runs by itself at the end of a
     backward pass; callable by hand after a pass that raised)."""
+    while _EARLY_DONE:
+        items, grads, side = _EARLY_DONE.pop(0)
+        torch.cuda.current_stream(items[0].gy.device).wait_stream(side)
+        with torch.no_grad():
+            _add_to_grads(items, grads)
     if not _WEIGHT_GRAD_QUEUE:
         return
     queue = list(_WEIGHT_GRAD_QUEUE)
@@ -170,13 +216,7 @@ def flush_weight_gradients() -> None:
         for (_, dt, gdt), items in groups.items():
             grads = _c3.conv3d_backward_weight_batch([(it.inp, it.wshape, it.gy, it.padding) for it in items],
                                                      grad_dtype=None if gdt is dt else gdt)
-            for it, gw in zip(items, grads):
-                p = it.param
-                if p.grad is None:
-                    # in the parameter's own layout, as the engine's accumulation would leave it
-                    p.grad = gw if gw.stride() == p.stride() else torch.empty_like(p).copy_(gw)
-                else:
-                    p.grad.add_(gw)
+            _add_to_grads(items, grads)
 
 
 # positions in _Conv3dFn.forward's argument list (after ctx): the gradients come back in this order
@@ -227,6 +267,7 @@ class _Conv3dFn(torch.autograd.Function):
                          weight.dtype is not wc.dtype)
         # the parameter whose .grad a deferred weight gradient is added to (see flush_weight_gradients)
         ctx.defer_param = weight if defer_weight_grad else None
+        ctx.defer_early = defer_weight_grad == 2
         return y
 
     @staticmethod
@@ -252,9 +293,10 @@ class _Conv3dFn(torch.autograd.Function):
                 if grad_b.dtype is not bias_dtype:
                     grad_b = grad_b.to(bias_dtype)
                 return grad_x, grad_w, grad_b, None, None, None, None, None, None, None, None, None, None, None
-        if needs_w and _deferrable(ctx.defer_param, x.shape, weight.shape, stride, padding, dilation, x.dtype):
+        family = _deferrable(ctx.defer_param, x.shape, weight.shape, stride, padding, dilation, x.dtype) if needs_w else 0
+        if family:
             _queue_weight_grad(_QueuedWeightGrad(ctx.defer_param, x, weight.shape, grad_output, padding,
-                                                 torch.float32 if master else x.dtype))
+                                                 torch.float32 if master else x.dtype, family, ctx.defer_early))
         elif needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight, x, weight.shape, grad_output, stride, padding, dilation, 1,
@@ -282,10 +324,13 @@ class _Conv3dFn(torch.autograd.Function):
                 grad_x = grad_x.narrow(2, ctx.halo, ctx.depth)
                 grad_second = grad_second.narrow(2, ctx.halo, ctx.depth)
         grad_w = None
-        if needs_w and _deferrable(ctx.defer_param, torch.Size((x.shape[0], x.shape[1] + second.shape[1], *x.shape[2:])), weight.shape,
-                                   stride, padding, dilation, x.dtype):
+        family = 0
+        if needs_w:
+            family = _deferrable(ctx.defer_param, torch.Size((x.shape[0], x.shape[1] + second.shape[1], *x.shape[2:])), weight.shape,
+                                 stride, padding, dilation, x.dtype)
+        if family:
             _queue_weight_grad(_QueuedWeightGrad(ctx.defer_param, (x, second), weight.shape, grad_output, padding,
-                                                 torch.float32 if master else x.dtype))
+                                                 torch.float32 if master else x.dtype, family, ctx.defer_early))
         elif needs_w:
             if master:
                 grad_w = _fp32_weight_grad(_c3.conv3d_backward_weight_pair, x, second, weight.shape, grad_output, stride, padding,
@@ -356,7 +401,9 @@ class FastConv3d(nn.Conv3d):
     #: GroupNorm's statistics on its result, where the kernel offers it, and the normalisation skips its statistics pass
     gn_groups = 0
     #: leave this module's weight gradient to the end of the backward pass, where all such gradients come from one launch
-    #: (see flush_weight_gradients); taken up only where the weight is the parameter itself and the library batches the shape
+    #: (see flush_weight_gradients); taken up only where the weight is the parameter itself and the library batches the shape.
+    #: 2 instead of True: besides, the large-row gradients queued when the pass reaches its first small volume are computed
+    #: there and then on a stream of their own, on half of the device, beside the rest of the pass
     defer_weight_grad = False
 
     def _pair_operands(self, x, second):
@@ -443,7 +490,7 @@ class FastConv3d(nn.Conv3d):
                                    second, slab2, self.defer_weight_grad)
         packs = _current_packs(w, w, in_shape, stride, padding, dilation) if w is weight else None
         return _Conv3dFn.apply(x, w, b, stride, padding, dilation, None, None, packs, slab, self.gn_groups, second,
-                               slab2, self.defer_weight_grad and w is weight)
+                               slab2, self.defer_weight_grad if w is weight else False)
 
     def forward(self, x: torch.Tensor, second: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``second``: the input is ``torch.cat([x, second], 1)``, read from the two tensors themselves (the decoder's skip

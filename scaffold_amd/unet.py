@@ -211,13 +211,17 @@ class UNet(nn.Module):
                 block.double_conv[4].out_halo = halo
         return self
 
-    def defer_weight_gradients(self, enabled: bool = True):
+    def defer_weight_gradients(self, enabled: bool = True, early: bool = False):
         """Leave the weight gradients of the 3x3x3 convolutions to the end of the backward pass, where one launch computes
         all that the library batches (``modules.flush_weight_gradients``): ``.grad`` is complete when ``backward()``
-        returns, as always; hooks on the parameters' gradient accumulation do not see these gradients."""
+        returns, as always; hooks on the parameters' gradient accumulation do not see these gradients.
+
+        ``early``: the gradients of the decoder's upper levels do not wait for the end: when the backward pass reaches the
+        deep levels (small volumes: kernels bound by latency, most of the device idle) they are computed on a stream of
+        their own, on half of the compute units, beside the rest of the pass, and joined where the others are computed."""
         for m in self.modules():
             if isinstance(m, FastConv3d):
-                m.defer_weight_grad = bool(enabled)
+                m.defer_weight_grad = (2 if early else True) if enabled else False
         return self
 
     def _run(self, block, *inputs):

@@ -188,18 +188,21 @@ def test_weight_gradient_batch_plan_and_refusals():
             it.desc = d
         return arr
 
-    one = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16)
-    two = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, ring), 2, bf16)
-    mixed = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, small), 2, bf16)
+    one = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16, 0)
+    two = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, ring), 2, bf16, 0)
+    mixed = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, small), 2, bf16, 0)
     assert one > 0 and two > 0 and mixed > 0
     # every workgroup writes one 32 x 32 x 27 fp32 slice per unit it touches: at least a slice a block, a few hundred at most
     block = 32 * 32 * 27 * 4
     assert 2 * block <= one <= 1024 * block
-    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16) == one        # a pure function of the list
-    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(small, small), 2, bf16) > 0   # nothing needed, still not 0
-    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, large16), 2, bf16) == 0
-    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 0, bf16) == 0
-    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(*([ring] * 17)), 17, bf16) == 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 1, bf16, 0) == one        # a pure function of the list
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(small, small), 2, bf16, 0) > 0   # nothing needed, still not 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, large16), 2, bf16, 0) == 0
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring), 0, bf16, 0) == 0
+    # half of the compute units for a batch that runs beside other work: fewer workgroups, no more slices
+    shared = L.sfh_conv3d_wgrad_batch_workspace_bytes(items(ring, ring), 2, bf16, _lib.SFH_FLAG_SHARE_DEVICE)
+    assert 0 < shared <= two
+    assert L.sfh_conv3d_wgrad_batch_workspace_bytes(items(*([ring] * 17)), 17, bf16, 0) == 0
     addr = ctypes.c_void_p(256)  # never dereferenced: every call below is refused before a launch
     bad = items(ring, large16)
     for it in bad:

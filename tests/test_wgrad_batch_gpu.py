@@ -77,6 +77,12 @@ def test_batch_against_the_oracle_and_the_single_calls(device, dtype, name):
         # the two sum the same products in different orders: fp32 rounding of sums of up to ~1e5 terms
         scale = single.abs().max().item()
         assert (g - single).abs().max().item() <= 2e-5 * scale
+    # on half of the compute units (a batch meant to run beside other work): another cut, the same sums
+    shared = sa.conv3d_backward_weight_batch(problems, grad_dtype=torch.float32, share_device=True)
+    shared2 = sa.conv3d_backward_weight_batch(problems, grad_dtype=torch.float32, share_device=True)
+    for g, s1, s2 in zip(got, shared, shared2):
+        assert torch.equal(s1, s2)
+        assert (g - s1).abs().max().item() <= 2e-5 * g.abs().max().item()
 
 
 def test_the_cut_depends_on_the_shapes_alone(device):
@@ -127,7 +133,7 @@ def test_what_is_refused(device):
         gws.append(gw)
         it.desc, it.x, it.x_second, it.cin_first, it.gy, it.gw = prob.desc, _lib.ptr(x), None, 0, _lib.ptr(gy), _lib.ptr(gw)
     code = c3._problem(good[0][0].shape, torch.Size(good[0][1]), 1, (1, 1, 1), 1, dtype).code
-    need = int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, 2, code))
+    need = int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, 2, code, 0))
     assert need > 0
     ws = torch.empty(need, dtype=torch.uint8, device=device)
     stream = _lib.stream_ptr(device)
@@ -138,13 +144,15 @@ def test_what_is_refused(device):
     torch.cuda.synchronize()
     assert torch.equal(gws[0], sa.conv3d_backward_weight_batch(good)[0])
     items[1].desc.sd = 2                                            # a strided problem in the list
-    assert int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, 2, code)) == 0
+    assert int(L.sfh_conv3d_wgrad_batch_workspace_bytes(items, 2, code, 0)) == 0
     assert L.sfh_conv3d_wgrad_batch(items, 2, code, _lib.ptr(ws), need, 0, stream) == _lib.SFH_ERR_UNSUPPORTED
 
 
-def _tiny_net(device, defer):
+def _tiny_net(device, defer, layers=2):
     torch.manual_seed(7)
-    net = sa.UNet(1, 3, layers=2, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
+    net = sa.UNet(1, 3, layers=layers, base_width=32).to(device).to(memory_format=CL).set_shard_halo(True)
+    if defer == "early":
+        return net.defer_weight_gradients(early=True)
     return net.defer_weight_gradients() if defer else net
 
 
@@ -271,3 +279,65 @@ def test_deferred_step_as_a_hip_graph_and_under_checkpointing(device):
     for n, g in grads[False].items():
         d = grads[True][n].float()
         assert (g.float() - d).abs().max().item() <= 2e-2 * max(g.float().abs().max().item(), 1e-30), n
+
+
+def test_early_weight_gradients_on_a_stream_of_their_own(device, monkeypatch):
+    """With ``defer_weight_gradients(early=True)`` the large-row gradients queued when the backward pass reaches its first
+    small volume leave on a side stream (half of the compute units) and are joined at the end of the pass: every gradient
+    is there when ``backward()`` returns, within summation-order rounding of the ordinary pass's; the captured step replays
+    to the eager step's losses."""
+    x = torch.randn(1, 1, 8, 32, 64, device=device).contiguous(memory_format=CL)
+    target = torch.randint(0, 3, (1, 8, 32, 64), device=device)
+    sent = []
+    real = modules._send_early
+    monkeypatch.setattr(modules, "_send_early", lambda items: (sent.append(len(items)), real(items))[1])
+    grads = {}
+    for defer in (False, "early"):
+        net = _tiny_net(device, defer, layers=3)
+        opt = sa.FusedClipAdam(net.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+        for rep in range(2):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                logits = net(x)
+            sa.ce_dice_loss(logits, target).backward()
+            assert not modules._WEIGHT_GRAD_QUEUE and not modules._EARLY_DONE
+        grads[defer] = {n: p.grad.detach().clone() for n, p in net.named_parameters()}
+    assert sent and all(n >= 2 for n in sent)                 # the side stream was used, once per pass
+    for n, g in grads[False].items():
+        d = grads["early"][n]
+        assert d.dtype is g.dtype and d.stride() == g.stride(), n
+        assert (g.float() - d.float()).abs().max().item() <= 2 * 2e-5 * max(g.float().abs().max().item(), 1e-30), n
+
+    def make():
+        net = _tiny_net(device, "early", layers=3)
+        opt = sa.FusedClipAdam(net.parameters(), lr=1e-3, max_norm=1.0, shadow_dtype=torch.bfloat16)
+
+        def step():
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                logits = net(x)
+            loss = sa.ce_dice_loss(logits, target)
+            loss.backward()
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+            return loss.detach()
+        return step
+
+    eager = make()
+    want = [eager().item() for _ in range(4)]
+    step2 = make()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        warm = step2().item()
+    torch.cuda.current_stream().wait_stream(side)
+    assert warm == want[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = step2()
+    got = []
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        got.append(static_loss.item())
+        torch.randn(1 << 16, device=device).sum().item()
+    assert got == want[1:]
+    assert not modules._WEIGHT_GRAD_QUEUE and not modules._EARLY_DONE
